@@ -1,0 +1,189 @@
+"""Pins oracle/llama_ref.py: (1) the batched/causal functions equal the literal
+single-token step of test/llama.py replayed with a real KV cache; (2) the
+closed-form adjoints equal the reference's per-op rules chained in trace order;
+(3) central finite differences; (4) an independent torch.autograd restatement;
+(5) closed-form special cases."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import llama_ref as L
+
+CFG = {"dim": 24, "hidden_dim": 40, "n_layers": 2, "n_heads": 3, "n_kv_heads": 3,
+       "vocab_size": 50, "seq_len": 8}
+
+
+def _weights(cfg, seed=0, uniform=False):
+    w = L.make_weights(cfg, seed, std=0.3, dtype=np.float64)
+    if uniform:   # the reference fixture draws uniform[0,1) (test/llama.py:266-291)
+        rng = np.random.default_rng(seed)
+        w = {k: rng.uniform(0, 1, size=v.shape) for k, v in w.items()}
+    return w
+
+
+@pytest.mark.parametrize("uniform", [False, True])
+def test_batched_forward_equals_step_form_replayed(uniform):
+    cfg, S = CFG, 6
+    w = _weights(cfg, 3, uniform)
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((1, S, cfg["dim"]))
+    kc = np.zeros((cfg["n_layers"], 0, cfg["dim"]))
+    vc = np.zeros((cfg["n_layers"], 0, cfg["dim"]))
+    outs = []
+    for t in range(S):
+        y, kc, vc = L.forward_step(x[0, t], cfg, w, kc, vc, return_caches=True)
+        outs.append(y)
+    got, _ = L.model_fwd(x, w, cfg, logits=False)
+    np.testing.assert_allclose(got[0], np.stack(outs), rtol=1e-10, atol=1e-12)
+
+
+def test_step_form_reference_fixture_shape():
+    """The shipped fixture: pos = 1 with an all-zero cached row (llama.py:299-301):
+    softmax weights are [1, e^s]/(1+e^s)."""
+    cfg = CFG
+    w = _weights(cfg, 1, uniform=True)
+    x = np.random.default_rng(2).uniform(0, 1, cfg["dim"])
+    kc = np.zeros((cfg["n_layers"], 1, cfg["dim"]))
+    y = L.forward_step(x, cfg, w, kc, kc.copy())
+    assert y.shape == (cfg["dim"],) and np.all(np.isfinite(y))
+
+
+def test_rule_chained_adjoints_equal_closed_forms():
+    rng = np.random.default_rng(7)
+    x, g, dy = rng.standard_normal(16), rng.uniform(0.5, 1.5, 16), rng.standard_normal(16)
+    dx_r, dg_r = L.rmsnorm_bwd_by_rules(x, g, dy)
+    dx_c, dg_c = L.rmsnorm_bwd(x[None], g, dy[None])
+    np.testing.assert_allclose(dx_c[0], dx_r, rtol=1e-12, atol=1e-14)
+    np.testing.assert_allclose(dg_c, dg_r, rtol=1e-12, atol=1e-14)
+    # softmax: rule chain (incl. the reduce-max path) vs P*(dP - sum(dP*P))
+    s, dp = rng.standard_normal(9), rng.standard_normal(9)
+    p = L.softmax(s)
+    np.testing.assert_allclose(L.softmax_bwd_by_rules(s, dp), p * (dp - np.sum(dp * p)), rtol=1e-12, atol=1e-14)
+    # ... also with a tie at the maximum (every arg-max gets the cotangent; it cancels)
+    s[3] = s[5] = s.max() + 1.0
+    p = L.softmax(s)
+    np.testing.assert_allclose(L.softmax_bwd_by_rules(s, dp), p * (dp - np.sum(dp * p)), rtol=1e-12, atol=1e-13)
+    a, b, dgv = rng.standard_normal(11), rng.standard_normal(11), rng.standard_normal(11)
+    da_r, db_r = L.silu_mul_bwd_by_rules(a, b, dgv)
+    da_c, db_c = L.swiglu_bwd(a, b, dgv)
+    np.testing.assert_allclose(da_c, da_r, rtol=1e-12)
+    np.testing.assert_allclose(db_c, db_r, rtol=1e-12)
+
+
+def test_special_cases():
+    # rmsnorm of a constant vector c: gamma * c / sqrt(c^2 + eps)
+    c, g = 3.0, np.linspace(0.5, 1.5, 8)
+    np.testing.assert_allclose(L.rmsnorm_fwd(np.full((1, 8), c), g), (g * c / np.sqrt(c * c + 1e-5))[None], rtol=1e-14)
+    # rope: position 0 is the identity; pair norms preserved; inverse undoes
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal((2, 5, 3, 8))
+    cos, sin = L.rope_angles(5, 8)
+    y = L.rope_fwd(x, cos, sin)
+    np.testing.assert_allclose(y[:, 0], x[:, 0], rtol=1e-14)
+    np.testing.assert_allclose(y[..., 0::2] ** 2 + y[..., 1::2] ** 2, x[..., 0::2] ** 2 + x[..., 1::2] ** 2, rtol=1e-12)
+    np.testing.assert_allclose(L.rope_fwd(y, cos, sin, inverse=True), x, rtol=1e-12, atol=1e-14)
+    # first frequency is 1 rad per position, last is theta^-(d-2)/d
+    assert np.isclose(cos[3, 0], np.cos(3.0)) and np.isclose(sin[4, 3], np.sin(4.0 * 10000 ** (-6 / 8)))
+    # attention with S = 1: out = v; softmax rows sum to one => lse consistent
+    q, k, v = (rng.standard_normal((1, 2, 1, 4)) for _ in range(3))
+    o, lse = L.attention_fwd(q, k, v)
+    np.testing.assert_allclose(o, v, rtol=1e-14)
+    # causal: the first query only sees key 0
+    q, k, v = (rng.standard_normal((1, 2, 6, 4)) for _ in range(3))
+    o, lse = L.attention_fwd(q, k, v)
+    np.testing.assert_allclose(o[:, :, 0], v[:, :, 0], rtol=1e-13)
+    s = np.einsum("bhqd,bhkd->bhqk", q, k) / 2.0
+    np.testing.assert_allclose(lse[0, 0, 2], np.log(np.sum(np.exp(s[0, 0, 2, :3]))), rtol=1e-13)
+
+
+def _fd(f, x, dy, h=1e-6):
+    g = np.zeros_like(x)
+    it = np.nditer(x, flags=["multi_index"])
+    for _ in it:
+        i = it.multi_index
+        xp, xm = x.copy(), x.copy()
+        xp[i] += h
+        xm[i] -= h
+        g[i] = np.sum((f(xp) - f(xm)) * dy) / (2 * h)
+    return g
+
+
+def test_layer_backward_matches_finite_differences():
+    cfg = {"dim": 8, "hidden_dim": 12, "n_layers": 1, "n_heads": 2}
+    rng = np.random.default_rng(11)
+    lw = {k: rng.standard_normal(s) * 0.4 for k, s in
+          [("rms_att_weight", (8,)), ("wq", (8, 8)), ("wk", (8, 8)), ("wv", (8, 8)), ("wo", (8, 8)),
+           ("rms_ffn_weight", (8,)), ("w1", (12, 8)), ("w2", (8, 12)), ("w3", (12, 8))]}
+    x = rng.standard_normal((2, 3, 8))
+    dy = rng.standard_normal((2, 3, 8))
+    y, cache = L.layer_fwd(x, lw, 2)
+    dx, gw = L.layer_bwd(dy, lw, cache, 2)
+    np.testing.assert_allclose(dx, _fd(lambda t: L.layer_fwd(t, lw, 2)[0], x, dy), rtol=2e-6, atol=2e-8)
+    for name in lw:
+        def f(wv, name=name):
+            l2 = dict(lw)
+            l2[name] = wv
+            return L.layer_fwd(x, l2, 2)[0]
+        np.testing.assert_allclose(gw[name], _fd(f, lw[name], dy), rtol=5e-6, atol=5e-8, err_msg=name)
+
+
+# ---- independent torch restatement (written against test/llama.py, not the oracle)
+
+def _torch_model(tokens, w, cfg, logits):
+    D, nh = cfg["dim"], cfg["n_heads"]
+    d = D // nh
+    x = w["token_embedding_table"][tokens]
+    B, S, _ = x.shape
+    pos = torch.arange(S, dtype=torch.float64)
+    freq = 1.0 / torch.pow(torch.tensor(10000.0, dtype=torch.float64), torch.arange(0, d, 2, dtype=torch.float64) / d)
+    ang = pos[:, None] * freq[None]
+    rot = torch.polar(torch.ones_like(ang), ang)      # complex rotation e^{i angle}
+
+    def norm(t, g):
+        return g * t * torch.rsqrt((t * t).mean(-1, keepdim=True) + 1e-5)
+
+    def rope(t):
+        tc = torch.view_as_complex(t.reshape(B, S, nh, d // 2, 2).contiguous())
+        return torch.view_as_real(tc * rot[None, :, None, :]).reshape(B, S, nh, d)
+
+    for i in range(cfg["n_layers"]):
+        xb = norm(x, w["rms_att_weight"][i])
+        q = rope((xb @ w["wq"][i].T).reshape(B, S, nh, d)).transpose(1, 2)
+        k = rope((xb @ w["wk"][i].T).reshape(B, S, nh, d)).transpose(1, 2)
+        v = (xb @ w["wv"][i].T).reshape(B, S, nh, d).transpose(1, 2)
+        o = torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True)
+        x = x + o.transpose(1, 2).reshape(B, S, D) @ w["wo"][i].T
+        xb = norm(x, w["rms_ffn_weight"][i])
+        x = x + (torch.nn.functional.silu(xb @ w["w1"][i].T) * (xb @ w["w3"][i].T)) @ w["w2"][i].T
+    x = norm(x, w["rms_final_weight"])
+    return x @ w["wcls"].T if logits else x
+
+
+@pytest.mark.parametrize("logits", [False, True])
+def test_model_forward_backward_matches_torch_autograd(logits):
+    cfg = CFG
+    w = _weights(cfg, 9)
+    rng = np.random.default_rng(4)
+    tokens = rng.integers(0, cfg["vocab_size"], size=(2, 7))
+    out, fc = L.model_fwd(tokens, w, cfg, logits=logits)
+    dout = rng.standard_normal(out.shape)
+    _, gw = L.model_bwd(dout, w, cfg, fc)
+    tw = {k: torch.tensor(v, dtype=torch.float64, requires_grad=True) for k, v in w.items()}
+    tout = _torch_model(torch.tensor(tokens), tw, cfg, logits)
+    np.testing.assert_allclose(out, tout.detach().numpy(), rtol=1e-9, atol=1e-11)
+    tout.backward(torch.tensor(dout))
+    for k in gw:
+        if k == "wcls" and not logits:
+            continue
+        np.testing.assert_allclose(gw[k], tw[k].grad.numpy(), rtol=1e-8, atol=1e-10, err_msg=k)
+
+
+def test_attention_backward_adjoint_identity():
+    """<J v, w> = <v, J^T w> with J v from a forward-difference of the forward."""
+    rng = np.random.default_rng(21)
+    q, k, v, do = (rng.standard_normal((1, 2, 5, 4)) for _ in range(4))
+    dq, dk, dv = L.attention_bwd(q, k, v, do)
+    tq, tk, tv = (rng.standard_normal(q.shape) for _ in range(3))
+    h = 1e-6
+    jp = (L.attention_fwd(q + h * tq, k + h * tk, v + h * tv)[0] - L.attention_fwd(q - h * tq, k - h * tk, v - h * tv)[0]) / (2 * h)
+    assert np.isclose(np.sum(jp * do), np.sum(tq * dq) + np.sum(tk * dk) + np.sum(tv * dv), rtol=1e-7)
