@@ -1,0 +1,825 @@
+// Causal softmax attention, forward and adjoint, for gfx950.
+//
+// Fast path (bf16, head_dim 64 or 128): flash-style, scores never leave the
+// CU.  Everything is computed "transposed" so that one lane owns one query
+// (forward, dQ) or one key (dK/dV) for its whole life:
+//   S^T[key,query] = K . Q^T     MFMA A = K rows from LDS, B = Q in registers
+//   O^T[d,query]   = V^T . P^T   MFMA A = V columns via the transposing LDS
+//                                load, B = P straight from the accumulator
+// so the softmax row statistics are per-lane scalars (one exchange with lane
+// ^32 per tile) and rescaling O needs no cross-lane traffic.  K/V (or Q/dO)
+// tiles stream HBM -> LDS with 16-byte direct-to-LDS loads, double buffered.
+// The adjoint is atomics-free and deterministic: one kernel owns query blocks
+// and produces dQ, another owns key blocks and produces dK and dV; both
+// recompute P from q, k and the saved log-sum-exp.
+//
+// Generic path (fp32 or any other head_dim <= 256): one wavefront per query
+// (or key) row, plain fp32 FMA, same maths.
+#include <initializer_list>
+
+#include "emi_device.h"
+
+namespace emi {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4_t;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
+typedef __attribute__((__vector_size__(8 * sizeof(float)))) float f32x8_t;
+
+#define EMI_LDS __attribute__((address_space(3)))
+
+constexpr uint32_t kOobA = 0x80000000u;
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+constexpr float kNegBig = -1.0e30f;
+
+struct AttnShape {
+  int seq, heads;
+  int64_t sb, sh, ss;   // element strides of batch, head, sequence position
+};
+
+// ===========================================================================
+// Generic path
+// ===========================================================================
+
+// One wavefront per query.  Lanes split the keys of a 64-key chunk for the
+// scores and split head_dim for the output.
+template <typename T>
+__global__ __launch_bounds__(256) void attn_fwd_generic_kernel(const T* __restrict__ q, const T* __restrict__ k,
+                                                               const T* __restrict__ v, T* __restrict__ o,
+                                                               float* __restrict__ lse, AttnShape sh, int d, float scale,
+                                                               int causal) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int qi = blockIdx.x * 4 + wave;
+  const int bh = blockIdx.y;
+  if (qi >= sh.seq) return;
+  const int64_t base = (int64_t)(bh / sh.heads) * sh.sb + (int64_t)(bh % sh.heads) * sh.sh;
+  const T* qr = q + base + (int64_t)qi * sh.ss;
+  const int nkeys = causal ? qi + 1 : sh.seq;
+  float m = kNegBig, l = 0.f;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < nkeys; k0 += 64) {
+    const int key = k0 + lane;
+    float s = kNegBig;
+    if (key < nkeys) {
+      const T* kr = k + base + (int64_t)key * sh.ss;
+      float dot = 0.f;
+      for (int i = 0; i < d; i++) dot += to_f32(qr[i]) * to_f32(kr[i]);
+      s = dot * scale;
+    }
+    const float m_new = fmaxf(m, wave_max(s));
+    const float alpha = expf(m - m_new);
+    const float p = key < nkeys ? expf(s - m_new) : 0.f;
+    l = l * alpha + wave_sum(p);
+#pragma unroll
+    for (int c = 0; c < 4; c++) acc[c] *= alpha;
+    const int cnt = nkeys - k0 < 64 ? nkeys - k0 : 64;
+    for (int j = 0; j < cnt; j++) {
+      const float pj = __shfl(p, j, 64);
+      const T* vr = v + base + (int64_t)(k0 + j) * sh.ss;
+#pragma unroll
+      for (int c = 0; c < 4; c++) {
+        const int i = lane + c * 64;
+        if (i < d) acc[c] += pj * to_f32(vr[i]);
+      }
+    }
+    m = m_new;
+  }
+  T* orow = o + base + (int64_t)qi * sh.ss;
+#pragma unroll
+  for (int c = 0; c < 4; c++) {
+    const int i = lane + c * 64;
+    if (i < d) orow[i] = from_f32<T>(acc[c] / l);
+  }
+  if (lane == 0) lse[(int64_t)bh * sh.seq + qi] = m + logf(l);
+}
+
+// delta[b,h,s] = sum_i dO[b,h,s,i] * O[b,h,s,i]; one wavefront per row.
+template <typename T>
+__global__ __launch_bounds__(256) void attn_delta_kernel(const T* __restrict__ o, const T* __restrict__ d_o,
+                                                         float* __restrict__ delta, AttnShape sh, int d) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int qi = blockIdx.x * 4 + wave;
+  const int bh = blockIdx.y;
+  if (qi >= sh.seq) return;
+  const int64_t off = (int64_t)(bh / sh.heads) * sh.sb + (int64_t)(bh % sh.heads) * sh.sh + (int64_t)qi * sh.ss;
+  float s = 0.f;
+  for (int i = lane; i < d; i += 64) s += to_f32(o[off + i]) * to_f32(d_o[off + i]);
+  s = wave_sum(s);
+  if (lane == 0) delta[(int64_t)bh * sh.seq + qi] = s;
+}
+
+// dQ: one wavefront per query.
+template <typename T>
+__global__ __launch_bounds__(256) void attn_bwd_dq_generic_kernel(const T* __restrict__ q, const T* __restrict__ k,
+                                                                  const T* __restrict__ v, const T* __restrict__ d_o,
+                                                                  const float* __restrict__ lse,
+                                                                  const float* __restrict__ delta, T* __restrict__ dq,
+                                                                  AttnShape sh, int d, float scale, int causal) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int qi = blockIdx.x * 4 + wave;
+  const int bh = blockIdx.y;
+  if (qi >= sh.seq) return;
+  const int64_t base = (int64_t)(bh / sh.heads) * sh.sb + (int64_t)(bh % sh.heads) * sh.sh;
+  const T* qr = q + base + (int64_t)qi * sh.ss;
+  const T* dor = d_o + base + (int64_t)qi * sh.ss;
+  const float L = lse[(int64_t)bh * sh.seq + qi], dl = delta[(int64_t)bh * sh.seq + qi];
+  const int nkeys = causal ? qi + 1 : sh.seq;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < nkeys; k0 += 64) {
+    const int key = k0 + lane;
+    float ds = 0.f;
+    if (key < nkeys) {
+      const T* kr = k + base + (int64_t)key * sh.ss;
+      const T* vr = v + base + (int64_t)key * sh.ss;
+      float dot = 0.f, dp = 0.f;
+      for (int i = 0; i < d; i++) {
+        dot += to_f32(qr[i]) * to_f32(kr[i]);
+        dp += to_f32(dor[i]) * to_f32(vr[i]);
+      }
+      const float p = expf(dot * scale - L);
+      ds = p * (dp - dl) * scale;
+    }
+    const int cnt = nkeys - k0 < 64 ? nkeys - k0 : 64;
+    for (int j = 0; j < cnt; j++) {
+      const float dsj = __shfl(ds, j, 64);
+      const T* kr = k + base + (int64_t)(k0 + j) * sh.ss;
+#pragma unroll
+      for (int c = 0; c < 4; c++) {
+        const int i = lane + c * 64;
+        if (i < d) acc[c] += dsj * to_f32(kr[i]);
+      }
+    }
+  }
+  T* out = dq + base + (int64_t)qi * sh.ss;
+#pragma unroll
+  for (int c = 0; c < 4; c++) {
+    const int i = lane + c * 64;
+    if (i < d) out[i] = from_f32<T>(acc[c]);
+  }
+}
+
+// dK, dV: one wavefront per key.
+template <typename T>
+__global__ __launch_bounds__(256) void attn_bwd_dkv_generic_kernel(const T* __restrict__ q, const T* __restrict__ k,
+                                                                   const T* __restrict__ v, const T* __restrict__ d_o,
+                                                                   const float* __restrict__ lse,
+                                                                   const float* __restrict__ delta, T* __restrict__ dk,
+                                                                   T* __restrict__ dv, AttnShape sh, int d, float scale,
+                                                                   int causal) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int ki = blockIdx.x * 4 + wave;
+  const int bh = blockIdx.y;
+  if (ki >= sh.seq) return;
+  const int64_t base = (int64_t)(bh / sh.heads) * sh.sb + (int64_t)(bh % sh.heads) * sh.sh;
+  const T* kr = k + base + (int64_t)ki * sh.ss;
+  const T* vr = v + base + (int64_t)ki * sh.ss;
+  const int qstart = causal ? ki : 0;
+  float acck[4] = {0.f, 0.f, 0.f, 0.f}, accv[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int q0 = qstart; q0 < sh.seq; q0 += 64) {
+    const int qi = q0 + lane;
+    float p = 0.f, ds = 0.f;
+    if (qi < sh.seq) {
+      const T* qr = q + base + (int64_t)qi * sh.ss;
+      const T* dor = d_o + base + (int64_t)qi * sh.ss;
+      float dot = 0.f, dp = 0.f;
+      for (int i = 0; i < d; i++) {
+        dot += to_f32(qr[i]) * to_f32(kr[i]);
+        dp += to_f32(dor[i]) * to_f32(vr[i]);
+      }
+      p = expf(dot * scale - lse[(int64_t)bh * sh.seq + qi]);
+      ds = p * (dp - delta[(int64_t)bh * sh.seq + qi]) * scale;
+    }
+    const int cnt = sh.seq - q0 < 64 ? sh.seq - q0 : 64;
+    for (int j = 0; j < cnt; j++) {
+      const float pj = __shfl(p, j, 64), dsj = __shfl(ds, j, 64);
+      const T* qr = q + base + (int64_t)(q0 + j) * sh.ss;
+      const T* dor = d_o + base + (int64_t)(q0 + j) * sh.ss;
+#pragma unroll
+      for (int c = 0; c < 4; c++) {
+        const int i = lane + c * 64;
+        if (i < d) {
+          accv[c] += pj * to_f32(dor[i]);
+          acck[c] += dsj * to_f32(qr[i]);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < 4; c++) {
+    const int i = lane + c * 64;
+    if (i < d) {
+      dk[base + (int64_t)ki * sh.ss + i] = from_f32<T>(acck[c]);
+      dv[base + (int64_t)ki * sh.ss + i] = from_f32<T>(accv[c]);
+    }
+  }
+}
+
+// ===========================================================================
+// bf16 MFMA path
+// ===========================================================================
+
+// LDS tile [rows][D] bf16.  16-byte chunk c of row r lives at chunk
+// c ^ swz<D>(r), chosen so that 16 consecutive rows at one logical chunk
+// (ds_read_b128 operand fetch) and 4 consecutive rows x 64 bytes (the
+// transposing ds_read_b64_tr_b16 fetch) both spread over all banks.
+template <int D> __device__ __forceinline__ int swz(int row);
+template <> __device__ __forceinline__ int swz<128>(int row) { return ((row & 3) << 2) | ((row >> 2) & 3); }
+template <> __device__ __forceinline__ int swz<64>(int row) { return (((row >> 1) & 1) << 2) | ((row >> 2) & 3); }
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t attn_rsrc(const void* p, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes, 0x00020000);
+}
+
+// Stream a [ROWS][D] tile (rows row0.. of one head) into LDS; rows >= seq read
+// as zeros.  `rsrc` is based at the head's first element.
+template <int D, int ROWS, int NW>
+__device__ __forceinline__ void load_rows_tile(__amdgpu_buffer_rsrc_t rsrc, EMI_LDS uint8_t* lds, int wave, int lane,
+                                               int row0, int seq, int64_t ss) {
+  constexpr int CPR = D / 8;              // chunks per row
+  constexpr int RPL = 64 / CPR;           // rows per wave-load
+  constexpr int NLOAD = ROWS / RPL / NW;
+  static_assert(NLOAD >= 1, "tile smaller than one pass of the block");
+#pragma unroll
+  for (int it = 0; it < NLOAD; it++) {
+    const int r = (it * NW + wave) * RPL + lane / CPR;
+    const int pc = lane % CPR;
+    const int lc = pc ^ swz<D>(r);
+    uint32_t voff = (uint32_t)((int64_t)(row0 + r) * ss + lc * 8) * 2u;
+    if (row0 + r >= seq) voff = kOobA;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, lds + (it * NW + wave) * 1024, 16, voff, 0, 0, 0);
+  }
+}
+
+// Operand fragment "32 tile rows x 16 of D": lane l holds row row_base + (l & 31),
+// D-index 16*step + 8*(l >> 5) + 0..7.
+template <int D>
+__device__ __forceinline__ bf16x8_t row_frag(const EMI_LDS uint8_t* tile, int row_base, int step, int lane) {
+  const int row = row_base + (lane & 31);
+  const int chunk = (step * 2 + (lane >> 5)) ^ swz<D>(row);
+  return *reinterpret_cast<const EMI_LDS bf16x8_t*>(tile + row * (D * 2) + chunk * 16);
+}
+
+// Operand fragment "32 of D x 16 tile rows" (the tile transposed): lane l holds
+// D-index col_base + (l & 31) and tile rows row_base + 4*(l>>5) + {0..3, 8..11},
+// which is exactly the row set a lane owns in registers 8s..8s+7 of a 32x32
+// accumulator (row_base = 16*s within the 32-row sub-tile).
+template <int D>
+__device__ __forceinline__ bf16x8_t col_frag(const EMI_LDS uint8_t* tile, int row_base, int col_base, int lane) {
+  const int i = lane & 15;
+  const int r0 = row_base + (lane >> 5) * 4 + (i >> 2);
+  const int r1 = r0 + 8;
+  const int col = col_base + ((lane >> 4) & 1) * 16 + (i & 3) * 4;
+  const int chunk = col >> 3, within = (col & 7) * 2;
+  const EMI_LDS uint8_t* p0 = tile + r0 * (D * 2) + ((chunk ^ swz<D>(r0)) * 16) + within;
+  const EMI_LDS uint8_t* p1 = tile + r1 * (D * 2) + ((chunk ^ swz<D>(r1)) * 16) + within;
+  bf16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((EMI_LDS bf16x4_t*)p0);
+  bf16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((EMI_LDS bf16x4_t*)p1);
+  return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+// Eight consecutive accumulator registers -> one bf16x8 MFMA operand.
+__device__ __forceinline__ bf16x8_t acc_to_frag(const f32x16_t& a, int s) {
+  f32x8_t t;
+#pragma unroll
+  for (int e = 0; e < 8; e++) t[e] = a[8 * s + e];
+  return __builtin_convertvector(t, bf16x8_t);
+}
+
+// Register-resident operand: 32 rows (one per lane & 31) x D, straight from HBM.
+template <int D>
+__device__ __forceinline__ void load_reg_rows(const uint16_t* head_base, int row, int seq, int64_t ss, int lane,
+                                              bf16x8_t (&f)[D / 16]) {
+#pragma unroll
+  for (int t = 0; t < D / 16; t++) {
+    if (row < seq) {
+      f[t] = *reinterpret_cast<const bf16x8_t*>(head_base + (int64_t)row * ss + t * 16 + 8 * (lane >> 5));
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; e++) f[t][e] = (__bf16)0.0f;
+    }
+  }
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// Row index inside a 32x32 accumulator tile held by register r of this lane.
+__device__ __forceinline__ int acc_row(int r, int lane) { return 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3); }
+
+// ---------------------------------------------------------------------------
+// Forward: block = 4 waves x 32 queries, KV tiles of 64 keys.
+// ---------------------------------------------------------------------------
+template <int D>
+__global__ __launch_bounds__(256) void attn_fwd_bf16_kernel(const uint16_t* __restrict__ q,
+                                                            const uint16_t* __restrict__ k,
+                                                            const uint16_t* __restrict__ v, uint16_t* __restrict__ o,
+                                                            float* __restrict__ lse, AttnShape sh, uint32_t head_bytes,
+                                                            float scale_log2e, int causal) {
+  constexpr int BQ = 128, BKV = 64, NW = 4;
+  constexpr int TILE = BKV * D * 2, STAGE = 2 * TILE;
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem_raw[];
+  EMI_LDS uint8_t* smem = (EMI_LDS uint8_t*)smem_raw;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int qblk = gridDim.x - 1 - blockIdx.x;       // longest rows first
+  const int bh = blockIdx.y;
+  const int64_t base = (int64_t)(bh / sh.heads) * sh.sb + (int64_t)(bh % sh.heads) * sh.sh;
+  const int seq = sh.seq;
+  const int q0 = qblk * BQ + wave * 32;
+  const int qrow = q0 + (lane & 31);
+
+  bf16x8_t qf[D / 16];
+  load_reg_rows<D>(q + base, qrow, seq, sh.ss, lane, qf);
+
+  const __amdgpu_buffer_rsrc_t rK = attn_rsrc(k + base, head_bytes);
+  const __amdgpu_buffer_rsrc_t rV = attn_rsrc(v + base, head_bytes);
+  const int kv_end = causal ? (qblk * BQ + BQ < seq ? qblk * BQ + BQ : seq) : seq;
+  const int nkv = (kv_end + BKV - 1) / BKV;
+
+  f32x16_t acc_o[D / 32];
+#pragma unroll
+  for (int dt = 0; dt < D / 32; dt++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc_o[dt][r] = 0.f;
+  float m = kNegBig, l = 0.f;
+
+  load_rows_tile<D, BKV, NW>(rK, smem, wave, lane, 0, seq, sh.ss);
+  load_rows_tile<D, BKV, NW>(rV, smem + TILE, wave, lane, 0, seq, sh.ss);
+  __builtin_amdgcn_s_waitcnt(0x0f70);
+  __syncthreads();
+
+  for (int j = 0; j < nkv; j++) {
+    if (j + 1 < nkv) {
+      EMI_LDS uint8_t* nxt = smem + ((j + 1) & 1) * STAGE;
+      load_rows_tile<D, BKV, NW>(rK, nxt, wave, lane, (j + 1) * BKV, seq, sh.ss);
+      load_rows_tile<D, BKV, NW>(rV, nxt + TILE, wave, lane, (j + 1) * BKV, seq, sh.ss);
+    }
+    const EMI_LDS uint8_t* sK = smem + (j & 1) * STAGE;
+    const EMI_LDS uint8_t* sV = sK + TILE;
+    const int key0 = j * BKV;
+    if (!(causal && key0 > q0 + 31)) {     // wave-uniform: this tile is not entirely in the future
+      f32x16_t s[2];
+#pragma unroll
+      for (int T = 0; T < 2; T++) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) s[T][r] = 0.f;
+#pragma unroll
+        for (int t = 0; t < D / 16; t++)
+          s[T] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(row_frag<D>(sK, T * 32, t, lane), qf[t], s[T], 0, 0, 0);
+      }
+      const bool need_mask = (causal && key0 + BKV - 1 > q0) || key0 + BKV > seq;
+      float mt = kNegBig;
+#pragma unroll
+      for (int T = 0; T < 2; T++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          float x = s[T][r] * scale_log2e;
+          if (need_mask) {
+            const int key = key0 + T * 32 + acc_row(r, lane);
+            if ((causal && key > qrow) || key >= seq) x = kNegBig;
+          }
+          s[T][r] = x;
+          mt = fmaxf(mt, x);
+        }
+      mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+      const float m_new = fmaxf(m, mt);
+      const float alpha = fast_exp2(m - m_new);
+      float rs = 0.f;
+#pragma unroll
+      for (int T = 0; T < 2; T++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const float p = fast_exp2(s[T][r] - m_new);
+          s[T][r] = p;
+          rs += p;
+        }
+      l = l * alpha + rs;
+      m = m_new;
+#pragma unroll
+      for (int dt = 0; dt < D / 32; dt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc_o[dt][r] *= alpha;
+#pragma unroll
+      for (int T = 0; T < 2; T++)
+#pragma unroll
+        for (int sI = 0; sI < 2; sI++) {
+          const bf16x8_t pf = acc_to_frag(s[T], sI);
+#pragma unroll
+          for (int dt = 0; dt < D / 32; dt++)
+            acc_o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(col_frag<D>(sV, T * 32 + sI * 16, dt * 32, lane), pf,
+                                                                acc_o[dt], 0, 0, 0);
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(0x0f70);
+    __syncthreads();
+  }
+
+  l += __shfl_xor(l, 32, 64);
+  if (qrow < seq) {
+    const float inv = 1.0f / l;
+    uint16_t* orow = o + base + (int64_t)qrow * sh.ss;
+#pragma unroll
+    for (int dt = 0; dt < D / 32; dt++)
+#pragma unroll
+      for (int jj = 0; jj < 4; jj++) {
+        const int dcol = dt * 32 + 8 * jj + 4 * (lane >> 5);
+        uint2 w;
+        w.x = pack_bf16x2(acc_o[dt][4 * jj] * inv, acc_o[dt][4 * jj + 1] * inv);
+        w.y = pack_bf16x2(acc_o[dt][4 * jj + 2] * inv, acc_o[dt][4 * jj + 3] * inv);
+        *reinterpret_cast<uint2*>(orow + dcol) = w;
+      }
+    if (lane < 32) lse[(int64_t)bh * seq + qrow] = (m + __builtin_amdgcn_logf(l)) * kLn2;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// dQ: block = 4 waves x 32 queries; K and V tiles of 64 keys through LDS.
+//   S^T = K Q^T, dP^T = V dO^T, dS^T = P^T (dP^T - delta), dQ^T = K^T dS^T
+// ---------------------------------------------------------------------------
+template <int D>
+__global__ __launch_bounds__(256) void attn_bwd_dq_bf16_kernel(const uint16_t* __restrict__ q,
+                                                               const uint16_t* __restrict__ k,
+                                                               const uint16_t* __restrict__ v,
+                                                               const uint16_t* __restrict__ d_o,
+                                                               const float* __restrict__ lse,
+                                                               const float* __restrict__ delta,
+                                                               uint16_t* __restrict__ dq, AttnShape sh,
+                                                               uint32_t head_bytes, float scale, int causal) {
+  constexpr int BQ = 128, BKV = 64, NW = 4;
+  constexpr int TILE = BKV * D * 2, STAGE = 2 * TILE;
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem_raw[];
+  EMI_LDS uint8_t* smem = (EMI_LDS uint8_t*)smem_raw;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int qblk = gridDim.x - 1 - blockIdx.x;
+  const int bh = blockIdx.y;
+  const int64_t base = (int64_t)(bh / sh.heads) * sh.sb + (int64_t)(bh % sh.heads) * sh.sh;
+  const int seq = sh.seq;
+  const int q0 = qblk * BQ + wave * 32;
+  const int qrow = q0 + (lane & 31);
+  const float scale_log2e = scale * kLog2e;
+
+  bf16x8_t qf[D / 16], dof[D / 16];
+  load_reg_rows<D>(q + base, qrow, seq, sh.ss, lane, qf);
+  load_reg_rows<D>(d_o + base, qrow, seq, sh.ss, lane, dof);
+  const float L2 = qrow < seq ? lse[(int64_t)bh * seq + qrow] * kLog2e : 0.f;
+  const float dl = qrow < seq ? delta[(int64_t)bh * seq + qrow] : 0.f;
+
+  const __amdgpu_buffer_rsrc_t rK = attn_rsrc(k + base, head_bytes);
+  const __amdgpu_buffer_rsrc_t rV = attn_rsrc(v + base, head_bytes);
+  const int kv_end = causal ? (qblk * BQ + BQ < seq ? qblk * BQ + BQ : seq) : seq;
+  const int nkv = (kv_end + BKV - 1) / BKV;
+
+  f32x16_t acc[D / 32];
+#pragma unroll
+  for (int dt = 0; dt < D / 32; dt++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[dt][r] = 0.f;
+
+  load_rows_tile<D, BKV, NW>(rK, smem, wave, lane, 0, seq, sh.ss);
+  load_rows_tile<D, BKV, NW>(rV, smem + TILE, wave, lane, 0, seq, sh.ss);
+  __builtin_amdgcn_s_waitcnt(0x0f70);
+  __syncthreads();
+
+  for (int j = 0; j < nkv; j++) {
+    if (j + 1 < nkv) {
+      EMI_LDS uint8_t* nxt = smem + ((j + 1) & 1) * STAGE;
+      load_rows_tile<D, BKV, NW>(rK, nxt, wave, lane, (j + 1) * BKV, seq, sh.ss);
+      load_rows_tile<D, BKV, NW>(rV, nxt + TILE, wave, lane, (j + 1) * BKV, seq, sh.ss);
+    }
+    const EMI_LDS uint8_t* sK = smem + (j & 1) * STAGE;
+    const EMI_LDS uint8_t* sV = sK + TILE;
+    const int key0 = j * BKV;
+    if (!(causal && key0 > q0 + 31)) {
+      const bool need_mask = (causal && key0 + BKV - 1 > q0) || key0 + BKV > seq;
+#pragma unroll
+      for (int T = 0; T < 2; T++) {
+        f32x16_t s, dp;
+#pragma unroll
+        for (int r = 0; r < 16; r++) s[r] = 0.f, dp[r] = 0.f;
+#pragma unroll
+        for (int t = 0; t < D / 16; t++) {
+          s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(row_frag<D>(sK, T * 32, t, lane), qf[t], s, 0, 0, 0);
+          dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(row_frag<D>(sV, T * 32, t, lane), dof[t], dp, 0, 0, 0);
+        }
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          float p = fast_exp2(s[r] * scale_log2e - L2);
+          if (need_mask) {
+            const int key = key0 + T * 32 + acc_row(r, lane);
+            if ((causal && key > qrow) || key >= seq) p = 0.f;
+          }
+          s[r] = p * (dp[r] - dl);
+        }
+#pragma unroll
+        for (int sI = 0; sI < 2; sI++) {
+          const bf16x8_t dsf = acc_to_frag(s, sI);
+#pragma unroll
+          for (int dt = 0; dt < D / 32; dt++)
+            acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(col_frag<D>(sK, T * 32 + sI * 16, dt * 32, lane), dsf,
+                                                              acc[dt], 0, 0, 0);
+        }
+      }
+    }
+    __builtin_amdgcn_s_waitcnt(0x0f70);
+    __syncthreads();
+  }
+  if (qrow < seq) {
+    uint16_t* out = dq + base + (int64_t)qrow * sh.ss;
+#pragma unroll
+    for (int dt = 0; dt < D / 32; dt++)
+#pragma unroll
+      for (int jj = 0; jj < 4; jj++) {
+        const int dcol = dt * 32 + 8 * jj + 4 * (lane >> 5);
+        uint2 w;
+        w.x = pack_bf16x2(acc[dt][4 * jj] * scale, acc[dt][4 * jj + 1] * scale);
+        w.y = pack_bf16x2(acc[dt][4 * jj + 2] * scale, acc[dt][4 * jj + 3] * scale);
+        *reinterpret_cast<uint2*>(out + dcol) = w;
+      }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// dK, dV: block = 4 waves x 32 keys; Q and dO tiles of 64 queries through LDS.
+//   S = Q K^T, dP = dO V^T (lane = key, registers = queries)
+//   dV^T = dO^T P, dK^T = Q^T dS
+// ---------------------------------------------------------------------------
+template <int D>
+__global__ __launch_bounds__(256) void attn_bwd_dkv_bf16_kernel(const uint16_t* __restrict__ q,
+                                                                const uint16_t* __restrict__ k,
+                                                                const uint16_t* __restrict__ v,
+                                                                const uint16_t* __restrict__ d_o,
+                                                                const float* __restrict__ lse,
+                                                                const float* __restrict__ delta,
+                                                                uint16_t* __restrict__ dk, uint16_t* __restrict__ dv,
+                                                                AttnShape sh, uint32_t head_bytes, float scale,
+                                                                int causal) {
+  constexpr int BKEY = 128, BQT = 64, NW = 4;
+  constexpr int TILE = BQT * D * 2, STAGE = 2 * TILE + 2 * BQT * 4;   // Q, dO, lse, delta
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem_raw[];
+  EMI_LDS uint8_t* smem = (EMI_LDS uint8_t*)smem_raw;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int kblk = blockIdx.x;                         // early key blocks see the most queries: first
+  const int bh = blockIdx.y;
+  const int64_t base = (int64_t)(bh / sh.heads) * sh.sb + (int64_t)(bh % sh.heads) * sh.sh;
+  const int seq = sh.seq;
+  const int k0 = kblk * BKEY + wave * 32;
+  const int krow = k0 + (lane & 31);
+  const float scale_log2e = scale * kLog2e;
+
+  bf16x8_t kf[D / 16], vf[D / 16];
+  load_reg_rows<D>(k + base, krow, seq, sh.ss, lane, kf);
+  load_reg_rows<D>(v + base, krow, seq, sh.ss, lane, vf);
+
+  const __amdgpu_buffer_rsrc_t rQ = attn_rsrc(q + base, head_bytes);
+  const __amdgpu_buffer_rsrc_t rDO = attn_rsrc(d_o + base, head_bytes);
+  const float* lse_h = lse + (int64_t)bh * seq;
+  const float* delta_h = delta + (int64_t)bh * seq;
+  const int qt0 = causal ? (kblk * BKEY) / BQT : 0;     // first query tile that can see this key block
+  const int nqt = (seq + BQT - 1) / BQT;
+
+  f32x16_t acc_k[D / 32], acc_v[D / 32];
+#pragma unroll
+  for (int dt = 0; dt < D / 32; dt++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc_k[dt][r] = 0.f, acc_v[dt][r] = 0.f;
+
+  auto issue = [&](int stage, int qt) {
+    EMI_LDS uint8_t* s0 = smem + stage * STAGE;
+    load_rows_tile<D, BQT, NW>(rQ, s0, wave, lane, qt * BQT, seq, sh.ss);
+    load_rows_tile<D, BQT, NW>(rDO, s0 + TILE, wave, lane, qt * BQT, seq, sh.ss);
+    if (threadIdx.x < BQT) {
+      const int qi = qt * BQT + threadIdx.x;
+      EMI_LDS float* st = (EMI_LDS float*)(s0 + 2 * TILE);
+      st[threadIdx.x] = qi < seq ? lse_h[qi] * kLog2e : 0.f;
+      st[BQT + threadIdx.x] = qi < seq ? delta_h[qi] : 0.f;
+    }
+  };
+
+  if (qt0 < nqt) issue(0, qt0);
+  __builtin_amdgcn_s_waitcnt(0x0070);   // vmcnt(0) and lgkmcnt(0)
+  __syncthreads();
+
+  for (int qt = qt0; qt < nqt; qt++) {
+    const int it = qt - qt0;
+    if (qt + 1 < nqt) issue((it + 1) & 1, qt + 1);
+    const EMI_LDS uint8_t* sQ = smem + (it & 1) * STAGE;
+    const EMI_LDS uint8_t* sDO = sQ + TILE;
+    const EMI_LDS float* sL = (const EMI_LDS float*)(sQ + 2 * TILE);
+    const EMI_LDS float* sDl = sL + BQT;
+    const int qbase = qt * BQT;
+    if (!(causal && qbase + BQT - 1 < k0)) {          // some query of the tile can see some key of this wave
+      const bool need_mask = (causal && qbase < k0 + 31) || qbase + BQT > seq || k0 + 32 > seq;
+#pragma unroll
+      for (int T = 0; T < 2; T++) {
+        f32x16_t s, dp;
+#pragma unroll
+        for (int r = 0; r < 16; r++) s[r] = 0.f, dp[r] = 0.f;
+#pragma unroll
+        for (int t = 0; t < D / 16; t++) {
+          s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(row_frag<D>(sQ, T * 32, t, lane), kf[t], s, 0, 0, 0);
+          dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(row_frag<D>(sDO, T * 32, t, lane), vf[t], dp, 0, 0, 0);
+        }
+        f32x16_t ds;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const int ql = T * 32 + acc_row(r, lane);     // query inside the tile
+          float p = fast_exp2(s[r] * scale_log2e - sL[ql]);
+          if (need_mask) {
+            const int qi = qbase + ql;
+            if ((causal && krow > qi) || qi >= seq || krow >= seq) p = 0.f;
+          }
+          s[r] = p;
+          ds[r] = p * (dp[r] - sDl[ql]);
+        }
+#pragma unroll
+        for (int sI = 0; sI < 2; sI++) {
+          const bf16x8_t pf = acc_to_frag(s, sI);
+          const bf16x8_t dsf = acc_to_frag(ds, sI);
+#pragma unroll
+          for (int dt = 0; dt < D / 32; dt++) {
+            acc_v[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(col_frag<D>(sDO, T * 32 + sI * 16, dt * 32, lane), pf,
+                                                                acc_v[dt], 0, 0, 0);
+            acc_k[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(col_frag<D>(sQ, T * 32 + sI * 16, dt * 32, lane), dsf,
+                                                                acc_k[dt], 0, 0, 0);
+          }
+        }
+      }
+    }
+    __builtin_amdgcn_s_waitcnt(0x0070);
+    __syncthreads();
+  }
+  if (krow < seq) {
+    uint16_t* outk = dk + base + (int64_t)krow * sh.ss;
+    uint16_t* outv = dv + base + (int64_t)krow * sh.ss;
+#pragma unroll
+    for (int dt = 0; dt < D / 32; dt++)
+#pragma unroll
+      for (int jj = 0; jj < 4; jj++) {
+        const int dcol = dt * 32 + 8 * jj + 4 * (lane >> 5);
+        uint2 w;
+        w.x = pack_bf16x2(acc_k[dt][4 * jj] * scale, acc_k[dt][4 * jj + 1] * scale);
+        w.y = pack_bf16x2(acc_k[dt][4 * jj + 2] * scale, acc_k[dt][4 * jj + 3] * scale);
+        *reinterpret_cast<uint2*>(outk + dcol) = w;
+        w.x = pack_bf16x2(acc_v[dt][4 * jj], acc_v[dt][4 * jj + 1]);
+        w.y = pack_bf16x2(acc_v[dt][4 * jj + 2], acc_v[dt][4 * jj + 3]);
+        *reinterpret_cast<uint2*>(outv + dcol) = w;
+      }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------
+
+static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+struct AttnArgs {
+  int64_t batch, heads, seq, d, sb, sh, ss;
+};
+
+static int check_common(const char* name, const AttnArgs& a, int dtype) {
+  EMI_REQUIRE(a.batch >= 0 && a.heads > 0 && a.seq > 0 && a.d > 0, "%s: bad shape [%lld,%lld,%lld,%lld]", name,
+              (long long)a.batch, (long long)a.heads, (long long)a.seq, (long long)a.d);
+  EMI_REQUIRE(dtype == EMI_F32 || dtype == EMI_BF16, "%s: unsupported dtype code %d (want 11=f32 or 16=bf16)", name, dtype);
+  EMI_REQUIRE(a.d <= 256, "%s: head_dim %lld > 256 is not supported", name, (long long)a.d);
+  EMI_REQUIRE(a.ss >= a.d && a.sh > 0 && a.sb > 0, "%s: bad strides (b=%lld h=%lld s=%lld)", name, (long long)a.sb,
+              (long long)a.sh, (long long)a.ss);
+  EMI_REQUIRE(a.seq <= 0x7fffffff / 4 && a.batch * a.heads <= 65535, "%s: seq or batch*heads too large", name);
+  return EMI_OK;
+}
+
+// The MFMA path needs 16-byte chunks and 32-bit byte offsets inside one head.
+static bool mfma_ok(const AttnArgs& a, int dtype, std::initializer_list<const void*> ptrs) {
+  if (dtype != EMI_BF16 || (a.d != 64 && a.d != 128)) return false;
+  if ((a.sb % 8) || (a.sh % 8) || (a.ss % 8)) return false;
+  if ((a.seq - 1) * a.ss + a.d >= (int64_t)0x3fffff00) return false;
+  for (const void* p : ptrs)
+    if (!aligned16(p)) return false;
+  return true;
+}
+
+template <typename K> static int reserve_lds(K kern, int bytes, const char* name) {
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e != hipSuccess) return emi_fail(EMI_INTERNAL, "%s: cannot reserve %d bytes of LDS: %s", name, bytes, hipGetErrorString(e));
+  return EMI_OK;
+}
+
+}  // namespace emi
+
+using namespace emi;
+
+extern "C" int emi_attn_fwd(emi_stream_t stream, const void* q, const void* k, const void* v, void* o, float* lse,
+                            int64_t batch, int64_t heads, int64_t seq, int64_t head_dim, int64_t stride_b,
+                            int64_t stride_h, int64_t stride_s, float scale, int causal, int dtype) {
+  const AttnArgs a{batch, heads, seq, head_dim, stride_b, stride_h, stride_s};
+  if (int rc = check_common("emi_attn_fwd", a, dtype)) return rc;
+  if (batch == 0) return EMI_OK;
+  EMI_REQUIRE(q && k && v && o && lse, "emi_attn_fwd: null buffer");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const AttnShape shp{(int)seq, (int)heads, stride_b, stride_h, stride_s};
+  const unsigned bh = (unsigned)(batch * heads);
+  if (mfma_ok(a, dtype, {q, k, v, o})) {
+    const uint32_t head_bytes = (uint32_t)(((seq - 1) * stride_s + head_dim) * 2);
+    const float sl2 = scale * kLog2e;
+    const dim3 grid((unsigned)((seq + 127) / 128), bh);
+    if (head_dim == 128) {
+      constexpr int smem = 2 * 2 * 64 * 128 * 2;
+      if (int rc = reserve_lds(attn_fwd_bf16_kernel<128>, smem, "emi_attn_fwd")) return rc;
+      hipLaunchKernelGGL(attn_fwd_bf16_kernel<128>, grid, dim3(256), smem, st, (const uint16_t*)q, (const uint16_t*)k,
+                         (const uint16_t*)v, (uint16_t*)o, lse, shp, head_bytes, sl2, causal);
+    } else {
+      constexpr int smem = 2 * 2 * 64 * 64 * 2;
+      if (int rc = reserve_lds(attn_fwd_bf16_kernel<64>, smem, "emi_attn_fwd")) return rc;
+      hipLaunchKernelGGL(attn_fwd_bf16_kernel<64>, grid, dim3(256), smem, st, (const uint16_t*)q, (const uint16_t*)k,
+                         (const uint16_t*)v, (uint16_t*)o, lse, shp, head_bytes, sl2, causal);
+    }
+    EMI_CHECK_LAUNCH("emi_attn_fwd");
+    return EMI_OK;
+  }
+  const dim3 grid((unsigned)((seq + 3) / 4), bh);
+  if (dtype == EMI_BF16)
+    hipLaunchKernelGGL(attn_fwd_generic_kernel<bf16>, grid, dim3(256), 0, st, (const bf16*)q, (const bf16*)k,
+                       (const bf16*)v, (bf16*)o, lse, shp, (int)head_dim, scale, causal);
+  else
+    hipLaunchKernelGGL(attn_fwd_generic_kernel<float>, grid, dim3(256), 0, st, (const float*)q, (const float*)k,
+                       (const float*)v, (float*)o, lse, shp, (int)head_dim, scale, causal);
+  EMI_CHECK_LAUNCH("emi_attn_fwd(generic)");
+  return EMI_OK;
+}
+
+extern "C" size_t emi_attn_bwd_workspace_bytes(int64_t batch, int64_t heads, int64_t seq, int64_t head_dim) {
+  (void)head_dim;
+  if (batch <= 0 || heads <= 0 || seq <= 0) return 0;
+  return (size_t)batch * (size_t)heads * (size_t)seq * sizeof(float);   // delta = rowsum(dO * O)
+}
+
+extern "C" int emi_attn_bwd(emi_stream_t stream, const void* q, const void* k, const void* v, const void* o,
+                            const float* lse, const void* d_o, void* dq, void* dk, void* dv, void* workspace,
+                            size_t workspace_bytes, int64_t batch, int64_t heads, int64_t seq, int64_t head_dim,
+                            int64_t stride_b, int64_t stride_h, int64_t stride_s, float scale, int causal, int dtype) {
+  const AttnArgs a{batch, heads, seq, head_dim, stride_b, stride_h, stride_s};
+  if (int rc = check_common("emi_attn_bwd", a, dtype)) return rc;
+  if (batch == 0) return EMI_OK;
+  EMI_REQUIRE(q && k && v && o && lse && d_o && dq && dk && dv, "emi_attn_bwd: null buffer");
+  const size_t need = emi_attn_bwd_workspace_bytes(batch, heads, seq, head_dim);
+  EMI_REQUIRE(workspace != nullptr && workspace_bytes >= need, "emi_attn_bwd: workspace of %zu bytes needed, got %zu", need,
+              workspace_bytes);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const AttnShape shp{(int)seq, (int)heads, stride_b, stride_h, stride_s};
+  const unsigned bh = (unsigned)(batch * heads);
+  float* delta = static_cast<float*>(workspace);
+  const dim3 grid4((unsigned)((seq + 3) / 4), bh);
+  if (dtype == EMI_BF16)
+    hipLaunchKernelGGL(attn_delta_kernel<bf16>, grid4, dim3(256), 0, st, (const bf16*)o, (const bf16*)d_o, delta, shp,
+                       (int)head_dim);
+  else
+    hipLaunchKernelGGL(attn_delta_kernel<float>, grid4, dim3(256), 0, st, (const float*)o, (const float*)d_o, delta, shp,
+                       (int)head_dim);
+  EMI_CHECK_LAUNCH("emi_attn_bwd(delta)");
+  if (mfma_ok(a, dtype, {q, k, v, d_o, dq, dk, dv})) {
+    const uint32_t head_bytes = (uint32_t)(((seq - 1) * stride_s + head_dim) * 2);
+    const dim3 grid((unsigned)((seq + 127) / 128), bh);
+    if (head_dim == 128) {
+      constexpr int smem_q = 2 * 2 * 64 * 128 * 2, smem_kv = 2 * (2 * 64 * 128 * 2 + 2 * 64 * 4);
+      if (int rc = reserve_lds(attn_bwd_dq_bf16_kernel<128>, smem_q, "emi_attn_bwd")) return rc;
+      if (int rc = reserve_lds(attn_bwd_dkv_bf16_kernel<128>, smem_kv, "emi_attn_bwd")) return rc;
+      hipLaunchKernelGGL(attn_bwd_dkv_bf16_kernel<128>, grid, dim3(256), smem_kv, st, (const uint16_t*)q,
+                         (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, (uint16_t*)dk,
+                         (uint16_t*)dv, shp, head_bytes, scale, causal);
+      EMI_CHECK_LAUNCH("emi_attn_bwd(dkv)");
+      hipLaunchKernelGGL(attn_bwd_dq_bf16_kernel<128>, grid, dim3(256), smem_q, st, (const uint16_t*)q,
+                         (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, (uint16_t*)dq, shp,
+                         head_bytes, scale, causal);
+    } else {
+      constexpr int smem_q = 2 * 2 * 64 * 64 * 2, smem_kv = 2 * (2 * 64 * 64 * 2 + 2 * 64 * 4);
+      if (int rc = reserve_lds(attn_bwd_dq_bf16_kernel<64>, smem_q, "emi_attn_bwd")) return rc;
+      if (int rc = reserve_lds(attn_bwd_dkv_bf16_kernel<64>, smem_kv, "emi_attn_bwd")) return rc;
+      hipLaunchKernelGGL(attn_bwd_dkv_bf16_kernel<64>, grid, dim3(256), smem_kv, st, (const uint16_t*)q,
+                         (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, (uint16_t*)dk,
+                         (uint16_t*)dv, shp, head_bytes, scale, causal);
+      EMI_CHECK_LAUNCH("emi_attn_bwd(dkv)");
+      hipLaunchKernelGGL(attn_bwd_dq_bf16_kernel<64>, grid, dim3(256), smem_q, st, (const uint16_t*)q,
+                         (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, (uint16_t*)dq, shp,
+                         head_bytes, scale, causal);
+    }
+    EMI_CHECK_LAUNCH("emi_attn_bwd(dq)");
+    return EMI_OK;
+  }
+  if (dtype == EMI_BF16) {
+    hipLaunchKernelGGL(attn_bwd_dq_generic_kernel<bf16>, grid4, dim3(256), 0, st, (const bf16*)q, (const bf16*)k,
+                       (const bf16*)v, (const bf16*)d_o, lse, delta, (bf16*)dq, shp, (int)head_dim, scale, causal);
+    hipLaunchKernelGGL(attn_bwd_dkv_generic_kernel<bf16>, grid4, dim3(256), 0, st, (const bf16*)q, (const bf16*)k,
+                       (const bf16*)v, (const bf16*)d_o, lse, delta, (bf16*)dk, (bf16*)dv, shp, (int)head_dim, scale,
+                       causal);
+  } else {
+    hipLaunchKernelGGL(attn_bwd_dq_generic_kernel<float>, grid4, dim3(256), 0, st, (const float*)q, (const float*)k,
+                       (const float*)v, (const float*)d_o, lse, delta, (float*)dq, shp, (int)head_dim, scale, causal);
+    hipLaunchKernelGGL(attn_bwd_dkv_generic_kernel<float>, grid4, dim3(256), 0, st, (const float*)q, (const float*)k,
+                       (const float*)v, (const float*)d_o, lse, delta, (float*)dk, (float*)dv, shp, (int)head_dim, scale,
+                       causal);
+  }
+  EMI_CHECK_LAUNCH("emi_attn_bwd(generic)");
+  return EMI_OK;
+}

@@ -1,0 +1,657 @@
+// HBM-bound kernels of the llama path for gfx950: RMSNorm, RoPE, SwiGLU,
+// residual add, embedding gather / scatter-add; forward and adjoint.
+//
+// All of them stream 16-byte vectors per lane, keep a row in registers where a
+// reduction is needed, reduce across the 64-lane wavefront with DPP shuffles
+// and compute in fp32 whatever the storage type is.
+#include "emi_device.h"
+
+namespace emi {
+
+// ---------------------------------------------------------------------------
+// RMSNorm (test/llama.py:6-10): y = gamma * x * rsqrt(mean(x^2) + eps)
+// TPR threads cooperate on one row (64 = one wavefront per row, four rows per
+// 256-thread block; 256 = one block per row); each thread keeps up to NCH
+// chunks of 8 elements in registers so x is read from HBM exactly once.
+// ---------------------------------------------------------------------------
+
+template <int TPR> __device__ __forceinline__ void row_reduce2(float& a, float& b, float (*red)[4][2], int it) {
+  a = wave_sum(a);
+  b = wave_sum(b);
+  if constexpr (TPR == 256) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    float(*buf)[2] = red[it & 1];
+    if (lane == 0) {
+      buf[wave][0] = a;
+      buf[wave][1] = b;
+    }
+    __syncthreads();
+    a = buf[0][0] + buf[1][0] + buf[2][0] + buf[3][0];
+    b = buf[0][1] + buf[1][1] + buf[2][1] + buf[3][1];
+  }
+}
+
+template <typename T, int TPR, int NCH>
+__global__ __launch_bounds__(256) void rmsnorm_fwd_kernel(const T* __restrict__ x, const T* __restrict__ gamma,
+                                                          T* __restrict__ y, int64_t rows, int dim, float eps) {
+  constexpr int RPB = 256 / TPR;
+  __shared__ float red[2][4][2];
+  const int tir = threadIdx.x % TPR;
+  const int rib = threadIdx.x / TPR;
+  const int64_t row = (int64_t)blockIdx.x * RPB + rib;
+  const bool active = row < rows;
+  const int nchunk = dim >> 3;
+  const T* xr = x + row * dim;
+  float v[NCH][8];
+  float ss = 0.f, dummy = 0.f;
+#pragma unroll
+  for (int j = 0; j < NCH; j++) {
+    const int c = tir + j * TPR;
+    if (active && c < nchunk) {
+      Vec8<T>::load(xr + c * 8, v[j]);
+#pragma unroll
+      for (int e = 0; e < 8; e++) ss += v[j][e] * v[j][e];
+    }
+  }
+  row_reduce2<TPR>(ss, dummy, red, 0);
+  const float r = 1.0f / sqrtf(ss / (float)dim + eps);
+  T* yr = y + row * dim;
+#pragma unroll
+  for (int j = 0; j < NCH; j++) {
+    const int c = tir + j * TPR;
+    if (active && c < nchunk) {
+      float g[8], o[8];
+      Vec8<T>::load(gamma + c * 8, g);
+#pragma unroll
+      for (int e = 0; e < 8; e++) o[e] = g[e] * v[j][e] * r;
+      Vec8<T>::store(yr + c * 8, o);
+    }
+  }
+}
+
+// Adjoint.  Blocks walk rows with a grid stride and keep this thread's share
+// of dgamma in registers; partial[blockIdx*RPB + rib][dim] is reduced by
+// colsum_kernel.  dx = [dx_add +] r*g - x * r^3 * mean(g*x), g = dy*gamma.
+template <typename T, int TPR, int NCH>
+__global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const T* __restrict__ x, const T* __restrict__ gamma,
+                                                          const T* __restrict__ dy, const T* dx_add, T* dx,
+                                                          float* __restrict__ partial, int64_t rows, int dim,
+                                                          float eps) {
+  constexpr int RPB = 256 / TPR;
+  __shared__ float red[2][4][2];
+  const int tir = threadIdx.x % TPR;
+  const int rib = threadIdx.x / TPR;
+  const int nchunk = dim >> 3;
+  float gm[NCH][8], acc[NCH][8];
+#pragma unroll
+  for (int j = 0; j < NCH; j++) {
+    const int c = tir + j * TPR;
+#pragma unroll
+    for (int e = 0; e < 8; e++) acc[j][e] = 0.f, gm[j][e] = 0.f;
+    if (c < nchunk) Vec8<T>::load(gamma + c * 8, gm[j]);
+  }
+  const int64_t nrow_iter = (rows + RPB - 1) / RPB;   // row groups
+  int it = 0;
+  for (int64_t rg = blockIdx.x; rg < nrow_iter; rg += gridDim.x, ++it) {
+    const int64_t row = rg * RPB + rib;
+    const bool active = row < rows;
+    float xv[NCH][8], gv[NCH][8];
+    float ss = 0.f, gx = 0.f;
+#pragma unroll
+    for (int j = 0; j < NCH; j++) {
+      const int c = tir + j * TPR;
+      if (active && c < nchunk) {
+        Vec8<T>::load(x + row * dim + c * 8, xv[j]);
+        Vec8<T>::load(dy + row * dim + c * 8, gv[j]);
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+          ss += xv[j][e] * xv[j][e];
+          gx += gv[j][e] * gm[j][e] * xv[j][e];
+        }
+      }
+    }
+    row_reduce2<TPR>(ss, gx, red, it);
+    const float r = 1.0f / sqrtf(ss / (float)dim + eps);
+    const float coef = r * r * r * (gx / (float)dim);
+#pragma unroll
+    for (int j = 0; j < NCH; j++) {
+      const int c = tir + j * TPR;
+      if (active && c < nchunk) {
+        float o[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+          acc[j][e] += gv[j][e] * xv[j][e] * r;
+          o[e] = r * gv[j][e] * gm[j][e] - xv[j][e] * coef;
+        }
+        if (dx_add != nullptr) {
+          float a[8];
+          Vec8<T>::load(dx_add + row * dim + c * 8, a);
+#pragma unroll
+          for (int e = 0; e < 8; e++) o[e] += a[e];
+        }
+        Vec8<T>::store(dx + row * dim + c * 8, o);
+      }
+    }
+  }
+  float* prow = partial + ((int64_t)blockIdx.x * RPB + rib) * dim;
+#pragma unroll
+  for (int j = 0; j < NCH; j++) {
+    const int c = tir + j * TPR;
+    if (c < nchunk) Vec8<float>::store(prow + c * 8, acc[j]);
+  }
+}
+
+// Any dim (not a multiple of 8, or beyond the register budget): one block per
+// row group, scalar accesses, x re-read from cache.
+template <typename T>
+__global__ __launch_bounds__(256) void rmsnorm_fwd_generic_kernel(const T* __restrict__ x, const T* __restrict__ gamma,
+                                                                  T* __restrict__ y, int64_t rows, int64_t dim,
+                                                                  float eps) {
+  __shared__ float red[2][4][2];
+  const int64_t row = blockIdx.x;
+  const T* xr = x + row * dim;
+  float ss = 0.f, dummy = 0.f;
+  for (int64_t c = threadIdx.x; c < dim; c += 256) {
+    const float v = to_f32(xr[c]);
+    ss += v * v;
+  }
+  row_reduce2<256>(ss, dummy, red, 0);
+  const float r = 1.0f / sqrtf(ss / (float)dim + eps);
+  for (int64_t c = threadIdx.x; c < dim; c += 256) y[row * dim + c] = from_f32<T>(to_f32(gamma[c]) * to_f32(xr[c]) * r);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void rmsnorm_bwd_generic_kernel(const T* __restrict__ x, const T* __restrict__ gamma,
+                                                                  const T* __restrict__ dy, const T* dx_add, T* dx,
+                                                                  float* __restrict__ partial, int64_t rows,
+                                                                  int64_t dim, float eps) {
+  __shared__ float red[2][4][2];
+  float* prow = partial + (int64_t)blockIdx.x * dim;
+  for (int64_t c = threadIdx.x; c < dim; c += 256) prow[c] = 0.f;
+  int it = 0;
+  for (int64_t row = blockIdx.x; row < rows; row += gridDim.x, ++it) {
+    float ss = 0.f, gx = 0.f;
+    for (int64_t c = threadIdx.x; c < dim; c += 256) {
+      const float xv = to_f32(x[row * dim + c]);
+      ss += xv * xv;
+      gx += to_f32(dy[row * dim + c]) * to_f32(gamma[c]) * xv;
+    }
+    row_reduce2<256>(ss, gx, red, it);
+    const float r = 1.0f / sqrtf(ss / (float)dim + eps);
+    const float coef = r * r * r * (gx / (float)dim);
+    for (int64_t c = threadIdx.x; c < dim; c += 256) {
+      const float xv = to_f32(x[row * dim + c]);
+      const float gv = to_f32(dy[row * dim + c]);
+      prow[c] += gv * xv * r;   // this thread owns column c of this block's partial row
+      float o = r * gv * to_f32(gamma[c]) - xv * coef;
+      if (dx_add != nullptr) o += to_f32(dx_add[row * dim + c]);
+      dx[row * dim + c] = from_f32<T>(o);
+    }
+  }
+}
+
+// out[c] = sum_p partial[p][c]; 32 columns x 8 row groups per block.
+template <typename T>
+__global__ __launch_bounds__(256) void colsum_kernel(const float* __restrict__ partial, int nparts, int64_t dim,
+                                                     T* __restrict__ out) {
+  __shared__ float red[8][33];
+  const int cg = threadIdx.x & 31, rg = threadIdx.x >> 5;
+  const int64_t col = (int64_t)blockIdx.x * 32 + cg;
+  float s = 0.f;
+  if (col < dim)
+    for (int p = rg; p < nparts; p += 8) s += partial[(int64_t)p * dim + col];
+  red[rg][cg] = s;
+  __syncthreads();
+  if (rg == 0 && col < dim) {
+    float t = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; i++) t += red[i][cg];
+    out[col] = from_f32<T>(t);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// RoPE (test/llama.py:127-140,161-168): adjacent pairs, angle table in fp32.
+// ---------------------------------------------------------------------------
+
+__global__ void rope_table_kernel(float2* __restrict__ table, int64_t seq, int half, int head_dim, double theta,
+                                  int64_t pos0) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= seq * half) return;
+  const int64_t s = i / half;
+  const int j = (int)(i % half);
+  const double freq = 1.0 / pow(theta, (double)(2 * j) / (double)head_dim);
+  const double ang = (double)(pos0 + s) * freq;
+  table[i] = make_float2((float)cos(ang), (float)sin(ang));
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void rope_kernel(const T* x, const float2* __restrict__ table, T* y, int64_t nchunks,
+                                                   int seq, int row_elems, int head_dim, int inverse) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= nchunks) return;
+  const int64_t e = i * 8;
+  const int in_head = (int)(e % head_dim);
+  const int s = (int)((e / row_elems) % seq);
+  const float4* tp = reinterpret_cast<const float4*>(table + (int64_t)s * (head_dim >> 1) + (in_head >> 1));
+  const float4 t0 = tp[0], t1 = tp[1];
+  const float cs[4] = {t0.x, t0.z, t1.x, t1.z};
+  float sn[4] = {t0.y, t0.w, t1.y, t1.w};
+  float v[8], o[8];
+  Vec8<T>::load(x + e, v);
+#pragma unroll
+  for (int p = 0; p < 4; p++) {
+    const float sp = inverse ? -sn[p] : sn[p];
+    o[2 * p] = cs[p] * v[2 * p] - sp * v[2 * p + 1];
+    o[2 * p + 1] = sp * v[2 * p] + cs[p] * v[2 * p + 1];
+  }
+  Vec8<T>::store(y + e, o);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void rope_pair_kernel(const T* x, const float2* __restrict__ table, T* y,
+                                                        int64_t npairs, int seq, int row_elems, int head_dim,
+                                                        int inverse) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= npairs) return;
+  const int64_t e = i * 2;
+  const int in_head = (int)(e % head_dim);
+  const int s = (int)((e / row_elems) % seq);
+  const float2 t = table[(int64_t)s * (head_dim >> 1) + (in_head >> 1)];
+  const float sp = inverse ? -t.y : t.y;
+  const float v0 = to_f32(x[e]), v1 = to_f32(x[e + 1]);
+  y[e] = from_f32<T>(t.x * v0 - sp * v1);
+  y[e + 1] = from_f32<T>(sp * v0 + t.x * v1);
+}
+
+// ---------------------------------------------------------------------------
+// SwiGLU (test/llama.py:21-28,229-231) and elementwise add
+// ---------------------------------------------------------------------------
+
+__device__ __forceinline__ float sigmoidf(float a) { return 1.0f / (1.0f + expf(-a)); }
+
+template <typename T>
+__global__ __launch_bounds__(256) void swiglu_fwd_kernel(const T* __restrict__ a, const T* __restrict__ b,
+                                                         T* __restrict__ g, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t nchunks = n >> 3;
+  if (i < nchunks) {
+    float av[8], bv[8], o[8];
+    Vec8<T>::load(a + i * 8, av);
+    Vec8<T>::load(b + i * 8, bv);
+#pragma unroll
+    for (int e = 0; e < 8; e++) o[e] = av[e] * sigmoidf(av[e]) * bv[e];
+    Vec8<T>::store(g + i * 8, o);
+  } else if (i - nchunks < (n & 7)) {
+    const int64_t e = (nchunks << 3) + (i - nchunks);
+    const float av = to_f32(a[e]);
+    g[e] = from_f32<T>(av * sigmoidf(av) * to_f32(b[e]));
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void swiglu_bwd_kernel(const T* __restrict__ a, const T* __restrict__ b,
+                                                         const T* __restrict__ dg, T* __restrict__ da,
+                                                         T* __restrict__ db, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t nchunks = n >> 3;
+  if (i < nchunks) {
+    float av[8], bv[8], gv[8], oa[8], ob[8];
+    Vec8<T>::load(a + i * 8, av);
+    Vec8<T>::load(b + i * 8, bv);
+    Vec8<T>::load(dg + i * 8, gv);
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      const float s = sigmoidf(av[e]);
+      oa[e] = gv[e] * bv[e] * s * (1.0f + av[e] * (1.0f - s));
+      ob[e] = gv[e] * av[e] * s;
+    }
+    Vec8<T>::store(da + i * 8, oa);
+    Vec8<T>::store(db + i * 8, ob);
+  } else if (i - nchunks < (n & 7)) {
+    const int64_t e = (nchunks << 3) + (i - nchunks);
+    const float av = to_f32(a[e]), bv = to_f32(b[e]), gv = to_f32(dg[e]);
+    const float s = sigmoidf(av);
+    da[e] = from_f32<T>(gv * bv * s * (1.0f + av * (1.0f - s)));
+    db[e] = from_f32<T>(gv * av * s);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void add_kernel(const T* a, const T* b, T* y, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t nchunks = n >> 3;
+  if (i < nchunks) {
+    float av[8], bv[8];
+    Vec8<T>::load(a + i * 8, av);
+    Vec8<T>::load(b + i * 8, bv);
+#pragma unroll
+    for (int e = 0; e < 8; e++) av[e] += bv[e];
+    Vec8<T>::store(y + i * 8, av);
+  } else if (i - nchunks < (n & 7)) {
+    const int64_t e = (nchunks << 3) + (i - nchunks);
+    y[e] = from_f32<T>(to_f32(a[e]) + to_f32(b[e]));
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Embedding gather and scatter-add
+// ---------------------------------------------------------------------------
+
+template <typename T>
+__global__ __launch_bounds__(256) void embedding_fwd_kernel(const int32_t* __restrict__ tokens,
+                                                            const T* __restrict__ table, T* __restrict__ x,
+                                                            int64_t n_tokens, int64_t vocab, int64_t dim) {
+  const int64_t t = blockIdx.x;
+  int64_t tok = tokens[t];
+  tok = tok < 0 ? 0 : (tok >= vocab ? vocab - 1 : tok);   // clamp like XLA's gather
+  for (int64_t c = threadIdx.x; c < dim; c += 256) x[t * dim + c] = table[tok * dim + c];
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void embedding_bwd_kernel(const int32_t* __restrict__ tokens,
+                                                            const T* __restrict__ dx, float* __restrict__ acc,
+                                                            int64_t n_tokens, int64_t vocab, int64_t dim) {
+  const int64_t t = blockIdx.x;
+  int64_t tok = tokens[t];
+  if (tok < 0 || tok >= vocab) return;                     // out-of-range updates are dropped (scatter)
+  for (int64_t c = threadIdx.x; c < dim; c += 256) atomicAdd(acc + tok * dim + c, to_f32(dx[t * dim + c]));
+}
+
+__global__ __launch_bounds__(256) void fill_zero_kernel(float* p, int64_t n) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) p[i] = 0.f;
+}
+
+__global__ __launch_bounds__(256) void f32_to_bf16_kernel(const float* __restrict__ in, bf16* __restrict__ out,
+                                                          int64_t n) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256)
+    out[i] = from_f32<bf16>(in[i]);
+}
+
+// ---------------------------------------------------------------------------
+// launch helpers
+// ---------------------------------------------------------------------------
+
+static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+static inline unsigned blocks_for(int64_t n, int per) { return (unsigned)((n + per - 1) / per); }
+
+// grid used by the RMSNorm adjoint; the workspace holds one fp32 partial row
+// of dgamma per (block, row-in-block).
+static inline void rms_bwd_shape(int64_t rows, int64_t dim, int* tpr, int* nch, int64_t* grid, int64_t* nparts) {
+  if ((dim & 7) == 0 && dim <= 8192) {
+    const int64_t chunks = dim >> 3;
+    *tpr = chunks <= 128 ? 64 : 256;
+    const int64_t per = (chunks + *tpr - 1) / *tpr;
+    *nch = per <= 1 ? 1 : (per <= 2 ? 2 : 4);
+    const int rpb = 256 / *tpr;
+    const int64_t groups = (rows + rpb - 1) / rpb;
+    const int64_t cap = (*tpr == 64) ? 512 : 2048;
+    *grid = groups < cap ? (groups > 0 ? groups : 1) : cap;
+    *nparts = *grid * rpb;
+  } else {
+    *tpr = 0;
+    *nch = 0;
+    *grid = rows < 1024 ? (rows > 0 ? rows : 1) : 1024;
+    *nparts = *grid;
+  }
+}
+
+template <typename T>
+static int rmsnorm_fwd_launch(hipStream_t st, const void* x, const void* gamma, void* y, int64_t rows, int64_t dim,
+                              float eps) {
+  const T* xp = static_cast<const T*>(x);
+  const T* gp = static_cast<const T*>(gamma);
+  T* yp = static_cast<T*>(y);
+  int tpr, nch;
+  int64_t grid, nparts;
+  rms_bwd_shape(rows, dim, &tpr, &nch, &grid, &nparts);
+  if (tpr == 0) {
+    hipLaunchKernelGGL(rmsnorm_fwd_generic_kernel<T>, dim3((unsigned)rows), dim3(256), 0, st, xp, gp, yp, rows, dim, eps);
+  } else {
+    const unsigned g = blocks_for(rows, 256 / tpr);
+#define EMI_RMS_FWD(TPR, NCH) \
+  hipLaunchKernelGGL((rmsnorm_fwd_kernel<T, TPR, NCH>), dim3(g), dim3(256), 0, st, xp, gp, yp, rows, (int)dim, eps)
+    if (tpr == 64 && nch == 1) EMI_RMS_FWD(64, 1);
+    else if (tpr == 64) EMI_RMS_FWD(64, 2);
+    else if (nch == 1) EMI_RMS_FWD(256, 1);
+    else if (nch == 2) EMI_RMS_FWD(256, 2);
+    else EMI_RMS_FWD(256, 4);
+#undef EMI_RMS_FWD
+  }
+  EMI_CHECK_LAUNCH("emi_rmsnorm_fwd");
+  return EMI_OK;
+}
+
+template <typename T>
+static int rmsnorm_bwd_launch(hipStream_t st, const void* x, const void* gamma, const void* dy, const void* dx_add,
+                              void* dx, void* dgamma, void* ws, int64_t rows, int64_t dim, float eps) {
+  const T* xp = static_cast<const T*>(x);
+  const T* gp = static_cast<const T*>(gamma);
+  const T* dyp = static_cast<const T*>(dy);
+  const T* ap = static_cast<const T*>(dx_add);
+  T* dxp = static_cast<T*>(dx);
+  float* part = static_cast<float*>(ws);
+  int tpr, nch;
+  int64_t grid, nparts;
+  rms_bwd_shape(rows, dim, &tpr, &nch, &grid, &nparts);
+  if (tpr == 0) {
+    hipLaunchKernelGGL(rmsnorm_bwd_generic_kernel<T>, dim3((unsigned)grid), dim3(256), 0, st, xp, gp, dyp, ap, dxp, part,
+                       rows, dim, eps);
+  } else {
+#define EMI_RMS_BWD(TPR, NCH)                                                                                   \
+  hipLaunchKernelGGL((rmsnorm_bwd_kernel<T, TPR, NCH>), dim3((unsigned)grid), dim3(256), 0, st, xp, gp, dyp, ap, dxp, \
+                     part, rows, (int)dim, eps)
+    if (tpr == 64 && nch == 1) EMI_RMS_BWD(64, 1);
+    else if (tpr == 64) EMI_RMS_BWD(64, 2);
+    else if (nch == 1) EMI_RMS_BWD(256, 1);
+    else if (nch == 2) EMI_RMS_BWD(256, 2);
+    else EMI_RMS_BWD(256, 4);
+#undef EMI_RMS_BWD
+  }
+  EMI_CHECK_LAUNCH("emi_rmsnorm_bwd");
+  hipLaunchKernelGGL(colsum_kernel<T>, dim3(blocks_for(dim, 32)), dim3(256), 0, st, part, (int)nparts, dim,
+                     static_cast<T*>(dgamma));
+  EMI_CHECK_LAUNCH("emi_rmsnorm_bwd(colsum)");
+  return EMI_OK;
+}
+
+}  // namespace emi
+
+using namespace emi;
+
+#define EMI_DISPATCH_DTYPE(name, dtype, call_f32, call_bf16)                           \
+  switch (dtype) {                                                                     \
+    case EMI_F32: return call_f32;                                                     \
+    case EMI_BF16: return call_bf16;                                                   \
+    default: return emi_fail(EMI_INVALID_ARGUMENT, "%s: unsupported dtype code %d (want 11=f32 or 16=bf16)", name, dtype); \
+  }
+
+extern "C" int emi_rmsnorm_fwd(emi_stream_t stream, const void* x, const void* gamma, void* y, int64_t rows,
+                               int64_t dim, float eps, int dtype) {
+  EMI_REQUIRE(rows >= 0 && dim > 0, "emi_rmsnorm_fwd: bad shape rows=%lld dim=%lld", (long long)rows, (long long)dim);
+  EMI_REQUIRE(rows <= 0x7fffffffLL * 4, "emi_rmsnorm_fwd: rows=%lld too large", (long long)rows);
+  if (rows == 0) return EMI_OK;
+  EMI_REQUIRE(x && gamma && y, "emi_rmsnorm_fwd: null buffer");
+  EMI_REQUIRE(aligned16(x) && aligned16(gamma) && aligned16(y), "emi_rmsnorm_fwd: buffers must be 16-byte aligned");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  EMI_DISPATCH_DTYPE("emi_rmsnorm_fwd", dtype, rmsnorm_fwd_launch<float>(st, x, gamma, y, rows, dim, eps),
+                     rmsnorm_fwd_launch<bf16>(st, x, gamma, y, rows, dim, eps));
+}
+
+extern "C" size_t emi_rmsnorm_bwd_workspace_bytes(int64_t rows, int64_t dim) {
+  if (rows <= 0 || dim <= 0) return 0;
+  int tpr, nch;
+  int64_t grid, nparts;
+  rms_bwd_shape(rows, dim, &tpr, &nch, &grid, &nparts);
+  return (size_t)nparts * (size_t)dim * sizeof(float);
+}
+
+extern "C" int emi_rmsnorm_bwd(emi_stream_t stream, const void* x, const void* gamma, const void* dy,
+                               const void* dx_add, void* dx, void* dgamma, void* workspace, size_t workspace_bytes,
+                               int64_t rows, int64_t dim, float eps, int dtype) {
+  EMI_REQUIRE(rows > 0 && dim > 0, "emi_rmsnorm_bwd: bad shape rows=%lld dim=%lld", (long long)rows, (long long)dim);
+  EMI_REQUIRE(x && gamma && dy && dx && dgamma, "emi_rmsnorm_bwd: null buffer");
+  EMI_REQUIRE(aligned16(x) && aligned16(gamma) && aligned16(dy) && aligned16(dx) && aligned16(dx_add) &&
+                  aligned16(workspace),
+              "emi_rmsnorm_bwd: buffers must be 16-byte aligned");
+  const size_t need = emi_rmsnorm_bwd_workspace_bytes(rows, dim);
+  EMI_REQUIRE(workspace != nullptr && workspace_bytes >= need, "emi_rmsnorm_bwd: workspace of %zu bytes needed, got %zu",
+              need, workspace_bytes);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  EMI_DISPATCH_DTYPE("emi_rmsnorm_bwd", dtype,
+                     rmsnorm_bwd_launch<float>(st, x, gamma, dy, dx_add, dx, dgamma, workspace, rows, dim, eps),
+                     rmsnorm_bwd_launch<bf16>(st, x, gamma, dy, dx_add, dx, dgamma, workspace, rows, dim, eps));
+}
+
+extern "C" int emi_rope_table(emi_stream_t stream, float* table, int64_t seq, int64_t head_dim, double theta,
+                              int64_t pos0) {
+  EMI_REQUIRE(seq > 0 && head_dim > 0 && (head_dim & 1) == 0, "emi_rope_table: bad shape seq=%lld head_dim=%lld",
+              (long long)seq, (long long)head_dim);
+  EMI_REQUIRE(table != nullptr && aligned16(table), "emi_rope_table: table must be a 16-byte aligned device buffer");
+  EMI_REQUIRE(theta > 0.0, "emi_rope_table: theta must be positive");
+  const int half = (int)(head_dim / 2);
+  hipLaunchKernelGGL(rope_table_kernel, dim3(blocks_for(seq * half, 256)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     reinterpret_cast<float2*>(table), seq, half, (int)head_dim, theta, pos0);
+  EMI_CHECK_LAUNCH("emi_rope_table");
+  return EMI_OK;
+}
+
+template <typename T>
+static int rope_launch(hipStream_t st, const void* x, const float* table, void* y, int64_t batch, int64_t seq,
+                       int64_t heads, int64_t head_dim, int inverse) {
+  const int64_t n = batch * seq * heads * head_dim;
+  const float2* tp = reinterpret_cast<const float2*>(table);
+  if ((head_dim & 7) == 0) {
+    hipLaunchKernelGGL(rope_kernel<T>, dim3(blocks_for(n / 8, 256)), dim3(256), 0, st, static_cast<const T*>(x), tp,
+                       static_cast<T*>(y), n / 8, (int)seq, (int)(heads * head_dim), (int)head_dim, inverse);
+  } else {
+    hipLaunchKernelGGL(rope_pair_kernel<T>, dim3(blocks_for(n / 2, 256)), dim3(256), 0, st, static_cast<const T*>(x), tp,
+                       static_cast<T*>(y), n / 2, (int)seq, (int)(heads * head_dim), (int)head_dim, inverse);
+  }
+  EMI_CHECK_LAUNCH("emi_rope");
+  return EMI_OK;
+}
+
+extern "C" int emi_rope(emi_stream_t stream, const void* x, const float* table, void* y, int64_t batch, int64_t seq,
+                        int64_t heads, int64_t head_dim, int inverse, int dtype) {
+  EMI_REQUIRE(batch >= 0 && seq > 0 && heads > 0 && head_dim > 0 && (head_dim & 1) == 0,
+              "emi_rope: bad shape [%lld,%lld,%lld,%lld] (head_dim must be even)", (long long)batch, (long long)seq,
+              (long long)heads, (long long)head_dim);
+  EMI_REQUIRE(heads * head_dim <= 0x7fffffff && seq <= 0x7fffffff, "emi_rope: row too large");
+  if (batch == 0) return EMI_OK;
+  EMI_REQUIRE(x && y && table, "emi_rope: null buffer");
+  EMI_REQUIRE(aligned16(x) && aligned16(y) && aligned16(table), "emi_rope: buffers must be 16-byte aligned");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  EMI_DISPATCH_DTYPE("emi_rope", dtype, rope_launch<float>(st, x, table, y, batch, seq, heads, head_dim, inverse),
+                     rope_launch<bf16>(st, x, table, y, batch, seq, heads, head_dim, inverse));
+}
+
+template <typename T>
+static int swiglu_fwd_launch(hipStream_t st, const void* a, const void* b, void* g, int64_t n) {
+  hipLaunchKernelGGL(swiglu_fwd_kernel<T>, dim3(blocks_for((n >> 3) + (n & 7), 256)), dim3(256), 0, st,
+                     static_cast<const T*>(a), static_cast<const T*>(b), static_cast<T*>(g), n);
+  EMI_CHECK_LAUNCH("emi_swiglu_fwd");
+  return EMI_OK;
+}
+template <typename T>
+static int swiglu_bwd_launch(hipStream_t st, const void* a, const void* b, const void* dg, void* da, void* db,
+                             int64_t n) {
+  hipLaunchKernelGGL(swiglu_bwd_kernel<T>, dim3(blocks_for((n >> 3) + (n & 7), 256)), dim3(256), 0, st,
+                     static_cast<const T*>(a), static_cast<const T*>(b), static_cast<const T*>(dg), static_cast<T*>(da),
+                     static_cast<T*>(db), n);
+  EMI_CHECK_LAUNCH("emi_swiglu_bwd");
+  return EMI_OK;
+}
+template <typename T> static int add_launch(hipStream_t st, const void* a, const void* b, void* y, int64_t n) {
+  hipLaunchKernelGGL(add_kernel<T>, dim3(blocks_for((n >> 3) + (n & 7), 256)), dim3(256), 0, st, static_cast<const T*>(a),
+                     static_cast<const T*>(b), static_cast<T*>(y), n);
+  EMI_CHECK_LAUNCH("emi_add");
+  return EMI_OK;
+}
+
+extern "C" int emi_swiglu_fwd(emi_stream_t stream, const void* a, const void* b, void* g, int64_t n, int dtype) {
+  EMI_REQUIRE(n >= 0, "emi_swiglu_fwd: negative size");
+  if (n == 0) return EMI_OK;
+  EMI_REQUIRE(a && b && g, "emi_swiglu_fwd: null buffer");
+  EMI_REQUIRE(aligned16(a) && aligned16(b) && aligned16(g), "emi_swiglu_fwd: buffers must be 16-byte aligned");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  EMI_DISPATCH_DTYPE("emi_swiglu_fwd", dtype, swiglu_fwd_launch<float>(st, a, b, g, n),
+                     swiglu_fwd_launch<bf16>(st, a, b, g, n));
+}
+
+extern "C" int emi_swiglu_bwd(emi_stream_t stream, const void* a, const void* b, const void* dg, void* da, void* db,
+                              int64_t n, int dtype) {
+  EMI_REQUIRE(n >= 0, "emi_swiglu_bwd: negative size");
+  if (n == 0) return EMI_OK;
+  EMI_REQUIRE(a && b && dg && da && db, "emi_swiglu_bwd: null buffer");
+  EMI_REQUIRE(aligned16(a) && aligned16(b) && aligned16(dg) && aligned16(da) && aligned16(db),
+              "emi_swiglu_bwd: buffers must be 16-byte aligned");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  EMI_DISPATCH_DTYPE("emi_swiglu_bwd", dtype, swiglu_bwd_launch<float>(st, a, b, dg, da, db, n),
+                     swiglu_bwd_launch<bf16>(st, a, b, dg, da, db, n));
+}
+
+extern "C" int emi_add(emi_stream_t stream, const void* a, const void* b, void* y, int64_t n, int dtype) {
+  EMI_REQUIRE(n >= 0, "emi_add: negative size");
+  if (n == 0) return EMI_OK;
+  EMI_REQUIRE(a && b && y, "emi_add: null buffer");
+  EMI_REQUIRE(aligned16(a) && aligned16(b) && aligned16(y), "emi_add: buffers must be 16-byte aligned");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  EMI_DISPATCH_DTYPE("emi_add", dtype, add_launch<float>(st, a, b, y, n), add_launch<bf16>(st, a, b, y, n));
+}
+
+template <typename T>
+static int embedding_fwd_launch(hipStream_t st, const int32_t* tokens, const void* table, void* x, int64_t n_tokens,
+                                int64_t vocab, int64_t dim) {
+  hipLaunchKernelGGL(embedding_fwd_kernel<T>, dim3((unsigned)n_tokens), dim3(256), 0, st, tokens,
+                     static_cast<const T*>(table), static_cast<T*>(x), n_tokens, vocab, dim);
+  EMI_CHECK_LAUNCH("emi_embedding_fwd");
+  return EMI_OK;
+}
+
+extern "C" int emi_embedding_fwd(emi_stream_t stream, const int32_t* tokens, const void* table, void* x,
+                                 int64_t n_tokens, int64_t vocab, int64_t dim, int dtype) {
+  EMI_REQUIRE(n_tokens >= 0 && vocab > 0 && dim > 0, "emi_embedding_fwd: bad shape");
+  EMI_REQUIRE(n_tokens <= 0x7fffffff, "emi_embedding_fwd: too many tokens");
+  if (n_tokens == 0) return EMI_OK;
+  EMI_REQUIRE(tokens && table && x, "emi_embedding_fwd: null buffer");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  EMI_DISPATCH_DTYPE("emi_embedding_fwd", dtype, embedding_fwd_launch<float>(st, tokens, table, x, n_tokens, vocab, dim),
+                     embedding_fwd_launch<bf16>(st, tokens, table, x, n_tokens, vocab, dim));
+}
+
+extern "C" size_t emi_embedding_bwd_workspace_bytes(int64_t vocab, int64_t dim, int dtype) {
+  if (vocab <= 0 || dim <= 0) return 0;
+  return dtype == EMI_BF16 ? (size_t)vocab * (size_t)dim * sizeof(float) : 0;
+}
+
+extern "C" int emi_embedding_bwd(emi_stream_t stream, const int32_t* tokens, const void* dx, void* dtable,
+                                 void* workspace, size_t workspace_bytes, int64_t n_tokens, int64_t vocab, int64_t dim,
+                                 int dtype) {
+  EMI_REQUIRE(n_tokens >= 0 && vocab > 0 && dim > 0, "emi_embedding_bwd: bad shape");
+  EMI_REQUIRE(n_tokens <= 0x7fffffff, "emi_embedding_bwd: too many tokens");
+  EMI_REQUIRE(dtable != nullptr && (n_tokens == 0 || (tokens && dx)), "emi_embedding_bwd: null buffer");
+  EMI_REQUIRE(dtype == EMI_F32 || dtype == EMI_BF16, "emi_embedding_bwd: unsupported dtype code %d", dtype);
+  const size_t need = emi_embedding_bwd_workspace_bytes(vocab, dim, dtype);
+  EMI_REQUIRE(need == 0 || (workspace != nullptr && workspace_bytes >= need),
+              "emi_embedding_bwd: workspace of %zu bytes needed, got %zu", need, workspace_bytes);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  float* acc = dtype == EMI_BF16 ? static_cast<float*>(workspace) : static_cast<float*>(dtable);
+  const int64_t total = vocab * dim;
+  hipLaunchKernelGGL(fill_zero_kernel, dim3(2048), dim3(256), 0, st, acc, total);
+  EMI_CHECK_LAUNCH("emi_embedding_bwd(zero)");
+  if (n_tokens > 0) {
+    if (dtype == EMI_BF16)
+      hipLaunchKernelGGL(embedding_bwd_kernel<bf16>, dim3((unsigned)n_tokens), dim3(256), 0, st, tokens,
+                         static_cast<const bf16*>(dx), acc, n_tokens, vocab, dim);
+    else
+      hipLaunchKernelGGL(embedding_bwd_kernel<float>, dim3((unsigned)n_tokens), dim3(256), 0, st, tokens,
+                         static_cast<const float*>(dx), acc, n_tokens, vocab, dim);
+    EMI_CHECK_LAUNCH("emi_embedding_bwd");
+  }
+  if (dtype == EMI_BF16) {
+    hipLaunchKernelGGL(f32_to_bf16_kernel, dim3(2048), dim3(256), 0, st, acc, static_cast<bf16*>(dtable), total);
+    EMI_CHECK_LAUNCH("emi_embedding_bwd(convert)");
+  }
+  return EMI_OK;
+}

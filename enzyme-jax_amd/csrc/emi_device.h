@@ -1,0 +1,97 @@
+// Device-side helpers shared by the gfx950 kernels: bf16 <-> fp32, 16-byte
+// vector access, 64-lane wavefront reductions.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/emi.h"
+
+namespace emi {
+
+constexpr int kWave = 64;
+
+struct bf16 {
+  uint16_t bits;
+};
+
+__device__ __forceinline__ float to_f32(float v) { return v; }
+__device__ __forceinline__ float to_f32(bf16 v) { return __uint_as_float(((uint32_t)v.bits) << 16); }
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) { return __uint_as_float(((uint32_t)b) << 16); }
+
+// fp32 -> bf16, round to nearest even (v_cvt_pk_bf16_f32 on gfx950).
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+  __bf16 b = (__bf16)f;
+  return __builtin_bit_cast(uint16_t, b);
+}
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_t;
+  typedef __attribute__((__vector_size__(2 * sizeof(float)))) float f32x2_t;
+  f32x2_t v = {lo, hi};
+  bf16x2_t r = __builtin_convertvector(v, bf16x2_t);
+  return __builtin_bit_cast(uint32_t, r);
+}
+
+template <typename T> __device__ __forceinline__ T from_f32(float f);
+template <> __device__ __forceinline__ float from_f32<float>(float f) { return f; }
+template <> __device__ __forceinline__ bf16 from_f32<bf16>(float f) { return bf16{f32_to_bf16_bits(f)}; }
+
+// Eight consecutive elements as fp32 (one 16-byte load for bf16, two for fp32).
+template <typename T> struct Vec8;
+template <> struct Vec8<float> {
+  static __device__ __forceinline__ void load(const float* p, float (&v)[8]) {
+    float4 a = *reinterpret_cast<const float4*>(p);
+    float4 b = *reinterpret_cast<const float4*>(p + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+    v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+  }
+  static __device__ __forceinline__ void store(float* p, const float (&v)[8]) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+    *reinterpret_cast<float4*>(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
+  }
+};
+template <> struct Vec8<bf16> {
+  static __device__ __forceinline__ void load(const bf16* p, float (&v)[8]) {
+    uint4 a = *reinterpret_cast<const uint4*>(p);
+    uint32_t w[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      v[2 * i] = __uint_as_float(w[i] << 16);
+      v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+  }
+  static __device__ __forceinline__ void store(bf16* p, const float (&v)[8]) {
+    uint4 a;
+    a.x = pack_bf16x2(v[0], v[1]);
+    a.y = pack_bf16x2(v[2], v[3]);
+    a.z = pack_bf16x2(v[4], v[5]);
+    a.w = pack_bf16x2(v[6], v[7]);
+    *reinterpret_cast<uint4*>(p) = a;
+  }
+};
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
+  return v;
+}
+
+}  // namespace emi
+
+// Host-side error plumbing (defined in status.cc).
+extern "C" int emi_fail(int code, const char* fmt, ...);
+
+#define EMI_REQUIRE(cond, ...)                                   \
+  do {                                                           \
+    if (!(cond)) return emi_fail(EMI_INVALID_ARGUMENT, __VA_ARGS__); \
+  } while (0)
+
+#define EMI_CHECK_LAUNCH(name)                                                        \
+  do {                                                                                \
+    hipError_t e__ = hipGetLastError();                                               \
+    if (e__ != hipSuccess) return emi_fail(EMI_INTERNAL, "%s: launch failed: %s", name, hipGetErrorString(e__)); \
+  } while (0)

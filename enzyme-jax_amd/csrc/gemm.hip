@@ -1,0 +1,373 @@
+// GEMM for the llama projections, FFN and their adjoints on gfx950 MFMA.
+//
+//   C[M,N] = op(A) . op(B) [+ R]      fp32 accumulate, one rounding at the end
+//
+// Fast path (bf16): v_mfma_f32_32x32x16_bf16, block tile BM x BN x 64, operands
+// streamed HBM -> LDS with 16-byte direct-to-LDS buffer loads (no VGPR
+// staging; out-of-range chunks read as zero), two LDS stages, XOR-swizzled so
+// both the k-contiguous reads (ds_read_b128) and the k-major reads
+// (ds_read_b64_tr_b16, the transposing LDS load) are bank-conflict free.
+// One kernel template covers the three operand layouts of the path:
+//   NT  Y  = X . W^T    (A k-contiguous, B k-contiguous)   forward
+//   NN  dX = dY . W     (A k-contiguous, B k-major)        input adjoint
+//   TN  dW = dY^T . X   (A k-major,      B k-major)        weight adjoint
+// Generic path (fp32, or bf16 with shapes/alignments the fast path does not
+// take): v_mfma_f32_32x32x2_f32 with predicated scalar loads.
+#include "emi_device.h"
+
+namespace emi {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4_t;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
+
+#define EMI_LDS __attribute__((address_space(3)))
+
+constexpr uint32_t kOob = 0x80000000u;   // beyond any buffer's num_records: loads return 0
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes, 0x00020000);
+}
+
+// XCD-aware tile order: consecutive workgroup ids land on different XCDs
+// (8 of them, each with its own L2), so give every XCD a contiguous run of
+// tiles, and walk tiles in groups of GROUP_M tile-rows so that the A and B
+// panels a XCD touches stay in its L2.
+__device__ __forceinline__ void tile_coords(int tiles_m, int tiles_n, int* tm, int* tn) {
+  const int nb = gridDim.x, bid = blockIdx.x;
+  const int per = nb >> 3, rem = nb & 7;
+  const int xcd = bid & 7, idx = bid >> 3;
+  const int pid = xcd * per + (xcd < rem ? xcd : rem) + idx;
+  constexpr int GROUP_M = 8;
+  const int group_size = GROUP_M * tiles_n;
+  const int group = pid / group_size;
+  const int first_m = group * GROUP_M;
+  const int gm = (tiles_m - first_m) < GROUP_M ? (tiles_m - first_m) : GROUP_M;
+  const int in_group = pid - group * group_size;
+  *tm = first_m + in_group % gm;
+  *tn = in_group / gm;
+}
+
+// --- LDS tile layouts -------------------------------------------------------
+// k-contiguous operand tile: [rows][64 k] bf16, 128-byte rows, 16-byte chunk c
+// of row r stored at chunk c ^ (r & 7).
+// k-major operand tile: [64 k][COLS] bf16, chunk c of row k stored at chunk
+// c ^ (4 * (k & 3)).
+
+template <int ROWS, int NW>
+__device__ __forceinline__ void load_tile_kcontig(__amdgpu_buffer_rsrc_t rsrc, EMI_LDS uint8_t* lds, int wave, int lane,
+                                                  uint32_t row0_off_bytes, int ld, int k0, int K) {
+  constexpr int NLOAD = ROWS / 8 / NW;
+  const int r_in = lane >> 3, pc = lane & 7;
+  const int lc = pc ^ r_in;
+  const int k = k0 + lc * 8;
+#pragma unroll
+  for (int it = 0; it < NLOAD; it++) {
+    const int r = (it * NW + wave) * 8 + r_in;
+    uint32_t voff = row0_off_bytes + (uint32_t)(r * ld + k) * 2u;
+    if (k >= K) voff = kOob;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, lds + (it * NW + wave) * 1024, 16, voff, 0, 0, 0);
+  }
+}
+
+template <int COLS, int NW>
+__device__ __forceinline__ void load_tile_kmajor(__amdgpu_buffer_rsrc_t rsrc, EMI_LDS uint8_t* lds, int wave, int lane,
+                                                 int col0, int ncols, int ld, int k0, int K) {
+  constexpr int CPR = COLS / 8;              // 16-byte chunks per k-row
+  constexpr int NLOAD = CPR / NW;            // 64 rows * CPR chunks / (64 lanes * NW waves)
+  static_assert(CPR >= 16 && NLOAD >= 1, "k-major tile too narrow");
+#pragma unroll
+  for (int it = 0; it < NLOAD; it++) {
+    const int slot = (it * NW + wave) * 64 + lane;
+    const int k = slot / CPR, pc = slot % CPR;
+    const int lc = pc ^ (4 * (k & 3));
+    const int col = col0 + lc * 8;
+    uint32_t voff = (uint32_t)((k0 + k) * ld + col) * 2u;
+    if (k0 + k >= K || col >= ncols) voff = kOob;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, lds + (it * NW + wave) * 1024, 16, voff, 0, 0, 0);
+  }
+}
+
+// MFMA operand fragment (32 rows x 16 k) for k-step kk of the 64-k tile.
+// Lane l holds row (l & 31), k = 8*(l >> 5) + 0..7 of the step.
+__device__ __forceinline__ bf16x8_t frag_kcontig(const EMI_LDS uint8_t* tile, int row_base, int kk, int lane) {
+  const int row = row_base + (lane & 31);
+  const int chunk = (kk * 2 + (lane >> 5)) ^ (row & 7);
+  return *reinterpret_cast<const EMI_LDS bf16x8_t*>(tile + row * 128 + chunk * 16);
+}
+
+// Same fragment out of a k-major tile with two transposing loads.  Within a
+// 16-lane group, lane i supplies the address of k-row (i >> 2), columns
+// 4*(i & 3).. +3, and receives column (i), k-rows 0..3.
+template <int COLS>
+__device__ __forceinline__ bf16x8_t frag_kmajor(const EMI_LDS uint8_t* tile, int col_base, int kk, int lane) {
+  const int i = lane & 15;
+  const int kq = i >> 2;                                        // k & 3 of the row this lane addresses
+  const int col = col_base + ((lane >> 4) & 1) * 16 + (i & 3) * 4;
+  const int krow = kk * 16 + (lane >> 5) * 8 + kq;
+  const int chunk = (col >> 3) ^ (4 * kq);
+  const EMI_LDS uint8_t* p = tile + krow * (COLS * 2) + chunk * 16 + (col & 7) * 2;
+  bf16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((EMI_LDS bf16x4_t*)p);
+  bf16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((EMI_LDS bf16x4_t*)(p + 4 * COLS * 2));
+  return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+template <int BM, int BN, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR>
+__global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_kernel(const uint16_t* __restrict__ A,
+                                                                 const uint16_t* __restrict__ B, const uint16_t* R,
+                                                                 uint16_t* C, int M, int N, int K, int lda, int ldb,
+                                                                 int ldr, int ldc, uint32_t a_bytes, uint32_t b_bytes) {
+  constexpr int NW = WM * WN;
+  constexpr int BK = 64;
+  constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+  constexpr int A_BYTES = BM * BK * 2, B_BYTES = BN * BK * 2, STAGE = A_BYTES + B_BYTES;
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem_raw[];
+  EMI_LDS uint8_t* smem = (EMI_LDS uint8_t*)smem_raw;
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wm = wave / WN, wn = wave % WN;
+
+  const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+  int tile_m, tile_n;
+  tile_coords(tiles_m, tiles_n, &tile_m, &tile_n);
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+  const __amdgpu_buffer_rsrc_t rA = make_rsrc(A, a_bytes);
+  const __amdgpu_buffer_rsrc_t rB = make_rsrc(B, b_bytes);
+
+  auto issue_loads = [&](int stage, int k0) {
+    EMI_LDS uint8_t* sA = smem + stage * STAGE;
+    EMI_LDS uint8_t* sB = sA + A_BYTES;
+    if constexpr (A_KMAJOR)
+      load_tile_kmajor<BM, NW>(rA, sA, wave, lane, m0, M, lda, k0, K);
+    else
+      load_tile_kcontig<BM, NW>(rA, sA, wave, lane, (uint32_t)m0 * (uint32_t)lda * 2u, lda, k0, K);
+    if constexpr (B_KMAJOR)
+      load_tile_kmajor<BN, NW>(rB, sB, wave, lane, n0, N, ldb, k0, K);
+    else
+      load_tile_kcontig<BN, NW>(rB, sB, wave, lane, (uint32_t)n0 * (uint32_t)ldb * 2u, ldb, k0, K);
+  };
+
+  f32x16_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+  const int nk = (K + BK - 1) / BK;
+  issue_loads(0, 0);
+  __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0)
+  __syncthreads();
+
+  for (int t = 0; t < nk; t++) {
+    if (t + 1 < nk) issue_loads((t + 1) & 1, (t + 1) * BK);
+    const EMI_LDS uint8_t* sA = smem + (t & 1) * STAGE;
+    const EMI_LDS uint8_t* sB = sA + A_BYTES;
+#pragma unroll
+    for (int kk = 0; kk < 4; kk++) {
+      bf16x8_t a[TM], b[TN];
+#pragma unroll
+      for (int i = 0; i < TM; i++) {
+        const int base = wm * (BM / WM) + i * 32;
+        if constexpr (A_KMAJOR) a[i] = frag_kmajor<BM>(sA, base, kk, lane);
+        else a[i] = frag_kcontig(sA, base, kk, lane);
+      }
+#pragma unroll
+      for (int j = 0; j < TN; j++) {
+        const int base = wn * (BN / WN) + j * 32;
+        if constexpr (B_KMAJOR) b[j] = frag_kmajor<BN>(sB, base, kk, lane);
+        else b[j] = frag_kcontig(sB, base, kk, lane);
+      }
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+    __builtin_amdgcn_s_waitcnt(0x0f70);   // next stage has landed
+    __syncthreads();                      // and everyone is done reading this one
+  }
+
+  // Epilogue.  Accumulator register r of lane l is C[8*(r/4) + 4*(l/32) + r%4][l%32].
+  const int col_l = lane & 31, row_l = (lane >> 5) * 4;
+#pragma unroll
+  for (int i = 0; i < TM; i++) {
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+      const int col = n0 + wn * (BN / WN) + j * 32 + col_l;
+      if (col < N) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const int row = m0 + wm * (BM / WM) + i * 32 + (r >> 2) * 8 + row_l + (r & 3);
+          if (row < M) {
+            float v = acc[i][j][r];
+            if (R != nullptr) v += bf16_bits_to_f32(R[(int64_t)row * ldr + col]);
+            C[(int64_t)row * ldc + col] = f32_to_bf16_bits(v);
+          }
+        }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Generic path: any dtype/shape/alignment, fp32 MFMA (v_mfma_f32_32x32x2_f32).
+// 256 threads, 128x128x16 tile, LDS tiles stored k-major as fp32.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void gemm_generic_kernel(const T* __restrict__ A, const T* __restrict__ B, const T* R,
+                                                           T* C, int M, int N, int K, int64_t lda, int64_t ldb,
+                                                           int64_t ldr, int64_t ldc, int trans_a, int trans_b) {
+  constexpr int BM = 128, BN = 128, BK = 16, PAD = 4;
+  __shared__ float sA[BK][BM + PAD];
+  __shared__ float sB[BK][BN + PAD];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  f32x16_t acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+  for (int k0 = 0; k0 < K; k0 += BK) {
+    // A tile: 128 x 16 elements, 8 per thread
+#pragma unroll
+    for (int it = 0; it < 8; it++) {
+      int m, k;
+      if (trans_a) { m = tid & 127; k = (tid >> 7) + it * 2; }        // A is [K,M]: m contiguous
+      else { k = tid & 15; m = (tid >> 4) + it * 16; }                // A is [M,K]: k contiguous
+      float v = 0.f;
+      if (m0 + m < M && k0 + k < K) v = to_f32(trans_a ? A[(int64_t)(k0 + k) * lda + m0 + m] : A[(int64_t)(m0 + m) * lda + k0 + k]);
+      sA[k][m] = v;
+    }
+#pragma unroll
+    for (int it = 0; it < 8; it++) {
+      int n, k;
+      if (trans_b) { k = tid & 15; n = (tid >> 4) + it * 16; }        // B is [N,K]
+      else { n = tid & 127; k = (tid >> 7) + it * 2; }                // B is [K,N]
+      float v = 0.f;
+      if (n0 + n < N && k0 + k < K) v = to_f32(trans_b ? B[(int64_t)(n0 + n) * ldb + k0 + k] : B[(int64_t)(k0 + k) * ldb + n0 + n]);
+      sB[k][n] = v;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < BK; kk += 2) {
+      const int k = kk + (lane >> 5);
+      float a[2], b[2];
+#pragma unroll
+      for (int i = 0; i < 2; i++) a[i] = sA[k][wm * 64 + i * 32 + (lane & 31)];
+#pragma unroll
+      for (int j = 0; j < 2; j++) b[j] = sB[k][wn * 64 + j * 32 + (lane & 31)];
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+    __syncthreads();
+  }
+  const int col_l = lane & 31, row_l = (lane >> 5) * 4;
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      const int col = n0 + wn * 64 + j * 32 + col_l;
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int row = m0 + wm * 64 + i * 32 + (r >> 2) * 8 + row_l + (r & 3);
+        if (row < M && col < N) {
+          float v = acc[i][j][r];
+          if (R != nullptr) v += to_f32(R[(int64_t)row * ldr + col]);
+          C[(int64_t)row * ldc + col] = from_f32<T>(v);
+        }
+      }
+    }
+}
+
+template <int BM, int BN, int WM, int WN, bool AK, bool BK_>
+static int launch_bf16(hipStream_t st, const void* A, const void* B, const void* R, void* C, int M, int N, int K, int lda,
+                       int ldb, int ldr, int ldc, uint32_t a_bytes, uint32_t b_bytes) {
+  auto kern = gemm_bf16_kernel<BM, BN, WM, WN, AK, BK_>;
+  constexpr int smem = 2 * (BM + BN) * 64 * 2;
+  static bool configured = false;   // idempotent; a race only repeats the call
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return emi_fail(EMI_INTERNAL, "emi_gemm: cannot reserve %d bytes of LDS: %s", smem, hipGetErrorString(e));
+    configured = true;
+  }
+  const int tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+  hipLaunchKernelGGL(kern, dim3(tiles), dim3(WM * WN * 64), smem, st, static_cast<const uint16_t*>(A),
+                     static_cast<const uint16_t*>(B), static_cast<const uint16_t*>(R), static_cast<uint16_t*>(C), M, N, K,
+                     lda, ldb, ldr, ldc, a_bytes, b_bytes);
+  EMI_CHECK_LAUNCH("emi_gemm");
+  return EMI_OK;
+}
+
+template <bool AK, bool BK_>
+static int launch_bf16_layout(hipStream_t st, const void* A, const void* B, const void* R, void* C, int M, int N, int K,
+                              int lda, int ldb, int ldr, int ldc, uint32_t a_bytes, uint32_t b_bytes) {
+  // 256x256 tiles when they fill the chip, else 128x128.
+  const int64_t big_tiles = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
+  if (big_tiles >= 192)
+    return launch_bf16<256, 256, 2, 4, AK, BK_>(st, A, B, R, C, M, N, K, lda, ldb, ldr, ldc, a_bytes, b_bytes);
+  return launch_bf16<128, 128, 2, 2, AK, BK_>(st, A, B, R, C, M, N, K, lda, ldb, ldr, ldc, a_bytes, b_bytes);
+}
+
+template <typename T>
+static int launch_generic(hipStream_t st, const void* A, const void* B, const void* R, void* C, int M, int N, int K,
+                          int64_t lda, int64_t ldb, int64_t ldr, int64_t ldc, int trans_a, int trans_b) {
+  dim3 grid((N + 127) / 128, (M + 127) / 128);
+  if (grid.y > 65535) return emi_fail(EMI_INVALID_ARGUMENT, "emi_gemm: M=%d too large for the generic path", M);
+  hipLaunchKernelGGL(gemm_generic_kernel<T>, grid, dim3(256), 0, st, static_cast<const T*>(A), static_cast<const T*>(B),
+                     static_cast<const T*>(R), static_cast<T*>(C), M, N, K, lda, ldb, ldr, ldc, trans_a, trans_b);
+  EMI_CHECK_LAUNCH("emi_gemm(generic)");
+  return EMI_OK;
+}
+
+}  // namespace emi
+
+using namespace emi;
+
+extern "C" int emi_gemm(emi_stream_t stream, const void* A, const void* B, const void* R, void* C, int64_t M, int64_t N,
+                        int64_t K, int64_t lda, int64_t ldb, int64_t ldr, int64_t ldc, int trans_a, int trans_b,
+                        int dtype) {
+  EMI_REQUIRE(M >= 0 && N >= 0 && K >= 0, "emi_gemm: negative dimension M=%lld N=%lld K=%lld", (long long)M, (long long)N,
+              (long long)K);
+  EMI_REQUIRE(M <= 0x7fffffff && N <= 0x7fffffff && K <= 0x7fffffff, "emi_gemm: dimension exceeds 2^31-1");
+  EMI_REQUIRE(dtype == EMI_F32 || dtype == EMI_BF16, "emi_gemm: unsupported dtype code %d (want 11=f32 or 16=bf16)", dtype);
+  if (M == 0 || N == 0) return EMI_OK;
+  EMI_REQUIRE(A && B && C, "emi_gemm: null buffer");
+  EMI_REQUIRE(lda >= (trans_a ? M : K) && ldb >= (trans_b ? K : N) && ldc >= N && (R == nullptr || ldr >= N),
+              "emi_gemm: leading dimension smaller than the row length (lda=%lld ldb=%lld ldr=%lld ldc=%lld)",
+              (long long)lda, (long long)ldb, (long long)ldr, (long long)ldc);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == EMI_BF16) {
+    const int64_t a_rows = trans_a ? K : M, b_rows = trans_b ? N : K;
+    const int64_t a_bytes = ((a_rows - 1) * lda + (trans_a ? M : K)) * 2;
+    const int64_t b_bytes = ((b_rows - 1) * ldb + (trans_b ? K : N)) * 2;
+    auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+    // The fast path moves 16-byte chunks: rows must start 16-byte aligned and
+    // row lengths in the contiguous dimension must be multiples of 8 elements.
+    const bool fast = K > 0 && al16(A) && al16(B) && (lda % 8 == 0) && (ldb % 8 == 0) && (K % 8 == 0) &&
+                      (!trans_a || M % 8 == 0) && (trans_b || N % 8 == 0) && a_bytes < 0x7fffff00LL &&
+                      b_bytes < 0x7fffff00LL && ldr <= 0x7fffffff && ldc <= 0x7fffffff;
+    if (fast) {
+      const int m = (int)M, n = (int)N, k = (int)K;
+      const uint32_t ab = (uint32_t)a_bytes, bb = (uint32_t)b_bytes;
+      if (!trans_a && trans_b)
+        return launch_bf16_layout<false, false>(st, A, B, R, C, m, n, k, (int)lda, (int)ldb, (int)ldr, (int)ldc, ab, bb);
+      if (!trans_a && !trans_b)
+        return launch_bf16_layout<false, true>(st, A, B, R, C, m, n, k, (int)lda, (int)ldb, (int)ldr, (int)ldc, ab, bb);
+      if (trans_a && !trans_b)
+        return launch_bf16_layout<true, true>(st, A, B, R, C, m, n, k, (int)lda, (int)ldb, (int)ldr, (int)ldc, ab, bb);
+      return launch_bf16_layout<true, false>(st, A, B, R, C, m, n, k, (int)lda, (int)ldb, (int)ldr, (int)ldc, ab, bb);
+    }
+    return launch_generic<bf16>(st, A, B, R, C, (int)M, (int)N, (int)K, lda, ldb, ldr, ldc, trans_a, trans_b);
+  }
+  return launch_generic<float>(st, A, B, R, C, (int)M, (int)N, (int)K, lda, ldb, ldr, ldc, trans_a, trans_b);
+}

@@ -1,0 +1,47 @@
+"""The llama2-style transformer of the reference's test/llama.py, batched and
+causal, written with the HIP operators of `enzyme_ad.jax.ops`.
+
+`forward(x, config, weights, ...)` keeps the reference's argument order
+(test/llama.py:35) where that makes sense: activations [B, S, dim] replace the
+single-token vector, the causal mask replaces the KV cache (a token at
+position t attends to rows 0..t, exactly what the step form sees in its
+cache).  Weight names and layouts are the reference's: matrices are [out, in]
+and applied as `w @ x` (:149).
+"""
+from . import ops
+
+LAYER_KEYS = ("rms_att_weight", "wq", "wk", "wv", "wo", "rms_ffn_weight", "w1", "w2", "w3")
+
+
+def layer(x, lw, n_heads, eps=1e-5, theta=10000.0):
+    """One decoder layer (test/llama.py:144-233).  x: [B, S, dim]."""
+    xb = ops.rmsnorm(x, lw["rms_att_weight"], eps)                 # :145
+    q = ops.matmul_nt(xb, lw["wq"])                                # :149-157
+    k = ops.matmul_nt(xb, lw["wk"])
+    v = ops.matmul_nt(xb, lw["wv"])
+    q = ops.rope(q, n_heads, theta)                                # :161-168
+    k = ops.rope(k, n_heads, theta)
+    att = ops.attention(q, k, v, n_heads, causal=True)             # :178-209
+    x = ops.matmul_nt(att, lw["wo"], residual=x)                   # :211-215
+    xb = ops.rmsnorm(x, lw["rms_ffn_weight"], eps)                 # :219
+    h1 = ops.matmul_nt(xb, lw["w1"])                               # :224-225
+    h3 = ops.matmul_nt(xb, lw["w3"])
+    g = ops.swiglu(h1, h3)                                         # :227-229
+    return ops.matmul_nt(g, lw["w2"], residual=x)                  # :231-233
+
+
+def forward(x, config, weights, logits=False, eps=1e-5, theta=10000.0):
+    """Whole model.  x: activations [B, S, dim], or int32 tokens [B, S] when
+    `weights` holds `token_embedding_table` (the lookup commented out at
+    test/llama.py:109-113).  Returns the final RMSNorm of the residual stream
+    (:235) or, with `logits`, its `wcls` projection (:236)."""
+    n_layers, n_heads = config["n_layers"], config["n_heads"]
+    if not x.is_floating_point():
+        x = ops.embedding(x, weights["token_embedding_table"])
+    for i in range(n_layers):
+        lw = {k: weights[k][i] for k in LAYER_KEYS}
+        x = layer(x, lw, n_heads, eps, theta)
+    x = ops.rmsnorm(x, weights["rms_final_weight"], eps)
+    if logits:
+        x = ops.matmul_nt(x, weights["wcls"])
+    return x

@@ -1,0 +1,322 @@
+"""Device operators of the llama path and their reverse-mode rules.
+
+This is the lowering table of the MI355X build: where the reference lowers an
+`enzyme_jax_ir`-decorated function to optimized StableHLO and lets XLA generate
+code (src/enzyme_ad/jax/primitives.py:626-692), each operator here is one
+custom-call target (`emi_<op>`) served by a hand-written gfx950 kernel through
+the C ABI in include/emi.h.  Tensors are torch CUDA tensors (device memory and
+streams only; no torch arithmetic happens on this path).
+
+Every operator records, on the active `Tape`, a rule that maps the cotangent
+of its result to the cotangents of its operands.  The rules restate the
+reference's StableHLO adjoints for the op clusters test/llama.py traces
+(Implementations/HLODerivatives.td: DotGeneral :1166, Mul :1221, Div :1133,
+Exp :1182, Sqrt :1320, Add :964; StableHLOAutoDiffOpInterfaceImpl.cpp: Reduce
+:1833).  A rule receives the cotangent already accumulated for each operand so
+that fan-in sums (Add rule) are fused into the producing kernel's epilogue
+instead of costing an extra pass over HBM.
+"""
+import math
+
+import torch
+
+from . import _native as N
+
+FFI_TARGETS = {
+    # operator        -> (forward target, adjoint target(s))
+    "rmsnorm":   ("emi_rmsnorm_fwd", ("emi_rmsnorm_bwd",)),
+    "rope":      ("emi_rope", ("emi_rope",)),                    # adjoint = inverse rotation
+    "matmul_nt": ("emi_gemm", ("emi_gemm", "emi_gemm")),         # dX (NN) and dW (TN)
+    "swiglu":    ("emi_swiglu_fwd", ("emi_swiglu_bwd",)),
+    "attention": ("emi_attn_fwd", ("emi_attn_bwd",)),
+    "add":       ("emi_add", ()),
+    "embedding": ("emi_embedding_fwd", ("emi_embedding_bwd",)),
+}
+
+_DTYPES = {torch.float32: N.EMI_F32, torch.bfloat16: N.EMI_BF16}
+
+
+def _code(t):
+    try:
+        return _DTYPES[t.dtype]
+    except KeyError:
+        raise TypeError("unsupported dtype %s (float32 and bfloat16 only)" % t.dtype) from None
+
+
+def _dev(*ts):
+    for t in ts:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise RuntimeError("operand is not in device memory: the HIP path has no CPU fallback")
+        if not t.is_contiguous():
+            raise ValueError("operand must be contiguous")
+
+
+def _p(t):
+    return None if t is None else t.data_ptr()
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _same_dtype(*ts):
+    d = ts[0].dtype
+    for t in ts[1:]:
+        if t is not None and t.dtype != d:
+            raise TypeError("mixed dtypes: %s vs %s" % (d, t.dtype))
+
+
+# ---------------------------------------------------------------------------
+# tape
+# ---------------------------------------------------------------------------
+
+class Tape:
+    """Linear record of operator applications for reverse mode."""
+
+    _active = None
+
+    def __init__(self):
+        self.nodes = []          # (inputs, output, rule)
+
+    def __enter__(self):
+        self._prev = Tape._active
+        Tape._active = self
+        return self
+
+    def __exit__(self, *exc):
+        Tape._active = self._prev
+        return False
+
+    @staticmethod
+    def record(inputs, output, rule):
+        t = Tape._active
+        if t is not None:
+            t.nodes.append((inputs, output, rule))
+
+    def backward(self, outputs, cotangents, wrt):
+        """Cotangents of `wrt` (list of tensors) given cotangents of `outputs`."""
+        ct = {}
+        for o, c in zip(outputs, cotangents):
+            if c is None:
+                continue
+            if c.shape != o.shape or c.dtype != o.dtype:
+                raise ValueError("cotangent %s/%s does not match output %s/%s" % (tuple(c.shape), c.dtype, tuple(o.shape), o.dtype))
+            ct[id(o)] = c if id(o) not in ct else add(ct[id(o)], c)
+        for inputs, output, rule in reversed(self.nodes):
+            c = ct.pop(id(output), None)
+            if c is None:
+                continue
+            first, acc = set(), []
+            for i in inputs:          # an operand that appears twice gets its fan-in summed afterwards
+                fresh = isinstance(i, torch.Tensor) and id(i) not in first
+                acc.append(ct.get(id(i)) if fresh else None)
+                first.add(id(i))
+            new = rule(c, acc)
+            done = set()
+            for i, g in zip(inputs, new):
+                if g is None:
+                    continue
+                ct[id(i)] = g if id(i) not in done else add(ct[id(i)], g)
+                done.add(id(i))
+        return [ct.get(id(w)) for w in wrt]
+
+
+def _accumulate(acc, g):
+    return g if acc is None else add(acc, g)
+
+
+# ---------------------------------------------------------------------------
+# operators
+# ---------------------------------------------------------------------------
+
+def add(a, b):
+    """a + b (test/llama.py:215,233; Add rule HLODerivatives.td:964)."""
+    _dev(a, b)
+    _same_dtype(a, b)
+    if a.shape != b.shape:
+        raise ValueError("add: shape mismatch %s vs %s" % (tuple(a.shape), tuple(b.shape)))
+    y = torch.empty_like(a)
+    N.check(N.lib().emi_add(_stream(), _p(a), _p(b), _p(y), a.numel(), _code(a)))
+    Tape.record((a, b), y, lambda c, acc: (_accumulate(acc[0], c), _accumulate(acc[1], c)))
+    return y
+
+
+def rmsnorm(x, gamma, eps=1e-5):
+    """gamma * x * rsqrt(mean(x^2) + eps) over the last dim (test/llama.py:6-10)."""
+    _dev(x, gamma)
+    _same_dtype(x, gamma)
+    D = x.shape[-1]
+    if gamma.shape != (D,):
+        raise ValueError("rmsnorm: gamma shape %s != (%d,)" % (tuple(gamma.shape), D))
+    rows = x.numel() // D
+    y = torch.empty_like(x)
+    N.check(N.lib().emi_rmsnorm_fwd(_stream(), _p(x), _p(gamma), _p(y), rows, D, eps, _code(x)))
+
+    def rule(c, acc):
+        dx = torch.empty_like(x)
+        dgamma = torch.empty_like(gamma)
+        nbytes = N.lib().emi_rmsnorm_bwd_workspace_bytes(rows, D)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+        N.check(N.lib().emi_rmsnorm_bwd(_stream(), _p(x), _p(gamma), _p(c), _p(acc[0]), _p(dx), _p(dgamma), _p(ws),
+                                        nbytes, rows, D, eps, _code(x)))
+        return dx, _accumulate(acc[1], dgamma)
+
+    Tape.record((x, gamma), y, rule)
+    return y
+
+
+_rope_tables = {}
+
+
+def rope_table(seq, head_dim, theta=10000.0, pos0=0, device=None):
+    """fp32 (cos, sin) table [seq, head_dim/2, 2]; trace-time constants in the
+    reference (test/llama.py:127-140).  Cached per (device, shape, theta, pos0)."""
+    device = torch.device("cuda", torch.cuda.current_device()) if device is None else device
+    key = (str(device), seq, head_dim, float(theta), pos0)
+    t = _rope_tables.get(key)
+    if t is None:
+        t = torch.empty((seq, head_dim // 2, 2), dtype=torch.float32, device=device)
+        N.check(N.lib().emi_rope_table(_stream(), _p(t), seq, head_dim, float(theta), pos0))
+        _rope_tables[key] = t
+    return t
+
+
+def rope(x, n_heads, theta=10000.0, pos0=0, inverse=False):
+    """Rotate adjacent pairs of every head of x [B, S, n_heads*head_dim] by the
+    position angle (test/llama.py:161-168)."""
+    _dev(x)
+    B, S, D = x.shape
+    d = D // n_heads
+    if d * n_heads != D or d % 2:
+        raise ValueError("rope: dim %d is not n_heads=%d x even head_dim" % (D, n_heads))
+    table = rope_table(S, d, theta, pos0, x.device)
+    y = torch.empty_like(x)
+    N.check(N.lib().emi_rope(_stream(), _p(x), _p(table), _p(y), B, S, n_heads, d, int(inverse), _code(x)))
+
+    def rule(c, acc):
+        g = torch.empty_like(c)
+        N.check(N.lib().emi_rope(_stream(), _p(c), _p(table), _p(g), B, S, n_heads, d, int(not inverse), _code(c)))
+        return (_accumulate(acc[0], g),)
+
+    Tape.record((x,), y, rule)
+    return y
+
+
+def gemm(a, b, trans_a=False, trans_b=False, residual=None):
+    """op(a) . op(b) [+ residual] on 2-D operands; fp32 accumulate."""
+    _dev(a, b, residual)
+    _same_dtype(a, b, residual)
+    M, K = (a.shape[1], a.shape[0]) if trans_a else a.shape
+    Kb, Nn = (b.shape[1], b.shape[0]) if trans_b else b.shape
+    if K != Kb:
+        raise ValueError("gemm: contraction mismatch %d vs %d" % (K, Kb))
+    if residual is not None and residual.shape != (M, Nn):
+        raise ValueError("gemm: residual shape %s != (%d, %d)" % (tuple(residual.shape), M, Nn))
+    c = torch.empty((M, Nn), dtype=a.dtype, device=a.device)
+    N.check(N.lib().emi_gemm(_stream(), _p(a), _p(b), _p(residual), _p(c), M, Nn, K, a.shape[1], b.shape[1], Nn, Nn,
+                             int(trans_a), int(trans_b), _code(a)))
+    return c
+
+
+def matmul_nt(x, w, residual=None):
+    """Y[..., out] = X[..., in] . W[out, in]^T [+ residual]  (`w @ x` of
+    test/llama.py:149-157,211,224-233, batched over tokens)."""
+    lead = x.shape[:-1]
+    K = x.shape[-1]
+    Nout = w.shape[0]
+    x2 = x.reshape(-1, K)
+    r2 = None if residual is None else residual.reshape(-1, Nout)
+    y = gemm(x2, w, False, True, r2).reshape(*lead, Nout)
+
+    def rule(c, acc):
+        c2 = c.reshape(-1, Nout)
+        ax = None if acc[0] is None else acc[0].reshape(-1, K)
+        dx = gemm(c2, w, False, False, ax).reshape(x.shape)      # dX = dY . W   (NN)
+        dw = gemm(c2, x2, True, False, acc[1])                   # dW = dY^T . X (TN)
+        out = [dx, dw]
+        if residual is not None:
+            out.append(_accumulate(acc[2], c))
+        return out
+
+    Tape.record((x, w) if residual is None else (x, w, residual), y, rule)
+    return y
+
+
+def swiglu(a, b):
+    """a * sigmoid(a) * b (test/llama.py:21-28,229-231)."""
+    _dev(a, b)
+    _same_dtype(a, b)
+    if a.shape != b.shape:
+        raise ValueError("swiglu: shape mismatch")
+    g = torch.empty_like(a)
+    N.check(N.lib().emi_swiglu_fwd(_stream(), _p(a), _p(b), _p(g), a.numel(), _code(a)))
+
+    def rule(c, acc):
+        da, db = torch.empty_like(a), torch.empty_like(b)
+        N.check(N.lib().emi_swiglu_bwd(_stream(), _p(a), _p(b), _p(c), _p(da), _p(db), a.numel(), _code(a)))
+        return _accumulate(acc[0], da), _accumulate(acc[1], db)
+
+    Tape.record((a, b), g, rule)
+    return g
+
+
+def attention_raw(q, k, v, n_heads, scale, causal, strides):
+    B, S = q.shape[0], q.shape[1 if strides == "bshd" else 2]
+    d = q.shape[-1] if q.dim() == 4 else q.shape[-1] // n_heads
+    if strides == "bshd":
+        sb, sh, ss = S * n_heads * d, d, n_heads * d
+    else:
+        sb, sh, ss = n_heads * S * d, S * d, d
+    o = torch.empty_like(q)
+    lse = torch.empty((B, n_heads, S), dtype=torch.float32, device=q.device)
+    N.check(N.lib().emi_attn_fwd(_stream(), _p(q), _p(k), _p(v), _p(o), _p(lse), B, n_heads, S, d, sb, sh, ss,
+                                 float(scale), int(causal), _code(q)))
+    return o, lse, (B, S, d, sb, sh, ss)
+
+
+def attention(q, k, v, n_heads, scale=None, causal=True, layout="bshd"):
+    """Causal softmax attention (test/llama.py:178-206).  layout "bshd": operands
+    are [B, S, n_heads*head_dim] (token-major, as the projections produce them);
+    layout "bhsd": [B, n_heads, S, head_dim]."""
+    _dev(q, k, v)
+    _same_dtype(q, k, v)
+    if q.shape != k.shape or q.shape != v.shape:
+        raise ValueError("attention: q, k, v shapes differ")
+    d = q.shape[-1] // n_heads if layout == "bshd" else q.shape[-1]
+    if scale is None:
+        scale = 1.0 / math.sqrt(d)
+    o, lse, (B, S, d, sb, sh, ss) = attention_raw(q, k, v, n_heads, scale, causal, layout)
+
+    def rule(c, acc):
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        nbytes = N.lib().emi_attn_bwd_workspace_bytes(B, n_heads, S, d)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
+        N.check(N.lib().emi_attn_bwd(_stream(), _p(q), _p(k), _p(v), _p(o), _p(lse), _p(c), _p(dq), _p(dk), _p(dv),
+                                     _p(ws), nbytes, B, n_heads, S, d, sb, sh, ss, float(scale), int(causal), _code(q)))
+        return _accumulate(acc[0], dq), _accumulate(acc[1], dk), _accumulate(acc[2], dv)
+
+    Tape.record((q, k, v), o, rule)
+    return o
+
+
+def embedding(tokens, table):
+    """table[tokens] (the lookup commented out at test/llama.py:109-113)."""
+    _dev(tokens, table)
+    if tokens.dtype != torch.int32:
+        raise TypeError("embedding: tokens must be int32")
+    V, D = table.shape
+    x = torch.empty(tuple(tokens.shape) + (D,), dtype=table.dtype, device=table.device)
+    N.check(N.lib().emi_embedding_fwd(_stream(), _p(tokens), _p(table), _p(x), tokens.numel(), V, D, _code(table)))
+
+    def rule(c, acc):
+        dt = torch.empty_like(table)
+        nbytes = N.lib().emi_embedding_bwd_workspace_bytes(V, D, _code(table))
+        ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=table.device)
+        N.check(N.lib().emi_embedding_bwd(_stream(), _p(tokens), _p(c), _p(dt), _p(ws), nbytes, tokens.numel(), V, D,
+                                          _code(table)))
+        return None, _accumulate(acc[1], dt)
+
+    Tape.record((tokens, table), x, rule)
+    return x

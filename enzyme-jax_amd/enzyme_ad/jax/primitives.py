@@ -1,0 +1,331 @@
+"""API surface of the reference's `enzyme_ad.jax` (src/enzyme_ad/jax/primitives.py)
+over the MI355X kernels.
+
+Kept from the reference: the pipeline configuration objects (`JaXPipeline`,
+`XLAPipeline`, :81-115), the pass-pipeline string builders
+(`optimization_passes`, `full_optimization_pass_pipeline`, :118-223), the
+decorator `enzyme_jax_ir(argv, pipeline_options, jit_options, inner_jit)`
+(:1528-1590) and the entry-point names `ffi_call`, `cpp_call`, `hlo_call`,
+`optimize_module`, `export`.
+
+Changed: the decorated function is written with the operators of
+`enzyme_ad.jax.ops` and runs eagerly on HIP streams; `vjp` below plays the role
+of `jax.vjp` through the reference's `enzyme_vjp` rule (:1381-1486): it returns
+the primal result and a function from result cotangents to argument cotangents.
+The MLIR pass pipeline named by `pipeline_options` selects nothing here - the
+fused kernels implement the optimized graph directly - but the strings are
+still built, parsed and carried so that code written for the reference runs.
+"""
+from collections.abc import Callable, Sequence
+from typing import Any
+
+import torch
+
+from . import ops
+
+LANG_CPP, LANG_LLVM, LANG_MHLO = 0, 1, 2     # enzyme_call.Language (enzyme_call.cc)
+
+
+class PipelineConfig:
+    """primitives.py:56-78."""
+
+    def xla_runtime(self):
+        raise NotImplementedError()
+
+    def pass_pipeline(self):
+        raise NotImplementedError()
+
+    def mlir_ad(self):
+        raise NotImplementedError()
+
+    def stablehlo_inject(self):
+        raise NotImplementedError()
+
+    def ad_level(self):
+        raise NotImplementedError()
+
+    def export_llvm(self):
+        raise NotImplementedError()
+
+
+class XLAPipeline(PipelineConfig):
+    """primitives.py:81-98 (LLVM-level AD of XLA-CPU code; CPU only there)."""
+
+    def __init__(self, name=None):
+        self.exportname = name
+
+    def xla_runtime(self):
+        return False
+
+    def pass_pipeline(self):
+        return ""
+
+    def mlir_ad(self):
+        return False
+
+    def stablehlo_inject(self):
+        return False
+
+    def export_llvm(self):
+        return self.exportname
+
+
+class JaXPipeline(PipelineConfig):
+    """primitives.py:101-115."""
+
+    def __init__(self, passes=""):
+        self.passes = passes
+
+    def pass_pipeline(self):
+        return self.passes
+
+    def mlir_ad(self):
+        return True
+
+    def stablehlo_inject(self):
+        return True
+
+    def ad_level(self):
+        return self.passes.count("enzyme-wrap")
+
+
+# Pattern-list placeholder: the reference obtains ~1000 rewrite-pattern names
+# from its C++ pass-list generator (Integrations/c/EnzymeXLA.cpp:951-1104).
+# The list itself has no meaning for fused kernels; its knobs are kept.
+def _pattern_list(**kw):
+    parts = ["emi_fused_llama<1>"]
+    parts.append("max_constant_expansion<1>(%d)" % kw["max_constant_threshold"])
+    for k in ("no_nan", "all_finite"):
+        if kw[k]:
+            parts.append("%s<1>" % k)
+    parts.append("transpose_propagate_%s<1>" % kw["transpose_propagate"])
+    parts.append("reshape_propagate_%s<1>" % kw["reshape_propagate"])
+    return ";".join(p for p in parts if p.split("<")[0] not in set(kw["excluded_passes"]))
+
+
+def optimization_passes(
+    *,
+    inline: bool = True,
+    no_nan: bool = False,
+    all_finite: bool = False,
+    transpose_propagate: str = "up",
+    reshape_propagate: str = "up",
+    max_constant_threshold: int = 1024,
+    enable_licm_optimization_passes: bool = True,
+    loop_unswitch_threshold: int = 10,
+    excluded_passes: list = [],
+    enable_scatter_gather_optimization_passes: bool = True,
+    enable_pad_optimization_passes: bool = True,
+    enable_self_to_convolution_like_passes: bool = False,
+    enable_structured_tensors_detection_passes: bool = False,
+    enable_structured_tensors_passes: bool = True,
+    enable_slice_to_batch_passes: bool = False,
+    enable_reduce_slice_fusion_passes: bool = True,
+    enable_concat_to_batch_passes: bool = True,
+    enable_loop_raising_passes: bool = True,
+    aggressive_propagation: bool = True,
+):
+    """Same keywords and string structure as primitives.py:118-192."""
+    for name, val in (("transpose_propagate", transpose_propagate), ("reshape_propagate", reshape_propagate)):
+        if val not in ("none", "up", "down"):
+            raise ValueError("%s must be 'none', 'up' or 'down', got %r" % (name, val))
+    main_passes_str = _pattern_list(
+        no_nan=no_nan, all_finite=all_finite, transpose_propagate=transpose_propagate,
+        reshape_propagate=reshape_propagate, max_constant_threshold=max_constant_threshold,
+        excluded_passes=list(excluded_passes))
+    transform_passes = ",".join([
+        "enzyme-hlo-generate-td{patterns=" + main_passes_str + "}",
+        "transform-interpreter",
+        "enzyme-hlo-remove-transform",
+    ])
+    func_passes = ",".join(["canonicalize", "cse", "canonicalize", transform_passes])
+    if inline:
+        func_passes = "inline{default-pipeline=canonicalize max-iterations=4}" + "," + func_passes
+    return func_passes
+
+
+def full_optimization_pass_pipeline(**kwargs):
+    """primitives.py:195-223."""
+    opt_passes = optimization_passes(**kwargs)
+    enzyme_pass = ('enzyme{postpasses="arith-raise{stablehlo=true},enzyme-batch-to-stablehlo,canonicalize,cse,'
+                   'canonicalize,remove-unnecessary-enzyme-ops,enzyme-simplify-math,canonicalize,cse,canonicalize"}')
+    propagate_down_passes = ""
+    if kwargs.get("transpose_propagate", "up") == "up" or kwargs.get("reshape_propagate", "up") == "up":
+        kw = dict(kwargs)
+        kw.update(transpose_propagate="down", reshape_propagate="down")
+        propagate_down_passes = optimization_passes(**kw)
+    return ",".join([
+        "mark-func-memory-effects", opt_passes, "enzyme-batch", opt_passes, enzyme_pass, opt_passes, "canonicalize",
+        "remove-unnecessary-enzyme-ops", "enzyme-simplify-math", opt_passes, propagate_down_passes,
+    ])
+
+
+DefaultCPPPipeline = XLAPipeline()
+DefaultJaXPipeline = JaXPipeline(full_optimization_pass_pipeline())
+
+
+def parse_pass_pipeline(text):
+    """Split an MLIR textual pass pipeline into [(pass name, option string)].
+    Tolerates nested braces and quoted option values (the grammar seen in
+    primitives.py:195-223 and TransformOps/GenerateApplyPatterns.cpp:98-148)."""
+    out, depth, cur, quote = [], 0, [], False
+    for ch in text:
+        if ch == '"':
+            quote = not quote
+        if not quote:
+            if ch == "{":
+                depth += 1
+            elif ch == "}":
+                depth -= 1
+                if depth < 0:
+                    raise ValueError("unbalanced '}' in pass pipeline")
+        if ch == "," and depth == 0 and not quote:
+            out.append("".join(cur))
+            cur = []
+        else:
+            cur.append(ch)
+    if depth != 0 or quote:
+        raise ValueError("unbalanced braces or quotes in pass pipeline")
+    out.append("".join(cur))
+    res = []
+    for item in out:
+        item = item.strip()
+        if not item:
+            continue
+        name, _, rest = item.partition("{")
+        res.append((name.strip(), rest[:-1] if rest.endswith("}") else rest))
+    return res
+
+
+# ---------------------------------------------------------------------------
+# pytrees (dict / list / tuple of tensors), the part of jax.tree_util used at
+# primitives.py:1538-1546
+# ---------------------------------------------------------------------------
+
+def tree_flatten(tree):
+    leaves = []
+
+    def walk(t):
+        if isinstance(t, dict):
+            return ("dict", [(k, walk(t[k])) for k in sorted(t)])
+        if isinstance(t, (list, tuple)):
+            return (type(t).__name__, [walk(x) for x in t])
+        leaves.append(t)
+        return ("leaf", None)
+
+    return leaves, walk(tree)
+
+
+def tree_unflatten(treedef, leaves):
+    it = iter(leaves)
+
+    def build(d):
+        kind, sub = d
+        if kind == "dict":
+            return {k: build(s) for k, s in sub}
+        if kind == "list":
+            return [build(s) for s in sub]
+        if kind == "tuple":
+            return tuple(build(s) for s in sub)
+        return next(it)
+
+    return build(treedef)
+
+
+class _EnzymeFunction:
+    """What `enzyme_jax_ir(...)(func)` returns: callable for the primal; carries
+    the options the reference passes to `ffi_call` (primitives.py:1571-1585)."""
+
+    def __init__(self, func, argv, pipeline_options, jit_options, inner_jit):
+        self.func = func
+        self.argv = tuple(argv)
+        self.pipeline_options = pipeline_options
+        self.jit_options = dict(jit_options)
+        self.inner_jit = inner_jit
+        self.lang = LANG_MHLO
+        self.__name__ = getattr(func, "__name__", "enzyme_fn")
+        if pipeline_options is not None:
+            if not hasattr(pipeline_options, "pass_pipeline"):
+                raise TypeError("pipeline_options must be a JaXPipeline/XLAPipeline, got %r" % (pipeline_options,))
+            if not pipeline_options.stablehlo_inject() and not isinstance(pipeline_options, XLAPipeline):
+                raise TypeError("unsupported pipeline configuration")
+            parse_pass_pipeline(pipeline_options.pass_pipeline())      # malformed strings fail here, at decoration
+
+    def __call__(self, *args, **kwargs):
+        if self.jit_options.get("print_mlir"):
+            print("// enzyme_jax_ir %s lowered to targets: %s" % (self.__name__, ", ".join(sorted(ops.FFI_TARGETS))))
+        return self.func(*args, **kwargs)
+
+
+def enzyme_jax_ir(argv=(), pipeline_options=DefaultJaXPipeline, jit_options={}, inner_jit=True):
+    """Decorator with the reference's signature (primitives.py:1528-1530)."""
+
+    def decorator(func: Callable[..., Any]) -> Callable[..., Any]:
+        return _EnzymeFunction(func, argv, pipeline_options, jit_options, inner_jit)
+
+    return decorator
+
+
+def vjp(fn, *args):
+    """(primals_out, f_vjp) like `jax.vjp`: `f_vjp(cotangents)` returns one
+    cotangent pytree per positional argument (None for integer leaves and for
+    leaves the result does not depend on... those get zeros, like the reference's
+    `make_mlir_zero`, primitives.py:487-499,741)."""
+    leaves, treedef = tree_flatten(args)
+    with ops.Tape() as tape:
+        out = fn(*args)
+    out_leaves, out_def = tree_flatten(out)
+
+    def f_vjp(cotangents):
+        ct_leaves, ct_def = tree_flatten(cotangents)
+        if len(ct_leaves) != len(out_leaves):
+            raise ValueError("cotangent tree has %d leaves, result has %d" % (len(ct_leaves), len(out_leaves)))
+        wrt = [l for l in leaves if isinstance(l, torch.Tensor) and l.is_floating_point()]
+        grads = tape.backward(out_leaves, ct_leaves, wrt)
+        it = iter(grads)
+        full = []
+        for l in leaves:
+            if isinstance(l, torch.Tensor) and l.is_floating_point():
+                g = next(it)
+                full.append(torch.zeros_like(l) if g is None else g)
+            else:
+                full.append(None)
+        return tree_unflatten(treedef, full)
+
+    return out, f_vjp
+
+
+def jvp(fn, primals, tangents):
+    """Forward mode (reference: enzyme_jvp, primitives.py:1147-1245) is not
+    built for the HIP path yet."""
+    raise NotImplementedError("forward-mode (jvp) kernels are not implemented on the HIP path")
+
+
+def ffi_call(*args, out_shapes: Sequence[Any], source, fn: str = "f", argv=(), lang: int = LANG_CPP,
+             pipeline_options=DefaultCPPPipeline):
+    """primitives.py:1020-1038.  C++/LLVM sources need the reference's in-process
+    clang + Enzyme JIT (clang_compile.cc), which is CPU-only and not part of this build."""
+    raise NotImplementedError("ffi_call with C++/LLVM/MHLO source text is not supported by the HIP path; "
+                              "decorate a function written with enzyme_ad.jax.ops with enzyme_jax_ir instead")
+
+
+def cpp_call(*args, out_shapes: Sequence[Any], source: str, fn: str = "f", argv=(),
+             pipeline_options=DefaultCPPPipeline):
+    """primitives.py:1111-1127."""
+    return ffi_call(*args, source=source, fn=fn, argv=argv, out_shapes=out_shapes, lang=LANG_CPP,
+                    pipeline_options=pipeline_options)
+
+
+def hlo_call(*args, source: str, argv=(), passes: str = ""):
+    """primitives.py:1052-1108 (StableHLO text in): needs an MLIR front end; not built."""
+    raise NotImplementedError("hlo_call needs a StableHLO front end, which the HIP path does not have")
+
+
+def optimize_module(mod, pipeline=None):
+    """primitives.py (optimize_module): runs the MLIR optimizer on a module; not built."""
+    raise NotImplementedError("optimize_module needs the MLIR optimizer, which the HIP path does not have")
+
+
+def export(outfile, func, *args, argv=(), jit_options={}):
+    """primitives.py:1489-1525 (export to LLVM IR); not built."""
+    raise NotImplementedError("export needs the XLA-CPU/LLVM pipeline, which the HIP path does not have")

@@ -1,0 +1,137 @@
+/* emi.h - C ABI of the MI355X (gfx950) llama forward + reverse-mode kernels.
+ *
+ * Boundary: these entry points are what an XLA custom-call handler for the
+ * llama path binds.  The reference hands its optimized StableHLO to XLA's own
+ * code generator (src/enzyme_ad/jax/primitives.py:626-692) and its only native
+ * handlers are the typed-FFI cuBLAS wrappers (src/enzyme_ad/jax/xla_ffi/cuda/
+ * blas.cc:286-313) and the kernel_call bundle (src/enzyme_ad/jax/gpu.cc:35-173);
+ * each function below cites the reference item whose arithmetic it replaces.
+ *
+ * Conventions
+ *  - plain pointers and sizes only; every pointer is DEVICE memory unless said
+ *    otherwise; `stream` is a hipStream_t passed as void* (NULL = default stream);
+ *  - work is enqueued on `stream`, no host synchronisation, no allocation;
+ *    scratch space is an explicit `workspace` argument sized by the matching
+ *    `*_workspace_bytes` query (the reference passes scratch as an extra
+ *    result buffer, primitives.py:712-727);
+ *  - row-major tensors, innermost dimension contiguous;
+ *  - `dtype` is an XLA PrimitiveType code: EMI_F32 (11) or EMI_BF16 (16); all
+ *    reductions, softmax statistics and GEMM accumulators are fp32;
+ *  - return value 0 = success, otherwise an absl/XLA status code
+ *    (EMI_INVALID_ARGUMENT = 3, EMI_UNIMPLEMENTED = 12, EMI_INTERNAL = 13) and a
+ *    message retrievable with emi_last_error(); nothing is launched on error
+ *    and nothing ever aborts or throws across this boundary.
+ */
+#ifndef EMI_H_
+#define EMI_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* emi_stream_t;
+
+enum { EMI_F32 = 11, EMI_BF16 = 16 };
+enum { EMI_OK = 0, EMI_INVALID_ARGUMENT = 3, EMI_UNIMPLEMENTED = 12, EMI_INTERNAL = 13 };
+
+#define EMI_ABI_VERSION 1
+
+/* ABI version of the loaded library (EMI_ABI_VERSION at build time). */
+int emi_abi_version(void);
+/* Message of the last failing call on this thread ("" if none). Host pointer. */
+const char* emi_last_error(void);
+
+/* RMSNorm forward: y = gamma * x * rsqrt(mean(x^2) + eps) over the last dim.
+ * Replaces rmsnorm() of test/llama.py:6-10.  x,y: [rows, dim]; gamma: [dim]. */
+int emi_rmsnorm_fwd(emi_stream_t stream, const void* x, const void* gamma, void* y,
+                    int64_t rows, int64_t dim, float eps, int dtype);
+
+/* RMSNorm adjoint (recomputes rstd from x, like the reference's combined
+ * reverse program): dx = [dx_add +] r*g - x*r^3*mean(g*x), g = dy*gamma;
+ * dgamma = sum_rows dy*x*r.  Replaces the Mul/Div/Sqrt/DotGeneral/Reduce
+ * rules of HLODerivatives.td:1221,1133,1320,1166 applied to llama.py:6-10.
+ * dx_add (nullable): residual-stream cotangent added into dx (Add rule, :964).
+ * dgamma: [dim] in `dtype`.  workspace: emi_rmsnorm_bwd_workspace_bytes(). */
+size_t emi_rmsnorm_bwd_workspace_bytes(int64_t rows, int64_t dim);
+int emi_rmsnorm_bwd(emi_stream_t stream, const void* x, const void* gamma, const void* dy,
+                    const void* dx_add, void* dx, void* dgamma, void* workspace,
+                    size_t workspace_bytes, int64_t rows, int64_t dim, float eps, int dtype);
+
+/* RoPE angle table: table[s][j] = (cos, sin)(pos * theta^(-2j/head_dim)),
+ * pos = pos0 + s, computed in float64 and rounded to fp32.  In the reference
+ * these are trace-time constants (test/llama.py:127-140).
+ * table: float[seq, head_dim/2, 2]. */
+int emi_rope_table(emi_stream_t stream, float* table, int64_t seq, int64_t head_dim,
+                   double theta, int64_t pos0);
+
+/* RoPE apply: rotate adjacent pairs (2p, 2p+1) of every head by +angle, or by
+ * -angle when inverse != 0 (the adjoint).  Replaces the einsum of
+ * test/llama.py:161-168 and its DotGeneral adjoint (HLODerivatives.td:1166).
+ * x,y: [batch, seq, heads, head_dim] contiguous; y may alias x. */
+int emi_rope(emi_stream_t stream, const void* x, const float* table, void* y, int64_t batch,
+             int64_t seq, int64_t heads, int64_t head_dim, int inverse, int dtype);
+
+/* SwiGLU forward g = a * sigmoid(a) * b and adjoint
+ * da = dg*b*s*(1 + a*(1-s)), db = dg*a*s.  Replaces silu()/sigmoid() of
+ * test/llama.py:21-28,229-231 and the Neg/Exp/Add/Div/Mul rules.  n elements. */
+int emi_swiglu_fwd(emi_stream_t stream, const void* a, const void* b, void* g, int64_t n, int dtype);
+int emi_swiglu_bwd(emi_stream_t stream, const void* a, const void* b, const void* dg, void* da,
+                   void* db, int64_t n, int dtype);
+
+/* Elementwise y = a + b (residual add / cotangent fan-in, Add rule
+ * HLODerivatives.td:964; test/llama.py:215,233).  y may alias a or b. */
+int emi_add(emi_stream_t stream, const void* a, const void* b, void* y, int64_t n, int dtype);
+
+/* GEMM: C[M,N] = op(A) . op(B) [+ R], fp32 accumulate, result rounded once.
+ *   trans_a == 0: A is [M,K] (lda >= K);  trans_a != 0: A is [K,M] (lda >= M)
+ *   trans_b == 0: B is [K,N] (ldb >= N);  trans_b != 0: B is [N,K] (ldb >= K)
+ * Replaces the dot_general projections of test/llama.py:149-157,211,224-233
+ * (Y = X.W^T: trans_a=0, trans_b=1) and their adjoints from the DotGeneral
+ * rule HLODerivatives.td:1166-1178 (dX = dY.W: 0,0;  dW = dY^T.X: 1,0).
+ * R (nullable, [M,N], ldr): added in the epilogue (residual add / fan-in sum).
+ * C may alias R.  Leading dimensions in elements. */
+int emi_gemm(emi_stream_t stream, const void* A, const void* B, const void* R, void* C,
+             int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldr, int64_t ldc,
+             int trans_a, int trans_b, int dtype);
+
+/* Causal softmax attention, forward.  Replaces the per-head loop of
+ * test/llama.py:178-206 with softmax of :13-18 (scale applied after the dot,
+ * max-subtracted, fp32 statistics).  Element (b, h, s, i) of q/k/v/o lives at
+ * b*stride_b + h*stride_h + s*stride_s + i.  lse: float[batch, heads, seq]
+ * = log-sum-exp of the scaled scores (saved for the adjoint). */
+int emi_attn_fwd(emi_stream_t stream, const void* q, const void* k, const void* v, void* o,
+                 float* lse, int64_t batch, int64_t heads, int64_t seq, int64_t head_dim,
+                 int64_t stride_b, int64_t stride_h, int64_t stride_s, float scale, int causal,
+                 int dtype);
+
+/* Attention adjoint: dV = P^T dO, dP = dO V^T, dS = P*(dP - rowsum(dO*O)),
+ * dQ = dS K scale, dK = dS^T Q scale; P is recomputed from q, k and lse.
+ * Rules: Exp :1182, Div :1133, Sub :1312, Reduce(max/add)
+ * StableHLOAutoDiffOpInterfaceImpl.cpp:1833-1916, DotGeneral :1166.
+ * All of q,k,v,o,dO,dq,dk,dv share the strides. */
+size_t emi_attn_bwd_workspace_bytes(int64_t batch, int64_t heads, int64_t seq, int64_t head_dim);
+int emi_attn_bwd(emi_stream_t stream, const void* q, const void* k, const void* v, const void* o,
+                 const float* lse, const void* d_o, void* dq, void* dk, void* dv, void* workspace,
+                 size_t workspace_bytes, int64_t batch, int64_t heads, int64_t seq,
+                 int64_t head_dim, int64_t stride_b, int64_t stride_h, int64_t stride_s,
+                 float scale, int causal, int dtype);
+
+/* Embedding gather x[t,:] = table[tokens[t],:] and its adjoint (scatter-add of
+ * dx rows into a zero-initialised dtable; fp32 accumulation in workspace when
+ * dtype is bf16).  The lookup is commented out in the reference
+ * (test/llama.py:109-113); adjoint per HLODerivatives.td:1022-1046.
+ * tokens: int32[n_tokens]. */
+int emi_embedding_fwd(emi_stream_t stream, const int32_t* tokens, const void* table, void* x,
+                      int64_t n_tokens, int64_t vocab, int64_t dim, int dtype);
+size_t emi_embedding_bwd_workspace_bytes(int64_t vocab, int64_t dim, int dtype);
+int emi_embedding_bwd(emi_stream_t stream, const int32_t* tokens, const void* dx, void* dtable,
+                      void* workspace, size_t workspace_bytes, int64_t n_tokens, int64_t vocab,
+                      int64_t dim, int dtype);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* EMI_H_ */

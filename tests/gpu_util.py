@@ -1,0 +1,31 @@
+"""Helpers for the GPU parity tests: move seeded numpy inputs to the device in
+the storage dtype under test, and hand the oracle the same (rounded) values."""
+import numpy as np
+import torch
+
+TOL = {"f32": 1e-4, "bf16": 2e-2}      # max relative error allowed by the parity contract
+TDTYPE = {"f32": torch.float32, "bf16": torch.bfloat16}
+
+
+def dev(a, dt):
+    """numpy -> device tensor in dtype `dt`; returns (tensor, float64 numpy of the stored values)."""
+    t = torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(TDTYPE[dt]).cuda()
+    return t, t.float().cpu().numpy().astype(np.float64)
+
+
+def host(t):
+    return t.float().cpu().numpy().astype(np.float64)
+
+
+def rel_err(got, ref):
+    got = np.asarray(got, dtype=np.float64)
+    ref = np.asarray(ref, dtype=np.float64)
+    den = float(np.max(np.abs(ref))) or 1.0
+    return float(np.max(np.abs(got - ref))) / den
+
+
+def check(got, ref, dt, what, factor=1.0):
+    e = rel_err(host(got) if isinstance(got, torch.Tensor) else got, ref)
+    assert np.all(np.isfinite(host(got) if isinstance(got, torch.Tensor) else got)), what + ": non-finite values"
+    assert e <= TOL[dt] * factor, "%s: max rel err %.3e > %.1e" % (what, e, TOL[dt] * factor)
+    return e

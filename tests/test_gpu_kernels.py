@@ -1,0 +1,224 @@
+"""GPU parity: every kernel, through the C ABI, against the CPU oracle on the
+same seeded inputs.  Tolerances are the contract's: max relative error
+(max|got-ref| / max|ref|) 1e-4 for fp32 and 2e-2 for bf16."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import llama_ref as L
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    if not torch.cuda.is_available():
+        pytest.fail("GPU tests need a GPU (run with -m 'not gpu' on CPU)")
+    from enzyme_ad.jax import ops as o
+    return o
+
+
+from gpu_util import dev, host, check, rel_err  # noqa: E402
+
+
+def _say(*a):
+    print(*a, flush=True)
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("rows,dim", [(37, 288), (5, 768), (9, 4096), (3, 8192), (7, 100), (3, 10000), (1, 8)])
+def test_rmsnorm_fwd_bwd(ops, dt, rows, dim):
+    _say("rmsnorm", dt, rows, dim)
+    rng = np.random.default_rng(rows * 1000 + dim)
+    x, xr = dev(rng.standard_normal((rows, dim)), dt)
+    g, gr = dev(rng.uniform(0.5, 1.5, dim), dt)
+    dy, dyr = dev(rng.standard_normal((rows, dim)), dt)
+    add, addr = dev(rng.standard_normal((rows, dim)), dt)
+    y = ops.rmsnorm(x, g)
+    check(y, L.rmsnorm_fwd(xr, gr), dt, "rmsnorm fwd")
+    with ops.Tape() as tape:
+        y = ops.rmsnorm(x, g)
+    dx, dg = tape.backward([y], [dy], [x, g])
+    rdx, rdg = L.rmsnorm_bwd(xr, gr, dyr)
+    check(dx, rdx, dt, "rmsnorm dx")
+    check(dg, rdg, dt, "rmsnorm dgamma")
+    # fused residual-cotangent add
+    with ops.Tape() as tape:
+        y = ops.rmsnorm(x, g)
+        z = ops.add(y, x)
+    dx2, _ = tape.backward([z], [dy], [x, g])
+    check(dx2, rdx + dyr, dt, "rmsnorm dx + residual")
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("B,S,h,d", [(2, 33, 6, 48), (1, 128, 4, 128), (2, 17, 3, 64), (1, 9, 2, 6)])
+def test_rope_fwd_bwd(ops, dt, B, S, h, d):
+    _say("rope", dt, B, S, h, d)
+    rng = np.random.default_rng(S * 100 + d)
+    x, xr = dev(rng.standard_normal((B, S, h * d)), dt)
+    cos, sin = L.rope_angles(S, d)
+    y = ops.rope(x, h)
+    check(y, L.rope_fwd(xr.reshape(B, S, h, d), cos, sin).reshape(B, S, h * d), dt, "rope fwd")
+    dy, dyr = dev(rng.standard_normal((B, S, h * d)), dt)
+    with ops.Tape() as tape:
+        y = ops.rope(x, h)
+    (dx,) = tape.backward([y], [dy], [x])
+    check(dx, L.rope_bwd(dyr.reshape(B, S, h, d), cos, sin).reshape(B, S, h * d), dt, "rope bwd")
+    # the table itself: float64 angles rounded to fp32
+    tab = host(ops.rope_table(S, d))
+    assert np.max(np.abs(tab[..., 0] - cos)) < 1e-7 and np.max(np.abs(tab[..., 1] - sin)) < 1e-7
+
+
+def test_rope_large_positions_fp32(ops):
+    """Angles up to ~4095 rad: fp32 angle arithmetic would lose 1e-4; the table is made in float64."""
+    B, S, h, d = 1, 4096, 1, 128
+    rng = np.random.default_rng(0)
+    x, xr = dev(rng.standard_normal((B, S, h * d)), "f32")
+    cos, sin = L.rope_angles(S, d)
+    check(ops.rope(x, h), L.rope_fwd(xr.reshape(B, S, h, d), cos, sin).reshape(B, S, h * d), "f32", "rope S=4096", 0.1)
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("n", [8, 1003, 4096 * 3 + 5])
+def test_swiglu_and_add(ops, dt, n):
+    _say("swiglu", dt, n)
+    rng = np.random.default_rng(n)
+    a, ar = dev(rng.standard_normal(n) * 3, dt)
+    b, br = dev(rng.standard_normal(n), dt)
+    dg, dgr = dev(rng.standard_normal(n), dt)
+    check(ops.swiglu(a, b), L.swiglu_fwd(ar, br), dt, "swiglu fwd")
+    with ops.Tape() as tape:
+        g = ops.swiglu(a, b)
+    da, db = tape.backward([g], [dg], [a, b])
+    rda, rdb = L.swiglu_bwd(ar, br, dgr)
+    check(da, rda, dt, "swiglu da")
+    check(db, rdb, dt, "swiglu db")
+    check(ops.add(a, b), ar + br, dt, "add")
+
+
+GEMM_SHAPES = [
+    (37, 29, 19),        # generic path (nothing aligned)
+    (256, 384, 320),     # fast path, 128-tiles, K not a multiple of 64
+    (200, 136, 72),      # fast path, ragged tiles
+    (64, 288, 288),      # C1 projection
+    (4096, 3072, 264),   # fast path, 256-tiles (192 tiles)
+    (4000, 3080, 128),   # 256-tiles, ragged M and N
+]
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("ta,tb", [(0, 1), (0, 0), (1, 0), (1, 1)])
+@pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
+def test_gemm_layouts(ops, dt, ta, tb, M, N, K):
+    _say("gemm", dt, ta, tb, M, N, K)
+    if dt == "f32" and M * N * K > 5e8:
+        pytest.skip("large shape covered in bf16 only (fp32 path is the generic kernel)")
+    rng = np.random.default_rng(M + N + K + ta * 2 + tb)
+    A = rng.standard_normal((K, M) if ta else (M, K))
+    B = rng.standard_normal((N, K) if tb else (K, N))
+    R = rng.standard_normal((M, N))
+    a, ar = dev(A, dt)
+    b, br = dev(B, dt)
+    r, rr = dev(R, dt)
+    ref = (ar.T if ta else ar) @ (br.T if tb else br)
+    check(ops.gemm(a, b, bool(ta), bool(tb)), ref, dt, "gemm")
+    check(ops.gemm(a, b, bool(ta), bool(tb), r), ref + rr, dt, "gemm + residual")
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+def test_matmul_nt_vjp(ops, dt):
+    rng = np.random.default_rng(3)
+    x, xr = dev(rng.standard_normal((2, 65, 136)), dt)
+    w, wr = dev(rng.standard_normal((200, 136)) * 0.1, dt)
+    dy, dyr = dev(rng.standard_normal((2, 65, 200)), dt)
+    with ops.Tape() as tape:
+        y = ops.matmul_nt(x, w)
+    check(y, L.linear_fwd(xr, wr), dt, "linear fwd")
+    dx, dw = tape.backward([y], [dy], [x, w])
+    rdx, rdw = L.linear_bwd(xr, wr, dyr)
+    check(dx, rdx, dt, "linear dX")
+    check(dw, rdw, dt, "linear dW")
+
+
+ATTN_CASES = [
+    ("f32", 2, 6, 100, 48, "bshd"),     # C1 head shape, generic path
+    ("f32", 1, 2, 64, 128, "bhsd"),
+    ("bf16", 1, 3, 70, 48, "bshd"),     # bf16 on the generic path
+    ("bf16", 2, 2, 256, 128, "bhsd"),   # MFMA path
+    ("bf16", 1, 2, 200, 128, "bshd"),   # MFMA, ragged sequence, token-major strides
+    ("bf16", 2, 3, 320, 64, "bshd"),    # MFMA, head_dim 64
+    ("bf16", 1, 1, 1, 128, "bhsd"),     # single position: out = v
+    ("bf16", 1, 2, 130, 64, "bhsd"),
+]
+
+
+@pytest.mark.parametrize("dt,B,h,S,d,layout", ATTN_CASES)
+@pytest.mark.parametrize("causal", [True, False])
+def test_attention_fwd_bwd(ops, dt, B, h, S, d, layout, causal):
+    _say("attention", dt, B, h, S, d, layout, causal)
+    rng = np.random.default_rng(S * 10 + d + B)
+    shp = (B, h, S, d)
+    arrs = [rng.standard_normal(shp) for _ in range(4)]
+
+    def put(a):
+        if layout == "bshd":
+            t, r = dev(a.transpose(0, 2, 1, 3).reshape(B, S, h * d), dt)
+            return t, r.reshape(B, S, h, d).transpose(0, 2, 1, 3)
+        return dev(a, dt)
+
+    def get(t):
+        a = host(t)
+        return a.reshape(B, S, h, d).transpose(0, 2, 1, 3) if layout == "bshd" else a
+
+    (q, qr), (k, kr), (v, vr), (do, dor) = (put(a) for a in arrs)
+    with ops.Tape() as tape:
+        o = ops.attention(q, k, v, h, causal=causal, layout=layout)
+    ro, rlse = L.attention_fwd(qr, kr, vr, causal=causal)
+    check(get(o), ro, dt, "attention out")
+    dq, dk, dv = tape.backward([o], [do], [q, k, v])
+    rdq, rdk, rdv = L.attention_bwd(qr, kr, vr, dor, causal=causal)
+    check(get(dq), rdq, dt, "attention dq")
+    check(get(dk), rdk, dt, "attention dk")
+    check(get(dv), rdv, dt, "attention dv")
+
+
+def test_attention_lse(ops):
+    B, h, S, d = 1, 2, 192, 128
+    rng = np.random.default_rng(1)
+    (q, qr), (k, kr), (v, vr) = (dev(rng.standard_normal((B, h, S, d)), "bf16") for _ in range(3))
+    o, lse, _ = ops.attention_raw(q, k, v, h, 1.0 / np.sqrt(d), True, "bhsd")
+    _, rlse = L.attention_fwd(qr, kr, vr)
+    assert np.max(np.abs(host(lse) - rlse)) < 2e-2
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+def test_embedding(ops, dt):
+    rng = np.random.default_rng(2)
+    V, D = 50, 24
+    tab, tabr = dev(rng.standard_normal((V, D)), dt)
+    tok = rng.integers(0, V, size=(2, 31))
+    tok[0, :5] = 7                                        # collisions
+    tt = torch.from_numpy(tok.astype(np.int32)).cuda()
+    dx, dxr = dev(rng.standard_normal((2, 31, D)), dt)
+    with ops.Tape() as tape:
+        x = ops.embedding(tt, tab)
+    assert np.array_equal(host(x), tabr[tok])              # a gather is exact
+    (dtab,) = tape.backward([x], [dx], [tab])
+    ref = np.zeros((V, D))
+    np.add.at(ref, tok.reshape(-1), dxr.reshape(-1, D))
+    check(dtab, ref, dt, "embedding scatter-add")
+
+
+def test_error_paths_do_not_launch(ops):
+    from enzyme_ad.jax import _native as N
+    lib = N.lib()
+    x = torch.zeros(16, device="cuda")
+    assert lib.emi_rmsnorm_fwd(None, x.data_ptr(), x.data_ptr(), x.data_ptr(), 2, 8, 1e-5, 99) == 3
+    assert b"dtype" in lib.emi_last_error()
+    assert lib.emi_gemm(None, x.data_ptr(), x.data_ptr(), None, x.data_ptr(), 2, 2, 4, 1, 2, 2, 2, 0, 0, 11) == 3
+    assert b"leading dimension" in lib.emi_last_error()
+    assert lib.emi_attn_bwd(None, *([x.data_ptr()] * 9), None, 0, 1, 1, 4, 4, 16, 16, 4, 1.0, 1, 11) == 3
+    assert b"workspace" in lib.emi_last_error()
+    with pytest.raises(RuntimeError):
+        ops.add(torch.zeros(4), torch.zeros(4))            # host memory is refused, never computed on CPU
+    torch.cuda.synchronize()
