@@ -310,7 +310,7 @@ __device__ __forceinline__ int acc_row(int r, int lane) { return 8 * (r >> 2) + 
 // Forward: block = 4 waves x 32 queries, KV tiles of 64 keys.
 // ---------------------------------------------------------------------------
 template <int D>
-__global__ __launch_bounds__(256) void attn_fwd_bf16_kernel(const uint16_t* __restrict__ q,
+__global__ __launch_bounds__(256, 2) void attn_fwd_bf16_kernel(const uint16_t* __restrict__ q,
                                                             const uint16_t* __restrict__ k,
                                                             const uint16_t* __restrict__ v, uint16_t* __restrict__ o,
                                                             float* __restrict__ lse, AttnShape sh, uint32_t head_bytes,
@@ -373,23 +373,21 @@ __global__ __launch_bounds__(256) void attn_fwd_bf16_kernel(const uint16_t* __re
       for (int T = 0; T < 2; T++)
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-          float x = s[T][r] * scale_log2e;
           if (need_mask) {
             const int key = key0 + T * 32 + acc_row(r, lane);
-            if ((causal && key > qrow) || key >= seq) x = kNegBig;
+            if ((causal && key > qrow) || key >= seq) s[T][r] = kNegBig;
           }
-          s[T][r] = x;
-          mt = fmaxf(mt, x);
+          mt = fmaxf(mt, s[T][r]);
         }
       mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
-      const float m_new = fmaxf(m, mt);
+      const float m_new = fmaxf(m, mt * scale_log2e);      // running max in the scaled log2 domain
       const float alpha = fast_exp2(m - m_new);
       float rs = 0.f;
 #pragma unroll
       for (int T = 0; T < 2; T++)
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-          const float p = fast_exp2(s[T][r] - m_new);
+          const float p = fast_exp2(fmaf(s[T][r], scale_log2e, -m_new));
           s[T][r] = p;
           rs += p;
         }
@@ -437,7 +435,7 @@ __global__ __launch_bounds__(256) void attn_fwd_bf16_kernel(const uint16_t* __re
 //   S^T = K Q^T, dP^T = V dO^T, dS^T = P^T (dP^T - delta), dQ^T = K^T dS^T
 // ---------------------------------------------------------------------------
 template <int D>
-__global__ __launch_bounds__(256) void attn_bwd_dq_bf16_kernel(const uint16_t* __restrict__ q,
+__global__ __launch_bounds__(256, 2) void attn_bwd_dq_bf16_kernel(const uint16_t* __restrict__ q,
                                                                const uint16_t* __restrict__ k,
                                                                const uint16_t* __restrict__ v,
                                                                const uint16_t* __restrict__ d_o,

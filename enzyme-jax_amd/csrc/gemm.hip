@@ -13,6 +13,8 @@
 //   TN  dW = dY^T . X   (A k-major,      B k-major)        weight adjoint
 // Generic path (fp32, or bf16 with shapes/alignments the fast path does not
 // take): v_mfma_f32_32x32x2_f32 with predicated scalar loads.
+#include <stdlib.h>
+
 #include "emi_device.h"
 
 namespace emi {
@@ -21,6 +23,8 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 
 #define EMI_LDS __attribute__((address_space(3)))
 
@@ -50,32 +54,44 @@ __device__ __forceinline__ void tile_coords(int tiles_m, int tiles_n, int* tm, i
 }
 
 // --- LDS tile layouts -------------------------------------------------------
-// k-contiguous operand tile: [rows][64 k] bf16, 128-byte rows, 16-byte chunk c
-// of row r stored at chunk c ^ (r & 7).
-// k-major operand tile: [64 k][COLS] bf16, chunk c of row k stored at chunk
-// c ^ (4 * (k & 3)).
+// The LDS serves 256 bytes (64 banks) per clock: 16 lanes of a ds_read_b128.
+// k-contiguous operand tile: [rows][BK] bf16.  Rows are 2*BK bytes, so 256/(2*BK)
+// rows share one 256-byte bank line; 16-byte chunk c of row r is stored at chunk
+// c ^ swz_kc(r), which spreads 16 consecutive rows at one logical chunk (one
+// MFMA operand fetch) over all 16 slots of the line.
+// k-major operand tile: [BK][COLS] bf16 (COLS*2-byte rows, a multiple of 256):
+// chunk c of row k is stored at chunk c ^ (4 * (k & 3)), which does the same for
+// the 4 rows x 64 bytes that 32 lanes of a transposing ds_read_b64_tr_b16 touch.
 
-template <int ROWS, int NW>
+template <int BK> __device__ __forceinline__ int swz_kc(int row) {
+  static_assert(BK == 64 || BK == 32, "BK");
+  return BK == 64 ? ((row >> 1) & 7) : ((row >> 2) & 3);
+}
+
+template <int ROWS, int BK, int NW>
 __device__ __forceinline__ void load_tile_kcontig(__amdgpu_buffer_rsrc_t rsrc, EMI_LDS uint8_t* lds, int wave, int lane,
                                                   uint32_t row0_off_bytes, int ld, int k0, int K) {
-  constexpr int NLOAD = ROWS / 8 / NW;
-  const int r_in = lane >> 3, pc = lane & 7;
-  const int lc = pc ^ r_in;
-  const int k = k0 + lc * 8;
+  constexpr int CPR = BK / 8;                 // 16-byte chunks per row
+  constexpr int RPW = 64 / CPR;               // rows per 1 KiB wave-load
+  constexpr int NLOAD = ROWS / RPW / NW;
+  static_assert(NLOAD >= 1, "tile smaller than one pass of the block");
+  const int r_in = lane / CPR, pc = lane % CPR;
 #pragma unroll
   for (int it = 0; it < NLOAD; it++) {
-    const int r = (it * NW + wave) * 8 + r_in;
+    const int r = (it * NW + wave) * RPW + r_in;
+    const int lc = pc ^ swz_kc<BK>(r);
+    const int k = k0 + lc * 8;
     uint32_t voff = row0_off_bytes + (uint32_t)(r * ld + k) * 2u;
     if (k >= K) voff = kOob;
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, lds + (it * NW + wave) * 1024, 16, voff, 0, 0, 0);
   }
 }
 
-template <int COLS, int NW>
+template <int COLS, int BK, int NW>
 __device__ __forceinline__ void load_tile_kmajor(__amdgpu_buffer_rsrc_t rsrc, EMI_LDS uint8_t* lds, int wave, int lane,
                                                  int col0, int ncols, int ld, int k0, int K) {
-  constexpr int CPR = COLS / 8;              // 16-byte chunks per k-row
-  constexpr int NLOAD = CPR / NW;            // 64 rows * CPR chunks / (64 lanes * NW waves)
+  constexpr int CPR = COLS / 8;               // 16-byte chunks per k-row
+  constexpr int NLOAD = BK * CPR / 64 / NW;
   static_assert(CPR >= 16 && NLOAD >= 1, "k-major tile too narrow");
 #pragma unroll
   for (int it = 0; it < NLOAD; it++) {
@@ -89,12 +105,13 @@ __device__ __forceinline__ void load_tile_kmajor(__amdgpu_buffer_rsrc_t rsrc, EM
   }
 }
 
-// MFMA operand fragment (32 rows x 16 k) for k-step kk of the 64-k tile.
+// MFMA operand fragment (32 rows x 16 k) for k-step kk of the tile.
 // Lane l holds row (l & 31), k = 8*(l >> 5) + 0..7 of the step.
+template <int BK>
 __device__ __forceinline__ bf16x8_t frag_kcontig(const EMI_LDS uint8_t* tile, int row_base, int kk, int lane) {
   const int row = row_base + (lane & 31);
-  const int chunk = (kk * 2 + (lane >> 5)) ^ (row & 7);
-  return *reinterpret_cast<const EMI_LDS bf16x8_t*>(tile + row * 128 + chunk * 16);
+  const int chunk = (kk * 2 + (lane >> 5)) ^ swz_kc<BK>(row);
+  return *reinterpret_cast<const EMI_LDS bf16x8_t*>(tile + row * (BK * 2) + chunk * 16);
 }
 
 // Same fragment out of a k-major tile with two transposing loads.  Within a
@@ -113,15 +130,31 @@ __device__ __forceinline__ bf16x8_t frag_kmajor(const EMI_LDS uint8_t* tile, int
   return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
-template <int BM, int BN, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR>
+// s_waitcnt vmcnt(N) with the other counters left alone.
+template <int N> __device__ __forceinline__ void wait_vmcnt() {
+  static_assert(N >= 0 && N < 64, "vmcnt");
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | 0x0f70);
+}
+
+// Software pipeline, NSTAGE == 2: tile t+1 streams into the other LDS stage while
+// tile t is multiplied; one barrier per tile.
+// NSTAGE == 4: tiles t+2 and t+3 are in flight while tile t is multiplied and
+// tile t+1 has already landed, so the operand fragments of the first k-step of
+// tile t+1 are fetched before the barrier and the MFMA stream never waits on LDS.
+// Loads past the end of K are still issued (they read as zeros) so that the
+// number of outstanding loads is a compile-time constant.
+template <int BM, int BN, int BK, int NSTAGE, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_kernel(const uint16_t* __restrict__ A,
                                                                  const uint16_t* __restrict__ B, const uint16_t* R,
                                                                  uint16_t* C, int M, int N, int K, int lda, int ldb,
-                                                                 int ldr, int ldc, uint32_t a_bytes, uint32_t b_bytes) {
+                                                                 int ldr, int ldc, uint32_t a_bytes, uint32_t b_bytes,
+                                                                 int vec_ok) {
   constexpr int NW = WM * WN;
-  constexpr int BK = 64;
+  constexpr int KS = BK / 16;
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
   constexpr int A_BYTES = BM * BK * 2, B_BYTES = BN * BK * 2, STAGE = A_BYTES + B_BYTES;
+  constexpr int LPT = (A_BYTES + B_BYTES) / 1024 / NW;      // direct-to-LDS loads per wave per tile
+  static_assert(NSTAGE == 2 || NSTAGE == 4, "NSTAGE");
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem_raw[];
   EMI_LDS uint8_t* smem = (EMI_LDS uint8_t*)smem_raw;
 
@@ -141,13 +174,13 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_kernel(const uint16_t* 
     EMI_LDS uint8_t* sA = smem + stage * STAGE;
     EMI_LDS uint8_t* sB = sA + A_BYTES;
     if constexpr (A_KMAJOR)
-      load_tile_kmajor<BM, NW>(rA, sA, wave, lane, m0, M, lda, k0, K);
+      load_tile_kmajor<BM, BK, NW>(rA, sA, wave, lane, m0, M, lda, k0, K);
     else
-      load_tile_kcontig<BM, NW>(rA, sA, wave, lane, (uint32_t)m0 * (uint32_t)lda * 2u, lda, k0, K);
+      load_tile_kcontig<BM, BK, NW>(rA, sA, wave, lane, (uint32_t)m0 * (uint32_t)lda * 2u, lda, k0, K);
     if constexpr (B_KMAJOR)
-      load_tile_kmajor<BN, NW>(rB, sB, wave, lane, n0, N, ldb, k0, K);
+      load_tile_kmajor<BN, BK, NW>(rB, sB, wave, lane, n0, N, ldb, k0, K);
     else
-      load_tile_kcontig<BN, NW>(rB, sB, wave, lane, (uint32_t)n0 * (uint32_t)ldb * 2u, ldb, k0, K);
+      load_tile_kcontig<BN, BK, NW>(rB, sB, wave, lane, (uint32_t)n0 * (uint32_t)ldb * 2u, ldb, k0, K);
   };
 
   f32x16_t acc[TM][TN];
@@ -158,56 +191,153 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_kernel(const uint16_t* 
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-  const int nk = (K + BK - 1) / BK;
-  issue_loads(0, 0);
-  __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0)
-  __syncthreads();
-
-  for (int t = 0; t < nk; t++) {
-    if (t + 1 < nk) issue_loads((t + 1) & 1, (t + 1) * BK);
-    const EMI_LDS uint8_t* sA = smem + (t & 1) * STAGE;
+  auto load_frags = [&](int stage, int kk, bf16x8_t (&a)[TM], bf16x8_t (&b)[TN]) {
+    const EMI_LDS uint8_t* sA = smem + stage * STAGE;
     const EMI_LDS uint8_t* sB = sA + A_BYTES;
 #pragma unroll
-    for (int kk = 0; kk < 4; kk++) {
-      bf16x8_t a[TM], b[TN];
-#pragma unroll
-      for (int i = 0; i < TM; i++) {
-        const int base = wm * (BM / WM) + i * 32;
-        if constexpr (A_KMAJOR) a[i] = frag_kmajor<BM>(sA, base, kk, lane);
-        else a[i] = frag_kcontig(sA, base, kk, lane);
-      }
-#pragma unroll
-      for (int j = 0; j < TN; j++) {
-        const int base = wn * (BN / WN) + j * 32;
-        if constexpr (B_KMAJOR) b[j] = frag_kmajor<BN>(sB, base, kk, lane);
-        else b[j] = frag_kcontig(sB, base, kk, lane);
-      }
-#pragma unroll
-      for (int i = 0; i < TM; i++)
-#pragma unroll
-        for (int j = 0; j < TN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+    for (int i = 0; i < TM; i++) {
+      const int base = wm * (BM / WM) + i * 32;
+      if constexpr (A_KMAJOR) a[i] = frag_kmajor<BM>(sA, base, kk, lane);
+      else a[i] = frag_kcontig<BK>(sA, base, kk, lane);
     }
-    __builtin_amdgcn_s_waitcnt(0x0f70);   // next stage has landed
-    __syncthreads();                      // and everyone is done reading this one
-  }
-
-  // Epilogue.  Accumulator register r of lane l is C[8*(r/4) + 4*(l/32) + r%4][l%32].
-  const int col_l = lane & 31, row_l = (lane >> 5) * 4;
-#pragma unroll
-  for (int i = 0; i < TM; i++) {
 #pragma unroll
     for (int j = 0; j < TN; j++) {
-      const int col = n0 + wn * (BN / WN) + j * 32 + col_l;
-      if (col < N) {
+      const int base = wn * (BN / WN) + j * 32;
+      if constexpr (B_KMAJOR) b[j] = frag_kmajor<BN>(sB, base, kk, lane);
+      else b[j] = frag_kcontig<BK>(sB, base, kk, lane);
+    }
+  };
+  // The MFMA operands are passed swapped (B fragment first): see the epilogue.
+  auto mfma_step = [&](const bf16x8_t (&a)[TM], const bf16x8_t (&b)[TN]) {
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-          const int row = m0 + wm * (BM / WM) + i * 32 + (r >> 2) * 8 + row_l + (r & 3);
-          if (row < M) {
-            float v = acc[i][j][r];
-            if (R != nullptr) v += bf16_bits_to_f32(R[(int64_t)row * ldr + col]);
-            C[(int64_t)row * ldc + col] = f32_to_bf16_bits(v);
-          }
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int j = 0; j < TN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[j], a[i], acc[i][j], 0, 0, 0);
+  };
+
+  const int nk = (K + BK - 1) / BK;
+  // Operand fragments are double buffered: the LDS reads of the next k-step are
+  // issued before the MFMAs of the current one so their latency hides behind them.
+  bf16x8_t fa[2][TM], fb[2][TN];
+  if constexpr (NSTAGE == 2) {
+    issue_loads(0, 0);
+    wait_vmcnt<0>();
+    __syncthreads();
+    for (int t = 0; t < nk; t++) {
+      if (t + 1 < nk) issue_loads((t + 1) & 1, (t + 1) * BK);
+      load_frags(t & 1, 0, fa[0], fb[0]);
+#pragma unroll
+      for (int kk = 0; kk < KS; kk++) {
+        if (kk + 1 < KS) load_frags(t & 1, kk + 1, fa[(kk + 1) & 1], fb[(kk + 1) & 1]);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_step(fa[kk & 1], fb[kk & 1]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      wait_vmcnt<0>();     // next stage has landed
+      __syncthreads();     // and everyone is done reading this one
+    }
+  } else {
+    static_assert(KS % 2 == 0, "fragment double buffering assumes an even number of k-steps per tile");
+    issue_loads(0, 0);
+    issue_loads(1, BK);
+    issue_loads(2, 2 * BK);
+    wait_vmcnt<LPT>();     // tiles 0 and 1 have landed
+    __syncthreads();
+    load_frags(0, 0, fa[0], fb[0]);
+    for (int t = 0; t < nk; t++) {
+      issue_loads((t + 3) & 3, (t + 3) * BK);
+#pragma unroll
+      for (int kk = 0; kk < KS; kk++) {
+        if (kk + 1 < KS) load_frags(t & 3, kk + 1, fa[(kk + 1) & 1], fb[(kk + 1) & 1]);
+        else load_frags((t + 1) & 3, 0, fa[0], fb[0]);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_step(fa[kk & 1], fb[kk & 1]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      wait_vmcnt<LPT>();   // everything but the newest tile (t+3) has landed: tiles <= t+2
+      __syncthreads();     // visible to all; tile t's stage may be refilled next iteration
+    }
+    wait_vmcnt<0>();       // drain the zero-filled loads past the end of K before LDS is reused
+    __syncthreads();
+  }
+
+  // Epilogue.  With swapped MFMA operands register r of lane l holds
+  // C[row = l%32][col = 8*(r/4) + 4*(l/32) + r%4] of its 32x32 tile: four
+  // consecutive columns per register quad.  Each wave stages its (BM/WM) x
+  // (BN/WN) sub-tile through its own slice of the now idle LDS as bf16 and writes
+  // it out with 16-byte, row-contiguous stores; the residual comes in the same way
+  // (16-byte loads -> LDS -> accumulator layout) and is added in fp32 before the
+  // single rounding.  Slice layout: rows of 2*WC bytes, chunk c of row r at chunk
+  // c ^ e_swz(r), the two 8-byte halves of a chunk swapped when (r>>4)&1, which
+  // makes the 8-byte column-quad accesses of 32 lanes (32 rows) conflict free.
+  constexpr int WR = BM / WM, WC = BN / WN;
+  static_assert(WC == 64 || WC == 128, "epilogue supports 64- or 128-column wave tiles");
+  static_assert(NW * WR * WC * 2 <= NSTAGE * STAGE, "epilogue staging does not fit in the LDS allocation");
+  constexpr int RSB = WC * 2, CH = WC / 8, RPP = 64 / CH;     // row bytes, chunks per row, rows per 64-lane pass
+  EMI_LDS uint8_t* wl = smem + wave * (WR * RSB);
+  const int lrow = lane & 31, lhalf = lane >> 5;
+  const int rbase = m0 + wm * WR, cbase = n0 + wn * WC;
+  auto e_swz = [](int row) { return WC == 64 ? ((row >> 1) & 7) : (row & 15); };
+  auto quad_slot = [&](int row, int chunk) {
+    return row * RSB + ((chunk ^ e_swz(row)) << 4) + ((lhalf ^ ((row >> 4) & 1)) << 3);
+  };
+  if (R != nullptr) {
+#pragma unroll
+    for (int it = 0; it < WR / RPP; it++) {
+      const int row = it * RPP + lane / CH, c = lane % CH;
+      const int grow = rbase + row, gcol = cbase + c * 8;
+      u32x4_t v = {0u, 0u, 0u, 0u};
+      if (grow < M && gcol < N) {
+        const uint16_t* src = R + (int64_t)grow * ldr + gcol;
+        if (vec_ok && gcol + 8 <= N) {
+          v = *reinterpret_cast<const u32x4_t*>(src);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; e++)
+            if (gcol + e < N) v[e >> 1] |= (uint32_t)src[e] << ((e & 1) * 16);
         }
+      }
+      if ((row >> 4) & 1) v = __builtin_shufflevector(v, v, 2, 3, 0, 1);
+      *reinterpret_cast<EMI_LDS u32x4_t*>(wl + row * RSB + ((c ^ e_swz(row)) << 4)) = v;
+    }
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int j = 0; j < TN; j++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          const u32x2_t w = *reinterpret_cast<const EMI_LDS u32x2_t*>(wl + quad_slot(i * 32 + lrow, j * 4 + q));
+          acc[i][j][4 * q + 0] += __uint_as_float(w[0] << 16);
+          acc[i][j][4 * q + 1] += __uint_as_float(w[0] & 0xffff0000u);
+          acc[i][j][4 * q + 2] += __uint_as_float(w[1] << 16);
+          acc[i][j][4 * q + 3] += __uint_as_float(w[1] & 0xffff0000u);
+        }
+  }
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        u32x2_t w;
+        w[0] = pack_bf16x2(acc[i][j][4 * q + 0], acc[i][j][4 * q + 1]);
+        w[1] = pack_bf16x2(acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+        *reinterpret_cast<EMI_LDS u32x2_t*>(wl + quad_slot(i * 32 + lrow, j * 4 + q)) = w;
+      }
+#pragma unroll
+  for (int it = 0; it < WR / RPP; it++) {
+    const int row = it * RPP + lane / CH, c = lane % CH;
+    const int grow = rbase + row, gcol = cbase + c * 8;
+    u32x4_t v = *reinterpret_cast<const EMI_LDS u32x4_t*>(wl + row * RSB + ((c ^ e_swz(row)) << 4));
+    if ((row >> 4) & 1) v = __builtin_shufflevector(v, v, 2, 3, 0, 1);
+    if (grow < M && gcol < N) {
+      uint16_t* dst = C + (int64_t)grow * ldc + gcol;
+      if (vec_ok && gcol + 8 <= N) {
+        *reinterpret_cast<u32x4_t*>(dst) = v;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; e++)
+          if (gcol + e < N) dst[e] = (uint16_t)(v[e >> 1] >> ((e & 1) * 16));
       }
     }
   }
@@ -289,11 +419,15 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const T* __restrict__
     }
 }
 
-template <int BM, int BN, int WM, int WN, bool AK, bool BK_>
+template <int BM, int BN, int BK, int NSTAGE, int WM, int WN, bool AK, bool BKM>
 static int launch_bf16(hipStream_t st, const void* A, const void* B, const void* R, void* C, int M, int N, int K, int lda,
                        int ldb, int ldr, int ldc, uint32_t a_bytes, uint32_t b_bytes) {
-  auto kern = gemm_bf16_kernel<BM, BN, WM, WN, AK, BK_>;
-  constexpr int smem = 2 * (BM + BN) * 64 * 2;
+  // 16-byte epilogue accesses need aligned rows of C (and R)
+  const int vec_ok = ((reinterpret_cast<uintptr_t>(C) & 15) == 0 && ldc % 8 == 0 &&
+                      (R == nullptr || ((reinterpret_cast<uintptr_t>(R) & 15) == 0 && ldr % 8 == 0)))
+                         ? 1 : 0;
+  auto kern = gemm_bf16_kernel<BM, BN, BK, NSTAGE, WM, WN, AK, BKM>;
+  constexpr int smem = NSTAGE * (BM + BN) * BK * 2;
   static bool configured = false;   // idempotent; a race only repeats the call
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
@@ -303,19 +437,40 @@ static int launch_bf16(hipStream_t st, const void* A, const void* B, const void*
   const int tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
   hipLaunchKernelGGL(kern, dim3(tiles), dim3(WM * WN * 64), smem, st, static_cast<const uint16_t*>(A),
                      static_cast<const uint16_t*>(B), static_cast<const uint16_t*>(R), static_cast<uint16_t*>(C), M, N, K,
-                     lda, ldb, ldr, ldc, a_bytes, b_bytes);
+                     lda, ldb, ldr, ldc, a_bytes, b_bytes, vec_ok);
   EMI_CHECK_LAUNCH("emi_gemm");
   return EMI_OK;
 }
 
-template <bool AK, bool BK_>
+// Tile configuration.  EMI_GEMM_TILE (read once) overrides the choice for tuning:
+//   0 = automatic, 1 = 256x256x64 2-stage 8 waves, 2 = 256x256x32 4-stage 4 waves,
+//   3 = 256x256x32 4-stage 8 waves, 4 = 128x128x64 2-stage 4 waves.
+static int tile_override() {
+  static int v = -1;
+  if (v < 0) {
+    const char* e = getenv("EMI_GEMM_TILE");
+    v = e ? atoi(e) : 0;
+  }
+  return v;
+}
+
+template <bool AK, bool BKM>
 static int launch_bf16_layout(hipStream_t st, const void* A, const void* B, const void* R, void* C, int M, int N, int K,
                               int lda, int ldb, int ldr, int ldc, uint32_t a_bytes, uint32_t b_bytes) {
-  // 256x256 tiles when they fill the chip, else 128x128.
-  const int64_t big_tiles = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
-  if (big_tiles >= 192)
-    return launch_bf16<256, 256, 2, 4, AK, BK_>(st, A, B, R, C, M, N, K, lda, ldb, ldr, ldc, a_bytes, b_bytes);
-  return launch_bf16<128, 128, 2, 2, AK, BK_>(st, A, B, R, C, M, N, K, lda, ldb, ldr, ldc, a_bytes, b_bytes);
+  int cfg = tile_override();
+  if (cfg == 0) {
+    // 256x256 tiles when they fill the chip, else 128x128.
+    const int64_t big_tiles = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
+    cfg = big_tiles >= 192 ? 1 : 4;
+  }
+#define EMI_GEMM_ARGS st, A, B, R, C, M, N, K, lda, ldb, ldr, ldc, a_bytes, b_bytes
+  switch (cfg) {
+    case 1: return launch_bf16<256, 256, 64, 2, 2, 4, AK, BKM>(EMI_GEMM_ARGS);
+    case 2: return launch_bf16<256, 256, 32, 4, 2, 2, AK, BKM>(EMI_GEMM_ARGS);
+    case 3: return launch_bf16<256, 256, 32, 4, 2, 4, AK, BKM>(EMI_GEMM_ARGS);
+    default: return launch_bf16<128, 128, 64, 2, 2, 2, AK, BKM>(EMI_GEMM_ARGS);
+  }
+#undef EMI_GEMM_ARGS
 }
 
 template <typename T>
