@@ -1,0 +1,178 @@
+"""CPU-only checks of the drop-in boundary: the C-ABI library loads and exports
+every symbol the headers declare; XLA-FFI handlers answer the metadata probe,
+ignore non-execute stages and reject malformed call frames without launching;
+the Python surface mirrors the reference's enzyme_ad.jax names."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+import ffi_frames as F
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _lib():
+    from enzyme_ad.jax import _native
+    return _native.lib()
+
+
+def _declared(header):
+    text = open(os.path.join(ROOT, "include", header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(emi_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib()
+    names = _declared("emi.h") + _declared("emi_ffi.h")
+    assert len(names) >= 30
+    for n in names:
+        assert hasattr(lib, n), "libemi_hip.so does not export " + n
+    assert lib.emi_abi_version() == 1
+    from enzyme_ad.jax import _native
+    assert set(_native.SIGNATURES) == set(_declared("emi.h"))      # the ctypes table covers emi.h exactly
+
+
+def test_plain_launchers_reject_bad_arguments_before_touching_the_gpu():
+    lib = _lib()
+    assert lib.emi_rmsnorm_fwd(None, 16, 16, 16, 4, 8, 1e-5, 10) == 3          # f16 is not supported
+    assert b"dtype" in lib.emi_last_error()
+    assert lib.emi_rmsnorm_fwd(None, None, 16, 16, 4, 8, 1e-5, 11) == 3
+    assert b"null" in lib.emi_last_error()
+    assert lib.emi_rope(None, 16, 16, 16, 1, 4, 2, 7, 0, 11) == 3             # odd head_dim
+    assert lib.emi_gemm(None, 16, 16, None, 16, 4, 4, -1, 4, 4, 4, 4, 0, 1, 16) == 3
+    assert lib.emi_attn_fwd(None, 16, 16, 16, 16, 16, 1, 1, 8, 512, 4096, 4096, 512, 1.0, 1, 16) == 3
+    assert b"head_dim" in lib.emi_last_error()
+    assert lib.emi_swiglu_fwd(None, 8, 16, 16, 64, 11) == 3                    # misaligned pointer
+    assert lib.emi_rmsnorm_bwd_workspace_bytes(32768, 4096) == 2048 * 4096 * 4
+
+
+def _handler(name):
+    lib = _lib()
+    fn = getattr(lib, name)
+    fn.restype, fn.argtypes = C.c_void_p, [C.POINTER(F.CallFrame)]
+    return fn
+
+
+def test_ffi_metadata_probe_and_stages():
+    xla = F.FakeXla()
+    md = F.Metadata(C.sizeof(F.Metadata), F.ApiVersion(0, None, -1, -1), 0)
+    ext = F.MetadataExt(F.ExtBase(C.sizeof(F.MetadataExt), 1, None), C.pointer(md))
+    cf = xla.frame([], [])
+    cf.extension_start = C.cast(C.pointer(ext), C.POINTER(F.ExtBase))
+    assert _handler("emi_gemm_ffi")(C.byref(cf)) is None
+    assert (md.api_version.major, md.api_version.minor) == (0, 1) and md.api_version.struct_size == C.sizeof(F.ApiVersion)
+    for stage in (0, 1, 2):                                  # instantiate / prepare / initialize do nothing
+        assert _handler("emi_attn_fwd_ffi")(C.byref(xla.frame([], [], stage=stage))) is None
+    assert xla.errors == []
+
+
+@pytest.mark.parametrize("name,args,rets,attrs,needle", [
+    ("emi_rmsnorm_fwd_ffi", [(F.F32, [4, 8]), (F.F32, [7])], [(F.F32, [4, 8])], {"eps": (F.F32, 1e-5)}, "gamma"),
+    ("emi_rmsnorm_fwd_ffi", [(F.F32, [4, 8]), (F.BF16, [8])], [(F.F32, [4, 8])], {"eps": (F.F32, 1e-5)}, "dtype"),
+    ("emi_rmsnorm_fwd_ffi", [(F.F32, [4, 8]), (F.F32, [8])], [(F.F32, [4, 8])], {}, "eps"),
+    ("emi_rmsnorm_fwd_ffi", [(F.F32, [4, 8])], [(F.F32, [4, 8])], {"eps": (F.F32, 1e-5)}, "operand"),
+    ("emi_rmsnorm_bwd_ffi", [(F.F32, [4, 8]), (F.F32, [8]), (F.F32, [4, 8])], [(F.F32, [4, 8]), (F.F32, [8]), (F.U8, [16])],
+     {"eps": (F.F32, 1e-5)}, "workspace"),
+    ("emi_rope_ffi", [(F.BF16, [2, 16, 4, 64]), (F.F32, [16, 16, 2])], [(F.BF16, [2, 16, 4, 64])], {}, "table"),
+    ("emi_gemm_ffi", [(F.BF16, [8, 16]), (F.BF16, [24, 8])], [(F.BF16, [8, 8])], {"trans_b": (F.PRED, 1)}, "contraction"),
+    ("emi_gemm_ffi", [(F.BF16, [8, 16]), (F.BF16, [8, 16])], [(F.BF16, [8, 9])], {"trans_b": (F.PRED, 1)}, "C (and R)"),
+    ("emi_attn_fwd_ffi", [(F.BF16, [1, 2, 64, 128])] * 3, [(F.BF16, [1, 2, 64, 128]), (F.F32, [1, 2, 63])],
+     {"scale": (F.F32, 0.1), "causal": (F.PRED, 1)}, "lse"),
+    ("emi_attn_fwd_ffi", [(F.BF16, [1, 2, 64, 128])] * 3, [(F.BF16, [1, 2, 64, 128]), (F.F32, [1, 2, 64])],
+     {"causal": (F.PRED, 1)}, "scale"),
+    ("emi_attn_bwd_ffi", [(F.BF16, [1, 2, 64, 128])] * 4 + [(F.F32, [1, 2, 64]), (F.BF16, [1, 2, 64, 128])],
+     [(F.BF16, [1, 2, 64, 128])] * 3 + [(F.U8, [8])], {"scale": (F.F32, 0.1)}, "workspace"),
+    ("emi_embedding_fwd_ffi", [(F.S64, [3]), (F.F32, [10, 4])], [(F.F32, [3, 4])], {}, "s32"),
+    ("emi_swiglu_bwd_ffi", [(F.F32, [8])] * 3, [(F.F32, [8]), (F.F32, [9])], {}, "shape"),
+])
+def test_ffi_rejects_malformed_frames(name, args, rets, attrs, needle):
+    xla = F.FakeXla()
+    cf = xla.frame([xla.buffer(*a) for a in args], [xla.buffer(*r) for r in rets], attrs)
+    err = _handler(name)(C.byref(cf))
+    assert err is not None and len(xla.errors) == 1
+    code, msg = xla.errors[0]
+    assert code == F.INVALID_ARGUMENT and needle in msg, msg
+
+
+def test_ffi_null_buffer_and_missing_stream_getter():
+    xla = F.FakeXla()
+    cf = xla.frame([xla.buffer(F.F32, [8], data=None), xla.buffer(F.F32, [8])], [xla.buffer(F.F32, [8])])
+    assert _handler("emi_add_ffi")(C.byref(cf)) is not None and "null" in xla.errors[-1][1]
+    xla.api.struct_size = 48                                  # an API table that ends before Stream_Get
+    cf = xla.frame([xla.buffer(F.F32, [8]), xla.buffer(F.F32, [8])], [xla.buffer(F.F32, [8])])
+    assert _handler("emi_add_ffi")(C.byref(cf)) is not None and "Stream_Get" in xla.errors[-1][1]
+
+
+def test_ffi_registration_lists_all_targets_for_rocm():
+    lib = _lib()
+    lib.emi_ffi_target_name.restype = C.c_char_p
+    lib.emi_ffi_target_handler.restype = C.c_void_p
+    n = lib.emi_ffi_target_count()
+    names = [lib.emi_ffi_target_name(i).decode() for i in range(n)]
+    assert n == 12 and "emi_attn_bwd" in names and all(lib.emi_ffi_target_handler(i) for i in range(n))
+    from enzyme_ad.jax import ops
+    used = {t for fwd, bwd in ops.FFI_TARGETS.values() for t in (fwd,) + tuple(bwd)}
+    assert used <= set(names)                                 # every target the lowering table names has a handler
+    xla = F.FakeXla()
+    lib.emi_register_ffi.argtypes = [C.POINTER(F.Api)]
+    assert lib.emi_register_ffi(C.byref(xla.api)) == 0
+    assert sorted(r[0] for r in xla.registered) == sorted(names) and {r[1] for r in xla.registered} == {"ROCM"}
+    assert lib.emi_register_ffi(C.byref(xla.api)) == 0 and len(xla.registered) == n     # once per process
+    assert lib.emi_register_ffi(None) == 3
+
+
+def test_python_surface_matches_reference_names():
+    import enzyme_ad.jax as ej
+    for name in ["cpp_call", "ffi_call", "hlo_call", "enzyme_jax_ir", "optimize_module", "export", "XLAPipeline",
+                 "JaXPipeline", "full_optimization_pass_pipeline", "optimization_passes"]:   # __init__.py:1-12
+        assert hasattr(ej, name), name
+    p = ej.JaXPipeline("inline,enzyme-wrap{infn=main outfn= retTys=enzyme_dup argTys=enzyme_dup mode=ForwardMode},cse")
+    assert p.mlir_ad() and p.stablehlo_inject() and p.ad_level() == 1 and p.pass_pipeline().startswith("inline")
+    x = ej.XLAPipeline("out.ll")
+    assert not x.mlir_ad() and not x.stablehlo_inject() and x.export_llvm() == "out.ll" and x.pass_pipeline() == ""
+    full = ej.full_optimization_pass_pipeline(inline=False, no_nan=True)
+    parsed = ej.parse_pass_pipeline(full)
+    names = [n for n, _ in parsed]
+    assert names[0] == "mark-func-memory-effects" and "enzyme-batch" in names and "enzyme" in names
+    enz = dict(parsed)["enzyme"]
+    assert enz.startswith('postpasses="arith-raise{stablehlo=true}')            # nested braces inside quotes survive
+    assert "inline" not in names and "no_nan<1>" in full
+    assert ej.optimization_passes().startswith("inline{default-pipeline=canonicalize max-iterations=4},canonicalize,cse")
+    with pytest.raises(ValueError):
+        ej.optimization_passes(transpose_propagate="sideways")
+    with pytest.raises(ValueError):
+        ej.parse_pass_pipeline("a{b")
+    with pytest.raises(TypeError):
+        ej.enzyme_jax_ir(pipeline_options="not a pipeline")(lambda x: x)
+    f = ej.enzyme_jax_ir(argv=("-O3",), pipeline_options=ej.JaXPipeline(), jit_options={"print_mlir": False}, inner_jit=False)(lambda x: x)
+    assert f(3) == 3 and f.argv == ("-O3",)
+    for call in (lambda: ej.cpp_call(out_shapes=[], source="void f(){}"), lambda: ej.hlo_call(source="module {}"),
+                 lambda: ej.jvp(f, (1,), (1,))):
+        with pytest.raises(NotImplementedError):
+            call()
+
+
+def test_operators_refuse_host_tensors():
+    import torch
+    from enzyme_ad.jax import ops
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        ops.rmsnorm(torch.zeros(2, 8), torch.ones(8))
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        ops.gemm(torch.zeros(2, 8), torch.zeros(8, 2))
+
+
+def test_tape_fan_in_without_gpu():
+    """The tape's bookkeeping, exercised with a stub operator (no kernels run)."""
+    import torch
+    from enzyme_ad.jax import ops
+    a, b = torch.ones(3), torch.ones(3)
+    with ops.Tape() as tape:
+        y = a * 2
+        ops.Tape.record((a,), y, lambda c, acc: (c * 2 if acc[0] is None else acc[0] + c * 2,))
+        z = y + a
+        ops.Tape.record((y, a), z, lambda c, acc: (c if acc[0] is None else acc[0] + c, c if acc[1] is None else acc[1] + c))
+    ga, gb = tape.backward([z], [torch.ones(3)], [a, b])
+    assert torch.equal(ga, torch.full((3,), 3.0)) and gb is None
