@@ -28,6 +28,10 @@ sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0     # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0         # MI355X HBM3E
+# HBM-side bytes per GEMM launch (average over the 21 launches of one step) from the
+# FETCH_SIZE and WRITE_SIZE counter runs summarised in
+# profiles/gemm_bf16_llama7b_layer_hbm_traffic.txt (only valid for the default workload).
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = 1.709e9
 
 C5 = dict(dim=4096, hidden_dim=11008, n_heads=32, batch=4, seq=4096)
 
@@ -206,6 +210,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel roofline table")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also run one emi_add over 3 x 512 MiB (reads 1 GiB, writes 512 MiB): the known-size kernel "
+                         "that FETCH_SIZE / WRITE_SIZE counter runs are scaled by")
     ap.add_argument("--seq", type=int, default=C5["seq"])
     ap.add_argument("--batch", type=int, default=C5["batch"])
     args = ap.parse_args()
@@ -218,6 +225,13 @@ def main():
     from enzyme_ad.jax import enzyme_jax_ir, JaXPipeline, vjp, llama
     from enzyme_ad.jax.profiling import pretty_print_table
 
+    if args.calibrate:
+        from enzyme_ad.jax import ops as _ops
+        ca = torch.ones(1 << 28, dtype=torch.bfloat16, device="cuda")
+        cb = torch.ones(1 << 28, dtype=torch.bfloat16, device="cuda")
+        _ops.add(ca, cb)
+        torch.cuda.synchronize()
+        del ca, cb
     cfg = dict(C5, seq=args.seq, batch=args.batch)
     x, lw, dy = make_layer_inputs(cfg)
     nh = cfg["n_heads"]
@@ -247,7 +261,8 @@ def main():
     t_gemm, gemm_fl, n_gemm, per_layout = bench_gemms(cfg, max(2, min(args.steps, 5)))
     roofline = dict(bound="mfma", kernel="gemm_bf16_kernel<256,256,2,4> (NT, NN, TN instantiations; %d launches per step)" % n_gemm,
                     achieved=gemm_fl / t_gemm / 1e12, peak=PEAK_BF16_TFLOPS, unit="TFLOP/s",
-                    frac=gemm_fl / t_gemm / 1e12 / PEAK_BF16_TFLOPS, traffic=None,
+                    frac=gemm_fl / t_gemm / 1e12 / PEAK_BF16_TFLOPS,
+                    traffic=GEMM_TRAFFIC_BYTES_PER_LAUNCH if (args.seq, args.batch) == (C5["seq"], C5["batch"]) else None,
                     avg_launch_us=t_gemm / n_gemm * 1e6, flops_per_launch=gemm_fl / n_gemm,
                     per_layout={k: dict(tflops=round(v["tflops"], 1), avg_launch_us=round(v["seconds"] / v["launches"] * 1e6, 1))
                                 for k, v in per_layout.items()})

@@ -490,7 +490,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_bf16_kernel(const uint16_t
     const int key0 = j * BKV;
     if (!(causal && key0 > q0 + 31)) {
       const bool need_mask = (causal && key0 + BKV - 1 > q0) || key0 + BKV > seq;
-#pragma unroll
+#pragma unroll 1
       for (int T = 0; T < 2; T++) {
         f32x16_t s, dp;
 #pragma unroll
@@ -609,7 +609,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_bf16_kernel(const uint16_t* 
     const int qbase = qt * BQT;
     if (!(causal && qbase + BQT - 1 < k0)) {          // some query of the tile can see some key of this wave
       const bool need_mask = (causal && qbase < k0 + 31) || qbase + BQT > seq || k0 + 32 > seq;
-#pragma unroll
+#pragma unroll 1
       for (int T = 0; T < 2; T++) {
         f32x16_t s, dp;
 #pragma unroll
