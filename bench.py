@@ -119,11 +119,18 @@ def bench_gemms(cfg, iters):
 
 
 def bench_kernels(cfg, iters):
-    """Roofline figures of the non-GEMM kernels at their configuration shapes."""
+    """Roofline figures of the non-GEMM kernels at their configuration shapes.  The
+    launchers are called straight through the C ABI on preallocated buffers so that
+    the HIP-event time is kernel time, not host allocation time."""
     import torch
     from enzyme_ad.jax import ops, _native as N
+    lib = N.lib()
+    st = torch.cuda.current_stream().cuda_stream
     out = {}
     bf = torch.bfloat16
+
+    def P(t):
+        return t.data_ptr()
 
     def hbm(name, fn, nbytes):
         t = event_time(fn, iters)
@@ -135,38 +142,45 @@ def bench_kernels(cfg, iters):
         out[name] = dict(bound="mfma", achieved=flops / t / 1e12, peak=PEAK_BF16_TFLOPS, unit="TFLOP/s",
                          frac=flops / t / 1e12 / PEAK_BF16_TFLOPS, us=t * 1e6)
 
-    # C2: x [16, 2048, 4096], bf16 and fp32
-    for dt, s in ((bf, 2), (torch.float32, 4)):
+    # C2: x [16, 2048, 4096], bf16 and fp32; RoPE over 32 heads x 128
+    for dt, s, code in ((bf, 2, N.EMI_BF16), (torch.float32, 4, N.EMI_F32)):
         tag = "bf16" if dt == bf else "f32"
-        x = torch.randn((16, 2048, 4096), device="cuda").to(dt)
-        gam = (torch.rand(4096, device="cuda") + 0.5).to(dt)
-        dy = torch.randn((16, 2048, 4096), device="cuda").to(dt)
+        rows, D = 16 * 2048, 4096
+        x = torch.randn((16, 2048, D), device="cuda").to(dt)
+        gam = (torch.rand(D, device="cuda") + 0.5).to(dt)
+        dy = torch.randn((16, 2048, D), device="cuda").to(dt)
+        y, dgam = torch.empty_like(x), torch.empty_like(gam)
+        wsb = lib.emi_rmsnorm_bwd_workspace_bytes(rows, D)
+        ws = torch.empty(wsb, dtype=torch.uint8, device="cuda")
+        table = ops.rope_table(2048, 128)
         n = x.numel()
-        hbm("rmsnorm_fwd_" + tag, lambda: ops.rmsnorm(x, gam), 2 * n * s)
-        with ops.Tape() as tape:
-            y = ops.rmsnorm(x, gam)
-        hbm("rmsnorm_bwd_" + tag, lambda: tape.backward([y], [dy], [x, gam]), 3 * n * s)
-        hbm("rope_fwd_" + tag, lambda: ops.rope(x, 32), 2 * n * s)
-        hbm("rope_bwd_" + tag, lambda: ops.rope(x, 32, inverse=True), 2 * n * s)
-        del x, dy, y, tape
+        hbm("rmsnorm_fwd_" + tag, lambda: N.check(lib.emi_rmsnorm_fwd(st, P(x), P(gam), P(y), rows, D, 1e-5, code)), 2 * n * s)
+        hbm("rmsnorm_bwd_" + tag, lambda: N.check(lib.emi_rmsnorm_bwd(st, P(x), P(gam), P(dy), None, P(y), P(dgam), P(ws), wsb,
+                                                                      rows, D, 1e-5, code)), 3 * n * s)
+        hbm("rope_fwd_" + tag, lambda: N.check(lib.emi_rope(st, P(x), P(table), P(y), 16, 2048, 32, 128, 0, code)), 2 * n * s)
+        hbm("rope_bwd_" + tag, lambda: N.check(lib.emi_rope(st, P(dy), P(table), P(y), 16, 2048, 32, 128, 1, code)), 2 * n * s)
+        del x, dy, y, ws
     # C5 SwiGLU: [16384, 11008] bf16
     T, H = cfg["batch"] * cfg["seq"], cfg["hidden_dim"]
-    a = torch.randn((T, H), device="cuda").to(bf)
-    b = torch.randn((T, H), device="cuda").to(bf)
-    dg = torch.randn((T, H), device="cuda").to(bf)
-    hbm("swiglu_fwd_bf16", lambda: ops.swiglu(a, b), 3 * a.numel() * 2)
-    with ops.Tape() as tape:
-        g = ops.swiglu(a, b)
-    hbm("swiglu_bwd_bf16", lambda: tape.backward([g], [dg], [a, b]), 5 * a.numel() * 2)
-    del a, b, dg, g, tape
+    a, b, dg = (torch.randn((T, H), device="cuda").to(bf) for _ in range(3))
+    da, db = torch.empty_like(a), torch.empty_like(a)
+    n = a.numel()
+    hbm("swiglu_fwd_bf16", lambda: N.check(lib.emi_swiglu_fwd(st, P(a), P(b), P(da), n, N.EMI_BF16)), 3 * n * 2)
+    hbm("swiglu_bwd_bf16", lambda: N.check(lib.emi_swiglu_bwd(st, P(a), P(b), P(dg), P(da), P(db), n, N.EMI_BF16)), 5 * n * 2)
+    del a, b, dg, da, db
     # C3: attention [8, 32, 2048, 128] bf16 causal
     B, h, S, d = 8, 32, 2048, 128
     q, k, v, do = (torch.randn((B, h, S, d), device="cuda").to(bf) for _ in range(4))
+    o, dq, dk, dv = (torch.empty_like(q) for _ in range(4))
+    lse = torch.empty((B, h, S), dtype=torch.float32, device="cuda")
+    wsb = lib.emi_attn_bwd_workspace_bytes(B, h, S, d)
+    ws = torch.empty(wsb, dtype=torch.uint8, device="cuda")
+    sc = d ** -0.5
     fl = 2.0 * B * h * S * S * d
-    mfma("attn_fwd_c3", lambda: ops.attention(q, k, v, h, layout="bhsd"), fl)
-    with ops.Tape() as tape:
-        o = ops.attention(q, k, v, h, layout="bhsd")
-    mfma("attn_bwd_c3", lambda: tape.backward([o], [do], [q, k, v]), 2.5 * fl)
+    mfma("attn_fwd_c3", lambda: N.check(lib.emi_attn_fwd(st, P(q), P(k), P(v), P(o), P(lse), B, h, S, d, h * S * d, S * d, d,
+                                                         sc, 1, N.EMI_BF16)), fl)
+    mfma("attn_bwd_c3", lambda: N.check(lib.emi_attn_bwd(st, P(q), P(k), P(v), P(o), P(lse), P(do), P(dq), P(dk), P(dv), P(ws), wsb,
+                                                         B, h, S, d, h * S * d, S * d, d, sc, 1, N.EMI_BF16)), 2.5 * fl)
     return out
 
 

@@ -91,6 +91,25 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const T* __restrict__ 
     if (c < nchunk) Vec8<T>::load(gamma + c * 8, gm[j]);
   }
   const int64_t nrow_iter = (rows + RPB - 1) / RPB;   // row groups
+  // Rows are software pipelined: the loads of the next row are issued before the
+  // reduction (shuffles, LDS, barrier) of the current one, which keeps twice the
+  // bytes in flight per block.
+  typename Vec8<T>::Raw xn[NCH], gn[NCH];      // kept in storage format to save registers
+  auto load_row = [&](int64_t rg) {
+    const int64_t row = rg * RPB + rib;
+#pragma unroll
+    for (int j = 0; j < NCH; j++) {
+      const int c = tir + j * TPR;
+      if (rg < nrow_iter && row < rows && c < nchunk) {
+        xn[j] = Vec8<T>::load_raw(x + row * dim + c * 8);
+        gn[j] = Vec8<T>::load_raw(dy + row * dim + c * 8);
+      } else {
+        xn[j] = Vec8<T>::zero_raw();
+        gn[j] = Vec8<T>::zero_raw();
+      }
+    }
+  };
+  load_row(blockIdx.x);
   int it = 0;
   for (int64_t rg = blockIdx.x; rg < nrow_iter; rg += gridDim.x, ++it) {
     const int64_t row = rg * RPB + rib;
@@ -99,17 +118,15 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const T* __restrict__ 
     float ss = 0.f, gx = 0.f;
 #pragma unroll
     for (int j = 0; j < NCH; j++) {
-      const int c = tir + j * TPR;
-      if (active && c < nchunk) {
-        Vec8<T>::load(x + row * dim + c * 8, xv[j]);
-        Vec8<T>::load(dy + row * dim + c * 8, gv[j]);
+      Vec8<T>::unpack(xn[j], xv[j]);
+      Vec8<T>::unpack(gn[j], gv[j]);
 #pragma unroll
-        for (int e = 0; e < 8; e++) {
-          ss += xv[j][e] * xv[j][e];
-          gx += gv[j][e] * gm[j][e] * xv[j][e];
-        }
+      for (int e = 0; e < 8; e++) {
+        ss += xv[j][e] * xv[j][e];
+        gx += gv[j][e] * gm[j][e] * xv[j][e];
       }
     }
+    load_row(rg + gridDim.x);
     row_reduce2<TPR>(ss, gx, red, it);
     const float r = 1.0f / sqrtf(ss / (float)dim + eps);
     const float coef = r * r * r * (gx / (float)dim);
@@ -190,23 +207,41 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_generic_kernel(const T* __res
   }
 }
 
-// out[c] = sum_p partial[p][c]; 32 columns x 8 row groups per block.
-template <typename T>
+// Column sums of partial[nparts][dim] in chunks of 128 rows: block (cb, rc) adds
+// rows [128*rc, 128*rc+128) of 128 columns (32 float4 columns x 8 row lanes, so a
+// wavefront reads 512 contiguous bytes of two rows) into row rc of `out`.
+// The launcher applies it until one row is left; the last pass writes type T.
+template <typename TO>
 __global__ __launch_bounds__(256) void colsum_kernel(const float* __restrict__ partial, int nparts, int64_t dim,
-                                                     T* __restrict__ out) {
-  __shared__ float red[8][33];
-  const int cg = threadIdx.x & 31, rg = threadIdx.x >> 5;
-  const int64_t col = (int64_t)blockIdx.x * 32 + cg;
-  float s = 0.f;
-  if (col < dim)
-    for (int p = rg; p < nparts; p += 8) s += partial[(int64_t)p * dim + col];
-  red[rg][cg] = s;
-  __syncthreads();
-  if (rg == 0 && col < dim) {
-    float t = 0.f;
+                                                     TO* __restrict__ out) {
+  __shared__ float red[8][128 + 4];
+  const int cq = threadIdx.x & 31, rl = threadIdx.x >> 5;
+  const int64_t col = (int64_t)blockIdx.x * 128 + cq * 4;
+  const int r0 = blockIdx.y * 128;
+  const int r1 = r0 + 128 < nparts ? r0 + 128 : nparts;
+  float s[4] = {0.f, 0.f, 0.f, 0.f};
+  if ((dim & 3) == 0 && col + 4 <= dim) {
+    for (int p = r0 + rl; p < r1; p += 8) {
+      const float4 v = *reinterpret_cast<const float4*>(partial + (int64_t)p * dim + col);
+      s[0] += v.x; s[1] += v.y; s[2] += v.z; s[3] += v.w;
+    }
+  } else {
+    for (int p = r0 + rl; p < r1; p += 8)
 #pragma unroll
-    for (int i = 0; i < 8; i++) t += red[i][cg];
-    out[col] = from_f32<T>(t);
+      for (int e = 0; e < 4; e++)
+        if (col + e < dim) s[e] += partial[(int64_t)p * dim + col + e];
+  }
+#pragma unroll
+  for (int e = 0; e < 4; e++) red[rl][cq * 4 + e] = s[e];
+  __syncthreads();
+  if (threadIdx.x < 128) {
+    const int64_t c = (int64_t)blockIdx.x * 128 + threadIdx.x;
+    if (c < dim) {
+      float t = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; i++) t += red[i][threadIdx.x];
+      out[(int64_t)blockIdx.y * dim + c] = from_f32<TO>(t);
+    }
   }
 }
 
@@ -385,7 +420,7 @@ static inline void rms_bwd_shape(int64_t rows, int64_t dim, int* tpr, int* nch, 
     *nch = per <= 1 ? 1 : (per <= 2 ? 2 : 4);
     const int rpb = 256 / *tpr;
     const int64_t groups = (rows + rpb - 1) / rpb;
-    const int64_t cap = (*tpr == 64) ? 512 : 2048;
+    const int64_t cap = (*tpr == 64) ? 256 : 1024;   // 4 resident blocks per CU, one wave of blocks
     *grid = groups < cap ? (groups > 0 ? groups : 1) : cap;
     *nparts = *grid * rpb;
   } else {
@@ -449,7 +484,20 @@ static int rmsnorm_bwd_launch(hipStream_t st, const void* x, const void* gamma, 
 #undef EMI_RMS_BWD
   }
   EMI_CHECK_LAUNCH("emi_rmsnorm_bwd");
-  hipLaunchKernelGGL(colsum_kernel<T>, dim3(blocks_for(dim, 32)), dim3(256), 0, st, part, (int)nparts, dim,
+  // [nparts, dim] -> [ceil(nparts/128), dim] -> ... -> dgamma
+  float* cur = part;
+  float* nxt = part + nparts * dim;
+  int64_t n = nparts;
+  while (n > 128) {
+    const int64_t m = (n + 127) / 128;
+    hipLaunchKernelGGL(colsum_kernel<float>, dim3(blocks_for(dim, 128), (unsigned)m), dim3(256), 0, st, cur, (int)n, dim, nxt);
+    EMI_CHECK_LAUNCH("emi_rmsnorm_bwd(colsum)");
+    float* t = cur;
+    cur = nxt;
+    nxt = t;
+    n = m;
+  }
+  hipLaunchKernelGGL(colsum_kernel<T>, dim3(blocks_for(dim, 128), 1), dim3(256), 0, st, cur, (int)n, dim,
                      static_cast<T*>(dgamma));
   EMI_CHECK_LAUNCH("emi_rmsnorm_bwd(colsum)");
   return EMI_OK;
@@ -483,7 +531,8 @@ extern "C" size_t emi_rmsnorm_bwd_workspace_bytes(int64_t rows, int64_t dim) {
   int tpr, nch;
   int64_t grid, nparts;
   rms_bwd_shape(rows, dim, &tpr, &nch, &grid, &nparts);
-  return (size_t)nparts * (size_t)dim * sizeof(float);
+  // first-level partial rows + one ping-pong area for the second level of the column sum
+  return ((size_t)nparts + (size_t)((nparts + 127) / 128)) * (size_t)dim * sizeof(float);
 }
 
 extern "C" int emi_rmsnorm_bwd(emi_stream_t stream, const void* x, const void* gamma, const void* dy,

@@ -38,6 +38,15 @@ template <> __device__ __forceinline__ bf16 from_f32<bf16>(float f) { return bf1
 // Eight consecutive elements as fp32 (one 16-byte load for bf16, two for fp32).
 template <typename T> struct Vec8;
 template <> struct Vec8<float> {
+  struct Raw { float4 a, b; };
+  static __device__ __forceinline__ Raw load_raw(const float* p) {
+    return Raw{*reinterpret_cast<const float4*>(p), *reinterpret_cast<const float4*>(p + 4)};
+  }
+  static __device__ __forceinline__ Raw zero_raw() { return Raw{make_float4(0, 0, 0, 0), make_float4(0, 0, 0, 0)}; }
+  static __device__ __forceinline__ void unpack(const Raw& r, float (&v)[8]) {
+    v[0] = r.a.x; v[1] = r.a.y; v[2] = r.a.z; v[3] = r.a.w;
+    v[4] = r.b.x; v[5] = r.b.y; v[6] = r.b.z; v[7] = r.b.w;
+  }
   static __device__ __forceinline__ void load(const float* p, float (&v)[8]) {
     float4 a = *reinterpret_cast<const float4*>(p);
     float4 b = *reinterpret_cast<const float4*>(p + 4);
@@ -50,6 +59,17 @@ template <> struct Vec8<float> {
   }
 };
 template <> struct Vec8<bf16> {
+  typedef uint4 Raw;
+  static __device__ __forceinline__ Raw load_raw(const bf16* p) { return *reinterpret_cast<const uint4*>(p); }
+  static __device__ __forceinline__ Raw zero_raw() { return make_uint4(0, 0, 0, 0); }
+  static __device__ __forceinline__ void unpack(const Raw& a, float (&v)[8]) {
+    const uint32_t w[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      v[2 * i] = __uint_as_float(w[i] << 16);
+      v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+  }
   static __device__ __forceinline__ void load(const bf16* p, float (&v)[8]) {
     uint4 a = *reinterpret_cast<const uint4*>(p);
     uint32_t w[4] = {a.x, a.y, a.z, a.w};
