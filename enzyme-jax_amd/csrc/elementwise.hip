@@ -404,6 +404,53 @@ __global__ __launch_bounds__(256) void f32_to_bf16_kernel(const float* __restric
 }
 
 // ---------------------------------------------------------------------------
+// 2-D transpose out[c][r] = in[r][c] through a padded 64x64 LDS tile.  Used to put
+// the contraction index of the adjoint GEMMs innermost (W -> W^T for dX = dY.W,
+// dY -> dY^T and X -> X^T for dW = dY^T.X) so that they run on the k-contiguous
+// MFMA path.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_kernel(const T* __restrict__ in, T* __restrict__ out, int64_t rows,
+                                                        int64_t cols, int vec_ok) {
+  constexpr int TS = 64, PADW = TS + (sizeof(T) == 2 ? 2 : 1);
+  __shared__ T tile[TS][PADW];
+  const int64_t r0 = (int64_t)blockIdx.y * TS, c0 = (int64_t)blockIdx.x * TS;
+  const int t = threadIdx.x;
+  if (vec_ok && r0 + TS <= rows && c0 + TS <= cols) {
+    constexpr int V = 16 / sizeof(T);            // elements per 16-byte access
+    constexpr int CPR = TS / V;                  // chunks per tile row
+#pragma unroll
+    for (int i = 0; i < TS * CPR / 256; i++) {
+      const int idx = t + i * 256, r = idx / CPR, c = (idx % CPR) * V;
+      const uint4 v = *reinterpret_cast<const uint4*>(in + (r0 + r) * cols + c0 + c);
+      const T* e = reinterpret_cast<const T*>(&v);
+#pragma unroll
+      for (int j = 0; j < V; j++) tile[r][c + j] = e[j];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < TS * CPR / 256; i++) {
+      const int idx = t + i * 256, c = idx / CPR, r = (idx % CPR) * V;
+      uint4 v;
+      T* e = reinterpret_cast<T*>(&v);
+#pragma unroll
+      for (int j = 0; j < V; j++) e[j] = tile[r + j][c];
+      *reinterpret_cast<uint4*>(out + (c0 + c) * rows + r0 + r) = v;
+    }
+  } else {
+    for (int idx = t; idx < TS * TS; idx += 256) {
+      const int r = idx / TS, c = idx % TS;
+      if (r0 + r < rows && c0 + c < cols) tile[r][c] = in[(r0 + r) * cols + c0 + c];
+    }
+    __syncthreads();
+    for (int idx = t; idx < TS * TS; idx += 256) {
+      const int c = idx / TS, r = idx % TS;
+      if (r0 + r < rows && c0 + c < cols) out[(c0 + c) * rows + r0 + r] = tile[r][c];
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
 // launch helpers
 // ---------------------------------------------------------------------------
 
@@ -703,4 +750,23 @@ extern "C" int emi_embedding_bwd(emi_stream_t stream, const int32_t* tokens, con
     EMI_CHECK_LAUNCH("emi_embedding_bwd(convert)");
   }
   return EMI_OK;
+}
+
+template <typename T> static int transpose_launch(hipStream_t st, const void* in, void* out, int64_t rows, int64_t cols) {
+  const int vec_ok = (aligned16(in) && aligned16(out) && rows % 8 == 0 && cols % 8 == 0) ? 1 : 0;
+  const dim3 grid(blocks_for(cols, 64), blocks_for(rows, 64));
+  hipLaunchKernelGGL(transpose_kernel<T>, grid, dim3(256), 0, st, static_cast<const T*>(in), static_cast<T*>(out), rows, cols,
+                     vec_ok);
+  EMI_CHECK_LAUNCH("emi_transpose");
+  return EMI_OK;
+}
+
+extern "C" int emi_transpose(emi_stream_t stream, const void* in, void* out, int64_t rows, int64_t cols, int dtype) {
+  EMI_REQUIRE(rows >= 0 && cols >= 0, "emi_transpose: negative size");
+  if (rows == 0 || cols == 0) return EMI_OK;
+  EMI_REQUIRE(in && out && in != out, "emi_transpose: null or aliased buffer");
+  EMI_REQUIRE((rows + 63) / 64 <= 65535, "emi_transpose: more than 65535*64 rows");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  EMI_DISPATCH_DTYPE("emi_transpose", dtype, transpose_launch<float>(st, in, out, rows, cols),
+                     transpose_launch<bf16>(st, in, out, rows, cols));
 }

@@ -68,41 +68,51 @@ template <int BK> __device__ __forceinline__ int swz_kc(int row) {
   return BK == 64 ? ((row >> 1) & 7) : ((row >> 2) & 3);
 }
 
+// One 1 KiB wave-load (number `it` of this wave) of a k-contiguous tile.
+template <int BK, int NW>
+__device__ __forceinline__ void load_one_kcontig(__amdgpu_buffer_rsrc_t rsrc, EMI_LDS uint8_t* lds, int wave, int lane,
+                                                 uint32_t row0_off_bytes, int ld, int k0, int K, int it) {
+  constexpr int CPR = BK / 8;                 // 16-byte chunks per row
+  constexpr int RPW = 64 / CPR;               // rows per 1 KiB wave-load
+  const int r_in = lane / CPR, pc = lane % CPR;
+  const int r = (it * NW + wave) * RPW + r_in;
+  const int lc = pc ^ swz_kc<BK>(r);
+  const int k = k0 + lc * 8;
+  uint32_t voff = row0_off_bytes + (uint32_t)(r * ld + k) * 2u;
+  if (k >= K) voff = kOob;
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, lds + (it * NW + wave) * 1024, 16, voff, 0, 0, 0);
+}
+
 template <int ROWS, int BK, int NW>
 __device__ __forceinline__ void load_tile_kcontig(__amdgpu_buffer_rsrc_t rsrc, EMI_LDS uint8_t* lds, int wave, int lane,
                                                   uint32_t row0_off_bytes, int ld, int k0, int K) {
-  constexpr int CPR = BK / 8;                 // 16-byte chunks per row
-  constexpr int RPW = 64 / CPR;               // rows per 1 KiB wave-load
-  constexpr int NLOAD = ROWS / RPW / NW;
+  constexpr int NLOAD = ROWS * BK * 2 / 1024 / NW;
   static_assert(NLOAD >= 1, "tile smaller than one pass of the block");
-  const int r_in = lane / CPR, pc = lane % CPR;
 #pragma unroll
-  for (int it = 0; it < NLOAD; it++) {
-    const int r = (it * NW + wave) * RPW + r_in;
-    const int lc = pc ^ swz_kc<BK>(r);
-    const int k = k0 + lc * 8;
-    uint32_t voff = row0_off_bytes + (uint32_t)(r * ld + k) * 2u;
-    if (k >= K) voff = kOob;
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, lds + (it * NW + wave) * 1024, 16, voff, 0, 0, 0);
-  }
+  for (int it = 0; it < NLOAD; it++) load_one_kcontig<BK, NW>(rsrc, lds, wave, lane, row0_off_bytes, ld, k0, K, it);
+}
+
+template <int COLS, int NW>
+__device__ __forceinline__ void load_one_kmajor(__amdgpu_buffer_rsrc_t rsrc, EMI_LDS uint8_t* lds, int wave, int lane,
+                                                int col0, int ncols, int ld, int k0, int K, int it) {
+  constexpr int CPR = COLS / 8;               // 16-byte chunks per k-row
+  static_assert(CPR >= 16, "k-major tile too narrow");
+  const int slot = (it * NW + wave) * 64 + lane;
+  const int k = slot / CPR, pc = slot % CPR;
+  const int lc = pc ^ (4 * (k & 3));
+  const int col = col0 + lc * 8;
+  uint32_t voff = (uint32_t)((k0 + k) * ld + col) * 2u;
+  if (k0 + k >= K || col >= ncols) voff = kOob;
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, lds + (it * NW + wave) * 1024, 16, voff, 0, 0, 0);
 }
 
 template <int COLS, int BK, int NW>
 __device__ __forceinline__ void load_tile_kmajor(__amdgpu_buffer_rsrc_t rsrc, EMI_LDS uint8_t* lds, int wave, int lane,
                                                  int col0, int ncols, int ld, int k0, int K) {
-  constexpr int CPR = COLS / 8;               // 16-byte chunks per k-row
-  constexpr int NLOAD = BK * CPR / 64 / NW;
-  static_assert(CPR >= 16 && NLOAD >= 1, "k-major tile too narrow");
+  constexpr int NLOAD = BK * COLS * 2 / 1024 / NW;
+  static_assert(NLOAD >= 1, "tile smaller than one pass of the block");
 #pragma unroll
-  for (int it = 0; it < NLOAD; it++) {
-    const int slot = (it * NW + wave) * 64 + lane;
-    const int k = slot / CPR, pc = slot % CPR;
-    const int lc = pc ^ (4 * (k & 3));
-    const int col = col0 + lc * 8;
-    uint32_t voff = (uint32_t)((k0 + k) * ld + col) * 2u;
-    if (k0 + k >= K || col >= ncols) voff = kOob;
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, lds + (it * NW + wave) * 1024, 16, voff, 0, 0, 0);
-  }
+  for (int it = 0; it < NLOAD; it++) load_one_kmajor<COLS, NW>(rsrc, lds, wave, lane, col0, ncols, ld, k0, K, it);
 }
 
 // MFMA operand fragment (32 rows x 16 k) for k-step kk of the tile.
@@ -443,8 +453,8 @@ static int launch_bf16(hipStream_t st, const void* A, const void* B, const void*
 }
 
 // Tile configuration.  EMI_GEMM_TILE (read once) overrides the choice for tuning:
-//   0 = automatic, 1 = 256x256x64 2-stage 8 waves, 2 = 256x256x32 4-stage 4 waves,
-//   3 = 256x256x32 4-stage 8 waves, 4 = 128x128x64 2-stage 4 waves.
+//   0 = automatic, 1 = 256x256x64 2-stage 8 waves, 2 = 256x256x32 4-stage 8 waves
+//   (slower: 64-byte rows double the cache-line requests per byte), 4 = 128x128x64.
 static int tile_override() {
   static int v = -1;
   if (v < 0) {
@@ -466,8 +476,7 @@ static int launch_bf16_layout(hipStream_t st, const void* A, const void* B, cons
 #define EMI_GEMM_ARGS st, A, B, R, C, M, N, K, lda, ldb, ldr, ldc, a_bytes, b_bytes
   switch (cfg) {
     case 1: return launch_bf16<256, 256, 64, 2, 2, 4, AK, BKM>(EMI_GEMM_ARGS);
-    case 2: return launch_bf16<256, 256, 32, 4, 2, 2, AK, BKM>(EMI_GEMM_ARGS);
-    case 3: return launch_bf16<256, 256, 32, 4, 2, 4, AK, BKM>(EMI_GEMM_ARGS);
+    case 2: return launch_bf16<256, 256, 32, 4, 2, 4, AK, BKM>(EMI_GEMM_ARGS);
     default: return launch_bf16<128, 128, 64, 2, 2, 2, AK, BKM>(EMI_GEMM_ARGS);
   }
 #undef EMI_GEMM_ARGS

@@ -28,6 +28,7 @@ SIGNATURES = {
     "emi_swiglu_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_int]),
     "emi_swiglu_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_int]),
     "emi_add": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_int]),
+    "emi_transpose": (c_int, [c_void_p, c_void_p, c_void_p, c_i64, c_i64, c_int]),
     "emi_gemm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64,
                          c_i64, c_int, c_int, c_int]),
     "emi_attn_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_i64, c_i64, c_i64,

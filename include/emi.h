@@ -85,6 +85,12 @@ int emi_swiglu_bwd(emi_stream_t stream, const void* a, const void* b, const void
  * HLODerivatives.td:964; test/llama.py:215,233).  y may alias a or b. */
 int emi_add(emi_stream_t stream, const void* a, const void* b, void* y, int64_t n, int dtype);
 
+/* out[cols, rows] = in[rows, cols]^T (Transpose rule HLODerivatives.td:1334: the adjoint
+ * dots of the DotGeneral rule :1166-1178 contract over the outer index of their
+ * row-major operands; transposing first puts the contraction index innermost).
+ * `out` must not alias `in`. */
+int emi_transpose(emi_stream_t stream, const void* in, void* out, int64_t rows, int64_t cols, int dtype);
+
 /* GEMM: C[M,N] = op(A) . op(B) [+ R], fp32 accumulate, result rounded once.
  *   trans_a == 0: A is [M,K] (lda >= K);  trans_a != 0: A is [K,M] (lda >= M)
  *   trans_b == 0: B is [K,N] (ldb >= N);  trans_b != 0: B is [N,K] (ldb >= K)

@@ -222,3 +222,11 @@ def test_error_paths_do_not_launch(ops):
     with pytest.raises(RuntimeError):
         ops.add(torch.zeros(4), torch.zeros(4))            # host memory is refused, never computed on CPU
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("rows,cols", [(64, 64), (128, 192), (70, 33), (1, 5), (4096, 1032)])
+def test_transpose(ops, dt, rows, cols):
+    rng = np.random.default_rng(rows + cols)
+    a, ar = dev(rng.standard_normal((rows, cols)), dt)
+    assert np.array_equal(host(ops.transpose(a)), ar.T)      # a pure permutation is exact
