@@ -146,6 +146,91 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | 0x0f70);
 }
 
+// Epilogue shared by the bf16 kernels.  With swapped MFMA operands register r of
+// lane l holds C[row = l%32][col = 8*(r/4) + 4*(l/32) + r%4] of its 32x32 tile:
+// four consecutive columns per register quad.  Each wave stages its WR x WC
+// sub-tile (rows rbase.., columns cbase..) through its own slice of the now idle
+// LDS as bf16 and writes it out with 16-byte, row-contiguous stores; the residual
+// comes in the same way (16-byte loads -> LDS -> accumulator layout) and is added
+// in fp32 before the single rounding.  Slice layout: rows of 2*WC bytes, chunk c
+// of row r at chunk c ^ e_swz(r), the two 8-byte halves of a chunk swapped when
+// (r>>4)&1, which makes the 8-byte column-quad accesses of 32 lanes (32 rows)
+// conflict free.
+template <int WR, int WC, int TM, int TN>
+__device__ __forceinline__ void epilogue_bf16(f32x16_t (&acc)[TM][TN], EMI_LDS uint8_t* smem, int wave, int lane,
+                                              int rbase, int cbase, const uint16_t* R, uint16_t* C, int M, int N,
+                                              int ldr, int ldc, int vec_ok) {
+  static_assert(WC == 64 || WC == 128, "epilogue supports 64- or 128-column wave tiles");
+  static_assert(WR == TM * 32 && WC == TN * 32, "wave tile");
+  constexpr int RSB = WC * 2, CH = WC / 8, RPP = 64 / CH;     // row bytes, chunks per row, rows per 64-lane pass
+  EMI_LDS uint8_t* wl = smem + wave * (WR * RSB);
+  const int lrow = lane & 31, lhalf = lane >> 5;
+  auto e_swz = [](int row) { return WC == 64 ? ((row >> 1) & 7) : (row & 15); };
+  auto quad_slot = [&](int row, int chunk) {
+    return row * RSB + ((chunk ^ e_swz(row)) << 4) + ((lhalf ^ ((row >> 4) & 1)) << 3);
+  };
+  if (R != nullptr) {
+#pragma unroll
+    for (int it = 0; it < WR / RPP; it++) {
+      const int row = it * RPP + lane / CH, c = lane % CH;
+      const int grow = rbase + row, gcol = cbase + c * 8;
+      u32x4_t v = {0u, 0u, 0u, 0u};
+      if (grow < M && gcol < N) {
+        const uint16_t* src = R + (int64_t)grow * ldr + gcol;
+        if (vec_ok && gcol + 8 <= N) {
+          v = *reinterpret_cast<const u32x4_t*>(src);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; e++)
+            if (gcol + e < N) v[e >> 1] |= (uint32_t)src[e] << ((e & 1) * 16);
+        }
+      }
+      if ((row >> 4) & 1) v = __builtin_shufflevector(v, v, 2, 3, 0, 1);
+      *reinterpret_cast<EMI_LDS u32x4_t*>(wl + row * RSB + ((c ^ e_swz(row)) << 4)) = v;
+    }
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int j = 0; j < TN; j++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          const u32x2_t w = *reinterpret_cast<const EMI_LDS u32x2_t*>(wl + quad_slot(i * 32 + lrow, j * 4 + q));
+          acc[i][j][4 * q + 0] += __uint_as_float(w[0] << 16);
+          acc[i][j][4 * q + 1] += __uint_as_float(w[0] & 0xffff0000u);
+          acc[i][j][4 * q + 2] += __uint_as_float(w[1] << 16);
+          acc[i][j][4 * q + 3] += __uint_as_float(w[1] & 0xffff0000u);
+        }
+  }
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        u32x2_t w;
+        w[0] = pack_bf16x2(acc[i][j][4 * q + 0], acc[i][j][4 * q + 1]);
+        w[1] = pack_bf16x2(acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+        *reinterpret_cast<EMI_LDS u32x2_t*>(wl + quad_slot(i * 32 + lrow, j * 4 + q)) = w;
+      }
+#pragma unroll
+  for (int it = 0; it < WR / RPP; it++) {
+    const int row = it * RPP + lane / CH, c = lane % CH;
+    const int grow = rbase + row, gcol = cbase + c * 8;
+    u32x4_t v = *reinterpret_cast<const EMI_LDS u32x4_t*>(wl + row * RSB + ((c ^ e_swz(row)) << 4));
+    if ((row >> 4) & 1) v = __builtin_shufflevector(v, v, 2, 3, 0, 1);
+    if (grow < M && gcol < N) {
+      uint16_t* dst = C + (int64_t)grow * ldc + gcol;
+      if (vec_ok && gcol + 8 <= N) {
+        *reinterpret_cast<u32x4_t*>(dst) = v;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; e++)
+          if (gcol + e < N) dst[e] = (uint16_t)(v[e >> 1] >> ((e & 1) * 16));
+      }
+    }
+  }
+}
+
 // Software pipeline, NSTAGE == 2: tile t+1 streams into the other LDS stage while
 // tile t is multiplied; one barrier per tile.
 // NSTAGE == 4: tiles t+2 and t+3 are in flight while tile t is multiplied and
@@ -271,30 +356,33 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_kernel(const uint16_t* 
     __syncthreads();
   }
 
-  // Epilogue.  With swapped MFMA operands register r of lane l holds
-  // C[row = l%32][col = 8*(r/4) + 4*(l/32) + r%4] of its 32x32 tile: four
-  // consecutive columns per register quad.  Each wave stages its (BM/WM) x
-  // (BN/WN) sub-tile through its own slice of the now idle LDS as bf16 and writes
-  // it out with 16-byte, row-contiguous stores; the residual comes in the same way
-  // (16-byte loads -> LDS -> accumulator layout) and is added in fp32 before the
-  // single rounding.  Slice layout: rows of 2*WC bytes, chunk c of row r at chunk
-  // c ^ e_swz(r), the two 8-byte halves of a chunk swapped when (r>>4)&1, which
-  // makes the 8-byte column-quad accesses of 32 lanes (32 rows) conflict free.
   constexpr int WR = BM / WM, WC = BN / WN;
-  static_assert(WC == 64 || WC == 128, "epilogue supports 64- or 128-column wave tiles");
   static_assert(NW * WR * WC * 2 <= NSTAGE * STAGE, "epilogue staging does not fit in the LDS allocation");
-  constexpr int RSB = WC * 2, CH = WC / 8, RPP = 64 / CH;     // row bytes, chunks per row, rows per 64-lane pass
+  epilogue_bf16<WR, WC, TM, TN>(acc, smem, wave, lane, m0 + wm * WR, n0 + wn * WC, R, C, M, N, ldr, ldc, vec_ok);
+}
+
+// Epilogue for accumulators of v_mfma_f32_16x16x32_bf16 with swapped operands:
+// register r of lane l holds C[row = l%16][col = 4*(l/16) + r] of its 16x16 tile.
+// The wave tile is (16*TM) x 64; rows of 128 bytes in the wave's LDS slice, 16-byte
+// chunk c of row r at chunk c ^ ((r >> 1) & 7): conflict free both for the 8-byte
+// column-quad accesses of the accumulator layout and for the 16-byte row accesses
+// of the global loads and stores.
+template <int TM, int TN>
+__device__ __forceinline__ void epilogue_bf16_t16(f32x4_t (&acc)[TM][TN], EMI_LDS uint8_t* smem, int wave, int lane,
+                                                  int rbase, int cbase, const uint16_t* R, uint16_t* C, int M, int N,
+                                                  int ldr, int ldc, int vec_ok) {
+  static_assert(TN == 4, "64-column wave tile");
+  constexpr int WR = TM * 16, RSB = 128;
   EMI_LDS uint8_t* wl = smem + wave * (WR * RSB);
-  const int lrow = lane & 31, lhalf = lane >> 5;
-  const int rbase = m0 + wm * WR, cbase = n0 + wn * WC;
-  auto e_swz = [](int row) { return WC == 64 ? ((row >> 1) & 7) : (row & 15); };
-  auto quad_slot = [&](int row, int chunk) {
-    return row * RSB + ((chunk ^ e_swz(row)) << 4) + ((lhalf ^ ((row >> 4) & 1)) << 3);
+  const int lrow = lane & 15, lq = lane >> 4;
+  auto quad_slot = [&](int row, int j) {      // 8-byte slot of columns 16*j + 4*lq .. +3
+    const int chunk = 2 * j + (lq >> 1);
+    return row * RSB + ((chunk ^ ((row >> 1) & 7)) << 4) + ((lq & 1) << 3);
   };
   if (R != nullptr) {
 #pragma unroll
-    for (int it = 0; it < WR / RPP; it++) {
-      const int row = it * RPP + lane / CH, c = lane % CH;
+    for (int it = 0; it < WR / 8; it++) {
+      const int row = it * 8 + (lane >> 3), c = lane & 7;
       const int grow = rbase + row, gcol = cbase + c * 8;
       u32x4_t v = {0u, 0u, 0u, 0u};
       if (grow < M && gcol < N) {
@@ -307,39 +395,33 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_kernel(const uint16_t* 
             if (gcol + e < N) v[e >> 1] |= (uint32_t)src[e] << ((e & 1) * 16);
         }
       }
-      if ((row >> 4) & 1) v = __builtin_shufflevector(v, v, 2, 3, 0, 1);
-      *reinterpret_cast<EMI_LDS u32x4_t*>(wl + row * RSB + ((c ^ e_swz(row)) << 4)) = v;
+      *reinterpret_cast<EMI_LDS u32x4_t*>(wl + row * RSB + ((c ^ ((row >> 1) & 7)) << 4)) = v;
     }
 #pragma unroll
     for (int i = 0; i < TM; i++)
 #pragma unroll
-      for (int j = 0; j < TN; j++)
-#pragma unroll
-        for (int q = 0; q < 4; q++) {
-          const u32x2_t w = *reinterpret_cast<const EMI_LDS u32x2_t*>(wl + quad_slot(i * 32 + lrow, j * 4 + q));
-          acc[i][j][4 * q + 0] += __uint_as_float(w[0] << 16);
-          acc[i][j][4 * q + 1] += __uint_as_float(w[0] & 0xffff0000u);
-          acc[i][j][4 * q + 2] += __uint_as_float(w[1] << 16);
-          acc[i][j][4 * q + 3] += __uint_as_float(w[1] & 0xffff0000u);
-        }
+      for (int j = 0; j < TN; j++) {
+        const u32x2_t w = *reinterpret_cast<const EMI_LDS u32x2_t*>(wl + quad_slot(i * 16 + lrow, j));
+        acc[i][j][0] += __uint_as_float(w[0] << 16);
+        acc[i][j][1] += __uint_as_float(w[0] & 0xffff0000u);
+        acc[i][j][2] += __uint_as_float(w[1] << 16);
+        acc[i][j][3] += __uint_as_float(w[1] & 0xffff0000u);
+      }
   }
 #pragma unroll
   for (int i = 0; i < TM; i++)
 #pragma unroll
-    for (int j = 0; j < TN; j++)
+    for (int j = 0; j < TN; j++) {
+      u32x2_t w;
+      w[0] = pack_bf16x2(acc[i][j][0], acc[i][j][1]);
+      w[1] = pack_bf16x2(acc[i][j][2], acc[i][j][3]);
+      *reinterpret_cast<EMI_LDS u32x2_t*>(wl + quad_slot(i * 16 + lrow, j)) = w;
+    }
 #pragma unroll
-      for (int q = 0; q < 4; q++) {
-        u32x2_t w;
-        w[0] = pack_bf16x2(acc[i][j][4 * q + 0], acc[i][j][4 * q + 1]);
-        w[1] = pack_bf16x2(acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
-        *reinterpret_cast<EMI_LDS u32x2_t*>(wl + quad_slot(i * 32 + lrow, j * 4 + q)) = w;
-      }
-#pragma unroll
-  for (int it = 0; it < WR / RPP; it++) {
-    const int row = it * RPP + lane / CH, c = lane % CH;
+  for (int it = 0; it < WR / 8; it++) {
+    const int row = it * 8 + (lane >> 3), c = lane & 7;
     const int grow = rbase + row, gcol = cbase + c * 8;
-    u32x4_t v = *reinterpret_cast<const EMI_LDS u32x4_t*>(wl + row * RSB + ((c ^ e_swz(row)) << 4));
-    if ((row >> 4) & 1) v = __builtin_shufflevector(v, v, 2, 3, 0, 1);
+    const u32x4_t v = *reinterpret_cast<const EMI_LDS u32x4_t*>(wl + row * RSB + ((c ^ ((row >> 1) & 7)) << 4));
     if (grow < M && gcol < N) {
       uint16_t* dst = C + (int64_t)grow * ldc + gcol;
       if (vec_ok && gcol + 8 <= N) {
@@ -351,6 +433,205 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_kernel(const uint16_t* 
       }
     }
   }
+}
+
+// ---------------------------------------------------------------------------
+// Ping-pong kernel for two k-contiguous operands (the NT layout): 256x256x64 block
+// tile, 8 wavefronts = two groups of four, one wavefront of each group per SIMD.
+// A tile step is cut into four slots separated by s_barrier; a wavefront
+// alternates memory slots (LDS -> register fragment reads, HBM -> LDS loads) and
+// compute slots (16 MFMAs), and the two groups run one slot apart, so on every SIMD
+// one wavefront always feeds the matrix core while the other one moves data.
+//
+// Each operand tile is held as two 128-row regions per LDS stage.  A wavefront's
+// 128x64 output tile is four 64x32 quadrants; a region is read into registers once
+// per tile step (for the whole BK) and is therefore free to be refilled two tile
+// steps ahead as soon as both groups have read it:
+//   region A_h : block rows  wm*128 + h*64 + [0,64)   for wm = 0,1
+//   region B_j : block cols  wn*64  + j*32 + [0,32)   for wn = 0..3
+//   slot  Ma: read B_0, B_1, A_0; refill B_1, A_1 of the other stage (tile t+1)
+//         Ca: quadrants (0,0), (0,1)
+//         Mb: read A_1; refill A_0, B_0 (tile t+2)         Cb: quadrants (1,0), (1,1)
+// A region written by loads issued in local slot L was last read in local slot
+// <= L-2 by both groups; a wavefront waits for its own loads (vmcnt) two local
+// slots before the first read of that region by either group.
+// ---------------------------------------------------------------------------
+#ifdef EMI_GEMM_TRACE
+__device__ unsigned long long emi_gemm_trace_buf[8 * 40];
+#define EMI_TRACE_MARK() do { if (tracing) ts[nts++] = __builtin_readcyclecounter(); } while (0)
+#if EMI_GEMM_TRACE > 1
+#define EMI_TRACE_MARK2() EMI_TRACE_MARK()
+#else
+#define EMI_TRACE_MARK2() do { } while (0)
+#endif
+#else
+#define EMI_TRACE_MARK() do { } while (0)
+#define EMI_TRACE_MARK2() do { } while (0)
+#endif
+
+__global__ __launch_bounds__(512) void gemm_bf16_nt_pingpong_kernel(const uint16_t* __restrict__ A,
+                                                                     const uint16_t* __restrict__ B, const uint16_t* R,
+                                                                     uint16_t* C, int M, int N, int K, int lda, int ldb,
+                                                                     int ldr, int ldc, uint32_t a_bytes, uint32_t b_bytes,
+                                                                     int vec_ok) {
+  constexpr int BM = 256, BN = 256, BK = 64;
+  constexpr int REGION = 128 * BK * 2, STAGE = 4 * REGION;      // 16 KiB, 64 KiB
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem_raw[];
+  EMI_LDS uint8_t* smem = (EMI_LDS uint8_t*)smem_raw;
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wm = wave >> 2, wn = wave & 3;
+
+  const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+  int tile_m, tile_n;
+  tile_coords(tiles_m, tiles_n, &tile_m, &tile_n);
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+  const __amdgpu_buffer_rsrc_t rA = make_rsrc(A, a_bytes);
+  const __amdgpu_buffer_rsrc_t rB = make_rsrc(B, b_bytes);
+
+  // HBM -> LDS: a region is 16 wave-loads of 1 KiB (8 rows x 128 bytes); wavefront w
+  // issues loads w and w+8 of every region.  Lane l of a wave-load fills physical
+  // chunk (l & 7) of region row q*8 + (l >> 3) and therefore fetches the logical
+  // chunk that the swizzle maps there.
+  const int lck = ((lane & 7) ^ (((lane >> 4) + 4 * (wave & 1)) & 7)) * 8;     // k offset of this lane's chunk
+  uint32_t voffA[2][2], voffB[2][2];
+#pragma unroll
+  for (int it = 0; it < 2; it++) {
+    const int rho = (it * 8 + wave) * 8 + (lane >> 3);
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+      const int grow = m0 + (rho >> 6) * 128 + h * 64 + (rho & 63);
+      voffA[h][it] = grow < M ? ((uint32_t)grow * (uint32_t)lda + (uint32_t)lck) * 2u : kOob;
+      const int gcol = n0 + (rho >> 5) * 64 + h * 32 + (rho & 31);
+      voffB[h][it] = gcol < N ? ((uint32_t)gcol * (uint32_t)ldb + (uint32_t)lck) * 2u : kOob;
+    }
+  }
+  auto refill = [&](__amdgpu_buffer_rsrc_t rsrc, const uint32_t (&voff)[2], int lds_off, int k0) {
+#pragma unroll
+    for (int it = 0; it < 2; it++) {
+      const uint32_t v = (k0 + lck < K) ? voff[it] + (uint32_t)k0 * 2u : kOob;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, smem + lds_off + (it * 8 + wave) * 1024, 16, v, 0, 0, 0);
+    }
+  };
+
+  // LDS -> registers.  Fragment of v_mfma_f32_16x16x32_bf16 (16 rows x 32 k): lane l
+  // reads row (l & 15), logical chunk 4*ks + (l >> 4) of k-step ks.
+  const int l15 = lane & 15, sw = l15 >> 1, kq = lane >> 4;
+  const int a_lane = (wm * 64 + l15) * (BK * 2);
+  const int b_lane = 2 * REGION + (wn * 32 + l15) * (BK * 2);
+  auto frag = [&](int base, int ks) {
+    return *reinterpret_cast<const EMI_LDS bf16x8_t*>(smem + base + (((ks * 4 + kq) ^ sw) << 4));
+  };
+
+  // acc[i][j]: 16x16 tile at wave rows 16*i, wave columns 16*j (i = 4*h + row block)
+  f32x4_t acc[8][4];
+#pragma unroll
+  for (int i = 0; i < 8; i++)
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) acc[i][j][r] = 0.f;
+
+  bf16x8_t fa[4][2], fb[4][2];               // [16-row block][k-step]; fb: 0,1 = B_0, 2,3 = B_1
+#ifdef EMI_GEMM_TRACE
+  unsigned long long ts[40];
+  int nts = 0;
+  bool tracing = false;
+#endif
+  auto slot_end = [&]() {
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();
+    EMI_TRACE_MARK();
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  // Compute slot: the 64 x 64 half of the wave tile that uses row half h (32 MFMAs).
+  // The operands are passed swapped so that a lane owns 4 consecutive C columns.
+  auto half_rows = [&](int h) {
+    __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+      for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+          acc[h * 4 + i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb[j][ks], fa[i][ks], acc[h * 4 + i][j], 0, 0, 0);
+    __builtin_amdgcn_s_setprio(0);
+    slot_end();
+  };
+  auto refill1 = [&](__amdgpu_buffer_rsrc_t rsrc, uint32_t voff, int lds_off, int it, int k0) {
+    const uint32_t v = (k0 + lck < K) ? voff + (uint32_t)k0 * 2u : kOob;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, smem + lds_off + (it * 8 + wave) * 1024, 16, v, 0, 0, 0);
+  };
+  auto tile_step = [&](int stage, int t) {
+    const int so = stage * STAGE, oo = (stage ^ 1) * STAGE;
+    // Ma: read B_0, A_0, B_1 of this stage; refill B_1, A_1 of the other stage (tile t+1).
+    // Loads and reads alternate so that the texture path and the LDS work in parallel.
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      if (q < 2) refill1(rB, voffB[1][q], oo + 3 * REGION, q, (t + 1) * BK);
+      else refill1(rA, voffA[1][q - 2], oo + REGION, q - 2, (t + 1) * BK);
+      const int ks = q >> 1, blk = q & 1;    // two 16-row blocks per q
+      fb[blk][ks] = frag(so + b_lane + blk * 16 * BK * 2, ks);
+      fa[2 * blk][ks] = frag(so + a_lane + (2 * blk) * 16 * BK * 2, ks);
+      fa[2 * blk + 1][ks] = frag(so + a_lane + (2 * blk + 1) * 16 * BK * 2, ks);
+      fb[2 + blk][ks] = frag(so + b_lane + REGION + blk * 16 * BK * 2, ks);
+    }
+    EMI_TRACE_MARK2();
+    wait_vmcnt<8>();                        // own part of A_1 of this tile has landed
+    EMI_TRACE_MARK2();
+    slot_end();
+    half_rows(0);                           // Ca
+    // Mb: read A_1; refill A_0, B_0 of this stage (tile t+2)
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      if (q < 2) refill1(rA, voffA[0][q], so, q, (t + 2) * BK);
+      else refill1(rB, voffB[0][q - 2], so + 2 * REGION, q - 2, (t + 2) * BK);
+      const int ks = q >> 1, blk = q & 1;
+      fa[2 * blk][ks] = frag(so + REGION + a_lane + (2 * blk) * 16 * BK * 2, ks);
+      fa[2 * blk + 1][ks] = frag(so + REGION + a_lane + (2 * blk + 1) * 16 * BK * 2, ks);
+    }
+    EMI_TRACE_MARK2();
+    wait_vmcnt<6>();                        // own part of A_0, B_0 and of B_1 of the next tile
+    EMI_TRACE_MARK2();
+    slot_end();
+    half_rows(1);                           // Cb
+  };
+
+  // Prologue: tile 0 into stage 0; A_0, B_0 of tile 1 into stage 1 (its A_1, B_1 are
+  // issued by the first memory slot).
+  refill(rA, voffA[0], 0, 0);
+  refill(rB, voffB[0], 2 * REGION, 0);
+  refill(rB, voffB[1], 3 * REGION, 0);
+  refill(rA, voffA[1], REGION, 0);
+  refill(rA, voffA[0], STAGE, BK);
+  refill(rB, voffB[0], STAGE + 2 * REGION, BK);
+  wait_vmcnt<0>();
+  slot_end();
+  if (wm == 1) slot_end();                  // second group runs one slot behind the first
+
+  const int nk = (K + BK - 1) / BK;
+  int t = 0;
+  for (; t + 1 < nk; t += 2) {
+#ifdef EMI_GEMM_TRACE
+    tracing = (blockIdx.x == 300 && (t == 16 || t == 18));
+#endif
+    tile_step(0, t);
+    tile_step(1, t + 1);
+  }
+#ifdef EMI_GEMM_TRACE
+  tracing = false;
+  if (blockIdx.x == 300 && lane == 0)
+    for (int i = 0; i < 40; i++) emi_gemm_trace_buf[wave * 40 + i] = i < nts ? ts[i] : 0ull;
+#endif
+  if (t < nk) tile_step(0, t);
+
+  if (wm == 0) slot_end();
+  wait_vmcnt<0>();                          // zero-filled loads past the end of K
+  slot_end();
+
+  epilogue_bf16_t16<8, 4>(acc, smem, wave, lane, m0 + wm * 128, n0 + wn * 64, R, C, M, N, ldr, ldc, vec_ok);
 }
 
 // ---------------------------------------------------------------------------
@@ -452,9 +733,31 @@ static int launch_bf16(hipStream_t st, const void* A, const void* B, const void*
   return EMI_OK;
 }
 
+static int launch_bf16_pingpong(hipStream_t st, const void* A, const void* B, const void* R, void* C, int M, int N, int K,
+                                int lda, int ldb, int ldr, int ldc, uint32_t a_bytes, uint32_t b_bytes) {
+  const int vec_ok = ((reinterpret_cast<uintptr_t>(C) & 15) == 0 && ldc % 8 == 0 &&
+                      (R == nullptr || ((reinterpret_cast<uintptr_t>(R) & 15) == 0 && ldr % 8 == 0)))
+                         ? 1 : 0;
+  constexpr int smem = 2 * 65536;
+  static bool configured = false;   // idempotent; a race only repeats the call
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_nt_pingpong_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return emi_fail(EMI_INTERNAL, "emi_gemm: cannot reserve %d bytes of LDS: %s", smem, hipGetErrorString(e));
+    configured = true;
+  }
+  const int tiles = ((M + 255) / 256) * ((N + 255) / 256);
+  hipLaunchKernelGGL(gemm_bf16_nt_pingpong_kernel, dim3(tiles), dim3(512), smem, st, static_cast<const uint16_t*>(A),
+                     static_cast<const uint16_t*>(B), static_cast<const uint16_t*>(R), static_cast<uint16_t*>(C), M, N, K,
+                     lda, ldb, ldr, ldc, a_bytes, b_bytes, vec_ok);
+  EMI_CHECK_LAUNCH("emi_gemm");
+  return EMI_OK;
+}
+
 // Tile configuration.  EMI_GEMM_TILE (read once) overrides the choice for tuning:
 //   0 = automatic, 1 = 256x256x64 2-stage 8 waves, 2 = 256x256x32 4-stage 8 waves
-//   (slower: 64-byte rows double the cache-line requests per byte), 4 = 128x128x64.
+//   (slower: 64-byte rows double the cache-line requests per byte), 4 = 128x128x64,
+//   5 = 256x256x64 ping-pong (NT layout only).
 static int tile_override() {
   static int v = -1;
   if (v < 0) {
@@ -469,13 +772,17 @@ static int launch_bf16_layout(hipStream_t st, const void* A, const void* B, cons
                               int lda, int ldb, int ldr, int ldc, uint32_t a_bytes, uint32_t b_bytes) {
   int cfg = tile_override();
   if (cfg == 0) {
-    // 256x256 tiles when they fill the chip, else 128x128.
+    // 256x256 tiles when they fill the chip (the ping-pong kernel for two
+    // k-contiguous operands), else 128x128.
     const int64_t big_tiles = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
-    cfg = big_tiles >= 192 ? 1 : 4;
+    cfg = big_tiles >= 192 ? ((!AK && !BKM) ? 5 : 1) : 4;
   }
 #define EMI_GEMM_ARGS st, A, B, R, C, M, N, K, lda, ldb, ldr, ldc, a_bytes, b_bytes
   switch (cfg) {
     case 1: return launch_bf16<256, 256, 64, 2, 2, 4, AK, BKM>(EMI_GEMM_ARGS);
+    case 5:
+      if constexpr (!AK && !BKM) return launch_bf16_pingpong(EMI_GEMM_ARGS);
+      else return launch_bf16<256, 256, 64, 2, 2, 4, AK, BKM>(EMI_GEMM_ARGS);
     case 2: return launch_bf16<256, 256, 32, 4, 2, 4, AK, BKM>(EMI_GEMM_ARGS);
     default: return launch_bf16<128, 128, 64, 2, 2, 2, AK, BKM>(EMI_GEMM_ARGS);
   }
@@ -496,6 +803,12 @@ static int launch_generic(hipStream_t st, const void* A, const void* B, const vo
 }  // namespace emi
 
 using namespace emi;
+
+#ifdef EMI_GEMM_TRACE
+extern "C" int emi_debug_gemm_trace(unsigned long long* out) {
+  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(emi_gemm_trace_buf), sizeof(unsigned long long) * 8 * 40);
+}
+#endif
 
 extern "C" int emi_gemm(emi_stream_t stream, const void* A, const void* B, const void* R, void* C, int64_t M, int64_t N,
                         int64_t K, int64_t lda, int64_t ldb, int64_t ldr, int64_t ldc, int trans_a, int trans_b,
