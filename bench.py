@@ -81,13 +81,15 @@ def layer_flops(cfg):
 
 
 def gemm_launches(cfg):
-    """(trans_a, trans_b, M, N, K) of the 21 GEMM launches of one fwd+VJP step."""
+    """(role, M, N, K) of the 21 GEMM launches of one fwd+VJP step.  All of them run in
+    the NT layout C[M,N] = A[M,K] . B[N,K]^T: the weight is transposed for dX and both
+    operands are transposed for dW (ops.matmul_nt)."""
     D, H, T = cfg["dim"], cfg["hidden_dim"], cfg["batch"] * cfg["seq"]
     out = []
     for (n_out, k_in) in [(D, D)] * 4 + [(H, D)] * 2 + [(D, H)]:
-        out.append((0, 1, T, n_out, k_in))        # Y  = X W^T
-        out.append((0, 1, T, k_in, n_out))        # dX = dY (W^T)^T, on the transposed weight
-        out.append((1, 0, n_out, k_in, T))        # dW = dY^T X
+        out.append(("Y", T, n_out, k_in))         # Y  = X W^T
+        out.append(("dX", T, k_in, n_out))        # dX = dY (W^T)^T
+        out.append(("dW", n_out, k_in, T))        # dW = dY^T (X^T)^T
     return out
 
 
@@ -96,26 +98,19 @@ def bench_gemms(cfg, iters):
     from enzyme_ad.jax import ops
     D, H, T = cfg["dim"], cfg["hidden_dim"], cfg["batch"] * cfg["seq"]
     big = max(D, H)
-    bufs = {"tok_a": torch.randn((T, big), device="cuda").to(torch.bfloat16),
-            "tok_b": torch.randn((T, big), device="cuda").to(torch.bfloat16),
-            "w": (torch.randn((big, big), device="cuda") * 0.02).to(torch.bfloat16)}
+    flat_a = torch.randn((T * big,), device="cuda").to(torch.bfloat16)
+    flat_b = (torch.randn((T * big,), device="cuda") * 0.02).to(torch.bfloat16)
     calls = []
-    for (ta, tb, M, N, K) in gemm_launches(cfg):
-        if not ta and tb:      # X[T,K] . W[N,K]^T
-            a, b = bufs["tok_a"][:, :K].contiguous(), bufs["w"][:N, :K].contiguous()
-        elif not ta and not tb:    # dY[T,K] . W[K,N]
-            a, b = bufs["tok_a"][:, :K].contiguous(), bufs["w"][:K, :N].contiguous()
-        else:                  # dY[T,M]^T . X[T,N]
-            a, b = bufs["tok_a"][:, :M].contiguous(), bufs["tok_b"][:, :N].contiguous()
-        calls.append((a, b, bool(ta), bool(tb), 2.0 * M * N * K))
-    per_layout = {}
-    for name, sel in (("NT", (False, True)), ("TN", (True, False))):
-        mine = [c for c in calls if (c[2], c[3]) == sel]
-        t = event_time(lambda: [ops.gemm(a, b, ta, tb) for (a, b, ta, tb, _) in mine], iters)
-        fl = sum(c[4] for c in mine)
-        per_layout[name] = dict(launches=len(mine), seconds=t, tflops=fl / t / 1e12)
-    t_all = event_time(lambda: [ops.gemm(a, b, ta, tb) for (a, b, ta, tb, _) in calls], iters)
-    return t_all, sum(c[4] for c in calls), len(calls), per_layout
+    for (role, M, N, K) in gemm_launches(cfg):
+        calls.append((role, flat_a[:M * K].view(M, K), flat_b[:N * K].view(N, K), 2.0 * M * N * K))
+    per_role = {}
+    for role in ("Y", "dX", "dW"):
+        mine = [c for c in calls if c[0] == role]
+        t = event_time(lambda: [ops.gemm(a, b, False, True) for (_, a, b, _) in mine], iters)
+        fl = sum(c[3] for c in mine)
+        per_role[role] = dict(launches=len(mine), seconds=t, tflops=fl / t / 1e12)
+    t_all = event_time(lambda: [ops.gemm(a, b, False, True) for (_, a, b, _) in calls], iters)
+    return t_all, sum(c[3] for c in calls), len(calls), per_role
 
 
 def bench_kernels(cfg, iters):
@@ -272,15 +267,15 @@ def main():
     pretty_print_table(name, "HIP", "rocm", "BothRev", dt) if False else log(
         "%s\tHIP\trocm\tPrimal+VJP\t%.6f s  (%.1f TFLOP/s over %.2f TFLOP algorithmic)" % (name, dt, fl["total"] / dt / 1e12, fl["total"] / 1e12))
 
-    t_gemm, gemm_fl, n_gemm, per_layout = bench_gemms(cfg, max(2, min(args.steps, 5)))
-    roofline = dict(bound="mfma", kernel="gemm_bf16_kernel<256,256,64,2,2,4> (14 NT + 7 TN launches per step; %d in all)" % n_gemm,
+    t_gemm, gemm_fl, n_gemm, per_layout = bench_gemms(cfg, max(5, min(args.steps, 20)))
+    roofline = dict(bound="mfma", kernel="gemm_bf16_nt_pingpong_kernel (256x256x64 tiles; %d launches per step: Y, dX, dW of 7 weights)" % n_gemm,
                     achieved=gemm_fl / t_gemm / 1e12, peak=PEAK_BF16_TFLOPS, unit="TFLOP/s",
                     frac=gemm_fl / t_gemm / 1e12 / PEAK_BF16_TFLOPS,
                     traffic=GEMM_TRAFFIC_BYTES_PER_LAUNCH if (args.seq, args.batch) == (C5["seq"], C5["batch"]) else None,
                     avg_launch_us=t_gemm / n_gemm * 1e6, flops_per_launch=gemm_fl / n_gemm,
-                    per_layout={k: dict(tflops=round(v["tflops"], 1), avg_launch_us=round(v["seconds"] / v["launches"] * 1e6, 1))
+                    per_role={k: dict(tflops=round(v["tflops"], 1), avg_launch_us=round(v["seconds"] / v["launches"] * 1e6, 1))
                                 for k, v in per_layout.items()})
-    log("GEMM: %.1f TFLOP/s (%.1f%% of bf16 MFMA peak); per layout %s" % (roofline["achieved"], 100 * roofline["frac"], roofline["per_layout"]))
+    log("GEMM: %.1f TFLOP/s (%.1f%% of bf16 MFMA peak); per role %s" % (roofline["achieved"], 100 * roofline["frac"], roofline["per_role"]))
 
     kernels = None
     if not args.no_kernels:

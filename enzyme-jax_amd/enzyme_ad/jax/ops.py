@@ -98,6 +98,7 @@ class Tape:
     def backward(self, outputs, cotangents, wrt):
         """Cotangents of `wrt` (list of tensors) given cotangents of `outputs`."""
         ct = {}
+        _transposed.clear()
         for o, c in zip(outputs, cotangents):
             if c is None:
                 continue
@@ -120,6 +121,7 @@ class Tape:
                     continue
                 ct[id(i)] = g if id(i) not in done else add(ct[id(i)], g)
                 done.add(id(i))
+        _transposed.clear()
         return [ct.get(id(w)) for w in wrt]
 
 
@@ -214,6 +216,22 @@ def transpose(a):
     return out
 
 
+_transposed = {}      # (data_ptr, shape) -> a^T, valid for the duration of one Tape.backward
+
+
+def _transpose_shared(a):
+    """a^T, computed once per reverse pass for an operand several adjoint GEMMs
+    share (the normed activations feed wq/wk/wv, and w1/w3)."""
+    key = (a.data_ptr(), tuple(a.shape), a.dtype)
+    hit = _transposed.get(key)
+    if hit is None:
+        rows, cols = a.shape
+        out = torch.empty((cols, rows), dtype=a.dtype, device=a.device)
+        N.check(N.lib().emi_transpose(_stream(), _p(a), _p(out), rows, cols, _code(a)))
+        hit = _transposed[key] = (out, a)       # keeps `a` alive so the pointer cannot be reused
+    return hit[0]
+
+
 def gemm(a, b, trans_a=False, trans_b=False, residual=None):
     """op(a) . op(b) [+ residual] on 2-D operands; fp32 accumulate."""
     _dev(a, b, residual)
@@ -246,8 +264,16 @@ def matmul_nt(x, w, residual=None):
         # dX = dY . W: W is transposed first (2|W| bytes of HBM traffic) so that the
         # contraction index is innermost in both operands and the GEMM runs on the
         # k-contiguous path, which is ~15% faster than the k-major one at these shapes.
-        dx = gemm(c2, transpose(w), False, True, ax).reshape(x.shape)
-        dw = gemm(c2, x2, True, False, acc[1])                   # dW = dY^T . X (TN)
+        dx = gemm(c2, _transpose_shared(w), False, True, ax).reshape(x.shape)
+        # dW = dY^T . X contracts over tokens, the slow index of both operands.  The
+        # k-major kernel has to fetch its fragments with the transposing LDS load,
+        # which makes it LDS-bound; transposing both operands in HBM and running the
+        # k-contiguous kernel is faster overall, and X^T is shared by the projections
+        # that read the same activations.
+        if c2.dtype == torch.bfloat16 and c2.shape[0] >= 2048:
+            dw = gemm(_transpose_shared(c2), _transpose_shared(x2), False, True, acc[1])
+        else:
+            dw = gemm(c2, x2, True, False, acc[1])               # dW = dY^T . X (TN)
         out = [dx, dw]
         if residual is not None:
             out.append(_accumulate(acc[2], c))
