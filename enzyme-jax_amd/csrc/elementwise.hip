@@ -69,16 +69,33 @@ __global__ __launch_bounds__(256) void rmsnorm_fwd_kernel(const T* __restrict__ 
   }
 }
 
-// Adjoint.  Blocks walk rows with a grid stride and keep this thread's share
-// of dgamma in registers; partial[blockIdx*RPB + rib][dim] is reduced by
-// colsum_kernel.  dx = [dx_add +] r*g - x * r^3 * mean(g*x), g = dy*gamma.
-template <typename T, int TPR, int NCH>
+// Sums of NV values over the TPR threads of a row with one barrier.
+template <int TPR, int NV> __device__ __forceinline__ void row_reduce_n(float (&v)[NV], float (*red)[4][NV], int it) {
+#pragma unroll
+  for (int i = 0; i < NV; i++) v[i] = wave_sum(v[i]);
+  if constexpr (TPR == 256) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    float(*buf)[NV] = red[it & 1];
+    if (lane == 0) {
+#pragma unroll
+      for (int i = 0; i < NV; i++) buf[wave][i] = v[i];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < NV; i++) v[i] = buf[0][i] + buf[1][i] + buf[2][i] + buf[3][i];
+  }
+}
+
+// Adjoint.  Blocks walk rows with a grid stride, NR rows per step, and keep this
+// thread's share of dgamma in registers; partial[blockIdx*RPB + rib][dim] is reduced
+// by colsum_kernel.  dx = [dx_add +] r*g - x * r^3 * mean(g*x), g = dy*gamma.
+template <typename T, int TPR, int NCH, int NR>
 __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const T* __restrict__ x, const T* __restrict__ gamma,
                                                           const T* __restrict__ dy, const T* dx_add, T* dx,
                                                           float* __restrict__ partial, int64_t rows, int dim,
                                                           float eps) {
   constexpr int RPB = 256 / TPR;
-  __shared__ float red[2][4][2];
+  __shared__ float red[2][4][2 * NR];
   const int tir = threadIdx.x % TPR;
   const int rib = threadIdx.x / TPR;
   const int nchunk = dim >> 3;
@@ -90,63 +107,80 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const T* __restrict__ 
     for (int e = 0; e < 8; e++) acc[j][e] = 0.f, gm[j][e] = 0.f;
     if (c < nchunk) Vec8<T>::load(gamma + c * 8, gm[j]);
   }
-  const int64_t nrow_iter = (rows + RPB - 1) / RPB;   // row groups
-  // Rows are software pipelined: the loads of the next row are issued before the
+  const int64_t nstep = (rows + RPB * NR - 1) / (RPB * NR);   // steps of RPB*NR rows
+  // Steps are software pipelined: the loads of the next step are issued before the
   // reduction (shuffles, LDS, barrier) of the current one, which keeps twice the
   // bytes in flight per block.
-  typename Vec8<T>::Raw xn[NCH], gn[NCH];      // kept in storage format to save registers
-  auto load_row = [&](int64_t rg) {
-    const int64_t row = rg * RPB + rib;
+  typename Vec8<T>::Raw xn[NR][NCH], gn[NR][NCH];      // kept in storage format to save registers
+  auto load_step = [&](int64_t sg) {
 #pragma unroll
-    for (int j = 0; j < NCH; j++) {
-      const int c = tir + j * TPR;
-      if (rg < nrow_iter && row < rows && c < nchunk) {
-        xn[j] = Vec8<T>::load_raw(x + row * dim + c * 8);
-        gn[j] = Vec8<T>::load_raw(dy + row * dim + c * 8);
-      } else {
-        xn[j] = Vec8<T>::zero_raw();
-        gn[j] = Vec8<T>::zero_raw();
+    for (int u = 0; u < NR; u++) {
+      const int64_t row = (sg * NR + u) * RPB + rib;
+#pragma unroll
+      for (int j = 0; j < NCH; j++) {
+        const int c = tir + j * TPR;
+        if (sg < nstep && row < rows && c < nchunk) {
+          xn[u][j] = Vec8<T>::load_raw(x + row * dim + c * 8);
+          gn[u][j] = Vec8<T>::load_raw(dy + row * dim + c * 8);
+        } else {
+          xn[u][j] = Vec8<T>::zero_raw();
+          gn[u][j] = Vec8<T>::zero_raw();
+        }
       }
     }
   };
-  load_row(blockIdx.x);
+  load_step(blockIdx.x);
   int it = 0;
-  for (int64_t rg = blockIdx.x; rg < nrow_iter; rg += gridDim.x, ++it) {
-    const int64_t row = rg * RPB + rib;
-    const bool active = row < rows;
-    float xv[NCH][8], gv[NCH][8];
-    float ss = 0.f, gx = 0.f;
+  for (int64_t sg = blockIdx.x; sg < nstep; sg += gridDim.x, ++it) {
+    typename Vec8<T>::Raw xc[NR][NCH], gc[NR][NCH];
+    float red_v[2 * NR];
 #pragma unroll
-    for (int j = 0; j < NCH; j++) {
-      Vec8<T>::unpack(xn[j], xv[j]);
-      Vec8<T>::unpack(gn[j], gv[j]);
+    for (int u = 0; u < NR; u++) {
+      float ss = 0.f, gx = 0.f;
 #pragma unroll
-      for (int e = 0; e < 8; e++) {
-        ss += xv[j][e] * xv[j][e];
-        gx += gv[j][e] * gm[j][e] * xv[j][e];
-      }
-    }
-    load_row(rg + gridDim.x);
-    row_reduce2<TPR>(ss, gx, red, it);
-    const float r = 1.0f / sqrtf(ss / (float)dim + eps);
-    const float coef = r * r * r * (gx / (float)dim);
-#pragma unroll
-    for (int j = 0; j < NCH; j++) {
-      const int c = tir + j * TPR;
-      if (active && c < nchunk) {
-        float o[8];
+      for (int j = 0; j < NCH; j++) {
+        xc[u][j] = xn[u][j];
+        gc[u][j] = gn[u][j];
+        float xv[8], gv[8];
+        Vec8<T>::unpack(xc[u][j], xv);
+        Vec8<T>::unpack(gc[u][j], gv);
 #pragma unroll
         for (int e = 0; e < 8; e++) {
-          acc[j][e] += gv[j][e] * xv[j][e] * r;
-          o[e] = r * gv[j][e] * gm[j][e] - xv[j][e] * coef;
+          ss += xv[e] * xv[e];
+          gx += gv[e] * gm[j][e] * xv[e];
         }
-        if (dx_add != nullptr) {
-          float a[8];
-          Vec8<T>::load(dx_add + row * dim + c * 8, a);
+      }
+      red_v[2 * u] = ss;
+      red_v[2 * u + 1] = gx;
+    }
+    load_step(sg + gridDim.x);
+    row_reduce_n<TPR, 2 * NR>(red_v, red, it);
 #pragma unroll
-          for (int e = 0; e < 8; e++) o[e] += a[e];
+    for (int u = 0; u < NR; u++) {
+      const int64_t row = (sg * NR + u) * RPB + rib;
+      const bool active = row < rows;
+      const float r = 1.0f / sqrtf(red_v[2 * u] / (float)dim + eps);
+      const float coef = r * r * r * (red_v[2 * u + 1] / (float)dim);
+#pragma unroll
+      for (int j = 0; j < NCH; j++) {
+        const int c = tir + j * TPR;
+        if (active && c < nchunk) {
+          float xv[8], gv[8], o[8];
+          Vec8<T>::unpack(xc[u][j], xv);
+          Vec8<T>::unpack(gc[u][j], gv);
+#pragma unroll
+          for (int e = 0; e < 8; e++) {
+            acc[j][e] += gv[e] * xv[e] * r;
+            o[e] = r * gv[e] * gm[j][e] - xv[e] * coef;
+          }
+          if (dx_add != nullptr) {
+            float a[8];
+            Vec8<T>::load(dx_add + row * dim + c * 8, a);
+#pragma unroll
+            for (int e = 0; e < 8; e++) o[e] += a[e];
+          }
+          Vec8<T>::store(dx + row * dim + c * 8, o);
         }
-        Vec8<T>::store(dx + row * dim + c * 8, o);
       }
     }
   }
@@ -207,26 +241,36 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_generic_kernel(const T* __res
   }
 }
 
-// Column sums of partial[nparts][dim] in chunks of 128 rows: block (cb, rc) adds
-// rows [128*rc, 128*rc+128) of 128 columns (32 float4 columns x 8 row lanes, so a
-// wavefront reads 512 contiguous bytes of two rows) into row rc of `out`.
-// The launcher applies it until one row is left; the last pass writes type T.
+// Column sums of partial[nparts][dim]: block (cb, rc) adds rows [CS_ROWS*rc, CS_ROWS*rc +
+// CS_ROWS) of 64 columns (16 float4 columns x 16 row lanes, so a wavefront reads 256
+// contiguous bytes of four rows) into row rc of `out`.  The launcher applies it
+// until one row is left (one pass for the grids the adjoint uses); the last pass
+// writes type T.
+constexpr int CS_ROWS = 512;
 template <typename TO>
 __global__ __launch_bounds__(256) void colsum_kernel(const float* __restrict__ partial, int nparts, int64_t dim,
                                                      TO* __restrict__ out) {
-  __shared__ float red[8][128 + 4];
-  const int cq = threadIdx.x & 31, rl = threadIdx.x >> 5;
-  const int64_t col = (int64_t)blockIdx.x * 128 + cq * 4;
-  const int r0 = blockIdx.y * 128;
-  const int r1 = r0 + 128 < nparts ? r0 + 128 : nparts;
+  __shared__ float red[16][64 + 4];
+  const int cq = threadIdx.x & 15, rl = threadIdx.x >> 4;
+  const int64_t col = (int64_t)blockIdx.x * 64 + cq * 4;
+  const int r0 = blockIdx.y * CS_ROWS;
+  const int r1 = r0 + CS_ROWS < nparts ? r0 + CS_ROWS : nparts;
   float s[4] = {0.f, 0.f, 0.f, 0.f};
   if ((dim & 3) == 0 && col + 4 <= dim) {
-    for (int p = r0 + rl; p < r1; p += 8) {
-      const float4 v = *reinterpret_cast<const float4*>(partial + (int64_t)p * dim + col);
-      s[0] += v.x; s[1] += v.y; s[2] += v.z; s[3] += v.w;
+    float4 v[4];
+    int p = r0 + rl;
+    for (; p + 48 < r1; p += 64) {           // four independent loads in flight
+#pragma unroll
+      for (int u = 0; u < 4; u++) v[u] = *reinterpret_cast<const float4*>(partial + (int64_t)(p + 16 * u) * dim + col);
+#pragma unroll
+      for (int u = 0; u < 4; u++) { s[0] += v[u].x; s[1] += v[u].y; s[2] += v[u].z; s[3] += v[u].w; }
+    }
+    for (; p < r1; p += 16) {
+      const float4 w = *reinterpret_cast<const float4*>(partial + (int64_t)p * dim + col);
+      s[0] += w.x; s[1] += w.y; s[2] += w.z; s[3] += w.w;
     }
   } else {
-    for (int p = r0 + rl; p < r1; p += 8)
+    for (int p = r0 + rl; p < r1; p += 16)
 #pragma unroll
       for (int e = 0; e < 4; e++)
         if (col + e < dim) s[e] += partial[(int64_t)p * dim + col + e];
@@ -234,12 +278,12 @@ __global__ __launch_bounds__(256) void colsum_kernel(const float* __restrict__ p
 #pragma unroll
   for (int e = 0; e < 4; e++) red[rl][cq * 4 + e] = s[e];
   __syncthreads();
-  if (threadIdx.x < 128) {
-    const int64_t c = (int64_t)blockIdx.x * 128 + threadIdx.x;
+  if (threadIdx.x < 64) {
+    const int64_t c = (int64_t)blockIdx.x * 64 + threadIdx.x;
     if (c < dim) {
       float t = 0.f;
 #pragma unroll
-      for (int i = 0; i < 8; i++) t += red[i][threadIdx.x];
+      for (int i = 0; i < 16; i++) t += red[i][threadIdx.x];
       out[(int64_t)blockIdx.y * dim + c] = from_f32<TO>(t);
     }
   }
@@ -467,7 +511,9 @@ static inline void rms_bwd_shape(int64_t rows, int64_t dim, int* tpr, int* nch, 
     *nch = per <= 1 ? 1 : (per <= 2 ? 2 : 4);
     const int rpb = 256 / *tpr;
     const int64_t groups = (rows + rpb - 1) / rpb;
-    const int64_t cap = (*tpr == 64) ? 256 : 1024;   // 4 resident blocks per CU, one wave of blocks
+    // Two resident blocks per CU: more blocks add partial rows (written here, read
+    // again by the column sum) without adding bandwidth.
+    const int64_t cap = (*tpr == 64) ? 128 : 512;
     *grid = groups < cap ? (groups > 0 ? groups : 1) : cap;
     *nparts = *grid * rpb;
   } else {
@@ -521,7 +567,7 @@ static int rmsnorm_bwd_launch(hipStream_t st, const void* x, const void* gamma, 
                        rows, dim, eps);
   } else {
 #define EMI_RMS_BWD(TPR, NCH)                                                                                   \
-  hipLaunchKernelGGL((rmsnorm_bwd_kernel<T, TPR, NCH>), dim3((unsigned)grid), dim3(256), 0, st, xp, gp, dyp, ap, dxp, \
+  hipLaunchKernelGGL((rmsnorm_bwd_kernel<T, TPR, NCH, (sizeof(T) == 2 ? 2 : 1)>), dim3((unsigned)grid), dim3(256), 0, st, xp, gp, dyp, ap, dxp, \
                      part, rows, (int)dim, eps)
     if (tpr == 64 && nch == 1) EMI_RMS_BWD(64, 1);
     else if (tpr == 64) EMI_RMS_BWD(64, 2);
@@ -531,20 +577,20 @@ static int rmsnorm_bwd_launch(hipStream_t st, const void* x, const void* gamma, 
 #undef EMI_RMS_BWD
   }
   EMI_CHECK_LAUNCH("emi_rmsnorm_bwd");
-  // [nparts, dim] -> [ceil(nparts/128), dim] -> ... -> dgamma
+  // [nparts, dim] -> [ceil(nparts/CS_ROWS), dim] -> ... -> dgamma
   float* cur = part;
   float* nxt = part + nparts * dim;
   int64_t n = nparts;
-  while (n > 128) {
-    const int64_t m = (n + 127) / 128;
-    hipLaunchKernelGGL(colsum_kernel<float>, dim3(blocks_for(dim, 128), (unsigned)m), dim3(256), 0, st, cur, (int)n, dim, nxt);
+  while (n > CS_ROWS) {
+    const int64_t m = (n + CS_ROWS - 1) / CS_ROWS;
+    hipLaunchKernelGGL(colsum_kernel<float>, dim3(blocks_for(dim, 64), (unsigned)m), dim3(256), 0, st, cur, (int)n, dim, nxt);
     EMI_CHECK_LAUNCH("emi_rmsnorm_bwd(colsum)");
     float* t = cur;
     cur = nxt;
     nxt = t;
     n = m;
   }
-  hipLaunchKernelGGL(colsum_kernel<T>, dim3(blocks_for(dim, 128), 1), dim3(256), 0, st, cur, (int)n, dim,
+  hipLaunchKernelGGL(colsum_kernel<T>, dim3(blocks_for(dim, 64), 1), dim3(256), 0, st, cur, (int)n, dim,
                      static_cast<T*>(dgamma));
   EMI_CHECK_LAUNCH("emi_rmsnorm_bwd(colsum)");
   return EMI_OK;
@@ -579,7 +625,7 @@ extern "C" size_t emi_rmsnorm_bwd_workspace_bytes(int64_t rows, int64_t dim) {
   int64_t grid, nparts;
   rms_bwd_shape(rows, dim, &tpr, &nch, &grid, &nparts);
   // first-level partial rows + one ping-pong area for the second level of the column sum
-  return ((size_t)nparts + (size_t)((nparts + 127) / 128)) * (size_t)dim * sizeof(float);
+  return ((size_t)nparts + (size_t)((nparts + CS_ROWS - 1) / CS_ROWS)) * (size_t)dim * sizeof(float);
 }
 
 extern "C" int emi_rmsnorm_bwd(emi_stream_t stream, const void* x, const void* gamma, const void* dy,
