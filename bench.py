@@ -172,8 +172,10 @@ def bench_kernels(cfg, iters):
     ws = torch.empty(wsb, dtype=torch.uint8, device="cuda")
     sc = d ** -0.5
     fl = 2.0 * B * h * S * S * d
-    mfma("attn_fwd_c3", lambda: N.check(lib.emi_attn_fwd(st, P(q), P(k), P(v), P(o), P(lse), B, h, S, d, h * S * d, S * d, d,
-                                                         sc, 1, N.EMI_BF16)), fl)
+    fwsb = lib.emi_attn_fwd_workspace_bytes(B, h, S, d)
+    fws = torch.empty(fwsb, dtype=torch.uint8, device="cuda")
+    mfma("attn_fwd_c3", lambda: N.check(lib.emi_attn_fwd_ws(st, P(q), P(k), P(v), P(o), P(lse), P(fws), fwsb, B, h, S, d,
+                                                            h * S * d, S * d, d, sc, 1, N.EMI_BF16)), fl)
     mfma("attn_bwd_c3", lambda: N.check(lib.emi_attn_bwd(st, P(q), P(k), P(v), P(o), P(lse), P(do), P(dq), P(dk), P(dv), P(ws), wsb,
                                                          B, h, S, d, h * S * d, S * d, d, sc, 1, N.EMI_BF16)), 2.5 * fl)
     return out

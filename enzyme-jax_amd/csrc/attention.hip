@@ -16,6 +16,8 @@
 // Generic path (fp32 or any other head_dim <= 256): one wavefront per query
 // (or key) row, plain fp32 FMA, same maths.
 #include <initializer_list>
+#include <type_traits>
+#include <stdlib.h>
 
 #include "emi_device.h"
 
@@ -37,6 +39,22 @@ struct AttnShape {
   int seq, heads;
   int64_t sb, sh, ss;   // element strides of batch, head, sequence position
 };
+
+// Work assignment of the MFMA kernels.  Consecutive workgroup ids go to different XCDs
+// (8 of them, each with its own L2), so a grid of (blocks per head) x (heads) that simply
+// used blockIdx would hand every XCD the same few block positions of every head: with a
+// causal mask that is a 2.4x imbalance between XCDs, and K/V of one head would be
+// fetched into all eight L2s.  Instead every XCD gets a contiguous run of heads with all
+// of their blocks, in the order given (longest first).
+__device__ __forceinline__ void attn_block_coords(int* blk, int* bh) {
+  const int nblk = gridDim.x, total = gridDim.x * gridDim.y;
+  const int lin = blockIdx.y * gridDim.x + blockIdx.x;
+  const int per = total >> 3, rem = total & 7;
+  const int xcd = lin & 7, idx = lin >> 3;
+  const int v = xcd * per + (xcd < rem ? xcd : rem) + idx;
+  *bh = v / nblk;
+  *blk = v - *bh * nblk;
+}
 
 // ===========================================================================
 // Generic path
@@ -321,8 +339,9 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_kernel(const uint16_t* _
   EMI_LDS uint8_t* smem = (EMI_LDS uint8_t*)smem_raw;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int qblk = gridDim.x - 1 - blockIdx.x;       // longest rows first
-  const int bh = blockIdx.y;
+  int blk, bh;
+  attn_block_coords(&blk, &bh);
+  const int qblk = gridDim.x - 1 - blk;              // longest rows first
   const int64_t base = (int64_t)(bh / sh.heads) * sh.sb + (int64_t)(bh % sh.heads) * sh.sh;
   const int seq = sh.seq;
   const int q0 = qblk * BQ + wave * 32;
@@ -430,6 +449,289 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_kernel(const uint16_t* _
   }
 }
 
+// V^T for the forward pass: vt[bh][d][s_pad] = v[b][s][h][d] (keys contiguous, rows
+// padded with zeros to a multiple of 64 keys), so that the P.V product can fetch its
+// V operand with plain 16-byte LDS reads instead of the slow transposing ones.
+template <int D>
+__global__ __launch_bounds__(256) void attn_vt_kernel(const uint16_t* __restrict__ v, uint16_t* __restrict__ vt,
+                                                      AttnShape sh, int s_pad) {
+  __shared__ uint16_t tile[64][66];
+  const int k0 = blockIdx.x * 64, d0 = blockIdx.y * 64, bh = blockIdx.z;
+  const int64_t base = (int64_t)(bh / sh.heads) * sh.sb + (int64_t)(bh % sh.heads) * sh.sh;
+#pragma unroll
+  for (int i = 0; i < 2; i++) {
+    const int idx = threadIdx.x + i * 256, r = idx >> 3, c = idx & 7;
+    uint4 w = make_uint4(0, 0, 0, 0);
+    if (k0 + r < sh.seq) w = *reinterpret_cast<const uint4*>(v + base + (int64_t)(k0 + r) * sh.ss + d0 + c * 8);
+    const uint32_t u[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+    for (int e = 0; e < 8; e++) tile[r][c * 8 + e] = (uint16_t)(u[e >> 1] >> ((e & 1) * 16));
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 2; i++) {
+    const int idx = threadIdx.x + i * 256, dd = idx >> 3, c = idx & 7;
+    uint32_t u[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) u[e] = (uint32_t)tile[c * 8 + 2 * e][dd] | ((uint32_t)tile[c * 8 + 2 * e + 1][dd] << 16);
+    *reinterpret_cast<uint4*>(vt + ((int64_t)bh * D + d0 + dd) * s_pad + k0 + c * 8) = make_uint4(u[0], u[1], u[2], u[3]);
+  }
+}
+
+// LDS tile [D][64 keys] of V^T: 128-byte rows, 16-byte chunk c of row r at chunk
+// c ^ ((r >> 1) & 7) (16 consecutive rows at one logical chunk cover all 64 banks).
+template <int D, int NW>
+__device__ __forceinline__ void load_vt_tile(__amdgpu_buffer_rsrc_t rsrc, EMI_LDS uint8_t* lds, int wave, int lane,
+                                             int key0, int s_pad) {
+  constexpr int NLOAD = D * 128 / 1024 / NW;       // wave-loads of 8 rows x 128 bytes
+  static_assert(NLOAD >= 1, "V^T tile smaller than one pass of the block");
+#pragma unroll
+  for (int it = 0; it < NLOAD; it++) {
+    const int r = (it * NW + wave) * 8 + (lane >> 3);
+    const int lc = (lane & 7) ^ ((r >> 1) & 7);
+    const uint32_t voff = (uint32_t)(r * s_pad + key0 + lc * 8) * 2u;      // key0 < s_pad always
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, lds + (it * NW + wave) * 1024, 16, voff, 0, 0, 0);
+  }
+}
+// Operand fragment "32 of D x 8 keys per lane": lane l holds D-index row_base + (l & 31),
+// keys 8*chunk .. +7 of the tile.
+__device__ __forceinline__ bf16x8_t vt_frag(const EMI_LDS uint8_t* tile, int row_base, int chunk, int lane) {
+  const int row = row_base + (lane & 31);
+  return *reinterpret_cast<const EMI_LDS bf16x8_t*>(tile + row * 128 + ((chunk ^ ((row >> 1) & 7)) << 4));
+}
+// Key permutation inside a 32-row score tile (swaps bits 2 and 3): MFMA row m holds key
+// perm_key(m), which makes registers 8s..8s+7 of a lane's accumulator eight consecutive
+// keys, the order a 16-byte read of a V^T row delivers.
+__device__ __forceinline__ int perm_key(int m) { return (m & ~12) | ((m & 4) << 1) | ((m & 8) >> 1); }
+
+// ---------------------------------------------------------------------------
+// Forward, ping-pong form: block = 8 waves x 32 queries in two groups of four, one
+// wavefront of each group per SIMD.  A key/value tile step is two phases separated by
+// s_barrier: a VALU phase (softmax of the scores in registers) and an MFMA phase (scores
+// of the next tile, then P.V of this one).  The groups run one phase apart, so on every
+// SIMD the softmax of one wavefront overlaps the matrix work of the other.
+//   bundle b(j) = {K tile j+1, V tile j}: what MFMA phase j reads; three bundles in LDS.
+//   MFMA phase j ends by issuing the loads of b(j+2) (its slot was last read two phases
+//   ago by both groups) and waiting for its own part of b(j+1) before the barrier.
+// The running maximum is only raised when some row's tile maximum exceeds it by more
+// than 8 (in log2 units), so the rescaling of O runs on a few early tiles only; P then
+// stays below 2^8 and the final O/l and log-sum-exp are exact for whatever m was used.
+// ---------------------------------------------------------------------------
+#ifdef EMI_ATTN_TRACE
+__device__ unsigned long long emi_attn_trace_buf[8 * 40];
+#define EMI_ATRACE() do { if (tracing && nts < 40) ts[nts++] = __builtin_readcyclecounter(); } while (0)
+#else
+#define EMI_ATRACE() do { } while (0)
+#endif
+template <int D, bool VT>
+__global__ __launch_bounds__(512) void attn_fwd_pp_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ k,
+                                                          const uint16_t* __restrict__ v, uint16_t* __restrict__ o,
+                                                          float* __restrict__ lse, AttnShape sh, uint32_t head_bytes,
+                                                          float scale_log2e, int causal, int s_pad) {
+  constexpr int BQ = 256, BKV = 64, NW = 8;
+  constexpr int TILE = BKV * D * 2, BUNDLE = 2 * TILE;
+  constexpr int LPB = 2 * (BKV * D * 2 / 1024 / NW);       // loads per wave per bundle
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem_raw[];
+  EMI_LDS uint8_t* smem = (EMI_LDS uint8_t*)smem_raw;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  int blk, bh;
+  attn_block_coords(&blk, &bh);
+  const int qblk = gridDim.x - 1 - blk;              // longest rows first
+  const int64_t base = (int64_t)(bh / sh.heads) * sh.sb + (int64_t)(bh % sh.heads) * sh.sh;
+  const int seq = sh.seq;
+  const int q0 = qblk * BQ + wave * 32;
+  const int qrow = q0 + (lane & 31);
+
+  bf16x8_t qf[D / 16];
+  load_reg_rows<D>(q + base, qrow, seq, sh.ss, lane, qf);
+
+  const __amdgpu_buffer_rsrc_t rK = attn_rsrc(k + base, head_bytes);
+  // VT: v is the transposed copy [bh][D][s_pad]
+  const __amdgpu_buffer_rsrc_t rV = VT ? attn_rsrc(v + (int64_t)bh * D * s_pad, (uint32_t)(D * s_pad * 2))
+                                       : attn_rsrc(v + base, head_bytes);
+  const int kv_end = causal ? (qblk * BQ + BQ < seq ? qblk * BQ + BQ : seq) : seq;
+  const int nt = (kv_end + BKV - 1) / BKV;
+  const int krow_l = VT ? perm_key(lane & 31) : (lane & 31);      // K row this lane feeds into the score MFMAs
+
+  f32x16_t acc_o[D / 32];
+#pragma unroll
+  for (int dt = 0; dt < D / 32; dt++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc_o[dt][r] = 0.f;
+  float m = kNegBig, l = 0.f;
+  f32x16_t s[2];
+  bf16x8_t pf[2][2];
+
+#ifdef EMI_ATTN_TRACE
+  unsigned long long ts[40];
+  int nts = 0;
+  bool tracing = false;
+#endif
+  auto phase_end = [&]() __attribute__((always_inline)) {
+    __builtin_amdgcn_sched_barrier(0);
+    EMI_ATRACE();
+    __builtin_amdgcn_s_barrier();
+    EMI_ATRACE();
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  auto issue_bundle = [&](int jb, int slot) __attribute__((always_inline)) {
+    EMI_LDS uint8_t* sK = smem + slot * TILE;
+    EMI_LDS uint8_t* sV = smem + 3 * TILE + slot * TILE;
+    load_rows_tile<D, BKV, NW>(rK, sK, wave, lane, (jb + 1) * BKV, seq, sh.ss);
+    const int vrow0 = jb < 0 ? 0 : jb * BKV;
+    if constexpr (VT) load_vt_tile<D, NW>(rV, sV, wave, lane, vrow0 < s_pad ? vrow0 : 0, s_pad);
+    else load_rows_tile<D, BKV, NW>(rV, sV, wave, lane, vrow0, seq, sh.ss);
+  };
+  // MFMA phase: scores of tile j+1 (DO_S) and P.V of tile j (DO_PV) out of bundle `slot`.
+  // The operand fragments go through a ring of DEPTH registers sets: the LDS read of
+  // operation i + DEPTH is issued right after the MFMA of operation i, so the LDS latency
+  // hides behind DEPTH MFMAs.
+  auto mfma_phase = [&](auto do_s_c, auto do_pv_c, int slot) __attribute__((always_inline)) {
+    constexpr bool DO_S = decltype(do_s_c)::value, DO_PV = decltype(do_pv_c)::value;
+    constexpr int NS = DO_S ? 2 * (D / 16) : 0, NPV = DO_PV ? 4 * (D / 32) : 0, NOP = NS + NPV, DEPTH = 6;
+    // K tiles of the three bundles first, then the V tiles: every fragment address is
+    // one of a few per-lane bases plus an immediate offset below 64 KiB
+    const EMI_LDS uint8_t* sK = smem + slot * TILE;
+    const EMI_LDS uint8_t* sV = smem + 3 * TILE + slot * TILE;
+    auto fetch = [&](int i) __attribute__((always_inline)) -> bf16x8_t {
+      if (i < NS) {
+        const int t = i >> 1, T = i & 1;
+        const int row = T * 32 + krow_l;
+        const int chunk = (t * 2 + (lane >> 5)) ^ swz<D>(row);
+        return *reinterpret_cast<const EMI_LDS bf16x8_t*>(sK + row * (D * 2) + chunk * 16);
+      }
+      const int x = i - NS, dt = x % (D / 32), sI = (x / (D / 32)) & 1, T = x / (2 * (D / 32));
+      if constexpr (VT) return vt_frag(sV, dt * 32, 4 * T + 2 * sI + (lane >> 5), lane);
+      else return col_frag<D>(sV, T * 32 + sI * 16, dt * 32, lane);
+    };
+    if constexpr (DO_S) {
+#pragma unroll
+      for (int T = 0; T < 2; T++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) s[T][r] = 0.f;
+    }
+    bf16x8_t ring[DEPTH];
+#pragma unroll
+    for (int i = 0; i < DEPTH && i < NOP; i++) ring[i] = fetch(i);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < NOP; i++) {
+      if (i < NS) {
+        s[i & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[i % DEPTH], qf[i >> 1], s[i & 1], 0, 0, 0);
+      } else {
+        const int x = i - NS, dt = x % (D / 32), sI = (x / (D / 32)) & 1, T = x / (2 * (D / 32));
+        acc_o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[i % DEPTH], pf[T][sI], acc_o[dt], 0, 0, 0);
+      }
+      if (i + DEPTH < NOP) ring[i % DEPTH] = fetch(i + DEPTH);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  auto softmax = [&](int j) __attribute__((always_inline)) {
+    const int key0 = j * BKV;
+    if ((causal && key0 + BKV - 1 > q0) || key0 + BKV > seq) {
+      asm volatile("" ::: "memory");     // keeps this a branch: most tiles need no mask
+#pragma unroll
+      for (int T = 0; T < 2; T++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const int mrow = acc_row(r, lane);
+          const int key = key0 + T * 32 + (VT ? perm_key(mrow) : mrow);
+          if ((causal && key > qrow) || key >= seq) s[T][r] = kNegBig;
+        }
+    }
+    float mt = s[0][0];
+#pragma unroll
+    for (int T = 0; T < 2; T++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) mt = fmaxf(mt, s[T][r]);
+    mt = fmaxf(mt, __shfl_xor(mt, 32, 64)) * scale_log2e;
+    if (__builtin_amdgcn_ballot_w64(mt > m + 8.0f) != 0) {      // wave-uniform, rare after the first tiles
+      const float m_new = fmaxf(m, mt);
+      const float alpha = fast_exp2(m - m_new);
+      l *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < D / 32; dt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc_o[dt][r] *= alpha;
+      m = m_new;
+    }
+    float rs = 0.f;
+#pragma unroll
+    for (int T = 0; T < 2; T++) {
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const float p = fast_exp2(fmaf(s[T][r], scale_log2e, -m));
+        s[T][r] = p;
+        rs += p;
+      }
+      pf[T][0] = acc_to_frag(s[T], 0);
+      pf[T][1] = acc_to_frag(s[T], 1);
+    }
+    l += rs;
+  };
+  // One tile step; bundle b(j) sits in slot (j + 1) % 3 = SLOT.  Every wavefront runs
+  // every step of its block (the barriers keep the eight in lockstep anyway); tiles in a
+  // wavefront's future are fully masked and contribute exact zeros, and the scores
+  // computed past the last tile are never used.
+  auto step = [&](auto slot_c, int j) __attribute__((always_inline)) {
+    constexpr int SLOT = decltype(slot_c)::value;
+    softmax(j);                                       // VALU phase
+    phase_end();
+    __builtin_amdgcn_s_setprio(1);                    // MFMA phase
+    mfma_phase(std::true_type{}, std::true_type{}, SLOT);
+    __builtin_amdgcn_s_setprio(0);
+    // After the LDS reads of this phase: the compiler orders every LDS read behind all
+    // outstanding direct-to-LDS loads, so loads issued earlier would be waited for here.
+    issue_bundle(j + 2, (SLOT + 2) % 3);
+    __builtin_amdgcn_s_waitcnt(0x0f70 | (LPB & 15));  // vmcnt(LPB): own part of b(j+1) has landed
+    phase_end();
+  };
+
+  issue_bundle(-1, 0);
+  issue_bundle(0, 1);
+  __builtin_amdgcn_s_waitcnt(0x0f70);                 // vmcnt(0)
+  issue_bundle(1, 2);
+  phase_end();
+  if (wave >= 4) phase_end();                         // second group runs one phase behind
+  __builtin_amdgcn_s_setprio(1);
+  mfma_phase(std::true_type{}, std::false_type{}, 0);      // MFMA phase -1
+  __builtin_amdgcn_s_setprio(0);
+  phase_end();
+  for (int j = 0; j < nt; j += 3) {
+#ifdef EMI_ATTN_TRACE
+    tracing = (blockIdx.x == 0 && blockIdx.y == 5 && j >= 30 && j < 36);
+#endif
+    step(std::integral_constant<int, 1>{}, j);
+    if (j + 1 < nt) step(std::integral_constant<int, 2>{}, j + 1);
+    if (j + 2 < nt) step(std::integral_constant<int, 0>{}, j + 2);
+  }
+#ifdef EMI_ATTN_TRACE
+  tracing = false;
+  if (blockIdx.x == 0 && blockIdx.y == 5 && lane == 0)
+    for (int i = 0; i < 40; i++) emi_attn_trace_buf[wave * 40 + i] = i < nts ? ts[i] : 0ull;
+#endif
+  if (wave < 4) phase_end();
+  __builtin_amdgcn_s_waitcnt(0x0f70);                 // loads past the last tile
+
+  l += __shfl_xor(l, 32, 64);
+  if (qrow < seq) {
+    const float inv = 1.0f / l;
+    uint16_t* orow = o + base + (int64_t)qrow * sh.ss;
+#pragma unroll
+    for (int dt = 0; dt < D / 32; dt++)
+#pragma unroll
+      for (int jj = 0; jj < 4; jj++) {
+        const int dcol = dt * 32 + 8 * jj + 4 * (lane >> 5);
+        uint2 w;
+        w.x = pack_bf16x2(acc_o[dt][4 * jj] * inv, acc_o[dt][4 * jj + 1] * inv);
+        w.y = pack_bf16x2(acc_o[dt][4 * jj + 2] * inv, acc_o[dt][4 * jj + 3] * inv);
+        *reinterpret_cast<uint2*>(orow + dcol) = w;
+      }
+    if (lane < 32) lse[(int64_t)bh * seq + qrow] = (m + __builtin_amdgcn_logf(l)) * kLn2;
+  }
+}
+
 // ---------------------------------------------------------------------------
 // dQ: block = 4 waves x 32 queries; K and V tiles of 64 keys through LDS.
 //   S^T = K Q^T, dP^T = V dO^T, dS^T = P^T (dP^T - delta), dQ^T = K^T dS^T
@@ -449,8 +751,9 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_bf16_kernel(const uint16_t
   EMI_LDS uint8_t* smem = (EMI_LDS uint8_t*)smem_raw;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int qblk = gridDim.x - 1 - blockIdx.x;
-  const int bh = blockIdx.y;
+  int blk, bh;
+  attn_block_coords(&blk, &bh);
+  const int qblk = gridDim.x - 1 - blk;
   const int64_t base = (int64_t)(bh / sh.heads) * sh.sb + (int64_t)(bh % sh.heads) * sh.sh;
   const int seq = sh.seq;
   const int q0 = qblk * BQ + wave * 32;
@@ -558,8 +861,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_bf16_kernel(const uint16_t* 
   EMI_LDS uint8_t* smem = (EMI_LDS uint8_t*)smem_raw;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int kblk = blockIdx.x;                         // early key blocks see the most queries: first
-  const int bh = blockIdx.y;
+  int kblk, bh;                                        // early key blocks see the most queries: first
+  attn_block_coords(&kblk, &bh);
   const int64_t base = (int64_t)(bh / sh.heads) * sh.sb + (int64_t)(bh % sh.heads) * sh.sh;
   const int seq = sh.seq;
   const int k0 = kblk * BKEY + wave * 32;
@@ -708,9 +1011,22 @@ template <typename K> static int reserve_lds(K kern, int bytes, const char* name
 
 using namespace emi;
 
-extern "C" int emi_attn_fwd(emi_stream_t stream, const void* q, const void* k, const void* v, void* o, float* lse,
-                            int64_t batch, int64_t heads, int64_t seq, int64_t head_dim, int64_t stride_b,
-                            int64_t stride_h, int64_t stride_s, float scale, int causal, int dtype) {
+#ifdef EMI_ATTN_TRACE
+extern "C" int emi_debug_attn_trace(unsigned long long* out) {
+  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(emi_attn_trace_buf), sizeof(unsigned long long) * 8 * 40);
+}
+#endif
+
+extern "C" size_t emi_attn_fwd_workspace_bytes(int64_t batch, int64_t heads, int64_t seq, int64_t head_dim) {
+  if (batch <= 0 || heads <= 0 || seq <= 0 || (head_dim != 64 && head_dim != 128)) return 0;
+  const int64_t s_pad = (seq + 63) / 64 * 64;
+  return (size_t)batch * (size_t)heads * (size_t)head_dim * (size_t)s_pad * 2;     // V^T, bf16
+}
+
+extern "C" int emi_attn_fwd_ws(emi_stream_t stream, const void* q, const void* k, const void* v, void* o, float* lse,
+                               void* workspace, size_t workspace_bytes, int64_t batch, int64_t heads, int64_t seq,
+                               int64_t head_dim, int64_t stride_b, int64_t stride_h, int64_t stride_s, float scale,
+                               int causal, int dtype) {
   const AttnArgs a{batch, heads, seq, head_dim, stride_b, stride_h, stride_s};
   if (int rc = check_common("emi_attn_fwd", a, dtype)) return rc;
   if (batch == 0) return EMI_OK;
@@ -721,6 +1037,39 @@ extern "C" int emi_attn_fwd(emi_stream_t stream, const void* q, const void* k, c
   if (mfma_ok(a, dtype, {q, k, v, o})) {
     const uint32_t head_bytes = (uint32_t)(((seq - 1) * stride_s + head_dim) * 2);
     const float sl2 = scale * kLog2e;
+    static const int fwd_variant = getenv("EMI_ATTN_FWD") ? atoi(getenv("EMI_ATTN_FWD")) : 1;
+    if (fwd_variant >= 1 && seq >= 256) {
+      const dim3 gridp((unsigned)((seq + 255) / 256), bh);
+      const int s_pad = (int)((seq + 63) / 64 * 64);
+      const size_t need = emi_attn_fwd_workspace_bytes(batch, heads, seq, head_dim);
+      // With a workspace V is transposed once (keys contiguous); without one the kernel
+      // falls back to transposing LDS reads of V.
+      const bool vt = fwd_variant == 1 && workspace != nullptr && workspace_bytes >= need && aligned16(workspace) &&
+                      (int64_t)head_dim * s_pad * 2 < 0x7fffff00LL && bh <= 65535;
+#define EMI_ATTN_FWD_PP(DD)                                                                                          \
+  do {                                                                                                               \
+    constexpr int smem = 3 * 2 * 64 * DD * 2;                                                                        \
+    if (vt) {                                                                                                        \
+      hipLaunchKernelGGL(attn_vt_kernel<DD>, dim3((unsigned)(s_pad / 64), DD / 64, bh), dim3(256), 0, st,            \
+                         (const uint16_t*)v, (uint16_t*)workspace, shp, s_pad);                                      \
+      EMI_CHECK_LAUNCH("emi_attn_fwd(vt)");                                                                          \
+      if (int rc = reserve_lds(attn_fwd_pp_kernel<DD, true>, smem, "emi_attn_fwd")) return rc;                       \
+      hipLaunchKernelGGL((attn_fwd_pp_kernel<DD, true>), gridp, dim3(512), smem, st, (const uint16_t*)q,             \
+                         (const uint16_t*)k, (const uint16_t*)workspace, (uint16_t*)o, lse, shp, head_bytes, sl2,    \
+                         causal, s_pad);                                                                             \
+    } else {                                                                                                         \
+      if (int rc = reserve_lds(attn_fwd_pp_kernel<DD, false>, smem, "emi_attn_fwd")) return rc;                      \
+      hipLaunchKernelGGL((attn_fwd_pp_kernel<DD, false>), gridp, dim3(512), smem, st, (const uint16_t*)q,            \
+                         (const uint16_t*)k, (const uint16_t*)v, (uint16_t*)o, lse, shp, head_bytes, sl2, causal,    \
+                         s_pad);                                                                                     \
+    }                                                                                                                \
+  } while (0)
+      if (head_dim == 128) EMI_ATTN_FWD_PP(128);
+      else EMI_ATTN_FWD_PP(64);
+#undef EMI_ATTN_FWD_PP
+      EMI_CHECK_LAUNCH("emi_attn_fwd");
+      return EMI_OK;
+    }
     const dim3 grid((unsigned)((seq + 127) / 128), bh);
     if (head_dim == 128) {
       constexpr int smem = 2 * 2 * 64 * 128 * 2;
@@ -745,6 +1094,13 @@ extern "C" int emi_attn_fwd(emi_stream_t stream, const void* q, const void* k, c
                        (const float*)v, (float*)o, lse, shp, (int)head_dim, scale, causal);
   EMI_CHECK_LAUNCH("emi_attn_fwd(generic)");
   return EMI_OK;
+}
+
+extern "C" int emi_attn_fwd(emi_stream_t stream, const void* q, const void* k, const void* v, void* o, float* lse,
+                            int64_t batch, int64_t heads, int64_t seq, int64_t head_dim, int64_t stride_b,
+                            int64_t stride_h, int64_t stride_s, float scale, int causal, int dtype) {
+  return emi_attn_fwd_ws(stream, q, k, v, o, lse, nullptr, 0, batch, heads, seq, head_dim, stride_b, stride_h, stride_s,
+                         scale, causal, dtype);
 }
 
 extern "C" size_t emi_attn_bwd_workspace_bytes(int64_t batch, int64_t heads, int64_t seq, int64_t head_dim) {

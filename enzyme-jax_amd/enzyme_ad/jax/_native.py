@@ -33,6 +33,9 @@ SIGNATURES = {
                          c_i64, c_int, c_int, c_int]),
     "emi_attn_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_i64, c_i64, c_i64,
                              c_i64, c_i64, c_i64, c_float, c_int, c_int]),
+    "emi_attn_fwd_workspace_bytes": (c_size_t, [c_i64, c_i64, c_i64, c_i64]),
+    "emi_attn_fwd_ws": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_i64,
+                                c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_float, c_int, c_int]),
     "emi_attn_bwd_workspace_bytes": (c_size_t, [c_i64, c_i64, c_i64, c_i64]),
     "emi_attn_bwd": (c_int, [c_void_p] * 10 + [c_void_p, c_size_t, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64,
                                                c_float, c_int, c_int]),

@@ -310,8 +310,10 @@ def attention_raw(q, k, v, n_heads, scale, causal, strides):
         sb, sh, ss = n_heads * S * d, S * d, d
     o = torch.empty_like(q)
     lse = torch.empty((B, n_heads, S), dtype=torch.float32, device=q.device)
-    N.check(N.lib().emi_attn_fwd(_stream(), _p(q), _p(k), _p(v), _p(o), _p(lse), B, n_heads, S, d, sb, sh, ss,
-                                 float(scale), int(causal), _code(q)))
+    nbytes = N.lib().emi_attn_fwd_workspace_bytes(B, n_heads, S, d) if q.dtype == torch.bfloat16 else 0
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device) if nbytes else None
+    N.check(N.lib().emi_attn_fwd_ws(_stream(), _p(q), _p(k), _p(v), _p(o), _p(lse), _p(ws), nbytes, B, n_heads, S, d,
+                                    sb, sh, ss, float(scale), int(causal), _code(q)))
     return o, lse, (B, S, d, sb, sh, ss)
 
 

@@ -113,6 +113,16 @@ int emi_attn_fwd(emi_stream_t stream, const void* q, const void* k, const void* 
                  int64_t stride_b, int64_t stride_h, int64_t stride_s, float scale, int causal,
                  int dtype);
 
+/* The same with a scratch buffer of emi_attn_fwd_workspace_bytes() bytes: the bf16
+ * MFMA kernel then transposes V once so that the P.V product reads keys
+ * contiguously (faster); a null or too small workspace selects the in-kernel
+ * transposing reads.  Results are identical up to rounding of P. */
+size_t emi_attn_fwd_workspace_bytes(int64_t batch, int64_t heads, int64_t seq, int64_t head_dim);
+int emi_attn_fwd_ws(emi_stream_t stream, const void* q, const void* k, const void* v, void* o,
+                    float* lse, void* workspace, size_t workspace_bytes, int64_t batch,
+                    int64_t heads, int64_t seq, int64_t head_dim, int64_t stride_b,
+                    int64_t stride_h, int64_t stride_s, float scale, int causal, int dtype);
+
 /* Attention adjoint: dV = P^T dO, dP = dO V^T, dS = P*(dP - rowsum(dO*O)),
  * dQ = dS K scale, dK = dS^T Q scale; P is recomputed from q, k and lse.
  * Rules: Exp :1182, Div :1133, Sub :1312, Reduce(max/add)
