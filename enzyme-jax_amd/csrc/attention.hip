@@ -27,6 +27,8 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
 typedef __attribute__((__vector_size__(8 * sizeof(float)))) float f32x8_t;
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 
 #define EMI_LDS __attribute__((address_space(3)))
 
@@ -47,13 +49,20 @@ struct AttnShape {
 // fetched into all eight L2s.  Instead every XCD gets a contiguous run of heads with all
 // of their blocks, in the order given (longest first).
 __device__ __forceinline__ void attn_block_coords(int* blk, int* bh) {
-  const int nblk = gridDim.x, total = gridDim.x * gridDim.y;
+  const int nblk = gridDim.x, nbh = gridDim.y, total = nblk * nbh;
   const int lin = blockIdx.y * gridDim.x + blockIdx.x;
   const int per = total >> 3, rem = total & 7;
   const int xcd = lin & 7, idx = lin >> 3;
   const int v = xcd * per + (xcd < rem ? xcd : rem) + idx;
-  *bh = v / nblk;
-  *blk = v - *bh * nblk;
+  // Heads are taken in groups of four and, inside a group, block positions go first
+  // (the four longest blocks, then the four next longest, ...): list scheduling of
+  // head-major order leaves the CUs of a XCD up to 10% apart at the end, this order
+  // does not, and four heads of K/V still fit in the L2.
+  constexpr int G = 4;
+  const int g = v / (G * nblk), r = v - g * G * nblk;
+  const int gh = nbh - g * G < G ? nbh - g * G : G;
+  *blk = r / gh;
+  *bh = g * G + (r - *blk * gh);
 }
 
 // ===========================================================================
@@ -431,21 +440,36 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_kernel(const uint16_t* _
     __syncthreads();
   }
 
+  // Epilogue.  A lane owns one query and, per register quad, four consecutive d: written
+  // straight to HBM that is 8 bytes per lane to 32 different rows.  Instead each wavefront
+  // stages its 32 x D tile through its slice of the (now idle) LDS and writes rows with
+  // 16-byte, row-contiguous stores.  Chunk c of row r sits at chunk c ^ (r % CH), the two
+  // 8-byte halves swapped when (r / CH) is odd: conflict free for both access shapes.
+  // (the loop ended with all loads landed and a barrier: the LDS is idle)
   l += __shfl_xor(l, 32, 64);
-  if (qrow < seq) {
+  {
+    constexpr int CH = D / 8, RB = D * 2;
+    EMI_LDS uint8_t* wl = smem + wave * (32 * RB);
     const float inv = 1.0f / l;
-    uint16_t* orow = o + base + (int64_t)qrow * sh.ss;
+    const int r = lane & 31, g = lane >> 5;
 #pragma unroll
     for (int dt = 0; dt < D / 32; dt++)
 #pragma unroll
       for (int jj = 0; jj < 4; jj++) {
-        const int dcol = dt * 32 + 8 * jj + 4 * (lane >> 5);
-        uint2 w;
-        w.x = pack_bf16x2(acc_o[dt][4 * jj] * inv, acc_o[dt][4 * jj + 1] * inv);
-        w.y = pack_bf16x2(acc_o[dt][4 * jj + 2] * inv, acc_o[dt][4 * jj + 3] * inv);
-        *reinterpret_cast<uint2*>(orow + dcol) = w;
+        u32x2_t w;
+        w[0] = pack_bf16x2(acc_o[dt][4 * jj] * inv, acc_o[dt][4 * jj + 1] * inv);
+        w[1] = pack_bf16x2(acc_o[dt][4 * jj + 2] * inv, acc_o[dt][4 * jj + 3] * inv);
+        const int c = dt * 4 + jj;
+        *reinterpret_cast<EMI_LDS u32x2_t*>(wl + r * RB + ((c ^ (r & (CH - 1))) << 4) + ((g ^ ((r / CH) & 1)) << 3)) = w;
       }
-    if (lane < 32) lse[(int64_t)bh * seq + qrow] = (m + __builtin_amdgcn_logf(l)) * kLn2;
+    if (qrow < seq && lane < 32) lse[(int64_t)bh * seq + qrow] = (m + __builtin_amdgcn_logf(l)) * kLn2;
+#pragma unroll
+    for (int it = 0; it < 32 * CH / 64; it++) {
+      const int row = it * (64 / CH) + lane / CH, c = lane % CH;
+      u32x4_t v4 = *reinterpret_cast<const EMI_LDS u32x4_t*>(wl + row * RB + ((c ^ (row & (CH - 1))) << 4));
+      if ((row / CH) & 1) v4 = __builtin_shufflevector(v4, v4, 2, 3, 0, 1);
+      if (q0 + row < seq) *reinterpret_cast<u32x4_t*>(o + base + (int64_t)(q0 + row) * sh.ss + c * 8) = v4;
+    }
   }
 }
 
@@ -517,6 +541,12 @@ __device__ __forceinline__ int perm_key(int m) { return (m & ~12) | ((m & 4) << 
 // than 8 (in log2 units), so the rescaling of O runs on a few early tiles only; P then
 // stays below 2^8 and the final O/l and log-sum-exp are exact for whatever m was used.
 // ---------------------------------------------------------------------------
+#ifdef EMI_ATTN_BLOCKLOG
+__device__ unsigned long long emi_attn_blocklog[4096 * 4];
+extern "C" int emi_debug_attn_blocklog(unsigned long long* out) {
+  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(emi_attn_blocklog), sizeof(unsigned long long) * 4096 * 4);
+}
+#endif
 #ifdef EMI_ATTN_TRACE
 __device__ unsigned long long emi_attn_trace_buf[8 * 40];
 #define EMI_ATRACE() do { if (tracing && nts < 40) ts[nts++] = __builtin_readcyclecounter(); } while (0)
@@ -538,6 +568,9 @@ __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(const uint16_t* __rest
   int blk, bh;
   attn_block_coords(&blk, &bh);
   const int qblk = gridDim.x - 1 - blk;              // longest rows first
+#ifdef EMI_ATTN_BLOCKLOG
+  const unsigned long long log_w0 = wall_clock64(), log_c0 = __builtin_readcyclecounter();
+#endif
   const int64_t base = (int64_t)(bh / sh.heads) * sh.sb + (int64_t)(bh % sh.heads) * sh.sh;
   const int seq = sh.seq;
   const int q0 = qblk * BQ + wave * 32;
@@ -688,11 +721,17 @@ __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(const uint16_t* __rest
     phase_end();
   };
 
+#ifdef EMI_ATTN_BLOCKLOG
+  const unsigned long long log_c1 = __builtin_readcyclecounter();
+#endif
   issue_bundle(-1, 0);
   issue_bundle(0, 1);
   __builtin_amdgcn_s_waitcnt(0x0f70);                 // vmcnt(0)
   issue_bundle(1, 2);
   phase_end();
+#ifdef EMI_ATTN_BLOCKLOG
+  const unsigned long long log_c2 = __builtin_readcyclecounter();
+#endif
   if (wave >= 4) phase_end();                         // second group runs one phase behind
   __builtin_amdgcn_s_setprio(1);
   mfma_phase(std::true_type{}, std::false_type{}, 0);      // MFMA phase -1
@@ -700,7 +739,7 @@ __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(const uint16_t* __rest
   phase_end();
   for (int j = 0; j < nt; j += 3) {
 #ifdef EMI_ATTN_TRACE
-    tracing = (blockIdx.x == 0 && blockIdx.y == 5 && j >= 30 && j < 36);
+    tracing = (blockIdx.x == 0 && blockIdx.y == 5 && j >= 9 && j < 18);
 #endif
     step(std::integral_constant<int, 1>{}, j);
     if (j + 1 < nt) step(std::integral_constant<int, 2>{}, j + 1);
@@ -713,23 +752,55 @@ __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(const uint16_t* __rest
 #endif
   if (wave < 4) phase_end();
   __builtin_amdgcn_s_waitcnt(0x0f70);                 // loads past the last tile
+#ifdef EMI_ATTN_BLOCKLOG
+  const unsigned long long log_c3 = __builtin_readcyclecounter();
+#endif
 
+  // Epilogue.  A lane owns one query and, per register quad, four consecutive d: written
+  // straight to HBM that is 8 bytes per lane to 32 different rows.  Instead each wavefront
+  // stages its 32 x D tile through its slice of the (now idle) LDS and writes rows with
+  // 16-byte, row-contiguous stores.  Chunk c of row r sits at chunk c ^ (r % CH), the two
+  // 8-byte halves swapped when (r / CH) is odd: conflict free for both access shapes.
+  phase_end();                                        // every wavefront's loads have landed
   l += __shfl_xor(l, 32, 64);
-  if (qrow < seq) {
+  {
+    constexpr int CH = D / 8, RB = D * 2;
+    EMI_LDS uint8_t* wl = smem + wave * (32 * RB);
     const float inv = 1.0f / l;
-    uint16_t* orow = o + base + (int64_t)qrow * sh.ss;
+    const int r = lane & 31, g = lane >> 5;
 #pragma unroll
     for (int dt = 0; dt < D / 32; dt++)
 #pragma unroll
       for (int jj = 0; jj < 4; jj++) {
-        const int dcol = dt * 32 + 8 * jj + 4 * (lane >> 5);
-        uint2 w;
-        w.x = pack_bf16x2(acc_o[dt][4 * jj] * inv, acc_o[dt][4 * jj + 1] * inv);
-        w.y = pack_bf16x2(acc_o[dt][4 * jj + 2] * inv, acc_o[dt][4 * jj + 3] * inv);
-        *reinterpret_cast<uint2*>(orow + dcol) = w;
+        u32x2_t w;
+        w[0] = pack_bf16x2(acc_o[dt][4 * jj] * inv, acc_o[dt][4 * jj + 1] * inv);
+        w[1] = pack_bf16x2(acc_o[dt][4 * jj + 2] * inv, acc_o[dt][4 * jj + 3] * inv);
+        const int c = dt * 4 + jj;
+        *reinterpret_cast<EMI_LDS u32x2_t*>(wl + r * RB + ((c ^ (r & (CH - 1))) << 4) + ((g ^ ((r / CH) & 1)) << 3)) = w;
       }
-    if (lane < 32) lse[(int64_t)bh * seq + qrow] = (m + __builtin_amdgcn_logf(l)) * kLn2;
+    if (qrow < seq && lane < 32) lse[(int64_t)bh * seq + qrow] = (m + __builtin_amdgcn_logf(l)) * kLn2;
+#pragma unroll
+    for (int it = 0; it < 32 * CH / 64; it++) {
+      const int row = it * (64 / CH) + lane / CH, c = lane % CH;
+      u32x4_t v4 = *reinterpret_cast<const EMI_LDS u32x4_t*>(wl + row * RB + ((c ^ (row & (CH - 1))) << 4));
+      if ((row / CH) & 1) v4 = __builtin_shufflevector(v4, v4, 2, 3, 0, 1);
+      if (q0 + row < seq) *reinterpret_cast<u32x4_t*>(o + base + (int64_t)(q0 + row) * sh.ss + c * 8) = v4;
+    }
   }
+#ifdef EMI_ATTN_BLOCKLOG
+  if (threadIdx.x == 0) {
+    const int lin = blockIdx.y * gridDim.x + blockIdx.x;
+    if (lin < 4096) {
+      emi_attn_blocklog[lin * 4 + 0] = log_w0;
+      emi_attn_blocklog[lin * 4 + 1] = wall_clock64();
+      const unsigned long long log_c4 = __builtin_readcyclecounter();
+      // packed: total cycles (24 bits) | q load (12, /16) | prologue (12, /16) | epilogue (12, /16)
+      emi_attn_blocklog[lin * 4 + 2] = (log_c4 - log_c0) | (((log_c1 - log_c0) >> 4) << 24) | (((log_c2 - log_c1) >> 4) << 36) |
+                                       (((log_c4 - log_c3) >> 4) << 48);
+      emi_attn_blocklog[lin * 4 + 3] = ((unsigned long long)qblk << 32) | (unsigned)bh;
+    }
+  }
+#endif
 }
 
 // ---------------------------------------------------------------------------
