@@ -27,6 +27,7 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
 typedef __attribute__((__vector_size__(8 * sizeof(float)))) float f32x8_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 
@@ -815,7 +816,8 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_bf16_kernel(const uint16_t
                                                                const float* __restrict__ lse,
                                                                const float* __restrict__ delta,
                                                                uint16_t* __restrict__ dq, AttnShape sh,
-                                                               uint32_t head_bytes, float scale, int causal) {
+                                                               uint32_t head_bytes, float scale, int causal,
+                                                               float delta_sign) {
   constexpr int BQ = 128, BKV = 64, NW = 4;
   constexpr int TILE = BKV * D * 2, STAGE = 2 * TILE;
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem_raw[];
@@ -835,7 +837,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_bf16_kernel(const uint16_t
   load_reg_rows<D>(q + base, qrow, seq, sh.ss, lane, qf);
   load_reg_rows<D>(d_o + base, qrow, seq, sh.ss, lane, dof);
   const float L2 = qrow < seq ? lse[(int64_t)bh * seq + qrow] * kLog2e : 0.f;
-  const float dl = qrow < seq ? delta[(int64_t)bh * seq + qrow] : 0.f;
+  const float dl = qrow < seq ? delta[(int64_t)bh * seq + qrow] * delta_sign : 0.f;
 
   const __amdgpu_buffer_rsrc_t rK = attn_rsrc(k + base, head_bytes);
   const __amdgpu_buffer_rsrc_t rV = attn_rsrc(v + base, head_bytes);
@@ -1042,6 +1044,274 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_bf16_kernel(const uint16_t* 
 }
 
 // ---------------------------------------------------------------------------
+// Adjoint pre-pass for the MFMA kernels: delta[row] = sum_i dO*O (times delta_sign) and
+// lse2[row] = lse * log2(e).  16-byte loads, D/8 lanes per row.
+// ---------------------------------------------------------------------------
+template <int D>
+__global__ __launch_bounds__(256) void attn_prep_kernel(const uint16_t* __restrict__ o, const uint16_t* __restrict__ d_o,
+                                                        const float* __restrict__ lse, float* __restrict__ delta,
+                                                        float* __restrict__ lse2, AttnShape sh, float delta_sign) {
+  constexpr int LPR = D / 8, RPB = 256 / LPR;          // lanes per row, rows per block
+  const int qi = blockIdx.x * RPB + threadIdx.x / LPR;
+  const int bh = blockIdx.y;
+  const int c = threadIdx.x % LPR;
+  float s = 0.f;
+  if (qi < sh.seq) {
+    const int64_t off = (int64_t)(bh / sh.heads) * sh.sb + (int64_t)(bh % sh.heads) * sh.sh + (int64_t)qi * sh.ss + c * 8;
+    float a[8], b[8];
+    Vec8<bf16>::load(reinterpret_cast<const bf16*>(o) + off, a);
+    Vec8<bf16>::load(reinterpret_cast<const bf16*>(d_o) + off, b);
+#pragma unroll
+    for (int e = 0; e < 8; e++) s += a[e] * b[e];
+  }
+#pragma unroll
+  for (int m = LPR / 2; m > 0; m >>= 1) s += __shfl_xor(s, m, 64);
+  if (qi < sh.seq && c == 0) {
+    delta[(int64_t)bh * sh.seq + qi] = s * delta_sign;
+    lse2[(int64_t)bh * sh.seq + qi] = lse[(int64_t)bh * sh.seq + qi] * kLog2e;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// dK, dV, software-pipelined form: block = 4 wavefronts x 32 keys, one wavefront per SIMD
+// (K, V fragments and both accumulators stay in registers).  Work proceeds in halves of a
+// 64-query tile (32 queries, index H):
+//   A(H): S, dP   = rows of Q, dO against K, V                (16 MFMAs)
+//   B(H): P = exp2(S*c - lse2), dS = P*(dP - delta)            (VALU)
+//   C(H): dV^T += dO^T P, dK^T += Q^T dS  (columns of dO, Q)   (16 MFMAs)
+// Iteration H runs A(H+1) interleaved with B(H), so the softmax arithmetic of one half
+// issues in the shadow of the MFMAs of the next, then C(H).  Tiles sit in a ring of
+// three LDS slots; once per tile the wavefronts meet at a barrier, after which the loads
+// of tile t+3 may overwrite tile t.  The column fragments are fetched with
+// ds_read_b64_tr_b16 through inline asm: the compiler orders every LDS read it knows of
+// behind all outstanding direct-to-LDS loads, which would serialise loading and compute.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ u32x2_t lds_read_tr_asm(uint32_t addr) {
+  u32x2_t r;
+  asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(r) : "v"(addr));
+  return r;
+}
+// s_waitcnt lgkmcnt(N) that the MFMA consuming `a`, `b` cannot be moved above.
+template <int N> __device__ __forceinline__ void lgkm_wait_for(u32x2_t& a, u32x2_t& b) {
+  asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N));
+}
+
+template <int D>
+__global__ __launch_bounds__(256) void attn_bwd_dkv_sp_kernel(const uint16_t* __restrict__ q,
+                                                              const uint16_t* __restrict__ k,
+                                                              const uint16_t* __restrict__ v,
+                                                              const uint16_t* __restrict__ d_o,
+                                                              const float* __restrict__ lse2,
+                                                              const float* __restrict__ delta, uint16_t* __restrict__ dk,
+                                                              uint16_t* __restrict__ dv, AttnShape sh,
+                                                              uint32_t head_bytes, float scale, int causal) {
+  constexpr int BKEY = 128, BQT = 64, NW = 4, NSLOT = 3;
+  constexpr int TILE = BQT * D * 2;
+  constexpr int STATS = 2 * NSLOT * TILE;                 // lse2 and delta of each slot: 2 x 256 bytes
+  constexpr int LPB = 2 * (TILE / 1024 / NW) + 1;         // loads per wavefront per tile
+  static_assert(LPB < 16, "vmcnt immediate");
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem_raw[];
+  EMI_LDS uint8_t* smem = (EMI_LDS uint8_t*)smem_raw;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  int kblk, bh;                                           // early key blocks see the most queries: first
+  attn_block_coords(&kblk, &bh);
+  const int64_t base = (int64_t)(bh / sh.heads) * sh.sb + (int64_t)(bh % sh.heads) * sh.sh;
+  const int seq = sh.seq;
+  const int k0 = kblk * BKEY + wave * 32;
+  const int krow = k0 + (lane & 31);
+  const float scale_log2e = scale * kLog2e;
+
+  bf16x8_t kf[D / 16], vf[D / 16];
+  load_reg_rows<D>(k + base, krow, seq, sh.ss, lane, kf);
+  load_reg_rows<D>(v + base, krow, seq, sh.ss, lane, vf);
+
+  const __amdgpu_buffer_rsrc_t rQ = attn_rsrc(q + base, head_bytes);
+  const __amdgpu_buffer_rsrc_t rDO = attn_rsrc(d_o + base, head_bytes);
+  const __amdgpu_buffer_rsrc_t rL = attn_rsrc(lse2 + (int64_t)bh * seq, (uint32_t)seq * 4u);
+  const __amdgpu_buffer_rsrc_t rDl = attn_rsrc(delta + (int64_t)bh * seq, (uint32_t)seq * 4u);
+  const int qt0 = causal ? (kblk * BKEY) / BQT : 0;       // first query tile that can see this key block
+  const int nt = (seq + BQT - 1) / BQT - qt0;             // >= 1: the block holds at least one key < seq
+
+  f32x16_t acc_k[D / 32], acc_v[D / 32];
+#pragma unroll
+  for (int dt = 0; dt < D / 32; dt++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc_k[dt][r] = 0.f, acc_v[dt][r] = 0.f;
+  bf16x8_t pf[2], dsf[2];
+
+  // tile ti (query tile qt0 + ti) -> slot; rows >= seq read as zeros
+  auto issue_tile = [&](int ti, int slot) __attribute__((always_inline)) {
+    const int row0 = (qt0 + ti) * BQT;
+    load_rows_tile<D, BQT, NW>(rQ, smem + slot * TILE, wave, lane, row0, seq, sh.ss);
+    load_rows_tile<D, BQT, NW>(rDO, smem + NSLOT * TILE + slot * TILE, wave, lane, row0, seq, sh.ss);
+    // one 256-byte load of lse2 (even wavefronts) or delta (odd ones); the copies are identical
+    const uint32_t voff = row0 + lane < seq ? (uint32_t)(row0 + lane) * 4u : kOobA;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds((wave & 1) ? rDl : rL, smem + STATS + slot * 512 + (wave & 1) * 256, 4, voff, 0, 0,
+                                             0);
+  };
+  // A(H+1) with B(H), interleaved by hand: after each of the 16 MFMAs of A (S and dP - delta
+  // of half (slot_n, Tn) into sn, dpn; the dP accumulator starts from the -delta of its rows,
+  // read from LDS, which saves a subtraction per score) comes the softmax arithmetic of one
+  // score of half (ti, slot_p, Tp) held in sp, dpp.  The scheduler is fenced after every
+  // step: left alone it issues all MFMAs first and the VALU work after them.
+  auto stage_ab = [&](auto masked_c, auto do_b_c, int slot_n, int Tn, f32x16_t& sn, f32x16_t& dpn, int ti, int slot_p,
+                      int Tp, f32x16_t& sp, f32x16_t& dpp) __attribute__((always_inline)) {
+    constexpr bool MASKED = decltype(masked_c)::value, DO_B = decltype(do_b_c)::value;
+    const EMI_LDS uint8_t* sQ = smem + slot_n * TILE;
+    const EMI_LDS uint8_t* sDO = smem + NSLOT * TILE + slot_n * TILE;
+    const EMI_LDS float* sNd = (const EMI_LDS float*)(smem + STATS + slot_n * 512) + 64 + Tn * 32 + 4 * (lane >> 5);
+    const EMI_LDS float* sL = (const EMI_LDS float*)(smem + STATS + slot_p * 512) + Tp * 32 + 4 * (lane >> 5);
+    const int qbase = (qt0 + ti) * BQT + Tp * 32;
+    constexpr int NOP = 2 * (D / 16), DEPTH = 4;
+    static_assert(NOP == 16 || NOP == 8, "one score per MFMA (or two)");
+    constexpr int EPM = 16 / NOP;                    // scores handled per MFMA
+    auto fetch = [&](int i) __attribute__((always_inline)) -> bf16x8_t {
+      return row_frag<D>((i & 1) ? sDO : sQ, Tn * 32, i >> 1, lane);
+    };
+    f32x4_t L4[4];
+#pragma unroll
+    for (int rq = 0; rq < 4; rq++) {
+      const f32x4_t nd = *reinterpret_cast<const EMI_LDS f32x4_t*>(sNd + 8 * rq);
+      if constexpr (DO_B) L4[rq] = *reinterpret_cast<const EMI_LDS f32x4_t*>(sL + 8 * rq);
+#pragma unroll
+      for (int e = 0; e < 4; e++) dpn[4 * rq + e] = nd[e];
+    }
+    const f32x16_t zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    bf16x8_t ring[DEPTH];
+#pragma unroll
+    for (int i = 0; i < DEPTH; i++) ring[i] = fetch(i);
+    f32x16_t ds;
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < NOP; i++) {
+      if (i & 1) dpn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[i % DEPTH], vf[i >> 1], dpn, 0, 0, 0);
+      else sn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[i % DEPTH], kf[i >> 1], i == 0 ? zero16 : sn, 0, 0, 0);
+      if (i + DEPTH < NOP) ring[i % DEPTH] = fetch(i + DEPTH);
+      if constexpr (DO_B) {
+#pragma unroll
+        for (int u = 0; u < EPM; u++) {
+          const int r = i * EPM + u;
+          float p = fast_exp2(fmaf(sp[r], scale_log2e, -L4[r >> 2][r & 3]));
+          if (MASKED && causal && krow > qbase + acc_row(r, lane)) p = 0.f;
+          sp[r] = p;
+          ds[r] = p * dpp[r];
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if constexpr (DO_B) {
+      pf[0] = acc_to_frag(sp, 0);
+      pf[1] = acc_to_frag(sp, 1);
+      dsf[0] = acc_to_frag(ds, 0);
+      dsf[1] = acc_to_frag(ds, 1);
+    }
+  };
+  // C: dV, dK contributions of half (slot, T).  16 column fragments, two asm reads each,
+  // ring of 4 fragments: after the reads of fragment i+4 are issued, fragments i..i+4 (10
+  // reads) are outstanding and lgkmcnt(8) means fragment i has arrived.
+  auto stage_c = [&](int slot, int T) __attribute__((always_inline)) {
+    const uint32_t aQ = (uint32_t)(uintptr_t)(smem + slot * TILE);
+    const uint32_t aDO = (uint32_t)(uintptr_t)(smem + NSLOT * TILE + slot * TILE);
+    // per-lane address of the first read of col_frag<D>(tile, row_base, col_base): see col_frag
+    const int li = lane & 15;
+    const int r0l = (lane >> 5) * 4 + (li >> 2);
+    const int coll = ((lane >> 4) & 1) * 16 + (li & 3) * 4;
+    auto addr = [&](uint32_t tile, int row, int col) __attribute__((always_inline)) {
+      return tile + (uint32_t)(row * (D * 2) + (((col >> 3) ^ swz<D>(row)) * 16) + (col & 7) * 2);
+    };
+    constexpr int NF = 4 * (D / 32), DEPTH = 4;
+    u32x2_t lo[DEPTH], hi[DEPTH];
+    auto fetch = [&](int i, int slot_i) __attribute__((always_inline)) {
+      const int which = i & 1, dt = (i >> 1) % (D / 32), sI = i / (2 * (D / 32));
+      const int row = T * 32 + sI * 16 + r0l, col = dt * 32 + coll;
+      lo[slot_i] = lds_read_tr_asm(addr(which ? aQ : aDO, row, col));
+      hi[slot_i] = lds_read_tr_asm(addr(which ? aQ : aDO, row + 8, col));
+    };
+    asm volatile("s_waitcnt lgkmcnt(0)");
+#pragma unroll
+    for (int i = 0; i < DEPTH; i++) fetch(i, i);
+#pragma unroll
+    for (int i = 0; i < NF; i++) {
+      const int which = i & 1, dt = (i >> 1) % (D / 32), sI = i / (2 * (D / 32));
+      const int rem = NF - 1 - i < DEPTH - 1 ? NF - 1 - i : DEPTH - 1;     // fragments still in flight behind i
+      if (rem == 3) lgkm_wait_for<6>(lo[i % DEPTH], hi[i % DEPTH]);
+      else if (rem == 2) lgkm_wait_for<4>(lo[i % DEPTH], hi[i % DEPTH]);
+      else if (rem == 1) lgkm_wait_for<2>(lo[i % DEPTH], hi[i % DEPTH]);
+      else lgkm_wait_for<0>(lo[i % DEPTH], hi[i % DEPTH]);
+      u32x4_t w = {lo[i % DEPTH][0], lo[i % DEPTH][1], hi[i % DEPTH][0], hi[i % DEPTH][1]};
+      const bf16x8_t af = __builtin_bit_cast(bf16x8_t, w);
+      if (which) acc_k[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, dsf[sI], acc_k[dt], 0, 0, 0);
+      else acc_v[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, pf[sI], acc_v[dt], 0, 0, 0);
+      if (i + DEPTH < NF) fetch(i + DEPTH, i % DEPTH);
+    }
+  };
+
+  issue_tile(0, 0);
+  issue_tile(1, 1);
+  __builtin_amdgcn_s_waitcnt(0x0f70);                 // vmcnt(0)
+  __syncthreads();
+  issue_tile(2, 2);
+
+  f32x16_t sA, dpA, sB, dpB;                          // scores of even / odd halves
+  stage_ab(std::false_type{}, std::false_type{}, 0, 0, sA, dpA, 0, 0, 0, sB, dpB);
+  int slot = 0;                                       // slot of tile ti
+  auto tile_step = [&](auto masked_c, int ti) __attribute__((always_inline)) {
+    const int nslot = slot == NSLOT - 1 ? 0 : slot + 1;
+    // iteration 2*ti: A(half 1 of this tile) with B(half 0), then C(half 0)
+    stage_ab(masked_c, std::true_type{}, slot, 1, sB, dpB, ti, slot, 0, sA, dpA);
+    stage_c(slot, 0);
+    // iteration 2*ti+1: A(half 0 of the next tile) with B(half 1), then C(half 1)
+    stage_ab(masked_c, std::true_type{}, nslot, 0, sA, dpA, ti, slot, 1, sB, dpB);
+    stage_c(slot, 1);
+    // Tile ti is finished.  Own part of tile ti+2 (issued one tile ago) must have landed;
+    // after the barrier every wavefront is done with tile ti and sees tile ti+2, and the
+    // loads of tile ti+3 may go into the slot of tile ti.
+    __builtin_amdgcn_s_waitcnt(0x0f70);               // vmcnt(0): only tile ti+2 is outstanding
+    __builtin_amdgcn_s_barrier();
+    issue_tile(ti + 3, slot);
+    slot = nslot;
+  };
+  // Only the first two query tiles of a key block can hold queries that precede its keys.
+  int ti = 0;
+  for (; ti < nt && ti < 2; ti++) tile_step(std::true_type{}, ti);
+  for (; ti < nt; ti++) tile_step(std::false_type{}, ti);
+  __builtin_amdgcn_s_waitcnt(0x0f70);                 // loads past the last tile
+  __syncthreads();
+
+  // Output through LDS for row-contiguous 16-byte stores (layout as in the forward kernel):
+  // dK (scaled), then dV, of this wavefront's 32 keys.
+  {
+    constexpr int CH = D / 8, RB = D * 2;
+    EMI_LDS uint8_t* wl = smem + wave * (32 * RB);
+    const int r = lane & 31, g = lane >> 5;
+#pragma unroll
+    for (int which = 0; which < 2; which++) {
+      const float mul = which ? 1.0f : scale;
+#pragma unroll
+      for (int dt = 0; dt < D / 32; dt++)
+#pragma unroll
+        for (int jj = 0; jj < 4; jj++) {
+          const f32x16_t& a = which ? acc_v[dt] : acc_k[dt];
+          u32x2_t w;
+          w[0] = pack_bf16x2(a[4 * jj] * mul, a[4 * jj + 1] * mul);
+          w[1] = pack_bf16x2(a[4 * jj + 2] * mul, a[4 * jj + 3] * mul);
+          const int c = dt * 4 + jj;
+          *reinterpret_cast<EMI_LDS u32x2_t*>(wl + r * RB + ((c ^ (r & (CH - 1))) << 4) + ((g ^ ((r / CH) & 1)) << 3)) = w;
+        }
+      uint16_t* out = which ? dv : dk;
+#pragma unroll
+      for (int it = 0; it < 32 * CH / 64; it++) {
+        const int row = it * (64 / CH) + lane / CH, c = lane % CH;
+        u32x4_t v4 = *reinterpret_cast<const EMI_LDS u32x4_t*>(wl + row * RB + ((c ^ (row & (CH - 1))) << 4));
+        if ((row / CH) & 1) v4 = __builtin_shufflevector(v4, v4, 2, 3, 0, 1);
+        if (k0 + row < seq) *reinterpret_cast<u32x4_t*>(out + base + (int64_t)(k0 + row) * sh.ss + c * 8) = v4;
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
 
@@ -1177,7 +1447,7 @@ extern "C" int emi_attn_fwd(emi_stream_t stream, const void* q, const void* k, c
 extern "C" size_t emi_attn_bwd_workspace_bytes(int64_t batch, int64_t heads, int64_t seq, int64_t head_dim) {
   (void)head_dim;
   if (batch <= 0 || heads <= 0 || seq <= 0) return 0;
-  return (size_t)batch * (size_t)heads * (size_t)seq * sizeof(float);   // delta = rowsum(dO * O)
+  return 2 * (size_t)batch * (size_t)heads * (size_t)seq * sizeof(float);   // delta = rowsum(dO * O), lse * log2(e)
 }
 
 extern "C" int emi_attn_bwd(emi_stream_t stream, const void* q, const void* k, const void* v, const void* o,
@@ -1195,40 +1465,54 @@ extern "C" int emi_attn_bwd(emi_stream_t stream, const void* q, const void* k, c
   const AttnShape shp{(int)seq, (int)heads, stride_b, stride_h, stride_s};
   const unsigned bh = (unsigned)(batch * heads);
   float* delta = static_cast<float*>(workspace);
+  float* lse2 = delta + (size_t)batch * heads * seq;
   const dim3 grid4((unsigned)((seq + 3) / 4), bh);
-  if (dtype == EMI_BF16)
+  const bool fast = mfma_ok(a, dtype, {q, k, v, o, d_o, dq, dk, dv});
+  // EMI_ATTN_BWD=0 selects the plain dK/dV kernel (for comparison); the software-pipelined
+  // one wants -delta in the workspace.
+  static const int bwd_variant = getenv("EMI_ATTN_BWD") ? atoi(getenv("EMI_ATTN_BWD")) : 1;
+  const float delta_sign = bwd_variant == 1 ? -1.0f : 1.0f;
+  if (fast) {
+    if (head_dim == 128)
+      hipLaunchKernelGGL(attn_prep_kernel<128>, dim3((unsigned)((seq + 15) / 16), bh), dim3(256), 0, st, (const uint16_t*)o,
+                         (const uint16_t*)d_o, lse, delta, lse2, shp, delta_sign);
+    else
+      hipLaunchKernelGGL(attn_prep_kernel<64>, dim3((unsigned)((seq + 31) / 32), bh), dim3(256), 0, st, (const uint16_t*)o,
+                         (const uint16_t*)d_o, lse, delta, lse2, shp, delta_sign);
+  } else if (dtype == EMI_BF16)
     hipLaunchKernelGGL(attn_delta_kernel<bf16>, grid4, dim3(256), 0, st, (const bf16*)o, (const bf16*)d_o, delta, shp,
                        (int)head_dim);
   else
     hipLaunchKernelGGL(attn_delta_kernel<float>, grid4, dim3(256), 0, st, (const float*)o, (const float*)d_o, delta, shp,
                        (int)head_dim);
   EMI_CHECK_LAUNCH("emi_attn_bwd(delta)");
-  if (mfma_ok(a, dtype, {q, k, v, d_o, dq, dk, dv})) {
+  if (fast) {
     const uint32_t head_bytes = (uint32_t)(((seq - 1) * stride_s + head_dim) * 2);
     const dim3 grid((unsigned)((seq + 127) / 128), bh);
-    if (head_dim == 128) {
-      constexpr int smem_q = 2 * 2 * 64 * 128 * 2, smem_kv = 2 * (2 * 64 * 128 * 2 + 2 * 64 * 4);
-      if (int rc = reserve_lds(attn_bwd_dq_bf16_kernel<128>, smem_q, "emi_attn_bwd")) return rc;
-      if (int rc = reserve_lds(attn_bwd_dkv_bf16_kernel<128>, smem_kv, "emi_attn_bwd")) return rc;
-      hipLaunchKernelGGL(attn_bwd_dkv_bf16_kernel<128>, grid, dim3(256), smem_kv, st, (const uint16_t*)q,
-                         (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, (uint16_t*)dk,
-                         (uint16_t*)dv, shp, head_bytes, scale, causal);
-      EMI_CHECK_LAUNCH("emi_attn_bwd(dkv)");
-      hipLaunchKernelGGL(attn_bwd_dq_bf16_kernel<128>, grid, dim3(256), smem_q, st, (const uint16_t*)q,
-                         (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, (uint16_t*)dq, shp,
-                         head_bytes, scale, causal);
-    } else {
-      constexpr int smem_q = 2 * 2 * 64 * 64 * 2, smem_kv = 2 * (2 * 64 * 64 * 2 + 2 * 64 * 4);
-      if (int rc = reserve_lds(attn_bwd_dq_bf16_kernel<64>, smem_q, "emi_attn_bwd")) return rc;
-      if (int rc = reserve_lds(attn_bwd_dkv_bf16_kernel<64>, smem_kv, "emi_attn_bwd")) return rc;
-      hipLaunchKernelGGL(attn_bwd_dkv_bf16_kernel<64>, grid, dim3(256), smem_kv, st, (const uint16_t*)q,
-                         (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, (uint16_t*)dk,
-                         (uint16_t*)dv, shp, head_bytes, scale, causal);
-      EMI_CHECK_LAUNCH("emi_attn_bwd(dkv)");
-      hipLaunchKernelGGL(attn_bwd_dq_bf16_kernel<64>, grid, dim3(256), smem_q, st, (const uint16_t*)q,
-                         (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, (uint16_t*)dq, shp,
-                         head_bytes, scale, causal);
-    }
+#define EMI_ATTN_BWD_LAUNCH(DD)                                                                                          \
+  do {                                                                                                                   \
+    constexpr int smem_q = 2 * 2 * 64 * DD * 2, smem_kv = 2 * (2 * 64 * DD * 2 + 2 * 64 * 4);                            \
+    constexpr int smem_sp = 6 * 64 * DD * 2 + 3 * 512;                                                                   \
+    if (bwd_variant == 1) {                                                                                              \
+      if (int rc = reserve_lds(attn_bwd_dkv_sp_kernel<DD>, smem_sp, "emi_attn_bwd")) return rc;                          \
+      hipLaunchKernelGGL(attn_bwd_dkv_sp_kernel<DD>, grid, dim3(256), smem_sp, st, (const uint16_t*)q,                   \
+                         (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse2, delta, (uint16_t*)dk,       \
+                         (uint16_t*)dv, shp, head_bytes, scale, causal);                                                 \
+    } else {                                                                                                             \
+      if (int rc = reserve_lds(attn_bwd_dkv_bf16_kernel<DD>, smem_kv, "emi_attn_bwd")) return rc;                        \
+      hipLaunchKernelGGL(attn_bwd_dkv_bf16_kernel<DD>, grid, dim3(256), smem_kv, st, (const uint16_t*)q,                 \
+                         (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, (uint16_t*)dk,        \
+                         (uint16_t*)dv, shp, head_bytes, scale, causal);                                                 \
+    }                                                                                                                    \
+    EMI_CHECK_LAUNCH("emi_attn_bwd(dkv)");                                                                               \
+    if (int rc = reserve_lds(attn_bwd_dq_bf16_kernel<DD>, smem_q, "emi_attn_bwd")) return rc;                            \
+    hipLaunchKernelGGL(attn_bwd_dq_bf16_kernel<DD>, grid, dim3(256), smem_q, st, (const uint16_t*)q, (const uint16_t*)k, \
+                       (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, (uint16_t*)dq, shp, head_bytes, scale,      \
+                       causal, delta_sign);                                                                              \
+  } while (0)
+    if (head_dim == 128) EMI_ATTN_BWD_LAUNCH(128);
+    else EMI_ATTN_BWD_LAUNCH(64);
+#undef EMI_ATTN_BWD_LAUNCH
     EMI_CHECK_LAUNCH("emi_attn_bwd(dq)");
     return EMI_OK;
   }
