@@ -284,8 +284,9 @@ bool attn_dims(const XLA_FFI_Buffer* q, int64_t bshd, AttnDims* d) {
 }  // namespace
 
 extern "C" XLA_FFI_Error* emi_attn_fwd_ffi(XLA_FFI_CallFrame* cf) {
-  EMI_FFI_BEGIN("emi_attn_fwd", 3, 3, 2, 2)
+  EMI_FFI_BEGIN("emi_attn_fwd", 3, 3, 2, 3)
   const XLA_FFI_Buffer *q = f.arg(0), *k = f.arg(1), *v = f.arg(2), *o = f.ret(0), *lse = f.ret(1);
+  const XLA_FFI_Buffer* ws = cf->rets.size == 3 ? f.ret(2) : nullptr;
   if (!is_float(q) || k->dtype != q->dtype || v->dtype != q->dtype || o->dtype != q->dtype)
     return f.invalid("q, k, v, o must share one dtype, f32 or bf16 (code %lld)", q->dtype);
   int64_t causal = 1, bshd = 0;
@@ -298,9 +299,16 @@ extern "C" XLA_FFI_Error* emi_attn_fwd_ffi(XLA_FFI_CallFrame* cf) {
     return f.invalid("q, k, v, o must be rank 4 with one shape (q rank %lld)", q->rank);
   if (lse->dtype != XLA_FFI_DataType_F32 || lse->rank != 3 || lse->dims[0] != d.B || lse->dims[1] != d.H || lse->dims[2] != d.S)
     return f.invalid("lse must be f32[batch, heads, seq] = [%lld, %lld, %lld]", d.B, d.H, d.S);
+  // The optional workspace result holds the transposed copy of V; a buffer smaller than the query is an error,
+  // not a silent fall back to the slower path.
+  if (ws != nullptr) {
+    const size_t need = emi_attn_fwd_workspace_bytes(d.B, d.H, d.S, d.D);
+    if (byte_size(ws) < need) return f.invalid("workspace result has %lld bytes, %lld needed", (long long)byte_size(ws), (long long)need);
+  }
   EMI_FFI_STREAM()
-  return f.from_status(emi_attn_fwd(stream, q->data, k->data, v->data, o->data, static_cast<float*>(lse->data), d.B, d.H, d.S,
-                                    d.D, d.sb, d.sh, d.ss, (float)scale, (int)causal, q->dtype));
+  return f.from_status(emi_attn_fwd_ws(stream, q->data, k->data, v->data, o->data, static_cast<float*>(lse->data),
+                                       ws ? ws->data : nullptr, ws ? byte_size(ws) : 0, d.B, d.H, d.S, d.D, d.sb, d.sh, d.ss,
+                                       (float)scale, (int)causal, q->dtype));
 }
 
 extern "C" XLA_FFI_Error* emi_attn_bwd_ffi(XLA_FFI_CallFrame* cf) {

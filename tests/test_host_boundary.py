@@ -46,7 +46,7 @@ def test_plain_launchers_reject_bad_arguments_before_touching_the_gpu():
     assert lib.emi_attn_fwd(None, 16, 16, 16, 16, 16, 1, 1, 8, 512, 4096, 4096, 512, 1.0, 1, 16) == 3
     assert b"head_dim" in lib.emi_last_error()
     assert lib.emi_swiglu_fwd(None, 8, 16, 16, 64, 11) == 3                    # misaligned pointer
-    assert lib.emi_rmsnorm_bwd_workspace_bytes(32768, 4096) == (1024 + 8) * 4096 * 4   # partial rows + second level
+    assert lib.emi_rmsnorm_bwd_workspace_bytes(32768, 4096) == (512 + 1) * 4096 * 4    # partial rows + second level
 
 
 def _handler(name):
@@ -83,6 +83,8 @@ def test_ffi_metadata_probe_and_stages():
      {"scale": (F.F32, 0.1), "causal": (F.PRED, 1)}, "lse"),
     ("emi_attn_fwd_ffi", [(F.BF16, [1, 2, 64, 128])] * 3, [(F.BF16, [1, 2, 64, 128]), (F.F32, [1, 2, 64])],
      {"causal": (F.PRED, 1)}, "scale"),
+    ("emi_attn_fwd_ffi", [(F.BF16, [1, 2, 512, 128])] * 3, [(F.BF16, [1, 2, 512, 128]), (F.F32, [1, 2, 512]), (F.U8, [64])],
+     {"scale": (F.F32, 0.1), "causal": (F.PRED, 1)}, "workspace"),
     ("emi_attn_bwd_ffi", [(F.BF16, [1, 2, 64, 128])] * 4 + [(F.F32, [1, 2, 64]), (F.BF16, [1, 2, 64, 128])],
      [(F.BF16, [1, 2, 64, 128])] * 3 + [(F.U8, [8])], {"scale": (F.F32, 0.1)}, "workspace"),
     ("emi_embedding_fwd_ffi", [(F.S64, [3]), (F.F32, [10, 4])], [(F.F32, [3, 4])], {}, "s32"),
