@@ -81,15 +81,15 @@ def layer_flops(cfg):
 
 
 def gemm_launches(cfg):
-    """(role, M, N, K) of the 21 GEMM launches of one fwd+VJP step.  All of them run in
-    the NT layout C[M,N] = A[M,K] . B[N,K]^T: the weight is transposed for dX and both
-    operands are transposed for dW (ops.matmul_nt)."""
+    """(role, M, N, K) of the 21 GEMM launches of one fwd+VJP step.  Y and dX run in the
+    NT layout C[M,N] = A[M,K] . B[N,K]^T (the weight is transposed for dX), dW in the TN
+    layout C[M,N] = A[K,M]^T . B[K,N] on dY and X as stored (ops.matmul_nt)."""
     D, H, T = cfg["dim"], cfg["hidden_dim"], cfg["batch"] * cfg["seq"]
     out = []
     for (n_out, k_in) in [(D, D)] * 4 + [(H, D)] * 2 + [(D, H)]:
         out.append(("Y", T, n_out, k_in))         # Y  = X W^T
         out.append(("dX", T, k_in, n_out))        # dX = dY (W^T)^T
-        out.append(("dW", n_out, k_in, T))        # dW = dY^T (X^T)^T
+        out.append(("dW", n_out, k_in, T))        # dW = dY^T X
     return out
 
 
@@ -102,14 +102,18 @@ def bench_gemms(cfg, iters):
     flat_b = (torch.randn((T * big,), device="cuda") * 0.02).to(torch.bfloat16)
     calls = []
     for (role, M, N, K) in gemm_launches(cfg):
-        calls.append((role, flat_a[:M * K].view(M, K), flat_b[:N * K].view(N, K), 2.0 * M * N * K))
+        if role == "dW":
+            calls.append((role, flat_a[:M * K].view(K, M), flat_b[:N * K].view(K, N), 2.0 * M * N * K))
+        else:
+            calls.append((role, flat_a[:M * K].view(M, K), flat_b[:N * K].view(N, K), 2.0 * M * N * K))
     per_role = {}
     for role in ("Y", "dX", "dW"):
         mine = [c for c in calls if c[0] == role]
-        t = event_time(lambda: [ops.gemm(a, b, False, True) for (_, a, b, _) in mine], iters)
+        ta, tb = (True, False) if role == "dW" else (False, True)
+        t = event_time(lambda: [ops.gemm(a, b, ta, tb) for (_, a, b, _) in mine], iters)
         fl = sum(c[3] for c in mine)
         per_role[role] = dict(launches=len(mine), seconds=t, tflops=fl / t / 1e12)
-    t_all = event_time(lambda: [ops.gemm(a, b, False, True) for (_, a, b, _) in calls], iters)
+    t_all = event_time(lambda: [ops.gemm(a, b, r == "dW", r != "dW") for (r, a, b, _) in calls], iters)
     return t_all, sum(c[3] for c in calls), len(calls), per_role
 
 
@@ -270,7 +274,7 @@ def main():
         "%s\tHIP\trocm\tPrimal+VJP\t%.6f s  (%.1f TFLOP/s over %.2f TFLOP algorithmic)" % (name, dt, fl["total"] / dt / 1e12, fl["total"] / 1e12))
 
     t_gemm, gemm_fl, n_gemm, per_layout = bench_gemms(cfg, max(5, min(args.steps, 20)))
-    roofline = dict(bound="mfma", kernel="gemm_bf16_nt_pingpong_kernel (256x256x64 tiles; %d launches per step: Y, dX, dW of 7 weights)" % n_gemm,
+    roofline = dict(bound="mfma", kernel="gemm_bf16_pingpong_kernel (256x256x64 tiles; %d launches per step: Y, dX in the NT form, dW in the TN form, 7 weights)" % n_gemm,
                     achieved=gemm_fl / t_gemm / 1e12, peak=PEAK_BF16_TFLOPS, unit="TFLOP/s",
                     frac=gemm_fl / t_gemm / 1e12 / PEAK_BF16_TFLOPS,
                     traffic=GEMM_TRAFFIC_BYTES_PER_LAUNCH if (args.seq, args.batch) == (C5["seq"], C5["batch"]) else None,

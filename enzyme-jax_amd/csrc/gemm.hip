@@ -14,6 +14,8 @@
 // Generic path (fp32, or bf16 with shapes/alignments the fast path does not
 // take): v_mfma_f32_32x32x2_f32 with predicated scalar loads.
 #include <stdlib.h>
+#include <type_traits>
+#include <utility>
 
 #include "emi_device.h"
 
@@ -366,8 +368,9 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_kernel(const uint16_t* 
 // The wave tile is (16*TM) x 64; rows of 128 bytes in the wave's LDS slice, 16-byte
 // chunk c of row r at chunk c ^ ((r >> 1) & 7): conflict free both for the 8-byte
 // column-quad accesses of the accumulator layout and for the 16-byte row accesses
-// of the global loads and stores.
-template <int TM, int TN>
+// of the global loads and stores.  CSPLIT: the wave tile's columns 32..63 lie CSPLIT
+// columns further right in C (two 32-column strips instead of one 64-column strip).
+template <int TM, int TN, int CSPLIT = 0>
 __device__ __forceinline__ void epilogue_bf16_t16(f32x4_t (&acc)[TM][TN], EMI_LDS uint8_t* smem, int wave, int lane,
                                                   int rbase, int cbase, const uint16_t* R, uint16_t* C, int M, int N,
                                                   int ldr, int ldc, int vec_ok) {
@@ -379,11 +382,59 @@ __device__ __forceinline__ void epilogue_bf16_t16(f32x4_t (&acc)[TM][TN], EMI_LD
     const int chunk = 2 * j + (lq >> 1);
     return row * RSB + ((chunk ^ ((row >> 1) & 7)) << 4) + ((lq & 1) << 3);
   };
+  // Whole wave tile inside C and 16-byte accesses allowed (wave-uniform): straight-line
+  // code, the residual comes in with direct-to-LDS loads that are all in flight at once.
+  if (vec_ok && rbase + WR <= M && cbase + CSPLIT + 64 <= N) {
+    // Wave-load it covers rows 8*it .. 8*it+7: lane l moves physical chunk (l & 7) of row 8*it + (l >> 3),
+    // whose swizzle term ((row >> 1) & 7) only depends on the parity of it.
+    const int prow = lane >> 3, pc = lane & 7;
+    const uint32_t ldsE = prow * RSB + ((pc ^ (prow >> 1)) << 4), ldsO = prow * RSB + ((pc ^ ((prow >> 1) + 4)) << 4);
+    if (R != nullptr) {
+      const uint8_t* rb = reinterpret_cast<const uint8_t*>(R + (int64_t)rbase * ldr + cbase);   // wave-uniform
+      const int cE = pc ^ (prow >> 1), cO = pc ^ ((prow >> 1) + 4);                            // logical chunks
+      const uint32_t gE = (uint32_t)prow * (uint32_t)ldr * 2u + (cE << 4) + (cE >= 4 ? CSPLIT * 2 : 0);
+      const uint32_t gO = (uint32_t)prow * (uint32_t)ldr * 2u + (cO << 4) + (cO >= 4 ? CSPLIT * 2 : 0);
+#pragma unroll
+      for (int it = 0; it < WR / 8; it++) {
+        const uint8_t* src = rb + (int64_t)it * 16 * ldr + ((it & 1) ? gO : gE);
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                         (EMI_LDS void*)(wl + it * 1024), 16, 0, 0);
+      }
+      wait_vmcnt<0>();
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+          const u32x2_t w = *reinterpret_cast<const EMI_LDS u32x2_t*>(wl + quad_slot(i * 16 + lrow, j));
+          acc[i][j][0] += __uint_as_float(w[0] << 16);
+          acc[i][j][1] += __uint_as_float(w[0] & 0xffff0000u);
+          acc[i][j][2] += __uint_as_float(w[1] << 16);
+          acc[i][j][3] += __uint_as_float(w[1] & 0xffff0000u);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int j = 0; j < TN; j++) {
+        u32x2_t w;
+        w[0] = pack_bf16x2(acc[i][j][0], acc[i][j][1]);
+        w[1] = pack_bf16x2(acc[i][j][2], acc[i][j][3]);
+        *reinterpret_cast<EMI_LDS u32x2_t*>(wl + quad_slot(i * 16 + lrow, j)) = w;
+      }
+    uint8_t* cb = reinterpret_cast<uint8_t*>(C + (int64_t)rbase * ldc + cbase);                  // wave-uniform
+    const uint32_t gC = (uint32_t)prow * (uint32_t)ldc * 2u + (pc << 4) + (pc >= 4 ? CSPLIT * 2 : 0);
+#pragma unroll
+    for (int it = 0; it < WR / 8; it++) {
+      const u32x4_t v = *reinterpret_cast<const EMI_LDS u32x4_t*>(wl + it * 1024 + ((it & 1) ? ldsO : ldsE));
+      *reinterpret_cast<u32x4_t*>(cb + (int64_t)it * 16 * ldc + gC) = v;
+    }
+    return;
+  }
   if (R != nullptr) {
 #pragma unroll
     for (int it = 0; it < WR / 8; it++) {
       const int row = it * 8 + (lane >> 3), c = lane & 7;
-      const int grow = rbase + row, gcol = cbase + c * 8;
+      const int grow = rbase + row, gcol = cbase + c * 8 + (c >= 4 ? CSPLIT : 0);
       u32x4_t v = {0u, 0u, 0u, 0u};
       if (grow < M && gcol < N) {
         const uint16_t* src = R + (int64_t)grow * ldr + gcol;
@@ -420,7 +471,7 @@ __device__ __forceinline__ void epilogue_bf16_t16(f32x4_t (&acc)[TM][TN], EMI_LD
 #pragma unroll
   for (int it = 0; it < WR / 8; it++) {
     const int row = it * 8 + (lane >> 3), c = lane & 7;
-    const int grow = rbase + row, gcol = cbase + c * 8;
+    const int grow = rbase + row, gcol = cbase + c * 8 + (c >= 4 ? CSPLIT : 0);
     const u32x4_t v = *reinterpret_cast<const EMI_LDS u32x4_t*>(wl + row * RSB + ((c ^ ((row >> 1) & 7)) << 4));
     if (grow < M && gcol < N) {
       uint16_t* dst = C + (int64_t)grow * ldc + gcol;
@@ -456,26 +507,55 @@ __device__ __forceinline__ void epilogue_bf16_t16(f32x4_t (&acc)[TM][TN], EMI_LD
 // <= L-2 by both groups; a wavefront waits for its own loads (vmcnt) two local
 // slots before the first read of that region by either group.
 // ---------------------------------------------------------------------------
-#ifdef EMI_GEMM_TRACE
-__device__ unsigned long long emi_gemm_trace_buf[8 * 40];
-#define EMI_TRACE_MARK() do { if (tracing) ts[nts++] = __builtin_readcyclecounter(); } while (0)
-#if EMI_GEMM_TRACE > 1
-#define EMI_TRACE_MARK2() EMI_TRACE_MARK()
-#else
-#define EMI_TRACE_MARK2() do { } while (0)
-#endif
-#else
-#define EMI_TRACE_MARK() do { } while (0)
-#define EMI_TRACE_MARK2() do { } while (0)
-#endif
+// Transposing LDS read through inline asm with an immediate offset: the compiler
+// orders every LDS read it knows of behind all outstanding direct-to-LDS loads,
+// which would serialise loading and compute.  The result is valid after the next
+// lds_tr_fence() over it.
+template <int OFF> __device__ __forceinline__ u32x2_t lds_tr_read(uint32_t addr) {
+  static_assert(OFF >= 0 && OFF < 65536, "ds offset field");
+  u32x2_t r;
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF));
+  return r;
+}
+// Waits for all LDS reads of this wavefront; the values passed in cannot be used
+// (or copied) by the compiler before the wait.
+__device__ __forceinline__ void lds_tr_fence(u32x2_t (&t)[4][2][2]) {
+  asm volatile("s_waitcnt lgkmcnt(0)"
+               : "+v"(t[0][0][0]), "+v"(t[0][0][1]), "+v"(t[0][1][0]), "+v"(t[0][1][1]), "+v"(t[1][0][0]), "+v"(t[1][0][1]),
+                 "+v"(t[1][1][0]), "+v"(t[1][1][1]));
+  asm volatile(""
+               : "+v"(t[2][0][0]), "+v"(t[2][0][1]), "+v"(t[2][1][0]), "+v"(t[2][1][1]), "+v"(t[3][0][0]), "+v"(t[3][0][1]),
+                 "+v"(t[3][1][0]), "+v"(t[3][1][1]));
+}
+template <typename F, int... Is>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, Is...>) {
+  (f(std::integral_constant<int, Is>{}), ...);
+}
+template <int N, typename F> __device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
 
-__global__ __launch_bounds__(512) void gemm_bf16_nt_pingpong_kernel(const uint16_t* __restrict__ A,
-                                                                     const uint16_t* __restrict__ B, const uint16_t* R,
-                                                                     uint16_t* C, int M, int N, int K, int lda, int ldb,
-                                                                     int ldr, int ldc, uint32_t a_bytes, uint32_t b_bytes,
-                                                                     int vec_ok) {
+// AKM / BKM: the operand is stored k-major (A as [K][M], B as [K][N]) instead of
+// k-contiguous (A as [M][K], B as [N][K]).  A k-major region holds [64 k][128 c]
+// (256-byte rows), chunk ch of k-row k at ch ^ 4(k&3) ^ 2((k>>3)&1).  For A, c runs over
+// the same block rows as the 128 rows of a k-contiguous region (two runs of 64; one run of
+// 128 measured slower).  For B, region B_j is the contiguous block columns 128j + [0,128)
+// and a wavefront owns the two 32-column strips 128j + 32*wn + [0,32) of C, so that every
+// k-row of a region is one 256-byte run in memory.  A k-major region is
+// read with two transposing loads per fragment: the 32 lanes that are served
+// together address k-rows {0..3} and {8..11} (+4 for the second load), 32 bytes
+// each, which the swizzle spreads over all 64 banks.
+template <bool AKM, bool BKM>
+__global__ __launch_bounds__(512) void gemm_bf16_pingpong_kernel(const uint16_t* __restrict__ A,
+                                                                  const uint16_t* __restrict__ B, const uint16_t* R,
+                                                                  uint16_t* C, int M, int N, int K, int lda, int ldb,
+                                                                  int ldr, int ldc, uint32_t a_bytes, uint32_t b_bytes,
+                                                                  int vec_ok) {
   constexpr int BM = 256, BN = 256, BK = 64;
-  constexpr int REGION = 128 * BK * 2, STAGE = 4 * REGION;      // 16 KiB, 64 KiB
+  constexpr int REGION = 128 * BK * 2;                          // 16 KiB
+  // LDS map: A_h of stage s at (2s + h) regions, B_j of stage s at 64 KiB + (2s + j) regions, so that
+  // every offset from a lane's A (or B) base address fits the 16-bit offset field of an LDS read.
+  constexpr int B_BASE = 4 * REGION;
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem_raw[];
   EMI_LDS uint8_t* smem = (EMI_LDS uint8_t*)smem_raw;
 
@@ -491,39 +571,72 @@ __global__ __launch_bounds__(512) void gemm_bf16_nt_pingpong_kernel(const uint16
   const __amdgpu_buffer_rsrc_t rA = make_rsrc(A, a_bytes);
   const __amdgpu_buffer_rsrc_t rB = make_rsrc(B, b_bytes);
 
-  // HBM -> LDS: a region is 16 wave-loads of 1 KiB (8 rows x 128 bytes); wavefront w
-  // issues loads w and w+8 of every region.  Lane l of a wave-load fills physical
-  // chunk (l & 7) of region row q*8 + (l >> 3) and therefore fetches the logical
-  // chunk that the swizzle maps there.
-  const int lck = ((lane & 7) ^ (((lane >> 4) + 4 * (wave & 1)) & 7)) * 8;     // k offset of this lane's chunk
+  // HBM -> LDS: a region is 16 wave-loads of 1 KiB; wavefront w issues loads w and w+8 of
+  // every region.  k-contiguous: a wave-load is 8 rows x 128 bytes, lane l fills physical
+  // chunk (l & 7) of region row 8q + (l >> 3).  k-major: 4 k-rows x 256 bytes, lane l fills
+  // physical chunk (l & 15) of k-row 4q + (l >> 4).  Either way the lane fetches the logical
+  // chunk that the swizzle maps to its slot.  lk: the k index (within the tile) of the chunk.
   uint32_t voffA[2][2], voffB[2][2];
+  int lkA[2], lkB[2];
+  const int lck = ((lane & 7) ^ (((lane >> 4) + 4 * (wave & 1)) & 7)) * 8;     // k-contiguous: k offset of the chunk
 #pragma unroll
   for (int it = 0; it < 2; it++) {
-    const int rho = (it * 8 + wave) * 8 + (lane >> 3);
+    const int q = it * 8 + wave;
+    const int rho = q * 8 + (lane >> 3);                                       // k-contiguous: region row
+    const int km = q * 4 + (lane >> 4);                                        // k-major: k-row
+    const int cm = ((lane & 15) ^ (4 * (km & 3)) ^ (2 * ((km >> 3) & 1))) * 8; // k-major: first of 8 columns
+    lkA[it] = AKM ? km : lck;
+    lkB[it] = BKM ? km : lck;
 #pragma unroll
     for (int h = 0; h < 2; h++) {
-      const int grow = m0 + (rho >> 6) * 128 + h * 64 + (rho & 63);
-      voffA[h][it] = grow < M ? ((uint32_t)grow * (uint32_t)lda + (uint32_t)lck) * 2u : kOob;
-      const int gcol = n0 + (rho >> 5) * 64 + h * 32 + (rho & 31);
-      voffB[h][it] = gcol < N ? ((uint32_t)gcol * (uint32_t)ldb + (uint32_t)lck) * 2u : kOob;
+      if constexpr (AKM) {
+        const int grow = m0 + (cm >> 6) * 128 + h * 64 + (cm & 63);
+        voffA[h][it] = grow < M ? ((uint32_t)km * (uint32_t)lda + (uint32_t)grow) * 2u : kOob;
+      } else {
+        const int grow = m0 + (rho >> 6) * 128 + h * 64 + (rho & 63);
+        voffA[h][it] = grow < M ? ((uint32_t)grow * (uint32_t)lda + (uint32_t)lck) * 2u : kOob;
+      }
+      if constexpr (BKM) {
+        const int gcol = n0 + h * 128 + cm;
+        voffB[h][it] = gcol < N ? ((uint32_t)km * (uint32_t)ldb + (uint32_t)gcol) * 2u : kOob;
+      } else {
+        const int gcol = n0 + (rho >> 5) * 64 + h * 32 + (rho & 31);
+        voffB[h][it] = gcol < N ? ((uint32_t)gcol * (uint32_t)ldb + (uint32_t)lck) * 2u : kOob;
+      }
     }
   }
-  auto refill = [&](__amdgpu_buffer_rsrc_t rsrc, const uint32_t (&voff)[2], int lds_off, int k0) {
-#pragma unroll
-    for (int it = 0; it < 2; it++) {
-      const uint32_t v = (k0 + lck < K) ? voff[it] + (uint32_t)k0 * 2u : kOob;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, smem + lds_off + (it * 8 + wave) * 1024, 16, v, 0, 0, 0);
-    }
+  const uint32_t kbytesA = AKM ? (uint32_t)lda * 2u : 2u, kbytesB = BKM ? (uint32_t)ldb * 2u : 2u;   // bytes per step in k
+  auto refillA = [&](int h, int lds_off, int it, int k0) __attribute__((always_inline)) {
+    const uint32_t v = (k0 + lkA[it] < K) ? voffA[h][it] + (uint32_t)k0 * kbytesA : kOob;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rA, smem + lds_off + (it * 8 + wave) * 1024, 16, v, 0, 0, 0);
+  };
+  auto refillB = [&](int j, int lds_off, int it, int k0) __attribute__((always_inline)) {
+    const uint32_t v = (k0 + lkB[it] < K) ? voffB[j][it] + (uint32_t)k0 * kbytesB : kOob;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rB, smem + lds_off + (it * 8 + wave) * 1024, 16, v, 0, 0, 0);
   };
 
-  // LDS -> registers.  Fragment of v_mfma_f32_16x16x32_bf16 (16 rows x 32 k): lane l
-  // reads row (l & 15), logical chunk 4*ks + (l >> 4) of k-step ks.
-  const int l15 = lane & 15, sw = l15 >> 1, kq = lane >> 4;
+  // LDS -> registers.  Fragment of v_mfma_f32_16x16x32_bf16 (16 rows x 32 k): lane l holds
+  // row (l & 15), k = 8*(l >> 4) .. +7 of k-step ks.
+  // k-contiguous: one 16-byte read of logical chunk 4*ks + (l >> 4).
+  const int l15 = lane & 15, sw = l15 >> 1, kq4 = lane >> 4;
   const int a_lane = (wm * 64 + l15) * (BK * 2);
-  const int b_lane = 2 * REGION + (wn * 32 + l15) * (BK * 2);
-  auto frag = [&](int base, int ks) {
-    return *reinterpret_cast<const EMI_LDS bf16x8_t*>(smem + base + (((ks * 4 + kq) ^ sw) << 4));
+  const int b_lane = B_BASE + (wn * 32 + l15) * (BK * 2);
+  auto frag = [&](int base, int ks) __attribute__((always_inline)) {
+    return *reinterpret_cast<const EMI_LDS bf16x8_t*>(smem + base + (((ks * 4 + kq4) ^ sw) << 4));
   };
+  // k-major: two transposing reads; within 16 lanes, lane i addresses k-row (i >> 2), columns
+  // 4*(i & 3).. +3 and receives column i, k-rows 0..3.  tadrA[blk] / tadrB[blk]: LDS address of
+  // this lane's 8 bytes for 16-row block blk, k-step 0, first read, region 0.
+  uint32_t tadrA[4], tadrB[2];
+  {
+    const int kq = l15 >> 2, g = lane >> 4, x = (l15 & 3) >> 1;
+    const int t = x ^ (4 * kq) ^ (2 * (g & 1));
+    const uint32_t lane_part = (uint32_t)(uintptr_t)smem + (uint32_t)((8 * g + kq) * 256 + (l15 & 1) * 8);
+#pragma unroll
+    for (int blk = 0; blk < 4; blk++) tadrA[blk] = lane_part + (uint32_t)(((wm * 8 + blk * 2) ^ t) << 4);
+#pragma unroll
+    for (int blk = 0; blk < 2; blk++) tadrB[blk] = lane_part + (uint32_t)B_BASE + (uint32_t)(((wn * 4 + blk * 2) ^ t) << 4);
+  }
 
   // acc[i][j]: 16x16 tile at wave rows 16*i, wave columns 16*j (i = 4*h + row block)
   f32x4_t acc[8][4];
@@ -535,20 +648,19 @@ __global__ __launch_bounds__(512) void gemm_bf16_nt_pingpong_kernel(const uint16
       for (int r = 0; r < 4; r++) acc[i][j][r] = 0.f;
 
   bf16x8_t fa[4][2], fb[4][2];               // [16-row block][k-step]; fb: 0,1 = B_0, 2,3 = B_1
-#ifdef EMI_GEMM_TRACE
-  unsigned long long ts[40];
-  int nts = 0;
-  bool tracing = false;
-#endif
-  auto slot_end = [&]() {
+  u32x2_t ta[4][2][2], tb[4][2][2];          // halves of k-major fragments in flight
+  auto join = [&](const u32x2_t (&t)[2]) __attribute__((always_inline)) {
+    const u32x4_t w = {t[0][0], t[0][1], t[1][0], t[1][1]};
+    return __builtin_bit_cast(bf16x8_t, w);
+  };
+  auto slot_end = [&]() __attribute__((always_inline)) {
     __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_barrier();
-    EMI_TRACE_MARK();
     __builtin_amdgcn_sched_barrier(0);
   };
   // Compute slot: the 64 x 64 half of the wave tile that uses row half h (32 MFMAs).
   // The operands are passed swapped so that a lane owns 4 consecutive C columns.
-  auto half_rows = [&](int h) {
+  auto half_rows = [&](int h) __attribute__((always_inline)) {
     __builtin_amdgcn_s_setprio(1);
 #pragma unroll
     for (int ks = 0; ks < 2; ks++)
@@ -560,53 +672,99 @@ __global__ __launch_bounds__(512) void gemm_bf16_nt_pingpong_kernel(const uint16
     __builtin_amdgcn_s_setprio(0);
     slot_end();
   };
-  auto refill1 = [&](__amdgpu_buffer_rsrc_t rsrc, uint32_t voff, int lds_off, int it, int k0) {
-    const uint32_t v = (k0 + lck < K) ? voff + (uint32_t)k0 * 2u : kOob;
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, smem + lds_off + (it * 8 + wave) * 1024, 16, v, 0, 0, 0);
+  // Read 16-row block blk (0..3) of region A_h / block blk (0..1) of region B_j of stage S, k-step ks.
+  auto readA = [&](auto S, auto h, auto blk, auto ks) __attribute__((always_inline)) {
+    constexpr int off = (2 * decltype(S)::value + decltype(h)::value) * REGION;
+    constexpr int b = decltype(blk)::value, k = decltype(ks)::value;
+    if constexpr (AKM) {
+      ta[b][k][0] = lds_tr_read<off + k * 32 * 256>(tadrA[b]);
+      ta[b][k][1] = lds_tr_read<off + k * 32 * 256 + 4 * 256>(tadrA[b]);
+    } else {
+      fa[b][k] = frag(off + a_lane + b * 16 * BK * 2, k);
+    }
   };
-  auto tile_step = [&](int stage, int t) {
-    const int so = stage * STAGE, oo = (stage ^ 1) * STAGE;
+  auto readB = [&](auto S, auto j, auto blk, auto ks) __attribute__((always_inline)) {
+    constexpr int off = (2 * decltype(S)::value + decltype(j)::value) * REGION;
+    constexpr int b = decltype(blk)::value, k = decltype(ks)::value, f = 2 * decltype(j)::value + b;
+    if constexpr (BKM) {
+      tb[f][k][0] = lds_tr_read<off + k * 32 * 256>(tadrB[b]);
+      tb[f][k][1] = lds_tr_read<off + k * 32 * 256 + 4 * 256>(tadrB[b]);
+    } else {
+      fb[f][k] = frag(off + b_lane + b * 16 * BK * 2, k);
+    }
+  };
+  using I0 = std::integral_constant<int, 0>;
+  using I1 = std::integral_constant<int, 1>;
+  auto tile_step = [&](auto S, int t) __attribute__((always_inline)) {
+    constexpr int s = decltype(S)::value, o = s ^ 1;
+    constexpr int offA0 = (2 * s) * REGION, offB0 = B_BASE + (2 * s) * REGION;                     // this stage
+    constexpr int offA1o = (2 * o + 1) * REGION, offB1o = B_BASE + (2 * o + 1) * REGION;           // other stage
     // Ma: read B_0, A_0, B_1 of this stage; refill B_1, A_1 of the other stage (tile t+1).
     // Loads and reads alternate so that the texture path and the LDS work in parallel.
+    static_for<4>([&](auto qc) __attribute__((always_inline)) {
+      constexpr int q = decltype(qc)::value;
+      if constexpr (q < 2) refillB(1, offB1o, q, (t + 1) * BK);
+      else refillA(1, offA1o, q - 2, (t + 1) * BK);
+      using KS = std::integral_constant<int, (q >> 1)>;
+      using BL = std::integral_constant<int, (q & 1)>;
+      using BA0 = std::integral_constant<int, 2 * (q & 1)>;
+      using BA1 = std::integral_constant<int, 2 * (q & 1) + 1>;
+      readB(S, I0{}, BL{}, KS{});
+      readA(S, I0{}, BA0{}, KS{});
+      readA(S, I0{}, BA1{}, KS{});
+      readB(S, I1{}, BL{}, KS{});
+    });
+    if constexpr (AKM) lds_tr_fence(ta);
+    if constexpr (BKM) lds_tr_fence(tb);
+    if constexpr (AKM) {
 #pragma unroll
-    for (int q = 0; q < 4; q++) {
-      if (q < 2) refill1(rB, voffB[1][q], oo + 3 * REGION, q, (t + 1) * BK);
-      else refill1(rA, voffA[1][q - 2], oo + REGION, q - 2, (t + 1) * BK);
-      const int ks = q >> 1, blk = q & 1;    // two 16-row blocks per q
-      fb[blk][ks] = frag(so + b_lane + blk * 16 * BK * 2, ks);
-      fa[2 * blk][ks] = frag(so + a_lane + (2 * blk) * 16 * BK * 2, ks);
-      fa[2 * blk + 1][ks] = frag(so + a_lane + (2 * blk + 1) * 16 * BK * 2, ks);
-      fb[2 + blk][ks] = frag(so + b_lane + REGION + blk * 16 * BK * 2, ks);
+      for (int b = 0; b < 4; b++)
+#pragma unroll
+        for (int k = 0; k < 2; k++) fa[b][k] = join(ta[b][k]);
     }
-    EMI_TRACE_MARK2();
+    if constexpr (BKM) {
+#pragma unroll
+      for (int b = 0; b < 4; b++)
+#pragma unroll
+        for (int k = 0; k < 2; k++) fb[b][k] = join(tb[b][k]);
+    }
     wait_vmcnt<8>();                        // own part of A_1 of this tile has landed
-    EMI_TRACE_MARK2();
     slot_end();
     half_rows(0);                           // Ca
     // Mb: read A_1; refill A_0, B_0 of this stage (tile t+2)
+    static_for<4>([&](auto qc) __attribute__((always_inline)) {
+      constexpr int q = decltype(qc)::value;
+      if constexpr (q < 2) refillA(0, offA0, q, (t + 2) * BK);
+      else refillB(0, offB0, q - 2, (t + 2) * BK);
+      using KS = std::integral_constant<int, (q >> 1)>;
+      using BA0 = std::integral_constant<int, 2 * (q & 1)>;
+      using BA1 = std::integral_constant<int, 2 * (q & 1) + 1>;
+      readA(S, I1{}, BA0{}, KS{});
+      readA(S, I1{}, BA1{}, KS{});
+    });
+    if constexpr (AKM) {
+      lds_tr_fence(ta);
 #pragma unroll
-    for (int q = 0; q < 4; q++) {
-      if (q < 2) refill1(rA, voffA[0][q], so, q, (t + 2) * BK);
-      else refill1(rB, voffB[0][q - 2], so + 2 * REGION, q - 2, (t + 2) * BK);
-      const int ks = q >> 1, blk = q & 1;
-      fa[2 * blk][ks] = frag(so + REGION + a_lane + (2 * blk) * 16 * BK * 2, ks);
-      fa[2 * blk + 1][ks] = frag(so + REGION + a_lane + (2 * blk + 1) * 16 * BK * 2, ks);
+      for (int b = 0; b < 4; b++)
+#pragma unroll
+        for (int k = 0; k < 2; k++) fa[b][k] = join(ta[b][k]);
     }
-    EMI_TRACE_MARK2();
     wait_vmcnt<6>();                        // own part of A_0, B_0 and of B_1 of the next tile
-    EMI_TRACE_MARK2();
     slot_end();
     half_rows(1);                           // Cb
   };
 
   // Prologue: tile 0 into stage 0; A_0, B_0 of tile 1 into stage 1 (its A_1, B_1 are
   // issued by the first memory slot).
-  refill(rA, voffA[0], 0, 0);
-  refill(rB, voffB[0], 2 * REGION, 0);
-  refill(rB, voffB[1], 3 * REGION, 0);
-  refill(rA, voffA[1], REGION, 0);
-  refill(rA, voffA[0], STAGE, BK);
-  refill(rB, voffB[0], STAGE + 2 * REGION, BK);
+#pragma unroll
+  for (int it = 0; it < 2; it++) {
+    refillA(0, 0, it, 0);
+    refillB(0, B_BASE, it, 0);
+    refillB(1, B_BASE + REGION, it, 0);
+    refillA(1, REGION, it, 0);
+    refillA(0, 2 * REGION, it, BK);
+    refillB(0, B_BASE + 2 * REGION, it, BK);
+  }
   wait_vmcnt<0>();
   slot_end();
   if (wm == 1) slot_end();                  // second group runs one slot behind the first
@@ -614,24 +772,17 @@ __global__ __launch_bounds__(512) void gemm_bf16_nt_pingpong_kernel(const uint16
   const int nk = (K + BK - 1) / BK;
   int t = 0;
   for (; t + 1 < nk; t += 2) {
-#ifdef EMI_GEMM_TRACE
-    tracing = (blockIdx.x == 300 && (t == 16 || t == 18));
-#endif
-    tile_step(0, t);
-    tile_step(1, t + 1);
+    tile_step(I0{}, t);
+    tile_step(I1{}, t + 1);
   }
-#ifdef EMI_GEMM_TRACE
-  tracing = false;
-  if (blockIdx.x == 300 && lane == 0)
-    for (int i = 0; i < 40; i++) emi_gemm_trace_buf[wave * 40 + i] = i < nts ? ts[i] : 0ull;
-#endif
-  if (t < nk) tile_step(0, t);
+  if (t < nk) tile_step(I0{}, t);
 
   if (wm == 0) slot_end();
   wait_vmcnt<0>();                          // zero-filled loads past the end of K
   slot_end();
 
-  epilogue_bf16_t16<8, 4>(acc, smem, wave, lane, m0 + wm * 128, n0 + wn * 64, R, C, M, N, ldr, ldc, vec_ok);
+  epilogue_bf16_t16<8, 4, (BKM ? 96 : 0)>(acc, smem, wave, lane, m0 + wm * 128, n0 + wn * (BKM ? 32 : 64), R, C, M, N, ldr,
+                                          ldc, vec_ok);
 }
 
 // ---------------------------------------------------------------------------
@@ -733,6 +884,7 @@ static int launch_bf16(hipStream_t st, const void* A, const void* B, const void*
   return EMI_OK;
 }
 
+template <bool AKM, bool BKM>
 static int launch_bf16_pingpong(hipStream_t st, const void* A, const void* B, const void* R, void* C, int M, int N, int K,
                                 int lda, int ldb, int ldr, int ldc, uint32_t a_bytes, uint32_t b_bytes) {
   const int vec_ok = ((reinterpret_cast<uintptr_t>(C) & 15) == 0 && ldc % 8 == 0 &&
@@ -741,13 +893,13 @@ static int launch_bf16_pingpong(hipStream_t st, const void* A, const void* B, co
   constexpr int smem = 2 * 65536;
   static bool configured = false;   // idempotent; a race only repeats the call
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_nt_pingpong_kernel),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_pingpong_kernel<AKM, BKM>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return emi_fail(EMI_INTERNAL, "emi_gemm: cannot reserve %d bytes of LDS: %s", smem, hipGetErrorString(e));
     configured = true;
   }
   const int tiles = ((M + 255) / 256) * ((N + 255) / 256);
-  hipLaunchKernelGGL(gemm_bf16_nt_pingpong_kernel, dim3(tiles), dim3(512), smem, st, static_cast<const uint16_t*>(A),
+  hipLaunchKernelGGL((gemm_bf16_pingpong_kernel<AKM, BKM>), dim3(tiles), dim3(512), smem, st, static_cast<const uint16_t*>(A),
                      static_cast<const uint16_t*>(B), static_cast<const uint16_t*>(R), static_cast<uint16_t*>(C), M, N, K,
                      lda, ldb, ldr, ldc, a_bytes, b_bytes, vec_ok);
   EMI_CHECK_LAUNCH("emi_gemm");
@@ -775,14 +927,12 @@ static int launch_bf16_layout(hipStream_t st, const void* A, const void* B, cons
     // 256x256 tiles when they fill the chip (the ping-pong kernel for two
     // k-contiguous operands), else 128x128.
     const int64_t big_tiles = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
-    cfg = big_tiles >= 192 ? ((!AK && !BKM) ? 5 : 1) : 4;
+    cfg = big_tiles >= 192 ? 5 : 4;
   }
 #define EMI_GEMM_ARGS st, A, B, R, C, M, N, K, lda, ldb, ldr, ldc, a_bytes, b_bytes
   switch (cfg) {
     case 1: return launch_bf16<256, 256, 64, 2, 2, 4, AK, BKM>(EMI_GEMM_ARGS);
-    case 5:
-      if constexpr (!AK && !BKM) return launch_bf16_pingpong(EMI_GEMM_ARGS);
-      else return launch_bf16<256, 256, 64, 2, 2, 4, AK, BKM>(EMI_GEMM_ARGS);
+    case 5: return launch_bf16_pingpong<AK, BKM>(EMI_GEMM_ARGS);
     case 2: return launch_bf16<256, 256, 32, 4, 2, 4, AK, BKM>(EMI_GEMM_ARGS);
     default: return launch_bf16<128, 128, 64, 2, 2, 2, AK, BKM>(EMI_GEMM_ARGS);
   }
@@ -804,11 +954,6 @@ static int launch_generic(hipStream_t st, const void* A, const void* B, const vo
 
 using namespace emi;
 
-#ifdef EMI_GEMM_TRACE
-extern "C" int emi_debug_gemm_trace(unsigned long long* out) {
-  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(emi_gemm_trace_buf), sizeof(unsigned long long) * 8 * 40);
-}
-#endif
 
 extern "C" int emi_gemm(emi_stream_t stream, const void* A, const void* B, const void* R, void* C, int64_t M, int64_t N,
                         int64_t K, int64_t lda, int64_t ldb, int64_t ldr, int64_t ldc, int trans_a, int trans_b,

@@ -220,8 +220,7 @@ _transposed = {}      # (data_ptr, shape) -> a^T, valid for the duration of one 
 
 
 def _transpose_shared(a):
-    """a^T, computed once per reverse pass for an operand several adjoint GEMMs
-    share (the normed activations feed wq/wk/wv, and w1/w3)."""
+    """a^T, computed once per reverse pass however many adjoint GEMMs read it."""
     key = (a.data_ptr(), tuple(a.shape), a.dtype)
     hit = _transposed.get(key)
     if hit is None:
@@ -261,19 +260,15 @@ def matmul_nt(x, w, residual=None):
     def rule(c, acc):
         c2 = c.reshape(-1, Nout)
         ax = None if acc[0] is None else acc[0].reshape(-1, K)
-        # dX = dY . W: W is transposed first (2|W| bytes of HBM traffic) so that the
-        # contraction index is innermost in both operands and the GEMM runs on the
-        # k-contiguous path, which is ~15% faster than the k-major one at these shapes.
+        # dX = dY . W: W is transposed first (2|W| bytes of HBM traffic, shared by nothing
+        # else) so that the contraction index is innermost in both operands: the
+        # k-contiguous kernel beats the k-major one by more than the transpose costs.
         dx = gemm(c2, _transpose_shared(w), False, True, ax).reshape(x.shape)
-        # dW = dY^T . X contracts over tokens, the slow index of both operands.  The
-        # k-major kernel has to fetch its fragments with the transposing LDS load,
-        # which makes it LDS-bound; transposing both operands in HBM and running the
-        # k-contiguous kernel is faster overall, and X^T is shared by the projections
-        # that read the same activations.
-        if c2.dtype == torch.bfloat16 and c2.shape[0] >= 2048:
-            dw = gemm(_transpose_shared(c2), _transpose_shared(x2), False, True, acc[1])
-        else:
-            dw = gemm(c2, x2, True, False, acc[1])               # dW = dY^T . X (TN)
+        # dW = dY^T . X contracts over tokens, the slow index of both operands: the
+        # k-major form of the GEMM kernel reads them in place (transposing LDS loads),
+        # 3-7% slower than the k-contiguous form but without two activation-sized
+        # transposes per projection.
+        dw = gemm(c2, x2, True, False, acc[1])
         out = [dx, dw]
         if residual is not None:
             out.append(_accumulate(acc[2], c))
