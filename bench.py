@@ -182,6 +182,35 @@ def bench_kernels(cfg, iters):
                                                             h * S * d, S * d, d, sc, 1, N.EMI_BF16)), fl)
     mfma("attn_bwd_c3", lambda: N.check(lib.emi_attn_bwd(st, P(q), P(k), P(v), P(o), P(lse), P(do), P(dq), P(dk), P(dv), P(ws), wsb,
                                                          B, h, S, d, h * S * d, S * d, d, sc, 1, N.EMI_BF16)), 2.5 * fl)
+    del q, k, v, do, o, dq, dk, dv, ws, fws
+    # Single-token (decode) step at the 7B layer's widths: mat-vec over W [11008, 4096] and its
+    # adjoints (weight read or written once), attention of one query per head over a
+    # 4096-row cache for 8 sequences (cache rows read once; the adjoint also writes dK, dV).
+    D = cfg["dim"]
+    w = (torch.randn((H, D), device="cuda") * 0.02).to(bf)
+    xv, yv, dyv, dxv = (torch.randn(n_, device="cuda").to(bf) for n_ in (D, H, H, D))
+    dw = torch.empty_like(w)
+    gm = lambda A, Bm, C, M_, N_, K_, lda, ldb, ta, tb: N.check(lib.emi_gemm(st, P(A), P(Bm), None, P(C), M_, N_, K_, lda, ldb,
+                                                                             N_, N_, ta, tb, N.EMI_BF16))
+    hbm("step_matvec_bf16", lambda: gm(xv, w, yv, 1, H, D, D, D, 0, 1), w.numel() * 2)
+    hbm("step_matvec_dx_bf16", lambda: gm(dyv, w, dxv, 1, D, H, H, D, 0, 0), w.numel() * 2)
+    hbm("step_matvec_dw_bf16", lambda: gm(dyv, xv, dw, H, D, 1, H, D, 1, 0), w.numel() * 2)
+    del w, dw
+    Bq, hq, Sk, dd = 8, 32, 4096, 128
+    Dq = hq * dd
+    qs, dos = (torch.randn((Bq, Dq), device="cuda").to(bf) for _ in range(2))
+    kc, vc = (torch.randn((Bq, Sk, Dq), device="cuda").to(bf) for _ in range(2))
+    os_, dqs = torch.empty_like(qs), torch.empty_like(qs)
+    dkc, dvc = torch.empty_like(kc), torch.empty_like(vc)
+    lses = torch.empty((Bq, hq), dtype=torch.float32, device="cuda")
+    strides = (Dq, dd, Sk * Dq, dd, Dq)
+    swb = lib.emi_attn_step_workspace_bytes(Bq, hq, Sk, dd)
+    sws = torch.empty(swb, dtype=torch.uint8, device="cuda")
+    hbm("step_attn_fwd_bf16", lambda: N.check(lib.emi_attn_step_fwd(st, P(qs), P(kc), P(vc), P(os_), P(lses), P(sws), swb, Bq, hq,
+                                                                    Sk, dd, *strides, dd ** -0.5, N.EMI_BF16)), 2 * kc.numel() * 2)
+    hbm("step_attn_bwd_bf16", lambda: N.check(lib.emi_attn_step_bwd(st, P(qs), P(kc), P(vc), P(os_), P(lses), P(dos), P(dqs),
+                                                                    P(dkc), P(dvc), P(sws), swb, Bq, hq, Sk, dd, *strides,
+                                                                    dd ** -0.5, N.EMI_BF16)), 4 * kc.numel() * 2)
     return out
 
 

@@ -1,0 +1,441 @@
+// Attention of the single-token (decode) step: one query per (batch, head) against the
+// seq_kv rows of that head's key/value cache, test/llama.py:178-206 with the softmax of
+// :13-18 (scale applied after the dot, max-subtracted).  HBM-bound: every cache row is read
+// once (forward and backward) and dK, dV are written once.  The keys of a head are split
+// over blocks of kKeysPerBlock (there are only batch*heads queries, far too few to fill
+// the chip); each block leaves a partial result (max, sum, unnormalised output; or its
+// share of dQ) in the workspace and a second small kernel combines them in a fixed order.
+// Inside a block 16 lanes share a key, each lane owning 16-byte chunks of the head
+// dimension, and every lane keeps four keys in flight.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "emi_device.h"
+
+namespace emi {
+namespace {
+
+constexpr int kRedFloats = 2048;                 // LDS floats for the reduction over key slots
+constexpr int kKeysPerBlock = 512, kUnroll = 4;
+
+template <typename T, bool VEC> struct Elems {   // VEC: 16-byte chunks; else single elements (any head_dim / alignment)
+  static constexpr int N = VEC ? Chunk<T>::N : 1;
+  static constexpr int MAXC = VEC ? 4 : 16;      // chunks per lane: head_dim <= 256 over 16 lanes
+  static __device__ __forceinline__ void load(const T* p, float (&v)[N]) {
+    if constexpr (VEC) Chunk<T>::load(p, v);
+    else v[0] = to_f32(p[0]);
+  }
+  static __device__ __forceinline__ void store(T* p, const float (&v)[N]) {
+    if constexpr (VEC) Chunk<T>::store(p, v);
+    else p[0] = from_f32<T>(v[0]);
+  }
+};
+
+struct StepShape {
+  int heads, seq_kv, head_dim;
+  int64_t q_sb, q_sh, kv_sb, kv_sh, kv_ss;
+};
+
+__device__ __forceinline__ float sum16(float v) {          // over the 16 lanes that share a key
+  v += __shfl_xor(v, 1, kWave);
+  v += __shfl_xor(v, 2, kWave);
+  v += __shfl_xor(v, 4, kWave);
+  v += __shfl_xor(v, 8, kWave);
+  return v;
+}
+
+// Block-wide reductions through a 4-float LDS scratch.
+__device__ __forceinline__ float block_max(float v, float* scratch) {
+  v = wave_max(v);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) scratch[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return fmaxf(fmaxf(scratch[0], scratch[1]), fmaxf(scratch[2], scratch[3]));
+}
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+  v = wave_sum(v);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) scratch[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return scratch[0] + scratch[1] + scratch[2] + scratch[3];
+}
+
+// Sum of per-lane chunk accumulators over the 16 key slots of the block (4 per wavefront:
+// lane bits 4, 5; then the 4 wavefronts through LDS).  Result valid in threads 0..15.
+template <int MAXC, int NE>
+__device__ __forceinline__ void reduce_keys(float (&acc)[MAXC][NE], int nch, float* red /* [4][MAXC][16][NE] */) {
+  static_assert(4 * MAXC * 16 * NE <= kRedFloats, "reduction scratch");
+  const int l16 = threadIdx.x & 15, wave = threadIdx.x >> 6;
+  __syncthreads();
+#pragma unroll
+  for (int c = 0; c < MAXC; c++)
+#pragma unroll
+    for (int e = 0; e < NE; e++) {
+      float v = acc[c][e];
+      v += __shfl_xor(v, 16, kWave);
+      v += __shfl_xor(v, 32, kWave);
+      if ((threadIdx.x & 63) < 16 && c < nch) red[(wave * MAXC + c) * 16 * NE + l16 * NE + e] = v;
+    }
+  __syncthreads();
+  if (threadIdx.x < 16) {
+#pragma unroll
+    for (int c = 0; c < MAXC; c++)
+#pragma unroll
+      for (int e = 0; e < NE; e++) {
+        float v = 0.f;
+        if (c < nch)
+          for (int w = 0; w < 4; w++) v += red[(w * MAXC + c) * 16 * NE + l16 * NE + e];
+        acc[c][e] = v;
+      }
+  }
+}
+
+template <typename T, bool VEC>
+__global__ __launch_bounds__(256) void attn_step_fwd_kernel(const T* __restrict__ q, const T* __restrict__ k,
+                                                            const T* __restrict__ v, float* __restrict__ part, StepShape sh,
+                                                            float scale) {
+  constexpr int NE = Elems<T, VEC>::N, MAXC = Elems<T, VEC>::MAXC;
+  __shared__ float scores[kKeysPerBlock];
+  __shared__ float scratch[4];
+  __shared__ float red[kRedFloats];
+  const int bh = blockIdx.y, b = bh / sh.heads, h = bh % sh.heads;
+  const int s0 = blockIdx.x * kKeysPerBlock;
+  const int s1 = s0 + kKeysPerBlock < sh.seq_kv ? s0 + kKeysPerBlock : sh.seq_kv;
+  const int l16 = threadIdx.x & 15, slot = threadIdx.x >> 4;       // 16 key slots per block
+  const int nchunks = sh.head_dim / NE;                            // chunks per row
+  const int nch = (nchunks - l16 + 15) / 16;                       // chunks of this lane: l16, l16 + 16, ...
+  const T* qrow = q + b * sh.q_sb + h * sh.q_sh;
+  const T* kbase = k + b * sh.kv_sb + h * sh.kv_sh;
+  const T* vbase = v + b * sh.kv_sb + h * sh.kv_sh;
+
+  float qf[MAXC][NE];
+#pragma unroll
+  for (int c = 0; c < MAXC; c++)
+    if (c < nch) Elems<T, VEC>::load(qrow + (l16 + 16 * c) * NE, qf[c]);
+
+  float mx = -INFINITY;
+  for (int sb = s0 + slot; sb < s1; sb += 16 * kUnroll) {
+    float dot[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; u++) {
+      const int s = sb + 16 * u;
+      dot[u] = 0.f;
+      if (s < s1) {
+        const T* krow = kbase + (int64_t)s * sh.kv_ss;
+#pragma unroll
+        for (int c = 0; c < MAXC; c++)
+          if (c < nch) {
+            float kf[NE];
+            Elems<T, VEC>::load(krow + (l16 + 16 * c) * NE, kf);
+#pragma unroll
+            for (int e = 0; e < NE; e++) dot[u] = fmaf(qf[c][e], kf[e], dot[u]);
+          }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; u++) {
+      const int s = sb + 16 * u;
+      const float d = sum16(dot[u]) * scale;
+      if (s < s1) {
+        if (l16 == 0) scores[s - s0] = d;
+        mx = fmaxf(mx, d);
+      }
+    }
+  }
+  mx = block_max(mx, scratch);
+  float sum = 0.f;
+  for (int s = threadIdx.x; s < s1 - s0; s += 256) {
+    const float p = __expf(scores[s] - mx);
+    scores[s] = p;
+    sum += p;
+  }
+  sum = block_sum(sum, scratch);                          // also orders the writes of p before the reads below
+
+  float acc[MAXC][NE];
+#pragma unroll
+  for (int c = 0; c < MAXC; c++)
+#pragma unroll
+    for (int e = 0; e < NE; e++) acc[c][e] = 0.f;
+  for (int sb = s0 + slot; sb < s1; sb += 16 * kUnroll) {
+    float vf[kUnroll][MAXC][NE];
+#pragma unroll
+    for (int u = 0; u < kUnroll; u++) {
+      const int s = sb + 16 * u;
+      if (s < s1) {
+        const T* vrow = vbase + (int64_t)s * sh.kv_ss;
+#pragma unroll
+        for (int c = 0; c < MAXC; c++)
+          if (c < nch) Elems<T, VEC>::load(vrow + (l16 + 16 * c) * NE, vf[u][c]);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; u++) {
+      const int s = sb + 16 * u;
+      if (s < s1) {
+        const float p = scores[s - s0];
+#pragma unroll
+        for (int c = 0; c < MAXC; c++)
+          if (c < nch) {
+#pragma unroll
+            for (int e = 0; e < NE; e++) acc[c][e] = fmaf(p, vf[u][c][e], acc[c][e]);
+          }
+      }
+    }
+  }
+  reduce_keys<MAXC, NE>(acc, nch, red);
+  if (threadIdx.x < 16) {
+    // partial of this block: [head_dim] unnormalised output, then max and sum
+    float* out = part + ((int64_t)bh * gridDim.x + blockIdx.x) * (sh.head_dim + 2);
+#pragma unroll
+    for (int c = 0; c < MAXC; c++)
+      if (c < nch) {
+#pragma unroll
+        for (int e = 0; e < NE; e++) out[(l16 + 16 * c) * NE + e] = acc[c][e];
+      }
+    if (threadIdx.x == 0) {
+      out[sh.head_dim] = mx;
+      out[sh.head_dim + 1] = sum;
+    }
+  }
+}
+
+// o = sum_i w_i o_i / sum_i w_i l_i with w_i = exp(m_i - max m); lse = max m + log(sum).
+template <typename T>
+__global__ __launch_bounds__(64) void attn_step_combine_kernel(const float* __restrict__ part, T* __restrict__ o,
+                                                               float* __restrict__ lse, StepShape sh, int nsplit) {
+  const int bh = blockIdx.x, b = bh / sh.heads, h = bh % sh.heads;
+  const float* p0 = part + (int64_t)bh * nsplit * (sh.head_dim + 2);
+  float mx = -INFINITY;
+  for (int i = 0; i < nsplit; i++) mx = fmaxf(mx, p0[i * (sh.head_dim + 2) + sh.head_dim]);
+  float l = 0.f;
+  for (int i = 0; i < nsplit; i++) l += p0[i * (sh.head_dim + 2) + sh.head_dim + 1] * __expf(p0[i * (sh.head_dim + 2) + sh.head_dim] - mx);
+  const float inv = 1.0f / l;
+  T* orow = o + b * sh.q_sb + h * sh.q_sh;
+  for (int e = threadIdx.x; e < sh.head_dim; e += 64) {
+    float acc = 0.f;
+    for (int i = 0; i < nsplit; i++) acc += p0[i * (sh.head_dim + 2) + e] * __expf(p0[i * (sh.head_dim + 2) + sh.head_dim] - mx);
+    orow[e] = from_f32<T>(acc * inv);
+  }
+  if (threadIdx.x == 0) lse[bh] = mx + __logf(l);
+}
+
+// dV_s = p_s dO; dP_s = dO . V_s; dS_s = p_s (dP_s - dO . O); dQ = scale sum_s dS_s K_s;
+// dK_s = scale dS_s Q.  p is recomputed from lse; one pass over the keys of the block.
+template <typename T, bool VEC>
+__global__ __launch_bounds__(256) void attn_step_bwd_kernel(const T* __restrict__ q, const T* __restrict__ k,
+                                                            const T* __restrict__ v, const T* __restrict__ o,
+                                                            const float* __restrict__ lse, const T* __restrict__ d_o,
+                                                            float* __restrict__ part, T* __restrict__ dk, T* __restrict__ dv,
+                                                            StepShape sh, float scale) {
+  constexpr int NE = Elems<T, VEC>::N, MAXC = Elems<T, VEC>::MAXC;
+  __shared__ float red[kRedFloats];
+  const int bh = blockIdx.y, b = bh / sh.heads, h = bh % sh.heads;
+  const int s0 = blockIdx.x * kKeysPerBlock;
+  const int s1 = s0 + kKeysPerBlock < sh.seq_kv ? s0 + kKeysPerBlock : sh.seq_kv;
+  const int l16 = threadIdx.x & 15, slot = threadIdx.x >> 4;
+  const int nchunks = sh.head_dim / NE;
+  const int nch = (nchunks - l16 + 15) / 16;
+  const int64_t qoff = b * sh.q_sb + h * sh.q_sh, kvoff = b * sh.kv_sb + h * sh.kv_sh;
+  const float L = lse[bh];
+
+  float qf[MAXC][NE], dof[MAXC][NE];
+  float delta = 0.f;
+#pragma unroll
+  for (int c = 0; c < MAXC; c++)
+    if (c < nch) {
+      float of[NE];
+      Elems<T, VEC>::load(q + qoff + (l16 + 16 * c) * NE, qf[c]);
+      Elems<T, VEC>::load(d_o + qoff + (l16 + 16 * c) * NE, dof[c]);
+      Elems<T, VEC>::load(o + qoff + (l16 + 16 * c) * NE, of);
+#pragma unroll
+      for (int e = 0; e < NE; e++) delta = fmaf(dof[c][e], of[e], delta);
+    }
+  delta = sum16(delta);
+
+  float acc[MAXC][NE];
+#pragma unroll
+  for (int c = 0; c < MAXC; c++)
+#pragma unroll
+    for (int e = 0; e < NE; e++) acc[c][e] = 0.f;
+  for (int sb = s0 + slot; sb < s1; sb += 16 * 2) {
+    float kf[2][MAXC][NE], vf[2][MAXC][NE];
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+      const int s = sb + 16 * u;
+      if (s < s1) {
+#pragma unroll
+        for (int c = 0; c < MAXC; c++)
+          if (c < nch) {
+            Elems<T, VEC>::load(k + kvoff + (int64_t)s * sh.kv_ss + (l16 + 16 * c) * NE, kf[u][c]);
+            Elems<T, VEC>::load(v + kvoff + (int64_t)s * sh.kv_ss + (l16 + 16 * c) * NE, vf[u][c]);
+          }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+      const int s = sb + 16 * u;
+      float dot = 0.f, dp = 0.f;
+      if (s < s1) {
+#pragma unroll
+        for (int c = 0; c < MAXC; c++)
+          if (c < nch) {
+#pragma unroll
+            for (int e = 0; e < NE; e++) {
+              dot = fmaf(qf[c][e], kf[u][c][e], dot);
+              dp = fmaf(dof[c][e], vf[u][c][e], dp);
+            }
+          }
+      }
+      dot = sum16(dot);
+      dp = sum16(dp);
+      if (s < s1) {
+        const float p = __expf(dot * scale - L);
+        const float ds = p * (dp - delta) * scale;
+        T* dkrow = dk + kvoff + (int64_t)s * sh.kv_ss;
+        T* dvrow = dv + kvoff + (int64_t)s * sh.kv_ss;
+#pragma unroll
+        for (int c = 0; c < MAXC; c++)
+          if (c < nch) {
+            float t[NE];
+#pragma unroll
+            for (int e = 0; e < NE; e++) acc[c][e] = fmaf(ds, kf[u][c][e], acc[c][e]);
+#pragma unroll
+            for (int e = 0; e < NE; e++) t[e] = ds * qf[c][e];
+            Elems<T, VEC>::store(dkrow + (l16 + 16 * c) * NE, t);
+#pragma unroll
+            for (int e = 0; e < NE; e++) t[e] = p * dof[c][e];
+            Elems<T, VEC>::store(dvrow + (l16 + 16 * c) * NE, t);
+          }
+      }
+    }
+  }
+  reduce_keys<MAXC, NE>(acc, nch, red);
+  if (threadIdx.x < 16) {
+    float* out = part + ((int64_t)bh * gridDim.x + blockIdx.x) * (sh.head_dim + 2);
+#pragma unroll
+    for (int c = 0; c < MAXC; c++)
+      if (c < nch) {
+#pragma unroll
+        for (int e = 0; e < NE; e++) out[(l16 + 16 * c) * NE + e] = acc[c][e];
+      }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(64) void attn_step_dq_kernel(const float* __restrict__ part, T* __restrict__ dq, StepShape sh,
+                                                          int nsplit) {
+  const int bh = blockIdx.x, b = bh / sh.heads, h = bh % sh.heads;
+  const float* p0 = part + (int64_t)bh * nsplit * (sh.head_dim + 2);
+  T* row = dq + b * sh.q_sb + h * sh.q_sh;
+  for (int e = threadIdx.x; e < sh.head_dim; e += 64) {
+    float acc = 0.f;
+    for (int i = 0; i < nsplit; i++) acc += p0[i * (sh.head_dim + 2) + e];
+    row[e] = from_f32<T>(acc);
+  }
+}
+
+bool al16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+int check_step(const char* name, int64_t batch, int64_t heads, int64_t seq_kv, int64_t head_dim, int64_t q_sb, int64_t q_sh,
+               int64_t kv_sb, int64_t kv_sh, int64_t kv_ss, int dtype) {
+  EMI_REQUIRE(batch >= 0 && heads > 0 && seq_kv > 0 && head_dim > 0, "%s: bad shape [%lld,%lld,%lld,%lld]", name, (long long)batch,
+              (long long)heads, (long long)seq_kv, (long long)head_dim);
+  EMI_REQUIRE(dtype == EMI_F32 || dtype == EMI_BF16, "%s: unsupported dtype code %d (want 11=f32 or 16=bf16)", name, dtype);
+  EMI_REQUIRE(head_dim <= 256, "%s: head_dim %lld > 256 is not supported", name, (long long)head_dim);
+  EMI_REQUIRE(q_sh >= head_dim && q_sb > 0 && kv_ss >= head_dim && kv_sh > 0 && kv_sb > 0, "%s: bad strides", name);
+  EMI_REQUIRE(batch * heads <= 65535 && seq_kv <= 0x7fffffff / 2, "%s: batch*heads or seq_kv too large", name);
+  return EMI_OK;
+}
+
+}  // namespace
+}  // namespace emi
+
+using namespace emi;
+
+extern "C" size_t emi_attn_step_workspace_bytes(int64_t batch, int64_t heads, int64_t seq_kv, int64_t head_dim) {
+  if (batch <= 0 || heads <= 0 || seq_kv <= 0 || head_dim <= 0) return 0;
+  const int64_t nsplit = (seq_kv + kKeysPerBlock - 1) / kKeysPerBlock;
+  return (size_t)(batch * heads * nsplit * (head_dim + 2)) * sizeof(float);
+}
+
+extern "C" int emi_attn_step_fwd(emi_stream_t stream, const void* q, const void* k, const void* v, void* o, float* lse,
+                                 void* workspace, size_t workspace_bytes, int64_t batch, int64_t heads, int64_t seq_kv,
+                                 int64_t head_dim, int64_t q_stride_b, int64_t q_stride_h, int64_t kv_stride_b,
+                                 int64_t kv_stride_h, int64_t kv_stride_s, float scale, int dtype) {
+  if (int rc = check_step("emi_attn_step_fwd", batch, heads, seq_kv, head_dim, q_stride_b, q_stride_h, kv_stride_b, kv_stride_h,
+                          kv_stride_s, dtype))
+    return rc;
+  if (batch == 0) return EMI_OK;
+  EMI_REQUIRE(q && k && v && o && lse, "emi_attn_step_fwd: null buffer");
+  const size_t need = emi_attn_step_workspace_bytes(batch, heads, seq_kv, head_dim);
+  EMI_REQUIRE(workspace != nullptr && workspace_bytes >= need, "emi_attn_step_fwd: workspace of %zu bytes needed, got %zu", need,
+              workspace_bytes);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const StepShape sh{(int)heads, (int)seq_kv, (int)head_dim, q_stride_b, q_stride_h, kv_stride_b, kv_stride_h, kv_stride_s};
+  const int ne = dtype == EMI_BF16 ? 8 : 4;
+  const bool vec = head_dim % ne == 0 && q_stride_b % ne == 0 && q_stride_h % ne == 0 && kv_stride_b % ne == 0 &&
+                   kv_stride_h % ne == 0 && kv_stride_s % ne == 0 && al16(q) && al16(k) && al16(v);
+  const int nsplit = (int)((seq_kv + kKeysPerBlock - 1) / kKeysPerBlock);
+  const dim3 grid((unsigned)nsplit, (unsigned)(batch * heads));
+  float* part = static_cast<float*>(workspace);
+#define EMI_STEP_FWD(T, VEC)                                                                                             \
+  do {                                                                                                                   \
+    hipLaunchKernelGGL((attn_step_fwd_kernel<T, VEC>), grid, dim3(256), 0, st, (const T*)q, (const T*)k, (const T*)v,    \
+                       part, sh, scale);                                                                                 \
+    EMI_CHECK_LAUNCH("emi_attn_step_fwd");                                                                               \
+    hipLaunchKernelGGL(attn_step_combine_kernel<T>, dim3((unsigned)(batch * heads)), dim3(64), 0, st, part, (T*)o, lse,  \
+                       sh, nsplit);                                                                                      \
+  } while (0)
+  if (dtype == EMI_BF16) {
+    if (vec) EMI_STEP_FWD(bf16, true);
+    else EMI_STEP_FWD(bf16, false);
+  } else {
+    if (vec) EMI_STEP_FWD(float, true);
+    else EMI_STEP_FWD(float, false);
+  }
+#undef EMI_STEP_FWD
+  EMI_CHECK_LAUNCH("emi_attn_step_fwd(combine)");
+  return EMI_OK;
+}
+
+extern "C" int emi_attn_step_bwd(emi_stream_t stream, const void* q, const void* k, const void* v, const void* o,
+                                 const float* lse, const void* d_o, void* dq, void* dk, void* dv, void* workspace,
+                                 size_t workspace_bytes, int64_t batch, int64_t heads, int64_t seq_kv, int64_t head_dim,
+                                 int64_t q_stride_b, int64_t q_stride_h, int64_t kv_stride_b, int64_t kv_stride_h,
+                                 int64_t kv_stride_s, float scale, int dtype) {
+  if (int rc = check_step("emi_attn_step_bwd", batch, heads, seq_kv, head_dim, q_stride_b, q_stride_h, kv_stride_b, kv_stride_h,
+                          kv_stride_s, dtype))
+    return rc;
+  if (batch == 0) return EMI_OK;
+  EMI_REQUIRE(q && k && v && o && lse && d_o && dq && dk && dv, "emi_attn_step_bwd: null buffer");
+  const size_t need = emi_attn_step_workspace_bytes(batch, heads, seq_kv, head_dim);
+  EMI_REQUIRE(workspace != nullptr && workspace_bytes >= need, "emi_attn_step_bwd: workspace of %zu bytes needed, got %zu", need,
+              workspace_bytes);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const StepShape sh{(int)heads, (int)seq_kv, (int)head_dim, q_stride_b, q_stride_h, kv_stride_b, kv_stride_h, kv_stride_s};
+  const int ne = dtype == EMI_BF16 ? 8 : 4;
+  const bool vec = head_dim % ne == 0 && q_stride_b % ne == 0 && q_stride_h % ne == 0 && kv_stride_b % ne == 0 &&
+                   kv_stride_h % ne == 0 && kv_stride_s % ne == 0 && al16(q) && al16(k) && al16(v) && al16(o) && al16(d_o) &&
+                   al16(dk) && al16(dv);
+  const int nsplit = (int)((seq_kv + kKeysPerBlock - 1) / kKeysPerBlock);
+  const dim3 grid((unsigned)nsplit, (unsigned)(batch * heads));
+  float* part = static_cast<float*>(workspace);
+#define EMI_STEP_BWD(T, VEC)                                                                                             \
+  do {                                                                                                                   \
+    hipLaunchKernelGGL((attn_step_bwd_kernel<T, VEC>), grid, dim3(256), 0, st, (const T*)q, (const T*)k, (const T*)v,    \
+                       (const T*)o, lse, (const T*)d_o, part, (T*)dk, (T*)dv, sh, scale);                                \
+    EMI_CHECK_LAUNCH("emi_attn_step_bwd");                                                                               \
+    hipLaunchKernelGGL(attn_step_dq_kernel<T>, dim3((unsigned)(batch * heads)), dim3(64), 0, st, part, (T*)dq, sh,       \
+                       nsplit);                                                                                          \
+  } while (0)
+  if (dtype == EMI_BF16) {
+    if (vec) EMI_STEP_BWD(bf16, true);
+    else EMI_STEP_BWD(bf16, false);
+  } else {
+    if (vec) EMI_STEP_BWD(float, true);
+    else EMI_STEP_BWD(float, false);
+  }
+#undef EMI_STEP_BWD
+  EMI_CHECK_LAUNCH("emi_attn_step_bwd(dq)");
+  return EMI_OK;
+}

@@ -336,6 +336,64 @@ extern "C" XLA_FFI_Error* emi_attn_bwd_ffi(XLA_FFI_CallFrame* cf) {
                                     (float)scale, (int)causal, q->dtype));
 }
 
+namespace {
+// q / o / dO / dq: [B, h, d]; caches and their cotangents: [B, S, h, d] (rows of one token contiguous).
+struct StepDims {
+  int64_t B, H, S, D;
+};
+bool step_dims(const XLA_FFI_Buffer* q, const XLA_FFI_Buffer* kc, StepDims* d) {
+  if (q->rank != 3 || kc->rank != 4) return false;
+  d->B = q->dims[0]; d->H = q->dims[1]; d->D = q->dims[2]; d->S = kc->dims[1];
+  return kc->dims[0] == d->B && kc->dims[2] == d->H && kc->dims[3] == d->D;
+}
+}  // namespace
+
+extern "C" XLA_FFI_Error* emi_attn_step_fwd_ffi(XLA_FFI_CallFrame* cf) {
+  EMI_FFI_BEGIN("emi_attn_step_fwd", 3, 3, 3, 3)
+  const XLA_FFI_Buffer *q = f.arg(0), *k = f.arg(1), *v = f.arg(2), *o = f.ret(0), *lse = f.ret(1), *ws = f.ret(2);
+  if (!is_float(q) || k->dtype != q->dtype || v->dtype != q->dtype || o->dtype != q->dtype)
+    return f.invalid("q, k, v, o must share one dtype, f32 or bf16 (code %lld)", q->dtype);
+  double scale;
+  if (!f.get_f("scale", &scale)) return f.invalid("missing f32/f64 attribute 'scale'");
+  StepDims d;
+  if (!step_dims(q, k, &d) || !same_shape(k, v) || !same_shape(q, o))
+    return f.invalid("q, o must be [batch, heads, head_dim] and k, v [batch, seq_kv, heads, head_dim] (q rank %lld)", q->rank);
+  if (lse->dtype != XLA_FFI_DataType_F32 || lse->rank != 2 || lse->dims[0] != d.B || lse->dims[1] != d.H)
+    return f.invalid("lse must be f32[batch, heads] = [%lld, %lld]", d.B, d.H);
+  const size_t need = emi_attn_step_workspace_bytes(d.B, d.H, d.S, d.D);
+  if (byte_size(ws) < need) return f.invalid("workspace result has %lld bytes, %lld needed", (long long)byte_size(ws), (long long)need);
+  EMI_FFI_STREAM()
+  return f.from_status(emi_attn_step_fwd(stream, q->data, k->data, v->data, o->data, static_cast<float*>(lse->data), ws->data,
+                                         byte_size(ws), d.B, d.H, d.S, d.D, d.H * d.D, d.D, d.S * d.H * d.D, d.D, d.H * d.D,
+                                         (float)scale, q->dtype));
+}
+
+extern "C" XLA_FFI_Error* emi_attn_step_bwd_ffi(XLA_FFI_CallFrame* cf) {
+  EMI_FFI_BEGIN("emi_attn_step_bwd", 6, 6, 4, 4)
+  const XLA_FFI_Buffer *q = f.arg(0), *k = f.arg(1), *v = f.arg(2), *o = f.arg(3), *lse = f.arg(4), *d_o = f.arg(5);
+  const XLA_FFI_Buffer *dq = f.ret(0), *dk = f.ret(1), *dv = f.ret(2), *ws = f.ret(3);
+  if (!is_float(q)) return f.invalid("q must be f32 or bf16 (code %lld)", q->dtype);
+  const XLA_FFI_Buffer* qlike[] = {o, d_o, dq};
+  const XLA_FFI_Buffer* klike[] = {v, dk, dv};
+  for (const XLA_FFI_Buffer* b : qlike)
+    if (b->dtype != q->dtype || !same_shape(q, b)) return f.invalid("q, o, do, dq must share dtype and shape");
+  for (const XLA_FFI_Buffer* b : klike)
+    if (b->dtype != q->dtype || !same_shape(k, b)) return f.invalid("k, v, dk, dv must share dtype and shape");
+  double scale;
+  if (!f.get_f("scale", &scale)) return f.invalid("missing f32/f64 attribute 'scale'");
+  StepDims d;
+  if (k->dtype != q->dtype || !step_dims(q, k, &d))
+    return f.invalid("q must be [batch, heads, head_dim] and k [batch, seq_kv, heads, head_dim] (q rank %lld)", q->rank);
+  if (lse->dtype != XLA_FFI_DataType_F32 || lse->rank != 2 || lse->dims[0] != d.B || lse->dims[1] != d.H)
+    return f.invalid("lse must be f32[batch, heads] = [%lld, %lld]", d.B, d.H);
+  const size_t need = emi_attn_step_workspace_bytes(d.B, d.H, d.S, d.D);
+  if (byte_size(ws) < need) return f.invalid("workspace result has %lld bytes, %lld needed", (long long)byte_size(ws), (long long)need);
+  EMI_FFI_STREAM()
+  return f.from_status(emi_attn_step_bwd(stream, q->data, k->data, v->data, o->data, static_cast<const float*>(lse->data),
+                                         d_o->data, dq->data, dk->data, dv->data, ws->data, byte_size(ws), d.B, d.H, d.S, d.D,
+                                         d.H * d.D, d.D, d.S * d.H * d.D, d.D, d.H * d.D, (float)scale, q->dtype));
+}
+
 extern "C" XLA_FFI_Error* emi_embedding_fwd_ffi(XLA_FFI_CallFrame* cf) {
   EMI_FFI_BEGIN("emi_embedding_fwd", 2, 2, 1, 1)
   const XLA_FFI_Buffer *tok = f.arg(0), *tab = f.arg(1), *x = f.ret(0);
@@ -375,6 +433,7 @@ const Target kTargets[] = {
     {"emi_swiglu_fwd", emi_swiglu_fwd_ffi},   {"emi_swiglu_bwd", emi_swiglu_bwd_ffi},
     {"emi_add", emi_add_ffi},                 {"emi_gemm", emi_gemm_ffi},
     {"emi_attn_fwd", emi_attn_fwd_ffi},       {"emi_attn_bwd", emi_attn_bwd_ffi},
+    {"emi_attn_step_fwd", emi_attn_step_fwd_ffi}, {"emi_attn_step_bwd", emi_attn_step_bwd_ffi},
     {"emi_embedding_fwd", emi_embedding_fwd_ffi}, {"emi_embedding_bwd", emi_embedding_bwd_ffi},
 };
 constexpr int kNumTargets = sizeof(kTargets) / sizeof(kTargets[0]);

@@ -950,6 +950,10 @@ static int launch_generic(hipStream_t st, const void* A, const void* B, const vo
   return EMI_OK;
 }
 
+// gemm_skinny.hip
+int launch_skinny(hipStream_t st, const void* A, const void* B, const void* R, void* C, int64_t M, int64_t N, int64_t K,
+                  int64_t lda, int64_t ldb, int64_t ldr, int64_t ldc, int trans_a, int trans_b, int dtype);
+
 }  // namespace emi
 
 using namespace emi;
@@ -968,6 +972,11 @@ extern "C" int emi_gemm(emi_stream_t stream, const void* A, const void* B, const
               "emi_gemm: leading dimension smaller than the row length (lda=%lld ldb=%lld ldr=%lld ldc=%lld)",
               (long long)lda, (long long)ldb, (long long)ldr, (long long)ldc);
   hipStream_t st = static_cast<hipStream_t>(stream);
+  if (K > 0 && (R == nullptr || ldr >= N)) {
+    // single-token forms (mat-vec and its adjoints): weight-bandwidth-bound kernels
+    const int rc = launch_skinny(st, A, B, R, C, M, N, K, lda, ldb, ldr, ldc, trans_a, trans_b, dtype);
+    if (rc >= 0) return rc;
+  }
   if (dtype == EMI_BF16) {
     const int64_t a_rows = trans_a ? K : M, b_rows = trans_b ? N : K;
     const int64_t a_bytes = ((a_rows - 1) * lda + (trans_a ? M : K)) * 2;

@@ -1,0 +1,205 @@
+// Skinny GEMMs of the single-token (decode) form of the llama step, all HBM-bound on
+// the weight matrix, which is read (or written) exactly once:
+//   mat-vec        y = W x            test/llama.py:149-157,211,224-233  (NT, M <= 8)
+//   its adjoints   dx = dy W          HLODerivatives.td:1166-1170        (NN, M <= 8)
+//                  dW = dy^T x                                           (TN, K <= 8)
+// emi_gemm routes here when the token dimension is at most 8; fp32 accumulation,
+// one rounding, optional residual like the large kernels.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "emi_device.h"
+
+namespace emi {
+namespace {
+
+// y[m][n] = sum_k A[m][k] B[n][k] (+ R[m][n]); one wavefront per row n of B, which streams
+// through in 16-byte chunks (four in flight per lane); A (M x K, a few KB) comes from cache.
+template <typename T, int MT>
+__global__ __launch_bounds__(256) void gemv_nt_kernel(const T* __restrict__ A, const T* __restrict__ B, const T* R, T* C, int M,
+                                                      int N, int K, int64_t lda, int64_t ldb, int64_t ldr, int64_t ldc) {
+  constexpr int V = Chunk<T>::N;
+  const int lane = threadIdx.x & 63;
+  const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (n >= N) return;
+  const T* brow = B + (int64_t)n * ldb;
+  float acc[MT];
+#pragma unroll
+  for (int m = 0; m < MT; m++) acc[m] = 0.f;
+  for (int k0 = lane * V; k0 < K; k0 += 64 * V * 4) {
+    float b[4][V];
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+      const int k = k0 + u * 64 * V;
+      if (k < K) Chunk<T>::load(brow + k, b[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+      const int k = k0 + u * 64 * V;
+      if (k < K) {
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+          if (m < M) {
+            float a[V];
+            Chunk<T>::load(A + (int64_t)m * lda + k, a);
+#pragma unroll
+            for (int e = 0; e < V; e++) acc[m] = fmaf(a[e], b[u][e], acc[m]);
+          }
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int m = 0; m < MT; m++) acc[m] = wave_sum(acc[m]);
+  if (lane == 0) {
+#pragma unroll
+    for (int m = 0; m < MT; m++)
+      if (m < M) {
+        float v = acc[m];
+        if (R != nullptr) v += to_f32(R[(int64_t)m * ldr + n]);
+        C[(int64_t)m * ldc + n] = from_f32<T>(v);
+      }
+  }
+}
+
+// y[m][n] = sum_k A[m][k] B[k][n] (+ R): a block owns 8 chunks = 128 bytes of every row of B
+// (8 lanes side by side) and its 128 row-lanes walk down the K rows with UN loads in flight
+// each (a block must keep tens of KB in flight: there are only N / 64 of them); the partial
+// sums meet through lane shuffles and LDS.  No atomics: the result does not depend on the
+// launch.
+template <typename T, int MT>
+__global__ __launch_bounds__(1024) void gemv_nn_kernel(const T* __restrict__ A, const T* __restrict__ B, const T* R, T* C, int M,
+                                                       int N, int K, int64_t lda, int64_t ldb, int64_t ldr, int64_t ldc) {
+  constexpr int V = Chunk<T>::N, UN = MT * V > 32 ? 4 : 8, ROWS = 128;
+  __shared__ float part[16][MT][8 * V];
+  const int cl = threadIdx.x & 7, rl = threadIdx.x >> 3;           // chunk lane, row lane (0..127)
+  const int n = (blockIdx.x * 8 + cl) * V;
+  float acc[MT][V];
+#pragma unroll
+  for (int m = 0; m < MT; m++)
+#pragma unroll
+    for (int e = 0; e < V; e++) acc[m][e] = 0.f;
+  if (n < N) {
+    for (int k0 = rl; k0 < K; k0 += ROWS * UN) {
+      float b[UN][V];
+#pragma unroll
+      for (int u = 0; u < UN; u++) {
+        const int k = k0 + u * ROWS;
+        if (k < K) Chunk<T>::load(B + (int64_t)k * ldb + n, b[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < UN; u++) {
+        const int k = k0 + u * ROWS;
+        if (k < K) {
+#pragma unroll
+          for (int m = 0; m < MT; m++) {
+            if (m < M) {
+              const float a = to_f32(A[(int64_t)m * lda + k]);
+#pragma unroll
+              for (int e = 0; e < V; e++) acc[m][e] = fmaf(a, b[u][e], acc[m][e]);
+            }
+          }
+        }
+      }
+    }
+  }
+  // the 8 row lanes of a wavefront differ in lane bits 3..5; then the 16 wavefronts meet in LDS
+#pragma unroll
+  for (int m = 0; m < MT; m++)
+#pragma unroll
+    for (int e = 0; e < V; e++) {
+      float v = acc[m][e];
+      v += __shfl_xor(v, 8, kWave);
+      v += __shfl_xor(v, 16, kWave);
+      v += __shfl_xor(v, 32, kWave);
+      if ((threadIdx.x & 63) < 8) part[threadIdx.x >> 6][m][cl * V + e] = v;
+    }
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < MT * 8 * V; idx += 1024) {
+    const int m = idx / (8 * V), c = idx % (8 * V);
+    const int col = blockIdx.x * 8 * V + c;
+    if (m < M && col < N) {
+      float v = 0.f;
+#pragma unroll
+      for (int w = 0; w < 16; w++) v += part[w][m][c];
+      if (R != nullptr) v += to_f32(R[(int64_t)m * ldr + col]);
+      C[(int64_t)m * ldc + col] = from_f32<T>(v);
+    }
+  }
+}
+
+// C[m][n] = sum_{k < K <= 8} A[k][m] B[k][n] (+ R): a sum of K outer products, one 16-byte
+// store per thread; bound by the write of C.
+template <typename T>
+__global__ __launch_bounds__(256) void outer_tn_kernel(const T* __restrict__ A, const T* __restrict__ B, const T* R, T* C, int M,
+                                                       int N, int K, int64_t lda, int64_t ldb, int64_t ldr, int64_t ldc) {
+  constexpr int V = Chunk<T>::N;
+  const int chunks = N / V;
+  const int64_t total = (int64_t)M * chunks;
+  for (int64_t i = blockIdx.x * (int64_t)256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int m = (int)(i / chunks), n = (int)(i % chunks) * V;
+    float acc[V];
+    if (R != nullptr) Chunk<T>::load(R + (int64_t)m * ldr + n, acc);
+    else {
+#pragma unroll
+      for (int e = 0; e < V; e++) acc[e] = 0.f;
+    }
+    for (int k = 0; k < K; k++) {
+      const float a = to_f32(A[(int64_t)k * lda + m]);
+      float b[V];
+      Chunk<T>::load(B + (int64_t)k * ldb + n, b);
+#pragma unroll
+      for (int e = 0; e < V; e++) acc[e] = fmaf(a, b[e], acc[e]);
+    }
+    Chunk<T>::store(C + (int64_t)m * ldc + n, acc);
+  }
+}
+
+bool al16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+template <typename T>
+int launch_skinny_t(hipStream_t st, const void* A_, const void* B_, const void* R_, void* C_, int64_t M, int64_t N, int64_t K,
+                    int64_t lda, int64_t ldb, int64_t ldr, int64_t ldc, int trans_a, int trans_b) {
+  constexpr int V = Chunk<T>::N;
+  const T* A = static_cast<const T*>(A_);
+  const T* B = static_cast<const T*>(B_);
+  const T* R = static_cast<const T*>(R_);
+  T* C = static_cast<T*>(C_);
+#define EMI_SKINNY_MT(KERNEL, GRID, BLOCK)                                                                              \
+  do {                                                                                                                  \
+    if (M <= 1) hipLaunchKernelGGL((KERNEL<T, 1>), GRID, dim3(BLOCK), 0, st, A, B, R, C, (int)M, (int)N, (int)K, lda, ldb, ldr, ldc); \
+    else if (M <= 2) hipLaunchKernelGGL((KERNEL<T, 2>), GRID, dim3(BLOCK), 0, st, A, B, R, C, (int)M, (int)N, (int)K, lda, ldb, ldr, ldc); \
+    else if (M <= 4) hipLaunchKernelGGL((KERNEL<T, 4>), GRID, dim3(BLOCK), 0, st, A, B, R, C, (int)M, (int)N, (int)K, lda, ldb, ldr, ldc); \
+    else hipLaunchKernelGGL((KERNEL<T, 8>), GRID, dim3(BLOCK), 0, st, A, B, R, C, (int)M, (int)N, (int)K, lda, ldb, ldr, ldc); \
+  } while (0)
+  if (!trans_a && trans_b) {                 // mat-vec: 16-byte chunks along K of both operands
+    if (M > 8 || K % V || lda % V || ldb % V || !al16(A) || !al16(B)) return -1;
+    EMI_SKINNY_MT(gemv_nt_kernel, dim3((unsigned)((N + 3) / 4)), 256);
+  } else if (!trans_a && !trans_b) {         // 16-byte chunks along N of B
+    if (M > 8 || N % V || ldb % V || !al16(B)) return -1;
+    EMI_SKINNY_MT(gemv_nn_kernel, dim3((unsigned)((N / V + 7) / 8)), 1024);
+  } else if (trans_a && !trans_b) {          // outer products: 16-byte chunks along N of B, C (and R)
+    if (K > 8 || N % V || ldb % V || ldc % V || !al16(B) || !al16(C) || (R != nullptr && (ldr % V || !al16(R)))) return -1;
+    const int64_t total = M * (N / V);
+    const unsigned grid = (unsigned)((total + 255) / 256 < 16384 ? (total + 255) / 256 : 16384);
+    hipLaunchKernelGGL(outer_tn_kernel<T>, dim3(grid), dim3(256), 0, st, A, B, R, C, (int)M, (int)N, (int)K, lda, ldb, ldr, ldc);
+  } else {
+    return -1;
+  }
+#undef EMI_SKINNY_MT
+  EMI_CHECK_LAUNCH("emi_gemm(skinny)");
+  return EMI_OK;
+}
+
+}  // namespace
+
+// Returns -1 when the shape is not one of the skinny forms (the caller then takes the tiled
+// kernels), otherwise a status code.
+int launch_skinny(hipStream_t st, const void* A, const void* B, const void* R, void* C, int64_t M, int64_t N, int64_t K,
+                  int64_t lda, int64_t ldb, int64_t ldr, int64_t ldc, int trans_a, int trans_b, int dtype) {
+  if (M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff) return -1;
+  if (dtype == EMI_BF16) return launch_skinny_t<bf16>(st, A, B, R, C, M, N, K, lda, ldb, ldr, ldc, trans_a, trans_b);
+  return launch_skinny_t<float>(st, A, B, R, C, M, N, K, lda, ldb, ldr, ldc, trans_a, trans_b);
+}
+
+}  // namespace emi

@@ -45,3 +45,35 @@ def forward(x, config, weights, logits=False, eps=1e-5, theta=10000.0):
     if logits:
         x = ops.matmul_nt(x, weights["wcls"])
     return x
+
+
+def forward_step(x, config, weights, key_cache, value_cache, eps=1e-5, theta=10000.0):
+    """The reference's own single-token form, argument for argument
+    (test/llama.py:35-238): x is the residual stream of one token [dim];
+    key_cache / value_cache are [n_layers, pos, kv_dim] and the token sits at
+    position pos = key_cache.shape[1].  Returns the final RMSNorm of the residual
+    stream.  Every projection is a mat-vec (weight-bandwidth-bound kernels)."""
+    n_layers, n_heads = config["n_layers"], config["n_heads"]
+    if config.get("n_kv_heads", n_heads) != n_heads:
+        # the reference reshapes k with `dim`, not `kv_dim` (:162,171): it only runs with equal head counts
+        raise ValueError("forward_step: n_kv_heads must equal n_heads")
+    dim = x.shape[-1]
+    pos = key_cache.shape[1]
+    for i in range(n_layers):
+        lw = {k: ops.select(weights[k], i) for k in LAYER_KEYS}
+        xb = ops.rmsnorm(x, lw["rms_att_weight"], eps)                                    # :145
+        q = ops.matmul_nt(xb, lw["wq"])                                                   # :149-157
+        k = ops.matmul_nt(xb, lw["wk"])
+        v = ops.matmul_nt(xb, lw["wv"])
+        q = ops.reshape(ops.rope(ops.reshape(q, (1, 1, dim)), n_heads, theta, pos0=pos), (dim,))   # :161-168
+        k = ops.reshape(ops.rope(ops.reshape(k, (1, 1, dim)), n_heads, theta, pos0=pos), (dim,))
+        key_cache_l = ops.append_row(ops.select(key_cache, i), k)                         # :170-175
+        value_cache_l = ops.append_row(ops.select(value_cache, i), v)
+        att = ops.attention_step(q, key_cache_l, value_cache_l, n_heads)                  # :178-209
+        x = ops.matmul_nt(att, lw["wo"], residual=x)                                      # :211-215
+        xb = ops.rmsnorm(x, lw["rms_ffn_weight"], eps)                                    # :219
+        h1 = ops.matmul_nt(xb, lw["w1"])                                                  # :224-225
+        h3 = ops.matmul_nt(xb, lw["w3"])
+        g = ops.swiglu(h1, h3)                                                            # :227-229
+        x = ops.matmul_nt(g, lw["w2"], residual=x)                                        # :231-233
+    return ops.rmsnorm(x, weights["rms_final_weight"], eps)                               # :235

@@ -29,6 +29,7 @@ FFI_TARGETS = {
     "matmul_nt": ("emi_gemm", ("emi_gemm", "emi_gemm")),         # dX (NN) and dW (TN)
     "swiglu":    ("emi_swiglu_fwd", ("emi_swiglu_bwd",)),
     "attention": ("emi_attn_fwd", ("emi_attn_bwd",)),
+    "attention_step": ("emi_attn_step_fwd", ("emi_attn_step_bwd",)),
     "add":       ("emi_add", ()),
     "embedding": ("emi_embedding_fwd", ("emi_embedding_bwd",)),
 }
@@ -334,6 +335,65 @@ def attention(q, k, v, n_heads, scale=None, causal=True, layout="bshd"):
         return _accumulate(acc[0], dq), _accumulate(acc[1], dk), _accumulate(acc[2], dv)
 
     Tape.record((q, k, v), o, rule)
+    return o
+
+
+def reshape(x, shape):
+    """x viewed with another shape (Reshape rule, HLODerivatives.td:1271: the cotangent is
+    reshaped back)."""
+    y = x.reshape(shape)
+    Tape.record((x,), y, lambda c, acc: (_accumulate(acc[0], c.reshape(x.shape)),))
+    return y
+
+
+def append_row(cache, row):
+    """[cache; row]: the key / value cache of one layer with the current token's row
+    appended (`jnp.append`, test/llama.py:170-175).  Adjoint: the cotangent is sliced
+    (Concatenate rule, StableHLOAutoDiffOpInterfaceImpl.cpp:2015-2059)."""
+    _dev(cache, row)
+    _same_dtype(cache, row)
+    if cache.dim() != 2 or row.shape != (cache.shape[1],):
+        raise ValueError("append_row: cache %s, row %s" % (tuple(cache.shape), tuple(row.shape)))
+    out = torch.cat([cache, row[None, :]], dim=0)          # device-to-device copies
+
+    def rule(c, acc):
+        n = cache.shape[0]
+        return _accumulate(acc[0], c[:n].contiguous()), _accumulate(acc[1], c[n].contiguous())
+
+    Tape.record((cache, row), out, rule)
+    return out
+
+
+def attention_step(q, k_cache, v_cache, n_heads, scale=None):
+    """Attention of one token against its layer's cache (test/llama.py:178-209): q is
+    [n_heads*head_dim], the caches are [seq_kv, n_heads*head_dim] and already hold the
+    token's own row.  Returns the concatenated per-head outputs [n_heads*head_dim]."""
+    _dev(q, k_cache, v_cache)
+    _same_dtype(q, k_cache, v_cache)
+    D = q.shape[-1]
+    if q.dim() != 1 or k_cache.dim() != 2 or k_cache.shape != v_cache.shape or k_cache.shape[1] != D or D % n_heads:
+        raise ValueError("attention_step: q %s, caches %s / %s, %d heads" %
+                         (tuple(q.shape), tuple(k_cache.shape), tuple(v_cache.shape), n_heads))
+    S, d = k_cache.shape[0], D // n_heads
+    if scale is None:
+        scale = 1.0 / math.sqrt(d)
+    k_cache, v_cache = k_cache.contiguous(), v_cache.contiguous()
+    o = torch.empty_like(q)
+    lse = torch.empty((1, n_heads), dtype=torch.float32, device=q.device)
+    strides = (D, d, S * D, d, D)              # q: batch, head; cache: batch, head, row
+    nbytes = N.lib().emi_attn_step_workspace_bytes(1, n_heads, S, d)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
+    N.check(N.lib().emi_attn_step_fwd(_stream(), _p(q), _p(k_cache), _p(v_cache), _p(o), _p(lse), _p(ws), nbytes, 1,
+                                      n_heads, S, d, *strides, float(scale), _code(q)))
+
+    def rule(c, acc):
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k_cache), torch.empty_like(v_cache)
+        N.check(N.lib().emi_attn_step_bwd(_stream(), _p(q), _p(k_cache), _p(v_cache), _p(o), _p(lse), _p(c), _p(dq),
+                                          _p(dk), _p(dv), _p(ws), nbytes, 1, n_heads, S, d, *strides, float(scale),
+                                          _code(q)))
+        return _accumulate(acc[0], dq), _accumulate(acc[1], dk), _accumulate(acc[2], dv)
+
+    Tape.record((q, k_cache, v_cache), o, rule)
     return o
 
 

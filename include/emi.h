@@ -135,6 +135,30 @@ int emi_attn_bwd(emi_stream_t stream, const void* q, const void* k, const void* 
                  int64_t head_dim, int64_t stride_b, int64_t stride_h, int64_t stride_s,
                  float scale, int causal, int dtype);
 
+/* Attention of the single-token step exactly as the reference writes it
+ * (test/llama.py:178-206, softmax :13-18): one query per (batch, head) against
+ * the seq_kv rows of that head's key / value cache (the cache already holds the
+ * row of the current token, :170-175).  Element (b, h, i) of q / o / dO / dq
+ * lives at b*q_stride_b + h*q_stride_h + i; element (b, h, s, i) of k / v / dk /
+ * dv at b*kv_stride_b + h*kv_stride_h + s*kv_stride_s + i.  lse: float[batch,
+ * heads].  The adjoint (rules as for emi_attn_bwd) returns the cotangent of
+ * every cache row.  The keys of a head are split over several blocks whose
+ * partial results meet in `workspace` (emi_attn_step_workspace_bytes, the same
+ * size forward and backward).  Query heads and key/value heads are equal in
+ * number, as in the reference (:162,171). */
+size_t emi_attn_step_workspace_bytes(int64_t batch, int64_t heads, int64_t seq_kv, int64_t head_dim);
+int emi_attn_step_fwd(emi_stream_t stream, const void* q, const void* k, const void* v, void* o,
+                      float* lse, void* workspace, size_t workspace_bytes, int64_t batch,
+                      int64_t heads, int64_t seq_kv, int64_t head_dim, int64_t q_stride_b,
+                      int64_t q_stride_h, int64_t kv_stride_b, int64_t kv_stride_h,
+                      int64_t kv_stride_s, float scale, int dtype);
+int emi_attn_step_bwd(emi_stream_t stream, const void* q, const void* k, const void* v,
+                      const void* o, const float* lse, const void* d_o, void* dq, void* dk,
+                      void* dv, void* workspace, size_t workspace_bytes, int64_t batch,
+                      int64_t heads, int64_t seq_kv, int64_t head_dim, int64_t q_stride_b,
+                      int64_t q_stride_h, int64_t kv_stride_b, int64_t kv_stride_h,
+                      int64_t kv_stride_s, float scale, int dtype);
+
 /* Embedding gather x[t,:] = table[tokens[t],:] and its adjoint (scatter-add of
  * dx rows into a zero-initialised dtable; fp32 accumulation in workspace when
  * dtype is bf16).  The lookup is commented out in the reference

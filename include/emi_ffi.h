@@ -26,6 +26,8 @@
  *  emi_gemm           A[.,.], B[.,.] [, R[M,N]]        C[M,N]                            trans_a:pred, trans_b:pred
  *  emi_attn_fwd       q, k, v  (rank 4)                o, lse f32[B,h,S] [, workspace:u8[n]]  scale:f32, causal:pred, bshd:pred
  *  emi_attn_bwd       q, k, v, o, lse, do              dq, dk, dv, workspace:u8[n]       scale:f32, causal:pred, bshd:pred
+ *  emi_attn_step_fwd  q[B,h,d], k, v [B,S,h,d]         o[B,h,d], lse f32[B,h], workspace:u8[n]  scale:f32
+ *  emi_attn_step_bwd  q, k, v, o, lse, do              dq, dk, dv, workspace:u8[n]       scale:f32
  *  emi_embedding_fwd  tokens s32[..], table[V,D]       x[..,D]                           -
  *  emi_embedding_bwd  tokens s32[..], dx[..,D]         dtable[V,D] [, workspace:u8[n]]   -
  *
@@ -54,6 +56,8 @@ struct XLA_FFI_Error* emi_add_ffi(struct XLA_FFI_CallFrame*);
 struct XLA_FFI_Error* emi_gemm_ffi(struct XLA_FFI_CallFrame*);
 struct XLA_FFI_Error* emi_attn_fwd_ffi(struct XLA_FFI_CallFrame*);
 struct XLA_FFI_Error* emi_attn_bwd_ffi(struct XLA_FFI_CallFrame*);
+struct XLA_FFI_Error* emi_attn_step_fwd_ffi(struct XLA_FFI_CallFrame*);
+struct XLA_FFI_Error* emi_attn_step_bwd_ffi(struct XLA_FFI_CallFrame*);
 struct XLA_FFI_Error* emi_embedding_fwd_ffi(struct XLA_FFI_CallFrame*);
 struct XLA_FFI_Error* emi_embedding_bwd_ffi(struct XLA_FFI_CallFrame*);
 

@@ -431,6 +431,66 @@ def model_bwd(dout, weights, config, fcache, eps=EPS):
 # 5. Seeded synthetic inputs for the benchmark configurations
 # ---------------------------------------------------------------------------
 
+def forward_step_vjp(x, config, weights, key_cache, value_cache, dy, eps=EPS, theta=ROPE_THETA):
+    """Reverse of `forward_step` (the program `jax.vjp` of test/llama.py:35-238 computes):
+    cotangents of x, of every weight and of both caches for the output cotangent dy.
+    Built from the batched closed forms on a one-token batch: the token at position pos
+    attends to the pos cache rows and to its own row, i.e. non-causal attention of one
+    query over pos+1 keys; the appended row's cotangent goes to k / v, the others to the
+    cache (Concatenate rule, StableHLOAutoDiffOpInterfaceImpl.cpp:2015-2059).  Returns
+    (y, dx, dweights, dkey_cache, dvalue_cache); y must equal forward_step's."""
+    n_layers, n_heads, D = config["n_layers"], config["n_heads"], config["dim"]
+    d = D // n_heads
+    pos = key_cache.shape[1]
+    scale = 1.0 / np.sqrt(d)
+    cos, sin = rope_angles(1, d, theta, pos, dtype=np.float64)
+    hd = lambda t: t.reshape(1, -1, n_heads, d).transpose(0, 2, 1, 3)          # [S, D] -> [1, h, S, d]
+    unhd = lambda t: t.transpose(0, 2, 1, 3).reshape(-1, D)                    # back to [S, D]
+    saved = []
+    x = np.asarray(x, dtype=np.float64).reshape(1, 1, D)
+    for i in range(n_layers):
+        lw = _layer_weights(weights, i)
+        xb = rmsnorm_fwd(x, lw["rms_att_weight"], eps)
+        q, k, v = linear_fwd(xb, lw["wq"]), linear_fwd(xb, lw["wk"]), linear_fwd(xb, lw["wv"])
+        qr = rope_fwd(_heads(q, n_heads), cos, sin).reshape(1, D)
+        kr = rope_fwd(_heads(k, n_heads), cos, sin).reshape(1, D)
+        K = np.concatenate([key_cache[i], kr], axis=0)
+        V = np.concatenate([value_cache[i], v.reshape(1, D)], axis=0)
+        o, _ = attention_fwd(hd(qr), hd(K), hd(V), scale, causal=False)
+        att = unhd(o).reshape(1, 1, D)
+        x1 = x + linear_fwd(att, lw["wo"])
+        xb2 = rmsnorm_fwd(x1, lw["rms_ffn_weight"], eps)
+        a1, a3 = linear_fwd(xb2, lw["w1"]), linear_fwd(xb2, lw["w3"])
+        g = swiglu_fwd(a1, a3)
+        saved.append(dict(x=x, xb=xb, qr=qr, K=K, V=V, att=att, x1=x1, xb2=xb2, a1=a1, a3=a3, g=g))
+        x = x1 + linear_fwd(g, lw["w2"])
+    y = rmsnorm_fwd(x, weights["rms_final_weight"], eps)
+
+    gw = {k: np.zeros_like(np.asarray(weights[k], dtype=np.float64)) for k in LAYER_KEYS}
+    dkc, dvc = np.zeros_like(key_cache, dtype=np.float64), np.zeros_like(value_cache, dtype=np.float64)
+    dx, gw["rms_final_weight"] = rmsnorm_bwd(x, weights["rms_final_weight"], np.asarray(dy, dtype=np.float64).reshape(1, 1, D), eps)
+    for i in reversed(range(n_layers)):
+        lw, c = _layer_weights(weights, i), saved[i]
+        dg, gw["w2"][i] = linear_bwd(c["g"], lw["w2"], dx)
+        da1, da3 = swiglu_bwd(c["a1"], c["a3"], dg)
+        dxa, gw["w1"][i] = linear_bwd(c["xb2"], lw["w1"], da1)
+        dxb, gw["w3"][i] = linear_bwd(c["xb2"], lw["w3"], da3)
+        dx1n, gw["rms_ffn_weight"][i] = rmsnorm_bwd(c["x1"], lw["rms_ffn_weight"], dxa + dxb, eps)
+        dx1 = dx + dx1n
+        datt, gw["wo"][i] = linear_bwd(c["att"], lw["wo"], dx1)
+        dq, dK, dV = attention_bwd(hd(c["qr"]), hd(c["K"]), hd(c["V"]), hd(datt.reshape(1, D)), scale, causal=False)
+        dq, dK, dV = unhd(dq), unhd(dK), unhd(dV)
+        dkc[i], dvc[i] = dK[:pos], dV[:pos]
+        dqp = rope_bwd(_heads(dq.reshape(1, 1, D), n_heads), cos, sin).reshape(1, 1, D)
+        dkp = rope_bwd(_heads(dK[pos:].reshape(1, 1, D), n_heads), cos, sin).reshape(1, 1, D)
+        dxq, gw["wq"][i] = linear_bwd(c["xb"], lw["wq"], dqp)
+        dxk, gw["wk"][i] = linear_bwd(c["xb"], lw["wk"], dkp)
+        dxv, gw["wv"][i] = linear_bwd(c["xb"], lw["wv"], dV[pos:].reshape(1, 1, D))
+        dxn, gw["rms_att_weight"][i] = rmsnorm_bwd(c["x"], lw["rms_att_weight"], dxq + dxk + dxv, eps)
+        dx = dx1 + dxn
+    return y.reshape(D), dx.reshape(D), gw, dkc, dvc
+
+
 def make_weights(config, seed, std=0.02, dtype=np.float32, embedding=True, norm_gain="normal"):
     """Weights drawn with numpy Generator(PCG64(seed)) in a fixed key order.
     `norm_gain`: "normal" draws the RMSNorm gains N(0, std) like every other

@@ -93,6 +93,25 @@ def test_ffi_handlers_launch_on_the_frame_stream():
         _call("emi_attn_fwd_ffi", xla, [_buf(xla, q), _buf(xla, k), _buf(xla, v)], [_buf(xla, o), _buf(xla, lse), _buf(xla, ws)], at)
         ro, _ = L.attention_fwd(tr(qr), tr(kr), tr(vr))
         check(tr(host(o)), ro, "bf16", "ffi attention with workspace")
+        # single-token attention over a cache: q [B, h, d], caches [B, S, h, d]
+        B, S, h, d = 2, 700, 3, 64
+        (q, qr), (do, dor) = (dev(rng.standard_normal((B, h, d)), "bf16") for _ in range(2))
+        (kc, kcr), (vc, vcr) = (dev(rng.standard_normal((B, S, h, d)), "bf16") for _ in range(2))
+        o, dq = torch.empty_like(q), torch.empty_like(q)
+        dk, dv = torch.empty_like(kc), torch.empty_like(vc)
+        lse = torch.empty((B, h), dtype=torch.float32, device="cuda")
+        ws = torch.empty(lib.emi_attn_step_workspace_bytes(B, h, S, d), dtype=torch.uint8, device="cuda")
+        at = {"scale": (F.F32, d ** -0.5)}
+        _call("emi_attn_step_fwd_ffi", xla, [_buf(xla, t) for t in (q, kc, vc)], [_buf(xla, t) for t in (o, lse, ws)], at)
+        q4, k4, v4, do4 = qr[:, :, None, :], kcr.transpose(0, 2, 1, 3), vcr.transpose(0, 2, 1, 3), dor[:, :, None, :]
+        ro, _ = L.attention_fwd(q4, k4, v4, causal=False)
+        check(o, ro[:, :, 0, :], "bf16", "ffi step attention")
+        _call("emi_attn_step_bwd_ffi", xla, [_buf(xla, t) for t in (q, kc, vc, o, lse, do)],
+              [_buf(xla, t) for t in (dq, dk, dv, ws)], at)
+        rdq, rdk, rdv = L.attention_bwd(q4, k4, v4, do4, causal=False)
+        check(dq, rdq[:, :, 0, :], "bf16", "ffi step dq")
+        check(dk, rdk.transpose(0, 2, 1, 3), "bf16", "ffi step dk")
+        check(dv, rdv.transpose(0, 2, 1, 3), "bf16", "ffi step dv")
         # swiglu, add, embedding
         a, ar = dev(rng.standard_normal(1000), "f32")
         b, br = dev(rng.standard_normal(1000), "f32")

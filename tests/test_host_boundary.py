@@ -87,6 +87,13 @@ def test_ffi_metadata_probe_and_stages():
      {"scale": (F.F32, 0.1), "causal": (F.PRED, 1)}, "workspace"),
     ("emi_attn_bwd_ffi", [(F.BF16, [1, 2, 64, 128])] * 4 + [(F.F32, [1, 2, 64]), (F.BF16, [1, 2, 64, 128])],
      [(F.BF16, [1, 2, 64, 128])] * 3 + [(F.U8, [8])], {"scale": (F.F32, 0.1)}, "workspace"),
+    ("emi_attn_step_fwd_ffi", [(F.F32, [1, 6, 48]), (F.F32, [1, 9, 6, 48]), (F.F32, [1, 9, 6, 48])],
+     [(F.F32, [1, 6, 48]), (F.F32, [1, 6]), (F.U8, [8])], {"scale": (F.F32, 0.1)}, "workspace"),
+    ("emi_attn_step_fwd_ffi", [(F.F32, [1, 6, 48]), (F.F32, [1, 9, 5, 48]), (F.F32, [1, 9, 5, 48])],
+     [(F.F32, [1, 6, 48]), (F.F32, [1, 6]), (F.U8, [4096])], {"scale": (F.F32, 0.1)}, "head_dim"),
+    ("emi_attn_step_bwd_ffi", [(F.F32, [1, 6, 48]), (F.F32, [1, 9, 6, 48]), (F.F32, [1, 9, 6, 48]), (F.F32, [1, 6, 48]),
+                               (F.F32, [1, 7]), (F.F32, [1, 6, 48])],
+     [(F.F32, [1, 6, 48]), (F.F32, [1, 9, 6, 48]), (F.F32, [1, 9, 6, 48]), (F.U8, [4096])], {"scale": (F.F32, 0.1)}, "lse"),
     ("emi_embedding_fwd_ffi", [(F.S64, [3]), (F.F32, [10, 4])], [(F.F32, [3, 4])], {}, "s32"),
     ("emi_swiglu_bwd_ffi", [(F.F32, [8])] * 3, [(F.F32, [8]), (F.F32, [9])], {}, "shape"),
 ])
@@ -114,7 +121,7 @@ def test_ffi_registration_lists_all_targets_for_rocm():
     lib.emi_ffi_target_handler.restype = C.c_void_p
     n = lib.emi_ffi_target_count()
     names = [lib.emi_ffi_target_name(i).decode() for i in range(n)]
-    assert n == 12 and "emi_attn_bwd" in names and all(lib.emi_ffi_target_handler(i) for i in range(n))
+    assert n == 14 and "emi_attn_bwd" in names and "emi_attn_step_bwd" in names and all(lib.emi_ffi_target_handler(i) for i in range(n))
     from enzyme_ad.jax import ops
     used = {t for fwd, bwd in ops.FFI_TARGETS.values() for t in (fwd,) + tuple(bwd)}
     assert used <= set(names)                                 # every target the lowering table names has a handler

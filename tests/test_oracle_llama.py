@@ -187,3 +187,39 @@ def test_attention_backward_adjoint_identity():
     h = 1e-6
     jp = (L.attention_fwd(q + h * tq, k + h * tk, v + h * tv)[0] - L.attention_fwd(q - h * tq, k - h * tk, v - h * tv)[0]) / (2 * h)
     assert np.isclose(np.sum(jp * do), np.sum(tq * dq) + np.sum(tk * dk) + np.sum(tv * dv), rtol=1e-7)
+
+
+@pytest.mark.parametrize("pos", [1, 4])
+def test_step_vjp_matches_literal_step_and_finite_differences(pos):
+    """`forward_step_vjp`: its forward value is the literal step's, and its cotangents are
+    the central finite differences of the literal step (float64) with respect to x, one
+    weight of every kind and both caches."""
+    cfg = CFG
+    w = _weights(cfg, 7)
+    rng = np.random.default_rng(11 + pos)
+    x = rng.standard_normal(cfg["dim"])
+    kc = rng.standard_normal((cfg["n_layers"], pos, cfg["dim"])) if pos > 1 else np.zeros((cfg["n_layers"], pos, cfg["dim"]))
+    vc = rng.standard_normal(kc.shape) if pos > 1 else np.zeros(kc.shape)
+    dy = rng.standard_normal(cfg["dim"])
+    y, dx, gw, dkc, dvc = L.forward_step_vjp(x, cfg, w, kc, vc, dy)
+    np.testing.assert_allclose(y, L.forward_step(x, cfg, w, kc, vc), rtol=1e-11, atol=1e-12)
+
+    def f(xx=x, ww=w, kk=kc, vv=vc):
+        return float(np.dot(L.forward_step(xx, cfg, ww, kk, vv), dy))
+
+    def fd(arr, idx, make, h=1e-6):
+        a = arr.copy(); a[idx] += h; up = f(**make(a))
+        a = arr.copy(); a[idx] -= h; dn = f(**make(a))
+        return (up - dn) / (2 * h)
+
+    picks = np.random.default_rng(3)
+    for idx in [tuple(picks.integers(0, n) for n in x.shape) for _ in range(4)]:
+        np.testing.assert_allclose(dx[idx], fd(x, idx, lambda a: dict(xx=a)), rtol=2e-5, atol=1e-7)
+    for name in list(L.LAYER_KEYS) + ["rms_final_weight"]:
+        for idx in [tuple(picks.integers(0, n) for n in w[name].shape) for _ in range(3)]:
+            got = gw[name][idx]
+            want = fd(w[name], idx, lambda a, name=name: dict(ww={**w, name: a}))
+            np.testing.assert_allclose(got, want, rtol=2e-5, atol=1e-7, err_msg=name)
+    for idx in [tuple(picks.integers(0, n) for n in kc.shape) for _ in range(4)]:
+        np.testing.assert_allclose(dkc[idx], fd(kc, idx, lambda a: dict(kk=a)), rtol=2e-5, atol=1e-7)
+        np.testing.assert_allclose(dvc[idx], fd(vc, idx, lambda a: dict(vv=a)), rtol=2e-5, atol=1e-7)
