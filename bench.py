@@ -193,9 +193,12 @@ def bench_kernels(cfg, iters):
     gm = lambda A, Bm, C, M_, N_, K_, lda, ldb, ta, tb: N.check(lib.emi_gemm(st, P(A), P(Bm), None, P(C), M_, N_, K_, lda, ldb,
                                                                              N_, N_, ta, tb, N.EMI_BF16))
     hbm("step_matvec_bf16", lambda: gm(xv, w, yv, 1, H, D, D, D, 0, 1), w.numel() * 2)
-    hbm("step_matvec_dx_bf16", lambda: gm(dyv, w, dxv, 1, D, H, H, D, 0, 0), w.numel() * 2)
+    gwb = lib.emi_gemm_workspace_bytes(1, D, H, 0, 0, N.EMI_BF16)
+    gws = torch.empty(gwb, dtype=torch.uint8, device="cuda")
+    hbm("step_matvec_dx_bf16", lambda: N.check(lib.emi_gemm_ws(st, P(dyv), P(w), None, P(dxv), P(gws), gwb, 1, D, H, H, D, D, D, 0, 0,
+                                                               N.EMI_BF16)), w.numel() * 2)
     hbm("step_matvec_dw_bf16", lambda: gm(dyv, xv, dw, H, D, 1, H, D, 1, 0), w.numel() * 2)
-    del w, dw
+    del w, dw, gws
     Bq, hq, Sk, dd = 8, 32, 4096, 128
     Dq = hq * dd
     qs, dos = (torch.randn((Bq, Dq), device="cuda").to(bf) for _ in range(2))

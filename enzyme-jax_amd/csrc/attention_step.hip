@@ -16,11 +16,10 @@ namespace emi {
 namespace {
 
 constexpr int kRedFloats = 2048;                 // LDS floats for the reduction over key slots
-constexpr int kKeysPerBlock = 512, kUnroll = 4;
+constexpr int kKeysPerBlock = 512;
 
 template <typename T, bool VEC> struct Elems {   // VEC: 16-byte chunks; else single elements (any head_dim / alignment)
   static constexpr int N = VEC ? Chunk<T>::N : 1;
-  static constexpr int MAXC = VEC ? 4 : 16;      // chunks per lane: head_dim <= 256 over 16 lanes
   static __device__ __forceinline__ void load(const T* p, float (&v)[N]) {
     if constexpr (VEC) Chunk<T>::load(p, v);
     else v[0] = to_f32(p[0]);
@@ -29,6 +28,18 @@ template <typename T, bool VEC> struct Elems {   // VEC: 16-byte chunks; else si
     if constexpr (VEC) Chunk<T>::store(p, v);
     else p[0] = from_f32<T>(v[0]);
   }
+};
+
+template <typename T> struct Vec16;              // 16 raw bytes of T, unpacked on use
+template <> struct Vec16<float> {
+  typedef float4 type;
+  static __device__ __forceinline__ float4 zero() { return make_float4(0.f, 0.f, 0.f, 0.f); }
+  static __device__ __forceinline__ void unpack(const float4& r, float (&v)[4]) { v[0] = r.x; v[1] = r.y; v[2] = r.z; v[3] = r.w; }
+};
+template <> struct Vec16<bf16> {
+  typedef uint4 type;
+  static __device__ __forceinline__ uint4 zero() { return make_uint4(0, 0, 0, 0); }
+  static __device__ __forceinline__ void unpack(const uint4& r, float (&v)[8]) { Vec8<bf16>::unpack(r, v); }
 };
 
 struct StepShape {
@@ -90,11 +101,13 @@ __device__ __forceinline__ void reduce_keys(float (&acc)[MAXC][NE], int nch, flo
   }
 }
 
-template <typename T, bool VEC>
+// NCH: 16-byte chunks (or single elements) of the head dimension per lane, 1, 2, 4 or 16; a
+// lane keeps 16 / NCH (at least 2) keys in flight.
+template <typename T, bool VEC, int NCH>
 __global__ __launch_bounds__(256) void attn_step_fwd_kernel(const T* __restrict__ q, const T* __restrict__ k,
                                                             const T* __restrict__ v, float* __restrict__ part, StepShape sh,
                                                             float scale) {
-  constexpr int NE = Elems<T, VEC>::N, MAXC = Elems<T, VEC>::MAXC;
+  constexpr int NE = Elems<T, VEC>::N, MAXC = NCH, kUnroll = NCH >= 8 ? 2 : 16 / NCH;
   __shared__ float scores[kKeysPerBlock];
   __shared__ float scratch[4];
   __shared__ float red[kRedFloats];
@@ -199,6 +212,98 @@ __global__ __launch_bounds__(256) void attn_step_fwd_kernel(const T* __restrict_
   }
 }
 
+// Forward for one 16-byte chunk per lane (head_dim 128 in bf16, 64 in fp32, and smaller):
+// the block loads all its K and V chunks up front (32 keys per slot, 16 loads of each kind
+// in flight per lane, kept as raw 16-byte vectors) and then works from registers, so the
+// memory system sees the whole request at once.
+template <typename T>
+__global__ __launch_bounds__(256) void attn_step_fwd1_kernel(const T* __restrict__ q, const T* __restrict__ k,
+                                                             const T* __restrict__ v, float* __restrict__ part, StepShape sh,
+                                                             float scale) {
+  constexpr int NE = Chunk<T>::N, KPS = kKeysPerBlock / 16 / 2;      // keys per slot and half
+  typedef typename Vec16<T>::type raw_t;
+  __shared__ float scratch[4];
+  __shared__ float red[kRedFloats];
+  const int bh = blockIdx.y, b = bh / sh.heads, h = bh % sh.heads;
+  const int l16 = threadIdx.x & 15, slot = threadIdx.x >> 4;
+  const bool mine = l16 * NE < sh.head_dim;                         // lanes beyond the head dimension idle
+  const T* qrow = q + b * sh.q_sb + h * sh.q_sh + l16 * NE;
+  const T* kbase = k + b * sh.kv_sb + h * sh.kv_sh + l16 * NE;
+  const T* vbase = v + b * sh.kv_sb + h * sh.kv_sh + l16 * NE;
+  float qf[NE];
+#pragma unroll
+  for (int e = 0; e < NE; e++) qf[e] = 0.f;
+  if (mine) Chunk<T>::load(qrow, qf);
+
+  float mx = -INFINITY, sum = 0.f;
+  float acc[1][NE];
+#pragma unroll
+  for (int e = 0; e < NE; e++) acc[0][e] = 0.f;
+  // two halves of 16 keys per slot: registers hold 16 K and 16 V chunks at a time
+#pragma unroll 1
+  for (int half = 0; half < 2; half++) {
+    const int s0 = blockIdx.x * kKeysPerBlock + half * (kKeysPerBlock / 2);
+    if (s0 >= sh.seq_kv) break;
+    raw_t kr[KPS], vr[KPS];
+#pragma unroll
+    for (int u = 0; u < KPS; u++) {
+      const int s = s0 + slot + 16 * u;
+      kr[u] = Vec16<T>::zero();
+      vr[u] = Vec16<T>::zero();
+      if (mine && s < sh.seq_kv) {
+        kr[u] = *reinterpret_cast<const raw_t*>(kbase + (int64_t)s * sh.kv_ss);
+        vr[u] = *reinterpret_cast<const raw_t*>(vbase + (int64_t)s * sh.kv_ss);
+      }
+    }
+    float sc[KPS];
+    float hm = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < KPS; u++) {
+      float kf[NE];
+      Vec16<T>::unpack(kr[u], kf);
+      float dot = 0.f;
+#pragma unroll
+      for (int e = 0; e < NE; e++) dot = fmaf(qf[e], kf[e], dot);
+      sc[u] = s0 + slot + 16 * u < sh.seq_kv ? sum16(dot) * scale : -INFINITY;
+      hm = fmaxf(hm, sc[u]);
+    }
+    // running maximum per slot (online softmax): rescale what has been accumulated so far
+    const float nm = fmaxf(mx, hm);
+    const float alpha = mx == -INFINITY ? 0.f : __expf(mx - nm);
+    sum *= alpha;
+#pragma unroll
+    for (int e = 0; e < NE; e++) acc[0][e] *= alpha;
+    mx = nm;
+#pragma unroll
+    for (int u = 0; u < KPS; u++) {
+      const float p = sc[u] == -INFINITY ? 0.f : __expf(sc[u] - mx);
+      sum += p;
+      float vf[NE];
+      Vec16<T>::unpack(vr[u], vf);
+#pragma unroll
+      for (int e = 0; e < NE; e++) acc[0][e] = fmaf(p, vf[e], acc[0][e]);
+    }
+  }
+  // the 16 slots have their own running maxima: bring them to the block maximum, then reduce
+  const float bm = block_max(mx, scratch);
+  const float w = mx == -INFINITY ? 0.f : __expf(mx - bm);
+#pragma unroll
+  for (int e = 0; e < NE; e++) acc[0][e] *= w;
+  float bsum = block_sum(l16 == 0 ? sum * w : 0.f, scratch);
+  reduce_keys<1, NE>(acc, mine ? 1 : 0, red);
+  if (threadIdx.x < 16) {
+    float* out = part + ((int64_t)bh * gridDim.x + blockIdx.x) * (sh.head_dim + 2);
+    if (mine) {
+#pragma unroll
+      for (int e = 0; e < NE; e++) out[l16 * NE + e] = acc[0][e];
+    }
+    if (threadIdx.x == 0) {
+      out[sh.head_dim] = bm;
+      out[sh.head_dim + 1] = bsum;
+    }
+  }
+}
+
 // o = sum_i w_i o_i / sum_i w_i l_i with w_i = exp(m_i - max m); lse = max m + log(sum).
 template <typename T>
 __global__ __launch_bounds__(64) void attn_step_combine_kernel(const float* __restrict__ part, T* __restrict__ o,
@@ -221,13 +326,13 @@ __global__ __launch_bounds__(64) void attn_step_combine_kernel(const float* __re
 
 // dV_s = p_s dO; dP_s = dO . V_s; dS_s = p_s (dP_s - dO . O); dQ = scale sum_s dS_s K_s;
 // dK_s = scale dS_s Q.  p is recomputed from lse; one pass over the keys of the block.
-template <typename T, bool VEC>
+template <typename T, bool VEC, int NCH>
 __global__ __launch_bounds__(256) void attn_step_bwd_kernel(const T* __restrict__ q, const T* __restrict__ k,
                                                             const T* __restrict__ v, const T* __restrict__ o,
                                                             const float* __restrict__ lse, const T* __restrict__ d_o,
                                                             float* __restrict__ part, T* __restrict__ dk, T* __restrict__ dv,
                                                             StepShape sh, float scale) {
-  constexpr int NE = Elems<T, VEC>::N, MAXC = Elems<T, VEC>::MAXC;
+  constexpr int NE = Elems<T, VEC>::N, MAXC = NCH, kUnroll = NCH >= 4 ? 2 : 8 / NCH;
   __shared__ float red[kRedFloats];
   const int bh = blockIdx.y, b = bh / sh.heads, h = bh % sh.heads;
   const int s0 = blockIdx.x * kKeysPerBlock;
@@ -257,10 +362,10 @@ __global__ __launch_bounds__(256) void attn_step_bwd_kernel(const T* __restrict_
   for (int c = 0; c < MAXC; c++)
 #pragma unroll
     for (int e = 0; e < NE; e++) acc[c][e] = 0.f;
-  for (int sb = s0 + slot; sb < s1; sb += 16 * 2) {
-    float kf[2][MAXC][NE], vf[2][MAXC][NE];
+  for (int sb = s0 + slot; sb < s1; sb += 16 * kUnroll) {
+    float kf[kUnroll][MAXC][NE], vf[kUnroll][MAXC][NE];
 #pragma unroll
-    for (int u = 0; u < 2; u++) {
+    for (int u = 0; u < kUnroll; u++) {
       const int s = sb + 16 * u;
       if (s < s1) {
 #pragma unroll
@@ -272,7 +377,7 @@ __global__ __launch_bounds__(256) void attn_step_bwd_kernel(const T* __restrict_
       }
     }
 #pragma unroll
-    for (int u = 0; u < 2; u++) {
+    for (int u = 0; u < kUnroll; u++) {
       const int s = sb + 16 * u;
       float dot = 0.f, dp = 0.f;
       if (s < s1) {
@@ -378,21 +483,34 @@ extern "C" int emi_attn_step_fwd(emi_stream_t stream, const void* q, const void*
   const int nsplit = (int)((seq_kv + kKeysPerBlock - 1) / kKeysPerBlock);
   const dim3 grid((unsigned)nsplit, (unsigned)(batch * heads));
   float* part = static_cast<float*>(workspace);
-#define EMI_STEP_FWD(T, VEC)                                                                                             \
+#define EMI_STEP_FWD(T, VEC, NCH)                                                                                       \
   do {                                                                                                                   \
-    hipLaunchKernelGGL((attn_step_fwd_kernel<T, VEC>), grid, dim3(256), 0, st, (const T*)q, (const T*)k, (const T*)v,    \
-                       part, sh, scale);                                                                                 \
+    hipLaunchKernelGGL((attn_step_fwd_kernel<T, VEC, NCH>), grid, dim3(256), 0, st, (const T*)q, (const T*)k,            \
+                       (const T*)v, part, sh, scale);                                                                    \
     EMI_CHECK_LAUNCH("emi_attn_step_fwd");                                                                               \
     hipLaunchKernelGGL(attn_step_combine_kernel<T>, dim3((unsigned)(batch * heads)), dim3(64), 0, st, part, (T*)o, lse,  \
                        sh, nsplit);                                                                                      \
   } while (0)
-  if (dtype == EMI_BF16) {
-    if (vec) EMI_STEP_FWD(bf16, true);
-    else EMI_STEP_FWD(bf16, false);
-  } else {
-    if (vec) EMI_STEP_FWD(float, true);
-    else EMI_STEP_FWD(float, false);
-  }
+#define EMI_STEP_FWD1(T)                                                                                                \
+  do {                                                                                                                   \
+    hipLaunchKernelGGL(attn_step_fwd1_kernel<T>, grid, dim3(256), 0, st, (const T*)q, (const T*)k, (const T*)v, part,    \
+                       sh, scale);                                                                                       \
+    EMI_CHECK_LAUNCH("emi_attn_step_fwd");                                                                               \
+    hipLaunchKernelGGL(attn_step_combine_kernel<T>, dim3((unsigned)(batch * heads)), dim3(64), 0, st, part, (T*)o, lse,  \
+                       sh, nsplit);                                                                                      \
+  } while (0)
+#define EMI_STEP_FWD_T(T)                                              \
+  do {                                                                 \
+    if (!vec) EMI_STEP_FWD(T, false, 16);                              \
+    else if (nch <= 1) EMI_STEP_FWD1(T);                               \
+    else if (nch <= 2) EMI_STEP_FWD(T, true, 2);                       \
+    else EMI_STEP_FWD(T, true, 4);                                     \
+  } while (0)
+  const int nch = (int)((head_dim / ne + 15) / 16);      // 16-byte chunks per lane
+  if (dtype == EMI_BF16) EMI_STEP_FWD_T(bf16);
+  else EMI_STEP_FWD_T(float);
+#undef EMI_STEP_FWD_T
+#undef EMI_STEP_FWD1
 #undef EMI_STEP_FWD
   EMI_CHECK_LAUNCH("emi_attn_step_fwd(combine)");
   return EMI_OK;
@@ -420,21 +538,25 @@ extern "C" int emi_attn_step_bwd(emi_stream_t stream, const void* q, const void*
   const int nsplit = (int)((seq_kv + kKeysPerBlock - 1) / kKeysPerBlock);
   const dim3 grid((unsigned)nsplit, (unsigned)(batch * heads));
   float* part = static_cast<float*>(workspace);
-#define EMI_STEP_BWD(T, VEC)                                                                                             \
+#define EMI_STEP_BWD(T, VEC, NCH)                                                                                       \
   do {                                                                                                                   \
-    hipLaunchKernelGGL((attn_step_bwd_kernel<T, VEC>), grid, dim3(256), 0, st, (const T*)q, (const T*)k, (const T*)v,    \
-                       (const T*)o, lse, (const T*)d_o, part, (T*)dk, (T*)dv, sh, scale);                                \
+    hipLaunchKernelGGL((attn_step_bwd_kernel<T, VEC, NCH>), grid, dim3(256), 0, st, (const T*)q, (const T*)k,            \
+                       (const T*)v, (const T*)o, lse, (const T*)d_o, part, (T*)dk, (T*)dv, sh, scale);                   \
     EMI_CHECK_LAUNCH("emi_attn_step_bwd");                                                                               \
     hipLaunchKernelGGL(attn_step_dq_kernel<T>, dim3((unsigned)(batch * heads)), dim3(64), 0, st, part, (T*)dq, sh,       \
                        nsplit);                                                                                          \
   } while (0)
-  if (dtype == EMI_BF16) {
-    if (vec) EMI_STEP_BWD(bf16, true);
-    else EMI_STEP_BWD(bf16, false);
-  } else {
-    if (vec) EMI_STEP_BWD(float, true);
-    else EMI_STEP_BWD(float, false);
-  }
+#define EMI_STEP_BWD_T(T)                                              \
+  do {                                                                 \
+    if (!vec) EMI_STEP_BWD(T, false, 16);                              \
+    else if (nch <= 1) EMI_STEP_BWD(T, true, 1);                       \
+    else if (nch <= 2) EMI_STEP_BWD(T, true, 2);                       \
+    else EMI_STEP_BWD(T, true, 4);                                     \
+  } while (0)
+  const int nch = (int)((head_dim / ne + 15) / 16);      // 16-byte chunks per lane
+  if (dtype == EMI_BF16) EMI_STEP_BWD_T(bf16);
+  else EMI_STEP_BWD_T(float);
+#undef EMI_STEP_BWD_T
 #undef EMI_STEP_BWD
   EMI_CHECK_LAUNCH("emi_attn_step_bwd(dq)");
   return EMI_OK;

@@ -93,6 +93,9 @@ template <> struct Vec8<bf16> {
 template <typename T> struct Chunk;
 template <> struct Chunk<float> {
   static constexpr int N = 4;
+  typedef float4 Raw;
+  static __device__ __forceinline__ Raw load_raw(const float* p) { return *reinterpret_cast<const float4*>(p); }
+  static __device__ __forceinline__ void unpack(const Raw& a, float (&v)[4]) { v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; }
   static __device__ __forceinline__ void load(const float* p, float (&v)[4]) {
     const float4 a = *reinterpret_cast<const float4*>(p);
     v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
@@ -103,6 +106,9 @@ template <> struct Chunk<float> {
 };
 template <> struct Chunk<bf16> {
   static constexpr int N = 8;
+  typedef uint4 Raw;
+  static __device__ __forceinline__ Raw load_raw(const bf16* p) { return *reinterpret_cast<const uint4*>(p); }
+  static __device__ __forceinline__ void unpack(const Raw& a, float (&v)[8]) { Vec8<bf16>::unpack(a, v); }
   static __device__ __forceinline__ void load(const bf16* p, float (&v)[8]) { Vec8<bf16>::load(p, v); }
   static __device__ __forceinline__ void store(bf16* p, const float (&v)[8]) { Vec8<bf16>::store(p, v); }
 };

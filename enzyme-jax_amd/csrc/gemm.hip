@@ -951,17 +951,29 @@ static int launch_generic(hipStream_t st, const void* A, const void* B, const vo
 }
 
 // gemm_skinny.hip
-int launch_skinny(hipStream_t st, const void* A, const void* B, const void* R, void* C, int64_t M, int64_t N, int64_t K,
-                  int64_t lda, int64_t ldb, int64_t ldr, int64_t ldc, int trans_a, int trans_b, int dtype);
+int launch_skinny(hipStream_t st, const void* A, const void* B, const void* R, void* C, void* workspace, size_t workspace_bytes,
+                  int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldr, int64_t ldc, int trans_a, int trans_b,
+                  int dtype);
+size_t skinny_workspace_bytes(int64_t M, int64_t N, int64_t K, int trans_a, int trans_b, int dtype);
 
 }  // namespace emi
 
 using namespace emi;
 
 
+extern "C" size_t emi_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int trans_a, int trans_b, int dtype) {
+  return skinny_workspace_bytes(M, N, K, trans_a, trans_b, dtype);
+}
+
 extern "C" int emi_gemm(emi_stream_t stream, const void* A, const void* B, const void* R, void* C, int64_t M, int64_t N,
                         int64_t K, int64_t lda, int64_t ldb, int64_t ldr, int64_t ldc, int trans_a, int trans_b,
                         int dtype) {
+  return emi_gemm_ws(stream, A, B, R, C, nullptr, 0, M, N, K, lda, ldb, ldr, ldc, trans_a, trans_b, dtype);
+}
+
+extern "C" int emi_gemm_ws(emi_stream_t stream, const void* A, const void* B, const void* R, void* C, void* workspace,
+                           size_t workspace_bytes, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldr,
+                           int64_t ldc, int trans_a, int trans_b, int dtype) {
   EMI_REQUIRE(M >= 0 && N >= 0 && K >= 0, "emi_gemm: negative dimension M=%lld N=%lld K=%lld", (long long)M, (long long)N,
               (long long)K);
   EMI_REQUIRE(M <= 0x7fffffff && N <= 0x7fffffff && K <= 0x7fffffff, "emi_gemm: dimension exceeds 2^31-1");
@@ -974,7 +986,7 @@ extern "C" int emi_gemm(emi_stream_t stream, const void* A, const void* B, const
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (K > 0 && (R == nullptr || ldr >= N)) {
     // single-token forms (mat-vec and its adjoints): weight-bandwidth-bound kernels
-    const int rc = launch_skinny(st, A, B, R, C, M, N, K, lda, ldb, ldr, ldc, trans_a, trans_b, dtype);
+    const int rc = launch_skinny(st, A, B, R, C, workspace, workspace_bytes, M, N, K, lda, ldb, ldr, ldc, trans_a, trans_b, dtype);
     if (rc >= 0) return rc;
   }
   if (dtype == EMI_BF16) {

@@ -128,6 +128,105 @@ __global__ __launch_bounds__(1024) void gemv_nn_kernel(const T* __restrict__ A, 
   }
 }
 
+// The same product with a workspace: the K rows are cut into bands, a block sums one band
+// for 256 chunks of columns (every row it reads is one contiguous run), writes fp32
+// partials [band][m][n], and a second kernel adds the bands in order.  Hundreds of blocks
+// instead of N / 64, and no 8 KB strides inside a wavefront.
+template <typename T, int MT>
+__global__ __launch_bounds__(256) void gemv_nn_bands_kernel(const T* __restrict__ A, const T* __restrict__ B,
+                                                            float* __restrict__ part, int M, int N, int K, int64_t lda,
+                                                            int64_t ldb, int rows_per_band) {
+  constexpr int V = Chunk<T>::N, UN = 16, AR = 256;
+  __shared__ float sa[MT][AR];                                    // A values of the rows being processed
+  const int n = (blockIdx.x * 256 + threadIdx.x) * V;
+  const int k_begin = blockIdx.y * rows_per_band;
+  const int k_end = k_begin + rows_per_band < K ? k_begin + rows_per_band : K;
+  const bool live = n < N;
+  float acc[MT][V];
+#pragma unroll
+  for (int m = 0; m < MT; m++)
+#pragma unroll
+    for (int e = 0; e < V; e++) acc[m][e] = 0.f;
+  for (int kc = k_begin; kc < k_end; kc += AR) {
+    __syncthreads();
+#pragma unroll
+    for (int m = 0; m < MT; m++)
+      if (m < M) sa[m][threadIdx.x] = kc + (int)threadIdx.x < k_end ? to_f32(A[(int64_t)m * lda + kc + threadIdx.x]) : 0.f;
+    __syncthreads();
+    const int kce = kc + AR < k_end ? kc + AR : k_end;
+    if (live) {
+      for (int k0 = kc; k0 < kce; k0 += UN) {
+        typename Chunk<T>::Raw b[UN];
+#pragma unroll
+        for (int u = 0; u < UN; u++)
+          if (k0 + u < kce) b[u] = Chunk<T>::load_raw(B + (int64_t)(k0 + u) * ldb + n);
+#pragma unroll
+        for (int u = 0; u < UN; u++)
+          if (k0 + u < kce) {
+            float bf[V];
+            Chunk<T>::unpack(b[u], bf);
+#pragma unroll
+            for (int m = 0; m < MT; m++)
+              if (m < M) {
+                const float a = sa[m][k0 + u - kc];
+#pragma unroll
+                for (int e = 0; e < V; e++) acc[m][e] = fmaf(a, bf[e], acc[m][e]);
+              }
+          }
+      }
+    }
+  }
+  if (!live) return;
+#pragma unroll
+  for (int m = 0; m < MT; m++)
+    if (m < M) {
+      float* dst = part + ((int64_t)blockIdx.y * M + m) * N + n;
+#pragma unroll
+      for (int e = 0; e < V; e += 4) *reinterpret_cast<float4*>(dst + e) = make_float4(acc[m][e], acc[m][e + 1], acc[m][e + 2], acc[m][e + 3]);
+    }
+}
+
+// C[m][n] = sum over bands (in a fixed order) + R: 64 columns per block, 4 band lanes each
+// with 8 loads in flight, met through LDS.
+template <typename T>
+__global__ __launch_bounds__(256) void gemv_bands_reduce_kernel(const float* __restrict__ part, const T* R, T* C, int M, int N,
+                                                                int bands, int64_t ldr, int64_t ldc) {
+  __shared__ float red[4][64];
+  const int col = threadIdx.x & 63, bl = threadIdx.x >> 6;
+  const int64_t i = blockIdx.x * (int64_t)64 + col;               // index into [M][N]
+  const bool live = i < (int64_t)M * N;
+  float v = 0.f;
+  if (live) {
+    const int m = (int)(i / N), n = (int)(i % N);
+    const float* p = part + (int64_t)m * N + n;
+    const int64_t bstride = (int64_t)M * N;
+    for (int b0 = bl; b0 < bands; b0 += 4 * 8) {
+      float t[8];
+#pragma unroll
+      for (int u = 0; u < 8; u++) t[u] = b0 + 4 * u < bands ? p[(int64_t)(b0 + 4 * u) * bstride] : 0.f;
+#pragma unroll
+      for (int u = 0; u < 8; u++) v += t[u];
+    }
+  }
+  red[bl][col] = v;
+  __syncthreads();
+  if (bl == 0 && live) {
+    const int m = (int)(i / N), n = (int)(i % N);
+    v = red[0][col] + red[1][col] + red[2][col] + red[3][col];
+    if (R != nullptr) v += to_f32(R[(int64_t)m * ldr + n]);
+    C[(int64_t)m * ldc + n] = from_f32<T>(v);
+  }
+}
+
+// Number of row bands for the workspace form (the same in the size query and the launch).
+int nn_bands(int64_t N, int64_t K, int V) {
+  const int64_t colgroups = (N / V + 255) / 256;
+  int64_t bands = (1024 + colgroups - 1) / colgroups;
+  if (bands > 256) bands = 256;
+  if (bands > (K + 7) / 8) bands = (K + 7) / 8;
+  return (int)(bands < 1 ? 1 : bands);
+}
+
 // C[m][n] = sum_{k < K <= 8} A[k][m] B[k][n] (+ R): a sum of K outer products, one 16-byte
 // store per thread; bound by the write of C.
 template <typename T>
@@ -158,8 +257,9 @@ __global__ __launch_bounds__(256) void outer_tn_kernel(const T* __restrict__ A, 
 bool al16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 template <typename T>
-int launch_skinny_t(hipStream_t st, const void* A_, const void* B_, const void* R_, void* C_, int64_t M, int64_t N, int64_t K,
-                    int64_t lda, int64_t ldb, int64_t ldr, int64_t ldc, int trans_a, int trans_b) {
+int launch_skinny_t(hipStream_t st, const void* A_, const void* B_, const void* R_, void* C_, void* workspace,
+                    size_t workspace_bytes, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldr, int64_t ldc,
+                    int trans_a, int trans_b) {
   constexpr int V = Chunk<T>::N;
   const T* A = static_cast<const T*>(A_);
   const T* B = static_cast<const T*>(B_);
@@ -177,7 +277,24 @@ int launch_skinny_t(hipStream_t st, const void* A_, const void* B_, const void* 
     EMI_SKINNY_MT(gemv_nt_kernel, dim3((unsigned)((N + 3) / 4)), 256);
   } else if (!trans_a && !trans_b) {         // 16-byte chunks along N of B
     if (M > 8 || N % V || ldb % V || !al16(B)) return -1;
-    EMI_SKINNY_MT(gemv_nn_kernel, dim3((unsigned)((N / V + 7) / 8)), 1024);
+    const int bands = nn_bands(N, K, V);
+    if (workspace != nullptr && al16(workspace) && workspace_bytes >= (size_t)bands * M * N * sizeof(float) && bands > 1) {
+      const int rpb = (int)((K + bands - 1) / bands);
+      const dim3 grid((unsigned)((N / V + 255) / 256), (unsigned)bands);
+      float* part = static_cast<float*>(workspace);
+#define EMI_BANDS(MT)                                                                                                   \
+  hipLaunchKernelGGL((gemv_nn_bands_kernel<T, MT>), grid, dim3(256), 0, st, A, B, part, (int)M, (int)N, (int)K, lda, ldb, rpb)
+      if (M <= 1) EMI_BANDS(1);
+      else if (M <= 2) EMI_BANDS(2);
+      else if (M <= 4) EMI_BANDS(4);
+      else EMI_BANDS(8);
+#undef EMI_BANDS
+      EMI_CHECK_LAUNCH("emi_gemm(skinny bands)");
+      hipLaunchKernelGGL(gemv_bands_reduce_kernel<T>, dim3((unsigned)((M * N + 63) / 64)), dim3(256), 0, st, part, R, C, (int)M,
+                         (int)N, bands, ldr, ldc);
+    } else {
+      EMI_SKINNY_MT(gemv_nn_kernel, dim3((unsigned)((N / V + 7) / 8)), 1024);
+    }
   } else if (trans_a && !trans_b) {          // outer products: 16-byte chunks along N of B, C (and R)
     if (K > 8 || N % V || ldb % V || ldc % V || !al16(B) || !al16(C) || (R != nullptr && (ldr % V || !al16(R)))) return -1;
     const int64_t total = M * (N / V);
@@ -195,11 +312,22 @@ int launch_skinny_t(hipStream_t st, const void* A_, const void* B_, const void* 
 
 // Returns -1 when the shape is not one of the skinny forms (the caller then takes the tiled
 // kernels), otherwise a status code.
-int launch_skinny(hipStream_t st, const void* A, const void* B, const void* R, void* C, int64_t M, int64_t N, int64_t K,
-                  int64_t lda, int64_t ldb, int64_t ldr, int64_t ldc, int trans_a, int trans_b, int dtype) {
+int launch_skinny(hipStream_t st, const void* A, const void* B, const void* R, void* C, void* workspace, size_t workspace_bytes,
+                  int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldr, int64_t ldc, int trans_a, int trans_b,
+                  int dtype) {
   if (M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff) return -1;
-  if (dtype == EMI_BF16) return launch_skinny_t<bf16>(st, A, B, R, C, M, N, K, lda, ldb, ldr, ldc, trans_a, trans_b);
-  return launch_skinny_t<float>(st, A, B, R, C, M, N, K, lda, ldb, ldr, ldc, trans_a, trans_b);
+  if (dtype == EMI_BF16)
+    return launch_skinny_t<bf16>(st, A, B, R, C, workspace, workspace_bytes, M, N, K, lda, ldb, ldr, ldc, trans_a, trans_b);
+  return launch_skinny_t<float>(st, A, B, R, C, workspace, workspace_bytes, M, N, K, lda, ldb, ldr, ldc, trans_a, trans_b);
+}
+
+// Bytes of workspace with which the skinny NN form runs its banded kernel (0: none useful).
+size_t skinny_workspace_bytes(int64_t M, int64_t N, int64_t K, int trans_a, int trans_b, int dtype) {
+  if (trans_a || trans_b || M < 1 || M > 8 || N < 1 || K < 1) return 0;
+  const int V = dtype == EMI_BF16 ? 8 : 4;
+  if (N % V) return 0;
+  const int bands = nn_bands(N, K, V);
+  return bands > 1 ? (size_t)bands * M * N * sizeof(float) : 0;
 }
 
 }  // namespace emi

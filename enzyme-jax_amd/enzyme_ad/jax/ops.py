@@ -243,8 +243,10 @@ def gemm(a, b, trans_a=False, trans_b=False, residual=None):
     if residual is not None and residual.shape != (M, Nn):
         raise ValueError("gemm: residual shape %s != (%d, %d)" % (tuple(residual.shape), M, Nn))
     c = torch.empty((M, Nn), dtype=a.dtype, device=a.device)
-    N.check(N.lib().emi_gemm(_stream(), _p(a), _p(b), _p(residual), _p(c), M, Nn, K, a.shape[1], b.shape[1], Nn, Nn,
-                             int(trans_a), int(trans_b), _code(a)))
+    nbytes = N.lib().emi_gemm_workspace_bytes(M, Nn, K, int(trans_a), int(trans_b), _code(a))
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=a.device) if nbytes else None
+    N.check(N.lib().emi_gemm_ws(_stream(), _p(a), _p(b), _p(residual), _p(c), _p(ws), nbytes, M, Nn, K, a.shape[1],
+                                b.shape[1], Nn, Nn, int(trans_a), int(trans_b), _code(a)))
     return c
 
 
@@ -264,7 +266,11 @@ def matmul_nt(x, w, residual=None):
         # dX = dY . W: W is transposed first (2|W| bytes of HBM traffic, shared by nothing
         # else) so that the contraction index is innermost in both operands: the
         # k-contiguous kernel beats the k-major one by more than the transpose costs.
-        dx = gemm(c2, _transpose_shared(w), False, True, ax).reshape(x.shape)
+        # With a handful of tokens (the single-token step) W is read in place, once.
+        if c2.shape[0] <= 8:
+            dx = gemm(c2, w, False, False, ax).reshape(x.shape)
+        else:
+            dx = gemm(c2, _transpose_shared(w), False, True, ax).reshape(x.shape)
         # dW = dY^T . X contracts over tokens, the slow index of both operands: the
         # k-major form of the GEMM kernel reads them in place (transposing LDS loads),
         # 3-7% slower than the k-contiguous form but without two activation-sized

@@ -103,6 +103,17 @@ int emi_gemm(emi_stream_t stream, const void* A, const void* B, const void* R, v
              int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldr, int64_t ldc,
              int trans_a, int trans_b, int dtype);
 
+/* The same with an optional scratch buffer.  Only the single-token adjoint
+ * dX = dY.W (trans_a = trans_b = 0, M <= 8) uses one: with
+ * emi_gemm_workspace_bytes() bytes it sums row bands of W in many blocks and
+ * adds the partial sums in a fixed order (about 3x faster); without, or for
+ * any other shape, the call is emi_gemm. */
+size_t emi_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int trans_a, int trans_b, int dtype);
+int emi_gemm_ws(emi_stream_t stream, const void* A, const void* B, const void* R, void* C,
+                void* workspace, size_t workspace_bytes, int64_t M, int64_t N, int64_t K,
+                int64_t lda, int64_t ldb, int64_t ldr, int64_t ldc, int trans_a, int trans_b,
+                int dtype);
+
 /* Causal softmax attention, forward.  Replaces the per-head loop of
  * test/llama.py:178-206 with softmax of :13-18 (scale applied after the dot,
  * max-subtracted, fp32 statistics).  Element (b, h, s, i) of q/k/v/o lives at

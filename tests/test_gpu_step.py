@@ -26,7 +26,12 @@ def test_skinny_gemm_forms(dt, m, n, k):
     rw, rwr = dev(rng.standard_normal((n, k)), dt)
     check(ops.gemm(x, w, False, True), xr @ wr.T, dt, "y")
     check(ops.gemm(x, w, False, True, r), xr @ wr.T + rr, dt, "y + r")
-    check(ops.gemm(dy, w, False, False), dyr @ wr, dt, "dx")
+    check(ops.gemm(dy, w, False, False), dyr @ wr, dt, "dx")                    # banded kernel (workspace)
+    plain = torch.empty((m, k), dtype=dy.dtype, device="cuda")                  # same product without a workspace
+    from enzyme_ad.jax import _native as N
+    N.check(N.lib().emi_gemm(torch.cuda.current_stream().cuda_stream, dy.data_ptr(), w.data_ptr(), None, plain.data_ptr(),
+                             m, k, n, n, k, k, k, 0, 0, ops._code(dy)))
+    check(plain, dyr @ wr, dt, "dx without workspace")
     check(ops.gemm(dy, w, False, False, rx), dyr @ wr + rxr, dt, "dx + r")
     check(ops.gemm(dy, x, True, False), dyr.T @ xr, dt, "dw")
     check(ops.gemm(dy, x, True, False, rw), dyr.T @ xr + rwr, dt, "dw + r")
