@@ -31,7 +31,7 @@ PEAK_HBM_GBS = 8000.0         # MI355X HBM3E
 # HBM-side bytes per GEMM launch (average over the 21 launches of one step) from the
 # FETCH_SIZE and WRITE_SIZE counter runs summarised in
 # profiles/gemm_bf16_llama7b_layer_hbm_traffic.txt (only valid for the default workload).
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = 1.890e9
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = 1.674e9
 
 C5 = dict(dim=4096, hidden_dim=11008, n_heads=32, batch=4, seq=4096)
 
