@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the llama forward + VJP path on one MI355X.
 
-Default workload (BASELINE.json configs[4], the one the metric is quoted on):
+Default workload (the configuration the metric is quoted on):
 one Llama-2-7B-shaped decoder layer, dim 4096, SwiGLU hidden 11008, 32 heads of
 128, batch 4 x seq 4096, bf16 weights N(0,0.02), activations and output
 cotangent N(0,1), RMSNorm eps 1e-5, RoPE theta 10000.  A step is one forward
@@ -156,6 +156,7 @@ def bench_kernels(cfg, iters):
         hbm("rmsnorm_fwd_" + tag, lambda: N.check(lib.emi_rmsnorm_fwd(st, P(x), P(gam), P(y), rows, D, 1e-5, code)), 2 * n * s)
         hbm("rmsnorm_bwd_" + tag, lambda: N.check(lib.emi_rmsnorm_bwd(st, P(x), P(gam), P(dy), None, P(y), P(dgam), P(ws), wsb,
                                                                       rows, D, 1e-5, code)), 3 * n * s)
+        hbm("rmsnorm_jvp_" + tag, lambda: N.check(lib.emi_rmsnorm_jvp(st, P(x), P(gam), P(dy), P(gam), P(y), rows, D, 1e-5, code)), 3 * n * s)
         hbm("rope_fwd_" + tag, lambda: N.check(lib.emi_rope(st, P(x), P(table), P(y), 16, 2048, 32, 128, 0, code)), 2 * n * s)
         hbm("rope_bwd_" + tag, lambda: N.check(lib.emi_rope(st, P(dy), P(table), P(y), 16, 2048, 32, 128, 1, code)), 2 * n * s)
         del x, dy, y, ws
@@ -165,6 +166,7 @@ def bench_kernels(cfg, iters):
     da, db = torch.empty_like(a), torch.empty_like(a)
     n = a.numel()
     hbm("swiglu_fwd_bf16", lambda: N.check(lib.emi_swiglu_fwd(st, P(a), P(b), P(da), n, N.EMI_BF16)), 3 * n * 2)
+    hbm("swiglu_jvp_bf16", lambda: N.check(lib.emi_swiglu_jvp(st, P(a), P(b), P(dg), P(db), P(da), n, N.EMI_BF16)), 5 * n * 2)
     hbm("swiglu_bwd_bf16", lambda: N.check(lib.emi_swiglu_bwd(st, P(a), P(b), P(dg), P(da), P(db), n, N.EMI_BF16)), 5 * n * 2)
     del a, b, dg, da, db
     # C3: attention [8, 32, 2048, 128] bf16 causal
@@ -182,6 +184,11 @@ def bench_kernels(cfg, iters):
                                                             h * S * d, S * d, d, sc, 1, N.EMI_BF16)), fl)
     mfma("attn_bwd_c3", lambda: N.check(lib.emi_attn_bwd(st, P(q), P(k), P(v), P(o), P(lse), P(do), P(dq), P(dk), P(dv), P(ws), wsb,
                                                          B, h, S, d, h * S * d, S * d, d, sc, 1, N.EMI_BF16)), 2.5 * fl)
+    # forward mode: tangent of the same attention on a quarter of the heads (one-wavefront-per-row kernel),
+    # counted like the adjoint at 2.5x the forward flops (5 matmuls)
+    hj = h // 4
+    mfma("attn_jvp_c3_quarter", lambda: N.check(lib.emi_attn_jvp(st, P(q), P(k), P(v), P(lse), P(do), P(dq), P(dk), P(dv), B, hj, S, d,
+                                                                 h * S * d, S * d, d, sc, 1, N.EMI_BF16)), 2.5 * fl * hj / h)
     del q, k, v, do, o, dq, dk, dv, ws, fws
     # Single-token (decode) step at the 7B layer's widths: mat-vec over W [11008, 4096] and its
     # adjoints (weight read or written once), attention of one query per head over a
@@ -333,7 +340,7 @@ def main():
         "value": tokens / dt, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": dt * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": "Llama-2-7B-shaped decoder layer fwd+VJP (BASELINE configs[4]): dim 4096, hidden 11008, "
+        "config": {"workload": "Llama-2-7B-shaped decoder layer fwd+VJP: dim 4096, hidden 11008, "
                                "32 heads x 128, batch %d x seq %d, bf16" % (cfg["batch"], cfg["seq"]),
                    "tokens_per_step": tokens, "algorithmic_tflop_per_step": fl["total"] / 1e12,
                    "step_tflops": fl["total"] / dt / 1e12},

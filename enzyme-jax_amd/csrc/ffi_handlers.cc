@@ -337,6 +337,55 @@ extern "C" XLA_FFI_Error* emi_attn_bwd_ffi(XLA_FFI_CallFrame* cf) {
                                     (float)scale, (int)causal, q->dtype));
 }
 
+// Forward mode: tangents are ordinary operands (a zero tangent is passed as zeros).
+extern "C" XLA_FFI_Error* emi_rmsnorm_jvp_ffi(XLA_FFI_CallFrame* cf) {
+  EMI_FFI_BEGIN("emi_rmsnorm_jvp", 4, 4, 1, 1)
+  const XLA_FFI_Buffer *x = f.arg(0), *g = f.arg(1), *tx = f.arg(2), *tg = f.arg(3), *ty = f.ret(0);
+  if (!is_float(x) || g->dtype != x->dtype || tx->dtype != x->dtype || tg->dtype != x->dtype || ty->dtype != x->dtype)
+    return f.invalid("all tensors must share one dtype, f32 or bf16 (x has code %lld)", x->dtype);
+  if (x->rank < 1 || g->rank != 1 || g->dims[0] != x->dims[x->rank - 1])
+    return f.invalid("gamma must be rank 1 with the last dimension of x (x rank %lld, gamma rank %lld)", x->rank, g->rank);
+  if (!same_shape(x, tx) || !same_shape(x, ty) || !same_shape(g, tg)) return f.invalid("tx, ty must have the shape of x and tgamma that of gamma");
+  double eps;
+  if (!f.get_f("eps", &eps)) return f.invalid("missing f32/f64 attribute 'eps'");
+  EMI_FFI_STREAM()
+  const int64_t D = g->dims[0];
+  return f.from_status(emi_rmsnorm_jvp(stream, x->data, g->data, tx->data, tg->data, ty->data, D ? numel(x) / D : 0, D, (float)eps,
+                                       x->dtype));
+}
+
+extern "C" XLA_FFI_Error* emi_swiglu_jvp_ffi(XLA_FFI_CallFrame* cf) {
+  EMI_FFI_BEGIN("emi_swiglu_jvp", 4, 4, 1, 1)
+  const XLA_FFI_Buffer *a = f.arg(0), *b = f.arg(1), *ta = f.arg(2), *tb = f.arg(3), *tg = f.ret(0);
+  if (!is_float(a) || b->dtype != a->dtype || ta->dtype != a->dtype || tb->dtype != a->dtype || tg->dtype != a->dtype)
+    return f.invalid("all tensors must share one dtype, f32 or bf16 (code %lld)", a->dtype);
+  if (!same_shape(a, b) || !same_shape(a, ta) || !same_shape(a, tb) || !same_shape(a, tg)) return f.invalid("all tensors must have one shape");
+  EMI_FFI_STREAM()
+  return f.from_status(emi_swiglu_jvp(stream, a->data, b->data, ta->data, tb->data, tg->data, numel(a), a->dtype));
+}
+
+extern "C" XLA_FFI_Error* emi_attn_jvp_ffi(XLA_FFI_CallFrame* cf) {
+  EMI_FFI_BEGIN("emi_attn_jvp", 7, 7, 1, 1)
+  const XLA_FFI_Buffer *q = f.arg(0), *k = f.arg(1), *v = f.arg(2), *lse = f.arg(3), *tq = f.arg(4), *tk = f.arg(5), *tv = f.arg(6);
+  const XLA_FFI_Buffer* to = f.ret(0);
+  if (!is_float(q)) return f.invalid("q must be f32 or bf16 (code %lld)", q->dtype);
+  const XLA_FFI_Buffer* same[] = {k, v, tq, tk, tv, to};
+  for (const XLA_FFI_Buffer* b : same)
+    if (b->dtype != q->dtype || !same_shape(q, b)) return f.invalid("q, k, v, tq, tk, tv, to must share dtype and shape");
+  int64_t causal = 1, bshd = 0;
+  double scale;
+  f.get_i("causal", &causal);
+  f.get_i("bshd", &bshd);
+  if (!f.get_f("scale", &scale)) return f.invalid("missing f32/f64 attribute 'scale'");
+  AttnDims d;
+  if (!attn_dims(q, bshd, &d)) return f.invalid("q must be rank 4 (rank %lld)", q->rank);
+  if (lse->dtype != XLA_FFI_DataType_F32 || lse->rank != 3 || lse->dims[0] != d.B || lse->dims[1] != d.H || lse->dims[2] != d.S)
+    return f.invalid("lse must be f32[batch, heads, seq] = [%lld, %lld, %lld]", d.B, d.H, d.S);
+  EMI_FFI_STREAM()
+  return f.from_status(emi_attn_jvp(stream, q->data, k->data, v->data, static_cast<const float*>(lse->data), tq->data, tk->data,
+                                    tv->data, to->data, d.B, d.H, d.S, d.D, d.sb, d.sh, d.ss, (float)scale, (int)causal, q->dtype));
+}
+
 namespace {
 // q / o / dO / dq: [B, h, d]; caches and their cotangents: [B, S, h, d] (rows of one token contiguous).
 struct StepDims {
@@ -435,6 +484,7 @@ const Target kTargets[] = {
     {"emi_add", emi_add_ffi},                 {"emi_gemm", emi_gemm_ffi},
     {"emi_attn_fwd", emi_attn_fwd_ffi},       {"emi_attn_bwd", emi_attn_bwd_ffi},
     {"emi_attn_step_fwd", emi_attn_step_fwd_ffi}, {"emi_attn_step_bwd", emi_attn_step_bwd_ffi},
+    {"emi_rmsnorm_jvp", emi_rmsnorm_jvp_ffi}, {"emi_swiglu_jvp", emi_swiglu_jvp_ffi}, {"emi_attn_jvp", emi_attn_jvp_ffi},
     {"emi_embedding_fwd", emi_embedding_fwd_ffi}, {"emi_embedding_bwd", emi_embedding_bwd_ffi},
 };
 constexpr int kNumTargets = sizeof(kTargets) / sizeof(kTargets[0]);

@@ -34,6 +34,12 @@ FFI_TARGETS = {
     "embedding": ("emi_embedding_fwd", ("emi_embedding_bwd",)),
 }
 
+# operator -> tangent target(s); linear operators push tangents through their forward target
+FFI_TANGENT_TARGETS = {
+    "rmsnorm": ("emi_rmsnorm_jvp",), "rope": ("emi_rope",), "matmul_nt": ("emi_gemm", "emi_gemm"),
+    "swiglu": ("emi_swiglu_jvp",), "attention": ("emi_attn_jvp",), "add": ("emi_add",), "embedding": ("emi_embedding_fwd",),
+}
+
 _DTYPES = {torch.float32: N.EMI_F32, torch.bfloat16: N.EMI_BF16}
 
 
@@ -126,6 +132,62 @@ class Tape:
         return [ct.get(id(w)) for w in wrt]
 
 
+class Forward:
+    """Forward mode: tangents travel with the primal values.  While a Forward context is
+    active every operator also computes the tangent of its result from the tangents of
+    its operands (None = zero) with the forward kernels; linear operators reuse their own
+    kernel on the tangent."""
+
+    _active = None
+
+    def __init__(self):
+        self.tan = {}            # id(primal tensor) -> tangent tensor
+        self.keep = []           # primal tensors kept alive so that ids stay unique
+
+    def __enter__(self):
+        self._prev = Forward._active
+        Forward._active = self
+        return self
+
+    def __exit__(self, *exc):
+        Forward._active = self._prev
+        return False
+
+    def seed(self, primal, tangent):
+        if tangent is None:
+            return
+        if tangent.shape != primal.shape or tangent.dtype != primal.dtype:
+            raise ValueError("tangent %s/%s does not match primal %s/%s" %
+                             (tuple(tangent.shape), tangent.dtype, tuple(primal.shape), primal.dtype))
+        self.tan[id(primal)] = tangent
+        self.keep.append(primal)
+
+    def get(self, primal):
+        return self.tan.get(id(primal))
+
+
+def _tan(*ts):
+    """Tangents of the operands (None each without an active Forward context)."""
+    f = Forward._active
+    return None if f is None else tuple(None if t is None else f.get(t) for t in ts)
+
+
+def _quiet(fn):
+    """Runs fn() without recording on the tape and without tangent propagation: used for
+    the kernel calls that compute a tangent."""
+    tape, fwd = Tape._active, Forward._active
+    Tape._active, Forward._active = None, None
+    try:
+        return fn()
+    finally:
+        Tape._active, Forward._active = tape, fwd
+
+
+def _set_tan(y, t):
+    if t is not None:
+        Forward._active.seed(y, t)
+
+
 def _accumulate(acc, g):
     return g if acc is None else add(acc, g)
 
@@ -143,6 +205,10 @@ def add(a, b):
     y = torch.empty_like(a)
     N.check(N.lib().emi_add(_stream(), _p(a), _p(b), _p(y), a.numel(), _code(a)))
     Tape.record((a, b), y, lambda c, acc: (_accumulate(acc[0], c), _accumulate(acc[1], c)))
+    tans = _tan(a, b)
+    if tans is not None and (tans[0] is not None or tans[1] is not None):
+        ta, tb = tans
+        _set_tan(y, tb if ta is None else ta if tb is None else _quiet(lambda: add(ta, tb)))
     return y
 
 
@@ -167,6 +233,11 @@ def rmsnorm(x, gamma, eps=1e-5):
         return dx, _accumulate(acc[1], dgamma)
 
     Tape.record((x, gamma), y, rule)
+    tans = _tan(x, gamma)
+    if tans is not None and (tans[0] is not None or tans[1] is not None):
+        ty = torch.empty_like(x)
+        N.check(N.lib().emi_rmsnorm_jvp(_stream(), _p(x), _p(gamma), _p(tans[0]), _p(tans[1]), _p(ty), rows, D, eps, _code(x)))
+        _set_tan(y, ty)
     return y
 
 
@@ -204,6 +275,10 @@ def rope(x, n_heads, theta=10000.0, pos0=0, inverse=False):
         return (_accumulate(acc[0], g),)
 
     Tape.record((x,), y, rule)
+    tans = _tan(x)
+    if tans is not None and tans[0] is not None:
+        tx = tans[0]
+        _set_tan(y, _quiet(lambda: rope(tx, n_heads, theta, pos0, inverse)))     # linear in x
     return y
 
 
@@ -282,6 +357,15 @@ def matmul_nt(x, w, residual=None):
         return out
 
     Tape.record((x, w) if residual is None else (x, w, residual), y, rule)
+    tans = _tan(x, w, residual)
+    if tans is not None and any(t is not None for t in tans):
+        tx, tw, tr = tans                                   # ty = tx W^T + x tW^T + tr
+        t = None if tr is None else tr.reshape(-1, Nout)
+        if tx is not None:
+            t = gemm(tx.reshape(-1, K), w, False, True, t)
+        if tw is not None:
+            t = gemm(x2, tw, False, True, t)
+        _set_tan(y, t.reshape(*lead, Nout))
     return y
 
 
@@ -300,6 +384,11 @@ def swiglu(a, b):
         return _accumulate(acc[0], da), _accumulate(acc[1], db)
 
     Tape.record((a, b), g, rule)
+    tans = _tan(a, b)
+    if tans is not None and (tans[0] is not None or tans[1] is not None):
+        tg = torch.empty_like(a)
+        N.check(N.lib().emi_swiglu_jvp(_stream(), _p(a), _p(b), _p(tans[0]), _p(tans[1]), _p(tg), a.numel(), _code(a)))
+        _set_tan(g, tg)
     return g
 
 
@@ -341,6 +430,12 @@ def attention(q, k, v, n_heads, scale=None, causal=True, layout="bshd"):
         return _accumulate(acc[0], dq), _accumulate(acc[1], dk), _accumulate(acc[2], dv)
 
     Tape.record((q, k, v), o, rule)
+    tans = _tan(q, k, v)
+    if tans is not None and any(t is not None for t in tans):
+        to = torch.empty_like(q)
+        N.check(N.lib().emi_attn_jvp(_stream(), _p(q), _p(k), _p(v), _p(lse), _p(tans[0]), _p(tans[1]), _p(tans[2]), _p(to),
+                                     B, n_heads, S, d, sb, sh, ss, float(scale), int(causal), _code(q)))
+        _set_tan(o, to)
     return o
 
 
@@ -349,6 +444,9 @@ def reshape(x, shape):
     reshaped back)."""
     y = x.reshape(shape)
     Tape.record((x,), y, lambda c, acc: (_accumulate(acc[0], c.reshape(x.shape)),))
+    tans = _tan(x)
+    if tans is not None and tans[0] is not None:
+        _set_tan(y, tans[0].reshape(shape))
     return y
 
 
@@ -367,6 +465,11 @@ def append_row(cache, row):
         return _accumulate(acc[0], c[:n].contiguous()), _accumulate(acc[1], c[n].contiguous())
 
     Tape.record((cache, row), out, rule)
+    tans = _tan(cache, row)
+    if tans is not None and (tans[0] is not None or tans[1] is not None):
+        tc = torch.zeros_like(cache) if tans[0] is None else tans[0]
+        tr = torch.zeros_like(row) if tans[1] is None else tans[1]
+        _set_tan(out, torch.cat([tc, tr[None, :]], dim=0))
     return out
 
 
@@ -400,6 +503,9 @@ def attention_step(q, k_cache, v_cache, n_heads, scale=None):
         return _accumulate(acc[0], dq), _accumulate(acc[1], dk), _accumulate(acc[2], dv)
 
     Tape.record((q, k_cache, v_cache), o, rule)
+    tans = _tan(q, k_cache, v_cache)
+    if tans is not None and any(t is not None for t in tans):
+        raise NotImplementedError("attention_step has no forward-mode kernel")
     return o
 
 
@@ -421,6 +527,10 @@ def embedding(tokens, table):
         return None, _accumulate(acc[1], dt)
 
     Tape.record((tokens, table), x, rule)
+    tans = _tan(table)
+    if tans is not None and tans[0] is not None:
+        tt = tans[0]
+        _set_tan(x, _quiet(lambda: embedding(tokens, tt)))                 # linear in the table
     return x
 
 
@@ -441,4 +551,7 @@ def select(w, i):
         return (g,)
 
     Tape.record((w,), y, rule)
+    tans = _tan(w)
+    if tans is not None and tans[0] is not None:
+        _set_tan(y, tans[0][i])
     return y

@@ -296,9 +296,26 @@ def vjp(fn, *args):
 
 
 def jvp(fn, primals, tangents):
-    """Forward mode (reference: enzyme_jvp, primitives.py:1147-1245) is not
-    built for the HIP path yet."""
-    raise NotImplementedError("forward-mode (jvp) kernels are not implemented on the HIP path")
+    """(primals_out, tangents_out) like `jax.jvp` (reference: enzyme_jvp,
+    primitives.py:1147-1245): `tangents` mirrors `primals`; a None leaf (and every
+    integer leaf) is a zero tangent.  Results the tangents do not reach get zeros."""
+    p_leaves, p_def = tree_flatten(tuple(primals))
+    t_leaves, t_def = tree_flatten(tuple(tangents))
+    if len(p_leaves) != len(t_leaves):
+        raise ValueError("tangent tree has %d leaves, primal tree has %d" % (len(t_leaves), len(p_leaves)))
+    with ops.Forward() as fwd:
+        for p, t in zip(p_leaves, t_leaves):
+            if t is not None:
+                if not (isinstance(p, torch.Tensor) and p.is_floating_point()):
+                    raise TypeError("a tangent was given for a leaf that is not a floating-point tensor")
+                fwd.seed(p, t)
+        out = fn(*primals)
+        out_leaves, out_def = tree_flatten(out)
+        t_out = []
+        for o in out_leaves:
+            t = fwd.get(o) if isinstance(o, torch.Tensor) else None
+            t_out.append(t if t is not None else (torch.zeros_like(o) if isinstance(o, torch.Tensor) else None))
+    return out, tree_unflatten(out_def, t_out)
 
 
 def ffi_call(*args, out_shapes: Sequence[Any], source, fn: str = "f", argv=(), lang: int = LANG_CPP,

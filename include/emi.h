@@ -170,6 +170,24 @@ int emi_attn_step_bwd(emi_stream_t stream, const void* q, const void* k, const v
                       int64_t q_stride_h, int64_t kv_stride_b, int64_t kv_stride_h,
                       int64_t kv_stride_s, float scale, int dtype);
 
+/* Forward mode (tangents), the other half of the reference API (enzyme_jvp,
+ * src/enzyme_ad/jax/primitives.py:1147-1245).  Linear operators (emi_gemm, emi_rope,
+ * emi_add, emi_embedding_fwd) carry tangents through their own forward entry
+ * points; the three below are the nonlinear ones.  A null tangent pointer is a
+ * zero tangent.
+ *   rmsnorm:  ty = gamma (r tx - x r^3 mean(x tx)) + tgamma x r
+ *   swiglu:   tg = ta b s (1 + a (1 - s)) + tb a s,  s = sigmoid(a)
+ *   attention (strides and lse as emi_attn_fwd):
+ *             tS = scale (tq k^T + q tk^T), tP = P (tS - rowsum(P tS)), to = tP v + P tv */
+int emi_rmsnorm_jvp(emi_stream_t stream, const void* x, const void* gamma, const void* tx,
+                    const void* tgamma, void* ty, int64_t rows, int64_t dim, float eps, int dtype);
+int emi_swiglu_jvp(emi_stream_t stream, const void* a, const void* b, const void* ta,
+                   const void* tb, void* tg, int64_t n, int dtype);
+int emi_attn_jvp(emi_stream_t stream, const void* q, const void* k, const void* v, const float* lse,
+                 const void* tq, const void* tk, const void* tv, void* to, int64_t batch,
+                 int64_t heads, int64_t seq, int64_t head_dim, int64_t stride_b, int64_t stride_h,
+                 int64_t stride_s, float scale, int causal, int dtype);
+
 /* Embedding gather x[t,:] = table[tokens[t],:] and its adjoint (scatter-add of
  * dx rows into a zero-initialised dtable; fp32 accumulation in workspace when
  * dtype is bf16).  The lookup is commented out in the reference

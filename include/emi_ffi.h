@@ -28,6 +28,9 @@
  *  emi_attn_bwd       q, k, v, o, lse, do              dq, dk, dv, workspace:u8[n]       scale:f32, causal:pred, bshd:pred
  *  emi_attn_step_fwd  q[B,h,d], k, v [B,S,h,d]         o[B,h,d], lse f32[B,h], workspace:u8[n]  scale:f32
  *  emi_attn_step_bwd  q, k, v, o, lse, do              dq, dk, dv, workspace:u8[n]       scale:f32
+ *  emi_rmsnorm_jvp    x, gamma, tx, tgamma             ty                                eps:f32
+ *  emi_swiglu_jvp     a, b, ta, tb                     tg                                -
+ *  emi_attn_jvp       q, k, v, lse, tq, tk, tv         to                                scale:f32, causal:pred, bshd:pred
  *  emi_embedding_fwd  tokens s32[..], table[V,D]       x[..,D]                           -
  *  emi_embedding_bwd  tokens s32[..], dx[..,D]         dtable[V,D] [, workspace:u8[n]]   -
  *
@@ -58,6 +61,9 @@ struct XLA_FFI_Error* emi_attn_fwd_ffi(struct XLA_FFI_CallFrame*);
 struct XLA_FFI_Error* emi_attn_bwd_ffi(struct XLA_FFI_CallFrame*);
 struct XLA_FFI_Error* emi_attn_step_fwd_ffi(struct XLA_FFI_CallFrame*);
 struct XLA_FFI_Error* emi_attn_step_bwd_ffi(struct XLA_FFI_CallFrame*);
+struct XLA_FFI_Error* emi_rmsnorm_jvp_ffi(struct XLA_FFI_CallFrame*);
+struct XLA_FFI_Error* emi_swiglu_jvp_ffi(struct XLA_FFI_CallFrame*);
+struct XLA_FFI_Error* emi_attn_jvp_ffi(struct XLA_FFI_CallFrame*);
 struct XLA_FFI_Error* emi_embedding_fwd_ffi(struct XLA_FFI_CallFrame*);
 struct XLA_FFI_Error* emi_embedding_bwd_ffi(struct XLA_FFI_CallFrame*);
 

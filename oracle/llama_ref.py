@@ -431,6 +431,81 @@ def model_bwd(dout, weights, config, fcache, eps=EPS):
 # 5. Seeded synthetic inputs for the benchmark configurations
 # ---------------------------------------------------------------------------
 
+# ---------------------------------------------------------------------------
+# 5. Forward mode (tangents): what `jax.jvp` of the same program computes
+#    (reference: enzyme_jvp, src/enzyme_ad/jax/primitives.py:1147-1245).  Pinned by
+#    <J v, w> = <v, J^T w> against the reverse-mode functions above and by central
+#    finite differences (tests/test_oracle_llama.py).
+# ---------------------------------------------------------------------------
+
+def rmsnorm_jvp(x, gamma, tx, tgamma, eps=EPS):
+    """ty = gamma (r tx - x r^3 mean(x tx)) + tgamma x r."""
+    r = 1.0 / np.sqrt(np.mean(x * x, axis=-1, keepdims=True) + eps)
+    return gamma * (r * tx - x * r ** 3 * np.mean(x * tx, axis=-1, keepdims=True)) + tgamma * x * r
+
+
+def linear_jvp(x, w, tx, tw):
+    return tx @ w.T + x @ tw.T
+
+
+def swiglu_jvp(a, b, ta, tb):
+    s = 1.0 / (1.0 + np.exp(-a))
+    return ta * b * s * (1.0 + a * (1.0 - s)) + tb * a * s
+
+
+def attention_jvp(q, k, v, tq, tk, tv, scale=None, causal=True):
+    """tS = scale (tq k^T + q tk^T); tP = P (tS - rowsum(P tS)); to = tP v + P tv."""
+    B, h, S, d = q.shape
+    if scale is None:
+        scale = 1.0 / np.sqrt(d)
+    s = np.einsum("bhqd,bhkd->bhqk", q, k) * scale
+    if causal:
+        mask = np.tril(np.ones((S, k.shape[2]), dtype=bool), k=k.shape[2] - S)
+        s = np.where(mask, s, -np.inf)
+    p = np.exp(s - np.max(s, axis=-1, keepdims=True))
+    p = p / np.sum(p, axis=-1, keepdims=True)
+    ts = (np.einsum("bhqd,bhkd->bhqk", tq, k) + np.einsum("bhqd,bhkd->bhqk", q, tk)) * scale
+    tp = p * (ts - np.sum(p * ts, axis=-1, keepdims=True))
+    return np.einsum("bhqk,bhkd->bhqd", tp, v) + np.einsum("bhqk,bhkd->bhqd", p, tv)
+
+
+def layer_jvp(x, lw, tx, tlw, n_heads, eps=EPS, theta=ROPE_THETA):
+    """Tangent of layer_fwd for tangents tx of x and tlw (same keys) of the weights."""
+    B, S, D = x.shape
+    d = D // n_heads
+    cos, sin = rope_angles(S, d, theta, 0, dtype=x.dtype)
+    tr = lambda t: _heads(t, n_heads).transpose(0, 2, 1, 3)
+    xb = rmsnorm_fwd(x, lw["rms_att_weight"], eps)
+    txb = rmsnorm_jvp(x, lw["rms_att_weight"], tx, tlw["rms_att_weight"], eps)
+    q, k, v = (linear_fwd(xb, lw[n]) for n in ("wq", "wk", "wv"))
+    tq, tk, tv = (linear_jvp(xb, lw[n], txb, tlw[n]) for n in ("wq", "wk", "wv"))
+    qr, kr = rope_fwd(_heads(q, n_heads), cos, sin), rope_fwd(_heads(k, n_heads), cos, sin)
+    tqr, tkr = rope_fwd(_heads(tq, n_heads), cos, sin), rope_fwd(_heads(tk, n_heads), cos, sin)     # linear
+    o, _ = attention_fwd(qr.transpose(0, 2, 1, 3), kr.transpose(0, 2, 1, 3), tr(v), 1.0 / np.sqrt(d), True)
+    to = attention_jvp(qr.transpose(0, 2, 1, 3), kr.transpose(0, 2, 1, 3), tr(v), tqr.transpose(0, 2, 1, 3),
+                       tkr.transpose(0, 2, 1, 3), tr(tv), 1.0 / np.sqrt(d), True)
+    att, tatt = o.transpose(0, 2, 1, 3).reshape(B, S, D), to.transpose(0, 2, 1, 3).reshape(B, S, D)
+    x1 = x + linear_fwd(att, lw["wo"])
+    tx1 = tx + linear_jvp(att, lw["wo"], tatt, tlw["wo"])
+    xb2 = rmsnorm_fwd(x1, lw["rms_ffn_weight"], eps)
+    txb2 = rmsnorm_jvp(x1, lw["rms_ffn_weight"], tx1, tlw["rms_ffn_weight"], eps)
+    a1, a3 = linear_fwd(xb2, lw["w1"]), linear_fwd(xb2, lw["w3"])
+    ta1, ta3 = linear_jvp(xb2, lw["w1"], txb2, tlw["w1"]), linear_jvp(xb2, lw["w3"], txb2, tlw["w3"])
+    g, tg = swiglu_fwd(a1, a3), swiglu_jvp(a1, a3, ta1, ta3)
+    y = x1 + linear_fwd(g, lw["w2"])
+    ty = tx1 + linear_jvp(g, lw["w2"], tg, tlw["w2"])
+    return y, ty
+
+
+def model_jvp(x, weights, tx, tweights, config, eps=EPS, theta=ROPE_THETA):
+    """Tangent of model_fwd (activations in, final RMSNorm out) for tangents of x and of every weight."""
+    t = tx
+    for i in range(config["n_layers"]):
+        x, t = layer_jvp(x, _layer_weights(weights, i), t, _layer_weights(tweights, i), config["n_heads"], eps, theta)
+    return (rmsnorm_fwd(x, weights["rms_final_weight"], eps),
+            rmsnorm_jvp(x, weights["rms_final_weight"], t, tweights["rms_final_weight"], eps))
+
+
 def forward_step_vjp(x, config, weights, key_cache, value_cache, dy, eps=EPS, theta=ROPE_THETA):
     """Reverse of `forward_step` (the program `jax.vjp` of test/llama.py:35-238 computes):
     cotangents of x, of every weight and of both caches for the output cotangent dy.

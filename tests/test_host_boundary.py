@@ -94,6 +94,10 @@ def test_ffi_metadata_probe_and_stages():
     ("emi_attn_step_bwd_ffi", [(F.F32, [1, 6, 48]), (F.F32, [1, 9, 6, 48]), (F.F32, [1, 9, 6, 48]), (F.F32, [1, 6, 48]),
                                (F.F32, [1, 7]), (F.F32, [1, 6, 48])],
      [(F.F32, [1, 6, 48]), (F.F32, [1, 9, 6, 48]), (F.F32, [1, 9, 6, 48]), (F.U8, [4096])], {"scale": (F.F32, 0.1)}, "lse"),
+    ("emi_rmsnorm_jvp_ffi", [(F.F32, [4, 8]), (F.F32, [8]), (F.F32, [4, 8]), (F.F32, [7])], [(F.F32, [4, 8])],
+     {"eps": (F.F32, 1e-5)}, "tgamma"),
+    ("emi_attn_jvp_ffi", [(F.BF16, [1, 2, 64, 128])] * 3 + [(F.F32, [1, 2, 64])] + [(F.BF16, [1, 2, 64, 128])] * 3,
+     [(F.BF16, [1, 2, 64, 128])], {"causal": (F.PRED, 1)}, "scale"),
     ("emi_embedding_fwd_ffi", [(F.S64, [3]), (F.F32, [10, 4])], [(F.F32, [3, 4])], {}, "s32"),
     ("emi_swiglu_bwd_ffi", [(F.F32, [8])] * 3, [(F.F32, [8]), (F.F32, [9])], {}, "shape"),
 ])
@@ -121,9 +125,10 @@ def test_ffi_registration_lists_all_targets_for_rocm():
     lib.emi_ffi_target_handler.restype = C.c_void_p
     n = lib.emi_ffi_target_count()
     names = [lib.emi_ffi_target_name(i).decode() for i in range(n)]
-    assert n == 14 and "emi_attn_bwd" in names and "emi_attn_step_bwd" in names and all(lib.emi_ffi_target_handler(i) for i in range(n))
+    assert n == 17 and "emi_attn_bwd" in names and "emi_attn_step_bwd" in names and "emi_attn_jvp" in names and all(lib.emi_ffi_target_handler(i) for i in range(n))
     from enzyme_ad.jax import ops
     used = {t for fwd, bwd in ops.FFI_TARGETS.values() for t in (fwd,) + tuple(bwd)}
+    used |= {t for ts in ops.FFI_TANGENT_TARGETS.values() for t in ts}
     assert used <= set(names)                                 # every target the lowering table names has a handler
     xla = F.FakeXla()
     lib.emi_register_ffi.argtypes = [C.POINTER(F.Api)]
@@ -158,10 +163,13 @@ def test_python_surface_matches_reference_names():
         ej.enzyme_jax_ir(pipeline_options="not a pipeline")(lambda x: x)
     f = ej.enzyme_jax_ir(argv=("-O3",), pipeline_options=ej.JaXPipeline(), jit_options={"print_mlir": False}, inner_jit=False)(lambda x: x)
     assert f(3) == 3 and f.argv == ("-O3",)
-    for call in (lambda: ej.cpp_call(out_shapes=[], source="void f(){}"), lambda: ej.hlo_call(source="module {}"),
-                 lambda: ej.jvp(f, (1,), (1,))):
+    for call in (lambda: ej.cpp_call(out_shapes=[], source="void f(){}"), lambda: ej.hlo_call(source="module {}")):
         with pytest.raises(NotImplementedError):
             call()
+    with pytest.raises(TypeError):                      # a tangent for a leaf that is not a floating-point tensor
+        ej.jvp(f, (1,), (1,))
+    out, tangent = ej.jvp(f, (3,), (None,))             # jax.jvp shape of the result: (primals_out, tangents_out)
+    assert out == 3 and tangent is None
 
 
 def test_operators_refuse_host_tensors():

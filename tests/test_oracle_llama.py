@@ -223,3 +223,26 @@ def test_step_vjp_matches_literal_step_and_finite_differences(pos):
     for idx in [tuple(picks.integers(0, n) for n in kc.shape) for _ in range(4)]:
         np.testing.assert_allclose(dkc[idx], fd(kc, idx, lambda a: dict(kk=a)), rtol=2e-5, atol=1e-7)
         np.testing.assert_allclose(dvc[idx], fd(vc, idx, lambda a: dict(vv=a)), rtol=2e-5, atol=1e-7)
+
+
+def test_forward_mode_matches_reverse_mode_and_finite_differences():
+    """`model_jvp`: <J v, w> = <v, J^T w> against `model_bwd` for random tangents of the input
+    and every weight, and J v = central finite difference of `model_fwd` along v (float64)."""
+    cfg, B, S = CFG, 2, 5
+    w = _weights(cfg, 13)
+    rng = np.random.default_rng(17)
+    x = rng.standard_normal((B, S, cfg["dim"]))
+    tx = rng.standard_normal(x.shape)
+    tw = {k: rng.standard_normal(np.shape(v)) for k, v in w.items()}
+    wvec = rng.standard_normal(x.shape)                       # cotangent on the output
+    y, ty = L.model_jvp(x, w, tx, tw, cfg)
+    y2, fc = L.model_fwd(x, w, cfg)
+    np.testing.assert_allclose(y, y2, rtol=1e-12, atol=1e-13)
+    gx, gw = L.model_bwd(wvec, w, cfg, fc)
+    lhs = float(np.sum(ty * wvec))
+    rhs = float(np.sum(gx * tx)) + sum(float(np.sum(gw[k] * tw[k])) for k in gw)
+    np.testing.assert_allclose(lhs, rhs, rtol=1e-9)
+    h = 1e-6
+    up, _ = L.model_fwd(x + h * tx, {k: w[k] + h * tw[k] for k in w}, cfg)
+    dn, _ = L.model_fwd(x - h * tx, {k: w[k] - h * tw[k] for k in w}, cfg)
+    np.testing.assert_allclose(ty, (up - dn) / (2 * h), rtol=2e-5, atol=1e-6)
