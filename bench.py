@@ -184,11 +184,9 @@ def bench_kernels(cfg, iters):
                                                             h * S * d, S * d, d, sc, 1, N.EMI_BF16)), fl)
     mfma("attn_bwd_c3", lambda: N.check(lib.emi_attn_bwd(st, P(q), P(k), P(v), P(o), P(lse), P(do), P(dq), P(dk), P(dv), P(ws), wsb,
                                                          B, h, S, d, h * S * d, S * d, d, sc, 1, N.EMI_BF16)), 2.5 * fl)
-    # forward mode: tangent of the same attention on a quarter of the heads (one-wavefront-per-row kernel),
-    # counted like the adjoint at 2.5x the forward flops (5 matmuls)
-    hj = h // 4
-    mfma("attn_jvp_c3_quarter", lambda: N.check(lib.emi_attn_jvp(st, P(q), P(k), P(v), P(lse), P(do), P(dq), P(dk), P(dv), B, hj, S, d,
-                                                                 h * S * d, S * d, d, sc, 1, N.EMI_BF16)), 2.5 * fl * hj / h)
+    # forward mode: tangent of the same attention, counted like the adjoint at 2.5x the forward flops
+    mfma("attn_jvp_c3", lambda: N.check(lib.emi_attn_jvp(st, P(q), P(k), P(v), P(lse), P(do), P(dq), P(dk), P(dv), B, h, S, d,
+                                                         h * S * d, S * d, d, sc, 1, N.EMI_BF16)), 2.5 * fl)
     del q, k, v, do, o, dq, dk, dv, ws, fws
     # Single-token (decode) step at the 7B layer's widths: mat-vec over W [11008, 4096] and its
     # adjoints (weight read or written once), attention of one query per head over a

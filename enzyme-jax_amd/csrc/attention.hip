@@ -1312,6 +1312,155 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_sp_kernel(const uint16_t* __
 }
 
 // ---------------------------------------------------------------------------
+// Forward mode (tangent) of attention on the matrix cores; same transposed formulation as
+// the forward kernel (lane = query).  Per 64-key tile and 32-key half:
+//   S^T = K Q^T,  tS^T = K tQ^T + tK Q^T,  p = exp2(S c - lse2),  w = p tS scale
+//   A_w^T += V^T w^T,  A_o^T += V^T p^T,  A_t^T += tV^T p^T,  mu += sum_keys w
+// and finally  to = A_w - mu A_o + A_t  (tP = P (tS - rowsum(P tS)), to = tP V + P tV).
+// Block = 4 wavefronts x 32 queries, one wavefront per SIMD (three output accumulators);
+// K, V, tK, tV tiles double-buffered in LDS.  A null tangent is zero and its products are
+// skipped (block-uniform branches).
+// ---------------------------------------------------------------------------
+template <int D>
+__global__ __launch_bounds__(256) void attn_jvp_bf16_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ k,
+                                                            const uint16_t* __restrict__ v, const float* __restrict__ lse,
+                                                            const uint16_t* __restrict__ tq, const uint16_t* __restrict__ tk,
+                                                            const uint16_t* __restrict__ tv, uint16_t* __restrict__ to,
+                                                            AttnShape sh, uint32_t head_bytes, float scale, int causal) {
+  constexpr int BQ = 128, BKV = 64, NW = 4;
+  constexpr int TILE = BKV * D * 2, STAGE = 4 * TILE;       // K, V, tK, tV
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem_raw[];
+  EMI_LDS uint8_t* smem = (EMI_LDS uint8_t*)smem_raw;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  int blk, bh;
+  attn_block_coords(&blk, &bh);
+  const int qblk = gridDim.x - 1 - blk;              // longest rows first
+  const int64_t base = (int64_t)(bh / sh.heads) * sh.sb + (int64_t)(bh % sh.heads) * sh.sh;
+  const int seq = sh.seq;
+  const int q0 = qblk * BQ + wave * 32;
+  const int qrow = q0 + (lane & 31);
+  const float scale_log2e = scale * kLog2e;
+  const bool has_tq = tq != nullptr, has_tk = tk != nullptr, has_tv = tv != nullptr;
+
+  bf16x8_t qf[D / 16], tqf[D / 16];
+  load_reg_rows<D>(q + base, qrow, seq, sh.ss, lane, qf);
+  if (has_tq) load_reg_rows<D>(tq + base, qrow, seq, sh.ss, lane, tqf);
+  const float L2 = qrow < seq ? lse[(int64_t)bh * seq + qrow] * kLog2e : 0.f;
+
+  const __amdgpu_buffer_rsrc_t rK = attn_rsrc(k + base, head_bytes);
+  const __amdgpu_buffer_rsrc_t rV = attn_rsrc(v + base, head_bytes);
+  const __amdgpu_buffer_rsrc_t rTK = attn_rsrc(has_tk ? tk + base : k + base, head_bytes);
+  const __amdgpu_buffer_rsrc_t rTV = attn_rsrc(has_tv ? tv + base : v + base, head_bytes);
+  const int kv_end = causal ? (qblk * BQ + BQ < seq ? qblk * BQ + BQ : seq) : seq;
+  const int nkv = (kv_end + BKV - 1) / BKV;
+
+  f32x16_t acc_w[D / 32], acc_o[D / 32], acc_t[D / 32];
+#pragma unroll
+  for (int dt = 0; dt < D / 32; dt++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc_w[dt][r] = 0.f, acc_o[dt][r] = 0.f, acc_t[dt][r] = 0.f;
+  float mu = 0.f;
+
+  auto issue = [&](int j, EMI_LDS uint8_t* dst) __attribute__((always_inline)) {
+    load_rows_tile<D, BKV, NW>(rK, dst, wave, lane, j * BKV, seq, sh.ss);
+    load_rows_tile<D, BKV, NW>(rV, dst + TILE, wave, lane, j * BKV, seq, sh.ss);
+    if (has_tk) load_rows_tile<D, BKV, NW>(rTK, dst + 2 * TILE, wave, lane, j * BKV, seq, sh.ss);
+    if (has_tv) load_rows_tile<D, BKV, NW>(rTV, dst + 3 * TILE, wave, lane, j * BKV, seq, sh.ss);
+  };
+  issue(0, smem);
+  __builtin_amdgcn_s_waitcnt(0x0f70);
+  __syncthreads();
+
+  for (int j = 0; j < nkv; j++) {
+    if (j + 1 < nkv) issue(j + 1, smem + ((j + 1) & 1) * STAGE);
+    const EMI_LDS uint8_t* sK = smem + (j & 1) * STAGE;
+    const EMI_LDS uint8_t* sV = sK + TILE;
+    const EMI_LDS uint8_t* sTK = sK + 2 * TILE;
+    const EMI_LDS uint8_t* sTV = sK + 3 * TILE;
+    const int key0 = j * BKV;
+    if (!(causal && key0 > q0 + 31)) {     // wave-uniform: this tile is not entirely in the future
+      const bool need_mask = (causal && key0 + BKV - 1 > q0) || key0 + BKV > seq;
+#pragma unroll 1
+      for (int T = 0; T < 2; T++) {
+        f32x16_t s, ts;
+#pragma unroll
+        for (int r = 0; r < 16; r++) s[r] = 0.f, ts[r] = 0.f;
+#pragma unroll
+        for (int t = 0; t < D / 16; t++) {
+          const bf16x8_t kf = row_frag<D>(sK, T * 32, t, lane);
+          s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[t], s, 0, 0, 0);
+          if (has_tq) ts = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, tqf[t], ts, 0, 0, 0);
+        }
+        if (has_tk) {
+#pragma unroll
+          for (int t = 0; t < D / 16; t++)
+            ts = __builtin_amdgcn_mfma_f32_32x32x16_bf16(row_frag<D>(sTK, T * 32, t, lane), qf[t], ts, 0, 0, 0);
+        }
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          float p = fast_exp2(fmaf(s[r], scale_log2e, -L2));
+          if (need_mask) {
+            const int key = key0 + T * 32 + acc_row(r, lane);
+            if ((causal && key > qrow) || key >= seq) p = 0.f;
+          }
+          const float w = p * ts[r] * scale;
+          mu += w;
+          s[r] = p;
+          ts[r] = w;
+        }
+#pragma unroll
+        for (int sI = 0; sI < 2; sI++) {
+          const bf16x8_t pf = acc_to_frag(s, sI), wf = acc_to_frag(ts, sI);
+#pragma unroll
+          for (int dt = 0; dt < D / 32; dt++) {
+            const bf16x8_t vt = col_frag<D>(sV, T * 32 + sI * 16, dt * 32, lane);
+            acc_o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vt, pf, acc_o[dt], 0, 0, 0);
+            if (has_tq || has_tk) acc_w[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vt, wf, acc_w[dt], 0, 0, 0);
+          }
+          if (has_tv) {
+#pragma unroll
+            for (int dt = 0; dt < D / 32; dt++)
+              acc_t[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(col_frag<D>(sTV, T * 32 + sI * 16, dt * 32, lane), pf,
+                                                                  acc_t[dt], 0, 0, 0);
+          }
+        }
+      }
+    }
+    __builtin_amdgcn_s_waitcnt(0x0f70);
+    __syncthreads();
+  }
+
+  // a lane pair (l, l ^ 32) holds the two halves of a query's keys
+  mu += __shfl_xor(mu, 32, 64);
+  {
+    constexpr int CH = D / 8, RB = D * 2;
+    EMI_LDS uint8_t* wl = smem + wave * (32 * RB);
+    const int r = lane & 31, g = lane >> 5;
+#pragma unroll
+    for (int dt = 0; dt < D / 32; dt++)
+#pragma unroll
+      for (int jj = 0; jj < 4; jj++) {
+        float o4[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) o4[e] = acc_w[dt][4 * jj + e] - mu * acc_o[dt][4 * jj + e] + acc_t[dt][4 * jj + e];
+        u32x2_t w;
+        w[0] = pack_bf16x2(o4[0], o4[1]);
+        w[1] = pack_bf16x2(o4[2], o4[3]);
+        const int c = dt * 4 + jj;
+        *reinterpret_cast<EMI_LDS u32x2_t*>(wl + r * RB + ((c ^ (r & (CH - 1))) << 4) + ((g ^ ((r / CH) & 1)) << 3)) = w;
+      }
+#pragma unroll
+    for (int it = 0; it < 32 * CH / 64; it++) {
+      const int row = it * (64 / CH) + lane / CH, c = lane % CH;
+      u32x4_t v4 = *reinterpret_cast<const EMI_LDS u32x4_t*>(wl + row * RB + ((c ^ (row & (CH - 1))) << 4));
+      if ((row / CH) & 1) v4 = __builtin_shufflevector(v4, v4, 2, 3, 0, 1);
+      if (q0 + row < seq) *reinterpret_cast<u32x4_t*>(to + base + (int64_t)(q0 + row) * sh.ss + c * 8) = v4;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
 
@@ -1345,6 +1494,31 @@ static bool mfma_ok(const AttnArgs& a, int dtype, std::initializer_list<const vo
 template <typename K> static int reserve_lds(K kern, int bytes, const char* name) {
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
   if (e != hipSuccess) return emi_fail(EMI_INTERNAL, "%s: cannot reserve %d bytes of LDS: %s", name, bytes, hipGetErrorString(e));
+  return EMI_OK;
+}
+
+// Tangent of attention on the MFMA path; -1 when the operands do not qualify (the caller
+// then takes the one-wavefront-per-row kernel).
+int launch_attn_jvp_mfma(hipStream_t st, const void* q, const void* k, const void* v, const float* lse, const void* tq,
+                         const void* tk, const void* tv, void* to, int64_t batch, int64_t heads, int64_t seq, int64_t head_dim,
+                         int64_t sb, int64_t shh, int64_t ss, float scale, int causal, int dtype) {
+  const AttnArgs a{batch, heads, seq, head_dim, sb, shh, ss};
+  if (!mfma_ok(a, dtype, {q, k, v, to, tq ? tq : q, tk ? tk : k, tv ? tv : v}) || seq < 128 || batch * heads > 65535) return -1;
+  const AttnShape shp{(int)seq, (int)heads, sb, shh, ss};
+  const uint32_t head_bytes = (uint32_t)(((seq - 1) * ss + head_dim) * 2);
+  const dim3 grid((unsigned)((seq + 127) / 128), (unsigned)(batch * heads));
+#define EMI_ATTN_JVP(DD)                                                                                                 \
+  do {                                                                                                                   \
+    constexpr int smem = 2 * 4 * 64 * DD * 2;                                                                            \
+    if (int rc = reserve_lds(attn_jvp_bf16_kernel<DD>, smem, "emi_attn_jvp")) return rc;                                 \
+    hipLaunchKernelGGL(attn_jvp_bf16_kernel<DD>, grid, dim3(256), smem, st, (const uint16_t*)q, (const uint16_t*)k,      \
+                       (const uint16_t*)v, lse, (const uint16_t*)tq, (const uint16_t*)tk, (const uint16_t*)tv,           \
+                       (uint16_t*)to, shp, head_bytes, scale, causal);                                                   \
+  } while (0)
+  if (head_dim == 128) EMI_ATTN_JVP(128);
+  else EMI_ATTN_JVP(64);
+#undef EMI_ATTN_JVP
+  EMI_CHECK_LAUNCH("emi_attn_jvp");
   return EMI_OK;
 }
 

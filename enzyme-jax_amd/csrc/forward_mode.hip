@@ -178,6 +178,11 @@ __global__ __launch_bounds__(256) void attn_jvp_kernel(const T* __restrict__ q, 
 bool al16(const void* p) { return p == nullptr || (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 }  // namespace
+
+// attention.hip
+int launch_attn_jvp_mfma(hipStream_t st, const void* q, const void* k, const void* v, const float* lse, const void* tq,
+                         const void* tk, const void* tv, void* to, int64_t batch, int64_t heads, int64_t seq, int64_t head_dim,
+                         int64_t sb, int64_t shh, int64_t ss, float scale, int causal, int dtype);
 }  // namespace emi
 
 using namespace emi;
@@ -238,6 +243,11 @@ extern "C" int emi_attn_jvp(emi_stream_t stream, const void* q, const void* k, c
   if (batch == 0) return EMI_OK;
   EMI_REQUIRE(q && k && v && lse && to, "emi_attn_jvp: null buffer");
   hipStream_t st = static_cast<hipStream_t>(stream);
+  {
+    const int rc = launch_attn_jvp_mfma(st, q, k, v, lse, tq, tk, tv, to, batch, heads, seq, head_dim, stride_b, stride_h,
+                                        stride_s, scale, causal, dtype);
+    if (rc >= 0) return rc;
+  }
   const JvpShape sh{(int)seq, (int)heads, stride_b, stride_h, stride_s};
   const dim3 grid((unsigned)((seq + 3) / 4), (unsigned)(batch * heads));
   if (dtype == EMI_BF16)
