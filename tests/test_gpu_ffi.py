@@ -112,6 +112,26 @@ def test_ffi_handlers_launch_on_the_frame_stream():
         check(dq, rdq[:, :, 0, :], "bf16", "ffi step dq")
         check(dk, rdk.transpose(0, 2, 1, 3), "bf16", "ffi step dk")
         check(dv, rdv.transpose(0, 2, 1, 3), "bf16", "ffi step dv")
+        # forward-mode targets: tangents are ordinary operands
+        x4, x4r = dev(rng.standard_normal((6, 512)), "bf16")
+        g4, g4r = dev(rng.uniform(0.5, 1.5, 512), "bf16")
+        tx4, tx4r = dev(rng.standard_normal((6, 512)), "bf16")
+        tg4, tg4r = dev(rng.standard_normal(512), "bf16")
+        ty4 = torch.empty_like(x4)
+        _call("emi_rmsnorm_jvp_ffi", xla, [_buf(xla, t) for t in (x4, g4, tx4, tg4)], [_buf(xla, ty4)], {"eps": (F.F32, 1e-5)})
+        check(ty4, L.rmsnorm_jvp(x4r, g4r, tx4r, tg4r), "bf16", "ffi rmsnorm tangent")
+        b4, b4r = dev(rng.standard_normal((6, 512)), "bf16")
+        tb4, tb4r = dev(rng.standard_normal((6, 512)), "bf16")
+        _call("emi_swiglu_jvp_ffi", xla, [_buf(xla, t) for t in (x4, b4, tx4, tb4)], [_buf(xla, ty4)], {})
+        check(ty4, L.swiglu_jvp(x4r, b4r, tx4r, tb4r), "bf16", "ffi swiglu tangent")
+        B, S, h, d = 1, 200, 2, 128
+        (q, qr), (k, kr), (v, vr), (tq, tqr), (tk, tkr), (tv, tvr) = (dev(rng.standard_normal((B, S, h, d)), "bf16") for _ in range(6))
+        o, to = torch.empty_like(q), torch.empty_like(q)
+        lse = torch.empty((B, h, S), dtype=torch.float32, device="cuda")
+        at = {"scale": (F.F32, d ** -0.5), "causal": (F.PRED, 1), "bshd": (F.PRED, 1)}
+        _call("emi_attn_fwd_ffi", xla, [_buf(xla, q), _buf(xla, k), _buf(xla, v)], [_buf(xla, o), _buf(xla, lse)], at)
+        _call("emi_attn_jvp_ffi", xla, [_buf(xla, t) for t in (q, k, v, lse, tq, tk, tv)], [_buf(xla, to)], at)
+        check(tr(host(to)), L.attention_jvp(tr(qr), tr(kr), tr(vr), tr(tqr), tr(tkr), tr(tvr)), "bf16", "ffi attention tangent")
         # swiglu, add, embedding
         a, ar = dev(rng.standard_normal(1000), "f32")
         b, br = dev(rng.standard_normal(1000), "f32")
