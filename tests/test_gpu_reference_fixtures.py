@@ -1,0 +1,110 @@
+"""The reference's small closed-form differentiation cases (test/bench_vs_xla.py:5-194) that
+can be written with the operators of the transformer path -- add, matrix product, reshape,
+row append -- run through `jvp` and `vjp` on the GPU and compared with answers worked out by
+hand from the inputs the reference's fixtures hold.  Sum, Cache and Slicing need elementwise
+products and broadcasts, which the path does not have; they are not covered."""
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import host
+
+pytestmark = pytest.mark.gpu
+
+
+def f32(a):
+    return torch.tensor(np.asarray(a, dtype=np.float32), device="cuda")
+
+
+def sq(lo, hi):
+    return sum(i * i for i in range(lo, hi))
+
+
+def test_add_two_inactive_argument():
+    """AddTwo (bench_vs_xla.py:32-52): f(x, z, y) = x + y; z gets a zero cotangent."""
+    from enzyme_ad.jax import enzyme_jax_ir, jvp, vjp, ops
+
+    @enzyme_jax_ir()
+    def add_two(x, z, y):
+        return ops.add(x, y)
+
+    ins = [f32([1, 2, 3]), f32([10, 20, 30]), f32([100, 200, 300])]
+    dins = [f32([0.1, 0.2, 0.3]), f32([50, 70, 110]), f32([1300, 1700, 1900])]
+    out, tan = jvp(add_two, ins, dins)
+    assert torch.equal(out, f32([101, 202, 303]))
+    np.testing.assert_allclose(host(tan), [1300.1, 1700.2, 1900.3], rtol=1e-7)
+    out, f_vjp = vjp(add_two, *ins)
+    gx, gz, gy = f_vjp(f32([500, 700, 110]))
+    assert torch.equal(gx, f32([500, 700, 110])) and torch.equal(gy, gx)
+    assert torch.equal(gz, torch.zeros_like(gz))
+
+
+def test_activity_mismatch():
+    """ActivityMismatch (bench_vs_xla.py:111-134): a constant row with an active row
+    appended; k = ones(12, 12) . x."""
+    from enzyme_ad.jax import enzyme_jax_ir, jvp, vjp, ops
+
+    dim = 12
+
+    @enzyme_jax_ir()
+    def f(x):
+        k = ops.matmul_nt(x, torch.ones(dim, dim, device="cuda"))
+        return ops.append_row(torch.zeros(1, dim, device="cuda"), k)
+
+    x = f32(range(dim))
+    dx = f32([i * i for i in range(dim)])
+    out, tan = jvp(f, (x,), (dx,))
+    assert out.shape == (2, dim)
+    assert torch.equal(out, f32([[0.0] * dim, [66.0] * dim]))
+    assert torch.equal(tan, f32([[0.0] * dim, [float(sq(0, dim))] * dim]))            # 506
+    out, f_vjp = vjp(f, x)
+    (gx,) = f_vjp(f32([i * i for i in range(2 * dim)]).reshape(2, dim))
+    assert torch.equal(gx, f32([float(sq(dim, 2 * dim))] * dim))                      # 3818
+
+
+def test_gen_dot():
+    """GenDot (bench_vs_xla.py:137-168): ones(12,12) . x, then a batched product with
+    ones(2,6,6) over the two halves, appended to a constant row."""
+    from enzyme_ad.jax import enzyme_jax_ir, jvp, vjp, ops
+
+    dim = 12
+    h = dim // 2
+
+    @enzyme_jax_ir()
+    def f(x):
+        k = ops.matmul_nt(x, torch.ones(dim, dim, device="cuda"))
+        k_tmp = ops.reshape(k, (2, h))
+        toconv2 = torch.ones(2, h, h, device="cuda")
+        rows = [ops.matmul_nt(ops.select(k_tmp, i), toconv2[i]) for i in range(2)]
+        k = ops.reshape(ops.append_row(ops.reshape(rows[0], (1, h)), rows[1]), (dim,))
+        return ops.append_row(torch.zeros(1, dim, device="cuda"), k)
+
+    x = f32(range(dim))
+    dx = f32([i * i for i in range(dim)])
+    out, tan = jvp(f, (x,), (dx,))
+    assert torch.equal(out, f32([[0.0] * dim, [6.0 * 66.0] * dim]))
+    assert torch.equal(tan, f32([[0.0] * dim, [6.0 * sq(0, dim)] * dim]))             # 3036
+    out, f_vjp = vjp(f, x)
+    (gx,) = f_vjp(f32([i * i for i in range(2 * dim)]).reshape(2, dim))
+    # d k_tmp[i, :] = sum of the cotangent over half i; dx = ones^T . dk = 6 (both halves)
+    assert torch.equal(gx, f32([6.0 * sq(dim, 2 * dim)] * dim))                        # 22908
+
+
+def test_concat():
+    """Concat (bench_vs_xla.py:171-194): two vectors joined; each cotangent is its slice."""
+    from enzyme_ad.jax import enzyme_jax_ir, jvp, vjp, ops
+
+    dim = 12
+
+    @enzyme_jax_ir()
+    def f(x, y):
+        return ops.reshape(ops.append_row(ops.reshape(x, (1, dim)), y), (2 * dim,))
+
+    x, y = f32(range(dim)), f32([10 * i for i in range(dim)])
+    dx, dy = f32([i * i for i in range(dim)]), f32([i * i * i / 3.0 for i in range(dim)])
+    out, tan = jvp(f, (x, y), (dx, dy))
+    assert torch.equal(out, torch.cat([x, y])) and torch.equal(tan, torch.cat([dx, dy]))
+    out, f_vjp = vjp(f, x, y)
+    c = f32([i * i for i in range(2 * dim)])
+    gx, gy = f_vjp(c)
+    assert torch.equal(gx, c[:dim]) and torch.equal(gy, c[dim:])
