@@ -29,6 +29,12 @@ SIGNATURES = {
     "emi_swiglu_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_int]),
     "emi_add": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_int]),
     "emi_transpose": (c_int, [c_void_p, c_void_p, c_void_p, c_i64, c_i64, c_int]),
+    "emi_map_binary": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_i64, c_int, c_int, c_int]),
+    "emi_map_unary": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_i64, c_int]),
+    "emi_convert": (c_int, [c_void_p, c_void_p, c_void_p, c_i64, c_int, c_int]),
+    "emi_strided_copy": (c_int, [c_void_p, c_void_p, c_void_p, c_int, ctypes.POINTER(c_i64), ctypes.POINTER(c_i64),
+                                 c_i64, ctypes.POINTER(c_i64), c_i64, c_int]),
+    "emi_reduce": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_i64, c_i64, c_i64, c_int]),
     "emi_gemm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64,
                          c_i64, c_int, c_int, c_int]),
     "emi_gemm_workspace_bytes": (c_size_t, [c_i64, c_i64, c_i64, c_int, c_int, c_int]),

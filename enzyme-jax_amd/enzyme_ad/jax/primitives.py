@@ -334,8 +334,24 @@ def cpp_call(*args, out_shapes: Sequence[Any], source: str, fn: str = "f", argv=
 
 
 def hlo_call(*args, source: str, argv=(), passes: str = ""):
-    """primitives.py:1052-1108 (StableHLO text in): needs an MLIR front end; not built."""
-    raise NotImplementedError("hlo_call needs a StableHLO front end, which the HIP path does not have")
+    """primitives.py:1052-1108: runs function `main` of a StableHLO module given as text on the
+    arguments (device tensors whose shapes and dtypes must equal the function's, as the
+    reference asserts) and returns the list of its results.  The text is parsed once per
+    distinct source, its llama clusters are matched to the fused kernels, and the operators
+    run on the HIP kernels with their differentiation rules, so `jvp` / `vjp` of a function
+    that calls `hlo_call` work.  `passes` is parsed for validity only: the HIP path has no
+    MLIR optimizer."""
+    from . import stablehlo
+
+    if passes:
+        parse_pass_pipeline(passes)
+    leaves, _ = tree_flatten(args)
+    # attention_step has no tangent kernel: under forward mode its cluster stays unfused
+    exe = stablehlo.compile_text(source, fuse=ops.Forward._active is None)
+    in_tys, _ = exe.signature("main")
+    if len(leaves) != len(in_tys):
+        raise AssertionError("main takes %d arguments, %d given" % (len(in_tys), len(leaves)))
+    return exe.run(leaves, "main")
 
 
 def optimize_module(mod, pipeline=None):

@@ -1,0 +1,845 @@
+"""StableHLO text front end: parse a module, match the llama clusters to the fused kernels,
+and run the rest operator by operator on the device.
+
+The reference hands StableHLO text (`hlo_call`, src/enzyme_ad/jax/primitives.py:1052-1108; the
+text of an `enzyme_jax_ir`-decorated function, :626-692) to MLIR passes and XLA's code
+generator.  Here the text is parsed into a small SSA graph (`parse_module`), rewritten by
+`fuse_clusters` (RMSNorm, SwiGLU and softmax-attention clusters of test/llama.py become one
+fused operator each), and executed by `Executable.run` through `enzyme_ad.jax.ops` /
+`hlo_ops`, whose operators carry the forward- and reverse-mode rules: `jvp` and `vjp` of a
+function that calls `hlo_call` differentiate through the parsed graph.
+
+The accepted text is MLIR's printed form of the operators JAX emits for such functions
+(pretty or quoted-generic operator names): constant, add, subtract, multiply, divide, maximum,
+minimum, power, negate, exponential, log, sqrt, rsqrt, logistic, tanh, sine, cosine, convert, reshape,
+transpose, broadcast_in_dim, reduce (add / maximum), dot_general, slice, concatenate, call,
+return.  Anything else raises `NotImplementedError` naming the operator.
+"""
+import math
+import re
+import struct
+
+import numpy as np
+import torch
+
+from . import hlo_ops as H
+from . import ops
+
+
+class ParseError(ValueError):
+    pass
+
+
+class TensorType:
+    __slots__ = ("shape", "dtype")
+
+    def __init__(self, shape, dtype):
+        self.shape, self.dtype = tuple(shape), dtype
+
+    def __eq__(self, o):
+        return isinstance(o, TensorType) and self.shape == o.shape and self.dtype == o.dtype
+
+    def __repr__(self):
+        return "tensor<%s>" % "x".join([str(s) for s in self.shape] + [self.dtype])
+
+
+class Op:
+    __slots__ = ("name", "results", "operands", "attrs", "types")
+
+    def __init__(self, name, results, operands, attrs, types):
+        self.name, self.results, self.operands, self.attrs, self.types = name, results, operands, attrs, types
+
+    def __repr__(self):
+        return "%s = %s(%s) %s" % (", ".join(self.results), self.name, ", ".join(self.operands), self.attrs)
+
+
+class Func:
+    def __init__(self, name, args, result_types, ops_):
+        self.name, self.args, self.result_types, self.ops = name, args, result_types, ops_
+
+
+TORCH_DTYPES = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16, "f64": torch.float64,
+                "i32": torch.int32, "i64": torch.int64, "i1": torch.bool, "ui32": torch.int32, "i8": torch.int8}
+NUMPY_DTYPES = {"f32": np.float32, "f64": np.float64, "f16": np.float16, "i32": np.int32, "i64": np.int64,
+                "i1": np.bool_, "ui32": np.uint32, "i8": np.int8}
+
+BINARY_OPS = {"add", "subtract", "multiply", "divide", "maximum", "minimum", "power"}
+UNARY_OPS = {"negate", "exponential", "log", "sqrt", "rsqrt", "logistic", "tanh", "sine", "cosine"}
+
+
+# ---------------------------------------------------------------------------
+# parser
+# ---------------------------------------------------------------------------
+
+_WS = re.compile(r"(?:\s+|//[^\n]*)*")
+_SSA = re.compile(r"%[A-Za-z0-9_.$-]+(?:#\d+)?")
+_SYM = re.compile(r"@[A-Za-z0-9_.$-]+|@\"[^\"]*\"")
+_IDENT = re.compile(r"[A-Za-z_][A-Za-z0-9_.$]*")
+_INT = re.compile(r"-?\d+")
+_OPEN = {"(": ")", "[": "]", "{": "}", "<": ">"}
+
+
+class _Scanner:
+    def __init__(self, text):
+        self.s, self.i = text, 0
+
+    def ws(self):
+        self.i = _WS.match(self.s, self.i).end()
+
+    def eof(self):
+        self.ws()
+        return self.i >= len(self.s)
+
+    def peek(self, lit):
+        self.ws()
+        return self.s.startswith(lit, self.i)
+
+    def accept(self, lit):
+        if self.peek(lit):
+            self.i += len(lit)
+            return True
+        return False
+
+    def expect(self, lit):
+        if not self.accept(lit):
+            self.fail("expected '%s'" % lit)
+
+    def match(self, rx):
+        self.ws()
+        m = rx.match(self.s, self.i)
+        if m:
+            self.i = m.end()
+            return m.group(0)
+        return None
+
+    def need(self, rx, what):
+        v = self.match(rx)
+        if v is None:
+            self.fail("expected %s" % what)
+        return v
+
+    def fail(self, msg):
+        line = self.s.count("\n", 0, self.i) + 1
+        near = self.s[self.i:self.i + 40].split("\n")[0]
+        raise ParseError("StableHLO text, line %d: %s near '%s'" % (line, msg, near))
+
+    def balanced(self):
+        """The text of one bracketed group starting at the cursor, brackets included.
+        '->' does not close an angle bracket; strings are skipped."""
+        self.ws()
+        start = self.i
+        stack = []
+        while self.i < len(self.s):
+            c = self.s[self.i]
+            if c == '"':
+                j = self.s.find('"', self.i + 1)
+                if j < 0:
+                    self.fail("unterminated string")
+                self.i = j + 1
+                continue
+            if c in _OPEN:
+                stack.append(_OPEN[c])
+            elif c in ")]}>":
+                if c == ">" and self.s[self.i - 1] == "-":
+                    self.i += 1
+                    continue
+                if not stack or stack[-1] != c:
+                    self.fail("unbalanced '%s'" % c)
+                stack.pop()
+                if not stack:
+                    self.i += 1
+                    return self.s[start:self.i]
+            self.i += 1
+        self.fail("unbalanced bracket")
+
+    def ints(self):
+        """[1, 2, 3] -> [1, 2, 3]"""
+        body = self.balanced()
+        if body[0] != "[":
+            self.fail("expected an integer list")
+        return [int(t) for t in re.findall(r"-?\d+", body)]
+
+    def type(self):
+        self.ws()
+        if not self.accept("tensor"):
+            self.fail("expected a tensor type")
+        body = self.balanced()[1:-1].strip()
+        parts = body.split("x")
+        dtype = parts[-1].strip()
+        # element types such as 'bf16' contain no 'x'; dimensions are integers
+        dims = []
+        for p in parts[:-1]:
+            p = p.strip()
+            if not re.fullmatch(r"\d+", p):
+                self.fail("dynamic or malformed dimension '%s'" % p)
+            dims.append(int(p))
+        if dtype not in TORCH_DTYPES:
+            self.fail("unsupported element type '%s'" % dtype)
+        return TensorType(dims, dtype)
+
+    def signature(self):
+        """': type' or ': (types) -> type | (types)': returns (operand types or None, result types)."""
+        self.expect(":")
+        if self.peek("("):
+            self.expect("(")
+            ins = []
+            if not self.accept(")"):
+                while True:
+                    ins.append(self.type())
+                    if self.accept(")"):
+                        break
+                    self.expect(",")
+            self.expect("->")
+            return ins, self.type_list()
+        first = self.type()
+        types = [first]
+        while self.accept(","):
+            types.append(self.type())
+        if self.accept("->"):
+            return types, self.type_list()
+        return None, types
+
+    def type_list(self):
+        if self.accept("("):
+            outs = []
+            if not self.accept(")"):
+                while True:
+                    outs.append(self.type())
+                    if self.peek("{"):
+                        self.balanced()
+                    if self.accept(")"):
+                        break
+                    self.expect(",")
+            return outs
+        return [self.type()]
+
+
+def _dense(body, ty):
+    """dense<...> payload -> numpy array of the tensor type."""
+    body = body.strip()
+    n = int(np.prod(ty.shape)) if ty.shape else 1
+    width = {"f32": 4, "bf16": 2, "f16": 2, "f64": 8, "i32": 4, "i64": 8, "i1": 1, "ui32": 4, "i8": 1}[ty.dtype]
+
+    def from_bits(raw):
+        if ty.dtype == "bf16":
+            u = np.frombuffer(raw, dtype="<u2").astype(np.uint32) << 16
+            return u.view(np.float32)
+        return np.frombuffer(raw, dtype=np.dtype(NUMPY_DTYPES[ty.dtype]).newbyteorder("<"))
+
+    if body.startswith('"'):                                   # "0x..." raw little-endian bytes
+        hexs = body.strip('"')
+        if not hexs.startswith("0x"):
+            raise ParseError("dense string payload must be hex")
+        raw = bytes.fromhex(hexs[2:])
+        arr = from_bits(raw)
+        if arr.size == 1 and n > 1:
+            arr = np.repeat(arr, n)
+        if arr.size != n:
+            raise ParseError("dense payload has %d elements, type %r wants %d" % (arr.size, ty, n))
+        return np.array(arr).reshape(ty.shape)
+
+    def scalar(tok):
+        tok = tok.strip()
+        if tok in ("true", "false"):
+            return tok == "true"
+        if tok.lower().startswith("0x") and ty.dtype in ("f32", "bf16", "f16", "f64"):
+            bits = int(tok, 16)
+            return from_bits(bits.to_bytes(width, "little"))[0]
+        if ty.dtype.startswith("f") or ty.dtype == "bf16":
+            return float(tok)
+        return int(tok, 0)
+
+    toks = [t for t in re.split(r"[\[\],\s]+", body) if t]
+    vals = [scalar(t) for t in toks]
+    if len(vals) == 1:
+        vals = vals * n
+    if len(vals) != n:
+        raise ParseError("dense payload has %d elements, type %r wants %d" % (len(vals), ty, n))
+    npdt = np.float32 if ty.dtype == "bf16" else NUMPY_DTYPES[ty.dtype]
+    return np.array(vals, dtype=npdt).reshape(ty.shape)
+
+
+def _i64_array(text, key):
+    """key = array<i64: 1, 0> or key = dense<[1, 0]> : tensor<2xi64> -> [1, 0]"""
+    m = re.search(key + r"\s*=\s*(array<i64:?([^>]*)>|dense<([^>]*)>)", text)
+    if not m:
+        raise ParseError("attribute %s not found" % key)
+    return [int(t) for t in re.findall(r"-?\d+", m.group(2) if m.group(2) is not None else m.group(3))]
+
+
+def _attr_lists(text, key):
+    m = re.search(key + r"\s*=\s*\[([^\]]*)\]", text)
+    return [int(t) for t in re.findall(r"-?\d+", m.group(1))] if m else []
+
+
+def _parse_op(sc):
+    results = []
+    save = sc.i
+    first = sc.match(_SSA)
+    if first is not None:
+        names = [first]
+        count = 1
+        if sc.accept(":"):
+            count = int(sc.need(_INT, "result count"))
+        while sc.accept(","):
+            names.append(sc.need(_SSA, "result name"))
+        sc.expect("=")
+        results = names if count == 1 else ["%s#%d" % (first, k) for k in range(count)]
+    else:
+        sc.i = save
+    generic = sc.peek('"')
+    if generic:
+        sc.expect('"')
+        name = sc.need(_IDENT, "operator name")
+        sc.expect('"')
+    else:
+        name = sc.need(_IDENT, "operator name")
+    short = name.split(".", 1)[1] if name.startswith(("stablehlo.", "mhlo.", "func.", "arith.")) else name
+    attrs = {}
+
+    def operand_list(close=None):
+        out = []
+        while True:
+            v = sc.match(_SSA)
+            if v is None:
+                break
+            out.append(v)
+            before = sc.i
+            if not sc.accept(","):
+                break
+            if not sc.peek("%"):
+                sc.i = before      # the comma belongs to a trailing attribute
+                break
+        return out
+
+    if short in ("return",):
+        operands = operand_list()
+        if operands:
+            sc.signature()
+        return Op("return", [], operands, attrs, [])
+
+    if generic:
+        sc.expect("(")
+        operands = operand_list()
+        sc.expect(")")
+        text = ""
+        while sc.peek("<{") or sc.peek("{"):
+            if sc.accept("<"):
+                text += sc.balanced()
+                sc.expect(">")
+            else:
+                text += sc.balanced()
+        if sc.peek("("):                                       # regions of a generic operator
+            sc.fail("regions of quoted operators are not supported")
+        _, types = sc.signature()
+        if short == "dot_general":
+            attrs = {"batch_a": _attr_lists(text, "lhs_batching_dimensions"),
+                     "batch_b": _attr_lists(text, "rhs_batching_dimensions"),
+                     "contract_a": _attr_lists(text, "lhs_contracting_dimensions"),
+                     "contract_b": _attr_lists(text, "rhs_contracting_dimensions")}
+        elif short == "transpose":
+            attrs = {"perm": _i64_array(text, "permutation")}
+        elif short == "broadcast_in_dim":
+            attrs = {"dims": _i64_array(text, "broadcast_dimensions")}
+        elif short == "concatenate":
+            attrs = {"dim": int(re.search(r"dimension\s*=\s*(\d+)", text).group(1))}
+        elif short == "constant":
+            m = re.search(r"value\s*=\s*dense<", text)
+            if not m:
+                sc.fail("constant without a dense value")
+            sub = _Scanner(text[m.end() - 1:])
+            attrs = {"value": _dense(sub.balanced()[1:-1], types[0])}
+        elif short in BINARY_OPS or short in UNARY_OPS or short in ("reshape", "convert"):
+            pass
+        else:
+            raise NotImplementedError("StableHLO operator '%s' in quoted form is not supported" % name)
+        return Op(short, results, operands, attrs, types)
+
+    if short == "constant":
+        sc.expect("dense")
+        body = sc.balanced()[1:-1]
+        _, types = sc.signature()
+        return Op("constant", results, [], {"value": _dense(body, types[0])}, types)
+    if short == "reduce":
+        sc.expect("(")
+        x = sc.need(_SSA, "operand")
+        sc.expect("init")
+        sc.expect(":")
+        init = sc.need(_SSA, "init value")
+        sc.expect(")")
+        body = None
+        if sc.accept("applies"):
+            body = sc.need(_IDENT, "reduction operator")
+        sc.expect("across")
+        sc.expect("dimensions")
+        sc.expect("=")
+        dims = sc.ints()
+        _, types = sc.signature()
+        if body is None:
+            sc.expect("reducer")
+            sc.balanced()                       # block arguments
+            region = sc.balanced()
+            found = re.findall(r"(?:stablehlo|mhlo)\.(add|maximum|minimum|multiply)\b", region)
+            if len(found) != 1:
+                sc.fail("reduce body must be one add or maximum")
+            body = found[0]
+        body = body.split(".")[-1]
+        return Op("reduce", results, [x, init], {"dims": dims, "body": body}, types)
+    if short == "call":
+        callee = sc.need(_SYM, "callee")
+        sc.expect("(")
+        operands = operand_list()
+        sc.expect(")")
+        if sc.peek("{"):
+            sc.balanced()
+        _, types = sc.signature()
+        return Op("call", results, operands, {"callee": callee[1:].strip('"')}, types)
+    if short == "slice":
+        x = sc.need(_SSA, "operand")
+        body = sc.balanced()
+        if body[0] != "[":
+            sc.fail("expected slice bounds")
+        start, limit, stride = [], [], []
+        for part in body[1:-1].split(","):
+            nums = [int(t) for t in part.strip().split(":")]
+            start.append(nums[0])
+            limit.append(nums[1])
+            stride.append(nums[2] if len(nums) > 2 else 1)
+        _, types = sc.signature()
+        return Op("slice", results, [x], {"start": start, "limit": limit, "stride": stride}, types)
+
+    operands = operand_list()
+    # trailing attributes: ', key = value'
+    while sc.accept(","):
+        key = sc.need(_IDENT, "attribute name")
+        sc.expect("=")
+        if sc.peek("["):
+            v = sc.ints() if not re.match(r"\s*\[\s*[A-Za-z]", sc.s[sc.i:]) else sc.balanced()
+            if sc.accept("x"):
+                v = (v, sc.ints())
+        elif sc.peek("<") or sc.peek("{") or sc.peek("("):
+            v = sc.balanced()
+        else:
+            v = sc.need(re.compile(r"[A-Za-z0-9_.+-]+"), "attribute value")
+        attrs[key] = v
+    if sc.peek("{"):
+        sc.balanced()                            # a discardable attribute dictionary
+    _, types = sc.signature()
+    if short == "dot_general":
+        b = attrs.get("batching_dims", ([], []))
+        c = attrs.get("contracting_dims", ([], []))
+        attrs = {"batch_a": b[0], "batch_b": b[1], "contract_a": c[0], "contract_b": c[1]}
+    elif short == "transpose":
+        attrs = {"perm": attrs["dims"]}
+    elif short == "broadcast_in_dim":
+        attrs = {"dims": attrs["dims"]}
+    elif short == "concatenate":
+        attrs = {"dim": int(attrs["dim"])}
+    elif short in BINARY_OPS or short in UNARY_OPS or short in ("reshape", "convert"):
+        attrs = {}
+    else:
+        raise NotImplementedError("StableHLO operator '%s' is not supported by the HIP front end" % name)
+    return Op(short, results, operands, attrs, types)
+
+
+def _parse_func(sc):
+    for vis in ("public", "private", "nested"):
+        sc.accept(vis)
+    name = sc.need(_SYM, "function name")[1:]
+    sc.expect("(")
+    args = []
+    if not sc.accept(")"):
+        while True:
+            a = sc.need(_SSA, "argument name")
+            sc.expect(":")
+            t = sc.type()
+            if sc.peek("{"):
+                sc.balanced()
+            args.append((a, t))
+            if sc.accept(")"):
+                break
+            sc.expect(",")
+    result_types = []
+    if sc.accept("->"):
+        result_types = sc.type_list()
+    if sc.accept("attributes"):
+        sc.balanced()
+    sc.expect("{")
+    body = []
+    while not sc.accept("}"):
+        body.append(_parse_op(sc))
+    return Func(name, args, result_types, body)
+
+
+def parse_module(text):
+    """{function name: Func} of a StableHLO module (or of bare func.func definitions)."""
+    sc = _Scanner(text)
+    funcs = {}
+    wrapped = False
+    if sc.accept("module"):
+        wrapped = True
+        sc.match(_SYM)
+        if sc.accept("attributes"):
+            sc.balanced()
+        sc.expect("{")
+    while not sc.eof():
+        if wrapped and sc.accept("}"):
+            break
+        if sc.accept("func.func"):
+            f = _parse_func(sc)
+            funcs[f.name] = f
+        else:
+            sc.fail("expected func.func")
+    if not funcs:
+        raise ParseError("StableHLO text holds no function")
+    return funcs
+
+
+# ---------------------------------------------------------------------------
+# cluster matcher
+# ---------------------------------------------------------------------------
+
+def _users(func):
+    use = {}
+    for op in func.ops:
+        for o in op.operands:
+            use.setdefault(o, []).append(op)
+    return use
+
+
+def _splat(op):
+    """The value of a constant whose elements are all equal, else None."""
+    if op is None or op.name != "constant":
+        return None
+    v = op.attrs["value"]
+    flat = np.asarray(v).reshape(-1)
+    if flat.size == 0 or not np.all(flat == flat[0]):
+        return None
+    return float(flat[0])
+
+
+def fuse_clusters(func):
+    """Rewrites, in place, the operator clusters test/llama.py traces into fused operators:
+
+      emi.rmsnorm  w * (x * (1 / sqrt(dot(x, x) / n + eps)))           (llama.py:6-10), also with
+                   rsqrt in place of 1 / sqrt (EnzymeHLOOpt.cpp:14907-14923)
+      emi.swiglu   a * (1 / (1 + exp(-a))) * b, or a * logistic(a) * b  (llama.py:21-28,229-231)
+      emi.softmax_dot  softmax(dot(K, q) / c) followed by the dot with V  (llama.py:13-18,193-204)
+
+    A cluster is fused only when none of its interior values is used outside it.  Returns
+    the number of clusters fused per kind."""
+    counts = {"rmsnorm": 0, "swiglu": 0, "softmax_dot": 0}
+    changed = True
+    while changed:
+        changed = False
+        defs = {r: op for op in func.ops for r in op.results}
+        use = _users(func)
+        rets = set(o for op in func.ops if op.name == "return" for o in op.operands)
+
+        def d(name):
+            return defs.get(name)
+
+        def through_broadcast(name):
+            """The rank-0 value behind a broadcast_in_dim (or the name itself)."""
+            op = d(name)
+            if op is not None and op.name == "broadcast_in_dim" and not op.attrs["dims"]:
+                return op.operands[0], op
+            return name, None
+
+        def only_used_by(names, inside):
+            ids = set(id(o) for o in inside)
+            for n in names:
+                if n in rets:
+                    return False
+                for u in use.get(n, []):
+                    if id(u) not in ids:
+                        return False
+            return True
+
+        for op in func.ops:
+            m = _match_rmsnorm(op, d, through_broadcast) or _match_swiglu(op, d, through_broadcast) or \
+                _match_softmax_dot(op, d, through_broadcast)
+            if m is None:
+                continue
+            kind, new_op, interior = m
+            inner_names = [r for o in interior if o is not op for r in o.results]
+            if not only_used_by(inner_names, interior):
+                continue
+            # drop interior operators whose results nobody else needs; keep shared constants
+            dead = set(id(o) for o in interior if o is not op)
+            func.ops = [new_op if o is op else o for o in func.ops if id(o) not in dead]
+            counts[kind] += 1
+            changed = True
+            break
+    return counts
+
+
+def _match_rmsnorm(op, d, tb):
+    # root: a product of three factors, (w * x) * bcast(ss) or w * (x * bcast(ss)) in any
+    # operand order, ss = 1 / sqrt(dot(x, x) / n + eps) or rsqrt(...)
+    if op.name != "multiply":
+        return None
+    for ii in (0, 1):
+        inner = d(op.operands[ii])
+        if inner is None or inner.name != "multiply":
+            continue
+        leaves = [op.operands[1 - ii]] + list(inner.operands)
+        for si, leaf in enumerate(leaves):
+            ss_name, bc = tb(leaf)
+            if bc is None:
+                continue
+            ss = d(ss_name)
+            if ss is None:
+                continue
+            interior = [op, inner, bc, ss]
+            if ss.name == "rsqrt":
+                arg = d(ss.operands[0])
+            elif ss.name == "divide" and _splat(d(ss.operands[0])) == 1.0:
+                sq = d(ss.operands[1])
+                if sq is None or sq.name != "sqrt":
+                    continue
+                interior.append(sq)
+                arg = d(sq.operands[0])
+            else:
+                continue
+            if arg is None or arg.name != "add":
+                continue
+            eps = mean = None
+            for ei in (0, 1):
+                e = _splat(d(arg.operands[ei]))
+                if e is not None:
+                    eps, mean = e, d(arg.operands[1 - ei])
+            if eps is None or mean is None or mean.name != "divide":
+                continue
+            n = _splat(d(mean.operands[1]))
+            dot = d(mean.operands[0])
+            if n is None or dot is None or dot.name != "dot_general":
+                continue
+            if dot.operands[0] != dot.operands[1] or dot.attrs["batch_a"] or len(dot.attrs["contract_a"]) != 1:
+                continue
+            x = dot.operands[0]
+            rest = [l for k, l in enumerate(leaves) if k != si]
+            if x not in rest:
+                continue
+            rest.remove(x)
+            w = rest[0]
+            xt = op.types[0]
+            if len(xt.shape) != 1 or n != float(xt.shape[0]):
+                continue
+            interior += [arg, mean, dot]
+            return "rmsnorm", Op("emi.rmsnorm", op.results, [x, w], {"eps": eps}, op.types), interior
+    return None
+
+
+def _match_sigmoid(name, d, tb):
+    """name = logistic(a) or 1 / (1 + exp(-a)): returns (a, interior ops) or None."""
+    s = d(name)
+    if s is None:
+        return None
+    if s.name == "logistic":
+        return s.operands[0], [s]
+    if s.name != "divide":
+        return None
+    num, nbc = tb(s.operands[0])
+    if _splat(d(num)) != 1.0:
+        return None
+    den = d(s.operands[1])
+    if den is None or den.name != "add":
+        return None
+    for oi in (0, 1):
+        one, obc = tb(den.operands[oi])
+        ex = d(den.operands[1 - oi])
+        if _splat(d(one)) != 1.0 or ex is None or ex.name != "exponential":
+            continue
+        ng = d(ex.operands[0])
+        if ng is None or ng.name != "negate":
+            continue
+        interior = [s, den, ex, ng] + [b for b in (nbc, obc) if b is not None]
+        return ng.operands[0], interior
+    return None
+
+
+def _match_swiglu(op, d, tb):
+    # root: multiply(multiply(a, sigmoid(a)), b) in any operand order
+    if op.name != "multiply":
+        return None
+    for bi in (0, 1):
+        b, inner = op.operands[bi], d(op.operands[1 - bi])
+        if inner is None or inner.name != "multiply":
+            continue
+        for ai in (0, 1):
+            a = inner.operands[ai]
+            sg = _match_sigmoid(inner.operands[1 - ai], d, tb)
+            if sg is None or sg[0] != a:
+                continue
+            return "swiglu", Op("emi.swiglu", op.results, [a, b], {}, op.types), [op, inner] + sg[1]
+    return None
+
+
+def _match_softmax_dot(op, d, tb):
+    # root: dot_general(att, V) or dot_general(V, att) contracting the sequence index, with
+    # att = e / bcast(sum(e)), e = exp(s - bcast(max(s))), s = dot_general(K, q) / c  (or * c)
+    if op.name != "dot_general" or op.attrs["batch_a"] or len(op.attrs["contract_a"]) != 1:
+        return None
+    for ai in (0, 1):
+        att, v = d(op.operands[ai]), op.operands[1 - ai]
+        if att is None or att.name != "divide":
+            continue
+        e = d(att.operands[0])
+        sum_name, sbc = tb(att.operands[1])
+        sm = d(sum_name)
+        if e is None or e.name != "exponential" or sbc is None or sm is None or sm.name != "reduce":
+            continue
+        if sm.attrs["body"] != "add" or sm.operands[0] != att.operands[0]:
+            continue
+        sub = d(e.operands[0])
+        if sub is None or sub.name != "subtract":
+            continue
+        s_name = sub.operands[0]
+        max_name, mbc = tb(sub.operands[1])
+        mx = d(max_name)
+        if mbc is None or mx is None or mx.name != "reduce" or mx.attrs["body"] != "maximum" or mx.operands[0] != s_name:
+            continue
+        s = d(s_name)
+        if s is None or s.name not in ("divide", "multiply"):
+            continue
+        c_name, cbc = tb(s.operands[1])
+        c = _splat(d(c_name))
+        sdot = d(s.operands[0])
+        if c is None or sdot is None or sdot.name != "dot_general" or sdot.attrs["batch_a"]:
+            continue
+        scale = 1.0 / c if s.name == "divide" else c
+        # K [S, d] . q [d] -> [S]
+        if sdot.attrs["contract_a"] != [1] or sdot.attrs["contract_b"] != [0]:
+            continue
+        k, q = sdot.operands
+        seq_type = s.types[0]
+        if len(seq_type.shape) != 1:
+            continue
+        # att [S] . V [S, d] -> [d]: contraction over index 0 of V
+        att_side, v_side = ("contract_a", "contract_b") if ai == 0 else ("contract_b", "contract_a")
+        if op.attrs[att_side] != [0] or op.attrs[v_side] != [0]:
+            continue
+        interior = [op, att, e, sbc, sm, sub, mbc, mx, s, sdot] + ([cbc] if cbc is not None else [])
+        return ("softmax_dot", Op("emi.softmax_dot", op.results, [q, k, v], {"scale": scale}, op.types), interior)
+    return None
+
+
+# ---------------------------------------------------------------------------
+# executor
+# ---------------------------------------------------------------------------
+
+class Executable:
+    """A parsed module ready to run on one device."""
+
+    def __init__(self, text, fuse=True):
+        self.funcs = parse_module(text)
+        self.fused = {}
+        if fuse:
+            for f in self.funcs.values():
+                for k, v in fuse_clusters(f).items():
+                    self.fused[k] = self.fused.get(k, 0) + v
+        self._consts = {}
+
+    def signature(self, fn="main"):
+        f = self._func(fn)
+        return [t for _, t in f.args], list(f.result_types)
+
+    def _func(self, fn):
+        if fn not in self.funcs:
+            raise AssertionError("Could not find desired function %s options are %s" % (fn, sorted(self.funcs)))
+        return self.funcs[fn]
+
+    def _const(self, op, device):
+        key = (id(op), str(device))
+        hit = self._consts.get(key)
+        if hit is None:
+            ty = op.types[0]
+            host = torch.from_numpy(np.array(op.attrs["value"]).reshape(-1)).reshape(ty.shape)
+            hit = self._consts[key] = host.to(TORCH_DTYPES[ty.dtype]).to(device)       # trace-time constant upload
+        return hit
+
+    def run(self, args, fn="main"):
+        f = self._func(fn)
+        if len(args) != len(f.args):
+            raise ValueError("%s takes %d arguments, %d given" % (fn, len(f.args), len(args)))
+        env = {}
+        device = None
+        if getattr(f, "defs", None) is None:
+            f.defs = {r: op for op in f.ops for r in op.results}
+        for (name, ty), a in zip(f.args, args):
+            if not isinstance(a, torch.Tensor):
+                raise TypeError("argument %s is not a tensor" % name)
+            if tuple(a.shape) != ty.shape or a.dtype != TORCH_DTYPES[ty.dtype]:
+                raise ValueError("argument %s is %s/%s, the module wants %r" % (name, tuple(a.shape), a.dtype, ty))
+            if not a.is_cuda:
+                raise RuntimeError("argument %s is not in device memory: the HIP path has no CPU fallback" % name)
+            device = a.device
+            env[name] = a
+        if device is None:
+            device = torch.device("cuda", torch.cuda.current_device())
+        for op in f.ops:
+            if op.name == "return":
+                return [env[o] for o in op.operands]
+            outs = self._apply(f, op, [env[o] for o in op.operands], device)
+            if len(outs) != len(op.results):
+                raise RuntimeError("%s produced %d values for %d results" % (op.name, len(outs), len(op.results)))
+            for r, v, ty in zip(op.results, outs, op.types):
+                if tuple(v.shape) != ty.shape:
+                    raise RuntimeError("%s: result %s has shape %s, the text says %r" % (op.name, r, tuple(v.shape), ty))
+                env[r] = v
+        raise ParseError("function %s has no return" % fn)
+
+    def _apply(self, f, op, xs, device):
+        n = op.name
+        if n == "constant":
+            return [self._const(op, device)]
+        if n in BINARY_OPS:
+            return [H.binary(n, xs[0], xs[1])]
+        if n in UNARY_OPS:
+            return [H.unary(n, xs[0])]
+        if n == "convert":
+            dt = TORCH_DTYPES[op.types[0].dtype]
+            return [xs[0] if xs[0].dtype == dt else H.convert(xs[0], dt)]
+        if n == "reshape":
+            return [ops.reshape(H._contig(xs[0]), op.types[0].shape)]
+        if n == "transpose":
+            return [H.transpose(xs[0], op.attrs["perm"])]
+        if n == "broadcast_in_dim":
+            return [H.broadcast_in_dim(xs[0], op.types[0].shape, op.attrs["dims"])]
+        if n == "reduce":
+            kind = op.attrs["body"]
+            y = H.reduce(kind, xs[0], op.attrs["dims"])
+            init = _splat(f.defs.get(op.operands[1]))
+            if init is not None and ((kind == "add" and init == 0.0) or (kind == "maximum" and init == -math.inf)):
+                return [y]
+            return [H.binary(kind, y, xs[1])]
+        if n == "dot_general":
+            return [H.dot_general(xs[0], xs[1], op.attrs["batch_a"], op.attrs["batch_b"], op.attrs["contract_a"],
+                                  op.attrs["contract_b"])]
+        if n == "slice":
+            return [H.slice_(xs[0], op.attrs["start"], op.attrs["limit"], op.attrs["stride"])]
+        if n == "concatenate":
+            return [H.concatenate(xs, op.attrs["dim"])]
+        if n == "call":
+            return self.run(xs, op.attrs["callee"])
+        if n == "emi.rmsnorm":
+            x, w = xs
+            return [ops.reshape(ops.rmsnorm(ops.reshape(x, (1, x.shape[0])), w, op.attrs["eps"]), tuple(x.shape))]
+        if n == "emi.swiglu":
+            return [ops.swiglu(H._contig(xs[0]), H._contig(xs[1]))]
+        if n == "emi.softmax_dot":
+            q, k, v = xs
+            return [ops.attention_step(q, H._contig(k), H._contig(v), 1, op.attrs["scale"])]
+        raise NotImplementedError("StableHLO operator '%s' is not supported by the HIP front end" % n)
+
+
+_CACHE = {}
+
+
+def compile_text(text, fuse=True):
+    key = (text, fuse)
+    exe = _CACHE.get(key)
+    if exe is None:
+        exe = _CACHE[key] = Executable(text, fuse)
+    return exe

@@ -188,6 +188,58 @@ int emi_attn_jvp(emi_stream_t stream, const void* q, const void* k, const void* 
                  int64_t heads, int64_t seq, int64_t head_dim, int64_t stride_b, int64_t stride_h,
                  int64_t stride_s, float scale, int causal, int dtype);
 
+/* ---- generic tensor operators -------------------------------------------
+ * What is left of a StableHLO module that arrives as text (hlo_call,
+ * src/enzyme_ad/jax/primitives.py:1052-1108; in the reference XLA's own code
+ * generator compiles these operators) once the llama clusters have been
+ * matched to the fused kernels above.  Operator codes: */
+enum {
+  /* binary: y = op(a, b) */
+  EMI_OP_ADD = 0, EMI_OP_SUB, EMI_OP_MUL, EMI_OP_DIV, EMI_OP_MAX, EMI_OP_MIN,
+  EMI_OP_GE,        /* 1.0 where a >= b else 0.0 (Max rule HLODerivatives.td:1205: ties go to a) */
+  EMI_OP_EQ,        /* 1.0 where a == b else 0.0 (reduce-max rule, StableHLOAutoDiffOpInterfaceImpl.cpp:1881-1916) */
+  EMI_OP_NMUL,      /* -(a * b) */
+  EMI_OP_POW,
+  /* binary derivative factors, a = incoming (co)tangent, b = the operator's saved value */
+  EMI_OP_D_SQRT,     /* b = sqrt(x):     b == 0 ? 0 : a / (2 b)   (Sqrt rule :1320 with its zero guard) */
+  EMI_OP_D_RSQRT,    /* b = rsqrt(x):    -a b^3 / 2               (Rsqrt rule :1283) */
+  EMI_OP_D_LOGISTIC, /* b = logistic(x): a b (1 - b) */
+  EMI_OP_D_TANH,     /* b = tanh(x):     a (1 - b^2) */
+  EMI_OP_D_SIN,      /* b = x:           a cos(b) */
+  EMI_OP_D_COS,      /* b = x:           -a sin(b) */
+  /* factors of the Pow rule (HLODerivatives.td:1237-1242) on the operands themselves */
+  EMI_OP_D_POW_A,    /* b pow(a, b - 1) */
+  EMI_OP_D_POW_B,    /* pow(a, b) log(a) */
+  /* unary: y = op(x) */
+  EMI_OP_NEG = 32, EMI_OP_EXP, EMI_OP_LOG, EMI_OP_SQRT, EMI_OP_RSQRT, EMI_OP_LOGISTIC, EMI_OP_TANH,
+  EMI_OP_SIN, EMI_OP_COS, EMI_OP_ABS, EMI_OP_COPY
+};
+
+/* y[i] = op(a[i], b[i]) for i < n, computed in fp32.  An operand flagged
+ * *_is_scalar is a single element broadcast to all i (a folded
+ * broadcast_in_dim of a rank-0 tensor).  y may alias a or b. */
+int emi_map_binary(emi_stream_t stream, int op, const void* a, const void* b, void* y, int64_t n,
+                   int a_is_scalar, int b_is_scalar, int dtype);
+/* y[i] = op(x[i]).  y may alias x. */
+int emi_map_unary(emi_stream_t stream, int op, const void* x, void* y, int64_t n, int dtype);
+/* stablehlo.convert between EMI_F32 and EMI_BF16 (round to nearest even). */
+int emi_convert(emi_stream_t stream, const void* x, void* y, int64_t n, int from_dtype, int to_dtype);
+/* out[out_offset + sum_d i_d out_strides[d]] = in[in_offset + sum_d i_d in_strides[d]] for every
+ * index 0 <= i_d < dims[d]: transpose (permuted strides), broadcast_in_dim
+ * (zero in_strides), slice (offset and strides; Slice rule
+ * StableHLOAutoDiffOpInterfaceImpl.cpp:1586-1620) and one operand of
+ * concatenate (Concatenate rule :2015-2059).  rank <= 8; strides and offsets in
+ * elements of elem_bytes (2, 4 or 8) bytes; dims / strides are HOST arrays.
+ * The boxes must not overlap. */
+int emi_strided_copy(emi_stream_t stream, const void* in, void* out, int rank, const int64_t* dims,
+                     const int64_t* in_strides, int64_t in_offset, const int64_t* out_strides,
+                     int64_t out_offset, int elem_bytes);
+/* y[o, i] = sum or max over r of x[o, r, i] (op = EMI_OP_ADD or EMI_OP_MAX), fp32
+ * accumulation (stablehlo.reduce with an add / maximum body; Reduce rule
+ * StableHLOAutoDiffOpInterfaceImpl.cpp:1833-1916).  x: [outer, red, inner] contiguous. */
+int emi_reduce(emi_stream_t stream, int op, const void* x, void* y, int64_t outer, int64_t red,
+               int64_t inner, int dtype);
+
 /* Embedding gather x[t,:] = table[tokens[t],:] and its adjoint (scatter-add of
  * dx rows into a zero-initialised dtable; fp32 accumulation in workspace when
  * dtype is bf16).  The lookup is commented out in the reference

@@ -1,0 +1,273 @@
+"""GPU parity of the StableHLO text front end: the generic tensor kernels against numpy, the
+reference's `hlo_call` fixture (test/testffi.py:6-49) against its closed-form answers, and the
+differentiation rules of the generic operators against the known-answer vectors of the
+reference's lit tests (tests/golden/diffrules.json), each driven through StableHLO text."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import TDTYPE, dev, host
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "diffrules.json")))
+
+
+def f32(a):
+    return torch.tensor(np.asarray(a, dtype=np.float32), device="cuda")
+
+
+def ulp_close(got, want, dt):
+    got, want = host(got), np.asarray(want, dtype=np.float64)
+    tol = 2e-6 if dt == "f32" else 8e-3                    # one bf16 ulp is 2^-8 relative
+    np.testing.assert_allclose(got, want, rtol=tol, atol=tol * 1e-3)
+
+
+# ---------------------------------------------------------------------------
+# kernels
+# ---------------------------------------------------------------------------
+
+NP_BINARY = {"add": np.add, "subtract": np.subtract, "multiply": np.multiply, "divide": np.divide,
+             "maximum": np.maximum, "minimum": np.minimum, "ge": lambda a, b: (a >= b).astype(np.float64),
+             "eq": lambda a, b: (a == b).astype(np.float64), "nmul": lambda a, b: -(a * b), "power": np.power,
+             "d_sqrt": lambda a, b: np.where(b == 0, 0.0, a / (2 * np.where(b == 0, 1.0, b))),
+             "d_rsqrt": lambda a, b: -0.5 * a * b ** 3, "d_logistic": lambda a, b: a * b * (1 - b),
+             "d_tanh": lambda a, b: a * (1 - b * b), "d_sin": lambda a, b: a * np.cos(b),
+             "d_cos": lambda a, b: -a * np.sin(b), "d_pow_a": lambda a, b: b * np.power(a, b - 1),
+             "d_pow_b": lambda a, b: np.power(a, b) * np.log(a)}
+NP_UNARY = {"negate": np.negative, "exponential": np.exp, "log": np.log, "sqrt": np.sqrt,
+            "rsqrt": lambda x: 1 / np.sqrt(x), "logistic": lambda x: 1 / (1 + np.exp(-x)), "tanh": np.tanh,
+            "sine": np.sin, "cosine": np.cos, "abs": np.abs, "copy": lambda x: x}
+POSITIVE = {"log", "sqrt", "rsqrt", "power", "d_pow_a", "d_pow_b"}
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("n", [1, 7, 1000, 4099])
+def test_elementwise_maps_match_numpy(dt, n):
+    from enzyme_ad.jax import hlo_ops as H
+
+    rng = np.random.default_rng(n)
+    for name, fn in NP_BINARY.items():
+        a = rng.uniform(0.5, 2.0, n) if name in POSITIVE else rng.normal(size=n)
+        b = rng.uniform(0.5, 2.0, n) if name in POSITIVE else rng.normal(size=n)
+        if name in ("ge", "eq", "maximum") and n > 2:
+            b[::3] = a[::3]                                             # ties
+        ta, ra = dev(a, dt)
+        tb, rb = dev(b, dt)
+        ulp_close(H._bin(name, ta, tb), fn(ra, rb), dt)
+        s, rs = torch.tensor(1.25, dtype=TDTYPE[dt], device="cuda"), 1.25    # rank-0 operand, either side
+        ulp_close(H._bin(name, ta, s), fn(ra, rs), dt)
+        ulp_close(H._bin(name, s, tb), fn(rs, rb), dt)
+    for name, fn in NP_UNARY.items():
+        x = rng.uniform(0.5, 2.0, n) if name in POSITIVE else rng.normal(size=n)
+        tx, rx = dev(x, dt)
+        ulp_close(H._un(name, tx), fn(rx), dt)
+    tx, rx = dev(rng.normal(size=n), "f32")
+    back = H._convert(H._convert(tx, torch.bfloat16), torch.float32)
+    assert torch.equal(back, tx.to(torch.bfloat16).float())
+
+
+def test_elementwise_maps_on_unaligned_views():
+    from enzyme_ad.jax import hlo_ops as H
+
+    base, ref = dev(np.arange(64, dtype=np.float32), "f32")
+    a, b = base[1:34], base[3:36]                                        # 4-byte aligned only
+    assert np.array_equal(host(H._bin("add", a, b)), ref[1:34] + ref[3:36])
+    assert np.array_equal(host(H._un("negate", a)), -ref[1:34])
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+def test_strided_copy_forms_match_numpy(dt):
+    from enzyme_ad.jax import hlo_ops as H
+
+    rng = np.random.default_rng(3)
+    x, rx = dev(rng.normal(size=(6, 8, 16)), dt)
+    for perm in ([0, 1, 2], [2, 1, 0], [1, 0, 2], [0, 2, 1], [2, 0, 1]):
+        assert np.array_equal(host(H._permute(x, perm)), rx.transpose(perm))
+    v, rv = dev(rng.normal(size=(8,)), dt)
+    assert np.array_equal(host(H._broadcast(v, (6, 8, 16), [1])), np.broadcast_to(rv[None, :, None], (6, 8, 16)))
+    r, rr = dev(rng.normal(size=(6, 1, 16)), dt)
+    assert np.array_equal(host(H._broadcast(r, (6, 8, 16), [0, 1, 2])), np.broadcast_to(rr, (6, 8, 16)))
+    s = torch.tensor(2.5, dtype=TDTYPE[dt], device="cuda")
+    assert np.array_equal(host(H._broadcast(s, (5, 3), [])), np.full((5, 3), 2.5))
+    assert np.array_equal(host(H._slice(x, [1, 0, 3], [6, 8, 16], [2, 3, 1])), rx[1:6:2, 0:8:3, 3:16])
+    assert np.array_equal(host(H._slice(x, [0, 0, 0], [6, 8, 8], [1, 1, 1])), rx[:, :, :8])
+    y, ry = dev(rng.normal(size=(6, 3, 16)), dt)
+    assert np.array_equal(host(H._concat([x, y], 1)), np.concatenate([rx, ry], 1))
+    z, rz = dev(rng.normal(size=(6, 8, 5)), dt)
+    assert np.array_equal(host(H._concat([x, z, x], 2)), np.concatenate([rx, rz, rx], 2))
+    box = H._scatter_box(H._slice(x, [1, 0, 3], [6, 8, 16], [2, 3, 1]), [6, 8, 16], [1, 0, 3], [2, 3, 1])
+    want = np.zeros_like(rx)
+    want[1:6:2, 0:8:3, 3:16] = rx[1:6:2, 0:8:3, 3:16]
+    assert np.array_equal(host(box), want)
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("shape,dims", [((37, 5000), [1]), ((37, 5000), [0]), ((4, 33, 7), [1]), ((4, 33, 7), [0, 2]),
+                                        ((2, 3, 4), [0, 1, 2]), ((300, 64), [1]), ((1, 100003), [1])])
+def test_reduce_matches_numpy(dt, shape, dims):
+    from enzyme_ad.jax import hlo_ops as H
+
+    x, rx = dev(np.random.default_rng(5).normal(size=shape), dt)
+    tol = 1e-5 if dt == "f32" else 8e-3
+    got = host(H._reduce("add", x, dims))
+    want = rx.sum(axis=tuple(dims))
+    assert np.max(np.abs(got - want)) <= tol * max(1.0, np.max(np.abs(want)))
+    assert np.array_equal(host(H._reduce("maximum", x, dims)), rx.max(axis=tuple(dims)))
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+def test_dot_general_forms_match_numpy(dt):
+    from enzyme_ad.jax import hlo_ops as H
+
+    rng = np.random.default_rng(11)
+    tol = 1e-5 if dt == "f32" else 1.5e-2
+    cases = [
+        ((2, 3), (4, 2), [], [], [0], [1], "ki,jk->ij"),
+        ((5, 7, 9), (5, 9, 4), [0], [0], [2], [1], "bmk,bkn->bmn"),
+        ((288, 288), (288,), [], [], [1], [0], "ok,k->o"),
+        ((144, 2, 2), (144, 2), [0], [0], [2], [1], "ijk,ik->ij"),
+        ((9, 48), (9,), [], [], [0], [0], "ij,i->j"),
+        ((3, 4, 5, 6), (6, 3, 5, 2), [0], [1], [2, 3], [2, 0], "bmxy,ybxn->bmn"),
+    ]
+    for sa, sb, ba, bb, ca, cb, spec in cases:
+        a, ra = dev(rng.normal(size=sa), dt)
+        b, rb = dev(rng.normal(size=sb), dt)
+        want = np.einsum(spec, ra, rb)
+        got = host(H._dot_general(a, b, ba, bb, ca, cb))
+        assert got.shape == want.shape, spec
+        assert np.max(np.abs(got - want)) <= tol * np.max(np.abs(want)), spec
+
+
+# ---------------------------------------------------------------------------
+# hlo_call
+# ---------------------------------------------------------------------------
+
+HLO_FFI = """
+module {
+func.func @main(%arg0: tensor<2x2xf32>, %arg1: tensor<f32>) -> (tensor<f32>, tensor<2x2xf32>) {
+%cst = stablehlo.constant dense<0.000000e+00> : tensor<f32>
+%0 = stablehlo.transpose %arg0, dims = [1, 0] : (tensor<2x2xf32>) -> tensor<2x2xf32>
+%1 = stablehlo.reduce(%0 init: %cst) applies stablehlo.add across dimensions = [0, 1] : (tensor<2x2xf32>, tensor<f32>) -> tensor<f32>
+%2 = stablehlo.broadcast_in_dim %arg1, dims = [] : (tensor<f32>) -> tensor<2x2xf32>
+%3 = stablehlo.multiply %0, %2 : tensor<2x2xf32>
+%4 = stablehlo.transpose %3, dims = [1, 0] : (tensor<2x2xf32>) -> tensor<2x2xf32>
+return %1, %4 : tensor<f32>, tensor<2x2xf32>
+}
+}
+"""
+
+
+def test_reference_hlo_call_fixture():
+    """test/testffi.py: a = sum(mat), b = mat * scalar on ones(2, 2) and 2.7, with the
+    fixture's tangents (5.0, 3.1) and cotangents (3.4, 7.0)."""
+    from enzyme_ad.jax import hlo_call, jvp, vjp
+
+    def do_something(mat, scalar):
+        a, b = hlo_call(mat, scalar, source=HLO_FFI)
+        return a, b
+
+    mat, scalar = f32(np.ones((2, 2))), f32(2.7)
+    a, b = do_something(mat, scalar)
+    assert a.shape == () and float(a) == 4.0
+    np.testing.assert_allclose(host(b), np.full((2, 2), 2.7), rtol=1e-7)
+    (a, b), (ta, tb) = jvp(do_something, (mat, scalar), (f32(np.full((2, 2), 5.0)), f32(3.1)))
+    assert float(ta) == 20.0
+    np.testing.assert_allclose(host(tb), np.full((2, 2), 5.0 * 2.7 + 3.1), rtol=1e-6)
+    _, f_vjp = vjp(do_something, mat, scalar)
+    gm, gs = f_vjp((f32(3.4), f32(np.full((2, 2), 7.0))))
+    np.testing.assert_allclose(host(gm), np.full((2, 2), 3.4 + 7.0 * 2.7), rtol=1e-6)
+    np.testing.assert_allclose(float(gs), 28.0, rtol=1e-6)
+
+
+def test_hlo_call_rejects_wrong_arguments():
+    from enzyme_ad.jax import hlo_call
+
+    with pytest.raises(ValueError):
+        hlo_call(f32(np.ones((2, 3))), f32(2.7), source=HLO_FFI)
+    with pytest.raises(AssertionError):
+        hlo_call(f32(np.ones((2, 2))), source=HLO_FFI)
+    with pytest.raises(AssertionError):
+        hlo_call(f32(1.0), source="func.func @f(%a: tensor<f32>) -> tensor<f32> {\n return %a : tensor<f32>\n}")
+    with pytest.raises(NotImplementedError):
+        hlo_call(f32(1.0), source="func.func @main(%a: tensor<f32>) -> tensor<f32> {\n %b = stablehlo.cbrt %a : tensor<f32>\n"
+                                  " return %b : tensor<f32>\n}")
+
+
+ELEMENTWISE = [k for k, v in GOLDEN.items() if isinstance(v, dict) and "grads" in v and "perm" not in v]
+
+
+@pytest.mark.parametrize("name", ELEMENTWISE)
+def test_rule_matches_reference_vector_through_text(name):
+    """The lit tests' operands, results and reverse-mode cotangents (all-ones result cotangent),
+    with the operator written as one line of StableHLO text."""
+    from enzyme_ad.jax import hlo_call, jvp, vjp
+
+    g = GOLDEN[name]
+    n = len(g["args"][0])
+    ty = "tensor<%dxf32>" % n
+    names = ["%a", "%b"][:len(g["args"])]
+    text = "func.func @main(%s) -> %s {\n  %%r = stablehlo.%s %s : %s\n  return %%r : %s\n}\n" % (
+        ", ".join("%s: %s" % (v, ty) for v in names), ty, name, ", ".join(names), ty, ty)
+    args = [f32(a) for a in g["args"]]
+    fn = lambda *xs: hlo_call(*xs, source=text)[0]
+    out, f_vjp = vjp(fn, *args)
+    np.testing.assert_allclose(host(out), g["out"], rtol=2e-6, atol=1e-7)
+    grads = f_vjp(f32(np.ones(n)))
+    for got, want in zip(grads, g["grads"]):
+        np.testing.assert_allclose(host(got), want, rtol=3e-6, atol=1e-7)
+    # forward mode against the same Jacobian: unit tangent on each operand in turn
+    for i, want in enumerate(g["grads"]):
+        tans = [f32(np.ones(n)) if j == i else None for j in range(len(args))]
+        _, t = jvp(fn, tuple(args), tuple(tans))
+        np.testing.assert_allclose(host(t), want, rtol=3e-6, atol=1e-7)
+
+
+def test_transpose_and_dot_general_rules_through_text():
+    from enzyme_ad.jax import hlo_call, vjp
+
+    g = GOLDEN["transpose"]
+    text = ("func.func @main(%a: tensor<2x3xf32>) -> tensor<3x2xf32> {\n"
+            "  %r = stablehlo.transpose %a, dims = [1, 0] : (tensor<2x3xf32>) -> tensor<3x2xf32>\n"
+            "  return %r : tensor<3x2xf32>\n}\n")
+    out, f_vjp = vjp(lambda a: hlo_call(a, source=text)[0], f32(g["args"][0]))
+    assert np.array_equal(host(out), np.asarray(g["out"]))
+    assert np.array_equal(host(f_vjp(f32(g["dret"]))[0]), np.asarray(g["grads"][0]))
+    # dot_general.mlir:4-37: c[3,4] = a[2,3] (dim 0) . b[4,2] (dim 1), quoted-generic spelling
+    text = ('func.func @main(%a : tensor<2x3xf32>, %b : tensor<4x2xf32>) -> tensor<3x4xf32> {\n'
+            '  %c = "stablehlo.dot_general"(%a, %b) {\n'
+            '    dot_dimension_numbers = #stablehlo.dot<\n'
+            '      lhs_batching_dimensions = [], rhs_batching_dimensions = [],\n'
+            '      lhs_contracting_dimensions = [0], rhs_contracting_dimensions = [1]>,\n'
+            '    precision_config = [#stablehlo<precision DEFAULT>, #stablehlo<precision DEFAULT>]\n'
+            '  } : (tensor<2x3xf32>, tensor<4x2xf32>) -> tensor<3x4xf32>\n'
+            '  func.return %c : tensor<3x4xf32>\n}\n')
+    rng = np.random.default_rng(0)
+    a, b, c = rng.normal(size=(2, 3)), rng.normal(size=(4, 2)), rng.normal(size=(3, 4))
+    out, f_vjp = vjp(lambda x, y: hlo_call(x, y, source=text)[0], f32(a), f32(b))
+    np.testing.assert_allclose(host(out), np.einsum("ki,jk->ij", a, b), rtol=1e-5, atol=1e-6)
+    da, db = f_vjp(f32(c))
+    np.testing.assert_allclose(host(da), np.einsum("ij,jk->ki", c, b), rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(host(db), np.einsum("ij,ki->jk", c, a), rtol=1e-5, atol=1e-6)
+
+
+def test_reduce_max_and_broadcast_rules_through_text():
+    """Reduce-maximum sends the cotangent to every maximal element, undivided
+    (StableHLOAutoDiffOpInterfaceImpl.cpp:1881-1916); broadcast_in_dim sums it back (:1474)."""
+    from enzyme_ad.jax import hlo_call, vjp
+
+    text = ("func.func @main(%x: tensor<2x4xf32>, %v: tensor<4xf32>) -> (tensor<2xf32>, tensor<2x4xf32>) {\n"
+            "  %m = stablehlo.constant dense<0xFF800000> : tensor<f32>\n"
+            "  %r = stablehlo.reduce(%x init: %m) applies stablehlo.maximum across dimensions = [1] : "
+            "(tensor<2x4xf32>, tensor<f32>) -> tensor<2xf32>\n"
+            "  %b = stablehlo.broadcast_in_dim %v, dims = [1] : (tensor<4xf32>) -> tensor<2x4xf32>\n"
+            "  return %r, %b : tensor<2xf32>, tensor<2x4xf32>\n}\n")
+    x = f32([[1.0, 3.0, 3.0, -1.0], [0.5, 0.25, -2.0, 0.125]])
+    (r, b), f_vjp = vjp(lambda x, v: tuple(hlo_call(x, v, source=text)), x, f32([1.0, 2.0, 3.0, 4.0]))
+    assert np.array_equal(host(r), [3.0, 0.5])
+    gx, gv = f_vjp((f32([10.0, 20.0]), f32(np.arange(8).reshape(2, 4))))
+    assert np.array_equal(host(gx), [[0, 10.0, 10.0, 0], [20.0, 0, 0, 0]])
+    assert np.array_equal(host(gv), [4.0, 6.0, 8.0, 10.0])

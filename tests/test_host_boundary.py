@@ -163,9 +163,12 @@ def test_python_surface_matches_reference_names():
         ej.enzyme_jax_ir(pipeline_options="not a pipeline")(lambda x: x)
     f = ej.enzyme_jax_ir(argv=("-O3",), pipeline_options=ej.JaXPipeline(), jit_options={"print_mlir": False}, inner_jit=False)(lambda x: x)
     assert f(3) == 3 and f.argv == ("-O3",)
-    for call in (lambda: ej.cpp_call(out_shapes=[], source="void f(){}"), lambda: ej.hlo_call(source="module {}")):
-        with pytest.raises(NotImplementedError):
-            call()
+    with pytest.raises(NotImplementedError):
+        ej.cpp_call(out_shapes=[], source="void f(){}")
+    with pytest.raises(ValueError):                     # a module without a function
+        ej.hlo_call(source="module {}")
+    with pytest.raises(RuntimeError):                   # host tensors: there is no CPU path
+        ej.hlo_call(torch.ones(2), source="func.func @main(%a: tensor<2xf32>) -> tensor<2xf32> {\n return %a : tensor<2xf32>\n}")
     with pytest.raises(TypeError):                      # a tangent for a leaf that is not a floating-point tensor
         ej.jvp(f, (1,), (1,))
     out, tangent = ej.jvp(f, (3,), (None,))             # jax.jvp shape of the result: (primals_out, tangents_out)
