@@ -7,6 +7,7 @@ import os
 import re
 
 import pytest
+import torch
 
 import ffi_frames as F
 
