@@ -125,6 +125,12 @@ def _broadcast(x, shape, dims):
 
 
 def _slice(x, start, limit, stride):
+    if all(st == 1 for st in stride):
+        v = x                                   # unit strides: a view, no kernel; consumers that
+        for d, (s, l) in enumerate(zip(start, limit)):     # need contiguous memory copy it then
+            if s != 0 or l != x.shape[d]:
+                v = v.narrow(d, s, max(0, l - s))
+        return v
     shape = [max(0, -(-(l - s) // st)) for s, l, st in zip(start, limit, stride)]
     out = torch.empty(shape, dtype=x.dtype, device=x.device)
     off = sum(s * xs for s, xs in zip(start, x.stride()))
@@ -220,6 +226,17 @@ def _dot_general(a, b, ba, bb, ca, cb):
     a3 = a.reshape(Bn, K, M) if ta else a.reshape(Bn, M, K)
     b3 = b.reshape(Bn, Nn, K) if tb else b.reshape(Bn, K, Nn)
     o3 = out.reshape(Bn, M, Nn)
+    if Bn >= 8 and M * Nn * K <= 256:
+        # many tiny products (the 2x2 rotations of test/llama.py:161-168 are 144 of them): one
+        # broadcast of each operand to [batch, M, N, K], one multiply, one sum over K
+        box = [Bn, M, Nn, K]
+        sa = (a3.stride(0), a3.stride(2), 0, a3.stride(1)) if ta else (a3.stride(0), a3.stride(1), 0, a3.stride(2))
+        sb = (b3.stride(0), 0, b3.stride(1), b3.stride(2)) if tb else (b3.stride(0), 0, b3.stride(2), b3.stride(1))
+        a4 = torch.empty(box, dtype=a.dtype, device=a.device)
+        b4 = torch.empty(box, dtype=a.dtype, device=a.device)
+        _copy_box(a3, box, sa, 0, a4, _contiguous_strides(box), 0)
+        _copy_box(b3, box, sb, 0, b4, _contiguous_strides(box), 0)
+        return _reduce("add", _bin("multiply", a4, b4), [3]).reshape(out_shape)
     for i in range(Bn):
         if Nn == 1 and M > 1:
             # matrix-vector product (`w @ x`, test/llama.py:149-157): as a one-row product the
@@ -338,6 +355,17 @@ def unary(name, x):
     return y
 
 
+def unary_copy(x):
+    """A fresh contiguous, aligned copy of x (the identity as far as differentiation goes)."""
+    y = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    _copy_box(x, list(x.shape), list(x.stride()), 0, y, _contiguous_strides(x.shape), 0)
+    Tape.record((x,), y, lambda c, acc: (_accumulate(acc[0], c),))
+    tans = _tan(x)
+    if tans is not None and tans[0] is not None:
+        _set_tan(y, tans[0])
+    return y
+
+
 def convert(x, dtype):
     y = _convert(x, dtype)
     Tape.record((x,), y, lambda c, acc: (_accumulate(acc[0], _convert(c, x.dtype)),))
@@ -451,6 +479,8 @@ def slice_(x, start, limit, stride=None):
     start, limit = [int(s) for s in start], [int(l) for l in limit]
     stride = [1] * len(start) if stride is None else [int(s) for s in stride]
     y = _slice(x, start, limit, stride)
+    if y is x:
+        return x
     Tape.record((x,), y, lambda c, acc: (_accumulate(acc[0], _scatter_box(c, list(x.shape), start, stride)),))
     tans = _tan(x)
     if tans is not None and tans[0] is not None:

@@ -282,6 +282,32 @@ def rope(x, n_heads, theta=10000.0, pos0=0, inverse=False):
     return y
 
 
+def rotate_pairs(x, table, inverse=False):
+    """Rotate the adjacent pairs (2p, 2p+1) of the last dimension of x by the angles of an
+    explicit fp32 (cos, sin) table [pairs, 2]: the batched 2x2 products of
+    test/llama.py:161-168 with their constant rotation matrices, as the StableHLO front end
+    finds them in a traced module.  Adjoint = rotation by the negated angles."""
+    _dev(x, table)
+    D = x.shape[-1]
+    if table.dtype != torch.float32 or tuple(table.shape) != (D // 2, 2) or D % 2:
+        raise ValueError("rotate_pairs: table %s/%s for a last dimension of %d" % (tuple(table.shape), table.dtype, D))
+    rows = x.numel() // D
+    y = torch.empty_like(x)
+    N.check(N.lib().emi_rope(_stream(), _p(x), _p(table), _p(y), rows, 1, 1, D, int(inverse), _code(x)))
+
+    def rule(c, acc):
+        g = torch.empty_like(c)
+        N.check(N.lib().emi_rope(_stream(), _p(c), _p(table), _p(g), rows, 1, 1, D, int(not inverse), _code(c)))
+        return (_accumulate(acc[0], g), None)
+
+    Tape.record((x, table), y, rule)
+    tans = _tan(x)
+    if tans is not None and tans[0] is not None:
+        tx = tans[0]
+        _set_tan(y, _quiet(lambda: rotate_pairs(tx, table, inverse)))      # linear in x
+    return y
+
+
 def transpose(a):
     """a^T for a 2-D operand (a fresh buffer; Transpose rule HLODerivatives.td:1334)."""
     _dev(a)

@@ -518,17 +518,81 @@ def _splat(op):
     return float(flat[0])
 
 
-def fuse_clusters(func):
+_FOLD_UNARY = {"negate": np.negative, "exponential": np.exp, "log": np.log, "sqrt": np.sqrt,
+               "rsqrt": lambda v: 1.0 / np.sqrt(v), "tanh": np.tanh, "sine": np.sin, "cosine": np.cos,
+               "logistic": lambda v: 1.0 / (1.0 + np.exp(-v))}
+_FOLD_BINARY = {"add": np.add, "subtract": np.subtract, "multiply": np.multiply, "divide": np.divide,
+                "maximum": np.maximum, "minimum": np.minimum, "power": np.power}
+
+
+def fold_constants(func, limit=4096):
+    """Evaluates, at parse time, operators whose operands are all constants (like
+    `jnp.sqrt(head_size)`, test/llama.py:196, which reaches the text as sqrt of a constant),
+    up to `limit` result elements, in the element type's precision; then drops operators
+    whose results nothing uses."""
+    defs = {}
+    out = []
+    for op in func.ops:
+        srcs = [defs.get(o) for o in op.operands]
+        ty = op.types[0] if op.types else None
+        new = None
+        if op.operands and all(c is not None and c.name == "constant" for c in srcs) and ty is not None \
+                and ty.dtype in ("f32", "bf16") and int(np.prod(ty.shape or (1,))) <= limit:
+            vals = [np.asarray(c.attrs["value"], dtype=np.float32) for c in srcs]
+            if op.name in _FOLD_UNARY:
+                new = _FOLD_UNARY[op.name](vals[0])
+            elif op.name in _FOLD_BINARY:
+                new = _FOLD_BINARY[op.name](vals[0], vals[1])
+            elif op.name == "reshape":
+                new = vals[0].reshape(ty.shape)
+            elif op.name == "transpose":
+                new = vals[0].transpose(op.attrs["perm"])
+            elif op.name == "broadcast_in_dim":
+                shape = [1] * len(ty.shape)
+                for i, d in enumerate(op.attrs["dims"]):
+                    shape[d] = vals[0].shape[i]
+                new = np.broadcast_to(vals[0].reshape(shape), ty.shape)
+            elif op.name == "convert":
+                new = vals[0]
+            if new is not None:
+                new = np.asarray(new, dtype=np.float32)
+                if ty.dtype == "bf16":
+                    new = torch.from_numpy(np.array(new)).to(torch.bfloat16).float().numpy()
+                op = Op("constant", op.results, [], {"value": np.array(new).reshape(ty.shape)}, op.types)
+        for r in op.results:
+            defs[r] = op
+        out.append(op)
+    func.ops = out
+    _drop_dead(func)
+
+
+def _drop_dead(func):
+    live = set()
+    kept = []
+    for op in reversed(func.ops):
+        if op.name == "return" or any(r in live for r in op.results):
+            kept.append(op)
+            live.update(op.operands)
+    func.ops = list(reversed(kept))
+
+
+def fuse_clusters(func, kinds=("rmsnorm", "swiglu", "rope", "softmax_dot", "attention_step")):
     """Rewrites, in place, the operator clusters test/llama.py traces into fused operators:
 
       emi.rmsnorm  w * (x * (1 / sqrt(dot(x, x) / n + eps)))           (llama.py:6-10), also with
                    rsqrt in place of 1 / sqrt (EnzymeHLOOpt.cpp:14907-14923)
       emi.swiglu   a * (1 / (1 + exp(-a))) * b, or a * logistic(a) * b  (llama.py:21-28,229-231)
+      emi.rope     reshape(dot_general(R, reshape(x, (P, 2)))) with constant 2x2 rotations R[P]
+                   (llama.py:127-140,161-168)
       emi.softmax_dot  softmax(dot(K, q) / c) followed by the dot with V  (llama.py:13-18,193-204)
+      emi.attention_step  the concatenation of emi.softmax_dot over consecutive head slices of
+                   one query and one pair of caches (llama.py:178-209)
 
     A cluster is fused only when none of its interior values is used outside it.  Returns
     the number of clusters fused per kind."""
-    counts = {"rmsnorm": 0, "swiglu": 0, "softmax_dot": 0}
+    counts = {"rmsnorm": 0, "swiglu": 0, "rope": 0, "softmax_dot": 0, "attention_step": 0}
+    matchers = [m for k, m in (("rmsnorm", _match_rmsnorm), ("swiglu", _match_swiglu), ("rope", _match_rope),
+                               ("softmax_dot", _match_softmax_dot), ("attention_step", _match_heads)) if k in kinds]
     changed = True
     while changed:
         changed = False
@@ -557,11 +621,15 @@ def fuse_clusters(func):
             return True
 
         for op in func.ops:
-            m = _match_rmsnorm(op, d, through_broadcast) or _match_swiglu(op, d, through_broadcast) or \
-                _match_softmax_dot(op, d, through_broadcast)
+            m = None
+            for matcher in matchers:
+                m = matcher(op, d, through_broadcast)
+                if m is not None:
+                    break
             if m is None:
                 continue
             kind, new_op, interior = m
+            interior = [o for o in interior if o.name != "constant"]
             inner_names = [r for o in interior if o is not op for r in o.results]
             if not only_used_by(inner_names, interior):
                 continue
@@ -571,6 +639,7 @@ def fuse_clusters(func):
             counts[kind] += 1
             changed = True
             break
+    _drop_dead(func)
     return counts
 
 
@@ -725,6 +794,72 @@ def _match_softmax_dot(op, d, tb):
     return None
 
 
+def _match_rope(op, d, tb):
+    # root: reshape(dot_general(R [P,2,2] constant, reshape(x, [P,2]), batch [0]x[0], contract [2]x[1])) -> [2P]
+    if op.name != "reshape" or len(op.types[0].shape) != 1:
+        return None
+    dot = d(op.operands[0])
+    if dot is None or dot.name != "dot_general" or dot.attrs["batch_a"] != [0] or dot.attrs["batch_b"] != [0]:
+        return None
+    if dot.attrs["contract_a"] != [2] or dot.attrs["contract_b"] != [1]:
+        return None
+    rot, inner = d(dot.operands[0]), d(dot.operands[1])
+    if rot is None or rot.name != "constant" or inner is None or inner.name != "reshape":
+        return None
+    R = np.asarray(rot.attrs["value"], dtype=np.float64)
+    P = op.types[0].shape[0] // 2
+    if R.shape != (P, 2, 2) or tuple(inner.types[0].shape) != (P, 2):
+        return None
+    c, s_ = R[:, 0, 0], R[:, 1, 0]
+    if not (np.array_equal(R[:, 1, 1], c) and np.array_equal(R[:, 0, 1], -s_)):
+        return None
+    if np.max(np.abs(c * c + s_ * s_ - 1.0)) > 1e-5:
+        return None
+    table = np.stack([c, s_], axis=1).astype(np.float32)
+    return "rope", Op("emi.rope", op.results, [inner.operands[0]], {"table": table}, op.types), [op, dot, inner]
+
+
+def _match_heads(op, d, tb):
+    # root: concatenate(dim 0) of emi.softmax_dot(q_h, K_h, V_h) over head slices h = 0..n-1
+    if op.name != "concatenate" or op.attrs["dim"] != 0 or len(op.operands) < 2:
+        return None
+    heads = [d(o) for o in op.operands]
+    if any(h is None or h.name != "emi.softmax_dot" for h in heads):
+        return None
+    scale = heads[0].attrs["scale"]
+    q = kc = vc = None
+    hs = heads[0].types[0].shape[0]
+    interior = [op]
+    for h, sd in enumerate(heads):
+        if sd.attrs["scale"] != scale or tuple(sd.types[0].shape) != (hs,):
+            return None
+        sl = [d(o) for o in sd.operands]
+        if any(x is None or x.name != "slice" for x in sl):
+            return None
+        qs, ks, vs = sl
+        if qs.attrs["start"] != [h * hs] or qs.attrs["limit"] != [(h + 1) * hs] or qs.attrs["stride"] != [1]:
+            return None
+        for cs in (ks, vs):
+            if len(cs.attrs["start"]) != 2 or cs.attrs["start"][0] != 0 or cs.attrs["stride"] != [1, 1]:
+                return None
+            if cs.attrs["start"][1] != h * hs or cs.attrs["limit"][1] != (h + 1) * hs:
+                return None
+        if h == 0:
+            q, kc, vc = qs.operands[0], ks.operands[0], vs.operands[0]
+            rows = ks.attrs["limit"][0]
+        if (qs.operands[0], ks.operands[0], vs.operands[0]) != (q, kc, vc):
+            return None
+        if ks.attrs["limit"][0] != rows or vs.attrs["limit"][0] != rows:
+            return None
+        interior += [sd, qs, ks, vs]
+    n = len(heads)
+    if tuple(op.types[0].shape) != (n * hs,):
+        return None
+    # the caches must be exactly [rows, n * hs] and the query [n * hs]: checked when run
+    new = Op("emi.attention_step", op.results, [q, kc, vc], {"scale": scale, "heads": n, "rows": rows}, op.types)
+    return "attention_step", new, interior
+
+
 # ---------------------------------------------------------------------------
 # executor
 # ---------------------------------------------------------------------------
@@ -733,11 +868,15 @@ class Executable:
     """A parsed module ready to run on one device."""
 
     def __init__(self, text, fuse=True):
+        """fuse: True (all clusters), False (none), or a tuple of cluster kinds."""
         self.funcs = parse_module(text)
         self.fused = {}
-        if fuse:
-            for f in self.funcs.values():
-                for k, v in fuse_clusters(f).items():
+        for f in self.funcs.values():
+            fold_constants(f)
+            if fuse:
+                kinds = fuse if isinstance(fuse, (tuple, list)) else \
+                    ("rmsnorm", "swiglu", "rope", "softmax_dot", "attention_step")
+                for k, v in fuse_clusters(f, kinds).items():
                     self.fused[k] = self.fused.get(k, 0) + v
         self._consts = {}
 
@@ -824,21 +963,42 @@ class Executable:
         if n == "call":
             return self.run(xs, op.attrs["callee"])
         if n == "emi.rmsnorm":
-            x, w = xs
+            x, w = _packed(xs[0]), _packed(xs[1])
             return [ops.reshape(ops.rmsnorm(ops.reshape(x, (1, x.shape[0])), w, op.attrs["eps"]), tuple(x.shape))]
         if n == "emi.swiglu":
-            return [ops.swiglu(H._contig(xs[0]), H._contig(xs[1]))]
+            return [ops.swiglu(_packed(xs[0]), _packed(xs[1]))]
+        if n == "emi.rope":
+            key = (id(op), "table", str(device))
+            table = self._consts.get(key)
+            if table is None:
+                table = self._consts[key] = torch.from_numpy(op.attrs["table"]).to(device)
+            return [ops.rotate_pairs(_packed(xs[0]), table)]
         if n == "emi.softmax_dot":
             q, k, v = xs
-            return [ops.attention_step(q, H._contig(k), H._contig(v), 1, op.attrs["scale"])]
+            return [ops.attention_step(_packed(q), _packed(k), _packed(v), 1, op.attrs["scale"])]
+        if n == "emi.attention_step":
+            q, k, v = xs
+            heads, rows = op.attrs["heads"], op.attrs["rows"]
+            if q.dim() != 1 or k.shape != (rows, q.shape[0]) or v.shape != k.shape:
+                raise RuntimeError("attention cluster: query %s, caches %s / %s do not form %d heads over %d rows" %
+                                   (tuple(q.shape), tuple(k.shape), tuple(v.shape), heads, rows))
+            return [ops.attention_step(_packed(q), _packed(k), _packed(v), heads, op.attrs["scale"])]
         raise NotImplementedError("StableHLO operator '%s' is not supported by the HIP front end" % n)
+
+
+def _packed(t):
+    """Contiguous and 16-byte aligned, as the fused kernels want their operands; a view that
+    is neither is copied (tracked, so cotangents flow back to the view's source)."""
+    if t.is_contiguous() and t.data_ptr() % 16 == 0:
+        return t
+    return H.unary_copy(t)
 
 
 _CACHE = {}
 
 
 def compile_text(text, fuse=True):
-    key = (text, fuse)
+    key = (text, tuple(fuse) if isinstance(fuse, (tuple, list)) else fuse)
     exe = _CACHE.get(key)
     if exe is None:
         exe = _CACHE[key] = Executable(text, fuse)
