@@ -160,6 +160,36 @@ def bench_kernels(cfg, iters):
         hbm("rope_fwd_" + tag, lambda: N.check(lib.emi_rope(st, P(x), P(table), P(y), 16, 2048, 32, 128, 0, code)), 2 * n * s)
         hbm("rope_bwd_" + tag, lambda: N.check(lib.emi_rope(st, P(dy), P(table), P(y), 16, 2048, 32, 128, 1, code)), 2 * n * s)
         del x, dy, y, ws
+    # Generic operators of the StableHLO front end at the C2 size [32768, 4096]: elementwise maps
+    # (multiply reads 2, writes 1; exponential reads 1, writes 1), convert, a row broadcast
+    # (writes N), the transpose through the strided copy, and sums over rows and columns.
+    from enzyme_ad.jax import hlo_ops as HO
+    import ctypes
+    rows, D = 16 * 2048, 4096
+    n = rows * D
+    i64 = lambda xs: (ctypes.c_int64 * len(xs))(*xs)
+    for dt, s, code in ((bf, 2, N.EMI_BF16), (torch.float32, 4, N.EMI_F32)):
+        tag = "bf16" if dt == bf else "f32"
+        a, b = (torch.randn((rows, D), device="cuda").to(dt) for _ in range(2))
+        y = torch.empty_like(a)
+        row = torch.randn(D, device="cuda").to(dt)
+        col = torch.empty(rows, device="cuda").to(dt)
+        hbm("map_multiply_" + tag, lambda: N.check(lib.emi_map_binary(st, HO.BINARY["multiply"], P(a), P(b), P(y), n, 0, 0, code)), 3 * n * s)
+        hbm("map_exp_" + tag, lambda: N.check(lib.emi_map_unary(st, HO.UNARY["exponential"], P(a), P(y), n, code)), 2 * n * s)
+        hbm("broadcast_row_" + tag, lambda: N.check(lib.emi_strided_copy(st, P(row), P(y), 2, i64([rows, D]), i64([0, 1]), 0,
+                                                                         i64([D, 1]), 0, s)), n * s)
+        hbm("transpose_copy_" + tag, lambda: N.check(lib.emi_strided_copy(st, P(a), P(y), 2, i64([D, rows]), i64([1, D]), 0,
+                                                                          i64([rows, 1]), 0, s)), 2 * n * s)
+        rwb = max(lib.emi_reduce_workspace_bytes(1, rows, D, code), lib.emi_reduce_workspace_bytes(1, n, 1, code), 16)
+        rws = torch.empty(rwb, dtype=torch.uint8, device="cuda")
+        hbm("reduce_rows_" + tag, lambda: N.check(lib.emi_reduce(st, HO.REDUCE["add"], P(a), P(col), None, 0, rows, D, 1, code)), n * s)
+        hbm("reduce_cols_" + tag, lambda: N.check(lib.emi_reduce(st, HO.REDUCE["add"], P(a), P(row), P(rws), rwb, 1, rows, D, code)), n * s)
+        hbm("reduce_all_" + tag, lambda: N.check(lib.emi_reduce(st, HO.REDUCE["add"], P(a), P(col), P(rws), rwb, 1, n, 1, code)), n * s)
+        if dt == torch.float32:
+            yb = torch.empty((rows, D), dtype=bf, device="cuda")
+            hbm("convert_f32_bf16", lambda: N.check(lib.emi_convert(st, P(a), P(yb), n, N.EMI_F32, N.EMI_BF16)), n * 6)
+            del yb
+        del a, b, y
     # C5 SwiGLU: [16384, 11008] bf16
     T, H = cfg["batch"] * cfg["seq"], cfg["hidden_dim"]
     a, b, dg = (torch.randn((T, H), device="cuda").to(bf) for _ in range(3))

@@ -12,6 +12,11 @@ constexpr int kBlock = 256;
 constexpr int kMaxRank = 8;
 
 inline bool al16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+// one lane per group of eight elements plus one per leftover element (VEC), or per element
+inline unsigned map_grid(int64_t n, bool vec) {
+  const int64_t lanes = vec ? (n >> 3) + (n & 7) : n;
+  return (unsigned)((lanes + kBlock - 1) / kBlock);
+}
 inline unsigned grid_for(int64_t items, int per_block) {
   int64_t g = (items + per_block - 1) / per_block;
   const int64_t cap = 256 * 32;  // 32 blocks per CU: grid-stride loops cover the rest
@@ -64,76 +69,72 @@ template <int OP> __device__ __forceinline__ float apply_unary(float a) {
 }
 
 // y[i] = op(a[i * sa], b[i * sb]); sa, sb in {0, 1} (0: the operand is one element).
-// VEC: chunks of 16 bytes per lane over the first n - n % N elements, lane-serial tail.
+// VEC: one group of eight elements per lane (16 bytes of bf16, 2 x 16 bytes of fp32), enough
+// workgroups to cover the tensor; the last n % 8 elements go to the lanes after the groups.
 template <typename T, bool VEC, int OP>
 __global__ void __launch_bounds__(kBlock) map_binary_kernel(const T* __restrict__ a, const T* __restrict__ b,
                                                             T* __restrict__ y, int64_t n, int sa, int sb) {
-  constexpr int N = Chunk<T>::N;
-  const int64_t tid = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  const int64_t nthreads = (int64_t)gridDim.x * kBlock;
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (VEC) {
-    const int64_t nchunks = n / N;
-    float fa[N], fb[N], fy[N];
-    if (!sa) { const float s = to_f32(a[0]);
+    const int64_t ngroups = n >> 3;
+    if (i < ngroups) {
+      float fa[8], fb[8];
+      if (sa) Vec8<T>::load(a + i * 8, fa);
+      if (sb) Vec8<T>::load(b + i * 8, fb);
+      if (!sa) { const float v = to_f32(a[0]);
 #pragma unroll
-      for (int j = 0; j < N; j++) fa[j] = s; }
-    if (!sb) { const float s = to_f32(b[0]);
+        for (int j = 0; j < 8; j++) fa[j] = v; }
+      if (!sb) { const float v = to_f32(b[0]);
 #pragma unroll
-      for (int j = 0; j < N; j++) fb[j] = s; }
-    for (int64_t c = tid; c < nchunks; c += nthreads) {
-      if (sa) Chunk<T>::load(a + c * N, fa);
-      if (sb) Chunk<T>::load(b + c * N, fb);
+        for (int j = 0; j < 8; j++) fb[j] = v; }
 #pragma unroll
-      for (int j = 0; j < N; j++) fy[j] = apply_binary<OP>(fa[j], fb[j]);
-      Chunk<T>::store(y + c * N, fy);
+      for (int j = 0; j < 8; j++) fa[j] = apply_binary<OP>(fa[j], fb[j]);
+      Vec8<T>::store(y + i * 8, fa);
+    } else if (i - ngroups < (n & 7)) {
+      const int64_t e = (ngroups << 3) + (i - ngroups);
+      y[e] = from_f32<T>(apply_binary<OP>(to_f32(a[sa ? e : 0]), to_f32(b[sb ? e : 0])));
     }
-    const int64_t i = nchunks * N + tid;
-    if (i < n) y[i] = from_f32<T>(apply_binary<OP>(to_f32(a[sa ? i : 0]), to_f32(b[sb ? i : 0])));
-  } else {
-    for (int64_t i = tid; i < n; i += nthreads)
-      y[i] = from_f32<T>(apply_binary<OP>(to_f32(a[sa ? i : 0]), to_f32(b[sb ? i : 0])));
+  } else if (i < n) {
+    y[i] = from_f32<T>(apply_binary<OP>(to_f32(a[sa ? i : 0]), to_f32(b[sb ? i : 0])));
   }
 }
 
 template <typename T, bool VEC, int OP>
 __global__ void __launch_bounds__(kBlock) map_unary_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t n) {
-  constexpr int N = Chunk<T>::N;
-  const int64_t tid = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  const int64_t nthreads = (int64_t)gridDim.x * kBlock;
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (VEC) {
-    const int64_t nchunks = n / N;
-    float fx[N], fy[N];
-    for (int64_t c = tid; c < nchunks; c += nthreads) {
-      Chunk<T>::load(x + c * N, fx);
+    const int64_t ngroups = n >> 3;
+    if (i < ngroups) {
+      float f[8];
+      Vec8<T>::load(x + i * 8, f);
 #pragma unroll
-      for (int j = 0; j < N; j++) fy[j] = apply_unary<OP>(fx[j]);
-      Chunk<T>::store(y + c * N, fy);
+      for (int j = 0; j < 8; j++) f[j] = apply_unary<OP>(f[j]);
+      Vec8<T>::store(y + i * 8, f);
+    } else if (i - ngroups < (n & 7)) {
+      const int64_t e = (ngroups << 3) + (i - ngroups);
+      y[e] = from_f32<T>(apply_unary<OP>(to_f32(x[e])));
     }
-    const int64_t i = nchunks * N + tid;
-    if (i < n) y[i] = from_f32<T>(apply_unary<OP>(to_f32(x[i])));
-  } else {
-    for (int64_t i = tid; i < n; i += nthreads) y[i] = from_f32<T>(apply_unary<OP>(to_f32(x[i])));
+  } else if (i < n) {
+    y[i] = from_f32<T>(apply_unary<OP>(to_f32(x[i])));
   }
 }
 
-template <typename TI, typename TO>
+template <typename TI, typename TO, bool VEC>
 __global__ void __launch_bounds__(kBlock) convert_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t n) {
-  const int64_t tid = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  const int64_t nthreads = (int64_t)gridDim.x * kBlock;
-  const int64_t nchunks = n / 8;
-  float v[8];
-  for (int64_t c = tid; c < nchunks; c += nthreads) {
-    Vec8<TI>::load(x + c * 8, v);
-    Vec8<TO>::store(y + c * 8, v);
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (VEC) {
+    const int64_t ngroups = n >> 3;
+    if (i < ngroups) {
+      float v[8];
+      Vec8<TI>::load(x + i * 8, v);
+      Vec8<TO>::store(y + i * 8, v);
+    } else if (i - ngroups < (n & 7)) {
+      const int64_t e = (ngroups << 3) + (i - ngroups);
+      y[e] = from_f32<TO>(to_f32(x[e]));
+    }
+  } else if (i < n) {
+    y[i] = from_f32<TO>(to_f32(x[i]));
   }
-  const int64_t i = nchunks * 8 + tid;
-  if (i < n) y[i] = from_f32<TO>(to_f32(x[i]));
-}
-
-template <typename TI, typename TO>
-__global__ void __launch_bounds__(kBlock) convert_scalar_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t n) {
-  const int64_t tid = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  for (int64_t i = tid; i < n; i += (int64_t)gridDim.x * kBlock) y[i] = from_f32<TO>(to_f32(x[i]));
 }
 
 // ---------------------------------------------------------------------------
@@ -193,8 +194,113 @@ __global__ void __launch_bounds__(kBlock) strided_copy32_kernel(const E* __restr
   }
 }
 
+// A permutation whose innermost result index is not the innermost source index: 64 x 64
+// tiles over (dt = the index that is contiguous in the source, last = the index that is
+// contiguous in the result) staged through LDS so that both sides move whole rows; the other
+// indices are enumerated by blockIdx.z.
+struct TilePlan {
+  int nouter;                  // indices other than dt and last
+  int64_t n_dt, n_last, is_last, os_dt;
+  int64_t dims[kMaxRank], is[kMaxRank], os[kMaxRank];
+};
+
+template <typename E>
+__global__ void __launch_bounds__(kBlock) tiled_permute_kernel(const E* __restrict__ in, E* __restrict__ out, TilePlan p,
+                                                               int vec_ok) {
+  constexpr int TS = 64, PADW = TS + (sizeof(E) == 2 ? 2 : 1);
+  __shared__ E tile[TS][PADW];
+  int64_t rem = blockIdx.z, ib = 0, ob = 0;
+#pragma unroll
+  for (int d = kMaxRank - 1; d >= 0; d--) {
+    if (d < p.nouter) {
+      const int64_t q = rem / p.dims[d], r = rem - q * p.dims[d];
+      ib += r * p.is[d];
+      ob += r * p.os[d];
+      rem = q;
+    }
+  }
+  in += ib;
+  out += ob;
+  const int64_t r0 = (int64_t)blockIdx.y * TS, c0 = (int64_t)blockIdx.x * TS;   // r: last index, c: dt index
+  const int t = threadIdx.x;
+  if (vec_ok && r0 + TS <= p.n_last && c0 + TS <= p.n_dt) {
+    constexpr int V = 16 / sizeof(E);
+    constexpr int CPR = TS / V;
+#pragma unroll
+    for (int i = 0; i < TS * CPR / kBlock; i++) {
+      const int idx = t + i * kBlock, r = idx / CPR, c = (idx % CPR) * V;
+      const uint4 v = *reinterpret_cast<const uint4*>(in + (r0 + r) * p.is_last + c0 + c);
+      const E* e = reinterpret_cast<const E*>(&v);
+#pragma unroll
+      for (int j = 0; j < V; j++) tile[r][c + j] = e[j];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < TS * CPR / kBlock; i++) {
+      const int idx = t + i * kBlock, c = idx / CPR, r = (idx % CPR) * V;
+      uint4 v;
+      E* e = reinterpret_cast<E*>(&v);
+#pragma unroll
+      for (int j = 0; j < V; j++) e[j] = tile[r + j][c];
+      *reinterpret_cast<uint4*>(out + (c0 + c) * p.os_dt + r0 + r) = v;
+    }
+  } else {
+    for (int idx = t; idx < TS * TS; idx += kBlock) {
+      const int r = idx / TS, c = idx % TS;
+      if (r0 + r < p.n_last && c0 + c < p.n_dt) tile[r][c] = in[(r0 + r) * p.is_last + c0 + c];
+    }
+    __syncthreads();
+    for (int idx = t; idx < TS * TS; idx += kBlock) {
+      const int c = idx / TS, r = idx % TS;
+      if (r0 + r < p.n_last && c0 + c < p.n_dt) out[(c0 + c) * p.os_dt + r0 + r] = tile[r][c];
+    }
+  }
+}
+
+// Tries the tiled form; returns false when the plan does not have it (then the generic
+// kernel runs).
+template <typename E>
+bool launch_tiled(hipStream_t st, const void* in, void* out, const CopyPlan& p, int* status) {
+  const int l = p.rank - 1;
+  if (p.rank < 2 || p.os[l] != 1 || p.is[l] == 1 || p.is[l] == 0) return false;
+  int dt = -1;
+  for (int d = 0; d < l; d++)
+    if (p.is[d] == 1 && p.dims[d] >= 16) dt = d;
+  if (dt < 0 || p.dims[l] < 16) return false;
+  TilePlan t;
+  t.nouter = 0;
+  t.n_dt = p.dims[dt];
+  t.n_last = p.dims[l];
+  t.is_last = p.is[l];
+  t.os_dt = p.os[dt];
+  int64_t nz = 1;
+  for (int d = 0; d < l; d++) {
+    if (d == dt) continue;
+    t.dims[t.nouter] = p.dims[d];
+    t.is[t.nouter] = p.is[d];
+    t.os[t.nouter] = p.os[d];
+    t.nouter++;
+    nz *= p.dims[d];
+  }
+  for (int d = t.nouter; d < kMaxRank; d++) { t.dims[d] = 1; t.is[d] = 0; t.os[d] = 0; }
+  const int64_t gx = (t.n_dt + 63) / 64, gy = (t.n_last + 63) / 64;
+  if (nz > 65535 || gy > 65535) return false;
+  constexpr int V = 16 / sizeof(E);
+  int vec_ok = sizeof(E) <= 4 && al16(in) && al16(out) && t.is_last % V == 0 && t.os_dt % V == 0;
+  for (int d = 0; d < t.nouter && vec_ok; d++) vec_ok = t.is[d] % V == 0 && t.os[d] % V == 0;
+  hipLaunchKernelGGL(tiled_permute_kernel<E>, dim3((unsigned)gx, (unsigned)gy, (unsigned)nz), dim3(kBlock), 0, st,
+                     static_cast<const E*>(in), static_cast<E*>(out), t, vec_ok);
+  hipError_t e = hipGetLastError();
+  *status = e == hipSuccess ? EMI_OK : emi_fail(EMI_INTERNAL, "emi_strided_copy: launch failed: %s", hipGetErrorString(e));
+  return true;
+}
+
 template <typename E>
 int launch_copy(hipStream_t st, const void* in, void* out, const CopyPlan& p) {
+  int status = EMI_OK;
+  if constexpr (sizeof(E) <= 8) {
+    if (launch_tiled<E>(st, in, out, p, &status)) return status;
+  }
   const unsigned grid = grid_for(p.total, kBlock);
   if (p.total < 0x7fffffffLL)
     hipLaunchKernelGGL(strided_copy32_kernel<E>, dim3(grid), dim3(kBlock), 0, st, static_cast<const E*>(in),
@@ -220,29 +326,47 @@ template <int OP> __device__ __forceinline__ float wave_red(float v) {
   return v;
 }
 
-// inner == 1: one workgroup of WAVES waves per row; lanes stride over 16-byte chunks when the
-// rows are 16-byte aligned (VEC), elements otherwise.
-template <typename T, int OP, int WAVES, bool VEC>
-__global__ void __launch_bounds__(WAVES * kWave) reduce_rows_kernel(const T* __restrict__ x, T* __restrict__ y,
-                                                                    int64_t rows, int64_t red) {
+// inner == 1.  Row `row` of x is split into `nsplit` segments of `seg` elements; workgroup
+// (row, s) reduces segment s with WAVES waves, lanes striding over 16-byte chunks (VEC: the
+// segments start 16-byte aligned) or elements, and writes either the result (nsplit == 1,
+// TO = T) or an fp32 partial [row, s] for the second stage.
+template <typename T, typename TO, int OP, int WAVES, bool VEC>
+__global__ void __launch_bounds__(WAVES * kWave) reduce_rows_kernel(const T* __restrict__ x, TO* __restrict__ y,
+                                                                    int64_t rows, int64_t red, int64_t seg, int nsplit) {
   constexpr int N = Chunk<T>::N;
   __shared__ float part[WAVES];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
-    const T* xr = x + row * red;
-    float acc = red_init<OP>();
+  for (int64_t item = blockIdx.x; item < rows * nsplit; item += gridDim.x) {
+    const int64_t row = item / nsplit, sidx = item - row * nsplit;
+    const int64_t lo = sidx * seg, hi = lo + seg < red ? lo + seg : red;
+    const T* xr = x + row * red + lo;
+    const int64_t len = hi - lo;
+    float a0 = red_init<OP>(), a1 = a0;
     if (VEC) {
-      const int64_t nchunks = red / N;
+      const int64_t nchunks = len / N;
+      typename Chunk<T>::Raw r0, r1;
       float v[N];
-      for (int64_t c = threadIdx.x; c < nchunks; c += WAVES * kWave) {
+      int64_t c = threadIdx.x;
+      for (; c + WAVES * kWave < nchunks; c += 2 * WAVES * kWave) {       // two loads in flight
+        r0 = Chunk<T>::load_raw(xr + c * N);
+        r1 = Chunk<T>::load_raw(xr + (c + WAVES * kWave) * N);
+        Chunk<T>::unpack(r0, v);
+#pragma unroll
+        for (int j = 0; j < N; j++) a0 = red_op<OP>(a0, v[j]);
+        Chunk<T>::unpack(r1, v);
+#pragma unroll
+        for (int j = 0; j < N; j++) a1 = red_op<OP>(a1, v[j]);
+      }
+      if (c < nchunks) {
         Chunk<T>::load(xr + c * N, v);
 #pragma unroll
-        for (int j = 0; j < N; j++) acc = red_op<OP>(acc, v[j]);
+        for (int j = 0; j < N; j++) a0 = red_op<OP>(a0, v[j]);
       }
+      for (int64_t i = nchunks * N + threadIdx.x; i < len; i += WAVES * kWave) a1 = red_op<OP>(a1, to_f32(xr[i]));
     } else {
-      for (int64_t i = threadIdx.x; i < red; i += WAVES * kWave) acc = red_op<OP>(acc, to_f32(xr[i]));
+      for (int64_t i = threadIdx.x; i < len; i += WAVES * kWave) a0 = red_op<OP>(a0, to_f32(xr[i]));
     }
-    acc = wave_red<OP>(acc);
+    float acc = wave_red<OP>(red_op<OP>(a0, a1));
     if (WAVES > 1) {
       __syncthreads();
       if (lane == 0) part[wave] = acc;
@@ -251,49 +375,174 @@ __global__ void __launch_bounds__(WAVES * kWave) reduce_rows_kernel(const T* __r
 #pragma unroll
       for (int w = 1; w < WAVES; w++) acc = red_op<OP>(acc, part[w]);
     }
-    if (threadIdx.x == 0) y[row] = from_f32<T>(acc);
+    if (threadIdx.x == 0) y[item] = from_f32<TO>(acc);
   }
 }
 
-// inner > 1: one lane per (outer, inner) result, coalesced over inner.
-template <typename T, int OP>
-__global__ void __launch_bounds__(kBlock) reduce_cols_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t outer,
-                                                             int64_t red, int64_t inner) {
-  const int64_t tid = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  const int64_t total = outer * inner;
-  for (int64_t i = tid; i < total; i += (int64_t)gridDim.x * kBlock) {
-    const int64_t o = i / inner, c = i - o * inner;
-    const T* p = x + o * red * inner + c;
-    float a0 = red_init<OP>(), a1 = a0, a2 = a0, a3 = a0;
-    int64_t r = 0;
-    for (; r + 4 <= red; r += 4) {
-      a0 = red_op<OP>(a0, to_f32(p[(r + 0) * inner]));
-      a1 = red_op<OP>(a1, to_f32(p[(r + 1) * inner]));
-      a2 = red_op<OP>(a2, to_f32(p[(r + 2) * inner]));
-      a3 = red_op<OP>(a3, to_f32(p[(r + 3) * inner]));
+// inner > 1: x [outer, red, inner].  Lane = one 16-byte chunk of columns (VEC) or one column;
+// blockIdx.y = band of `band` rows, blockIdx.z = outer.  Writes the result (nsplit == 1) or
+// an fp32 partial [band, outer, inner].
+template <typename T, typename TO, int OP, bool VEC>
+__global__ void __launch_bounds__(kBlock) reduce_cols_kernel(const T* __restrict__ x, TO* __restrict__ y, int64_t outer,
+                                                             int64_t red, int64_t inner, int64_t band) {
+  constexpr int N = VEC ? Chunk<T>::N : 1;
+  const int64_t col = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * N;
+  if (col >= inner) return;
+  const int64_t o = blockIdx.z, r0 = (int64_t)blockIdx.y * band, r1 = r0 + band < red ? r0 + band : red;
+  const T* p = x + (o * red + r0) * inner + col;
+  float acc[N], acc2[N];
+#pragma unroll
+  for (int j = 0; j < N; j++) acc[j] = acc2[j] = red_init<OP>();
+  int64_t r = r0;
+  if (VEC) {
+    float v[Chunk<T>::N];
+    constexpr int UN = 8;                                   // row loads in flight per lane
+    for (; r + UN <= r1; r += UN) {
+      typename Chunk<T>::Raw q[UN];
+#pragma unroll
+      for (int u = 0; u < UN; u++) q[u] = Chunk<T>::load_raw(p + u * inner);
+      p += UN * inner;
+#pragma unroll
+      for (int u = 0; u < UN; u++) {
+        Chunk<T>::unpack(q[u], v);
+        if (u & 1) {
+#pragma unroll
+          for (int j = 0; j < N; j++) acc2[j] = red_op<OP>(acc2[j], v[j]);
+        } else {
+#pragma unroll
+          for (int j = 0; j < N; j++) acc[j] = red_op<OP>(acc[j], v[j]);
+        }
+      }
     }
-    for (; r < red; r++) a0 = red_op<OP>(a0, to_f32(p[r * inner]));
-    y[i] = from_f32<T>(red_op<OP>(red_op<OP>(a0, a1), red_op<OP>(a2, a3)));
-  }
-}
-
-template <typename T, int OP>
-int launch_reduce(hipStream_t st, const void* x, void* y, int64_t outer, int64_t red, int64_t inner) {
-  const T* xp = static_cast<const T*>(x);
-  T* yp = static_cast<T*>(y);
-  if (inner == 1) {
-    const bool vec = al16(x) && red % Chunk<T>::N == 0;
-    const unsigned grid = (unsigned)(outer < 65536 ? outer : 65536);
-    if (red <= 2048) {
-      if (vec) hipLaunchKernelGGL((reduce_rows_kernel<T, OP, 1, true>), dim3(grid), dim3(64), 0, st, xp, yp, outer, red);
-      else hipLaunchKernelGGL((reduce_rows_kernel<T, OP, 1, false>), dim3(grid), dim3(64), 0, st, xp, yp, outer, red);
-    } else {
-      if (vec) hipLaunchKernelGGL((reduce_rows_kernel<T, OP, 16, true>), dim3(grid), dim3(1024), 0, st, xp, yp, outer, red);
-      else hipLaunchKernelGGL((reduce_rows_kernel<T, OP, 16, false>), dim3(grid), dim3(1024), 0, st, xp, yp, outer, red);
+    for (; r < r1; r++, p += inner) {
+      Chunk<T>::load(p, v);
+#pragma unroll
+      for (int j = 0; j < N; j++) acc[j] = red_op<OP>(acc[j], v[j]);
     }
   } else {
-    hipLaunchKernelGGL((reduce_cols_kernel<T, OP>), dim3(grid_for(outer * inner, kBlock)), dim3(kBlock), 0, st, xp, yp,
-                       outer, red, inner);
+    for (; r < r1; r++, p += inner) acc[0] = red_op<OP>(acc[0], to_f32(*p));
+  }
+  TO* yp = y + ((int64_t)blockIdx.y * outer + o) * inner + col;
+#pragma unroll
+  for (int j = 0; j < N; j++) yp[j] = from_f32<TO>(red_op<OP>(acc[j], acc2[j]));
+}
+
+// second stage of the column form: y[m] = reduce over s of part[s, m].  A workgroup owns 64
+// columns; its 16 waves take the partial rows s = wave, wave + 16, ... with eight loads in
+// flight each and meet in LDS, so the pass costs a few round trips to memory, not nsplit.
+template <typename T, int OP>
+__global__ void __launch_bounds__(1024) reduce_partials_kernel(const float* __restrict__ part, T* __restrict__ y,
+                                                               int64_t m, int nsplit) {
+  __shared__ float sh[16][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t i = (int64_t)blockIdx.x * 64 + lane;
+  float acc = red_init<OP>();
+  if (i < m) {
+    int s = wave;
+    for (; s + 7 * 16 < nsplit; s += 8 * 16) {
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; u++) v[u] = part[(int64_t)(s + u * 16) * m + i];
+#pragma unroll
+      for (int u = 0; u < 8; u++) acc = red_op<OP>(acc, v[u]);
+    }
+    for (; s < nsplit; s += 16) acc = red_op<OP>(acc, part[(int64_t)s * m + i]);
+  }
+  sh[wave][lane] = acc;
+  __syncthreads();
+  if (wave == 0 && i < m) {
+#pragma unroll
+    for (int w = 1; w < 16; w++) acc = red_op<OP>(acc, sh[w][lane]);
+    y[i] = from_f32<T>(acc);
+  }
+}
+
+struct ReducePlan {
+  int nsplit;          // 1: single pass
+  int64_t seg;         // rows form: elements per segment; column form: rows per band
+};
+
+// Enough workgroups to fill 256 CUs a few times over; segments keep 16-byte alignment.
+template <typename T>
+ReducePlan reduce_plan(int64_t outer, int64_t red, int64_t inner) {
+  ReducePlan p{1, red};
+  const int64_t want = 2048;
+  if (inner == 1) {
+    if (outer >= want / 2 || red < 16384) return p;
+    int64_t ns = (want + outer - 1) / outer;
+    int64_t seg = (red + ns - 1) / ns;
+    seg = (seg + 1023) / 1024 * 1024;                       // multiple of every chunk size
+    if (seg < 8192) seg = 8192;
+    ns = (red + seg - 1) / seg;
+    if (ns > 1) { p.nsplit = (int)ns; p.seg = seg; }
+  } else {
+    const int64_t lanes = (inner + Chunk<T>::N - 1) / Chunk<T>::N;
+    const int64_t blocks = ((lanes + kBlock - 1) / kBlock) * outer;
+    if (blocks >= want / 2 || red < 64) return p;
+    int64_t ns = (want + blocks - 1) / blocks;
+    int64_t band = (red + ns - 1) / ns;
+    if (band < 64) band = 64;
+    ns = (red + band - 1) / band;
+    if (ns > 1024) { ns = 1024; band = (red + ns - 1) / ns; ns = (red + band - 1) / band; }
+    if (ns > 1) { p.nsplit = (int)ns; p.seg = band; }
+  }
+  return p;
+}
+
+template <typename T>
+size_t reduce_workspace(int64_t outer, int64_t red, int64_t inner) {
+  const ReducePlan p = reduce_plan<T>(outer, red, inner);
+  return p.nsplit == 1 ? 0 : (size_t)p.nsplit * (size_t)outer * (size_t)inner * sizeof(float);
+}
+
+template <typename T, typename TO, int OP>
+void launch_rows(hipStream_t st, const T* x, TO* y, int64_t rows, int64_t red, int64_t seg, int nsplit) {
+  const int64_t items = rows * nsplit;
+  const unsigned grid = (unsigned)(items < 262144 ? items : 262144);
+  const bool vec = al16(x) && red % Chunk<T>::N == 0 && seg % Chunk<T>::N == 0;
+  const int64_t chunks = seg / Chunk<T>::N;
+#define EMI_ROWS(W)                                                                                              \
+  do {                                                                                                           \
+    if (vec) hipLaunchKernelGGL((reduce_rows_kernel<T, TO, OP, W, true>), dim3(grid), dim3(W * 64), 0, st, x, y, rows, red, seg, nsplit); \
+    else hipLaunchKernelGGL((reduce_rows_kernel<T, TO, OP, W, false>), dim3(grid), dim3(W * 64), 0, st, x, y, rows, red, seg, nsplit);   \
+  } while (0)
+  if (chunks <= 128) EMI_ROWS(1);
+  else if (chunks <= 1024) EMI_ROWS(4);
+  else EMI_ROWS(16);
+#undef EMI_ROWS
+}
+
+template <typename T, int OP>
+int launch_reduce(hipStream_t st, const void* x, void* y, void* ws, size_t ws_bytes, int64_t outer, int64_t red,
+                  int64_t inner) {
+  const T* xp = static_cast<const T*>(x);
+  T* yp = static_cast<T*>(y);
+  ReducePlan p = reduce_plan<T>(outer, red, inner);
+  if (p.nsplit > 1 && (ws == nullptr || ws_bytes < reduce_workspace<T>(outer, red, inner))) p = ReducePlan{1, red};
+  float* part = static_cast<float*>(ws);
+  if (inner == 1) {
+    if (p.nsplit == 1) {
+      launch_rows<T, T, OP>(st, xp, yp, outer, red, red, 1);
+    } else {
+      launch_rows<T, float, OP>(st, xp, part, outer, red, p.seg, p.nsplit);
+      EMI_CHECK_LAUNCH("emi_reduce");
+      launch_rows<float, T, OP>(st, part, yp, outer, p.nsplit, p.nsplit, 1);
+    }
+  } else {
+    const bool vec = al16(x) && inner % Chunk<T>::N == 0;
+    const int64_t lanes = vec ? inner / Chunk<T>::N : inner;
+    const dim3 grid((unsigned)((lanes + kBlock - 1) / kBlock), (unsigned)p.nsplit, (unsigned)outer);
+    if (p.nsplit == 1) {
+      if (vec) hipLaunchKernelGGL((reduce_cols_kernel<T, T, OP, true>), grid, dim3(kBlock), 0, st, xp, yp, outer, red, inner, red);
+      else hipLaunchKernelGGL((reduce_cols_kernel<T, T, OP, false>), grid, dim3(kBlock), 0, st, xp, yp, outer, red, inner, red);
+    } else {
+      if (vec) hipLaunchKernelGGL((reduce_cols_kernel<T, float, OP, true>), grid, dim3(kBlock), 0, st, xp, part, outer, red, inner, p.seg);
+      else hipLaunchKernelGGL((reduce_cols_kernel<T, float, OP, false>), grid, dim3(kBlock), 0, st, xp, part, outer, red, inner, p.seg);
+      EMI_CHECK_LAUNCH("emi_reduce");
+      const int64_t m = outer * inner;
+      hipLaunchKernelGGL((reduce_partials_kernel<T, OP>), dim3((unsigned)((m + 63) / 64)), dim3(1024), 0, st, part, yp, m,
+                         p.nsplit);
+    }
   }
   EMI_CHECK_LAUNCH("emi_reduce");
   return EMI_OK;
@@ -319,8 +568,8 @@ int launch_binary_op(hipStream_t st, int op, unsigned grid, const T* a, const T*
 
 template <typename T>
 int launch_binary(hipStream_t st, int op, const void* a, const void* b, void* y, int64_t n, int sa, int sb) {
-  const bool vec = al16(a) && al16(b) && al16(y) && n >= Chunk<T>::N;
-  const unsigned grid = grid_for(vec ? n / Chunk<T>::N : n, kBlock);
+  const bool vec = al16(a) && al16(b) && al16(y);
+  const unsigned grid = map_grid(n, vec);
   const T* ap = static_cast<const T*>(a);
   const T* bp = static_cast<const T*>(b);
   T* yp = static_cast<T*>(y);
@@ -347,8 +596,8 @@ int launch_unary_op(hipStream_t st, int op, unsigned grid, const T* x, T* y, int
 
 template <typename T>
 int launch_unary(hipStream_t st, int op, const void* x, void* y, int64_t n) {
-  const bool vec = al16(x) && al16(y) && n >= Chunk<T>::N;
-  const unsigned grid = grid_for(vec ? n / Chunk<T>::N : n, kBlock);
+  const bool vec = al16(x) && al16(y);
+  const unsigned grid = map_grid(n, vec);
   const T* xp = static_cast<const T*>(x);
   T* yp = static_cast<T*>(y);
   return vec ? launch_unary_op<T, true>(st, op, grid, xp, yp, n) : launch_unary_op<T, false>(st, op, grid, xp, yp, n);
@@ -356,13 +605,14 @@ int launch_unary(hipStream_t st, int op, const void* x, void* y, int64_t n) {
 
 template <typename TI, typename TO>
 int launch_convert(hipStream_t st, const void* x, void* y, int64_t n) {
-  const bool vec = al16(x) && al16(y) && n >= 8;
+  const bool vec = al16(x) && al16(y);
+  const unsigned grid = map_grid(n, vec);
   if (vec)
-    hipLaunchKernelGGL((convert_kernel<TI, TO>), dim3(grid_for(n / 8, kBlock)), dim3(kBlock), 0, st,
-                       static_cast<const TI*>(x), static_cast<TO*>(y), n);
+    hipLaunchKernelGGL((convert_kernel<TI, TO, true>), dim3(grid), dim3(kBlock), 0, st, static_cast<const TI*>(x),
+                       static_cast<TO*>(y), n);
   else
-    hipLaunchKernelGGL((convert_scalar_kernel<TI, TO>), dim3(grid_for(n, kBlock)), dim3(kBlock), 0, st,
-                       static_cast<const TI*>(x), static_cast<TO*>(y), n);
+    hipLaunchKernelGGL((convert_kernel<TI, TO, false>), dim3(grid), dim3(kBlock), 0, st, static_cast<const TI*>(x),
+                       static_cast<TO*>(y), n);
   EMI_CHECK_LAUNCH("emi_convert");
   return EMI_OK;
 }
@@ -375,7 +625,7 @@ using namespace emi;
 extern "C" int emi_map_binary(emi_stream_t stream, int op, const void* a, const void* b, void* y, int64_t n,
                               int a_is_scalar, int b_is_scalar, int dtype) {
   EMI_REQUIRE(op >= EMI_OP_ADD && op <= EMI_OP_D_POW_B, "emi_map_binary: unknown operator code %d", op);
-  EMI_REQUIRE(n >= 0, "emi_map_binary: negative size");
+  EMI_REQUIRE(n >= 0 && n < (int64_t)1 << 39, "emi_map_binary: size out of range");
   if (n == 0) return EMI_OK;
   EMI_REQUIRE(a && b && y, "emi_map_binary: null buffer");
   hipStream_t st = static_cast<hipStream_t>(stream);
@@ -389,7 +639,7 @@ extern "C" int emi_map_binary(emi_stream_t stream, int op, const void* a, const 
 
 extern "C" int emi_map_unary(emi_stream_t stream, int op, const void* x, void* y, int64_t n, int dtype) {
   EMI_REQUIRE(op >= EMI_OP_NEG && op <= EMI_OP_COPY, "emi_map_unary: unknown operator code %d", op);
-  EMI_REQUIRE(n >= 0, "emi_map_unary: negative size");
+  EMI_REQUIRE(n >= 0 && n < (int64_t)1 << 39, "emi_map_unary: size out of range");
   if (n == 0) return EMI_OK;
   EMI_REQUIRE(x && y, "emi_map_unary: null buffer");
   hipStream_t st = static_cast<hipStream_t>(stream);
@@ -401,7 +651,7 @@ extern "C" int emi_map_unary(emi_stream_t stream, int op, const void* x, void* y
 }
 
 extern "C" int emi_convert(emi_stream_t stream, const void* x, void* y, int64_t n, int from_dtype, int to_dtype) {
-  EMI_REQUIRE(n >= 0, "emi_convert: negative size");
+  EMI_REQUIRE(n >= 0 && n < (int64_t)1 << 39, "emi_convert: size out of range");
   if (n == 0) return EMI_OK;
   EMI_REQUIRE(x && y, "emi_convert: null buffer");
   hipStream_t st = static_cast<hipStream_t>(stream);
@@ -466,19 +716,26 @@ extern "C" int emi_strided_copy(emi_stream_t stream, const void* in, void* out, 
   return launch_copy<uint64_t>(st, ip, op, p);
 }
 
-extern "C" int emi_reduce(emi_stream_t stream, int op, const void* x, void* y, int64_t outer, int64_t red,
-                          int64_t inner, int dtype) {
+extern "C" size_t emi_reduce_workspace_bytes(int64_t outer, int64_t red, int64_t inner, int dtype) {
+  if (outer <= 0 || red <= 0 || inner <= 0) return 0;
+  return dtype == EMI_BF16 ? reduce_workspace<bf16>(outer, red, inner) : reduce_workspace<float>(outer, red, inner);
+}
+
+extern "C" int emi_reduce(emi_stream_t stream, int op, const void* x, void* y, void* workspace, size_t workspace_bytes,
+                          int64_t outer, int64_t red, int64_t inner, int dtype) {
   EMI_REQUIRE(op == EMI_OP_ADD || op == EMI_OP_MAX, "emi_reduce: operator code %d (want add or max)", op);
   EMI_REQUIRE(outer >= 0 && red > 0 && inner > 0, "emi_reduce: bad shape [%lld, %lld, %lld]", (long long)outer,
               (long long)red, (long long)inner);
+  EMI_REQUIRE(outer <= 65535 || inner == 1, "emi_reduce: more than 65535 outer slices with inner > 1");
   if (outer == 0) return EMI_OK;
   EMI_REQUIRE(x && y, "emi_reduce: null buffer");
+  EMI_REQUIRE(workspace == nullptr || al16(workspace), "emi_reduce: workspace must be 16-byte aligned");
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (dtype == EMI_F32)
-    return op == EMI_OP_ADD ? launch_reduce<float, EMI_OP_ADD>(st, x, y, outer, red, inner)
-                            : launch_reduce<float, EMI_OP_MAX>(st, x, y, outer, red, inner);
+    return op == EMI_OP_ADD ? launch_reduce<float, EMI_OP_ADD>(st, x, y, workspace, workspace_bytes, outer, red, inner)
+                            : launch_reduce<float, EMI_OP_MAX>(st, x, y, workspace, workspace_bytes, outer, red, inner);
   if (dtype == EMI_BF16)
-    return op == EMI_OP_ADD ? launch_reduce<bf16, EMI_OP_ADD>(st, x, y, outer, red, inner)
-                            : launch_reduce<bf16, EMI_OP_MAX>(st, x, y, outer, red, inner);
+    return op == EMI_OP_ADD ? launch_reduce<bf16, EMI_OP_ADD>(st, x, y, workspace, workspace_bytes, outer, red, inner)
+                            : launch_reduce<bf16, EMI_OP_MAX>(st, x, y, workspace, workspace_bytes, outer, red, inner);
   return emi_fail(EMI_INVALID_ARGUMENT, "emi_reduce: unsupported dtype code %d", dtype);
 }

@@ -34,7 +34,8 @@ SIGNATURES = {
     "emi_convert": (c_int, [c_void_p, c_void_p, c_void_p, c_i64, c_int, c_int]),
     "emi_strided_copy": (c_int, [c_void_p, c_void_p, c_void_p, c_int, ctypes.POINTER(c_i64), ctypes.POINTER(c_i64),
                                  c_i64, ctypes.POINTER(c_i64), c_i64, c_int]),
-    "emi_reduce": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_i64, c_i64, c_i64, c_int]),
+    "emi_reduce_workspace_bytes": (c_size_t, [c_i64, c_i64, c_i64, c_int]),
+    "emi_reduce": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_size_t, c_i64, c_i64, c_i64, c_int]),
     "emi_gemm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64,
                          c_i64, c_int, c_int, c_int]),
     "emi_gemm_workspace_bytes": (c_size_t, [c_i64, c_i64, c_i64, c_int, c_int, c_int]),

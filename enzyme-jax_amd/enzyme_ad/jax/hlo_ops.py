@@ -178,7 +178,11 @@ def _reduce(kind, x, dims):
     if y.numel():
         if red == 0:
             raise ValueError("reduce over an empty dimension")
-        N.check(N.lib().emi_reduce(_stream(), REDUCE[kind], _p(x), _p(y), outer, red, inner, _code(x)))
+        if inner > 1 and outer > 65535:
+            raise ValueError("reduce: more than 65535 leading slices")
+        nbytes = N.lib().emi_reduce_workspace_bytes(outer, red, inner, _code(x))
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device) if nbytes else None
+        N.check(N.lib().emi_reduce(_stream(), REDUCE[kind], _p(x), _p(y), _p(ws), nbytes, outer, red, inner, _code(x)))
     return y
 
 

@@ -217,10 +217,10 @@ enum {
 
 /* y[i] = op(a[i], b[i]) for i < n, computed in fp32.  An operand flagged
  * *_is_scalar is a single element broadcast to all i (a folded
- * broadcast_in_dim of a rank-0 tensor).  y may alias a or b. */
+ * broadcast_in_dim of a rank-0 tensor).  y must not overlap a or b. */
 int emi_map_binary(emi_stream_t stream, int op, const void* a, const void* b, void* y, int64_t n,
                    int a_is_scalar, int b_is_scalar, int dtype);
-/* y[i] = op(x[i]).  y may alias x. */
+/* y[i] = op(x[i]).  y must not overlap x. */
 int emi_map_unary(emi_stream_t stream, int op, const void* x, void* y, int64_t n, int dtype);
 /* stablehlo.convert between EMI_F32 and EMI_BF16 (round to nearest even). */
 int emi_convert(emi_stream_t stream, const void* x, void* y, int64_t n, int from_dtype, int to_dtype);
@@ -236,9 +236,14 @@ int emi_strided_copy(emi_stream_t stream, const void* in, void* out, int rank, c
                      int64_t out_offset, int elem_bytes);
 /* y[o, i] = sum or max over r of x[o, r, i] (op = EMI_OP_ADD or EMI_OP_MAX), fp32
  * accumulation (stablehlo.reduce with an add / maximum body; Reduce rule
- * StableHLOAutoDiffOpInterfaceImpl.cpp:1833-1916).  x: [outer, red, inner] contiguous. */
-int emi_reduce(emi_stream_t stream, int op, const void* x, void* y, int64_t outer, int64_t red,
-               int64_t inner, int dtype);
+ * StableHLOAutoDiffOpInterfaceImpl.cpp:1833-1916).  x: [outer, red, inner] contiguous.
+ * Shapes with few results and long reductions run in two stages through fp32
+ * partials in `workspace` (emi_reduce_workspace_bytes(); 0 when one stage is used);
+ * with a null or short workspace the single-stage kernel runs (same result, slower).
+ * outer <= 65535 when inner > 1. */
+size_t emi_reduce_workspace_bytes(int64_t outer, int64_t red, int64_t inner, int dtype);
+int emi_reduce(emi_stream_t stream, int op, const void* x, void* y, void* workspace,
+               size_t workspace_bytes, int64_t outer, int64_t red, int64_t inner, int dtype);
 
 /* Embedding gather x[t,:] = table[tokens[t],:] and its adjoint (scatter-add of
  * dx rows into a zero-initialised dtable; fp32 accumulation in workspace when
