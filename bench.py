@@ -252,6 +252,50 @@ def bench_kernels(cfg, iters):
     return out
 
 
+def bench_frontend(iters):
+    """The reference's own case (dim 288, hidden 768, 6 layers, 6 heads, fp32) handed over as
+    StableHLO text: fwd + VJP of one token at position 255 through the parsed graph, with the
+    clusters matched to the fused kernels and operator by operator.  Launch-bound at this size;
+    the figure of interest is the ratio."""
+    import torch
+    from enzyme_ad.jax import stablehlo, vjp
+    from enzyme_ad.jax.llama_text import WEIGHT_ORDER, llama_step_text
+    cfg = dict(dim=288, hidden_dim=768, n_layers=6, n_heads=6, n_kv_heads=6)
+    pos = 255
+    text, order = llama_step_text(cfg, pos)
+    g = torch.Generator(device="cuda").manual_seed(1)
+    shapes = {"x": (288,), "rms_att_weight": (6, 288), "wq": (6, 288, 288), "wk": (6, 288, 288), "wv": (6, 288, 288),
+              "wo": (6, 288, 288), "rms_ffn_weight": (6, 288), "w1": (6, 768, 288), "w2": (6, 288, 768), "w3": (6, 768, 288),
+              "rms_final_weight": (288,), "key_cache": (6, pos, 288), "value_cache": (6, pos, 288)}
+    args = [torch.randn(shapes[n], device="cuda", generator=g) * (0.05 if len(shapes[n]) == 3 and n[0] == "w" else 1.0)
+            for n in order]
+    dy = torch.randn(288, device="cuda", generator=g)
+    out = {}
+    for tag, fuse in (("fused", True), ("unfused", False)):
+        exe = stablehlo.compile_text(text, fuse=fuse)
+
+        def step():
+            y, f_vjp = vjp(lambda *a: exe.run(list(a))[0], *args)
+            return f_vjp(dy)
+
+        t = event_time(step, iters)
+        out["llama_step_text_" + tag] = dict(us_per_step=round(t * 1e6, 1), operators=len(exe.funcs["main"].ops) - 1,
+                                             clusters=exe.fused)
+    # the same step written by hand against the operator table (no text, no matcher)
+    from enzyme_ad.jax import llama
+    named = dict(zip(order, args))
+    weights = {k: named[k] for k in WEIGHT_ORDER}
+    hcfg = dict(cfg, vocab_size=32000, seq_len=256)
+
+    def hand():
+        y, f_vjp = vjp(lambda x, w, kc, vc: llama.forward_step(x, hcfg, w, kc, vc), named["x"], weights,
+                       named["key_cache"], named["value_cache"])
+        return f_vjp(dy)
+
+    out["llama_step_hand_wired"] = dict(us_per_step=round(event_time(hand, iters) * 1e6, 1))
+    return out
+
+
 def cpu_baseline(cfg, seconds_hint=20):
     """The numpy oracle of the same layer (fwd + bwd) on a bounded sample."""
     import numpy as np
@@ -358,6 +402,12 @@ def main():
         kernels = {k: dict(bound=v["bound"], achieved=round(v["achieved"], 1), unit=v["unit"], frac=round(v["frac"], 4))
                    for k, v in kernels.items()}
 
+    frontend = None
+    if not args.no_kernels:
+        frontend = bench_frontend(5)
+        for k, v in frontend.items():
+            log("%-24s %9.1f us per fwd+VJP step, %s operators" % (k, v["us_per_step"], v.get("operators", "-")))
+
     cpu = None
     if not args.no_cpu_baseline:
         cpu = cpu_baseline(cfg)
@@ -372,7 +422,7 @@ def main():
                                "32 heads x 128, batch %d x seq %d, bf16" % (cfg["batch"], cfg["seq"]),
                    "tokens_per_step": tokens, "algorithmic_tflop_per_step": fl["total"] / 1e12,
                    "step_tflops": fl["total"] / dt / 1e12},
-        "roofline": roofline, "kernels": kernels, "cpu_baseline": cpu,
+        "roofline": roofline, "kernels": kernels, "stablehlo_frontend": frontend, "cpu_baseline": cpu,
     }))
 
 

@@ -485,7 +485,28 @@ def slice_(x, start, limit, stride=None):
     y = _slice(x, start, limit, stride)
     if y is x:
         return x
-    Tape.record((x,), y, lambda c, acc: (_accumulate(acc[0], _scatter_box(c, list(x.shape), start, stride)),))
+
+    # only a leaf's cotangent is never handed on to another rule, so only there may a buffer be
+    # updated in place
+    leaf = Tape._active is not None and id(x) not in Tape._active.produced
+
+    def rule(c, acc):
+        g = acc[0]
+        if leaf and g is not None and getattr(g, "_emi_slice_owned", False) and all(st == 1 for st in stride):
+            box = _slice(g, start, limit, stride)
+            if box.is_contiguous() and box.data_ptr() % 16 == 0:
+                # the accumulated cotangent is a buffer an earlier slice rule zero-filled and nobody
+                # else holds (the per-layer slices of one stacked weight): add the block in place
+                c = _contig(c)
+                N.check(N.lib().emi_add(_stream(), _p(box), _p(c), _p(box), c.numel(), _code(c)))
+                return (g,)
+        fresh = _scatter_box(c, list(x.shape), start, stride)
+        if g is None:
+            fresh._emi_slice_owned = leaf
+            return (fresh,)
+        return (_accumulate(g, fresh),)
+
+    Tape.record((x,), y, rule)
     tans = _tan(x)
     if tans is not None and tans[0] is not None:
         _set_tan(y, _quiet(lambda: _slice(tans[0], start, limit, stride)))

@@ -1,9 +1,11 @@
-"""Writes the single-token llama step of the reference (test/llama.py:35-238) as StableHLO
+"""The single-token llama step of the reference (test/llama.py:35-238) written out as StableHLO
 text, operator by operator in the order the Python source applies them, the way a trace of
 that function prints: per-layer weight slices, `w @ x` as dot_general, the batched 2x2
 rotations against constant matrices, cache append as concatenate, a per-head loop of
 dot / softmax / dot, the sigmoid spelled 1 / (1 + exp(-x)), and `jnp.sqrt(head_size)` as a
-sqrt of a constant.  Test input for the StableHLO front end; nothing here computes."""
+sqrt of a constant.  For callers that have no tracer at hand (`hlo_call(*args,
+source=llama_step_text(config, pos)[0])`), for the front end's tests and for its benchmark;
+nothing here computes."""
 import numpy as np
 
 

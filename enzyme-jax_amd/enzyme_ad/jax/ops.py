@@ -86,6 +86,7 @@ class Tape:
 
     def __init__(self):
         self.nodes = []          # (inputs, output, rule)
+        self.produced = set()    # ids of operator results (everything else is a leaf)
 
     def __enter__(self):
         self._prev = Tape._active
@@ -101,6 +102,7 @@ class Tape:
         t = Tape._active
         if t is not None:
             t.nodes.append((inputs, output, rule))
+            t.produced.add(id(output))
 
     def backward(self, outputs, cotangents, wrt):
         """Cotangents of `wrt` (list of tensors) given cotangents of `outputs`."""

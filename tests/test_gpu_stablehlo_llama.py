@@ -8,7 +8,7 @@ import torch
 
 from oracle import llama_ref as L
 from gpu_util import check, dev, host
-from stablehlo_llama import WEIGHT_ORDER, llama_step_text
+from enzyme_ad.jax.llama_text import WEIGHT_ORDER, llama_step_text
 
 pytestmark = pytest.mark.gpu
 

@@ -5,7 +5,7 @@ from collections import Counter
 import numpy as np
 import pytest
 
-from stablehlo_llama import llama_step_text
+from enzyme_ad.jax.llama_text import llama_step_text
 
 CFG = {"dim": 288, "hidden_dim": 768, "n_layers": 2, "n_heads": 6, "n_kv_heads": 6}
 
