@@ -336,6 +336,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel roofline table")
+    ap.add_argument("--no-frontend", action="store_true", help="skip the StableHLO front end timing (thousands of tiny launches)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run one emi_add over 3 x 512 MiB (reads 1 GiB, writes 512 MiB): the known-size kernel "
                          "that FETCH_SIZE / WRITE_SIZE counter runs are scaled by")
@@ -403,7 +404,7 @@ def main():
                    for k, v in kernels.items()}
 
     frontend = None
-    if not args.no_kernels:
+    if not args.no_kernels and not args.no_frontend:
         frontend = bench_frontend(5)
         for k, v in frontend.items():
             log("%-24s %9.1f us per fwd+VJP step, %s operators" % (k, v["us_per_step"], v.get("operators", "-")))
