@@ -48,6 +48,23 @@ def test_plain_launchers_reject_bad_arguments_before_touching_the_gpu():
     assert b"head_dim" in lib.emi_last_error()
     assert lib.emi_swiglu_fwd(None, 8, 16, 16, 64, 11) == 3                    # misaligned pointer
     assert lib.emi_rmsnorm_bwd_workspace_bytes(32768, 4096) == (512 + 1) * 4096 * 4    # partial rows + second level
+    # generic tensor operators
+    i64 = lambda *xs: (C.c_int64 * len(xs))(*xs)
+    assert lib.emi_map_binary(None, 99, 16, 16, 16, 8, 0, 0, 11) == 3 and b"operator" in lib.emi_last_error()
+    assert lib.emi_map_unary(None, 0, 16, 16, 8, 11) == 3                      # a binary code on the unary entry point
+    assert lib.emi_map_binary(None, 0, 16, 16, 16, 8, 0, 0, 5) == 3 and b"dtype" in lib.emi_last_error()
+    assert lib.emi_convert(None, 16, 16, 8, 11, 12) == 3                       # f64 is not supported
+    assert lib.emi_strided_copy(None, 16, 16, 9, i64(*[1] * 9), i64(*[1] * 9), 0, i64(*[1] * 9), 0, 4) == 3
+    assert b"rank" in lib.emi_last_error()
+    assert lib.emi_strided_copy(None, 16, 16, 1, i64(4), i64(1), 0, i64(1), 0, 3) == 3         # element size
+    assert lib.emi_strided_copy(None, 16, 16, 1, i64(4), i64(-1), 0, i64(1), 0, 4) == 3        # negative stride
+    assert lib.emi_strided_copy(None, None, None, 2, i64(0, 4), i64(4, 1), 0, i64(4, 1), 0, 4) == 0   # empty box: nothing to do
+    assert lib.emi_reduce(None, 2, 16, 16, None, 0, 4, 4, 1, 11) == 3 and b"add or max" in lib.emi_last_error()
+    assert lib.emi_reduce(None, 0, 16, 16, None, 0, 70000, 4, 2, 11) == 3      # too many outer slices for the column form
+    assert lib.emi_reduce(None, 0, 16, 16, None, 0, 4, 0, 1, 11) == 3          # empty reduction
+    assert lib.emi_reduce_workspace_bytes(32768, 4096, 1, 16) == 0             # plenty of rows: one stage
+    assert lib.emi_reduce_workspace_bytes(1, 1 << 27, 1, 16) == 2048 * 4       # full sum: 2048 fp32 partials
+    assert lib.emi_reduce_workspace_bytes(1, 32768, 4096, 11) == 512 * 4096 * 4   # column sum: 512 bands of 64 rows
 
 
 def _handler(name):
