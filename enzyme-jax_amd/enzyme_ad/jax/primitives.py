@@ -232,6 +232,62 @@ def tree_unflatten(treedef, leaves):
     return build(treedef)
 
 
+def arg_activity_from_pipeline(pass_pipeline):
+    """(text up to and including 'argTys=', the activities, the text after them); the list ends
+    at the next space (primitives.py:502-508)."""
+    start = pass_pipeline.index("argTys=")
+    end = pass_pipeline.index(" ", start)
+    acts = pass_pipeline[start + len("argTys="):end].split(",")
+    return pass_pipeline[:start + len("argTys=")], acts, pass_pipeline[end:]
+
+
+def ret_activity_from_pipeline(pass_pipeline):
+    """Same for 'retTys=' (primitives.py:511-517)."""
+    start = pass_pipeline.index("retTys=")
+    end = pass_pipeline.index(" ", start)
+    acts = pass_pipeline[start + len("retTys="):end].split(",")
+    return pass_pipeline[:start + len("retTys=")], acts, pass_pipeline[end:]
+
+
+def forward_mode_pipeline(pipeline_options, arg_active, n_results):
+    """The pipeline `enzyme_jvp` builds for forward mode (primitives.py:1176-1203): an
+    `enzyme-wrap{... mode=ForwardMode}` pass with one activity per argument (`enzyme_dup`
+    where a tangent is given, `enzyme_const` for a zero tangent) and `enzyme_dup` per result,
+    spliced into a pipeline that already differentiates (one more AD level) or put in front of
+    one that does not."""
+    arg_act = ",".join("enzyme_dup" if a else "enzyme_const" for a in arg_active)
+    ret_act = ",".join(["enzyme_dup"] * n_results)
+    afterad = "arith-raise{stablehlo=true},enzyme-batch-to-stablehlo, " + optimization_passes() + ", cse, canonicalize"
+    newpasses = ("inline{default-pipeline=canonicalize max-iterations=4}," + optimization_passes() +
+                 ", cse,enzyme-wrap{infn=main outfn= retTys=" + ret_act + " argTys=" + arg_act + " mode=ForwardMode}," + afterad)
+    old = pipeline_options.pass_pipeline()
+    if old != "":
+        if "enzyme-wrap" in old:
+            start = old.rindex("enzyme-wrap{")
+            end = old.index("}", start)
+            newpasses = old[:end] + afterad + newpasses + old[end:]
+        else:
+            newpasses = newpasses + "," + old
+    return JaXPipeline(newpasses)
+
+
+def reverse_mode_pipeline(forward_pipeline, ret_active):
+    """The pipeline `enzyme_vjp` derives from the forward-mode one (primitives.py:1385-1419):
+    the last `enzyme-wrap` pass switches to `ReverseModeCombined`, `enzyme_dup` arguments become
+    `enzyme_active`, each result is `enzyme_active` where a cotangent arrives and
+    `enzyme_const` where it is zero, and the cleanup passes follow."""
+    passes = forward_pipeline.pass_pipeline()
+    start = passes.rindex("enzyme-wrap{")
+    end = passes.index("}", start)
+    prev_passes, post_passes = passes[:start], passes[end + 1:]
+    ad_pass = passes[start:end + 1].replace("enzyme_dup", "enzyme_active").replace("ForwardMode", "ReverseModeCombined")
+    preret, _, postret = ret_activity_from_pipeline(ad_pass)
+    ad_pass = preret + ",".join("enzyme_active" if a else "enzyme_const" for a in ret_active) + postret
+    return JaXPipeline(prev_passes + ad_pass +
+                       ",arith-raise{stablehlo=true},enzyme-batch-to-stablehlo,canonicalize, remove-unnecessary-enzyme-ops, "
+                       "enzyme-simplify-math, " + optimization_passes() + ", canonicalize, cse" + post_passes)
+
+
 class _EnzymeFunction:
     """What `enzyme_jax_ir(...)(func)` returns: callable for the primal; carries
     the options the reference passes to `ffi_call` (primitives.py:1571-1585)."""
@@ -266,6 +322,17 @@ def enzyme_jax_ir(argv=(), pipeline_options=DefaultJaXPipeline, jit_options={}, 
     return decorator
 
 
+def _ad_pipeline(fn, arg_active, n_results):
+    """Forward-mode pipeline for an `enzyme_jax_ir` function whose pipeline differentiates in
+    MLIR, recorded as `fn.last_pipeline` (what the reference would hand to its optimizer; the
+    HIP path reads only the activities from it)."""
+    if not isinstance(fn, _EnzymeFunction) or fn.pipeline_options is None or not fn.pipeline_options.mlir_ad():
+        return None
+    fwd = forward_mode_pipeline(fn.pipeline_options, arg_active, n_results)
+    fn.last_pipeline = fwd
+    return fwd
+
+
 def vjp(fn, *args):
     """(primals_out, f_vjp) like `jax.vjp`: `f_vjp(cotangents)` returns one
     cotangent pytree per positional argument (None for integer leaves and for
@@ -275,11 +342,15 @@ def vjp(fn, *args):
     with ops.Tape() as tape:
         out = fn(*args)
     out_leaves, out_def = tree_flatten(out)
+    active = [isinstance(l, torch.Tensor) and l.is_floating_point() for l in leaves]
+    forward = _ad_pipeline(fn, active, len(out_leaves))
 
     def f_vjp(cotangents):
         ct_leaves, ct_def = tree_flatten(cotangents)
         if len(ct_leaves) != len(out_leaves):
             raise ValueError("cotangent tree has %d leaves, result has %d" % (len(ct_leaves), len(out_leaves)))
+        if forward is not None:
+            fn.last_pipeline = reverse_mode_pipeline(forward, [c is not None for c in ct_leaves])
         wrt = [l for l in leaves if isinstance(l, torch.Tensor) and l.is_floating_point()]
         grads = tape.backward(out_leaves, ct_leaves, wrt)
         it = iter(grads)
@@ -311,6 +382,7 @@ def jvp(fn, primals, tangents):
                 fwd.seed(p, t)
         out = fn(*primals)
         out_leaves, out_def = tree_flatten(out)
+        _ad_pipeline(fn, [t is not None for t in t_leaves], len(out_leaves))
         t_out = []
         for o in out_leaves:
             t = fwd.get(o) if isinstance(o, torch.Tensor) else None

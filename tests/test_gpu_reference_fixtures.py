@@ -37,6 +37,9 @@ def test_add_two_inactive_argument():
     gx, gz, gy = f_vjp(f32([500, 700, 110]))
     assert torch.equal(gx, f32([500, 700, 110])) and torch.equal(gy, gx)
     assert torch.equal(gz, torch.zeros_like(gz))
+    # the pipeline the reference would run for this reverse pass (primitives.py:1385-1419)
+    assert ("retTys=enzyme_active argTys=enzyme_active,enzyme_active,enzyme_active mode=ReverseModeCombined"
+            in add_two.last_pipeline.pass_pipeline())
 
 
 def test_activity_mismatch():

@@ -214,3 +214,48 @@ def test_tape_fan_in_without_gpu():
         ops.Tape.record((y, a), z, lambda c, acc: (c if acc[0] is None else acc[0] + c, c if acc[1] is None else acc[1] + c))
     ga, gb = tape.backward([z], [torch.ones(3)], [a, b])
     assert torch.equal(ga, torch.full((3,), 3.0)) and gb is None
+
+
+def test_activity_pipeline_strings_round_trip():
+    """The strings `enzyme_jvp` / `enzyme_vjp` build (primitives.py:502-517,1176-1203,1385-1419):
+    activities per argument and result, ForwardMode -> ReverseModeCombined, and the splice into
+    a pipeline that already differentiates."""
+    from enzyme_ad.jax import primitives as P
+
+    fwd = P.forward_mode_pipeline(P.JaXPipeline(), [True, False, True], 2)
+    s = fwd.pass_pipeline()
+    wrap = "enzyme-wrap{infn=main outfn= retTys=enzyme_dup,enzyme_dup argTys=enzyme_dup,enzyme_const,enzyme_dup mode=ForwardMode}"
+    assert wrap in s and s.startswith("inline{default-pipeline=canonicalize max-iterations=4},")
+    assert s.endswith(", cse, canonicalize") and fwd.ad_level() == 1
+    pre, acts, post = P.arg_activity_from_pipeline(s)
+    assert acts == ["enzyme_dup", "enzyme_const", "enzyme_dup"] and pre.endswith("argTys=") and post.startswith(" mode=ForwardMode}")
+    assert pre + ",".join(acts) + post == s                                  # lossless split
+    pre, acts, post = P.ret_activity_from_pipeline(s)
+    assert acts == ["enzyme_dup", "enzyme_dup"] and pre + ",".join(acts) + post == s
+    rev = P.reverse_mode_pipeline(fwd, [True, False]).pass_pipeline()
+    assert ("enzyme-wrap{infn=main outfn= retTys=enzyme_active,enzyme_const argTys=enzyme_active,enzyme_const,enzyme_active "
+            "mode=ReverseModeCombined}") in rev
+    assert "ForwardMode" not in rev and "enzyme_dup" not in rev
+    assert ",arith-raise{stablehlo=true},enzyme-batch-to-stablehlo,canonicalize, remove-unnecessary-enzyme-ops, enzyme-simplify-math, " in rev
+    assert [n for n, _ in P.parse_pass_pipeline(rev)].count("enzyme-wrap") == 1
+    # a user pipeline without AD is appended; one with AD gets the new pass spliced after its own
+    plain = P.forward_mode_pipeline(P.JaXPipeline("canonicalize,cse"), [True], 1).pass_pipeline()
+    assert plain.endswith(", cse, canonicalize,canonicalize,cse")
+    twice = P.forward_mode_pipeline(fwd, [True, False, True, True, True], 4)
+    assert twice.ad_level() == 2
+    assert P.arg_activity_from_pipeline(twice.pass_pipeline())[1] == ["enzyme_dup", "enzyme_const", "enzyme_dup"]   # first pass kept
+    with pytest.raises(ValueError):
+        P.arg_activity_from_pipeline("canonicalize")
+
+
+def test_vjp_and_jvp_record_the_reference_pipeline():
+    import enzyme_ad.jax as ej
+
+    f = ej.enzyme_jax_ir(pipeline_options=ej.JaXPipeline(), inner_jit=False)(lambda a, b: a)
+    ej.jvp(f, (3, 4), (None, None))
+    assert "argTys=enzyme_const,enzyme_const mode=ForwardMode" in f.last_pipeline.pass_pipeline()
+    out, f_vjp = ej.vjp(f, 3, 4)
+    assert "mode=ForwardMode" in f.last_pipeline.pass_pipeline()
+    g = ej.enzyme_jax_ir(pipeline_options=ej.XLAPipeline(), inner_jit=False)(lambda a: a)     # no MLIR AD: nothing recorded
+    ej.jvp(g, (3,), (None,))
+    assert not hasattr(g, "last_pipeline")
