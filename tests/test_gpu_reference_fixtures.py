@@ -1,8 +1,8 @@
-"""The reference's small closed-form differentiation cases (test/bench_vs_xla.py:5-194) that
-can be written with the operators of the transformer path -- add, matrix product, reshape,
-row append -- run through `jvp` and `vjp` on the GPU and compared with answers worked out by
-hand from the inputs the reference's fixtures hold.  Sum, Cache and Slicing need elementwise
-products and broadcasts, which the path does not have; they are not covered."""
+"""The reference's small closed-form differentiation cases (test/bench_vs_xla.py:5-194) run through
+`jvp` and `vjp` on the GPU and compared with answers worked out by hand from the inputs the
+reference's fixtures hold: AddTwo, ActivityMismatch, GenDot and Concat written with the
+operators of the transformer path, Sum, Cache and Slicing (which need reductions, broadcasts
+and elementwise products) as StableHLO text through `hlo_call`."""
 import numpy as np
 import pytest
 import torch
@@ -111,3 +111,59 @@ def test_concat():
     c = f32([i * i for i in range(2 * dim)])
     gx, gy = f_vjp(c)
     assert torch.equal(gx, c[:dim]) and torch.equal(gy, c[dim:])
+
+
+def _text_case(text, ins, dins, douts):
+    from enzyme_ad.jax import hlo_call, jvp, vjp
+
+    fn = lambda *a: hlo_call(*a, source=text)[0]
+    out, tan = jvp(fn, tuple(ins), tuple(dins))
+    _, f_vjp = vjp(fn, *ins)
+    return out, tan, f_vjp(douts)
+
+
+def test_sum():
+    """Sum (bench_vs_xla.py:55-69): jnp.sum over range(50)."""
+    text = """func.func @main(%x: tensor<50xf32>) -> tensor<f32> {
+      %z = stablehlo.constant dense<0.000000e+00> : tensor<f32>
+      %r = stablehlo.reduce(%x init: %z) applies stablehlo.add across dimensions = [0] : (tensor<50xf32>, tensor<f32>) -> tensor<f32>
+      return %r : tensor<f32>
+    }"""
+    out, tan, (gx,) = _text_case(text, [f32(range(50))], [f32([i * i for i in range(50)])], f32(1.0))
+    assert float(out) == 1225.0 and float(tan) == float(sq(0, 50))                    # 40425
+    assert torch.equal(gx, f32([1.0] * 50))
+
+
+def test_cache():
+    """Cache (bench_vs_xla.py:72-91): x * x[0] with x = range(288): x[0] = 0, so the output and
+    the tangent vanish and the whole cotangent lands on x[0]: sum_j dout_j x_j = sum j^3."""
+    dim = 288
+    text = """func.func @main(%x: tensor<288xf32>) -> tensor<288xf32> {
+      %s = stablehlo.slice %x [0:1] : (tensor<288xf32>) -> tensor<1xf32>
+      %h = stablehlo.reshape %s : (tensor<1xf32>) -> tensor<f32>
+      %b = stablehlo.broadcast_in_dim %h, dims = [] : (tensor<f32>) -> tensor<288xf32>
+      %r = stablehlo.multiply %x, %b : tensor<288xf32>
+      return %r : tensor<288xf32>
+    }"""
+    sqs = f32([i * i for i in range(dim)])
+    out, tan, (gx,) = _text_case(text, [f32(range(dim))], [sqs], sqs)
+    assert torch.equal(out, torch.zeros_like(out)) and torch.equal(tan, torch.zeros_like(tan))
+    want = np.zeros(dim)
+    want[0] = float(sum(j ** 3 for j in range(dim)))                                  # 1708003584
+    np.testing.assert_allclose(host(gx), want, rtol=1e-5)                             # the reference's own rtol (:90)
+
+
+def test_slicing():
+    """Slicing (bench_vs_xla.py:94-108): x[0, 0:1, 0] * ones(3) on x = range(3) shaped (1, 3, 1)."""
+    text = """func.func @main(%x: tensor<1x3x1xf32>) -> tensor<3xf32> {
+      %s = stablehlo.slice %x [0:1, 0:1, 0:1] : (tensor<1x3x1xf32>) -> tensor<1x1x1xf32>
+      %h = stablehlo.reshape %s : (tensor<1x1x1xf32>) -> tensor<1xf32>
+      %one = stablehlo.constant dense<1.000000e+00> : tensor<3xf32>
+      %b = stablehlo.broadcast_in_dim %h, dims = [0] : (tensor<1xf32>) -> tensor<3xf32>
+      %r = stablehlo.multiply %b, %one : tensor<3xf32>
+      return %r : tensor<3xf32>
+    }"""
+    x = f32(range(3)).reshape(1, 3, 1)
+    out, tan, (gx,) = _text_case(text, [x], [f32([0.0, 1.0, 4.0]).reshape(1, 3, 1)], f32([0.0, 1.0, 4.0]))
+    assert torch.equal(out, f32([0.0] * 3)) and torch.equal(tan, f32([0.0] * 3))
+    assert torch.equal(gx, f32([5.0, 0.0, 0.0]).reshape(1, 3, 1))
