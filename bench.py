@@ -249,6 +249,12 @@ def bench_kernels(cfg, iters):
     hbm("step_attn_bwd_bf16", lambda: N.check(lib.emi_attn_step_bwd(st, P(qs), P(kc), P(vc), P(os_), P(lses), P(dos), P(dqs),
                                                                     P(dkc), P(dvc), P(sws), swb, Bq, hq, Sk, dd, *strides,
                                                                     dd ** -0.5, N.EMI_BF16)), 4 * kc.numel() * 2)
+    tqs = torch.randn((Bq, Dq), device="cuda").to(bf)
+    tkc, tvc = (torch.randn((Bq, Sk, Dq), device="cuda").to(bf) for _ in range(2))
+    del dkc, dvc
+    hbm("step_attn_jvp_bf16", lambda: N.check(lib.emi_attn_step_jvp(st, P(qs), P(kc), P(vc), P(os_), P(lses), P(tqs), P(tkc), P(tvc),
+                                                                    P(dqs), P(sws), swb, Bq, hq, Sk, dd, *strides, dd ** -0.5,
+                                                                    N.EMI_BF16)), 4 * kc.numel() * 2)
     return out
 
 

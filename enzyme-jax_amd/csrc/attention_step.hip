@@ -439,6 +439,118 @@ __global__ __launch_bounds__(64) void attn_step_dq_kernel(const float* __restric
   }
 }
 
+// Forward mode of the step: with p_s = exp(scale q.k_s - lse) from the saved lse,
+// tS_s = scale (tq.k_s + q.tk_s), mu = sum_s p_s tS_s:
+//   to = sum_s p_s (tS_s v_s + tv_s) - mu o.
+// One pass over the keys of the block (k, v and the tangent caches read once); the block's
+// partial sum and its share of mu go to `part`, the combine kernel finishes.  A null tangent
+// pointer is a zero tangent.
+template <typename T, bool VEC, int NCH>
+__global__ __launch_bounds__(256) void attn_step_jvp_kernel(const T* __restrict__ q, const T* __restrict__ k,
+                                                            const T* __restrict__ v, const float* __restrict__ lse,
+                                                            const T* __restrict__ tq, const T* __restrict__ tk,
+                                                            const T* __restrict__ tv, float* __restrict__ part, StepShape sh,
+                                                            float scale) {
+  constexpr int NE = Elems<T, VEC>::N, MAXC = NCH, kUnroll = NCH >= 4 ? 1 : 4 / NCH;
+  __shared__ float red[kRedFloats];
+  __shared__ float scratch[4];
+  const int bh = blockIdx.y, b = bh / sh.heads, h = bh % sh.heads;
+  const int s0 = blockIdx.x * kKeysPerBlock;
+  const int s1 = s0 + kKeysPerBlock < sh.seq_kv ? s0 + kKeysPerBlock : sh.seq_kv;
+  const int l16 = threadIdx.x & 15, slot = threadIdx.x >> 4;
+  const int nchunks = sh.head_dim / NE;
+  const int nch = (nchunks - l16 + 15) / 16;
+  const int64_t qoff = b * sh.q_sb + h * sh.q_sh, kvoff = b * sh.kv_sb + h * sh.kv_sh;
+  const float L = lse[bh];
+
+  float qf[MAXC][NE], tqf[MAXC][NE];
+#pragma unroll
+  for (int c = 0; c < MAXC; c++) {
+#pragma unroll
+    for (int e = 0; e < NE; e++) qf[c][e] = tqf[c][e] = 0.f;
+    if (c < nch) {
+      Elems<T, VEC>::load(q + qoff + (l16 + 16 * c) * NE, qf[c]);
+      if (tq) Elems<T, VEC>::load(tq + qoff + (l16 + 16 * c) * NE, tqf[c]);
+    }
+  }
+  float acc[MAXC][NE];
+#pragma unroll
+  for (int c = 0; c < MAXC; c++)
+#pragma unroll
+    for (int e = 0; e < NE; e++) acc[c][e] = 0.f;
+  float mu = 0.f;
+  for (int sb = s0 + slot; sb < s1; sb += 16 * kUnroll) {
+    float kf[kUnroll][MAXC][NE], vf[kUnroll][MAXC][NE], tkf[kUnroll][MAXC][NE], tvf[kUnroll][MAXC][NE];
+#pragma unroll
+    for (int u = 0; u < kUnroll; u++) {
+      const int s = sb + 16 * u;
+#pragma unroll
+      for (int c = 0; c < MAXC; c++) {
+#pragma unroll
+        for (int e = 0; e < NE; e++) kf[u][c][e] = vf[u][c][e] = tkf[u][c][e] = tvf[u][c][e] = 0.f;
+        if (s < s1 && c < nch) {
+          const int64_t off = kvoff + (int64_t)s * sh.kv_ss + (l16 + 16 * c) * NE;
+          Elems<T, VEC>::load(k + off, kf[u][c]);
+          Elems<T, VEC>::load(v + off, vf[u][c]);
+          if (tk) Elems<T, VEC>::load(tk + off, tkf[u][c]);
+          if (tv) Elems<T, VEC>::load(tv + off, tvf[u][c]);
+        }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; u++) {
+      const int s = sb + 16 * u;
+      float dot = 0.f, tdot = 0.f;
+#pragma unroll
+      for (int c = 0; c < MAXC; c++)
+#pragma unroll
+        for (int e = 0; e < NE; e++) {
+          dot = fmaf(qf[c][e], kf[u][c][e], dot);
+          tdot = fmaf(tqf[c][e], kf[u][c][e], tdot);
+          tdot = fmaf(qf[c][e], tkf[u][c][e], tdot);
+        }
+      dot = sum16(dot);
+      tdot = sum16(tdot);
+      if (s < s1) {
+        const float p = __expf(dot * scale - L);
+        const float w = p * tdot * scale;
+        if (l16 == 0) mu += w;
+#pragma unroll
+        for (int c = 0; c < MAXC; c++)
+#pragma unroll
+          for (int e = 0; e < NE; e++) acc[c][e] = fmaf(w, vf[u][c][e], fmaf(p, tvf[u][c][e], acc[c][e]));
+      }
+    }
+  }
+  mu = block_sum(mu, scratch);
+  reduce_keys<MAXC, NE>(acc, nch, red);
+  float* out = part + ((int64_t)bh * gridDim.x + blockIdx.x) * (sh.head_dim + 2);
+  if (threadIdx.x < 16) {
+#pragma unroll
+    for (int c = 0; c < MAXC; c++)
+      if (c < nch) {
+#pragma unroll
+        for (int e = 0; e < NE; e++) out[(l16 + 16 * c) * NE + e] = acc[c][e];
+      }
+  }
+  if (threadIdx.x == 0) out[sh.head_dim] = mu;
+}
+
+template <typename T>
+__global__ __launch_bounds__(64) void attn_step_jvp_combine_kernel(const float* __restrict__ part, const T* __restrict__ o,
+                                                                   T* __restrict__ to, StepShape sh, int nsplit) {
+  const int bh = blockIdx.x, b = bh / sh.heads, h = bh % sh.heads;
+  const float* p0 = part + (int64_t)bh * nsplit * (sh.head_dim + 2);
+  const int64_t off = b * sh.q_sb + h * sh.q_sh;
+  float mu = 0.f;
+  for (int i = 0; i < nsplit; i++) mu += p0[i * (sh.head_dim + 2) + sh.head_dim];
+  for (int e = threadIdx.x; e < sh.head_dim; e += 64) {
+    float acc = 0.f;
+    for (int i = 0; i < nsplit; i++) acc += p0[i * (sh.head_dim + 2) + e];
+    to[off + e] = from_f32<T>(acc - mu * to_f32(o[off + e]));
+  }
+}
+
 bool al16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 int check_step(const char* name, int64_t batch, int64_t heads, int64_t seq_kv, int64_t head_dim, int64_t q_sb, int64_t q_sh,
@@ -559,5 +671,51 @@ extern "C" int emi_attn_step_bwd(emi_stream_t stream, const void* q, const void*
 #undef EMI_STEP_BWD_T
 #undef EMI_STEP_BWD
   EMI_CHECK_LAUNCH("emi_attn_step_bwd(dq)");
+  return EMI_OK;
+}
+
+extern "C" int emi_attn_step_jvp(emi_stream_t stream, const void* q, const void* k, const void* v, const void* o,
+                                 const float* lse, const void* tq, const void* tk, const void* tv, void* to, void* workspace,
+                                 size_t workspace_bytes, int64_t batch, int64_t heads, int64_t seq_kv, int64_t head_dim,
+                                 int64_t q_stride_b, int64_t q_stride_h, int64_t kv_stride_b, int64_t kv_stride_h,
+                                 int64_t kv_stride_s, float scale, int dtype) {
+  if (int rc = check_step("emi_attn_step_jvp", batch, heads, seq_kv, head_dim, q_stride_b, q_stride_h, kv_stride_b, kv_stride_h,
+                          kv_stride_s, dtype))
+    return rc;
+  if (batch == 0) return EMI_OK;
+  EMI_REQUIRE(q && k && v && o && lse && to, "emi_attn_step_jvp: null buffer");
+  const size_t need = emi_attn_step_workspace_bytes(batch, heads, seq_kv, head_dim);
+  EMI_REQUIRE(workspace != nullptr && workspace_bytes >= need, "emi_attn_step_jvp: workspace of %zu bytes needed, got %zu", need,
+              workspace_bytes);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const StepShape sh{(int)heads, (int)seq_kv, (int)head_dim, q_stride_b, q_stride_h, kv_stride_b, kv_stride_h, kv_stride_s};
+  const int ne = dtype == EMI_BF16 ? 8 : 4;
+  const bool vec = head_dim % ne == 0 && q_stride_b % ne == 0 && q_stride_h % ne == 0 && kv_stride_b % ne == 0 &&
+                   kv_stride_h % ne == 0 && kv_stride_s % ne == 0 && al16(q) && al16(k) && al16(v) && al16(tq) && al16(tk) &&
+                   al16(tv);
+  const int nsplit = (int)((seq_kv + kKeysPerBlock - 1) / kKeysPerBlock);
+  const dim3 grid((unsigned)nsplit, (unsigned)(batch * heads));
+  float* part = static_cast<float*>(workspace);
+#define EMI_STEP_JVP(T, VEC, NCH)                                                                                       \
+  do {                                                                                                                   \
+    hipLaunchKernelGGL((attn_step_jvp_kernel<T, VEC, NCH>), grid, dim3(256), 0, st, (const T*)q, (const T*)k,            \
+                       (const T*)v, lse, (const T*)tq, (const T*)tk, (const T*)tv, part, sh, scale);                     \
+    EMI_CHECK_LAUNCH("emi_attn_step_jvp");                                                                               \
+    hipLaunchKernelGGL(attn_step_jvp_combine_kernel<T>, dim3((unsigned)(batch * heads)), dim3(64), 0, st, part,          \
+                       (const T*)o, (T*)to, sh, nsplit);                                                                 \
+  } while (0)
+#define EMI_STEP_JVP_T(T)                                              \
+  do {                                                                 \
+    if (!vec) EMI_STEP_JVP(T, false, 16);                              \
+    else if (nch <= 1) EMI_STEP_JVP(T, true, 1);                       \
+    else if (nch <= 2) EMI_STEP_JVP(T, true, 2);                       \
+    else EMI_STEP_JVP(T, true, 4);                                     \
+  } while (0)
+  const int nch = (int)((head_dim / ne + 15) / 16);      // 16-byte chunks per lane
+  if (dtype == EMI_BF16) EMI_STEP_JVP_T(bf16);
+  else EMI_STEP_JVP_T(float);
+#undef EMI_STEP_JVP_T
+#undef EMI_STEP_JVP
+  EMI_CHECK_LAUNCH("emi_attn_step_jvp(combine)");
   return EMI_OK;
 }

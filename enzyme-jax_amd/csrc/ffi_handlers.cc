@@ -444,6 +444,33 @@ extern "C" XLA_FFI_Error* emi_attn_step_bwd_ffi(XLA_FFI_CallFrame* cf) {
                                          d.H * d.D, d.D, d.S * d.H * d.D, d.D, d.H * d.D, (float)scale, q->dtype));
 }
 
+extern "C" XLA_FFI_Error* emi_attn_step_jvp_ffi(XLA_FFI_CallFrame* cf) {
+  EMI_FFI_BEGIN("emi_attn_step_jvp", 8, 8, 2, 2)
+  const XLA_FFI_Buffer *q = f.arg(0), *k = f.arg(1), *v = f.arg(2), *o = f.arg(3), *lse = f.arg(4), *tq = f.arg(5), *tk = f.arg(6),
+                       *tv = f.arg(7);
+  const XLA_FFI_Buffer *to = f.ret(0), *ws = f.ret(1);
+  if (!is_float(q)) return f.invalid("q must be f32 or bf16 (code %lld)", q->dtype);
+  const XLA_FFI_Buffer* qlike[] = {o, tq, to};
+  const XLA_FFI_Buffer* klike[] = {v, tk, tv};
+  for (const XLA_FFI_Buffer* b : qlike)
+    if (b->dtype != q->dtype || !same_shape(q, b)) return f.invalid("q, o, tq, to must share dtype and shape");
+  for (const XLA_FFI_Buffer* b : klike)
+    if (b->dtype != q->dtype || !same_shape(k, b)) return f.invalid("k, v, tk, tv must share dtype and shape");
+  double scale;
+  if (!f.get_f("scale", &scale)) return f.invalid("missing f32/f64 attribute 'scale'");
+  StepDims d;
+  if (k->dtype != q->dtype || !step_dims(q, k, &d))
+    return f.invalid("q must be [batch, heads, head_dim] and k [batch, seq_kv, heads, head_dim] (q rank %lld)", q->rank);
+  if (lse->dtype != XLA_FFI_DataType_F32 || lse->rank != 2 || lse->dims[0] != d.B || lse->dims[1] != d.H)
+    return f.invalid("lse must be f32[batch, heads] = [%lld, %lld]", d.B, d.H);
+  const size_t need = emi_attn_step_workspace_bytes(d.B, d.H, d.S, d.D);
+  if (byte_size(ws) < need) return f.invalid("workspace result has %lld bytes, %lld needed", (long long)byte_size(ws), (long long)need);
+  EMI_FFI_STREAM()
+  return f.from_status(emi_attn_step_jvp(stream, q->data, k->data, v->data, o->data, static_cast<const float*>(lse->data),
+                                         tq->data, tk->data, tv->data, to->data, ws->data, byte_size(ws), d.B, d.H, d.S, d.D,
+                                         d.H * d.D, d.D, d.S * d.H * d.D, d.D, d.H * d.D, (float)scale, q->dtype));
+}
+
 extern "C" XLA_FFI_Error* emi_embedding_fwd_ffi(XLA_FFI_CallFrame* cf) {
   EMI_FFI_BEGIN("emi_embedding_fwd", 2, 2, 1, 1)
   const XLA_FFI_Buffer *tok = f.arg(0), *tab = f.arg(1), *x = f.ret(0);
@@ -485,6 +512,7 @@ const Target kTargets[] = {
     {"emi_attn_fwd", emi_attn_fwd_ffi},       {"emi_attn_bwd", emi_attn_bwd_ffi},
     {"emi_attn_step_fwd", emi_attn_step_fwd_ffi}, {"emi_attn_step_bwd", emi_attn_step_bwd_ffi},
     {"emi_rmsnorm_jvp", emi_rmsnorm_jvp_ffi}, {"emi_swiglu_jvp", emi_swiglu_jvp_ffi}, {"emi_attn_jvp", emi_attn_jvp_ffi},
+    {"emi_attn_step_jvp", emi_attn_step_jvp_ffi},
     {"emi_embedding_fwd", emi_embedding_fwd_ffi}, {"emi_embedding_bwd", emi_embedding_bwd_ffi},
 };
 constexpr int kNumTargets = sizeof(kTargets) / sizeof(kTargets[0]);

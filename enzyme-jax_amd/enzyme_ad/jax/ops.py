@@ -37,7 +37,8 @@ FFI_TARGETS = {
 # operator -> tangent target(s); linear operators push tangents through their forward target
 FFI_TANGENT_TARGETS = {
     "rmsnorm": ("emi_rmsnorm_jvp",), "rope": ("emi_rope",), "matmul_nt": ("emi_gemm", "emi_gemm"),
-    "swiglu": ("emi_swiglu_jvp",), "attention": ("emi_attn_jvp",), "add": ("emi_add",), "embedding": ("emi_embedding_fwd",),
+    "swiglu": ("emi_swiglu_jvp",), "attention": ("emi_attn_jvp",), "attention_step": ("emi_attn_step_jvp",),
+    "add": ("emi_add",), "embedding": ("emi_embedding_fwd",),
 }
 
 _DTYPES = {torch.float32: N.EMI_F32, torch.bfloat16: N.EMI_BF16}
@@ -533,7 +534,11 @@ def attention_step(q, k_cache, v_cache, n_heads, scale=None):
     Tape.record((q, k_cache, v_cache), o, rule)
     tans = _tan(q, k_cache, v_cache)
     if tans is not None and any(t is not None for t in tans):
-        raise NotImplementedError("attention_step has no forward-mode kernel")
+        tq, tk, tv = (None if t is None else t.contiguous() for t in tans)
+        to = torch.empty_like(q)
+        N.check(N.lib().emi_attn_step_jvp(_stream(), _p(q), _p(k_cache), _p(v_cache), _p(o), _p(lse), _p(tq), _p(tk), _p(tv),
+                                          _p(to), _p(ws), nbytes, 1, n_heads, S, d, *strides, float(scale), _code(q)))
+        _set_tan(o, to)
     return o
 
 

@@ -418,9 +418,7 @@ def hlo_call(*args, source: str, argv=(), passes: str = ""):
     if passes:
         parse_pass_pipeline(passes)
     leaves, _ = tree_flatten(args)
-    # attention_step has no tangent kernel: under forward mode its cluster stays unfused
-    fuse = True if ops.Forward._active is None else ("rmsnorm", "swiglu", "rope")
-    exe = stablehlo.compile_text(source, fuse=fuse)
+    exe = stablehlo.compile_text(source)
     in_tys, _ = exe.signature("main")
     if len(leaves) != len(in_tys):
         raise AssertionError("main takes %d arguments, %d given" % (len(in_tys), len(leaves)))

@@ -188,6 +188,16 @@ int emi_attn_jvp(emi_stream_t stream, const void* q, const void* k, const void* 
                  int64_t heads, int64_t seq, int64_t head_dim, int64_t stride_b, int64_t stride_h,
                  int64_t stride_s, float scale, int causal, int dtype);
 
+/* Forward mode of the single-token attention (emi_attn_step_fwd's layout, o and lse from
+ * it): to = sum_s p_s (tS_s v_s + tv_s) - (sum_s p_s tS_s) o with tS_s = scale (tq.k_s + q.tk_s).
+ * Null tq / tk / tv = zero tangent.  workspace: emi_attn_step_workspace_bytes(). */
+int emi_attn_step_jvp(emi_stream_t stream, const void* q, const void* k, const void* v, const void* o,
+                      const float* lse, const void* tq, const void* tk, const void* tv, void* to,
+                      void* workspace, size_t workspace_bytes, int64_t batch, int64_t heads,
+                      int64_t seq_kv, int64_t head_dim, int64_t q_stride_b, int64_t q_stride_h,
+                      int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s, float scale,
+                      int dtype);
+
 /* ---- generic tensor operators -------------------------------------------
  * What is left of a StableHLO module that arrives as text (hlo_call,
  * src/enzyme_ad/jax/primitives.py:1052-1108; in the reference XLA's own code

@@ -31,6 +31,7 @@
  *  emi_rmsnorm_jvp    x, gamma, tx, tgamma             ty                                eps:f32
  *  emi_swiglu_jvp     a, b, ta, tb                     tg                                -
  *  emi_attn_jvp       q, k, v, lse, tq, tk, tv         to                                scale:f32, causal:pred, bshd:pred
+ *  emi_attn_step_jvp  q, k, v, o, lse, tq, tk, tv      to, workspace:u8[n]               scale:f32
  *  emi_embedding_fwd  tokens s32[..], table[V,D]       x[..,D]                           -
  *  emi_embedding_bwd  tokens s32[..], dx[..,D]         dtable[V,D] [, workspace:u8[n]]   -
  *
@@ -64,6 +65,7 @@ struct XLA_FFI_Error* emi_attn_step_bwd_ffi(struct XLA_FFI_CallFrame*);
 struct XLA_FFI_Error* emi_rmsnorm_jvp_ffi(struct XLA_FFI_CallFrame*);
 struct XLA_FFI_Error* emi_swiglu_jvp_ffi(struct XLA_FFI_CallFrame*);
 struct XLA_FFI_Error* emi_attn_jvp_ffi(struct XLA_FFI_CallFrame*);
+struct XLA_FFI_Error* emi_attn_step_jvp_ffi(struct XLA_FFI_CallFrame*);
 struct XLA_FFI_Error* emi_embedding_fwd_ffi(struct XLA_FFI_CallFrame*);
 struct XLA_FFI_Error* emi_embedding_bwd_ffi(struct XLA_FFI_CallFrame*);
 

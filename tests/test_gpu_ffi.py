@@ -112,6 +112,14 @@ def test_ffi_handlers_launch_on_the_frame_stream():
         check(dq, rdq[:, :, 0, :], "bf16", "ffi step dq")
         check(dk, rdk.transpose(0, 2, 1, 3), "bf16", "ffi step dk")
         check(dv, rdv.transpose(0, 2, 1, 3), "bf16", "ffi step dv")
+        # tangent of the step attention: same layout, tangents are ordinary operands
+        (tq, tqr), = (dev(rng.standard_normal((B, h, d)), "bf16"),)
+        (tkc, tkcr), (tvc, tvcr) = (dev(rng.standard_normal((B, S, h, d)), "bf16") for _ in range(2))
+        to = torch.empty_like(q)
+        _call("emi_attn_step_jvp_ffi", xla, [_buf(xla, t) for t in (q, kc, vc, o, lse, tq, tkc, tvc)],
+              [_buf(xla, to), _buf(xla, ws)], at)
+        rto = L.attention_jvp(q4, k4, v4, tqr[:, :, None, :], tkcr.transpose(0, 2, 1, 3), tvcr.transpose(0, 2, 1, 3), causal=False)
+        check(to, rto[:, :, 0, :], "bf16", "ffi step attention tangent")
         # forward-mode targets: tangents are ordinary operands
         x4, x4r = dev(rng.standard_normal((6, 512)), "bf16")
         g4, g4r = dev(rng.uniform(0.5, 1.5, 512), "bf16")

@@ -121,3 +121,44 @@ def test_step_form_bf16_llama_head_shape():
     check(gvc, rdvc, "bf16", "dvalue_cache")
     for k in rgw:
         check(gw[k], rgw[k], "bf16", "grad " + k)
+
+
+@pytest.mark.parametrize("dt,heads,d,s", [("f32", 6, 48, 2), ("f32", 6, 48, 301), ("bf16", 4, 128, 1000), ("bf16", 3, 64, 77),
+                                            ("f32", 2, 50, 33), ("bf16", 2, 36, 5)])
+def test_attention_step_tangent(dt, heads, d, s):
+    """Forward mode of the step attention against the oracle's attention_jvp (one query, no
+    mask), with all tangents and with single ones (null pointers are zero tangents)."""
+    from enzyme_ad.jax import ops, jvp
+    D = heads * d
+    rng = np.random.Generator(np.random.PCG64(s * 11 + d))
+    (q, qr), (tq, tqr) = (dev(rng.standard_normal(D), dt) for _ in range(2))
+    (kc, kcr), (vc, vcr), (tk, tkr), (tv, tvr) = (dev(rng.standard_normal((s, D)), dt) for _ in range(4))
+    hd = lambda t: t.reshape(1, -1, heads, d).transpose(0, 2, 1, 3)
+    fn = lambda a, b, c: ops.attention_step(a, b, c, heads)
+    for mask in ((1, 1, 1), (1, 0, 0), (0, 1, 0), (0, 0, 1)):
+        tans = tuple(t if m else None for t, m in zip((tq, tk, tv), mask))
+        o, to = jvp(fn, (q, kc, vc), tans)
+        ref = L.attention_jvp(hd(qr), hd(kcr), hd(vcr), mask[0] * hd(tqr), mask[1] * hd(tkr), mask[2] * hd(tvr), causal=False)
+        check(to, ref.transpose(0, 2, 1, 3).reshape(D), dt, "step tangent %s" % (mask,))
+
+
+def test_step_form_forward_mode_adjoint_identity():
+    """<J v, w> from forward mode of the whole step = <v, J^T w> from its reverse mode."""
+    from enzyme_ad.jax import jvp, vjp, llama
+    cfg = {"dim": 288, "hidden_dim": 768, "n_layers": 3, "n_heads": 6, "n_kv_heads": 6, "vocab_size": 32000, "seq_len": 256}
+    pos = 9
+    rng = np.random.Generator(np.random.PCG64(61))
+    w = L.make_weights(cfg, 61, std=0.05, embedding=False, norm_gain="uniform")
+    wd = {k: dev(a, "f32")[0] for k, a in w.items()}
+    tw = {k: dev(rng.standard_normal(a.shape) * 0.05, "f32")[0] for k, a in w.items()}
+    x, tx, dy = (dev(rng.standard_normal(cfg["dim"]), "f32")[0] for _ in range(3))
+    shape = (cfg["n_layers"], pos, cfg["dim"])
+    kc, vc, tkc, tvc = (dev(rng.standard_normal(shape), "f32")[0] for _ in range(4))
+    fn = lambda x, w, kc, vc: llama.forward_step(x, cfg, w, kc, vc)
+    y, ty = jvp(fn, (x, wd, kc, vc), (tx, tw, tkc, tvc))
+    y2, f_vjp = vjp(fn, x, wd, kc, vc)
+    gx, gw, gkc, gvc = f_vjp(dy)
+    lhs = float(np.dot(host(ty), host(dy)))
+    rhs = float(np.sum(host(gx) * host(tx)) + np.sum(host(gkc) * host(tkc)) + np.sum(host(gvc) * host(tvc)) +
+                sum(np.sum(host(gw[k]) * host(tw[k])) for k in w))
+    assert abs(lhs - rhs) <= 1e-4 * max(abs(lhs), abs(rhs)), (lhs, rhs)
