@@ -14,7 +14,7 @@ namespace emi {
 namespace {
 
 // y[m][n] = sum_k A[m][k] B[n][k] (+ R[m][n]); one wavefront per row n of B, which streams
-// through in 16-byte chunks (four in flight per lane); A (M x K, a few KB) comes from cache.
+// through in 16-byte chunks (eight in flight per lane); A (M x K, a few KB) comes from cache.
 template <typename T, int MT>
 __global__ __launch_bounds__(256) void gemv_nt_kernel(const T* __restrict__ A, const T* __restrict__ B, const T* R, T* C, int M,
                                                       int N, int K, int64_t lda, int64_t ldb, int64_t ldr, int64_t ldc) {
@@ -26,24 +26,27 @@ __global__ __launch_bounds__(256) void gemv_nt_kernel(const T* __restrict__ A, c
   float acc[MT];
 #pragma unroll
   for (int m = 0; m < MT; m++) acc[m] = 0.f;
-  for (int k0 = lane * V; k0 < K; k0 += 64 * V * 4) {
-    float b[4][V];
+  constexpr int UN = 8;                      // 16-byte loads of the row in flight per lane
+  for (int k0 = lane * V; k0 < K; k0 += 64 * V * UN) {
+    typename Chunk<T>::Raw raw[UN];
 #pragma unroll
-    for (int u = 0; u < 4; u++) {
+    for (int u = 0; u < UN; u++) {
       const int k = k0 + u * 64 * V;
-      if (k < K) Chunk<T>::load(brow + k, b[u]);
+      if (k < K) raw[u] = Chunk<T>::load_raw(brow + k);
     }
 #pragma unroll
-    for (int u = 0; u < 4; u++) {
+    for (int u = 0; u < UN; u++) {
       const int k = k0 + u * 64 * V;
       if (k < K) {
+        float b[V];
+        Chunk<T>::unpack(raw[u], b);
 #pragma unroll
         for (int m = 0; m < MT; m++) {
           if (m < M) {
             float a[V];
             Chunk<T>::load(A + (int64_t)m * lda + k, a);
 #pragma unroll
-            for (int e = 0; e < V; e++) acc[m] = fmaf(a[e], b[u][e], acc[m]);
+            for (int e = 0; e < V; e++) acc[m] = fmaf(a[e], b[e], acc[m]);
           }
         }
       }
