@@ -426,8 +426,18 @@ def hlo_call(*args, source: str, argv=(), passes: str = ""):
 
 
 def optimize_module(mod, pipeline=None):
-    """primitives.py (optimize_module): runs the MLIR optimizer on a module; not built."""
-    raise NotImplementedError("optimize_module needs the MLIR optimizer, which the HIP path does not have")
+    """primitives.py:280-284 runs the MLIR optimizer over a module in place.  Here `mod` is the
+    module's StableHLO text and the result is returned: constants folded, the llama clusters
+    replaced by `stablehlo.custom_call @emi_*` (api_version 4, scalars in `backend_config`), the
+    other operators printed back unchanged.  An XLA client with this library's FFI handlers
+    registered can compile the result; `hlo_call` runs it as well.  `pipeline` is parsed for
+    validity only."""
+    from . import stablehlo
+
+    parse_pass_pipeline(full_optimization_pass_pipeline() if pipeline is None else pipeline)
+    if not isinstance(mod, str):
+        raise TypeError("optimize_module takes the module as StableHLO text (str); there are no MLIR module objects here")
+    return stablehlo.lower_to_custom_calls(mod)[0]
 
 
 def export(outfile, func, *args, argv=(), jit_options={}):

@@ -267,6 +267,26 @@ def _i64_array(text, key):
     return [int(t) for t in re.findall(r"-?\d+", m.group(2) if m.group(2) is not None else m.group(3))]
 
 
+def _backend_config(text):
+    """{name: value} of the `backend_config = {...}` dictionary of a custom call (numbers and
+    booleans; the wire format of typed-FFI calls, Passes/LowerEnzymeXLABLAS.cpp:463-479)."""
+    m = re.search(r"backend_config\s*=\s*\{", text)
+    if not m:
+        return {}
+    body = _Scanner(text[m.end() - 1:]).balanced()[1:-1]
+    out = {}
+    for key, val in re.findall(r"([A-Za-z_][A-Za-z0-9_]*)\s*=\s*([^,:}]+)", body):
+        val = val.strip()
+        if val in ("true", "false"):
+            out[key] = val == "true"
+        else:
+            try:
+                out[key] = int(val)
+            except ValueError:
+                out[key] = float(val)
+    return out
+
+
 def _attr_lists(text, key):
     m = re.search(key + r"\s*=\s*\[([^\]]*)\]", text)
     return [int(t) for t in re.findall(r"-?\d+", m.group(1))] if m else []
@@ -385,6 +405,14 @@ def _parse_op(sc):
             body = found[0]
         body = body.split(".")[-1]
         return Op("reduce", results, [x, init], {"dims": dims, "body": body}, types)
+    if short == "custom_call":
+        target = sc.need(_SYM, "custom-call target")[1:].strip('"')
+        sc.expect("(")
+        operands = operand_list()
+        sc.expect(")")
+        text = sc.balanced() if sc.peek("{") else "{}"
+        _, types = sc.signature()
+        return Op("custom_call", results, operands, {"target": target, "config": _backend_config(text)}, types)
     if short == "call":
         callee = sc.need(_SYM, "callee")
         sc.expect("(")
@@ -924,7 +952,7 @@ class Executable:
             if len(outs) != len(op.results):
                 raise RuntimeError("%s produced %d values for %d results" % (op.name, len(outs), len(op.results)))
             for r, v, ty in zip(op.results, outs, op.types):
-                if tuple(v.shape) != ty.shape:
+                if v is not None and tuple(v.shape) != ty.shape:
                     raise RuntimeError("%s: result %s has shape %s, the text says %r" % (op.name, r, tuple(v.shape), ty))
                 env[r] = v
         raise ParseError("function %s has no return" % fn)
@@ -962,6 +990,8 @@ class Executable:
             return [H.concatenate(xs, op.attrs["dim"])]
         if n == "call":
             return self.run(xs, op.attrs["callee"])
+        if n == "custom_call":
+            return self._custom_call(op, xs)
         if n == "emi.rmsnorm":
             x, w = _packed(xs[0]), _packed(xs[1])
             return [ops.reshape(ops.rmsnorm(ops.reshape(x, (1, x.shape[0])), w, op.attrs["eps"]), tuple(x.shape))]
@@ -986,12 +1016,219 @@ class Executable:
         raise NotImplementedError("StableHLO operator '%s' is not supported by the HIP front end" % n)
 
 
+def _custom_call_impl(self, op, xs):
+    """Typed-FFI custom calls to this library's targets (the form `lower_to_custom_calls` prints),
+    run through the same operators the matcher would have picked."""
+    target, cfg = op.attrs["target"], op.attrs["config"]
+    if target == "emi_rmsnorm_fwd":
+        x, w = _packed(xs[0]), _packed(xs[1])
+        y = ops.rmsnorm(ops.reshape(x, (-1, x.shape[-1])), w, cfg.get("eps", 1e-5))
+        return [ops.reshape(y, tuple(x.shape))]
+    if target == "emi_swiglu_fwd":
+        return [ops.swiglu(_packed(xs[0]), _packed(xs[1]))]
+    if target == "emi_add":
+        return [ops.add(_packed(xs[0]), _packed(xs[1]))]
+    if target == "emi_rope":
+        x, table = _packed(xs[0]), xs[1]
+        if x.dim() != 4 or x.shape[1] != 1 or tuple(table.shape) != (1, x.shape[3] // 2, 2):
+            raise NotImplementedError("custom call emi_rope is run for one position per call (seq = 1)")
+        y = ops.rotate_pairs(ops.reshape(x, (-1, x.shape[3])), table.reshape(-1, 2).contiguous(), bool(cfg.get("inverse", False)))
+        return [ops.reshape(y, tuple(x.shape))]
+    if target == "emi_attn_step_fwd":
+        q, k, v = (_packed(t) for t in xs)
+        if q.dim() != 3 or q.shape[0] != 1 or k.dim() != 4:
+            raise NotImplementedError("custom call emi_attn_step_fwd is run for one sequence per call (batch = 1)")
+        h, d = q.shape[1], q.shape[2]
+        o = ops.attention_step(ops.reshape(q, (h * d,)), ops.reshape(k, (k.shape[1], h * d)), ops.reshape(v, (v.shape[1], h * d)),
+                               h, cfg["scale"])
+        return [ops.reshape(o, (1, h, d))] + [None] * (len(op.results) - 1)       # lse and workspace stay inside the operator
+    raise NotImplementedError("custom call target '%s' is not one of this library's" % target)
+
+
+Executable._custom_call = _custom_call_impl
+
+
 def _packed(t):
     """Contiguous and 16-byte aligned, as the fused kernels want their operands; a view that
     is neither is copied (tracked, so cotangents flow back to the view's source)."""
     if t.is_contiguous() and t.data_ptr() % 16 == 0:
         return t
     return H.unary_copy(t)
+
+
+# ---------------------------------------------------------------------------
+# printer: the module with its clusters lowered to typed-FFI custom calls
+# ---------------------------------------------------------------------------
+
+def _fmt_float(v):
+    v = float(v)
+    if v == math.inf:
+        return "0x7F800000"
+    if v == -math.inf:
+        return "0xFF800000"
+    return "%.9e" % v
+
+
+def _dense_text(value, ty):
+    a = np.asarray(value)
+    flat = a.reshape(-1)
+    is_float = ty.dtype in ("f32", "bf16", "f16", "f64")
+    one = (lambda x: _fmt_float(x)) if is_float else (lambda x: str(bool(x)).lower() if ty.dtype == "i1" else str(int(x)))
+    if flat.size and np.all(flat == flat[0]) and not (is_float and np.isinf(flat[0]) and ty.dtype != "f32"):
+        return one(flat[0])
+
+    def lit(x):
+        return "[" + ", ".join(lit(y) for y in x) + "]" if x.ndim else one(x)
+
+    return lit(a)
+
+
+def _layouts(types):
+    def one(t):
+        r = len(t.shape)
+        body = "" if r == 0 else "0" if r == 1 else "[" + ", ".join(str(i) for i in reversed(range(r))) + "]"
+        return "dense<%s> : tensor<%dxindex>" % (body, r)
+    return "[" + ", ".join(one(t) for t in types) + "]"
+
+
+class _Printer:
+    def __init__(self, func):
+        self.f, self.lines, self.n = func, [], 0
+        self.types = {a: t for a, t in func.args}
+        for op in func.ops:
+            for r, t in zip(op.results, op.types):
+                self.types[r] = t
+
+    def fresh(self, ty):
+        name = "%%emi%d" % self.n
+        self.n += 1
+        self.types[name] = ty
+        return name
+
+    def emit(self, text):
+        self.lines.append("    " + text)
+
+    def reshape(self, v, shape):
+        ty = TensorType(shape, self.types[v].dtype)
+        if self.types[v].shape == ty.shape:
+            return v
+        r = self.fresh(ty)
+        self.emit("%s = stablehlo.reshape %s : (%r) -> %r" % (r, v, self.types[v], ty))
+        return r
+
+    def custom_call(self, results, target, operands, config, out_types):
+        cfg = ", ".join("%s = %s" % (k, ("true" if v else "false") if isinstance(v, bool) else
+                                     ("%d : i64" % v if isinstance(v, int) else "%s : f32" % _fmt_float(v))) for k, v in config.items())
+        lhs = results[0] if len(results) == 1 else "%s:%d" % (results[0].split("#")[0], len(results))
+        outs = repr(out_types[0]) if len(out_types) == 1 else "(" + ", ".join(repr(t) for t in out_types) + ")"
+        self.emit("%s = stablehlo.custom_call @%s(%s) {api_version = 4 : i32, backend_config = {%s}, operand_layouts = %s, "
+                  "result_layouts = %s} : (%s) -> %s" % (lhs, target, ", ".join(operands), cfg,
+                                                       _layouts([self.types[o] for o in operands]), _layouts(out_types),
+                                                       ", ".join(repr(self.types[o]) for o in operands), outs))
+
+    def op(self, op):
+        T = self.types
+        n, r = op.name, (op.results[0] if op.results else None)
+        ty = op.types[0] if op.types else None
+        if n == "return":
+            self.emit("return %s : %s" % (", ".join(op.operands), ", ".join(repr(T[o]) for o in op.operands)))
+        elif n == "constant":
+            self.emit("%s = stablehlo.constant dense<%s> : %r" % (r, _dense_text(op.attrs["value"], ty), ty))
+        elif n in BINARY_OPS:
+            self.emit("%s = stablehlo.%s %s, %s : %r" % (r, n, op.operands[0], op.operands[1], ty))
+        elif n in UNARY_OPS:
+            self.emit("%s = stablehlo.%s %s : %r" % (r, n, op.operands[0], ty))
+        elif n in ("reshape", "convert"):
+            self.emit("%s = stablehlo.%s %s : (%r) -> %r" % (r, n, op.operands[0], T[op.operands[0]], ty))
+        elif n == "transpose":
+            self.emit("%s = stablehlo.transpose %s, dims = %s : (%r) -> %r" % (r, op.operands[0], list(op.attrs["perm"]), T[op.operands[0]], ty))
+        elif n == "broadcast_in_dim":
+            self.emit("%s = stablehlo.broadcast_in_dim %s, dims = %s : (%r) -> %r" % (r, op.operands[0], list(op.attrs["dims"]), T[op.operands[0]], ty))
+        elif n == "reduce":
+            self.emit("%s = stablehlo.reduce(%s init: %s) applies stablehlo.%s across dimensions = %s : (%r, %r) -> %r" % (
+                r, op.operands[0], op.operands[1], op.attrs["body"], list(op.attrs["dims"]), T[op.operands[0]], T[op.operands[1]], ty))
+        elif n == "dot_general":
+            a = op.attrs
+            dims = ("batching_dims = %s x %s, " % (list(a["batch_a"]), list(a["batch_b"])) if a["batch_a"] else "") + \
+                "contracting_dims = %s x %s" % (list(a["contract_a"]), list(a["contract_b"]))
+            self.emit("%s = stablehlo.dot_general %s, %s, %s, precision = [DEFAULT, DEFAULT] : (%r, %r) -> %r" % (
+                r, op.operands[0], op.operands[1], dims, T[op.operands[0]], T[op.operands[1]], ty))
+        elif n == "slice":
+            a = op.attrs
+            self.emit("%s = stablehlo.slice %s [%s] : (%r) -> %r" % (r, op.operands[0], ", ".join(
+                "%d:%d" % (s_, l) if st == 1 else "%d:%d:%d" % (s_, l, st) for s_, l, st in zip(a["start"], a["limit"], a["stride"])),
+                T[op.operands[0]], ty))
+        elif n == "concatenate":
+            self.emit("%s = stablehlo.concatenate %s, dim = %d : (%s) -> %r" % (r, ", ".join(op.operands), op.attrs["dim"],
+                                                                                ", ".join(repr(T[o]) for o in op.operands), ty))
+        elif n == "call":
+            lhs = r if len(op.results) == 1 else "%s:%d" % (op.results[0].split("#")[0], len(op.results))
+            outs = repr(ty) if len(op.types) == 1 else "(" + ", ".join(repr(t) for t in op.types) + ")"
+            self.emit("%s = call @%s(%s) : (%s) -> %s" % (lhs, op.attrs["callee"], ", ".join(op.operands),
+                                                         ", ".join(repr(T[o]) for o in op.operands), outs))
+        elif n == "custom_call":
+            self.custom_call(op.results, op.attrs["target"], op.operands, op.attrs["config"], op.types)
+        elif n == "emi.rmsnorm":
+            x, w = op.operands
+            D = ty.shape[-1]
+            x2 = self.reshape(x, (1, D))
+            y2 = self.fresh(TensorType((1, D), ty.dtype))
+            self.custom_call([y2], "emi_rmsnorm_fwd", [x2, w], {"eps": op.attrs["eps"]}, [T[y2]])
+            self.emit("%s = stablehlo.reshape %s : (%r) -> %r" % (r, y2, T[y2], ty))
+        elif n == "emi.swiglu":
+            self.custom_call([r], "emi_swiglu_fwd", list(op.operands), {}, [ty])
+        elif n == "emi.rope":
+            P = ty.shape[0] // 2
+            tab_ty = TensorType((1, P, 2), "f32")
+            tab = self.fresh(tab_ty)
+            self.emit("%s = stablehlo.constant dense<%s> : %r" % (tab, _dense_text(op.attrs["table"].reshape(1, P, 2), tab_ty), tab_ty))
+            x4 = self.reshape(op.operands[0], (1, 1, 1, 2 * P))
+            y4 = self.fresh(T[x4])
+            self.custom_call([y4], "emi_rope", [x4, tab], {"inverse": False}, [T[y4]])
+            self.emit("%s = stablehlo.reshape %s : (%r) -> %r" % (r, y4, T[y4], ty))
+        elif n in ("emi.softmax_dot", "emi.attention_step"):
+            q, k, v = op.operands
+            h = op.attrs.get("heads", 1)
+            d = T[q].shape[0] // h
+            S = T[k].shape[0]
+            q3, k4, v4 = self.reshape(q, (1, h, d)), self.reshape(k, (1, S, h, d)), self.reshape(v, (1, S, h, d))
+            nsplit = (S + 511) // 512
+            outs = [TensorType((1, h, d), ty.dtype), TensorType((1, h), "f32"), TensorType((h * nsplit * (d + 2) * 4,), "i8")]
+            base = self.fresh(outs[0])
+            names = ["%s#%d" % (base, i) for i in range(3)]
+            for nm, t in zip(names, outs):
+                T[nm] = t
+            self.custom_call([base, None, None], "emi_attn_step_fwd", [q3, k4, v4], {"scale": op.attrs["scale"]}, outs)
+            self.emit("%s = stablehlo.reshape %s : (%r) -> %r" % (r, names[0], outs[0], ty))
+        else:
+            raise NotImplementedError("cannot print operator '%s'" % n)
+
+
+def print_module(funcs):
+    """StableHLO text of parsed (and possibly rewritten) functions; fused clusters are printed
+    as `stablehlo.custom_call @emi_*` with `api_version = 4` and their scalars in
+    `backend_config` (the wire format of include/emi_ffi.h), wrapped in the reshapes that bring
+    the operands to the handlers' layouts."""
+    out = ["module {"]
+    for f in funcs.values():
+        p = _Printer(f)
+        for op in f.ops:
+            p.op(op)
+        rets = [o for op in f.ops if op.name == "return" for o in op.operands]
+        out.append("  func.func %s@%s(%s) -> (%s) {" % ("public " if f.name == "main" else "private ", f.name,
+                                                      ", ".join("%s: %r" % (a, t) for a, t in f.args),
+                                                      ", ".join(repr(p.types[o]) for o in rets)))
+        out += p.lines
+        out.append("  }")
+    out.append("}")
+    return "\n".join(out) + "\n"
+
+
+def lower_to_custom_calls(text):
+    """Parse, fold constants, match the llama clusters, and print the module back with the
+    clusters as typed-FFI custom calls to this library's targets."""
+    exe = Executable(text, fuse=True)
+    return print_module(exe.funcs), dict(exe.fused)
 
 
 _CACHE = {}

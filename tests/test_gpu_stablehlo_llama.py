@@ -87,3 +87,24 @@ def test_llama_step_text_through_hlo_call_and_forward_mode():
     lhs = float(np.dot(host(ty), host(dy)))
     rhs = sum(float(np.sum(host(g) * host(t))) for g, t in zip(grads, tans))
     assert abs(lhs - rhs) <= 1e-4 * max(abs(lhs), abs(rhs)), (lhs, rhs)
+
+
+def test_optimized_module_runs_and_matches_the_fused_run():
+    """optimize_module's text (clusters as custom calls to this library's FFI targets) through
+    hlo_call: value and every gradient equal those of the matched graph bit for bit."""
+    from enzyme_ad.jax import hlo_call, optimize_module, vjp
+
+    cfg = dict(STORIES, n_layers=2)
+    text, order = llama_step_text(cfg, 5, "f32")
+    low = optimize_module(text)
+    assert low.count("stablehlo.custom_call") == 2 * 6 + 1 and "stablehlo.exponential" not in low
+    (x, wd, kc, vc, dy), (xr, wr, kcr, vcr, dyr) = _inputs(cfg, 5, "f32", 88, False, 0.05)
+    args = [x] + [wd[k] for k in WEIGHT_ORDER] + [kc, vc]
+    outs = []
+    for src in (text, low):
+        y, f_vjp = vjp(lambda *a: hlo_call(*a, source=src)[0], *args)
+        outs.append((y, f_vjp(dy)))
+    check(outs[1][0], L.forward_step(xr, cfg, wr, kcr, vcr), "f32", "y of the lowered module")
+    assert torch.equal(outs[0][0], outs[1][0])
+    for a, b in zip(outs[0][1], outs[1][1]):
+        assert torch.equal(a, b)

@@ -113,3 +113,35 @@ def test_matcher_leaves_clusters_with_outside_uses_alone():
       return %y : tensor<4xf32>
     }"""
     assert S.Executable(bad).fused["rope"] == 0
+
+
+def test_optimize_module_prints_typed_ffi_custom_calls():
+    """optimize_module: clusters come back as stablehlo.custom_call @emi_* in the typed-FFI wire
+    format (api_version 4, scalars in backend_config, row-major layouts); the printed module
+    parses again and printing it once more changes nothing."""
+    import enzyme_ad.jax as ej
+    from enzyme_ad.jax import stablehlo as S
+
+    text, order = llama_step_text(dict(CFG, n_layers=1), pos=3)
+    low = ej.optimize_module(text)
+    calls = [l.strip() for l in low.splitlines() if "stablehlo.custom_call" in l]
+    assert Counter(l.split("@")[1].split("(")[0] for l in calls) == {"emi_rmsnorm_fwd": 3, "emi_rope": 2, "emi_attn_step_fwd": 1, "emi_swiglu_fwd": 1}
+    assert all("api_version = 4 : i32" in l and "backend_config = {" in l and "operand_layouts = [" in l for l in calls)
+    rms = [l for l in calls if "emi_rmsnorm_fwd" in l][0]
+    assert "backend_config = {eps = 9.999999747e-06 : f32}" in rms
+    assert "operand_layouts = [dense<[1, 0]> : tensor<2xindex>, dense<0> : tensor<1xindex>]" in rms
+    assert ": (tensor<1x288xf32>, tensor<288xf32>) -> tensor<1x288xf32>" in rms
+    att = [l for l in calls if "emi_attn_step_fwd" in l][0]
+    assert ":3 = stablehlo.custom_call" in att and "scale = 1.443375647e-01 : f32" in att or "scale = 1.4433756" in att
+    assert "-> (tensor<1x6x48xf32>, tensor<1x6xf32>, tensor<1200xi8>)" in att          # o, lse, workspace (1 split of 512 keys)
+    for gone in ("stablehlo.exponential", "stablehlo.sqrt", "stablehlo.reduce", "stablehlo.divide"):
+        assert gone not in low
+    again = S.parse_module(low)
+    ccs = [o for o in again["main"].ops if o.name == "custom_call"]
+    assert ccs[0].attrs["target"] == "emi_rmsnorm_fwd" and abs(ccs[0].attrs["config"]["eps"] - 1e-5) < 1e-11
+    assert [o.attrs["config"] for o in ccs if o.attrs["target"] == "emi_rope"][0] == {"inverse": False}
+    assert S.print_module(again) == low
+    with pytest.raises(TypeError):
+        ej.optimize_module(object())
+    with pytest.raises(ValueError):
+        ej.optimize_module(text, pipeline="a{b")
