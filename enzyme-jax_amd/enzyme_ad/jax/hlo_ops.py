@@ -533,3 +533,23 @@ def concatenate(xs, dim):
         parts = [torch.zeros_like(x) if t is None else t for x, t in zip(xs, tans)]
         _set_tan(y, _quiet(lambda: _concat(parts, dim)))
     return y
+
+
+def pad(x, low, high, interior, shape):
+    """stablehlo.pad with a zero padding value: x placed at offset `low` with `interior` zeros
+    between neighbours (Pad is the adjoint of Slice, StableHLOAutoDiffOpInterfaceImpl.cpp:1586-1620,
+    and the other way round)."""
+    low, high, interior = [int(v) for v in low], [int(v) for v in high], [int(v) for v in interior]
+    if any(v < 0 for v in low + high + interior):
+        raise NotImplementedError("stablehlo.pad with negative padding")
+    stride = [i + 1 for i in interior]
+    want = [l + h + (n - 1) * st + 1 if n else l + h for l, h, n, st in zip(low, high, x.shape, stride)]
+    if list(shape) != want:
+        raise ValueError("pad: result shape %s, operands give %s" % (list(shape), want))
+    y = _scatter_box(x, list(shape), low, stride)
+    limit = [l + (n - 1) * st + 1 for l, n, st in zip(low, x.shape, stride)]
+    Tape.record((x,), y, lambda c, acc: (_accumulate(acc[0], _contig(_slice(c, low, limit, stride))),))
+    tans = _tan(x)
+    if tans is not None and tans[0] is not None:
+        _set_tan(y, _quiet(lambda: _scatter_box(tans[0], list(shape), low, stride)))
+    return y

@@ -502,10 +502,11 @@ def append_row(cache, row):
     return out
 
 
-def attention_step(q, k_cache, v_cache, n_heads, scale=None):
+def attention_step(q, k_cache, v_cache, n_heads, scale=None, return_lse=False):
     """Attention of one token against its layer's cache (test/llama.py:178-209): q is
     [n_heads*head_dim], the caches are [seq_kv, n_heads*head_dim] and already hold the
-    token's own row.  Returns the concatenated per-head outputs [n_heads*head_dim]."""
+    token's own row.  Returns the concatenated per-head outputs [n_heads*head_dim] (with
+    return_lse also the fp32 log-sum-exp per head, [1, n_heads], which the adjoint reads)."""
     _dev(q, k_cache, v_cache)
     _same_dtype(q, k_cache, v_cache)
     D = q.shape[-1]
@@ -539,7 +540,7 @@ def attention_step(q, k_cache, v_cache, n_heads, scale=None):
         N.check(N.lib().emi_attn_step_jvp(_stream(), _p(q), _p(k_cache), _p(v_cache), _p(o), _p(lse), _p(tq), _p(tk), _p(tv),
                                           _p(to), _p(ws), nbytes, 1, n_heads, S, d, *strides, float(scale), _code(q)))
         _set_tan(o, to)
-    return o
+    return (o, lse) if return_lse else o
 
 
 def embedding(tokens, table):

@@ -16,6 +16,7 @@ The MLIR pass pipeline named by `pipeline_options` selects nothing here - the
 fused kernels implement the optimized graph directly - but the strings are
 still built, parsed and carried so that code written for the reference runs.
 """
+import re
 from collections.abc import Callable, Sequence
 from typing import Any
 
@@ -429,15 +430,30 @@ def optimize_module(mod, pipeline=None):
     """primitives.py:280-284 runs the MLIR optimizer over a module in place.  Here `mod` is the
     module's StableHLO text and the result is returned: constants folded, the llama clusters
     replaced by `stablehlo.custom_call @emi_*` (api_version 4, scalars in `backend_config`), the
-    other operators printed back unchanged.  An XLA client with this library's FFI handlers
-    registered can compile the result; `hlo_call` runs it as well.  `pipeline` is parsed for
-    validity only."""
-    from . import stablehlo
+    other operators printed back unchanged.  When the pipeline's last `enzyme-wrap` pass asks
+    for `mode=ReverseModeCombined` (the string `enzyme_vjp` builds, :1385-1419) the result is
+    the reverse-mode program instead: main(args..., cotangents of the active results) ->
+    cotangents of the active arguments, with the clusters' adjoints as custom calls.  An XLA
+    client with this library's FFI handlers registered can compile either; `hlo_call` runs
+    them as well.  The other passes of the pipeline are parsed for validity only."""
+    from . import stablehlo, stablehlo_ad
 
-    parse_pass_pipeline(full_optimization_pass_pipeline() if pipeline is None else pipeline)
+    passes = parse_pass_pipeline(full_optimization_pass_pipeline() if pipeline is None else pipeline)
     if not isinstance(mod, str):
         raise TypeError("optimize_module takes the module as StableHLO text (str); there are no MLIR module objects here")
-    return stablehlo.lower_to_custom_calls(mod)[0]
+    wraps = [opts for name, opts in passes if name == "enzyme-wrap"]
+    if not wraps:
+        return stablehlo.lower_to_custom_calls(mod)[0]
+    wrap = "enzyme-wrap{" + wraps[-1] + " }"
+    mode = re.search(r"mode=(\w+)", wrap)
+    if mode is None or mode.group(1) != "ReverseModeCombined":
+        raise NotImplementedError("optimize_module differentiates symbolically in mode=ReverseModeCombined only "
+                                  "(forward mode runs on the tape: jvp); got %s" % (mode.group(1) if mode else "no mode"))
+    fn = re.search(r"infn=(\w+)", wrap)
+    active = lambda acts: [a != "enzyme_const" for a in acts]
+    return stablehlo_ad.reverse_module_text(mod, fn.group(1) if fn else "main",
+                                            arg_active=active(arg_activity_from_pipeline(wrap)[1]),
+                                            ret_active=active(ret_activity_from_pipeline(wrap)[1]))
 
 
 def export(outfile, func, *args, argv=(), jit_options={}):

@@ -12,8 +12,8 @@ function that calls `hlo_call` differentiate through the parsed graph.
 The accepted text is MLIR's printed form of the operators JAX emits for such functions
 (pretty or quoted-generic operator names): constant, add, subtract, multiply, divide, maximum,
 minimum, power, negate, exponential, log, sqrt, rsqrt, logistic, tanh, sine, cosine, convert, reshape,
-transpose, broadcast_in_dim, reduce (add / maximum), dot_general, slice, concatenate, call,
-return.  Anything else raises `NotImplementedError` naming the operator.
+transpose, broadcast_in_dim, reduce (add / maximum), dot_general, slice, pad, concatenate, call,
+custom_call (this library's targets), return.  Anything else raises `NotImplementedError` naming the operator.
 """
 import math
 import re
@@ -22,6 +22,7 @@ import struct
 import numpy as np
 import torch
 
+from . import _native as N
 from . import hlo_ops as H
 from . import ops
 
@@ -463,6 +464,8 @@ def _parse_op(sc):
         attrs = {"dims": attrs["dims"]}
     elif short == "concatenate":
         attrs = {"dim": int(attrs["dim"])}
+    elif short == "pad":
+        attrs = {"low": attrs["low"], "high": attrs["high"], "interior": attrs.get("interior", [0] * len(attrs["low"]))}
     elif short in BINARY_OPS or short in UNARY_OPS or short in ("reshape", "convert"):
         attrs = {}
     else:
@@ -988,6 +991,10 @@ class Executable:
             return [H.slice_(xs[0], op.attrs["start"], op.attrs["limit"], op.attrs["stride"])]
         if n == "concatenate":
             return [H.concatenate(xs, op.attrs["dim"])]
+        if n == "pad":
+            if _splat(f.defs.get(op.operands[1])) != 0.0:
+                raise NotImplementedError("stablehlo.pad with a padding value other than a zero constant")
+            return [H.pad(xs[0], op.attrs["low"], op.attrs["high"], op.attrs["interior"], op.types[0].shape)]
         if n == "call":
             return self.run(xs, op.attrs["callee"])
         if n == "custom_call":
@@ -1039,9 +1046,38 @@ def _custom_call_impl(self, op, xs):
         if q.dim() != 3 or q.shape[0] != 1 or k.dim() != 4:
             raise NotImplementedError("custom call emi_attn_step_fwd is run for one sequence per call (batch = 1)")
         h, d = q.shape[1], q.shape[2]
-        o = ops.attention_step(ops.reshape(q, (h * d,)), ops.reshape(k, (k.shape[1], h * d)), ops.reshape(v, (v.shape[1], h * d)),
-                               h, cfg["scale"])
-        return [ops.reshape(o, (1, h, d))] + [None] * (len(op.results) - 1)       # lse and workspace stay inside the operator
+        o, lse = ops.attention_step(ops.reshape(q, (h * d,)), ops.reshape(k, (k.shape[1], h * d)),
+                                    ops.reshape(v, (v.shape[1], h * d)), h, cfg["scale"], return_lse=True)
+        return [ops.reshape(o, (1, h, d)), lse, None][:len(op.results)]           # the workspace stays inside the operator
+    # adjoint targets: what a reverse-mode module calls; they run the kernels directly and are
+    # not themselves differentiable
+    lib, st = N.lib(), ops._stream()
+    P = lambda t: None if t is None else t.data_ptr()
+    if target == "emi_rmsnorm_bwd":
+        x, w, dy = (_packed(t) for t in xs[:3])
+        rows, dim = x.numel() // x.shape[-1], x.shape[-1]
+        dx, dg = torch.empty_like(x), torch.empty_like(w)
+        nbytes = lib.emi_rmsnorm_bwd_workspace_bytes(rows, dim)
+        ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=x.device)
+        N.check(lib.emi_rmsnorm_bwd(st, P(x), P(w), P(dy), None, P(dx), P(dg), P(ws), nbytes, rows, dim, float(cfg.get("eps", 1e-5)),
+                                    ops._code(x)))
+        return [dx, dg, None][:len(op.results)]
+    if target == "emi_swiglu_bwd":
+        a, b_, dg = (_packed(t) for t in xs)
+        da, db = torch.empty_like(a), torch.empty_like(a)
+        N.check(lib.emi_swiglu_bwd(st, P(a), P(b_), P(dg), P(da), P(db), a.numel(), ops._code(a)))
+        return [da, db]
+    if target == "emi_attn_step_bwd":
+        q, k, v, o, lse, do = (_packed(t) for t in xs)
+        if q.dim() != 3 or q.shape[0] != 1 or k.dim() != 4:
+            raise NotImplementedError("custom call emi_attn_step_bwd is run for one sequence per call (batch = 1)")
+        h, d, S = q.shape[1], q.shape[2], k.shape[1]
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        nbytes = lib.emi_attn_step_workspace_bytes(1, h, S, d)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
+        N.check(lib.emi_attn_step_bwd(st, P(q), P(k), P(v), P(o), P(lse), P(do), P(dq), P(dk), P(dv), P(ws), nbytes, 1, h, S, d,
+                                      h * d, d, S * h * d, d, h * d, float(cfg["scale"]), ops._code(q)))
+        return [dq, dk, dv, None][:len(op.results)]
     raise NotImplementedError("custom call target '%s' is not one of this library's" % target)
 
 
@@ -1168,38 +1204,11 @@ class _Printer:
                                                          ", ".join(repr(T[o]) for o in op.operands), outs))
         elif n == "custom_call":
             self.custom_call(op.results, op.attrs["target"], op.operands, op.attrs["config"], op.types)
-        elif n == "emi.rmsnorm":
-            x, w = op.operands
-            D = ty.shape[-1]
-            x2 = self.reshape(x, (1, D))
-            y2 = self.fresh(TensorType((1, D), ty.dtype))
-            self.custom_call([y2], "emi_rmsnorm_fwd", [x2, w], {"eps": op.attrs["eps"]}, [T[y2]])
-            self.emit("%s = stablehlo.reshape %s : (%r) -> %r" % (r, y2, T[y2], ty))
-        elif n == "emi.swiglu":
-            self.custom_call([r], "emi_swiglu_fwd", list(op.operands), {}, [ty])
-        elif n == "emi.rope":
-            P = ty.shape[0] // 2
-            tab_ty = TensorType((1, P, 2), "f32")
-            tab = self.fresh(tab_ty)
-            self.emit("%s = stablehlo.constant dense<%s> : %r" % (tab, _dense_text(op.attrs["table"].reshape(1, P, 2), tab_ty), tab_ty))
-            x4 = self.reshape(op.operands[0], (1, 1, 1, 2 * P))
-            y4 = self.fresh(T[x4])
-            self.custom_call([y4], "emi_rope", [x4, tab], {"inverse": False}, [T[y4]])
-            self.emit("%s = stablehlo.reshape %s : (%r) -> %r" % (r, y4, T[y4], ty))
-        elif n in ("emi.softmax_dot", "emi.attention_step"):
-            q, k, v = op.operands
-            h = op.attrs.get("heads", 1)
-            d = T[q].shape[0] // h
-            S = T[k].shape[0]
-            q3, k4, v4 = self.reshape(q, (1, h, d)), self.reshape(k, (1, S, h, d)), self.reshape(v, (1, S, h, d))
-            nsplit = (S + 511) // 512
-            outs = [TensorType((1, h, d), ty.dtype), TensorType((1, h), "f32"), TensorType((h * nsplit * (d + 2) * 4,), "i8")]
-            base = self.fresh(outs[0])
-            names = ["%s#%d" % (base, i) for i in range(3)]
-            for nm, t in zip(names, outs):
-                T[nm] = t
-            self.custom_call([base, None, None], "emi_attn_step_fwd", [q3, k4, v4], {"scale": op.attrs["scale"]}, outs)
-            self.emit("%s = stablehlo.reshape %s : (%r) -> %r" % (r, names[0], outs[0], ty))
+        elif n == "pad":
+            a = op.attrs
+            self.emit("%s = stablehlo.pad %s, %s, low = %s, high = %s, interior = %s : (%r, %r) -> %r" % (
+                r, op.operands[0], op.operands[1], list(a["low"]), list(a["high"]), list(a["interior"]), T[op.operands[0]],
+                T[op.operands[1]], ty))
         else:
             raise NotImplementedError("cannot print operator '%s'" % n)
 
@@ -1209,8 +1218,11 @@ def print_module(funcs):
     as `stablehlo.custom_call @emi_*` with `api_version = 4` and their scalars in
     `backend_config` (the wire format of include/emi_ffi.h), wrapped in the reshapes that bring
     the operands to the handlers' layouts."""
+    from .stablehlo_ad import lower_fused
+
     out = ["module {"]
     for f in funcs.values():
+        f = lower_fused(f)
         p = _Printer(f)
         for op in f.ops:
             p.op(op)

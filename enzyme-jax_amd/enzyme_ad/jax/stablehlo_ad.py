@@ -1,0 +1,394 @@
+"""Rewrites on parsed StableHLO functions: lowering of matched clusters to typed-FFI custom calls,
+and symbolic reverse mode.
+
+`reverse_function` is the counterpart, for the operators of the llama path, of the reference's
+`enzyme-wrap{... mode=ReverseModeCombined}` pass (src/enzyme_ad/jax/primitives.py:1385-1419): from a
+function f(args) -> results it builds f_rev(args, cotangents of results) -> cotangents of args,
+recomputing the forward values and then walking the operators backwards with the reference's
+rules (Implementations/HLODerivatives.td: Add :964, Div :1133, DotGeneral :1166, Exp :1182,
+Mul :1221, Neg :1228, Reshape :1271, Rsqrt :1283, Convert :1290, Sub :1312, Sqrt :1320,
+Transpose :1334; StableHLOAutoDiffOpInterfaceImpl.cpp: BroadcastInDim :1474, Slice :1586,
+Reduce :1833, Concatenate :2015).  Clusters that were matched to fused kernels differentiate
+into the matching adjoint custom calls (`emi_rmsnorm_bwd`, `emi_swiglu_bwd`, `emi_rope` with
+`inverse`, `emi_attn_step_bwd`), so the printed reverse module is what an XLA client with this
+library's handlers would compile for `jax.vjp`.
+"""
+import re
+
+import numpy as np
+
+from .stablehlo import BINARY_OPS, UNARY_OPS, Func, Op, TensorType, _drop_dead, _splat
+
+FLOAT = ("f32", "bf16", "f16", "f64")
+
+
+def _types_of(func):
+    types = {a: t for a, t in func.args}
+    for op in func.ops:
+        for r, t in zip(op.results, op.types):
+            types[r] = t
+    return types
+
+
+class _Builder:
+    def __init__(self, func, prefix):
+        self.ops, self.types, self.prefix = [], _types_of(func), prefix
+        used = [int(m.group(1)) for n in self.types for m in [re.fullmatch(r"%%%s(\d+)(?:#\d+)?" % prefix, n)] if m]
+        self.n = max(used) + 1 if used else 0
+
+    def new(self, ty):
+        name = "%%%s%d" % (self.prefix, self.n)
+        self.n += 1
+        self.types[name] = ty
+        return name
+
+    def emit(self, name, operands, attrs, ty):
+        r = self.new(ty)
+        self.ops.append(Op(name, [r], list(operands), attrs, [ty]))
+        return r
+
+    def const(self, value, ty):
+        return self.emit("constant", [], {"value": np.full(ty.shape, value, dtype=np.float32)}, ty)
+
+    def reshape(self, v, shape):
+        ty = TensorType(shape, self.types[v].dtype)
+        return v if self.types[v].shape == ty.shape else self.emit("reshape", [v], {}, ty)
+
+    def custom_call(self, target, operands, config, tys):
+        base = self.new(tys[0])
+        names = [base] if len(tys) == 1 else ["%s#%d" % (base, i) for i in range(len(tys))]
+        for n, t in zip(names, tys):
+            self.types[n] = t
+        self.ops.append(Op("custom_call", names, list(operands), {"target": target, "config": dict(config)}, list(tys)))
+        return names
+
+    def binary(self, name, a, b):
+        return self.emit(name, [a, b], {}, self.types[a])
+
+    def unary(self, name, a):
+        return self.emit(name, [a], {}, self.types[a])
+
+
+def _step_workspace(heads, rows, head_dim):
+    return heads * ((rows + 511) // 512) * (head_dim + 2) * 4          # emi_attn_step_workspace_bytes for one sequence
+
+
+def lower_fused(func):
+    """A copy of `func` with the matcher's fused operators written as custom calls to this
+    library's FFI targets (api_version 4; scalars in backend_config), wrapped in the reshapes
+    that bring the operands to the handlers' layouts."""
+    if not any(op.name.startswith("emi.") for op in func.ops):
+        return func
+    b = _Builder(func, "emi")
+    T = b.types
+    for op in func.ops:
+        n = op.name
+        ty = op.types[0] if op.types else None
+        if n == "emi.rmsnorm":
+            x, w = op.operands
+            D = ty.shape[-1]
+            y2, = b.custom_call("emi_rmsnorm_fwd", [b.reshape(x, (1, D)), w], {"eps": op.attrs["eps"]}, [TensorType((1, D), ty.dtype)])
+            b.ops.append(Op("reshape", op.results, [y2], {}, op.types))
+        elif n == "emi.swiglu":
+            b.ops.append(Op("custom_call", op.results, list(op.operands), {"target": "emi_swiglu_fwd", "config": {}}, op.types))
+        elif n == "emi.rope":
+            P = ty.shape[0] // 2
+            tab = b.emit("constant", [], {"value": np.asarray(op.attrs["table"], dtype=np.float32).reshape(1, P, 2)},
+                         TensorType((1, P, 2), "f32"))
+            x4 = b.reshape(op.operands[0], (1, 1, 1, 2 * P))
+            y4, = b.custom_call("emi_rope", [x4, tab], {"inverse": False}, [T[x4]])
+            b.ops.append(Op("reshape", op.results, [y4], {}, op.types))
+        elif n in ("emi.softmax_dot", "emi.attention_step"):
+            q, k, v = op.operands
+            h = op.attrs.get("heads", 1)
+            d, S = T[q].shape[0] // h, T[k].shape[0]
+            outs = [TensorType((1, h, d), ty.dtype), TensorType((1, h), "f32"), TensorType((_step_workspace(h, S, d),), "i8")]
+            o3, _, _ = b.custom_call("emi_attn_step_fwd", [b.reshape(q, (1, h, d)), b.reshape(k, (1, S, h, d)), b.reshape(v, (1, S, h, d))],
+                                     {"scale": op.attrs["scale"]}, outs)
+            b.ops.append(Op("reshape", op.results, [o3], {}, op.types))
+        else:
+            b.ops.append(op)
+    return Func(func.name, func.args, func.result_types, b.ops)
+
+
+def inline_calls(funcs, fn="main"):
+    """`fn` with every `call` replaced by the callee's operators (renamed), recursively."""
+    counter = [0]
+
+    def inline(f, depth=0):
+        if depth > 32:
+            raise RecursionError("call depth over 32 (recursive functions are not supported)")
+        out = []
+        for op in f.ops:
+            if op.name != "call":
+                out.append(op)
+                continue
+            callee = inline(funcs[op.attrs["callee"]], depth + 1)
+            counter[0] += 1
+            tag = "%%c%d_" % counter[0]
+            ren = {a: o for (a, _), o in zip(callee.args, op.operands)}
+            for cop in callee.ops:
+                if cop.name == "return":
+                    for r, o, t in zip(op.results, cop.operands, op.types):
+                        out.append(Op("reshape", [r], [ren.get(o, o)], {}, [t]))        # identity: binds the call's result names
+                    continue
+                res = [tag + r[1:] for r in cop.results]
+                ren.update(zip(cop.results, res))
+                out.append(Op(cop.name, res, [ren.get(o, o) for o in cop.operands], cop.attrs, cop.types))
+        return Func(f.name, f.args, f.result_types, out)
+
+    return inline(funcs[fn])
+
+
+def reverse_function(func, name=None, arg_active=None, ret_active=None):
+    """f_rev(args..., one cotangent per active result) -> one cotangent per active argument
+    (default: every floating-point argument and result; `enzyme_const` entries of the
+    reference's activity lists are the inactive ones).  `func` must be call-free (see
+    `inline_calls`); fused operators are lowered first."""
+    func = lower_fused(func)
+    b = _Builder(func, "r")
+    T = b.types
+    ret = [op for op in func.ops if op.name == "return"]
+    if len(ret) != 1:
+        raise ValueError("reverse mode needs exactly one return")
+    results = list(ret[0].operands)
+    primal = [op for op in func.ops if op.name != "return"]
+    b.ops = list(primal)
+    ct_args = []
+    ct = {}
+
+    def accum(v, g):
+        if T[v].dtype not in FLOAT:
+            return
+        if T[g] != T[v]:
+            raise RuntimeError("cotangent %r for a value of type %r" % (T[g], T[v]))
+        ct[v] = g if v not in ct else b.binary("add", ct[v], g)
+
+    if ret_active is None:
+        ret_active = [T[r].dtype in FLOAT for r in results]
+    if arg_active is None:
+        arg_active = [t.dtype in FLOAT for _, t in func.args]
+    if len(ret_active) != len(results) or len(arg_active) != len(func.args):
+        raise ValueError("activity lists do not match the function: %d results, %d arguments" % (len(results), len(func.args)))
+    for i, r in enumerate(results):
+        if not ret_active[i]:
+            continue
+        a = "%%ct%d" % i
+        T[a] = T[r]
+        ct_args.append((a, T[r]))
+        accum(r, a)
+
+    def splat_like(v, value):
+        return b.const(value, T[v])
+
+    for op in reversed(primal):
+        cs = [ct.pop(r, None) for r in op.results]
+        if all(c is None for c in cs):
+            continue
+        c = cs[0]
+        n, xs = op.name, op.operands
+        r = op.results[0]
+        if n == "constant":
+            continue
+        if n == "add":
+            accum(xs[0], c)
+            accum(xs[1], c)
+        elif n == "subtract":
+            accum(xs[0], c)
+            accum(xs[1], b.unary("negate", c))
+        elif n == "multiply":
+            accum(xs[0], b.binary("multiply", c, xs[1]))
+            accum(xs[1], b.binary("multiply", c, xs[0]))
+        elif n == "divide":
+            q = b.binary("divide", c, xs[1])
+            accum(xs[0], q)
+            accum(xs[1], b.unary("negate", b.binary("multiply", q, r)))
+        elif n == "negate":
+            accum(xs[0], b.unary("negate", c))
+        elif n == "exponential":
+            accum(xs[0], b.binary("multiply", c, r))
+        elif n == "log":
+            accum(xs[0], b.binary("divide", c, xs[0]))
+        elif n == "sqrt":
+            # c / (2 sqrt(x)); the reference also selects 0 where x == 0 (Sqrt rule :1320), which
+            # needs compare / select and is not reproduced here
+            accum(xs[0], b.binary("divide", c, b.binary("multiply", splat_like(r, 2.0), r)))
+        elif n == "rsqrt":
+            cube = b.binary("multiply", b.binary("multiply", r, r), r)
+            accum(xs[0], b.binary("multiply", b.binary("multiply", splat_like(r, -0.5), c), cube))
+        elif n == "logistic":
+            accum(xs[0], b.binary("multiply", b.binary("multiply", c, r), b.binary("subtract", splat_like(r, 1.0), r)))
+        elif n == "tanh":
+            accum(xs[0], b.binary("multiply", c, b.binary("subtract", splat_like(r, 1.0), b.binary("multiply", r, r))))
+        elif n == "sine":
+            accum(xs[0], b.binary("multiply", c, b.unary("cosine", xs[0])))
+        elif n == "cosine":
+            accum(xs[0], b.unary("negate", b.binary("multiply", c, b.unary("sine", xs[0]))))
+        elif n == "convert":
+            accum(xs[0], c if T[xs[0]].dtype == T[c].dtype else b.emit("convert", [c], {}, T[xs[0]]))
+        elif n == "reshape":
+            accum(xs[0], b.reshape(c, T[xs[0]].shape))
+        elif n == "transpose":
+            perm = list(op.attrs["perm"])
+            accum(xs[0], b.emit("transpose", [c], {"perm": [perm.index(i) for i in range(len(perm))]}, T[xs[0]]))
+        elif n == "broadcast_in_dim":
+            dims, xt, ot = list(op.attrs["dims"]), T[xs[0]], T[r]
+            red = [d for d in range(len(ot.shape)) if d not in dims] + \
+                  [d for i, d in enumerate(dims) if xt.shape[i] == 1 and ot.shape[d] != 1]
+            g = c
+            if red:
+                kept = [ot.shape[d] for d in range(len(ot.shape)) if d not in red]
+                zero = b.const(0.0, TensorType((), ot.dtype))
+                g = b.emit("reduce", [c, zero], {"dims": sorted(red), "body": "add"}, TensorType(kept, ot.dtype))
+                order = [d for d in dims if d not in red]
+                if order != sorted(order):
+                    rank = sorted(order)
+                    perm = [rank.index(d) for d in order]
+                    g = b.emit("transpose", [g], {"perm": perm}, TensorType([kept[p] for p in perm], ot.dtype))
+            accum(xs[0], b.reshape(g, xt.shape))
+        elif n == "reduce":
+            if op.attrs["body"] != "add":
+                raise NotImplementedError("symbolic reverse mode of reduce with a %s body" % op.attrs["body"])
+            xt = T[xs[0]]
+            kept = [d for d in range(len(xt.shape)) if d not in op.attrs["dims"]]
+            accum(xs[0], b.emit("broadcast_in_dim", [c], {"dims": kept}, xt))
+        elif n == "dot_general":
+            _reverse_dot_general(b, op, c, accum)
+        elif n == "slice":
+            xt, a = T[xs[0]], op.attrs
+            shape = T[r].shape
+            high = [xt.shape[i] - (a["start"][i] + (shape[i] - 1) * a["stride"][i] + 1) if shape[i] else xt.shape[i] - a["start"][i]
+                    for i in range(len(shape))]
+            zero = b.const(0.0, TensorType((), xt.dtype))
+            accum(xs[0], b.emit("pad", [c, zero], {"low": list(a["start"]), "high": high, "interior": [s - 1 for s in a["stride"]]}, xt))
+        elif n == "pad":
+            a, xt = op.attrs, T[xs[0]]
+            stride = [i + 1 for i in a["interior"]]
+            limit = [l + (m - 1) * st + 1 for l, m, st in zip(a["low"], xt.shape, stride)]
+            accum(xs[0], b.emit("slice", [c], {"start": list(a["low"]), "limit": limit, "stride": stride}, xt))
+        elif n == "concatenate":
+            dim, at = op.attrs["dim"], 0
+            for x in xs:
+                xt = T[x]
+                start = [0] * len(xt.shape)
+                limit = list(T[r].shape)
+                start[dim], limit[dim] = at, at + xt.shape[dim]
+                at += xt.shape[dim]
+                accum(x, b.emit("slice", [c], {"start": start, "limit": limit, "stride": [1] * len(start)}, xt))
+        elif n == "custom_call":
+            _reverse_custom_call(b, op, cs, accum)
+        elif n == "call":
+            raise NotImplementedError("symbolic reverse mode needs a call-free function (inline_calls)")
+        else:
+            raise NotImplementedError("symbolic reverse mode of stablehlo.%s" % n)
+
+    outs = []
+    for (a, t), active in zip(func.args, arg_active):
+        if not active:
+            continue
+        if t.dtype not in FLOAT:
+            raise ValueError("argument %s of type %r cannot be active" % (a, t))
+        outs.append(ct[a] if a in ct else b.const(0.0, t))
+    b.ops.append(Op("return", [], outs, {}, []))
+    rev = Func(name or func.name + "_rev", list(func.args) + ct_args, [T[o] for o in outs], b.ops)
+    _drop_dead(rev)
+    return rev
+
+
+def _reverse_dot_general(b, op, c, accum):
+    T = b.types
+    a_, b_ = op.operands
+    at, bt = T[a_], T[b_]
+    ba, bb, ca, cb = (list(op.attrs[k]) for k in ("batch_a", "batch_b", "contract_a", "contract_b"))
+    fa = [d for d in range(len(at.shape)) if d not in ba and d not in ca]
+    fb = [d for d in range(len(bt.shape)) if d not in bb and d not in cb]
+    nb, nfa, nfb = len(ba), len(fa), len(fb)
+
+    def grad(other, ot, obatch, ofree, ocontract, mine_t, mine_batch, mine_free, mine_contract, cfree_at):
+        # contract c with `other` over other's free dims: batch, my free dims, other's contracting dims (in its order)
+        rest = sorted(ocontract)
+        shape = [ot.shape[d] for d in obatch] + [mine_t.shape[d] for d in mine_free] + [ot.shape[d] for d in rest]
+        g = b.emit("dot_general", [c, other], {"batch_a": list(range(nb)), "batch_b": list(obatch),
+                                                "contract_a": list(range(cfree_at, cfree_at + len(ofree))), "contract_b": list(ofree)},
+                   TensorType(shape, mine_t.dtype))
+        src = {}
+        for i, d in enumerate(mine_batch):
+            src[d] = i
+        for i, d in enumerate(mine_free):
+            src[d] = nb + i
+        for i, d in enumerate(rest):
+            src[mine_contract[ocontract.index(d)]] = nb + len(mine_free) + i
+        perm = [src[d] for d in range(len(mine_t.shape))]
+        if perm != list(range(len(perm))):
+            g = b.emit("transpose", [g], {"perm": perm}, mine_t)
+        return g
+
+    # c dims: batch (nb), free of a (nfa), free of b (nfb)
+    accum(a_, grad(b_, bt, bb, fb, cb, at, ba, fa, ca, nb + nfa))
+    # for b: c's free-of-a dims are contracted with a's free dims; the product's free dims are c's free-of-b dims
+    rest = sorted(ca)
+    shape = [at.shape[d] for d in ba] + [bt.shape[d] for d in fb] + [at.shape[d] for d in rest]
+    g = b.emit("dot_general", [c, a_], {"batch_a": list(range(nb)), "batch_b": list(ba),
+                                        "contract_a": list(range(nb, nb + nfa)), "contract_b": list(fa)}, TensorType(shape, bt.dtype))
+    src = {}
+    for i, d in enumerate(bb):
+        src[d] = i
+    for i, d in enumerate(fb):
+        src[d] = nb + i
+    for i, d in enumerate(rest):
+        src[cb[ca.index(d)]] = nb + nfb + i
+    perm = [src[d] for d in range(len(bt.shape))]
+    if perm != list(range(len(perm))):
+        g = b.emit("transpose", [g], {"perm": perm}, bt)
+    accum(b_, g)
+
+
+def _reverse_custom_call(b, op, cs, accum):
+    T = b.types
+    target, cfg, xs = op.attrs["target"], op.attrs["config"], op.operands
+    c = cs[0]
+    if target == "emi_rmsnorm_fwd":
+        from . import _native as N
+        x, w = xs
+        rows = int(np.prod(T[x].shape[:-1])) if len(T[x].shape) > 1 else 1
+        nbytes = int(N.lib().emi_rmsnorm_bwd_workspace_bytes(rows, T[x].shape[-1]))
+        dx, dg, _ = b.custom_call("emi_rmsnorm_bwd", [x, w, c], {"eps": cfg.get("eps", 1e-5)},
+                                  [T[x], T[w], TensorType((nbytes,), "i8")])
+        accum(x, dx)
+        accum(w, dg)
+    elif target == "emi_swiglu_fwd":
+        da, db = b.custom_call("emi_swiglu_bwd", [xs[0], xs[1], c], {}, [T[xs[0]], T[xs[1]]])
+        accum(xs[0], da)
+        accum(xs[1], db)
+    elif target == "emi_add":
+        accum(xs[0], c)
+        accum(xs[1], c)
+    elif target == "emi_rope":
+        g, = b.custom_call("emi_rope", [c, xs[1]], {"inverse": not cfg.get("inverse", False)}, [T[xs[0]]])
+        accum(xs[0], g)
+    elif target == "emi_attn_step_fwd":
+        if cs[1] is not None or (len(cs) > 2 and cs[2] is not None):
+            raise NotImplementedError("cotangents of the log-sum-exp or workspace results of emi_attn_step_fwd")
+        if c is None:
+            return
+        q, k, v = xs
+        o, lse, ws = op.results
+        dq, dk, dv, _ = b.custom_call("emi_attn_step_bwd", [q, k, v, o, lse, c], {"scale": cfg["scale"]}, [T[q], T[k], T[v], T[ws]])
+        accum(q, dq)
+        accum(k, dk)
+        accum(v, dv)
+    else:
+        raise NotImplementedError("symbolic reverse mode of custom call '%s'" % target)
+
+
+def reverse_module_text(text, fn="main", arg_active=None, ret_active=None):
+    """StableHLO text in, StableHLO text of the reverse-mode program out: calls inlined,
+    constants folded, clusters matched, `reverse_function`, printed with the fused operators
+    and their adjoints as typed-FFI custom calls."""
+    from .stablehlo import fold_constants, fuse_clusters, parse_module, print_module
+
+    f = inline_calls(parse_module(text), fn)
+    fold_constants(f)
+    fuse_clusters(f)
+    rev = reverse_function(f, name="main", arg_active=arg_active, ret_active=ret_active)
+    return print_module({"main": rev})

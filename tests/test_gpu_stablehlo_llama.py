@@ -108,3 +108,67 @@ def test_optimized_module_runs_and_matches_the_fused_run():
     assert torch.equal(outs[0][0], outs[1][0])
     for a, b in zip(outs[0][1], outs[1][1]):
         assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("dt,pos", [("f32", 1), ("f32", 7), ("bf16", 40)])
+def test_reverse_module_of_the_llama_step(dt, pos):
+    """The symbolic reverse-mode module (forward recomputation + adjoint custom calls, printed
+    as StableHLO text) run through hlo_call: its 13 cotangents against the oracle's
+    forward_step_vjp and against the tape's vjp of the same text."""
+    from enzyme_ad.jax import hlo_call, stablehlo_ad, vjp
+
+    cfg = dict(STORIES, n_layers=3)
+    text, order = llama_step_text(cfg, pos, dt)
+    rev = stablehlo_ad.reverse_module_text(text)
+    (x, wd, kc, vc, dy), (xr, wr, kcr, vcr, dyr) = _inputs(cfg, pos, dt, 90 + pos, pos == 1, 0.05)
+    args = [x] + [wd[k] for k in WEIGHT_ORDER] + [kc, vc]
+    grads = hlo_call(*(args + [dy]), source=rev)
+    assert len(grads) == len(args)
+    ry, rdx, rgw, rdkc, rdvc = L.forward_step_vjp(xr, cfg, wr, kcr, vcr, dyr)
+    want = [rdx] + [rgw[k] for k in WEIGHT_ORDER] + [rdkc, rdvc]
+    for name, g, w in zip(order, grads, want):
+        check(g, w, dt, "reverse module, cotangent of " + name)
+    _, f_vjp = vjp(lambda *a: hlo_call(*a, source=text)[0], *args)
+    for name, g, t in zip(order, grads, f_vjp(dy)):
+        check(g, host(t), dt, "reverse module vs tape, " + name, factor=0.1 if dt == "f32" else 1.0)
+
+
+def test_reverse_module_of_generic_operators_matches_the_tape():
+    """A module of generic operators only (broadcasts, reductions, transposes, slices with
+    strides, concatenation, a batched product, unary maps): symbolic reverse mode against the
+    tape's reverse mode."""
+    from enzyme_ad.jax import hlo_call, stablehlo_ad, vjp
+
+    text = """
+    func.func @main(%a: tensor<4x6xf32>, %b: tensor<6xf32>, %w: tensor<2x3x5xf32>) -> (tensor<4x6xf32>, tensor<2x4x5xf32>, tensor<f32>) {
+      %bb = stablehlo.broadcast_in_dim %b, dims = [1] : (tensor<6xf32>) -> tensor<4x6xf32>
+      %m = stablehlo.multiply %a, %bb : tensor<4x6xf32>
+      %e = stablehlo.exponential %m : tensor<4x6xf32>
+      %t = stablehlo.tanh %a : tensor<4x6xf32>
+      %d = stablehlo.divide %e, %t : tensor<4x6xf32>
+      %z = stablehlo.constant dense<0.000000e+00> : tensor<f32>
+      %rs = stablehlo.reduce(%d init: %z) applies stablehlo.add across dimensions = [1] : (tensor<4x6xf32>, tensor<f32>) -> tensor<4xf32>
+      %rb = stablehlo.broadcast_in_dim %rs, dims = [0] : (tensor<4xf32>) -> tensor<4x6xf32>
+      %lg = stablehlo.logistic %rb : tensor<4x6xf32>
+      %o1 = stablehlo.subtract %d, %lg : tensor<4x6xf32>
+      %s0 = stablehlo.slice %a [0:4, 0:6:2] : (tensor<4x6xf32>) -> tensor<4x3xf32>
+      %s1 = stablehlo.slice %m [0:4, 3:6] : (tensor<4x6xf32>) -> tensor<4x3xf32>
+      %cc = stablehlo.concatenate %s0, %s1, dim = 0 : (tensor<4x3xf32>, tensor<4x3xf32>) -> tensor<8x3xf32>
+      %c3 = stablehlo.reshape %cc : (tensor<8x3xf32>) -> tensor<2x4x3xf32>
+      %o2 = stablehlo.dot_general %c3, %w, batching_dims = [0] x [0], contracting_dims = [2] x [1] : (tensor<2x4x3xf32>, tensor<2x3x5xf32>) -> tensor<2x4x5xf32>
+      %tr = stablehlo.transpose %o2, dims = [2, 0, 1] : (tensor<2x4x5xf32>) -> tensor<5x2x4xf32>
+      %sq = stablehlo.multiply %tr, %tr : tensor<5x2x4xf32>
+      %o3 = stablehlo.reduce(%sq init: %z) applies stablehlo.add across dimensions = [0, 1, 2] : (tensor<5x2x4xf32>, tensor<f32>) -> tensor<f32>
+      return %o1, %o2, %o3 : tensor<4x6xf32>, tensor<2x4x5xf32>, tensor<f32>
+    }"""
+    rng = np.random.Generator(np.random.PCG64(7))
+    a = dev(rng.uniform(0.5, 1.5, (4, 6)), "f32")[0]
+    b = dev(rng.standard_normal(6) * 0.3, "f32")[0]
+    w = dev(rng.standard_normal((2, 3, 5)), "f32")[0]
+    cts = (dev(rng.standard_normal((4, 6)), "f32")[0], dev(rng.standard_normal((2, 4, 5)), "f32")[0], dev(rng.standard_normal(()), "f32")[0].reshape(()))
+    outs, f_vjp = vjp(lambda *xs: tuple(hlo_call(*xs, source=text)), a, b, w)
+    tape = f_vjp(cts)
+    rev = stablehlo_ad.reverse_module_text(text)
+    sym = hlo_call(a, b, w, *cts, source=rev)
+    for name, g, t in zip("abw", sym, tape):
+        check(g, host(t), "f32", "symbolic vs tape, " + name, factor=0.1)

@@ -145,3 +145,85 @@ def test_optimize_module_prints_typed_ffi_custom_calls():
         ej.optimize_module(object())
     with pytest.raises(ValueError):
         ej.optimize_module(text, pipeline="a{b")
+
+
+def _ops_of(text, fn="main"):
+    from enzyme_ad.jax import stablehlo as S
+    return [(o.name, tuple(o.operands), {k: v for k, v in o.attrs.items() if k != "value"}) for o in S.parse_module(text)[fn].ops]
+
+
+def test_symbolic_reverse_mode_has_the_reference_ir_form():
+    """The reverse programs the reference's lit tests expect (their REVERSE check lines, minus
+    the additions of zero constants and identity transposes): dot_general.mlir:25-37 and
+    divide.mlir:21-27."""
+    from enzyme_ad.jax import stablehlo_ad as A
+
+    dot = """func.func @main(%a: tensor<2x3xf32>, %b: tensor<4x2xf32>) -> tensor<3x4xf32> {
+      %c = stablehlo.dot_general %a, %b, contracting_dims = [0] x [1] : (tensor<2x3xf32>, tensor<4x2xf32>) -> tensor<3x4xf32>
+      return %c : tensor<3x4xf32>
+    }"""
+    ops = _ops_of(A.reverse_module_text(dot))
+    assert [o[0] for o in ops] == ["dot_general", "transpose", "dot_general", "return"]
+    assert ops[0][1] == ("%ct0", "%b") and ops[0][2] == {"batch_a": [], "batch_b": [], "contract_a": [1], "contract_b": [0]}
+    assert ops[1][2] == {"perm": [1, 0]}
+    assert ops[2][1] == ("%ct0", "%a") and ops[2][2] == {"batch_a": [], "batch_b": [], "contract_a": [0], "contract_b": [1]}
+    div = """func.func @main(%a: tensor<2xf32>, %b: tensor<2xf32>) -> tensor<2xf32> {
+      %c = stablehlo.divide %a, %b : tensor<2xf32>
+      return %c : tensor<2xf32>
+    }"""
+    ops = _ops_of(A.reverse_module_text(div))
+    # %0 = ct / b; %1 = a / b; %2 = %0 * %1; %3 = -%2; return %0, %3
+    assert sorted(o[0] for o in ops) == ["divide", "divide", "multiply", "negate", "return"]
+    by = {o[0]: o for o in ops if o[0] in ("multiply", "negate", "return")}
+    q = [o for o in ops if o[0] == "divide" and o[1][0] == "%ct0"]
+    assert len(q) == 1 and q[0][1][1] == "%b" and by["multiply"][1][1] == "%c"
+    # activities: an inactive argument gets no result, an inactive result no cotangent argument
+    rev = A.reverse_module_text(div, arg_active=[False, True])
+    f = __import__("enzyme_ad.jax.stablehlo", fromlist=["x"]).parse_module(rev)["main"]
+    assert len(f.result_types) == 1 and [a for a, _ in f.args] == ["%a", "%b", "%ct0"]
+    with pytest.raises(NotImplementedError):
+        A.reverse_module_text("""func.func @main(%a: tensor<2xf32>, %b: tensor<2xf32>) -> tensor<2xf32> {
+          %c = stablehlo.maximum %a, %b : tensor<2xf32>
+          return %c : tensor<2xf32>
+        }""")
+
+
+def test_symbolic_reverse_of_the_llama_step_calls_the_adjoint_targets():
+    from enzyme_ad.jax import stablehlo as S, stablehlo_ad as A
+
+    text, order = llama_step_text(dict(CFG, n_layers=1), pos=3)
+    rev = A.reverse_module_text(text)
+    f = S.parse_module(rev)["main"]
+    targets = Counter(o.attrs["target"] for o in f.ops if o.name == "custom_call")
+    # forward values the adjoints need are recomputed (the final RMSNorm's output is not needed)
+    assert targets == {"emi_rope": 4, "emi_rmsnorm_bwd": 3, "emi_rmsnorm_fwd": 2, "emi_attn_step_fwd": 1, "emi_swiglu_fwd": 1,
+                       "emi_swiglu_bwd": 1, "emi_attn_step_bwd": 1}
+    assert sorted(o.attrs["config"]["inverse"] for o in f.ops if o.name == "custom_call" and o.attrs["target"] == "emi_rope") == \
+        [False, False, True, True]
+    assert len(f.args) == len(order) + 1 and f.args[-1][1].shape == (288,)
+    assert [t.shape for t in f.result_types] == [t.shape for _, t in f.args[:-1]]
+    assert S.print_module(S.parse_module(rev)) == rev
+    bwd = [o for o in f.ops if o.name == "custom_call" and o.attrs["target"] == "emi_attn_step_bwd"][0]
+    fwd = [o for o in f.ops if o.name == "custom_call" and o.attrs["target"] == "emi_attn_step_fwd"][0]
+    assert bwd.operands[3:5] == fwd.results[:2]                                  # o and lse of the forward call
+
+
+def test_optimize_module_differentiates_when_the_pipeline_says_so():
+    """The pipeline strings enzyme_jvp / enzyme_vjp build select the program optimize_module
+    returns: lowering only, or the reverse-mode program with the listed activities."""
+    import enzyme_ad.jax as ej
+    from enzyme_ad.jax import primitives as P, stablehlo as S
+
+    text = """func.func @main(%a: tensor<2xf32>, %b: tensor<2xf32>) -> tensor<2xf32> {
+      %c = stablehlo.divide %a, %b : tensor<2xf32>
+      return %c : tensor<2xf32>
+    }"""
+    fwd = P.forward_mode_pipeline(P.JaXPipeline(), [False, True], 1)
+    rev = P.reverse_mode_pipeline(fwd, [True])
+    out = S.parse_module(ej.optimize_module(text, rev.pass_pipeline()))["main"]
+    assert [a for a, _ in out.args] == ["%a", "%b", "%ct0"] and len(out.result_types) == 1      # a is enzyme_const
+    assert sorted(o.name for o in out.ops) == ["divide", "divide", "multiply", "negate", "return"]
+    plain = S.parse_module(ej.optimize_module(text))["main"]
+    assert [o.name for o in plain.ops] == ["divide", "return"]
+    with pytest.raises(NotImplementedError, match="ForwardMode"):
+        ej.optimize_module(text, fwd.pass_pipeline())
