@@ -433,7 +433,9 @@ def optimize_module(mod, pipeline=None):
     other operators printed back unchanged.  When the pipeline's last `enzyme-wrap` pass asks
     for `mode=ReverseModeCombined` (the string `enzyme_vjp` builds, :1385-1419) the result is
     the reverse-mode program instead: main(args..., cotangents of the active results) ->
-    cotangents of the active arguments, with the clusters' adjoints as custom calls.  An XLA
+    cotangents of the active arguments, with the clusters' adjoints as custom calls; for
+    `mode=ForwardMode` (`enzyme_jvp`, :1176-1203) it is main(arg, tangent of arg, ...) ->
+    (result, tangent of result, ...) with the clusters' tangent targets.  An XLA
     client with this library's FFI handlers registered can compile either; `hlo_call` runs
     them as well.  The other passes of the pipeline are parsed for validity only."""
     from . import stablehlo, stablehlo_ad
@@ -446,11 +448,14 @@ def optimize_module(mod, pipeline=None):
         return stablehlo.lower_to_custom_calls(mod)[0]
     wrap = "enzyme-wrap{" + wraps[-1] + " }"
     mode = re.search(r"mode=(\w+)", wrap)
-    if mode is None or mode.group(1) != "ReverseModeCombined":
-        raise NotImplementedError("optimize_module differentiates symbolically in mode=ReverseModeCombined only "
-                                  "(forward mode runs on the tape: jvp); got %s" % (mode.group(1) if mode else "no mode"))
     fn = re.search(r"infn=(\w+)", wrap)
     active = lambda acts: [a != "enzyme_const" for a in acts]
+    if mode is not None and mode.group(1) == "ForwardMode":
+        return stablehlo_ad.forward_module_text(mod, fn.group(1) if fn else "main",
+                                                arg_active=active(arg_activity_from_pipeline(wrap)[1]))
+    if mode is None or mode.group(1) != "ReverseModeCombined":
+        raise NotImplementedError("optimize_module differentiates in mode=ForwardMode or mode=ReverseModeCombined; got %s" %
+                                  (mode.group(1) if mode else "no mode"))
     return stablehlo_ad.reverse_module_text(mod, fn.group(1) if fn else "main",
                                             arg_active=active(arg_activity_from_pipeline(wrap)[1]),
                                             ret_active=active(ret_activity_from_pipeline(wrap)[1]))

@@ -1053,6 +1053,28 @@ def _custom_call_impl(self, op, xs):
     # not themselves differentiable
     lib, st = N.lib(), ops._stream()
     P = lambda t: None if t is None else t.data_ptr()
+    if target == "emi_rmsnorm_jvp":
+        x, w, tx, tw = (_packed(t) for t in xs)
+        ty = torch.empty_like(x)
+        N.check(lib.emi_rmsnorm_jvp(st, P(x), P(w), P(tx), P(tw), P(ty), x.numel() // x.shape[-1], x.shape[-1],
+                                    float(cfg.get("eps", 1e-5)), ops._code(x)))
+        return [ty]
+    if target == "emi_swiglu_jvp":
+        a, b_, ta, tb = (_packed(t) for t in xs)
+        tg = torch.empty_like(a)
+        N.check(lib.emi_swiglu_jvp(st, P(a), P(b_), P(ta), P(tb), P(tg), a.numel(), ops._code(a)))
+        return [tg]
+    if target == "emi_attn_step_jvp":
+        q, k, v, o, lse, tq, tk, tv = (_packed(t) for t in xs)
+        if q.dim() != 3 or q.shape[0] != 1 or k.dim() != 4:
+            raise NotImplementedError("custom call emi_attn_step_jvp is run for one sequence per call (batch = 1)")
+        h, d, S = q.shape[1], q.shape[2], k.shape[1]
+        to = torch.empty_like(q)
+        nbytes = lib.emi_attn_step_workspace_bytes(1, h, S, d)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
+        N.check(lib.emi_attn_step_jvp(st, P(q), P(k), P(v), P(o), P(lse), P(tq), P(tk), P(tv), P(to), P(ws), nbytes, 1, h, S, d,
+                                      h * d, d, S * h * d, d, h * d, float(cfg["scale"]), ops._code(q)))
+        return [to, None][:len(op.results)]
     if target == "emi_rmsnorm_bwd":
         x, w, dy = (_packed(t) for t in xs[:3])
         rows, dim = x.numel() // x.shape[-1], x.shape[-1]

@@ -295,6 +295,130 @@ def reverse_function(func, name=None, arg_active=None, ret_active=None):
     return rev
 
 
+def forward_function(func, name=None, arg_active=None):
+    """f_fwd(arg0[, tangent of arg0], arg1[, ...]) -> (result0, tangent of result0, ...): the
+    program of the reference's `enzyme-wrap{... mode=ForwardMode}` pass with `enzyme_dup`
+    arguments (each followed by its tangent), `enzyme_const` arguments (no tangent) and
+    `enzyme_dup` results (primitives.py:1160-1203).  Every operator is followed by the
+    operators of its tangent; matched clusters call the tangent targets (`emi_rmsnorm_jvp`,
+    `emi_swiglu_jvp`, `emi_attn_step_jvp`, `emi_rope` on the tangent)."""
+    func = lower_fused(func)
+    b = _Builder(func, "f")
+    T = b.types
+    if arg_active is None:
+        arg_active = [t.dtype in FLOAT for _, t in func.args]
+    if len(arg_active) != len(func.args):
+        raise ValueError("activity list does not match the function: %d arguments" % len(func.args))
+    args, tan = [], {}
+    for (a, t), active in zip(func.args, arg_active):
+        args.append((a, t))
+        if active:
+            if t.dtype not in FLOAT:
+                raise ValueError("argument %s of type %r cannot be active" % (a, t))
+            ta = "%%t_%s" % a[1:]
+            T[ta] = t
+            args.append((ta, t))
+            tan[a] = ta
+
+    def zero(ty):
+        return b.const(0.0, ty)
+
+    def tz(v):
+        return tan[v] if v in tan else zero(T[v])
+
+    def add(x, y):
+        return y if x is None else x if y is None else b.binary("add", x, y)
+
+    outs = None
+    for op in func.ops:
+        n, xs = op.name, op.operands
+        if n == "return":
+            outs = []
+            for o in xs:
+                outs += [o, tz(o)]
+            continue
+        b.ops.append(op)
+        ts = [tan.get(x) for x in xs]
+        if all(t is None for t in ts) or not op.results:
+            continue
+        r = op.results[0]
+        t = ts[0]
+        if n == "add":
+            tan[r] = add(ts[0], ts[1])
+        elif n == "subtract":
+            tan[r] = ts[0] if ts[1] is None else b.unary("negate", ts[1]) if ts[0] is None else b.binary("subtract", ts[0], ts[1])
+        elif n == "multiply":
+            tan[r] = add(None if ts[0] is None else b.binary("multiply", ts[0], xs[1]),
+                         None if ts[1] is None else b.binary("multiply", ts[1], xs[0]))
+        elif n == "divide":
+            # (ta b - tb a) / b^2, the form of the reference's FORWARD lines (divide.mlir:9-17)
+            num = None if ts[0] is None else b.binary("multiply", ts[0], xs[1])
+            if ts[1] is not None:
+                sub = b.binary("multiply", ts[1], xs[0])
+                num = b.unary("negate", sub) if num is None else b.binary("subtract", num, sub)
+            tan[r] = b.binary("divide", num, b.binary("multiply", xs[1], xs[1]))
+        elif n == "negate":
+            tan[r] = b.unary("negate", t)
+        elif n == "exponential":
+            tan[r] = b.binary("multiply", t, r)
+        elif n == "log":
+            tan[r] = b.binary("divide", t, xs[0])
+        elif n == "sqrt":
+            tan[r] = b.binary("divide", t, b.binary("multiply", b.const(2.0, T[r]), r))
+        elif n == "rsqrt":
+            tan[r] = b.binary("multiply", b.binary("multiply", b.const(-0.5, T[r]), t), b.binary("multiply", b.binary("multiply", r, r), r))
+        elif n == "logistic":
+            tan[r] = b.binary("multiply", b.binary("multiply", t, r), b.binary("subtract", b.const(1.0, T[r]), r))
+        elif n == "tanh":
+            tan[r] = b.binary("multiply", t, b.binary("subtract", b.const(1.0, T[r]), b.binary("multiply", r, r)))
+        elif n == "sine":
+            tan[r] = b.binary("multiply", t, b.unary("cosine", xs[0]))
+        elif n == "cosine":
+            tan[r] = b.unary("negate", b.binary("multiply", t, b.unary("sine", xs[0])))
+        elif n in ("convert", "reshape", "transpose", "broadcast_in_dim", "slice"):
+            tan[r] = b.emit(n, [t], op.attrs, T[r])
+        elif n == "reduce":
+            if op.attrs["body"] != "add":
+                raise NotImplementedError("symbolic forward mode of reduce with a %s body" % op.attrs["body"])
+            if t is not None:
+                tan[r] = b.emit("reduce", [t, zero(TensorType((), T[r].dtype))], op.attrs, T[r])
+        elif n == "pad":
+            if t is not None:
+                tan[r] = b.emit("pad", [t, zero(TensorType((), T[r].dtype))], op.attrs, T[r])
+        elif n == "concatenate":
+            tan[r] = b.emit("concatenate", [tz(x) for x in xs], op.attrs, T[r])
+        elif n == "dot_general":
+            tan[r] = add(None if ts[0] is None else b.emit("dot_general", [ts[0], xs[1]], op.attrs, T[r]),
+                         None if ts[1] is None else b.emit("dot_general", [xs[0], ts[1]], op.attrs, T[r]))
+        elif n == "custom_call":
+            target, cfg = op.attrs["target"], op.attrs["config"]
+            if target == "emi_rmsnorm_fwd":
+                tan[r], = b.custom_call("emi_rmsnorm_jvp", [xs[0], xs[1], tz(xs[0]), tz(xs[1])], {"eps": cfg.get("eps", 1e-5)}, [T[r]])
+            elif target == "emi_swiglu_fwd":
+                tan[r], = b.custom_call("emi_swiglu_jvp", [xs[0], xs[1], tz(xs[0]), tz(xs[1])], {}, [T[r]])
+            elif target == "emi_add":
+                tan[r] = add(ts[0], ts[1])
+            elif target == "emi_rope":
+                if ts[0] is not None:
+                    tan[r], = b.custom_call("emi_rope", [ts[0], xs[1]], dict(cfg), [T[r]])
+            elif target == "emi_attn_step_fwd":
+                o, lse, ws = op.results
+                tan[o], _ = b.custom_call("emi_attn_step_jvp", [xs[0], xs[1], xs[2], o, lse, tz(xs[0]), tz(xs[1]), tz(xs[2])],
+                                          {"scale": cfg["scale"]}, [T[o], T[ws]])
+            else:
+                raise NotImplementedError("symbolic forward mode of custom call '%s'" % target)
+        elif n == "call":
+            raise NotImplementedError("symbolic forward mode needs a call-free function (inline_calls)")
+        else:
+            raise NotImplementedError("symbolic forward mode of stablehlo.%s" % n)
+    if outs is None:
+        raise ValueError("forward mode needs a return")
+    b.ops.append(Op("return", [], outs, {}, []))
+    fwd = Func(name or func.name + "_fwd", args, [T[o] for o in outs], b.ops)
+    _drop_dead(fwd)
+    return fwd
+
+
 def _reverse_dot_general(b, op, c, accum):
     T = b.types
     a_, b_ = op.operands
@@ -392,3 +516,13 @@ def reverse_module_text(text, fn="main", arg_active=None, ret_active=None):
     fuse_clusters(f)
     rev = reverse_function(f, name="main", arg_active=arg_active, ret_active=ret_active)
     return print_module({"main": rev})
+
+
+def forward_module_text(text, fn="main", arg_active=None):
+    """StableHLO text in, StableHLO text of the forward-mode program out (see `forward_function`)."""
+    from .stablehlo import fold_constants, fuse_clusters, parse_module, print_module
+
+    f = inline_calls(parse_module(text), fn)
+    fold_constants(f)
+    fuse_clusters(f)
+    return print_module({"main": forward_function(f, name="main", arg_active=arg_active)})

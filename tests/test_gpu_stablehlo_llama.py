@@ -172,3 +172,27 @@ def test_reverse_module_of_generic_operators_matches_the_tape():
     sym = hlo_call(a, b, w, *cts, source=rev)
     for name, g, t in zip("abw", sym, tape):
         check(g, host(t), "f32", "symbolic vs tape, " + name, factor=0.1)
+
+
+def test_forward_module_of_the_llama_step():
+    """The symbolic forward-mode module (each argument followed by its tangent; results
+    interleaved with their tangents) through hlo_call against the tape's jvp of the same text,
+    with every argument active and with only the weights active."""
+    from enzyme_ad.jax import hlo_call, jvp, stablehlo_ad
+
+    cfg = dict(STORIES, n_layers=2)
+    text, order = llama_step_text(cfg, 6, "f32")
+    (x, wd, kc, vc, dy), _ = _inputs(cfg, 6, "f32", 71, False, 0.05)
+    args = [x] + [wd[k] for k in WEIGHT_ORDER] + [kc, vc]
+    rng = np.random.Generator(np.random.PCG64(8))
+    tans = [dev(rng.standard_normal(tuple(a.shape)) * (0.05 if a.dim() > 1 else 1.0), "f32")[0] for a in args]
+    fn = lambda *a: hlo_call(*a, source=text)[0]
+    for active in ([True] * len(args), [False] + [True] * (len(args) - 3) + [False, False]):
+        fwd = stablehlo_ad.forward_module_text(text, arg_active=active)
+        flat = []
+        for a, t, on in zip(args, tans, active):
+            flat += [a, t] if on else [a]
+        y, ty = hlo_call(*flat, source=fwd)
+        y_ref, ty_ref = jvp(fn, tuple(args), tuple(t if on else None for t, on in zip(tans, active)))
+        check(y, host(y_ref), "f32", "forward module, primal", factor=0.1)
+        check(ty, host(ty_ref), "f32", "forward module, tangent", factor=0.1)

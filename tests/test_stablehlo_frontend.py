@@ -225,5 +225,12 @@ def test_optimize_module_differentiates_when_the_pipeline_says_so():
     assert sorted(o.name for o in out.ops) == ["divide", "divide", "multiply", "negate", "return"]
     plain = S.parse_module(ej.optimize_module(text))["main"]
     assert [o.name for o in plain.ops] == ["divide", "return"]
-    with pytest.raises(NotImplementedError, match="ForwardMode"):
-        ej.optimize_module(text, fwd.pass_pipeline())
+    # forward mode: (ta b - tb a) / b^2 with a inactive -> -(tb a) / (b b), primal last (divide.mlir:9-17)
+    f = S.parse_module(ej.optimize_module(text, fwd.pass_pipeline()))["main"]
+    assert [a for a, _ in f.args] == ["%a", "%b", "%t_b"] and len(f.result_types) == 2
+    assert sorted(o.name for o in f.ops) == ["divide", "divide", "multiply", "multiply", "negate", "return"]
+    both = S.parse_module(ej.optimize_module(text, P.forward_mode_pipeline(P.JaXPipeline(), [True, True], 1).pass_pipeline()))["main"]
+    assert [a for a, _ in both.args] == ["%a", "%t_a", "%b", "%t_b"]
+    assert sorted(o.name for o in both.ops) == ["divide", "divide", "multiply", "multiply", "multiply", "return", "subtract"]
+    with pytest.raises(NotImplementedError, match="ForwardModeSplit"):
+        ej.optimize_module(text, fwd.pass_pipeline().replace("mode=ForwardMode", "mode=ForwardModeSplit"))
