@@ -137,6 +137,74 @@ __global__ void __launch_bounds__(kBlock) convert_kernel(const TI* __restrict__ 
   }
 }
 
+// compare: mask[i] = dir(a[i * sa], b[i * sb]) as one byte (0 / 1); select: y[i] = mask ? a : b.
+__device__ __forceinline__ bool cmp(int dir, float a, float b) {
+  switch (dir) {
+    case EMI_CMP_EQ: return a == b;
+    case EMI_CMP_NE: return a != b;
+    case EMI_CMP_GE: return a >= b;
+    case EMI_CMP_GT: return a > b;
+    case EMI_CMP_LE: return a <= b;
+    default: return a < b;
+  }
+}
+
+template <typename T, bool VEC>
+__global__ void __launch_bounds__(kBlock) compare_kernel(int dir, const T* __restrict__ a, const T* __restrict__ b,
+                                                         uint8_t* __restrict__ mask, int64_t n, int sa, int sb) {
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (VEC) {
+    const int64_t ngroups = n >> 3;
+    if (i < ngroups) {
+      float fa[8], fb[8];
+      if (sa) Vec8<T>::load(a + i * 8, fa);
+      if (sb) Vec8<T>::load(b + i * 8, fb);
+      const float va = sa ? 0.f : to_f32(a[0]), vb = sb ? 0.f : to_f32(b[0]);
+      uint32_t lo = 0, hi = 0;
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        lo |= (uint32_t)cmp(dir, sa ? fa[j] : va, sb ? fb[j] : vb) << (8 * j);
+        hi |= (uint32_t)cmp(dir, sa ? fa[j + 4] : va, sb ? fb[j + 4] : vb) << (8 * j);
+      }
+      *reinterpret_cast<uint2*>(mask + i * 8) = make_uint2(lo, hi);
+    } else if (i - ngroups < (n & 7)) {
+      const int64_t e = (ngroups << 3) + (i - ngroups);
+      mask[e] = cmp(dir, to_f32(a[sa ? e : 0]), to_f32(b[sb ? e : 0]));
+    }
+  } else if (i < n) {
+    mask[i] = cmp(dir, to_f32(a[sa ? i : 0]), to_f32(b[sb ? i : 0]));
+  }
+}
+
+template <typename T, bool VEC>
+__global__ void __launch_bounds__(kBlock) select_kernel(const uint8_t* __restrict__ mask, const T* __restrict__ a,
+                                                        const T* __restrict__ b, T* __restrict__ y, int64_t n, int sm, int sa,
+                                                        int sb) {
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (VEC) {
+    const int64_t ngroups = n >> 3;
+    if (i < ngroups) {
+      float fa[8], fb[8];
+      if (sa) Vec8<T>::load(a + i * 8, fa);
+      if (sb) Vec8<T>::load(b + i * 8, fb);
+      const float va = sa ? 0.f : to_f32(a[0]), vb = sb ? 0.f : to_f32(b[0]);
+      uint2 m = sm ? *reinterpret_cast<const uint2*>(mask + i * 8) : make_uint2(mask[0] ? 0x01010101u : 0u, mask[0] ? 0x01010101u : 0u);
+      float out[8];
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        out[j] = ((m.x >> (8 * j)) & 0xff) ? (sa ? fa[j] : va) : (sb ? fb[j] : vb);
+        out[j + 4] = ((m.y >> (8 * j)) & 0xff) ? (sa ? fa[j + 4] : va) : (sb ? fb[j + 4] : vb);
+      }
+      Vec8<T>::store(y + i * 8, out);
+    } else if (i - ngroups < (n & 7)) {
+      const int64_t e = (ngroups << 3) + (i - ngroups);
+      y[e] = mask[sm ? e : 0] ? a[sa ? e : 0] : b[sb ? e : 0];
+    }
+  } else if (i < n) {
+    y[i] = mask[sm ? i : 0] ? a[sa ? i : 0] : b[sb ? i : 0];
+  }
+}
+
 // ---------------------------------------------------------------------------
 // strided copy: out[o0 + sum_d i_d * os_d] = in[i0 + sum_d i_d * is_d] over the index box
 // dims[0..rank).  Covers transpose (permuted strides), broadcast_in_dim (zero strides),
@@ -738,4 +806,49 @@ extern "C" int emi_reduce(emi_stream_t stream, int op, const void* x, void* y, v
     return op == EMI_OP_ADD ? launch_reduce<bf16, EMI_OP_ADD>(st, x, y, workspace, workspace_bytes, outer, red, inner)
                             : launch_reduce<bf16, EMI_OP_MAX>(st, x, y, workspace, workspace_bytes, outer, red, inner);
   return emi_fail(EMI_INVALID_ARGUMENT, "emi_reduce: unsupported dtype code %d", dtype);
+}
+
+extern "C" int emi_compare(emi_stream_t stream, int direction, const void* a, const void* b, void* mask, int64_t n,
+                           int a_is_scalar, int b_is_scalar, int dtype) {
+  EMI_REQUIRE(direction >= EMI_CMP_EQ && direction <= EMI_CMP_LT, "emi_compare: unknown direction code %d", direction);
+  EMI_REQUIRE(n >= 0 && n < (int64_t)1 << 39, "emi_compare: size out of range");
+  if (n == 0) return EMI_OK;
+  EMI_REQUIRE(a && b && mask, "emi_compare: null buffer");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int sa = a_is_scalar ? 0 : 1, sb = b_is_scalar ? 0 : 1;
+  const bool vec = al16(a) && al16(b) && (reinterpret_cast<uintptr_t>(mask) & 7) == 0;
+  const unsigned grid = map_grid(n, vec);
+#define EMI_CMP_LAUNCH(T)                                                                                             \
+  do {                                                                                                                 \
+    if (vec) hipLaunchKernelGGL((compare_kernel<T, true>), dim3(grid), dim3(kBlock), 0, st, direction, (const T*)a, (const T*)b, (uint8_t*)mask, n, sa, sb); \
+    else hipLaunchKernelGGL((compare_kernel<T, false>), dim3(grid), dim3(kBlock), 0, st, direction, (const T*)a, (const T*)b, (uint8_t*)mask, n, sa, sb);    \
+  } while (0)
+  if (dtype == EMI_F32) EMI_CMP_LAUNCH(float);
+  else if (dtype == EMI_BF16) EMI_CMP_LAUNCH(bf16);
+  else return emi_fail(EMI_INVALID_ARGUMENT, "emi_compare: unsupported dtype code %d", dtype);
+#undef EMI_CMP_LAUNCH
+  EMI_CHECK_LAUNCH("emi_compare");
+  return EMI_OK;
+}
+
+extern "C" int emi_select(emi_stream_t stream, const void* mask, const void* a, const void* b, void* y, int64_t n,
+                          int mask_is_scalar, int a_is_scalar, int b_is_scalar, int dtype) {
+  EMI_REQUIRE(n >= 0 && n < (int64_t)1 << 39, "emi_select: size out of range");
+  if (n == 0) return EMI_OK;
+  EMI_REQUIRE(mask && a && b && y, "emi_select: null buffer");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int sm = mask_is_scalar ? 0 : 1, sa = a_is_scalar ? 0 : 1, sb = b_is_scalar ? 0 : 1;
+  const bool vec = al16(a) && al16(b) && al16(y) && (reinterpret_cast<uintptr_t>(mask) & 7) == 0;
+  const unsigned grid = map_grid(n, vec);
+#define EMI_SEL_LAUNCH(T)                                                                                             \
+  do {                                                                                                                 \
+    if (vec) hipLaunchKernelGGL((select_kernel<T, true>), dim3(grid), dim3(kBlock), 0, st, (const uint8_t*)mask, (const T*)a, (const T*)b, (T*)y, n, sm, sa, sb); \
+    else hipLaunchKernelGGL((select_kernel<T, false>), dim3(grid), dim3(kBlock), 0, st, (const uint8_t*)mask, (const T*)a, (const T*)b, (T*)y, n, sm, sa, sb);    \
+  } while (0)
+  if (dtype == EMI_F32) EMI_SEL_LAUNCH(float);
+  else if (dtype == EMI_BF16) EMI_SEL_LAUNCH(bf16);
+  else return emi_fail(EMI_INVALID_ARGUMENT, "emi_select: unsupported dtype code %d", dtype);
+#undef EMI_SEL_LAUNCH
+  EMI_CHECK_LAUNCH("emi_select");
+  return EMI_OK;
 }

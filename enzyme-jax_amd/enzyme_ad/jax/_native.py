@@ -31,6 +31,8 @@ SIGNATURES = {
     "emi_transpose": (c_int, [c_void_p, c_void_p, c_void_p, c_i64, c_i64, c_int]),
     "emi_map_binary": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_i64, c_int, c_int, c_int]),
     "emi_map_unary": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_i64, c_int]),
+    "emi_compare": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_i64, c_int, c_int, c_int]),
+    "emi_select": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_int, c_int, c_int, c_int]),
     "emi_convert": (c_int, [c_void_p, c_void_p, c_void_p, c_i64, c_int, c_int]),
     "emi_strided_copy": (c_int, [c_void_p, c_void_p, c_void_p, c_int, ctypes.POINTER(c_i64), ctypes.POINTER(c_i64),
                                  c_i64, ctypes.POINTER(c_i64), c_i64, c_int]),

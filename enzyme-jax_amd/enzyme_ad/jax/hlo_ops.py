@@ -103,6 +103,43 @@ def _convert(x, dtype):
     return y
 
 
+COMPARE = {"EQ": 0, "NE": 1, "GE": 2, "GT": 3, "LE": 4, "LT": 5}
+
+
+def _compare(direction, a, b):
+    """i1 tensor (torch.bool, one byte per element) of direction(a, b); rank-0 operands broadcast."""
+    _need_cuda(a, b)
+    if a.dtype != b.dtype:
+        raise TypeError("compare: mixed dtypes %s and %s" % (a.dtype, b.dtype))
+    a, b = _contig(a), _contig(b)
+    sa = a.dim() == 0 and b.dim() > 0
+    sb = b.dim() == 0 and a.dim() > 0
+    if not (sa or sb) and a.shape != b.shape:
+        raise ValueError("compare: shapes %s and %s" % (tuple(a.shape), tuple(b.shape)))
+    m = torch.empty(b.shape if sa else a.shape, dtype=torch.bool, device=a.device)
+    N.check(N.lib().emi_compare(_stream(), COMPARE[direction], _p(a), _p(b), _p(m), m.numel(), int(sa), int(sb), _code(a)))
+    return m
+
+
+def _select(m, a, b):
+    _need_cuda(m, a, b)
+    if m.dtype != torch.bool or a.dtype != b.dtype:
+        raise TypeError("select: predicate %s, values %s and %s" % (m.dtype, a.dtype, b.dtype))
+    m, a, b = _contig(m), _contig(a), _contig(b)
+    shape = max((tuple(t.shape) for t in (m, a, b)), key=len)
+    flags = []
+    for t in (m, a, b):
+        if tuple(t.shape) == shape:
+            flags.append(0)
+        elif t.dim() == 0:
+            flags.append(1)
+        else:
+            raise ValueError("select: shapes %s, %s, %s" % (tuple(m.shape), tuple(a.shape), tuple(b.shape)))
+    y = torch.empty(shape, dtype=a.dtype, device=a.device)
+    N.check(N.lib().emi_select(_stream(), _p(m), _p(a), _p(b), _p(y), y.numel(), flags[0], flags[1], flags[2], _code(a)))
+    return y
+
+
 def _permute(x, perm):
     out = torch.empty([x.shape[p] for p in perm], dtype=x.dtype, device=x.device)
     _copy_box(x, list(out.shape), [x.stride(p) for p in perm], 0, out, _contiguous_strides(out.shape), 0)
@@ -552,4 +589,32 @@ def pad(x, low, high, interior, shape):
     tans = _tan(x)
     if tans is not None and tans[0] is not None:
         _set_tan(y, _quiet(lambda: _scatter_box(tans[0], list(shape), low, stride)))
+    return y
+
+
+def compare(direction, a, b):
+    """stablehlo.compare: no derivative (the result is an i1 tensor)."""
+    return _compare(direction, a, b)
+
+
+def select(m, a, b):
+    """stablehlo.select (Select rule HLODerivatives.td:1297): the cotangent goes to the chosen
+    side, zero to the other."""
+    y = _select(m, a, b)
+    zero = lambda like: torch.zeros((), dtype=like.dtype, device=like.device)
+
+    def rule(c, acc):
+        ga = _select(m, c, zero(c))
+        gb = _select(m, zero(c), c)
+        return None, _accumulate(acc[1], _fit(ga, a)), _accumulate(acc[2], _fit(gb, b))
+
+    Tape.record((m, a, b), y, rule)
+    tans = _tan(a, b)
+    if tans is not None and (tans[0] is not None or tans[1] is not None):
+        ta = zero(y) if tans[0] is None else tans[0]
+        tb = zero(y) if tans[1] is None else tans[1]
+        t = _quiet(lambda: _select(m, ta, tb))
+        if t.shape != y.shape:
+            t = _broadcast(t, list(y.shape), [])
+        _set_tan(y, t)
     return y

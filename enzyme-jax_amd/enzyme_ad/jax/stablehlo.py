@@ -12,7 +12,8 @@ function that calls `hlo_call` differentiate through the parsed graph.
 The accepted text is MLIR's printed form of the operators JAX emits for such functions
 (pretty or quoted-generic operator names): constant, add, subtract, multiply, divide, maximum,
 minimum, power, negate, exponential, log, sqrt, rsqrt, logistic, tanh, sine, cosine, convert, reshape,
-transpose, broadcast_in_dim, reduce (add / maximum), dot_general, slice, pad, concatenate, call,
+transpose, broadcast_in_dim, reduce (add / maximum), dot_general, slice, pad, concatenate, compare,
+select, call,
 custom_call (this library's targets), return.  Anything else raises `NotImplementedError` naming the operator.
 """
 import math
@@ -414,6 +415,20 @@ def _parse_op(sc):
         text = sc.balanced() if sc.peek("{") else "{}"
         _, types = sc.signature()
         return Op("custom_call", results, operands, {"target": target, "config": _backend_config(text)}, types)
+    if short == "compare":
+        direction = sc.need(_IDENT, "comparison direction")
+        sc.expect(",")
+        operands = operand_list()
+        if sc.accept(","):
+            sc.need(_IDENT, "comparison type")               # FLOAT / TOTALORDER / SIGNED: floats compare as IEEE here
+        _, types = sc.signature()
+        if direction not in H.COMPARE:
+            sc.fail("unknown comparison direction '%s'" % direction)
+        return Op("compare", results, operands, {"direction": direction}, types[-1:])
+    if short == "select":
+        operands = operand_list()
+        _, types = sc.signature()
+        return Op("select", results, operands, {}, types[-1:])
     if short == "call":
         callee = sc.need(_SYM, "callee")
         sc.expect("(")
@@ -991,6 +1006,10 @@ class Executable:
             return [H.slice_(xs[0], op.attrs["start"], op.attrs["limit"], op.attrs["stride"])]
         if n == "concatenate":
             return [H.concatenate(xs, op.attrs["dim"])]
+        if n == "compare":
+            return [H.compare(op.attrs["direction"], xs[0], xs[1])]
+        if n == "select":
+            return [H.select(xs[0], xs[1], xs[2])]
         if n == "pad":
             if _splat(f.defs.get(op.operands[1])) != 0.0:
                 raise NotImplementedError("stablehlo.pad with a padding value other than a zero constant")
@@ -1226,6 +1245,12 @@ class _Printer:
                                                          ", ".join(repr(T[o]) for o in op.operands), outs))
         elif n == "custom_call":
             self.custom_call(op.results, op.attrs["target"], op.operands, op.attrs["config"], op.types)
+        elif n == "compare":
+            self.emit("%s = stablehlo.compare %s, %s, %s, FLOAT : (%r, %r) -> %r" % (r, op.attrs["direction"], op.operands[0],
+                                                                                 op.operands[1], T[op.operands[0]], T[op.operands[1]], ty))
+        elif n == "select":
+            self.emit("%s = stablehlo.select %s, %s, %s : (%s) -> %r" % (r, op.operands[0], op.operands[1], op.operands[2],
+                                                                        ", ".join(repr(T[o]) for o in op.operands), ty))
         elif n == "pad":
             a = op.attrs
             self.emit("%s = stablehlo.pad %s, %s, low = %s, high = %s, interior = %s : (%r, %r) -> %r" % (

@@ -65,6 +65,9 @@ class _Builder:
     def binary(self, name, a, b):
         return self.emit(name, [a, b], {}, self.types[a])
 
+    def compare(self, direction, a, b):
+        return self.emit("compare", [a, b], {"direction": direction}, TensorType(self.types[a].shape, "i1"))
+
     def unary(self, name, a):
         return self.emit(name, [a], {}, self.types[a])
 
@@ -210,9 +213,26 @@ def reverse_function(func, name=None, arg_active=None, ret_active=None):
         elif n == "log":
             accum(xs[0], b.binary("divide", c, xs[0]))
         elif n == "sqrt":
-            # c / (2 sqrt(x)); the reference also selects 0 where x == 0 (Sqrt rule :1320), which
-            # needs compare / select and is not reproduced here
-            accum(xs[0], b.binary("divide", c, b.binary("multiply", splat_like(r, 2.0), r)))
+            # select(x == 0, 0, c / (2 sqrt(x)))  (Sqrt rule :1320 with its zero guard)
+            g = b.binary("divide", c, b.binary("multiply", splat_like(r, 2.0), r))
+            accum(xs[0], b.emit("select", [b.compare("EQ", xs[0], splat_like(r, 0.0)), splat_like(r, 0.0), g], {}, T[r]))
+        elif n in ("maximum", "minimum"):
+            # ties go to the first operand (Max rule :1205, maximum.mlir:25-34)
+            m = b.compare("GE" if n == "maximum" else "LE", xs[0], xs[1])
+            z = splat_like(r, 0.0)
+            accum(xs[0], b.emit("select", [m, c, z], {}, T[r]))
+            accum(xs[1], b.emit("select", [m, z, c], {}, T[r]))
+        elif n == "power":
+            # c y x^(y-1) and c x^y log x (Pow rule :1237-1242)
+            ym1 = b.binary("subtract", xs[1], splat_like(r, 1.0))
+            accum(xs[0], b.binary("multiply", c, b.binary("multiply", xs[1], b.binary("power", xs[0], ym1))))
+            accum(xs[1], b.binary("multiply", c, b.binary("multiply", r, b.unary("log", xs[0]))))
+        elif n == "compare":
+            continue
+        elif n == "select":
+            z = splat_like(r, 0.0)
+            accum(xs[1], b.emit("select", [xs[0], c, z], {}, T[r]))
+            accum(xs[2], b.emit("select", [xs[0], z, c], {}, T[r]))
         elif n == "rsqrt":
             cube = b.binary("multiply", b.binary("multiply", r, r), r)
             accum(xs[0], b.binary("multiply", b.binary("multiply", splat_like(r, -0.5), c), cube))
@@ -247,11 +267,18 @@ def reverse_function(func, name=None, arg_active=None, ret_active=None):
                     g = b.emit("transpose", [g], {"perm": perm}, TensorType([kept[p] for p in perm], ot.dtype))
             accum(xs[0], b.reshape(g, xt.shape))
         elif n == "reduce":
-            if op.attrs["body"] != "add":
-                raise NotImplementedError("symbolic reverse mode of reduce with a %s body" % op.attrs["body"])
             xt = T[xs[0]]
             kept = [d for d in range(len(xt.shape)) if d not in op.attrs["dims"]]
-            accum(xs[0], b.emit("broadcast_in_dim", [c], {"dims": kept}, xt))
+            back = b.emit("broadcast_in_dim", [c], {"dims": kept}, xt)
+            if op.attrs["body"] == "add":
+                accum(xs[0], back)
+            elif op.attrs["body"] == "maximum":
+                # every element equal to the maximum gets the cotangent, undivided
+                # (StableHLOAutoDiffOpInterfaceImpl.cpp:1881-1916)
+                m = b.compare("EQ", xs[0], b.emit("broadcast_in_dim", [r], {"dims": kept}, xt))
+                accum(xs[0], b.emit("select", [m, back, b.const(0.0, xt)], {}, xt))
+            else:
+                raise NotImplementedError("symbolic reverse mode of reduce with a %s body" % op.attrs["body"])
         elif n == "dot_general":
             _reverse_dot_general(b, op, c, accum)
         elif n == "slice":
@@ -364,7 +391,20 @@ def forward_function(func, name=None, arg_active=None):
         elif n == "log":
             tan[r] = b.binary("divide", t, xs[0])
         elif n == "sqrt":
-            tan[r] = b.binary("divide", t, b.binary("multiply", b.const(2.0, T[r]), r))
+            g = b.binary("divide", t, b.binary("multiply", b.const(2.0, T[r]), r))
+            tan[r] = b.emit("select", [b.compare("EQ", xs[0], b.const(0.0, T[r])), b.const(0.0, T[r]), g], {}, T[r])
+        elif n in ("maximum", "minimum"):
+            m = b.compare("GE" if n == "maximum" else "LE", xs[0], xs[1])
+            tan[r] = b.emit("select", [m, tz(xs[0]), tz(xs[1])], {}, T[r])
+        elif n == "power":
+            ym1 = b.binary("subtract", xs[1], b.const(1.0, T[r]))
+            tan[r] = add(None if ts[0] is None else b.binary("multiply", ts[0], b.binary("multiply", xs[1], b.binary("power", xs[0], ym1))),
+                         None if ts[1] is None else b.binary("multiply", ts[1], b.binary("multiply", r, b.unary("log", xs[0]))))
+        elif n == "compare":
+            continue
+        elif n == "select":
+            if ts[1] is not None or ts[2] is not None:
+                tan[r] = b.emit("select", [xs[0], tz(xs[1]), tz(xs[2])], {}, T[r])
         elif n == "rsqrt":
             tan[r] = b.binary("multiply", b.binary("multiply", b.const(-0.5, T[r]), t), b.binary("multiply", b.binary("multiply", r, r), r))
         elif n == "logistic":
@@ -378,10 +418,20 @@ def forward_function(func, name=None, arg_active=None):
         elif n in ("convert", "reshape", "transpose", "broadcast_in_dim", "slice"):
             tan[r] = b.emit(n, [t], op.attrs, T[r])
         elif n == "reduce":
-            if op.attrs["body"] != "add":
+            if t is None:
+                continue
+            z0 = zero(TensorType((), T[r].dtype))
+            if op.attrs["body"] == "add":
+                tan[r] = b.emit("reduce", [t, z0], op.attrs, T[r])
+            elif op.attrs["body"] == "maximum":
+                # the transpose of the reverse rule: tangents of all maximal elements, summed
+                xt = T[xs[0]]
+                kept = [d for d in range(len(xt.shape)) if d not in op.attrs["dims"]]
+                m = b.compare("EQ", xs[0], b.emit("broadcast_in_dim", [r], {"dims": kept}, xt))
+                tan[r] = b.emit("reduce", [b.emit("select", [m, t, b.const(0.0, xt)], {}, xt), z0],
+                                {"dims": op.attrs["dims"], "body": "add"}, T[r])
+            else:
                 raise NotImplementedError("symbolic forward mode of reduce with a %s body" % op.attrs["body"])
-            if t is not None:
-                tan[r] = b.emit("reduce", [t, zero(TensorType((), T[r].dtype))], op.attrs, T[r])
         elif n == "pad":
             if t is not None:
                 tan[r] = b.emit("pad", [t, zero(TensorType((), T[r].dtype))], op.attrs, T[r])

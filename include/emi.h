@@ -234,6 +234,15 @@ int emi_map_binary(emi_stream_t stream, int op, const void* a, const void* b, vo
 int emi_map_unary(emi_stream_t stream, int op, const void* x, void* y, int64_t n, int dtype);
 /* stablehlo.convert between EMI_F32 and EMI_BF16 (round to nearest even). */
 int emi_convert(emi_stream_t stream, const void* x, void* y, int64_t n, int from_dtype, int to_dtype);
+/* stablehlo.compare on floating-point operands: mask[i] = direction(a[i], b[i]) as one byte
+ * (0 or 1, the storage of an i1 tensor); stablehlo.select: y[i] = mask[i] ? a[i] : b[i]
+ * (Select rule HLODerivatives.td:1297; the guards of the Sqrt :1320 and Max :1205 rules are
+ * selects on compares).  *_is_scalar operands are one element broadcast to all i. */
+enum { EMI_CMP_EQ = 0, EMI_CMP_NE, EMI_CMP_GE, EMI_CMP_GT, EMI_CMP_LE, EMI_CMP_LT };
+int emi_compare(emi_stream_t stream, int direction, const void* a, const void* b, void* mask, int64_t n,
+                int a_is_scalar, int b_is_scalar, int dtype);
+int emi_select(emi_stream_t stream, const void* mask, const void* a, const void* b, void* y, int64_t n,
+               int mask_is_scalar, int a_is_scalar, int b_is_scalar, int dtype);
 /* out[out_offset + sum_d i_d out_strides[d]] = in[in_offset + sum_d i_d in_strides[d]] for every
  * index 0 <= i_d < dims[d]: transpose (permuted strides), broadcast_in_dim
  * (zero in_strides), slice (offset and strides; Slice rule

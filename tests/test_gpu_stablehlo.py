@@ -70,6 +70,32 @@ def test_elementwise_maps_match_numpy(dt, n):
     assert torch.equal(back, tx.to(torch.bfloat16).float())
 
 
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("n", [1, 9, 4099])
+def test_compare_and_select_match_numpy(dt, n):
+    from enzyme_ad.jax import hlo_ops as H
+
+    rng = np.random.default_rng(n + 1)
+    a, b = rng.normal(size=n), rng.normal(size=n)
+    b[::3] = a[::3]
+    (ta, ra), (tb, rb) = dev(a, dt), dev(b, dt)
+    s = torch.tensor(0.25, dtype=TDTYPE[dt], device="cuda")
+    fns = {"EQ": np.equal, "NE": np.not_equal, "GE": np.greater_equal, "GT": np.greater, "LE": np.less_equal, "LT": np.less}
+    for d, fn in fns.items():
+        m = H._compare(d, ta, tb)
+        assert m.dtype == torch.bool and np.array_equal(m.cpu().numpy(), fn(ra, rb)), d
+        assert np.array_equal(H._compare(d, ta, s).cpu().numpy(), fn(ra, 0.25)), d
+        assert np.array_equal(H._compare(d, s, tb).cpu().numpy(), fn(0.25, rb)), d
+    m = H._compare("GT", ta, tb)
+    assert np.array_equal(host(H._select(m, ta, tb)), np.where(ra > rb, ra, rb))
+    assert np.array_equal(host(H._select(m, s, tb)), np.where(ra > rb, 0.25, rb))
+    assert np.array_equal(host(H._select(m, ta, s)), np.where(ra > rb, ra, 0.25))
+    one = torch.tensor(True, device="cuda")
+    assert np.array_equal(host(H._select(one, ta, tb)), ra)
+    inf = torch.full_like(ta, float("inf"))
+    assert np.array_equal(host(H._select(m, ta, inf)), np.where(ra > rb, ra, np.inf))         # no 0 * inf
+
+
 def test_elementwise_maps_on_unaligned_views():
     from enzyme_ad.jax import hlo_ops as H
 
@@ -219,6 +245,17 @@ def test_rule_matches_reference_vector_through_text(name):
     grads = f_vjp(f32(np.ones(n)))
     for got, want in zip(grads, g["grads"]):
         np.testing.assert_allclose(host(got), want, rtol=3e-6, atol=1e-7)
+    # the symbolic programs (what optimize_module prints for the reference's AD pipelines)
+    if True:
+        from enzyme_ad.jax import stablehlo_ad
+        sym = hlo_call(*args, f32(np.ones(n)), source=stablehlo_ad.reverse_module_text(text))
+        for got, want in zip(sym, g["grads"]):
+            np.testing.assert_allclose(host(got), want, rtol=3e-6, atol=1e-7)
+        fwd = stablehlo_ad.forward_module_text(text)
+        flat = [v for a in args for v in (a, f32(np.ones(n)))]
+        out2, tan2 = hlo_call(*flat, source=fwd)
+        np.testing.assert_allclose(host(out2), g["out"], rtol=2e-6, atol=1e-7)
+        np.testing.assert_allclose(host(tan2), np.sum(np.asarray(g["grads"]), axis=0), rtol=3e-6, atol=1e-7)
     # forward mode against the same Jacobian: unit tangent on each operand in turn
     for i, want in enumerate(g["grads"]):
         tans = [f32(np.ones(n)) if j == i else None for j in range(len(args))]
@@ -271,3 +308,49 @@ def test_reduce_max_and_broadcast_rules_through_text():
     gx, gv = f_vjp((f32([10.0, 20.0]), f32(np.arange(8).reshape(2, 4))))
     assert np.array_equal(host(gx), [[0, 10.0, 10.0, 0], [20.0, 0, 0, 0]])
     assert np.array_equal(host(gv), [4.0, 6.0, 8.0, 10.0])
+
+
+def test_compare_select_and_reduce_max_through_text_in_all_three_modes():
+    """relu-like select on a compare, and a softmax spelled out (reduce-max, exp, reduce-add):
+    tape reverse mode, symbolic reverse module and symbolic forward module agree."""
+    from enzyme_ad.jax import hlo_call, jvp, stablehlo_ad, vjp
+
+    text = """
+    func.func @main(%x: tensor<3x5xf32>, %y: tensor<3x5xf32>) -> (tensor<3x5xf32>, tensor<3x5xf32>) {
+      %z = stablehlo.constant dense<0.000000e+00> : tensor<3x5xf32>
+      %p = stablehlo.compare GT, %x, %z, FLOAT : (tensor<3x5xf32>, tensor<3x5xf32>) -> tensor<3x5xi1>
+      %r = stablehlo.select %p, %x, %y : tensor<3x5xi1>, tensor<3x5xf32>
+      %ninf = stablehlo.constant dense<0xFF800000> : tensor<f32>
+      %zero = stablehlo.constant dense<0.000000e+00> : tensor<f32>
+      %mx = stablehlo.reduce(%r init: %ninf) applies stablehlo.maximum across dimensions = [1] : (tensor<3x5xf32>, tensor<f32>) -> tensor<3xf32>
+      %mb = stablehlo.broadcast_in_dim %mx, dims = [0] : (tensor<3xf32>) -> tensor<3x5xf32>
+      %e = stablehlo.exponential %r : tensor<3x5xf32>
+      %sh = stablehlo.subtract %r, %mb : tensor<3x5xf32>
+      %e2 = stablehlo.exponential %sh : tensor<3x5xf32>
+      %sm = stablehlo.reduce(%e2 init: %zero) applies stablehlo.add across dimensions = [1] : (tensor<3x5xf32>, tensor<f32>) -> tensor<3xf32>
+      %sb = stablehlo.broadcast_in_dim %sm, dims = [0] : (tensor<3xf32>) -> tensor<3x5xf32>
+      %soft = stablehlo.divide %e2, %sb : tensor<3x5xf32>
+      %mm = stablehlo.maximum %soft, %y : tensor<3x5xf32>
+      return %mm, %mb : tensor<3x5xf32>, tensor<3x5xf32>
+    }"""
+    rng = np.random.default_rng(4)
+    x, y = f32(rng.normal(size=(3, 5))), f32(rng.normal(size=(3, 5)) * 0.3)
+    c1, c2 = f32(rng.normal(size=(3, 5))), f32(rng.normal(size=(3, 5)))
+    tx, ty = f32(rng.normal(size=(3, 5))), f32(rng.normal(size=(3, 5)))
+    fn = lambda a, b: tuple(hlo_call(a, b, source=text))
+    outs, f_vjp = vjp(fn, x, y)
+    r = np.where(host(x) > 0, host(x), host(y))
+    e = np.exp(r - r.max(1, keepdims=True))
+    np.testing.assert_allclose(host(outs[0]), np.maximum(e / e.sum(1, keepdims=True), host(y)), rtol=1e-6)
+    tape = f_vjp((c1, c2))
+    sym = hlo_call(x, y, c1, c2, source=stablehlo_ad.reverse_module_text(text))
+    for g, t in zip(sym, tape):
+        np.testing.assert_allclose(host(g), host(t), rtol=1e-5, atol=1e-6)
+    _, tans = jvp(fn, (x, y), (tx, ty))
+    fo = hlo_call(x, tx, y, ty, source=stablehlo_ad.forward_module_text(text))
+    np.testing.assert_allclose(host(fo[1]), host(tans[0]), rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(host(fo[3]), host(tans[1]), rtol=1e-5, atol=1e-6)
+    # adjoint identity between the two symbolic programs
+    lhs = float(np.sum(host(fo[1]) * host(c1)) + np.sum(host(fo[3]) * host(c2)))
+    rhs = float(np.sum(host(sym[0]) * host(tx)) + np.sum(host(sym[1]) * host(ty)))
+    assert abs(lhs - rhs) <= 1e-5 * max(abs(lhs), abs(rhs), 1.0)

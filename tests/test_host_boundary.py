@@ -59,6 +59,9 @@ def test_plain_launchers_reject_bad_arguments_before_touching_the_gpu():
     assert lib.emi_strided_copy(None, 16, 16, 1, i64(4), i64(1), 0, i64(1), 0, 3) == 3         # element size
     assert lib.emi_strided_copy(None, 16, 16, 1, i64(4), i64(-1), 0, i64(1), 0, 4) == 3        # negative stride
     assert lib.emi_strided_copy(None, None, None, 2, i64(0, 4), i64(4, 1), 0, i64(4, 1), 0, 4) == 0   # empty box: nothing to do
+    assert lib.emi_compare(None, 6, 16, 16, 16, 8, 0, 0, 11) == 3 and b"direction" in lib.emi_last_error()
+    assert lib.emi_compare(None, 0, 16, 16, None, 8, 0, 0, 11) == 3 and b"null" in lib.emi_last_error()
+    assert lib.emi_select(None, 16, 16, 16, 16, 8, 0, 0, 0, 12) == 3 and b"dtype" in lib.emi_last_error()
     assert lib.emi_reduce(None, 2, 16, 16, None, 0, 4, 4, 1, 11) == 3 and b"add or max" in lib.emi_last_error()
     assert lib.emi_reduce(None, 0, 16, 16, None, 0, 70000, 4, 2, 11) == 3      # too many outer slices for the column form
     assert lib.emi_reduce(None, 0, 16, 16, None, 0, 4, 0, 1, 11) == 3          # empty reduction

@@ -181,11 +181,13 @@ def test_symbolic_reverse_mode_has_the_reference_ir_form():
     rev = A.reverse_module_text(div, arg_active=[False, True])
     f = __import__("enzyme_ad.jax.stablehlo", fromlist=["x"]).parse_module(rev)["main"]
     assert len(f.result_types) == 1 and [a for a, _ in f.args] == ["%a", "%b", "%ct0"]
-    with pytest.raises(NotImplementedError):
-        A.reverse_module_text("""func.func @main(%a: tensor<2xf32>, %b: tensor<2xf32>) -> tensor<2xf32> {
-          %c = stablehlo.maximum %a, %b : tensor<2xf32>
-          return %c : tensor<2xf32>
-        }""")
+    # maximum: a compare and two selects (ties to the first operand, maximum.mlir:25-34)
+    ops = _ops_of(A.reverse_module_text("""func.func @main(%a: tensor<2xf32>, %b: tensor<2xf32>) -> tensor<2xf32> {
+      %c = stablehlo.maximum %a, %b : tensor<2xf32>
+      return %c : tensor<2xf32>
+    }"""))
+    assert sorted(o[0] for o in ops) == ["compare", "constant", "return", "select", "select"]
+    assert [o[2] for o in ops if o[0] == "compare"] == [{"direction": "GE"}]
 
 
 def test_symbolic_reverse_of_the_llama_step_calls_the_adjoint_targets():
