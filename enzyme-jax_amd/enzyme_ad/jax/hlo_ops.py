@@ -12,7 +12,6 @@ Slice :1586, Reduce :1833-1916, Concatenate :2015).  The rules themselves are co
 the same kernels, outside the tape.
 """
 import ctypes
-import math
 
 import torch
 

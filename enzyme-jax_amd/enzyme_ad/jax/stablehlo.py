@@ -18,7 +18,6 @@ custom_call (this library's targets), return.  Anything else raises `NotImplemen
 """
 import math
 import re
-import struct
 
 import numpy as np
 import torch
@@ -319,7 +318,7 @@ def _parse_op(sc):
     short = name.split(".", 1)[1] if name.startswith(("stablehlo.", "mhlo.", "func.", "arith.")) else name
     attrs = {}
 
-    def operand_list(close=None):
+    def operand_list():
         out = []
         while True:
             v = sc.match(_SSA)

@@ -17,7 +17,7 @@ import re
 
 import numpy as np
 
-from .stablehlo import BINARY_OPS, UNARY_OPS, Func, Op, TensorType, _drop_dead, _splat
+from .stablehlo import Func, Op, TensorType, _drop_dead
 
 FLOAT = ("f32", "bf16", "f16", "f64")
 
@@ -499,22 +499,8 @@ def _reverse_dot_general(b, op, c, accum):
 
     # c dims: batch (nb), free of a (nfa), free of b (nfb)
     accum(a_, grad(b_, bt, bb, fb, cb, at, ba, fa, ca, nb + nfa))
-    # for b: c's free-of-a dims are contracted with a's free dims; the product's free dims are c's free-of-b dims
-    rest = sorted(ca)
-    shape = [at.shape[d] for d in ba] + [bt.shape[d] for d in fb] + [at.shape[d] for d in rest]
-    g = b.emit("dot_general", [c, a_], {"batch_a": list(range(nb)), "batch_b": list(ba),
-                                        "contract_a": list(range(nb, nb + nfa)), "contract_b": list(fa)}, TensorType(shape, bt.dtype))
-    src = {}
-    for i, d in enumerate(bb):
-        src[d] = i
-    for i, d in enumerate(fb):
-        src[d] = nb + i
-    for i, d in enumerate(rest):
-        src[cb[ca.index(d)]] = nb + nfb + i
-    perm = [src[d] for d in range(len(bt.shape))]
-    if perm != list(range(len(perm))):
-        g = b.emit("transpose", [g], {"perm": perm}, bt)
-    accum(b_, g)
+    # for b: c's free-of-a dims (from position nb) meet a's free dims; c's free-of-b dims stay
+    accum(b_, grad(a_, at, ba, fa, ca, bt, bb, fb, cb, nb))
 
 
 def _reverse_custom_call(b, op, cs, accum):
