@@ -299,6 +299,25 @@ def bench_frontend(iters):
         return f_vjp(dy)
 
     out["llama_step_hand_wired"] = dict(us_per_step=round(event_time(hand, iters) * 1e6, 1))
+    # the same two programs captured once into a HIP graph and replayed (the counterpart of the
+    # reference's compiled executable): launch and host overhead gone, kernel time left
+    from enzyme_ad.jax.graph import capture
+
+    def hand_fn(x, w, kc, vc, dy_):
+        y, f_vjp = vjp(lambda a, b, c, d: llama.forward_step(a, hcfg, b, c, d), x, w, kc, vc)
+        return y, f_vjp(dy_)
+
+    g = capture(hand_fn, named["x"], weights, named["key_cache"], named["value_cache"], dy)
+    out["llama_step_hand_wired_graph"] = dict(
+        us_per_step=round(event_time(lambda: g(named["x"], weights, named["key_cache"], named["value_cache"], dy), 4 * iters) * 1e6, 1))
+    exe = stablehlo.compile_text(text, fuse=True)
+
+    def text_fn(dy_, *a):
+        y, f_vjp = vjp(lambda *b: exe.run(list(b))[0], *a)
+        return y, f_vjp(dy_)
+
+    gt = capture(text_fn, dy, *args)
+    out["llama_step_text_fused_graph"] = dict(us_per_step=round(event_time(lambda: gt(dy, *args), 4 * iters) * 1e6, 1))
     return out
 
 
