@@ -375,7 +375,6 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible; the HIP path has no CPU fallback")
     from enzyme_ad.jax import enzyme_jax_ir, JaXPipeline, vjp, llama
-    from enzyme_ad.jax.profiling import pretty_print_table
 
     if args.calibrate:
         from enzyme_ad.jax import ops as _ops
@@ -407,8 +406,7 @@ def main():
     tokens = cfg["batch"] * cfg["seq"]
     fl = layer_flops(cfg)
     name = "llama7b_layer_B%d_S%d" % (cfg["batch"], cfg["seq"])
-    pretty_print_table(name, "HIP", "rocm", "BothRev", dt) if False else log(
-        "%s\tHIP\trocm\tPrimal+VJP\t%.6f s  (%.1f TFLOP/s over %.2f TFLOP algorithmic)" % (name, dt, fl["total"] / dt / 1e12, fl["total"] / 1e12))
+    log("%s\tHIP\trocm\tPrimal+VJP\t%.6f s  (%.1f TFLOP/s over %.2f TFLOP algorithmic)" % (name, dt, fl["total"] / dt / 1e12, fl["total"] / 1e12))
 
     t_gemm, gemm_fl, n_gemm, per_layout = bench_gemms(cfg, max(5, min(args.steps, 20)))
     roofline = dict(bound="mfma", kernel="gemm_bf16_pingpong_kernel (256x256x64 tiles; %d launches per step: Y, dX in the NT form, dW in the TN form, 7 weights)" % n_gemm,

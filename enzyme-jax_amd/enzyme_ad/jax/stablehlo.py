@@ -516,9 +516,44 @@ def _parse_func(sc):
     return Func(name, args, result_types, body)
 
 
+def _strip_locations(text):
+    """Debug locations (`loc(...)` trailers, nested to any depth, and `#loc = ...` alias lines)
+    carry nothing the executor uses."""
+    if "loc(" not in text:
+        return text
+    text = "\n".join(l for l in text.split("\n") if not l.lstrip().startswith("#loc"))
+    out, i, n = [], 0, len(text)
+    while i < n:
+        j = text.find("loc(", i)
+        if j < 0:
+            out.append(text[i:])
+            break
+        if j > 0 and (text[j - 1].isalnum() or text[j - 1] in "_.#"):
+            out.append(text[i:j + 4])                      # part of a longer name
+            i = j + 4
+            continue
+        out.append(text[i:j])
+        k, depth = j + 3, 0
+        while k < n:
+            c = text[k]
+            if c == '"':
+                k = text.find('"', k + 1)
+                if k < 0:
+                    raise ParseError("unterminated string in a location")
+            elif c == "(":
+                depth += 1
+            elif c == ")":
+                depth -= 1
+                if depth == 0:
+                    break
+            k += 1
+        i = k + 1
+    return "".join(out)
+
+
 def parse_module(text):
     """{function name: Func} of a StableHLO module (or of bare func.func definitions)."""
-    sc = _Scanner(text)
+    sc = _Scanner(_strip_locations(text))
     funcs = {}
     wrapped = False
     if sc.accept("module"):

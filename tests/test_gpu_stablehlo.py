@@ -354,3 +354,36 @@ def test_compare_select_and_reduce_max_through_text_in_all_three_modes():
     lhs = float(np.sum(host(fo[1]) * host(c1)) + np.sum(host(fo[3]) * host(c2)))
     rhs = float(np.sum(host(sym[0]) * host(tx)) + np.sum(host(sym[1]) * host(ty)))
     assert abs(lhs - rhs) <= 1e-5 * max(abs(lhs), abs(rhs), 1.0)
+
+
+def test_calls_between_functions_run_and_differentiate():
+    """A private function called twice (what nested jit leaves in a traced module): tape modes
+    run through the call, the symbolic programs inline it."""
+    from enzyme_ad.jax import hlo_call, jvp, stablehlo_ad, vjp
+
+    text = """module @jit_f {
+      func.func public @main(%x: tensor<4xf32>, %y: tensor<4xf32>) -> (tensor<4xf32> {jax.result_info = ""}) {
+        %0 = call @scale(%x, %y) : (tensor<4xf32>, tensor<4xf32>) -> tensor<4xf32>
+        %1 = call @scale(%0, %x) : (tensor<4xf32>, tensor<4xf32>) -> tensor<4xf32>
+        return %1 : tensor<4xf32>
+      }
+      func.func private @scale(%a: tensor<4xf32>, %b: tensor<4xf32>) -> tensor<4xf32> {
+        %e = stablehlo.exponential %b : tensor<4xf32>
+        %r = stablehlo.multiply %a, %e : tensor<4xf32>
+        return %r : tensor<4xf32>
+      }
+    }"""
+    x, y, c, tx, ty = (f32(v) for v in ([0.1, 0.2, -0.3, 0.4], [1.0, -1.0, 0.5, 0.0], [1.0, 2.0, 3.0, 4.0], [0.5, 0.5, 0.5, 0.5], [1.0, 0.0, -1.0, 2.0]))
+    fn = lambda a, b: hlo_call(a, b, source=text)[0]
+    out, f_vjp = vjp(fn, x, y)
+    xr, yr = host(x), host(y)
+    np.testing.assert_allclose(host(out), xr * np.exp(yr) * np.exp(xr), rtol=1e-6)
+    gx, gy = f_vjp(c)
+    np.testing.assert_allclose(host(gx), host(c) * np.exp(yr) * np.exp(xr) * (1 + xr), rtol=1e-5)
+    np.testing.assert_allclose(host(gy), host(c) * host(out), rtol=1e-5)
+    sym = hlo_call(x, y, c, source=stablehlo_ad.reverse_module_text(text))
+    np.testing.assert_allclose(host(sym[0]), host(gx), rtol=1e-6)
+    np.testing.assert_allclose(host(sym[1]), host(gy), rtol=1e-6)
+    _, t = jvp(fn, (x, y), (tx, ty))
+    fo = hlo_call(x, tx, y, ty, source=stablehlo_ad.forward_module_text(text))
+    np.testing.assert_allclose(host(fo[1]), host(t), rtol=1e-6)

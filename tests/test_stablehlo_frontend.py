@@ -236,3 +236,26 @@ def test_optimize_module_differentiates_when_the_pipeline_says_so():
     assert sorted(o.name for o in both.ops) == ["divide", "divide", "multiply", "multiply", "multiply", "return", "subtract"]
     with pytest.raises(NotImplementedError, match="ForwardModeSplit"):
         ej.optimize_module(text, fwd.pass_pipeline().replace("mode=ForwardMode", "mode=ForwardModeSplit"))
+
+
+def test_parser_drops_debug_locations():
+    from enzyme_ad.jax import stablehlo as S
+
+    text = """#loc = loc(unknown)
+module @jit_f attributes {mhlo.num_partitions = 1 : i32, mhlo.num_replicas = 1 : i32} {
+  func.func public @main(%arg0: tensor<4xf32> {mhlo.layout_mode = "default"} loc(unknown)) -> (tensor<4xf32> {jax.result_info = ""}) {
+    %0 = stablehlo.multiply %arg0, %arg0 : tensor<4xf32> loc(#loc2)
+    %1 = call @inner(%0) : (tensor<4xf32>) -> tensor<4xf32> loc(#loc3)
+    return %1 : tensor<4xf32> loc(#loc)
+  } loc(#loc)
+  func.func private @inner(%arg0: tensor<4xf32> loc("x(1)"(callsite("f"("a.py":3:0) at "g"("b.py":7:1))))) -> tensor<4xf32> {
+    %0 = stablehlo.negate %arg0 : tensor<4xf32> loc(#loc4)
+    return %0 : tensor<4xf32> loc(#loc)
+  } loc(#loc)
+} loc(#loc)
+#loc1 = loc("a.py":3:0)
+#loc2 = loc("jit(f)/mul"(#loc1))
+"""
+    funcs = S.parse_module(text)
+    assert [o.name for o in funcs["main"].ops] == ["multiply", "call", "return"]
+    assert [o.name for o in funcs["inner"].ops] == ["negate", "return"]
