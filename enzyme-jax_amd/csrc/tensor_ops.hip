@@ -275,7 +275,7 @@ struct TilePlan {
 template <typename E>
 __global__ void __launch_bounds__(kBlock) tiled_permute_kernel(const E* __restrict__ in, E* __restrict__ out, TilePlan p,
                                                                int vec_ok) {
-  constexpr int TS = 64, PADW = TS + (sizeof(E) == 2 ? 2 : 1);
+  constexpr int TS = 64, PADW = TS + (sizeof(E) == 1 ? 4 : sizeof(E) == 2 ? 2 : 1);
   __shared__ E tile[TS][PADW];
   int64_t rem = blockIdx.z, ib = 0, ob = 0;
 #pragma unroll
@@ -734,7 +734,8 @@ extern "C" int emi_strided_copy(emi_stream_t stream, const void* in, void* out, 
                                 const int64_t* in_strides, int64_t in_offset, const int64_t* out_strides,
                                 int64_t out_offset, int elem_bytes) {
   EMI_REQUIRE(rank >= 0 && rank <= kMaxRank, "emi_strided_copy: rank %d (at most %d)", rank, kMaxRank);
-  EMI_REQUIRE(elem_bytes == 2 || elem_bytes == 4 || elem_bytes == 8, "emi_strided_copy: element size %d", elem_bytes);
+  EMI_REQUIRE(elem_bytes == 1 || elem_bytes == 2 || elem_bytes == 4 || elem_bytes == 8, "emi_strided_copy: element size %d",
+              elem_bytes);
   EMI_REQUIRE(rank == 0 || (dims && in_strides && out_strides), "emi_strided_copy: null shape");
   EMI_REQUIRE(in_offset >= 0 && out_offset >= 0, "emi_strided_copy: negative offset");
   int64_t total = 1;
@@ -779,6 +780,7 @@ extern "C" int emi_strided_copy(emi_stream_t stream, const void* in, void* out, 
     for (int d = 0; d < l; d++) { q.is[d] /= N; q.os[d] /= N; }
     return launch_copy<uint4>(st, ip, op, q);
   }
+  if (elem_bytes == 1) return launch_copy<uint8_t>(st, ip, op, p);
   if (elem_bytes == 2) return launch_copy<uint16_t>(st, ip, op, p);
   if (elem_bytes == 4) return launch_copy<uint32_t>(st, ip, op, p);
   return launch_copy<uint64_t>(st, ip, op, p);

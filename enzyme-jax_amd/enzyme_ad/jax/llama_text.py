@@ -75,6 +75,50 @@ class Builder:
         return self.emit(shape, "stablehlo.reduce(%s init: %s) applies stablehlo.%s across dimensions = [%s] : (%s, %s) -> %s" % (
             a, init, kind, ", ".join(str(d) for d in dims), self.t(a), self.ty(()), self.ty(shape)))
 
+    def blob(self, array, dtype=None):
+        """A constant too large to spell out: raw little-endian bytes as a hex string."""
+        a = np.ascontiguousarray(array, dtype=np.float32)
+        shape = a.shape
+        if (dtype or self.dtype) == "bf16":
+            bits = a.view(np.uint32)
+            raw = ((bits + 0x7FFF + ((bits >> 16) & 1)) >> 16).astype("<u2").tobytes()      # round to nearest even
+        else:
+            raw = a.astype("<f4").tobytes()
+        ty = "tensor<%s>" % "x".join([str(s) for s in shape] + [dtype or self.dtype])
+        r = self.new(shape)
+        self.lines.append('    %s = stablehlo.constant dense<"0x%s"> : %s' % (r, raw.hex().upper(), ty))
+        return r
+
+    def transpose(self, a, perm):
+        shape = [self.types[a][p] for p in perm]
+        return self.emit(shape, "stablehlo.transpose %s, dims = [%s] : (%s) -> %s" % (
+            a, ", ".join(str(p) for p in perm), self.t(a), self.ty(shape)))
+
+    def iota(self, shape, dim):
+        r = self.new(shape)
+        self.lines.append("    %s = stablehlo.iota dim = %d : tensor<%s>" % (r, dim, "x".join([str(s) for s in shape] + ["i32"])))
+        return r
+
+    def compare(self, direction, a, b, kind="SIGNED", elem="i32"):
+        shape = self.types[a]
+        ty = "tensor<%s>" % "x".join([str(s) for s in shape] + [elem])
+        r = self.new(shape)
+        self.lines.append("    %s = stablehlo.compare %s, %s, %s, %s : (%s, %s) -> tensor<%s>" % (
+            r, direction, a, b, kind, ty, ty, "x".join([str(s) for s in shape] + ["i1"])))
+        return r
+
+    def bcast_pred(self, a, shape, dims):
+        r = self.new(shape)
+        i1 = lambda sh: "tensor<%s>" % "x".join([str(s) for s in sh] + ["i1"])
+        self.lines.append("    %s = stablehlo.broadcast_in_dim %s, dims = [%s] : (%s) -> %s" % (
+            r, a, ", ".join(str(d) for d in dims), i1(self.types[a]), i1(shape)))
+        return r
+
+    def select(self, p, a, b):
+        shape = self.types[a]
+        i1 = "tensor<%s>" % "x".join([str(s) for s in shape] + ["i1"])
+        return self.emit(shape, "stablehlo.select %s, %s, %s : %s, %s" % (p, a, b, i1, self.t(a)))
+
     def dot(self, a, b, batch=((), ()), contract=((), ())):
         sa, sb = self.types[a], self.types[b]
         shape = [sa[d] for d in batch[0]] + [s for i, s in enumerate(sa) if i not in batch[0] and i not in contract[0]] + \
@@ -175,3 +219,76 @@ def llama_step_text(config, pos, dtype="f32"):
         ", ".join("%s: %s" % (a[n], b.ty(shapes[n])) for n in order), b.ty((dim,)))
     text = head + "\n".join(b.lines) + "\n    return %s : %s\n  }\n}\n" % (x, b.ty((dim,)))
     return text, order
+
+
+LAYER_ORDER = ["rms_att_weight", "wq", "wk", "wv", "wo", "rms_ffn_weight", "w1", "w2", "w3"]
+
+
+def llama_layer_text(config, batch, seq, dtype="f32", eps=1e-5, theta=10000.0):
+    """(text, argument names): one decoder layer of test/llama.py:144-233 over a whole batch of
+    sequences, main(x [B, S, dim], <weights in LAYER_ORDER>) -> x, written the way the batched
+    form of that function traces: RMSNorm as sum(x*x) / dim over the last index, projections as
+    dot_general against [out, in] weights, the pair rotation with cos / sin tables [S, hs/2]
+    (constants: positions are static), scores per head from a batched dot_general, a causal mask
+    from two iotas and a compare, softmax over the keys, and the SwiGLU FFN."""
+    dim, hidden, H = config["dim"], config["hidden_dim"], config["n_heads"]
+    hs = dim // H
+    B, S = batch, seq
+    b = Builder(dtype)
+    shapes = {"x": (B, S, dim), "rms_att_weight": (dim,), "wq": (dim, dim), "wk": (dim, dim), "wv": (dim, dim), "wo": (dim, dim),
+              "rms_ffn_weight": (dim,), "w1": (hidden, dim), "w2": (dim, hidden), "w3": (hidden, dim)}
+    order = ["x"] + LAYER_ORDER
+    a = {n: b.arg("%" + n, shapes[n]) for n in order}
+
+    def rmsnorm(x, w):
+        ss = b.reduce(b.binary("multiply", x, x), "add", [2])                          # [B, S]
+        ss = b.binary("divide", ss, b.bcast(b.const(float(dim)), (B, S)))
+        ss = b.binary("add", ss, b.bcast(b.const(eps), (B, S)))
+        ss = b.binary("divide", b.bcast(b.const(1.0), (B, S)), b.unary("sqrt", ss))
+        xn = b.binary("multiply", x, b.bcast(ss, (B, S, dim), (0, 1)))
+        return b.binary("multiply", xn, b.bcast(w, (B, S, dim), (2,)))
+
+    def linear(x, w):
+        return b.dot(x, w, contract=((len(b.types[x]) - 1,), (1,)))
+
+    pos = np.arange(S, dtype=np.float64)[:, None]
+    freq = 1.0 / np.power(theta, (2.0 * np.arange(hs // 2, dtype=np.float64)) / hs)[None, :]
+    cos_c, sin_c = b.blob(np.cos(pos * freq), "f32"), b.blob(np.sin(pos * freq), "f32")
+    if dtype != "f32":
+        cos_c = b.emit((S, hs // 2), "stablehlo.convert %s : (tensor<%dx%dxf32>) -> %s" % (cos_c, S, hs // 2, b.ty((S, hs // 2))))
+        sin_c = b.emit((S, hs // 2), "stablehlo.convert %s : (tensor<%dx%dxf32>) -> %s" % (sin_c, S, hs // 2, b.ty((S, hs // 2))))
+
+    def rope(x):
+        xr = b.reshape(x, (B, S, H, hs // 2, 2))
+        half = (B, S, H, hs // 2)
+        x0 = b.reshape(b.slice(xr, [0, 0, 0, 0, 0], [B, S, H, hs // 2, 1]), half)
+        x1 = b.reshape(b.slice(xr, [0, 0, 0, 0, 1], [B, S, H, hs // 2, 2]), half)
+        cb, sb = b.bcast(cos_c, half, (1, 3)), b.bcast(sin_c, half, (1, 3))
+        o0 = b.binary("subtract", b.binary("multiply", x0, cb), b.binary("multiply", x1, sb))
+        o1 = b.binary("add", b.binary("multiply", x0, sb), b.binary("multiply", x1, cb))
+        both = b.concat([b.reshape(o0, half + (1,)), b.reshape(o1, half + (1,))], 4)
+        return b.reshape(both, (B, S, dim))
+
+    x = a["x"]
+    xb = rmsnorm(x, a["rms_att_weight"])
+    q, k, v = rope(linear(xb, a["wq"])), rope(linear(xb, a["wk"])), linear(xb, a["wv"])
+    heads = lambda t: b.transpose(b.reshape(t, (B, S, H, hs)), [0, 2, 1, 3])                 # [B, H, S, hs]
+    qh, kh, vh = heads(q), heads(k), heads(v)
+    att = b.dot(qh, kh, batch=((0, 1), (0, 1)), contract=((3,), (3,)))                      # [B, H, S, S]
+    att = b.binary("divide", att, b.bcast(b.unary("sqrt", b.const(float(hs))), (B, H, S, S)))
+    causal = b.compare("GE", b.iota((S, S), 0), b.iota((S, S), 1))                           # key <= query
+    att = b.select(b.bcast_pred(causal, (B, H, S, S), (2, 3)), att, b.bcast(b.const(-np.inf), (B, H, S, S)))
+    mx = b.reduce(att, "maximum", [3])
+    e = b.unary("exponential", b.binary("subtract", att, b.bcast(mx, (B, H, S, S), (0, 1, 2))))
+    p = b.binary("divide", e, b.bcast(b.reduce(e, "add", [3]), (B, H, S, S), (0, 1, 2)))
+    o = b.dot(p, vh, batch=((0, 1), (0, 1)), contract=((3,), (2,)))                         # [B, H, S, hs]
+    o = b.reshape(b.transpose(o, [0, 2, 1, 3]), (B, S, dim))
+    x = b.binary("add", x, linear(o, a["wo"]))
+    xb = rmsnorm(x, a["rms_ffn_weight"])
+    hb, hb2 = linear(xb, a["w1"]), linear(xb, a["w3"])
+    one = b.bcast(b.const(1.0), (B, S, hidden))
+    sig = b.binary("divide", one, b.binary("add", one, b.unary("exponential", b.unary("negate", hb))))
+    x = b.binary("add", x, linear(b.binary("multiply", b.binary("multiply", hb, sig), hb2), a["w2"]))
+    head = "module @jit_layer {\n  func.func public @main(%s) -> (%s {jax.result_info = \"\"}) {\n" % (
+        ", ".join("%s: %s" % (a[n], b.ty(shapes[n])) for n in order), b.ty((B, S, dim)))
+    return head + "\n".join(b.lines) + "\n    return %s : %s\n  }\n}\n" % (x, b.ty((B, S, dim))), order

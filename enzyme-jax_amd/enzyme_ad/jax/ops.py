@@ -311,6 +311,31 @@ def rotate_pairs(x, table, inverse=False):
     return y
 
 
+def rope_rows(x, n_heads, table, inverse=False):
+    """RoPE over a batch of sequences with an explicit fp32 (cos, sin) table [S, head_dim/2, 2]
+    (what the StableHLO front end recovers from a traced module's constants): x is
+    [B, S, n_heads*head_dim], position = index along S.  Adjoint = inverse rotation."""
+    _dev(x, table)
+    B, S, D = x.shape
+    d = D // n_heads
+    if table.dtype != torch.float32 or tuple(table.shape) != (S, d // 2, 2) or d * n_heads != D or d % 2:
+        raise ValueError("rope_rows: table %s for x %s with %d heads" % (tuple(table.shape), tuple(x.shape), n_heads))
+    y = torch.empty_like(x)
+    N.check(N.lib().emi_rope(_stream(), _p(x), _p(table), _p(y), B, S, n_heads, d, int(inverse), _code(x)))
+
+    def rule(c, acc):
+        g = torch.empty_like(c)
+        N.check(N.lib().emi_rope(_stream(), _p(c), _p(table), _p(g), B, S, n_heads, d, int(not inverse), _code(c)))
+        return (_accumulate(acc[0], g), None)
+
+    Tape.record((x, table), y, rule)
+    tans = _tan(x)
+    if tans is not None and tans[0] is not None:
+        tx = tans[0]
+        _set_tan(y, _quiet(lambda: rope_rows(tx, n_heads, table, inverse)))
+    return y
+
+
 def transpose(a):
     """a^T for a 2-D operand (a fresh buffer; Transpose rule HLODerivatives.td:1334)."""
     _dev(a)

@@ -414,6 +414,12 @@ def _parse_op(sc):
         text = sc.balanced() if sc.peek("{") else "{}"
         _, types = sc.signature()
         return Op("custom_call", results, operands, {"target": target, "config": _backend_config(text)}, types)
+    if short == "iota":
+        sc.expect("dim")
+        sc.expect("=")
+        dim = int(sc.need(_INT, "iota dimension"))
+        _, types = sc.signature()
+        return Op("iota", results, [], {"dim": dim}, types)
     if short == "compare":
         direction = sc.need(_IDENT, "comparison direction")
         sc.expect(",")
@@ -605,6 +611,11 @@ _FOLD_BINARY = {"add": np.add, "subtract": np.subtract, "multiply": np.multiply,
                 "maximum": np.maximum, "minimum": np.minimum, "power": np.power}
 
 
+_FOLD_COMPARE = {"EQ": np.equal, "NE": np.not_equal, "GE": np.greater_equal, "GT": np.greater, "LE": np.less_equal,
+                 "LT": np.less}
+MASK_LIMIT = 1 << 25          # elements of a trace-time mask (iota / compare / broadcast of i1) folded at parse
+
+
 def fold_constants(func, limit=4096):
     """Evaluates, at parse time, operators whose operands are all constants (like
     `jnp.sqrt(head_size)`, test/llama.py:196, which reaches the text as sqrt of a constant),
@@ -616,6 +627,27 @@ def fold_constants(func, limit=4096):
         srcs = [defs.get(o) for o in op.operands]
         ty = op.types[0] if op.types else None
         new = None
+        # masks that depend on no argument (`jnp.tril`-style causal masks: iota, iota, compare)
+        if ty is not None and int(np.prod(ty.shape or (1,))) <= MASK_LIMIT and all(c is not None and c.name == "constant" for c in srcs):
+            mask = None
+            if op.name == "iota" and ty.dtype in ("i32", "i64"):
+                shape = [1] * len(ty.shape)
+                shape[op.attrs["dim"]] = ty.shape[op.attrs["dim"]]
+                mask = np.broadcast_to(np.arange(ty.shape[op.attrs["dim"]], dtype=NUMPY_DTYPES[ty.dtype]).reshape(shape), ty.shape)
+            elif op.name == "compare" and ty.dtype == "i1":
+                mask = _FOLD_COMPARE[op.attrs["direction"]](np.asarray(srcs[0].attrs["value"]), np.asarray(srcs[1].attrs["value"]))
+            elif op.name == "broadcast_in_dim" and ty.dtype == "i1":
+                v = np.asarray(srcs[0].attrs["value"])
+                shape = [1] * len(ty.shape)
+                for i, d in enumerate(op.attrs["dims"]):
+                    shape[d] = v.shape[i]
+                mask = np.broadcast_to(v.reshape(shape), ty.shape)
+            if mask is not None:
+                op = Op("constant", op.results, [], {"value": mask}, op.types)
+                for r in op.results:
+                    defs[r] = op
+                out.append(op)
+                continue
         if op.operands and all(c is not None and c.name == "constant" for c in srcs) and ty is not None \
                 and ty.dtype in ("f32", "bf16") and int(np.prod(ty.shape or (1,))) <= limit:
             vals = [np.asarray(c.attrs["value"], dtype=np.float32) for c in srcs]
@@ -627,11 +659,8 @@ def fold_constants(func, limit=4096):
                 new = vals[0].reshape(ty.shape)
             elif op.name == "transpose":
                 new = vals[0].transpose(op.attrs["perm"])
-            elif op.name == "broadcast_in_dim":
-                shape = [1] * len(ty.shape)
-                for i, d in enumerate(op.attrs["dims"]):
-                    shape[d] = vals[0].shape[i]
-                new = np.broadcast_to(vals[0].reshape(shape), ty.shape)
+            elif op.name == "broadcast_in_dim" and _splat(srcs[0]) is not None:
+                new = np.full(ty.shape, vals[0].reshape(-1)[0], dtype=np.float32)       # tables stay tables
             elif op.name == "convert":
                 new = vals[0]
             if new is not None:
@@ -656,7 +685,10 @@ def _drop_dead(func):
     func.ops = list(reversed(kept))
 
 
-def fuse_clusters(func, kinds=("rmsnorm", "swiglu", "rope", "softmax_dot", "attention_step")):
+ALL_KINDS = ("rmsnorm", "swiglu", "rope", "softmax_dot", "attention_step", "rmsnorm_rows", "rope_rows", "attention")
+
+
+def fuse_clusters(func, kinds=ALL_KINDS):
     """Rewrites, in place, the operator clusters test/llama.py traces into fused operators:
 
       emi.rmsnorm  w * (x * (1 / sqrt(dot(x, x) / n + eps)))           (llama.py:6-10), also with
@@ -670,9 +702,12 @@ def fuse_clusters(func, kinds=("rmsnorm", "swiglu", "rope", "softmax_dot", "atte
 
     A cluster is fused only when none of its interior values is used outside it.  Returns
     the number of clusters fused per kind."""
-    counts = {"rmsnorm": 0, "swiglu": 0, "rope": 0, "softmax_dot": 0, "attention_step": 0}
+    counts = {"rmsnorm": 0, "swiglu": 0, "rope": 0, "softmax_dot": 0, "attention_step": 0, "rmsnorm_rows": 0, "rope_rows": 0,
+              "attention": 0}
     matchers = [m for k, m in (("rmsnorm", _match_rmsnorm), ("swiglu", _match_swiglu), ("rope", _match_rope),
-                               ("softmax_dot", _match_softmax_dot), ("attention_step", _match_heads)) if k in kinds]
+                               ("softmax_dot", _match_softmax_dot), ("attention_step", _match_heads),
+                               ("rmsnorm_rows", _match_rmsnorm_rows), ("rope_rows", _match_rope_rows),
+                               ("attention", _match_attention)) if k in kinds]
     changed = True
     while changed:
         changed = False
@@ -874,6 +909,209 @@ def _match_softmax_dot(op, d, tb):
     return None
 
 
+def _bcast(name, d, dims=None):
+    """(operand, op) when `name` is a broadcast_in_dim (with the given dims), else (None, None)."""
+    op = d(name)
+    if op is not None and op.name == "broadcast_in_dim" and (dims is None or list(op.attrs["dims"]) == list(dims)):
+        return op.operands[0], op
+    return None, None
+
+
+def _match_rmsnorm_rows(op, d, tb):
+    # batched form: (x * bcast(1 / sqrt(sum(x * x, last) / n + eps))) * bcast(w, last), x [..., n]
+    if op.name != "multiply":
+        return None
+    rank = len(op.types[0].shape)
+    if rank < 2:
+        return None
+    lead = list(range(rank - 1))
+    for wi in (0, 1):
+        w, wb = _bcast(op.operands[wi], d, [rank - 1])
+        inner = d(op.operands[1 - wi])
+        if wb is None or inner is None or inner.name != "multiply":
+            continue
+        for xi in (0, 1):
+            x = inner.operands[xi]
+            r_name, rb = _bcast(inner.operands[1 - xi], d, lead)
+            if rb is None:
+                continue
+            ss = d(r_name)
+            if ss is None:
+                continue
+            interior = [op, wb, inner, rb, ss]
+            if ss.name == "rsqrt":
+                arg = d(ss.operands[0])
+            elif ss.name == "divide" and _splat(d(tb(ss.operands[0])[0])) == 1.0:
+                sq = d(ss.operands[1])
+                if sq is None or sq.name != "sqrt":
+                    continue
+                interior += [sq] + [o for o in [tb(ss.operands[0])[1]] if o is not None]
+                arg = d(sq.operands[0])
+            else:
+                continue
+            if arg is None or arg.name != "add":
+                continue
+            eps = mean = None
+            for ei in (0, 1):
+                en, eb = tb(arg.operands[ei])
+                e = _splat(d(en))
+                if e is not None:
+                    eps, mean = e, d(arg.operands[1 - ei])
+                    interior += [o for o in [eb] if o is not None]
+            if eps is None or mean is None or mean.name != "divide":
+                continue
+            nn, nbc = tb(mean.operands[1])
+            n = _splat(d(nn))
+            red = d(mean.operands[0])
+            if n is None or red is None or red.name != "reduce" or red.attrs["body"] != "add" or list(red.attrs["dims"]) != [rank - 1]:
+                continue
+            sq2 = d(red.operands[0])
+            if sq2 is None or sq2.name != "multiply" or sq2.operands != [x, x] or n != float(op.types[0].shape[-1]):
+                continue
+            interior += [arg, mean, red, sq2] + [o for o in [nbc] if o is not None]
+            return "rmsnorm_rows", Op("emi.rmsnorm_rows", op.results, [x, w], {"eps": eps}, op.types), interior
+    return None
+
+
+def _match_rope_rows(op, d, tb):
+    # reshape(concat([reshape(x0 c - x1 s), reshape(x0 s + x1 c)], last)) with x0 / x1 the even / odd
+    # elements of reshape(x, [B, S, h, P, 2]) and c, s constant tables [S, P] broadcast over dims (1, 3)
+    if op.name != "reshape" or len(op.types[0].shape) != 3:
+        return None
+    cat = d(op.operands[0])
+    if cat is None or cat.name != "concatenate" or cat.attrs["dim"] != 4 or len(cat.operands) != 2:
+        return None
+    r0, r1 = d(cat.operands[0]), d(cat.operands[1])
+    if r0 is None or r1 is None or r0.name != "reshape" or r1.name != "reshape":
+        return None
+    o0, o1 = d(r0.operands[0]), d(r1.operands[0])
+    if o0 is None or o1 is None or o0.name != "subtract" or o1.name != "add":
+        return None
+    m = [d(o) for o in (o0.operands[0], o0.operands[1], o1.operands[0], o1.operands[1])]
+    if any(t is None or t.name != "multiply" for t in m):
+        return None
+    (x0, cb0), (x1, sb0), (x0b, sb1), (x1b, cb1) = (t.operands for t in m)
+    if x0 != x0b or x1 != x1b or cb0 != cb1 or sb0 != sb1:
+        return None
+    cn, cbc = _bcast(cb0, d, [1, 3])
+    sn, sbc = _bcast(sb0, d, [1, 3])
+    if cbc is None or sbc is None:
+        return None
+    extra = []
+
+    def table_const(name):
+        op_ = d(name)
+        if op_ is not None and op_.name == "convert":           # fp32 tables converted to the storage dtype
+            extra.append(op_)
+            op_ = d(op_.operands[0])
+        return op_
+
+    cconst, sconst = table_const(cn), table_const(sn)
+    if cconst is None or sconst is None or cconst.name != "constant" or sconst.name != "constant":
+        return None
+    e0, e1 = d(x0), d(x1)
+    if e0 is None or e1 is None or e0.name != "reshape" or e1.name != "reshape":
+        return None
+    s0, s1 = d(e0.operands[0]), d(e1.operands[0])
+    if s0 is None or s1 is None or s0.name != "slice" or s1.name != "slice" or s0.operands != s1.operands:
+        return None
+    xr = d(s0.operands[0])
+    if xr is None or xr.name != "reshape" or len(xr.types[0].shape) != 5 or xr.types[0].shape[4] != 2:
+        return None
+    B, S, h, P, _ = xr.types[0].shape
+    if s0.attrs["start"] != [0, 0, 0, 0, 0] or s0.attrs["limit"] != [B, S, h, P, 1] or s1.attrs["start"] != [0, 0, 0, 0, 1] or \
+            s1.attrs["limit"] != [B, S, h, P, 2]:
+        return None
+    c, s_ = np.asarray(cconst.attrs["value"], dtype=np.float64), np.asarray(sconst.attrs["value"], dtype=np.float64)
+    if c.shape != (S, P) or s_.shape != (S, P) or np.max(np.abs(c * c + s_ * s_ - 1.0)) > 2e-2:
+        return None
+    if tuple(op.types[0].shape) != (B, S, h * 2 * P):
+        return None
+    table = np.stack([c, s_], axis=2).astype(np.float32)                      # [S, P, 2]
+    # the converts of the tables may serve other clusters too: they stay until nothing uses them
+    interior = [op, cat, r0, r1, o0, o1] + m + [cbc, sbc, e0, e1, s0, s1, xr]
+    return "rope_rows", Op("emi.rope_rows", op.results, [xr.operands[0]], {"table": table, "heads": h}, op.types), interior
+
+
+def _match_attention(op, d, tb):
+    # reshape(transpose(dot(P, Vh))) with P = softmax over keys of select(mask, dot(Qh, Kh) / c, -inf),
+    # Xh = transpose(reshape(X, [B, S, h, d]), [0, 2, 1, 3]); mask constant, lower triangular or all true
+    if op.name != "reshape" or len(op.types[0].shape) != 3:
+        return None
+    tr = d(op.operands[0])
+    if tr is None or tr.name != "transpose" or list(tr.attrs["perm"]) != [0, 2, 1, 3]:
+        return None
+    pv = d(tr.operands[0])
+    if pv is None or pv.name != "dot_general" or pv.attrs["batch_a"] != [0, 1] or pv.attrs["batch_b"] != [0, 1] or \
+            pv.attrs["contract_a"] != [3] or pv.attrs["contract_b"] != [2]:
+        return None
+    p, vh = d(pv.operands[0]), d(pv.operands[1])
+    if p is None or p.name != "divide":
+        return None
+    e = d(p.operands[0])
+    sum_name, sbc = _bcast(p.operands[1], d, [0, 1, 2])
+    sm = d(sum_name) if sbc is not None else None
+    if e is None or e.name != "exponential" or sm is None or sm.name != "reduce" or sm.attrs["body"] != "add" or \
+            list(sm.attrs["dims"]) != [3] or sm.operands[0] != p.operands[0]:
+        return None
+    sub = d(e.operands[0])
+    if sub is None or sub.name != "subtract":
+        return None
+    s_name = sub.operands[0]
+    max_name, mbc = _bcast(sub.operands[1], d, [0, 1, 2])
+    mx = d(max_name) if mbc is not None else None
+    if mx is None or mx.name != "reduce" or mx.attrs["body"] != "maximum" or list(mx.attrs["dims"]) != [3] or mx.operands[0] != s_name:
+        return None
+    interior = [op, tr, pv, p, e, sbc, sm, sub, mbc, mx]
+    s = d(s_name)
+    causal = False
+    if s is not None and s.name == "select":
+        fill_name, fill_bc = tb(s.operands[2])
+        mask = d(s.operands[0])
+        mask_bc = None
+        if mask is not None and mask.name == "broadcast_in_dim" and list(mask.attrs["dims"]) == [2, 3]:
+            mask_bc, mask = mask, d(mask.operands[0])                   # a [S, S] mask shared by every batch and head
+        if mask is None or mask.name != "constant" or _splat(d(fill_name)) != -np.inf:
+            return None
+        interior += [o for o in (fill_bc, mask_bc) if o is not None]
+        mv = np.asarray(mask.attrs["value"])
+        S = mv.shape[-1]
+        m2 = mv.reshape(-1, S, S)
+        if not np.all(m2 == m2[0]):
+            return None
+        if np.array_equal(m2[0], np.tril(np.ones((S, S), dtype=bool))):
+            causal = True
+        elif not np.all(m2[0]):
+            return None
+        interior.append(s)
+        s = d(s.operands[1])
+    if s is None or s.name not in ("divide", "multiply"):
+        return None
+    c_name, cbc = tb(s.operands[1])
+    c = _splat(d(c_name))
+    qk = d(s.operands[0])
+    if c is None or qk is None or qk.name != "dot_general" or qk.attrs["batch_a"] != [0, 1] or qk.attrs["batch_b"] != [0, 1] or \
+            qk.attrs["contract_a"] != [3] or qk.attrs["contract_b"] != [3]:
+        return None
+    scale = 1.0 / c if s.name == "divide" else c
+    interior += [s, qk] + ([cbc] if cbc is not None else [])
+    srcs = []
+    for hname in (qk.operands[0], qk.operands[1], pv.operands[1]):
+        ht = d(hname)
+        if ht is None or ht.name != "transpose" or list(ht.attrs["perm"]) != [0, 2, 1, 3]:
+            return None
+        rs = d(ht.operands[0])
+        if rs is None or rs.name != "reshape" or len(rs.types[0].shape) != 4:
+            return None
+        interior += [ht, rs]
+        srcs.append(rs.operands[0])
+    B, h, S, hd = qk.types[0].shape[0], qk.types[0].shape[1], qk.types[0].shape[2], d(qk.operands[0]).types[0].shape[3]
+    if tuple(op.types[0].shape) != (B, S, h * hd):
+        return None
+    new = Op("emi.attention", op.results, srcs, {"scale": scale, "heads": h, "causal": causal}, op.types)
+    return "attention", new, interior
+
+
 def _match_rope(op, d, tb):
     # root: reshape(dot_general(R [P,2,2] constant, reshape(x, [P,2]), batch [0]x[0], contract [2]x[1])) -> [2P]
     if op.name != "reshape" or len(op.types[0].shape) != 1:
@@ -954,8 +1192,7 @@ class Executable:
         for f in self.funcs.values():
             fold_constants(f)
             if fuse:
-                kinds = fuse if isinstance(fuse, (tuple, list)) else \
-                    ("rmsnorm", "swiglu", "rope", "softmax_dot", "attention_step")
+                kinds = fuse if isinstance(fuse, (tuple, list)) else ALL_KINDS
                 for k, v in fuse_clusters(f, kinds).items():
                     self.fused[k] = self.fused.get(k, 0) + v
         self._consts = {}
@@ -974,7 +1211,7 @@ class Executable:
         hit = self._consts.get(key)
         if hit is None:
             ty = op.types[0]
-            host = torch.from_numpy(np.array(op.attrs["value"]).reshape(-1)).reshape(ty.shape)
+            host = torch.from_numpy(np.ascontiguousarray(op.attrs["value"]).reshape(-1)).reshape(ty.shape)
             hit = self._consts[key] = host.to(TORCH_DTYPES[ty.dtype]).to(device)       # trace-time constant upload
         return hit
 
@@ -1021,7 +1258,8 @@ class Executable:
             dt = TORCH_DTYPES[op.types[0].dtype]
             return [xs[0] if xs[0].dtype == dt else H.convert(xs[0], dt)]
         if n == "reshape":
-            return [ops.reshape(H._contig(xs[0]), op.types[0].shape)]
+            x = xs[0] if xs[0].is_contiguous() else H.unary_copy(xs[0])      # a tracked copy: cotangents reach the view
+            return [ops.reshape(x, op.types[0].shape)]
         if n == "transpose":
             return [H.transpose(xs[0], op.attrs["perm"])]
         if n == "broadcast_in_dim":
@@ -1040,7 +1278,11 @@ class Executable:
             return [H.slice_(xs[0], op.attrs["start"], op.attrs["limit"], op.attrs["stride"])]
         if n == "concatenate":
             return [H.concatenate(xs, op.attrs["dim"])]
+        if n == "iota":
+            raise NotImplementedError("stablehlo.iota of type %r (integer iotas feeding masks are folded at parse time)" % op.types[0])
         if n == "compare":
+            if not xs[0].is_floating_point():
+                raise NotImplementedError("stablehlo.compare on integer operands that are not trace-time constants")
             return [H.compare(op.attrs["direction"], xs[0], xs[1])]
         if n == "select":
             return [H.select(xs[0], xs[1], xs[2])]
@@ -1052,6 +1294,18 @@ class Executable:
             return self.run(xs, op.attrs["callee"])
         if n == "custom_call":
             return self._custom_call(op, xs)
+        if n == "emi.rmsnorm_rows":
+            x, w = _packed(xs[0]), _packed(xs[1])
+            return [ops.rmsnorm(x, w, op.attrs["eps"])]
+        if n == "emi.rope_rows":
+            key = (id(op), "table", str(device))
+            table = self._consts.get(key)
+            if table is None:
+                table = self._consts[key] = torch.from_numpy(op.attrs["table"]).to(device)
+            return [ops.rope_rows(_packed(xs[0]), op.attrs["heads"], table)]
+        if n == "emi.attention":
+            q, k, v = (_packed(t) for t in xs)
+            return [ops.attention(q, k, v, op.attrs["heads"], op.attrs["scale"], causal=op.attrs["causal"], layout="bshd")]
         if n == "emi.rmsnorm":
             x, w = _packed(xs[0]), _packed(xs[1])
             return [ops.reshape(ops.rmsnorm(ops.reshape(x, (1, x.shape[0])), w, op.attrs["eps"]), tuple(x.shape))]

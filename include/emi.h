@@ -248,7 +248,7 @@ int emi_select(emi_stream_t stream, const void* mask, const void* a, const void*
  * (zero in_strides), slice (offset and strides; Slice rule
  * StableHLOAutoDiffOpInterfaceImpl.cpp:1586-1620) and one operand of
  * concatenate (Concatenate rule :2015-2059).  rank <= 8; strides and offsets in
- * elements of elem_bytes (2, 4 or 8) bytes; dims / strides are HOST arrays.
+ * elements of elem_bytes (1, 2, 4 or 8) bytes; dims / strides are HOST arrays.
  * The boxes must not overlap. */
 int emi_strided_copy(emi_stream_t stream, const void* in, void* out, int rank, const int64_t* dims,
                      const int64_t* in_strides, int64_t in_offset, const int64_t* out_strides,
