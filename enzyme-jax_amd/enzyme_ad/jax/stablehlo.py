@@ -1194,7 +1194,8 @@ class Executable:
             if fuse:
                 kinds = fuse if isinstance(fuse, (tuple, list)) else ALL_KINDS
                 for k, v in fuse_clusters(f, kinds).items():
-                    self.fused[k] = self.fused.get(k, 0) + v
+                    if v:
+                        self.fused[k] = self.fused.get(k, 0) + v
         self._consts = {}
 
     def signature(self, fn="main"):
