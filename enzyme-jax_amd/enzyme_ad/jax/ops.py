@@ -462,7 +462,7 @@ def attention_raw(q, k, v, n_heads, scale, causal, strides):
     return o, lse, (B, S, d, sb, sh, ss)
 
 
-def attention(q, k, v, n_heads, scale=None, causal=True, layout="bshd"):
+def attention(q, k, v, n_heads, scale=None, causal=True, layout="bshd", return_lse=False):
     """Causal softmax attention (test/llama.py:178-206).  layout "bshd": operands
     are [B, S, n_heads*head_dim] (token-major, as the projections produce them);
     layout "bhsd": [B, n_heads, S, head_dim]."""
@@ -490,7 +490,7 @@ def attention(q, k, v, n_heads, scale=None, causal=True, layout="bshd"):
         N.check(N.lib().emi_attn_jvp(_stream(), _p(q), _p(k), _p(v), _p(lse), _p(tans[0]), _p(tans[1]), _p(tans[2]), _p(to),
                                      B, n_heads, S, d, sb, sh, ss, float(scale), int(causal), _code(q)))
         _set_tan(o, to)
-    return o
+    return (o, lse) if return_lse else o
 
 
 def reshape(x, shape):

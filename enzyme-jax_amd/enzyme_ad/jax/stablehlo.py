@@ -1344,11 +1344,25 @@ def _custom_call_impl(self, op, xs):
     if target == "emi_add":
         return [ops.add(_packed(xs[0]), _packed(xs[1]))]
     if target == "emi_rope":
-        x, table = _packed(xs[0]), xs[1]
-        if x.dim() != 4 or x.shape[1] != 1 or tuple(table.shape) != (1, x.shape[3] // 2, 2):
-            raise NotImplementedError("custom call emi_rope is run for one position per call (seq = 1)")
-        y = ops.rotate_pairs(ops.reshape(x, (-1, x.shape[3])), table.reshape(-1, 2).contiguous(), bool(cfg.get("inverse", False)))
+        x, table = _packed(xs[0]), _packed(xs[1])
+        if x.dim() != 4 or tuple(table.shape) != (x.shape[1], x.shape[3] // 2, 2):
+            raise ValueError("custom call emi_rope: x %s, table %s" % (tuple(x.shape), tuple(table.shape)))
+        B_, S_, h, d = x.shape
+        y = ops.rope_rows(ops.reshape(x, (B_, S_, h * d)), h, table, bool(cfg.get("inverse", False)))
         return [ops.reshape(y, tuple(x.shape))]
+    if target == "emi_attn_fwd":
+        q, k, v = (_packed(t) for t in xs)
+        if q.dim() != 4:
+            raise ValueError("custom call emi_attn_fwd: rank-4 operands wanted")
+        if cfg.get("bshd", False):
+            B_, S_, h, d = q.shape
+            flat = lambda t: ops.reshape(t, (B_, S_, h * d))
+            o, lse = ops.attention(flat(q), flat(k), flat(v), h, cfg["scale"], causal=bool(cfg.get("causal", True)), layout="bshd",
+                                   return_lse=True)
+            o = ops.reshape(o, (B_, S_, h, d))
+        else:
+            o, lse = ops.attention(q, k, v, q.shape[1], cfg["scale"], causal=bool(cfg.get("causal", True)), layout="bhsd", return_lse=True)
+        return [o, lse, None][:len(op.results)]
     if target == "emi_attn_step_fwd":
         q, k, v = (_packed(t) for t in xs)
         if q.dim() != 3 or q.shape[0] != 1 or k.dim() != 4:
@@ -1383,6 +1397,25 @@ def _custom_call_impl(self, op, xs):
         N.check(lib.emi_attn_step_jvp(st, P(q), P(k), P(v), P(o), P(lse), P(tq), P(tk), P(tv), P(to), P(ws), nbytes, 1, h, S, d,
                                       h * d, d, S * h * d, d, h * d, float(cfg["scale"]), ops._code(q)))
         return [to, None][:len(op.results)]
+    if target in ("emi_attn_bwd", "emi_attn_jvp"):
+        bshd = bool(cfg.get("bshd", False))
+        q = _packed(xs[0])
+        B_, S_, h, d = (q.shape if bshd else (q.shape[0], q.shape[2], q.shape[1], q.shape[3]))
+        sb, sh, ss = (S_ * h * d, d, h * d) if bshd else (h * S_ * d, S_ * d, d)
+        causal = int(bool(cfg.get("causal", True)))
+        if target == "emi_attn_bwd":
+            q, k, v, o, lse, do = (_packed(t) for t in xs)
+            dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+            nbytes = lib.emi_attn_bwd_workspace_bytes(B_, h, S_, d)
+            ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
+            N.check(lib.emi_attn_bwd(st, P(q), P(k), P(v), P(o), P(lse), P(do), P(dq), P(dk), P(dv), P(ws), nbytes, B_, h, S_, d,
+                                     sb, sh, ss, float(cfg["scale"]), causal, ops._code(q)))
+            return [dq, dk, dv, None][:len(op.results)]
+        q, k, v, lse, tq, tk, tv = (_packed(t) for t in xs)
+        to = torch.empty_like(q)
+        N.check(lib.emi_attn_jvp(st, P(q), P(k), P(v), P(lse), P(tq), P(tk), P(tv), P(to), B_, h, S_, d, sb, sh, ss,
+                                 float(cfg["scale"]), causal, ops._code(q)))
+        return [to]
     if target == "emi_rmsnorm_bwd":
         x, w, dy = (_packed(t) for t in xs[:3])
         rows, dim = x.numel() // x.shape[-1], x.shape[-1]
@@ -1442,6 +1475,13 @@ def _dense_text(value, ty):
     one = (lambda x: _fmt_float(x)) if is_float else (lambda x: str(bool(x)).lower() if ty.dtype == "i1" else str(int(x)))
     if flat.size and np.all(flat == flat[0]) and not (is_float and np.isinf(flat[0]) and ty.dtype != "f32"):
         return one(flat[0])
+
+    if flat.size > 1024 and ty.dtype in ("f32", "bf16"):           # large tables: raw little-endian bytes as hex
+        if ty.dtype == "bf16":
+            raw = torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(torch.bfloat16).view(torch.int16).numpy().astype("<i2").tobytes()
+        else:
+            raw = np.ascontiguousarray(a, dtype="<f4").tobytes()
+        return '"0x%s"' % raw.hex().upper()
 
     def lit(x):
         return "[" + ", ".join(lit(y) for y in x) + "]" if x.ndim else one(x)

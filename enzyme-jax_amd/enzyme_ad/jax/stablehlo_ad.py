@@ -101,6 +101,24 @@ def lower_fused(func):
             x4 = b.reshape(op.operands[0], (1, 1, 1, 2 * P))
             y4, = b.custom_call("emi_rope", [x4, tab], {"inverse": False}, [T[x4]])
             b.ops.append(Op("reshape", op.results, [y4], {}, op.types))
+        elif n == "emi.rmsnorm_rows":
+            b.ops.append(Op("custom_call", op.results, list(op.operands), {"target": "emi_rmsnorm_fwd", "config": {"eps": op.attrs["eps"]}},
+                            op.types))
+        elif n == "emi.rope_rows":
+            B_, S_, D_ = ty.shape
+            h = op.attrs["heads"]
+            tab = b.emit("constant", [], {"value": np.asarray(op.attrs["table"], dtype=np.float32)},
+                         TensorType(op.attrs["table"].shape, "f32"))
+            x4 = b.reshape(op.operands[0], (B_, S_, h, D_ // h))
+            y4, = b.custom_call("emi_rope", [x4, tab], {"inverse": False}, [T[x4]])
+            b.ops.append(Op("reshape", op.results, [y4], {}, op.types))
+        elif n == "emi.attention":
+            B_, S_, D_ = ty.shape
+            h = op.attrs["heads"]
+            q4, k4, v4 = (b.reshape(o_, (B_, S_, h, D_ // h)) for o_ in op.operands)
+            o4, _ = b.custom_call("emi_attn_fwd", [q4, k4, v4], {"scale": op.attrs["scale"], "causal": bool(op.attrs["causal"]), "bshd": True},
+                                  [T[q4], TensorType((B_, h, S_), "f32")])
+            b.ops.append(Op("reshape", op.results, [o4], {}, op.types))
         elif n in ("emi.softmax_dot", "emi.attention_step"):
             q, k, v = op.operands
             h = op.attrs.get("heads", 1)
@@ -451,6 +469,11 @@ def forward_function(func, name=None, arg_active=None):
             elif target == "emi_rope":
                 if ts[0] is not None:
                     tan[r], = b.custom_call("emi_rope", [ts[0], xs[1]], dict(cfg), [T[r]])
+            elif target == "emi_attn_fwd":
+                o, lse = op.results[:2]
+                tan[o], = b.custom_call("emi_attn_jvp", [xs[0], xs[1], xs[2], lse, tz(xs[0]), tz(xs[1]), tz(xs[2])],
+                                        {"scale": cfg["scale"], "causal": bool(cfg.get("causal", True)), "bshd": bool(cfg.get("bshd", False))},
+                                        [T[o]])
             elif target == "emi_attn_step_fwd":
                 o, lse, ws = op.results
                 tan[o], _ = b.custom_call("emi_attn_step_jvp", [xs[0], xs[1], xs[2], o, lse, tz(xs[0]), tz(xs[1]), tz(xs[2])],
@@ -526,6 +549,24 @@ def _reverse_custom_call(b, op, cs, accum):
     elif target == "emi_rope":
         g, = b.custom_call("emi_rope", [c, xs[1]], {"inverse": not cfg.get("inverse", False)}, [T[xs[0]]])
         accum(xs[0], g)
+    elif target == "emi_attn_fwd":
+        if any(x is not None for x in cs[1:]):
+            raise NotImplementedError("cotangents of the log-sum-exp or workspace results of emi_attn_fwd")
+        if c is None:
+            return
+        from . import _native as N
+        q, k, v = xs
+        o, lse = op.results[:2]
+        bshd = bool(cfg.get("bshd", False))
+        qs = T[q].shape
+        B_, S_, h, d = (qs[0], qs[1], qs[2], qs[3]) if bshd else (qs[0], qs[2], qs[1], qs[3])
+        nbytes = int(N.lib().emi_attn_bwd_workspace_bytes(B_, h, S_, d))
+        dq, dk, dv, _ = b.custom_call("emi_attn_bwd", [q, k, v, o, lse, c],
+                                      {"scale": cfg["scale"], "causal": bool(cfg.get("causal", True)), "bshd": bshd},
+                                      [T[q], T[k], T[v], TensorType((nbytes,), "i8")])
+        accum(q, dq)
+        accum(k, dk)
+        accum(v, dv)
     elif target == "emi_attn_step_fwd":
         if cs[1] is not None or (len(cs) > 2 and cs[2] is not None):
             raise NotImplementedError("cotangents of the log-sum-exp or workspace results of emi_attn_step_fwd")

@@ -73,3 +73,41 @@ def test_layer_text_forward_mode_adjoint_identity():
     lhs = float(np.sum(host(ty) * host(dy)))
     rhs = sum(float(np.sum(host(g) * host(t))) for g, t in zip(grads, tans))
     assert abs(lhs - rhs) <= 1e-4 * max(abs(lhs), abs(rhs)), (lhs, rhs)
+
+
+def test_layer_text_lowered_and_symbolic_programs():
+    """optimize_module's three programs for the batched layer (clusters as emi_rmsnorm_fwd /
+    emi_rope / emi_attn_fwd / emi_swiglu_fwd custom calls; the reverse program with emi_attn_bwd
+    & co.; the forward program with emi_attn_jvp & co.) through hlo_call against the tape."""
+    from enzyme_ad.jax import hlo_call, jvp, optimize_module, stablehlo_ad, vjp
+    from enzyme_ad.jax import primitives as P
+
+    cfg = {"dim": 256, "hidden_dim": 704, "n_heads": 2}
+    for dt, tol in (("f32", 1e-5), ("bf16", 2e-2)):
+        text, order = llama_layer_text(cfg, 2, 70, dt)
+        rng = np.random.Generator(np.random.PCG64(3))
+        shapes = [(2, 70, 256), (256,), (256, 256), (256, 256), (256, 256), (256, 256), (256,), (704, 256), (256, 704), (704, 256)]
+        args = [dev(rng.uniform(0.5, 1.5, s) if len(s) == 1 else rng.standard_normal(s) * (1.0 if len(s) == 3 else 0.05), dt)[0] for s in shapes]
+        tans = [dev(rng.standard_normal(s) * (1.0 if len(s) != 2 else 0.05), dt)[0] for s in shapes]
+        dy = dev(rng.standard_normal(shapes[0]), dt)[0]
+        fn = lambda *a: hlo_call(*a, source=text)[0]
+        y, f_vjp = vjp(fn, *args)
+        grads = f_vjp(dy)
+        low = optimize_module(text)
+        assert low.count("stablehlo.custom_call") == 6 and "stablehlo.exponential" not in low
+        y_low = hlo_call(*args, source=low)[0]
+        assert torch.equal(y_low, y)
+        fwd_pipe = P.forward_mode_pipeline(P.JaXPipeline(), [True] * len(args), 1)
+        rev = optimize_module(text, P.reverse_mode_pipeline(fwd_pipe, [True]).pass_pipeline())
+        assert rev.count("@emi_attn_bwd") == 1 and rev.count("@emi_rmsnorm_bwd") == 2
+        sym = hlo_call(*(args + [dy]), source=rev)
+        for name, g, t in zip(order, sym, grads):
+            e = float((g.float() - t.float()).abs().max() / t.float().abs().max())
+            assert e <= tol, "reverse program, %s: %.3e" % (name, e)
+        fwd = optimize_module(text, fwd_pipe.pass_pipeline())
+        assert fwd.count("@emi_attn_jvp") == 1
+        flat = [v for a, t in zip(args, tans) for v in (a, t)]
+        y_f, ty_f = hlo_call(*flat, source=fwd)
+        _, ty = jvp(fn, tuple(args), tuple(tans))
+        e = float((ty_f.float() - ty.float()).abs().max() / ty.float().abs().max())
+        assert torch.equal(y_f, y) and e <= tol, "forward program: %.3e" % e
