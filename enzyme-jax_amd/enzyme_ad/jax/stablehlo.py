@@ -685,7 +685,7 @@ def _drop_dead(func):
     func.ops = list(reversed(kept))
 
 
-ALL_KINDS = ("rmsnorm", "swiglu", "rope", "softmax_dot", "attention_step", "rmsnorm_rows", "rope_rows", "attention")
+ALL_KINDS = ("rmsnorm", "swiglu", "rope", "softmax_dot", "attention_step", "rmsnorm_rows", "rope_rows", "attention", "linear")
 
 
 def fuse_clusters(func, kinds=ALL_KINDS):
@@ -703,11 +703,12 @@ def fuse_clusters(func, kinds=ALL_KINDS):
     A cluster is fused only when none of its interior values is used outside it.  Returns
     the number of clusters fused per kind."""
     counts = {"rmsnorm": 0, "swiglu": 0, "rope": 0, "softmax_dot": 0, "attention_step": 0, "rmsnorm_rows": 0, "rope_rows": 0,
-              "attention": 0}
+              "attention": 0, "linear": 0}
     matchers = [m for k, m in (("rmsnorm", _match_rmsnorm), ("swiglu", _match_swiglu), ("rope", _match_rope),
                                ("softmax_dot", _match_softmax_dot), ("attention_step", _match_heads),
                                ("rmsnorm_rows", _match_rmsnorm_rows), ("rope_rows", _match_rope_rows),
                                ("attention", _match_attention)) if k in kinds]
+    want_linear = "linear" in kinds
     changed = True
     while changed:
         changed = False
@@ -754,6 +755,31 @@ def fuse_clusters(func, kinds=ALL_KINDS):
             counts[kind] += 1
             changed = True
             break
+    if want_linear:
+        changed = True
+        while changed:
+            changed = False
+            defs = {r: op for op in func.ops for r in op.results}
+            use = _users(func)
+            rets = set(o for op in func.ops if op.name == "return" for o in op.operands)
+            types = {a: t for a, t in func.args}
+            for op in func.ops:
+                for r, t in zip(op.results, op.types):
+                    types[r] = t
+            for op in func.ops:
+                m = _match_linear(op, defs.get, None, types.get)
+                if m is None:
+                    continue
+                kind, new_op, interior = m
+                inner = [o for o in interior if o is not op]
+                if any(r in rets or any(u is not op for u in use.get(r, [])) for o in inner for r in o.results):
+                    continue
+                dead = set(id(o) for o in inner)
+                func.ops = [new_op if o is op else o for o in func.ops if id(o) not in dead]
+                if not inner:
+                    counts["linear"] += 1
+                changed = True
+                break
     _drop_dead(func)
     return counts
 
@@ -1112,6 +1138,40 @@ def _match_attention(op, d, tb):
     return "attention", new, interior
 
 
+def _linear_form(op, types):
+    """(x, w) when dot_general `op` is y = x . w^T for a weight w [out, in]: either x[..., in]
+    contracted over its last index with index 1 of w (batched form), or w contracted over
+    index 1 with a vector x[in] (the step's `w @ x`, test/llama.py:149-157)."""
+    if op is None or op.name != "dot_general" or op.attrs["batch_a"] or len(op.attrs["contract_a"]) != 1:
+        return None
+    a, b_ = op.operands
+    ta, tb_ = types(a), types(b_)
+    if ta is None or tb_ is None or ta.dtype not in ("f32", "bf16"):
+        return None
+    ca, cb = op.attrs["contract_a"][0], op.attrs["contract_b"][0]
+    if len(tb_.shape) == 2 and cb == 1 and ca == len(ta.shape) - 1 and len(ta.shape) >= 1:
+        return a, b_
+    if len(ta.shape) == 2 and ca == 1 and len(tb_.shape) == 1 and cb == 0:
+        return b_, a
+    return None
+
+
+def _match_linear(op, d, tb, types=None):
+    # root: add(r, dot) with the product used only here -> projection with the residual added in
+    # the GEMM epilogue (test/llama.py:211-215,231-233); or a bare projection
+    if op.name == "add":
+        for di in (0, 1):
+            inner = d(op.operands[di])
+            if inner is not None and inner.name == "emi.linear" and len(inner.operands) == 2:
+                new = Op("emi.linear", op.results, list(inner.operands) + [op.operands[1 - di]], {}, op.types)
+                return "linear", new, [op, inner]
+        return None
+    lf = _linear_form(op, types)
+    if lf is None:
+        return None
+    return "linear", Op("emi.linear", op.results, [lf[0], lf[1]], {}, op.types), [op]
+
+
 def _match_rope(op, d, tb):
     # root: reshape(dot_general(R [P,2,2] constant, reshape(x, [P,2]), batch [0]x[0], contract [2]x[1])) -> [2P]
     if op.name != "reshape" or len(op.types[0].shape) != 1:
@@ -1295,6 +1355,10 @@ class Executable:
             return self.run(xs, op.attrs["callee"])
         if n == "custom_call":
             return self._custom_call(op, xs)
+        if n == "emi.linear":
+            x, w = _packed(xs[0]), _packed(xs[1])
+            r = _packed(xs[2]) if len(xs) > 2 else None
+            return [ops.matmul_nt(x, w, residual=r)]
         if n == "emi.rmsnorm_rows":
             x, w = _packed(xs[0]), _packed(xs[1])
             return [ops.rmsnorm(x, w, op.attrs["eps"])]
@@ -1341,6 +1405,13 @@ def _custom_call_impl(self, op, xs):
         return [ops.reshape(y, tuple(x.shape))]
     if target == "emi_swiglu_fwd":
         return [ops.swiglu(_packed(xs[0]), _packed(xs[1]))]
+    if target == "emi_gemm":
+        a, b_ = _packed(xs[0]), _packed(xs[1])
+        r = _packed(xs[2]) if len(xs) > 2 else None
+        ta, tb_ = bool(cfg.get("trans_a", False)), bool(cfg.get("trans_b", False))
+        if not ta and tb_:
+            return [ops.matmul_nt(a, b_, residual=r)]                   # the projection form: differentiable on the tape
+        return [ops.gemm(a, b_, ta, tb_, r)]                            # the forms derivative programs use
     if target == "emi_add":
         return [ops.add(_packed(xs[0]), _packed(xs[1]))]
     if target == "emi_rope":

@@ -101,6 +101,13 @@ def lower_fused(func):
             x4 = b.reshape(op.operands[0], (1, 1, 1, 2 * P))
             y4, = b.custom_call("emi_rope", [x4, tab], {"inverse": False}, [T[x4]])
             b.ops.append(Op("reshape", op.results, [y4], {}, op.types))
+        elif n == "emi.linear":
+            x, w = op.operands[:2]
+            K, Nn = T[x].shape[-1], T[w].shape[0]
+            rows = int(np.prod(T[x].shape[:-1])) if len(T[x].shape) > 1 else 1
+            operands = [b.reshape(x, (rows, K)), w] + [b.reshape(r_, (rows, Nn)) for r_ in op.operands[2:]]
+            c2, = b.custom_call("emi_gemm", operands, {"trans_a": False, "trans_b": True}, [TensorType((rows, Nn), ty.dtype)])
+            b.ops.append(Op("reshape", op.results, [c2], {}, op.types))
         elif n == "emi.rmsnorm_rows":
             b.ops.append(Op("custom_call", op.results, list(op.operands), {"target": "emi_rmsnorm_fwd", "config": {"eps": op.attrs["eps"]}},
                             op.types))
@@ -469,6 +476,15 @@ def forward_function(func, name=None, arg_active=None):
             elif target == "emi_rope":
                 if ts[0] is not None:
                     tan[r], = b.custom_call("emi_rope", [ts[0], xs[1]], dict(cfg), [T[r]])
+            elif target == "emi_gemm":
+                flags = {"trans_a": bool(cfg.get("trans_a", False)), "trans_b": bool(cfg.get("trans_b", False))}
+                acc_t = ts[2] if len(xs) > 2 else None
+                if ts[0] is not None:
+                    acc_t, = b.custom_call("emi_gemm", [ts[0], xs[1]] + ([acc_t] if acc_t is not None else []), flags, [T[r]])
+                if ts[1] is not None:
+                    acc_t, = b.custom_call("emi_gemm", [xs[0], ts[1]] + ([acc_t] if acc_t is not None else []), flags, [T[r]])
+                if acc_t is not None:
+                    tan[r] = acc_t
             elif target == "emi_attn_fwd":
                 o, lse = op.results[:2]
                 tan[o], = b.custom_call("emi_attn_jvp", [xs[0], xs[1], xs[2], lse, tz(xs[0]), tz(xs[1]), tz(xs[2])],
@@ -549,6 +565,15 @@ def _reverse_custom_call(b, op, cs, accum):
     elif target == "emi_rope":
         g, = b.custom_call("emi_rope", [c, xs[1]], {"inverse": not cfg.get("inverse", False)}, [T[xs[0]]])
         accum(xs[0], g)
+    elif target == "emi_gemm":
+        # C = op(A) . op(B) [+ R]: the DotGeneral rule (HLODerivatives.td:1166-1178) in the GEMM's own flags
+        ta, tb_ = bool(cfg.get("trans_a", False)), bool(cfg.get("trans_b", False))
+        A, Bm = xs[0], xs[1]
+        gemm = lambda p, q, fa, fb, ty: b.custom_call("emi_gemm", [p, q], {"trans_a": fa, "trans_b": fb}, [ty])[0]
+        accum(A, gemm(c, Bm, False, not tb_, T[A]) if not ta else gemm(Bm, c, tb_, True, T[A]))
+        accum(Bm, gemm(A, c, not ta, False, T[Bm]) if not tb_ else gemm(c, A, True, ta, T[Bm]))
+        if len(xs) > 2:
+            accum(xs[2], c)
     elif target == "emi_attn_fwd":
         if any(x is not None for x in cs[1:]):
             raise NotImplementedError("cotangents of the log-sum-exp or workspace results of emi_attn_fwd")

@@ -55,7 +55,8 @@ def test_llama_step_text_stories15m_fp32(pos, zero_cache, fuse):
     exe, errs = _run(STORIES, pos, "f32", 40 + pos, zero_cache, 0.05, fuse)
     if fuse:
         L_ = STORIES["n_layers"]
-        assert exe.fused == {"rmsnorm": 2 * L_ + 1, "swiglu": L_, "rope": 2 * L_, "softmax_dot": 6 * L_, "attention_step": L_}
+        assert exe.fused == {"rmsnorm": 2 * L_ + 1, "swiglu": L_, "rope": 2 * L_, "softmax_dot": 6 * L_, "attention_step": L_,
+                             "linear": 7 * L_}
     else:
         assert exe.fused == {}
     print("llama text fuse=%s max rel errors" % fuse, {k: "%.2e" % v for k, v in errs.items()}, flush=True)
@@ -97,7 +98,7 @@ def test_optimized_module_runs_and_matches_the_fused_run():
     cfg = dict(STORIES, n_layers=2)
     text, order = llama_step_text(cfg, 5, "f32")
     low = optimize_module(text)
-    assert low.count("stablehlo.custom_call") == 2 * 6 + 1 and "stablehlo.exponential" not in low
+    assert low.count("stablehlo.custom_call") == 2 * (6 + 7) + 1 and "stablehlo.exponential" not in low
     (x, wd, kc, vc, dy), (xr, wr, kcr, vcr, dyr) = _inputs(cfg, 5, "f32", 88, False, 0.05)
     args = [x] + [wd[k] for k in WEIGHT_ORDER] + [kc, vc]
     outs = []

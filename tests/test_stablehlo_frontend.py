@@ -73,11 +73,13 @@ def test_llama_text_clusters_are_matched():
     text, order = llama_step_text(CFG, pos=3)
     exe = S.Executable(text)
     L = CFG["n_layers"]
-    assert exe.fused == {"rmsnorm": 2 * L + 1, "swiglu": L, "rope": 2 * L, "softmax_dot": 6 * L, "attention_step": L}
+    assert exe.fused == {"rmsnorm": 2 * L + 1, "swiglu": L, "rope": 2 * L, "softmax_dot": 6 * L, "attention_step": L,
+                         "linear": 7 * L}
     left = Counter(o.name for o in exe.funcs["main"].ops)
-    # what stays generic: weight slices / reshapes, the seven projections per layer, the two
-    # cache appends per layer, the two residual adds per layer
-    assert left["dot_general"] == 7 * L and left["concatenate"] == 2 * L and left["add"] == 2 * L
+    # what stays generic: weight slices / reshapes and the two cache appends per layer; the seven
+    # projections per layer are emi.linear, two of them with the residual add folded in
+    assert left["emi.linear"] == 7 * L and left["concatenate"] == 2 * L and "add" not in left and "dot_general" not in left
+    assert sum(len(o.operands) == 3 for o in exe.funcs["main"].ops if o.name == "emi.linear") == 2 * L
     assert not any(k in left for k in ("exponential", "reduce", "sqrt", "divide", "multiply", "broadcast_in_dim", "constant"))
     att = [o for o in exe.funcs["main"].ops if o.name == "emi.attention_step"][0]
     assert att.attrs["heads"] == 6 and att.attrs["rows"] == 4 and abs(att.attrs["scale"] - 1 / np.sqrt(48)) < 1e-7
@@ -125,7 +127,8 @@ def test_optimize_module_prints_typed_ffi_custom_calls():
     text, order = llama_step_text(dict(CFG, n_layers=1), pos=3)
     low = ej.optimize_module(text)
     calls = [l.strip() for l in low.splitlines() if "stablehlo.custom_call" in l]
-    assert Counter(l.split("@")[1].split("(")[0] for l in calls) == {"emi_rmsnorm_fwd": 3, "emi_rope": 2, "emi_attn_step_fwd": 1, "emi_swiglu_fwd": 1}
+    assert Counter(l.split("@")[1].split("(")[0] for l in calls) == {"emi_rmsnorm_fwd": 3, "emi_rope": 2, "emi_attn_step_fwd": 1, "emi_swiglu_fwd": 1,
+                                                                     "emi_gemm": 7}
     assert all("api_version = 4 : i32" in l and "backend_config = {" in l and "operand_layouts = [" in l for l in calls)
     rms = [l for l in calls if "emi_rmsnorm_fwd" in l][0]
     assert "backend_config = {eps = 9.999999747e-06 : f32}" in rms
@@ -199,7 +202,7 @@ def test_symbolic_reverse_of_the_llama_step_calls_the_adjoint_targets():
     targets = Counter(o.attrs["target"] for o in f.ops if o.name == "custom_call")
     # forward values the adjoints need are recomputed (the final RMSNorm's output is not needed)
     assert targets == {"emi_rope": 4, "emi_rmsnorm_bwd": 3, "emi_rmsnorm_fwd": 2, "emi_attn_step_fwd": 1, "emi_swiglu_fwd": 1,
-                       "emi_swiglu_bwd": 1, "emi_attn_step_bwd": 1}
+                       "emi_swiglu_bwd": 1, "emi_attn_step_bwd": 1, "emi_gemm": 7 + 14}      # 7 projections, dX and dW of each
     assert sorted(o.attrs["config"]["inverse"] for o in f.ops if o.name == "custom_call" and o.attrs["target"] == "emi_rope") == \
         [False, False, True, True]
     assert len(f.args) == len(order) + 1 and f.args[-1][1].shape == (288,)
