@@ -426,6 +426,19 @@ def main():
     name = "llama7b_layer_B%d_S%d" % (cfg["batch"], cfg["seq"])
     log("%s\tHIP\trocm\tPrimal+VJP\t%.6f s  (%.1f TFLOP/s over %.2f TFLOP algorithmic)" % (name, dt, fl["total"] / dt / 1e12, fl["total"] / 1e12))
 
+    # the other two programs the reference's harness times next to reverse mode (test/test_utils.py:626-735):
+    # the primal alone, and forward mode with a tangent on the input and on every weight
+    from enzyme_ad.jax import jvp
+    modes = None
+    if not args.no_kernels:
+        tx = torch.randn_like(x)
+        tlw = {k: torch.randn_like(v) * 0.02 for k, v in lw.items()}
+        t_primal = event_time(lambda: layer_fn(x, lw), 5)
+        t_forward = event_time(lambda: jvp(layer_fn, (x, lw), (tx, tlw)), 5)
+        modes = {"Primal_ms": round(t_primal * 1e3, 3), "Forward_ms": round(t_forward * 1e3, 3), "BothRev_ms": round(dt * 1e3, 3)}
+        log("layer programs:", modes)
+        del tx, tlw
+
     t_gemm, gemm_fl, n_gemm, per_layout = bench_gemms(cfg, max(5, min(args.steps, 20)))
     roofline = dict(bound="mfma", kernel="gemm_bf16_pingpong_kernel (256x256x64 tiles; %d launches per step: Y, dX in the NT form, dW in the TN form, 7 weights)" % n_gemm,
                     achieved=gemm_fl / t_gemm / 1e12, peak=PEAK_BF16_TFLOPS, unit="TFLOP/s",
@@ -464,7 +477,7 @@ def main():
                                "32 heads x 128, batch %d x seq %d, bf16" % (cfg["batch"], cfg["seq"]),
                    "tokens_per_step": tokens, "algorithmic_tflop_per_step": fl["total"] / 1e12,
                    "step_tflops": fl["total"] / dt / 1e12},
-        "roofline": roofline, "kernels": kernels, "stablehlo_frontend": frontend, "cpu_baseline": cpu,
+        "roofline": roofline, "programs": modes, "kernels": kernels, "stablehlo_frontend": frontend, "cpu_baseline": cpu,
     }))
 
 
