@@ -185,6 +185,10 @@ def bench_kernels(cfg, iters):
         hbm("reduce_rows_" + tag, lambda: N.check(lib.emi_reduce(st, HO.REDUCE["add"], P(a), P(col), None, 0, rows, D, 1, code)), n * s)
         hbm("reduce_cols_" + tag, lambda: N.check(lib.emi_reduce(st, HO.REDUCE["add"], P(a), P(row), P(rws), rwb, 1, rows, D, code)), n * s)
         hbm("reduce_all_" + tag, lambda: N.check(lib.emi_reduce(st, HO.REDUCE["add"], P(a), P(col), P(rws), rwb, 1, n, 1, code)), n * s)
+        mask = torch.empty((rows, D), dtype=torch.bool, device="cuda")
+        hbm("compare_" + tag, lambda: N.check(lib.emi_compare(st, HO.COMPARE["GT"], P(a), P(b), P(mask), n, 0, 0, code)), n * (2 * s + 1))
+        hbm("select_" + tag, lambda: N.check(lib.emi_select(st, P(mask), P(a), P(b), P(y), n, 0, 0, 0, code)), n * (3 * s + 1))
+        del mask
         if dt == torch.float32:
             yb = torch.empty((rows, D), dtype=bf, device="cuda")
             hbm("convert_f32_bf16", lambda: N.check(lib.emi_convert(st, P(a), P(yb), n, N.EMI_F32, N.EMI_BF16)), n * 6)
