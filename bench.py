@@ -343,6 +343,54 @@ def bench_frontend(iters):
     return out
 
 
+def bench_models(iters):
+    """The two whole-model configurations: tokens in, logits out, fwd + VJP with a cotangent on the
+    logits.  C4 stories110M (dim 768, hidden 2048, 12 layers, 12 heads x 64, vocab 32000, seq 1024,
+    batch 8, bf16) and C1 stories15M (dim 288, hidden 768, 6 layers, 6 heads x 48, seq 256, batch 1,
+    fp32)."""
+    import torch
+    from enzyme_ad.jax import enzyme_jax_ir, JaXPipeline, vjp, llama
+    out = {}
+    for name, cfg, B, S, dt in (("c4_stories110m_bf16", dict(dim=768, hidden_dim=2048, n_layers=12, n_heads=12, n_kv_heads=12,
+                                                            vocab_size=32000, seq_len=1024), 8, 1024, torch.bfloat16),
+                                ("c1_stories15m_f32", dict(dim=288, hidden_dim=768, n_layers=6, n_heads=6, n_kv_heads=6,
+                                                          vocab_size=32000, seq_len=256), 1, 256, torch.float32)):
+        g = torch.Generator(device="cuda").manual_seed(4)
+        L_, D, H, V = cfg["n_layers"], cfg["dim"], cfg["hidden_dim"], cfg["vocab_size"]
+        n = lambda *shape: (torch.randn(shape, generator=g, device="cuda") * 0.02).to(dt)
+        w = {"rms_att_weight": n(L_, D) + 1, "wq": n(L_, D, D), "wk": n(L_, D, D), "wv": n(L_, D, D), "wo": n(L_, D, D),
+             "rms_ffn_weight": n(L_, D) + 1, "w1": n(L_, H, D), "w2": n(L_, D, H), "w3": n(L_, H, D), "rms_final_weight": n(D) + 1,
+             "token_embedding_table": n(V, D), "wcls": n(V, D)}
+        tok = torch.randint(0, V, (B, S), generator=g, device="cuda", dtype=torch.int32)
+        dlogits = torch.randn((B, S, V), generator=g, device="cuda").to(dt)
+
+        @enzyme_jax_ir(pipeline_options=JaXPipeline(), inner_jit=False)
+        def fn(weights):
+            return llama.forward(tok, cfg, weights, logits=True)
+
+        def step():
+            y, f_vjp = vjp(fn, w)
+            return f_vjp(dlogits)
+
+        t = event_time(step, iters, warmup=2)
+        out[name] = dict(ms_per_step=round(t * 1e3, 3), tokens_per_s=round(B * S / t, 1), tokens_per_step=B * S)
+        if B * S <= 1024:
+            # small enough to be bound by launches and host code: the same step replayed from a HIP graph
+            from enzyme_ad.jax.graph import capture
+
+            def step_fn(weights, dl):
+                y, f_vjp = vjp(lambda ww: llama.forward(tok, cfg, ww, logits=True), weights)
+                return f_vjp(dl)
+
+            gr = capture(step_fn, w, dlogits)
+            tg = event_time(lambda: gr(w, dlogits), 4 * iters)
+            out[name]["graph_replay_ms_per_step"] = round(tg * 1e3, 3)
+            out[name]["graph_replay_tokens_per_s"] = round(B * S / tg, 1)
+            del gr
+        del w, dlogits
+    return out
+
+
 def cpu_baseline(cfg, seconds_hint=20):
     """The numpy oracle of the same layer (fwd + bwd) on a bounded sample."""
     import numpy as np
@@ -467,6 +515,12 @@ def main():
         for k, v in frontend.items():
             log("%-28s %s" % (k, {a: b for a, b in v.items() if a != "clusters"}))
 
+    models = None
+    if not args.no_kernels and not args.no_frontend:
+        models = bench_models(5)
+        for k, v in models.items():
+            log("%-24s %s" % (k, v))
+
     cpu = None
     if not args.no_cpu_baseline:
         cpu = cpu_baseline(cfg)
@@ -481,7 +535,7 @@ def main():
                                "32 heads x 128, batch %d x seq %d, bf16" % (cfg["batch"], cfg["seq"]),
                    "tokens_per_step": tokens, "algorithmic_tflop_per_step": fl["total"] / 1e12,
                    "step_tflops": fl["total"] / dt / 1e12},
-        "roofline": roofline, "programs": modes, "kernels": kernels, "stablehlo_frontend": frontend, "cpu_baseline": cpu,
+        "roofline": roofline, "programs": modes, "kernels": kernels, "stablehlo_frontend": frontend, "whole_models": models, "cpu_baseline": cpu,
     }))
 
 

@@ -789,40 +789,48 @@ __global__ __launch_bounds__(512) void gemm_bf16_pingpong_kernel(const uint16_t*
 // Generic path: any dtype/shape/alignment, fp32 MFMA (v_mfma_f32_32x32x2_f32).
 // 256 threads, 128x128x16 tile, LDS tiles stored k-major as fp32.
 // ---------------------------------------------------------------------------
-template <typename T>
+// WT: 32x32 MFMA tiles per wavefront and dimension: 2 -> 128x128 block tiles, 1 -> 64x64 (small problems: more
+// blocks, shorter iterations).
+template <typename T, int WT>
 __global__ __launch_bounds__(256) void gemm_generic_kernel(const T* __restrict__ A, const T* __restrict__ B, const T* R,
                                                            T* C, int M, int N, int K, int64_t lda, int64_t ldb,
-                                                           int64_t ldr, int64_t ldc, int trans_a, int trans_b) {
-  constexpr int BM = 128, BN = 128, BK = 16, PAD = 4;
+                                                           int64_t ldr, int64_t ldc, int trans_a, int trans_b,
+                                                           float* __restrict__ part, int k_per_split) {
+  constexpr int BM = 64 * WT, BN = 64 * WT, BK = 16, PAD = 4;
   __shared__ float sA[BK][BM + PAD];
   __shared__ float sB[BK][BN + PAD];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
-  f32x16_t acc[2][2];
+  f32x16_t acc[WT][WT];
 #pragma unroll
-  for (int i = 0; i < 2; i++)
+  for (int i = 0; i < WT; i++)
 #pragma unroll
-    for (int j = 0; j < 2; j++)
+    for (int j = 0; j < WT; j++)
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-  for (int k0 = 0; k0 < K; k0 += BK) {
-    // A tile: 128 x 16 elements, 8 per thread
+  // split-K (part != nullptr): block z owns k in [z * k_per_split, ...) and writes an fp32 partial
+  // tile to part[z][M][N]; a second kernel adds the partials (and R) in fixed order
+  const int k_lo = part ? blockIdx.z * k_per_split : 0;
+  const int k_hi = part ? (k_lo + k_per_split < K ? k_lo + k_per_split : K) : K;
+  K = k_hi;
+  for (int k0 = k_lo; k0 < K; k0 += BK) {
+    // A tile: BM x 16 elements, BM / 16 per thread
 #pragma unroll
-    for (int it = 0; it < 8; it++) {
+    for (int it = 0; it < BM / 16; it++) {
       int m, k;
-      if (trans_a) { m = tid & 127; k = (tid >> 7) + it * 2; }        // A is [K,M]: m contiguous
+      if (trans_a) { m = tid & (BM - 1); k = tid / BM + it * (256 / BM); }   // A is [K,M]: m contiguous
       else { k = tid & 15; m = (tid >> 4) + it * 16; }                // A is [M,K]: k contiguous
       float v = 0.f;
       if (m0 + m < M && k0 + k < K) v = to_f32(trans_a ? A[(int64_t)(k0 + k) * lda + m0 + m] : A[(int64_t)(m0 + m) * lda + k0 + k]);
       sA[k][m] = v;
     }
 #pragma unroll
-    for (int it = 0; it < 8; it++) {
+    for (int it = 0; it < BN / 16; it++) {
       int n, k;
       if (trans_b) { k = tid & 15; n = (tid >> 4) + it * 16; }        // B is [N,K]
-      else { n = tid & 127; k = (tid >> 7) + it * 2; }                // B is [K,N]
+      else { n = tid & (BN - 1); k = tid / BN + it * (256 / BN); }    // B is [K,N]
       float v = 0.f;
       if (n0 + n < N && k0 + k < K) v = to_f32(trans_b ? B[(int64_t)(n0 + n) * ldb + k0 + k] : B[(int64_t)(k0 + k) * ldb + n0 + n]);
       sB[k][n] = v;
@@ -831,34 +839,64 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const T* __restrict__
 #pragma unroll
     for (int kk = 0; kk < BK; kk += 2) {
       const int k = kk + (lane >> 5);
-      float a[2], b[2];
+      float a[WT], b[WT];
 #pragma unroll
-      for (int i = 0; i < 2; i++) a[i] = sA[k][wm * 64 + i * 32 + (lane & 31)];
+      for (int i = 0; i < WT; i++) a[i] = sA[k][wm * 32 * WT + i * 32 + (lane & 31)];
 #pragma unroll
-      for (int j = 0; j < 2; j++) b[j] = sB[k][wn * 64 + j * 32 + (lane & 31)];
+      for (int j = 0; j < WT; j++) b[j] = sB[k][wn * 32 * WT + j * 32 + (lane & 31)];
 #pragma unroll
-      for (int i = 0; i < 2; i++)
+      for (int i = 0; i < WT; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+        for (int j = 0; j < WT; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
     }
     __syncthreads();
   }
   const int col_l = lane & 31, row_l = (lane >> 5) * 4;
 #pragma unroll
-  for (int i = 0; i < 2; i++)
+  for (int i = 0; i < WT; i++)
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
-      const int col = n0 + wn * 64 + j * 32 + col_l;
+    for (int j = 0; j < WT; j++) {
+      const int col = n0 + wn * 32 * WT + j * 32 + col_l;
 #pragma unroll
       for (int r = 0; r < 16; r++) {
-        const int row = m0 + wm * 64 + i * 32 + (r >> 2) * 8 + row_l + (r & 3);
+        const int row = m0 + wm * 32 * WT + i * 32 + (r >> 2) * 8 + row_l + (r & 3);
         if (row < M && col < N) {
           float v = acc[i][j][r];
-          if (R != nullptr) v += to_f32(R[(int64_t)row * ldr + col]);
-          C[(int64_t)row * ldc + col] = from_f32<T>(v);
+          if (part != nullptr) {
+            part[((int64_t)blockIdx.z * M + row) * N + col] = v;
+          } else {
+            if (R != nullptr) v += to_f32(R[(int64_t)row * ldr + col]);
+            C[(int64_t)row * ldc + col] = from_f32<T>(v);
+          }
         }
       }
     }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __restrict__ part, const T* R, T* C, int M, int N,
+                                                                 int splits, int64_t ldr, int64_t ldc) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (int64_t)M * N) return;
+  const int row = (int)(i / N), col = (int)(i - (int64_t)row * N);
+  float v = 0.f;
+  for (int z = 0; z < splits; z++) v += part[(int64_t)z * M * N + i];
+  if (R != nullptr) v += to_f32(R[(int64_t)row * ldr + col]);
+  C[(int64_t)row * ldc + col] = from_f32<T>(v);
+}
+
+// Few output tiles and a long contraction (the logits adjoint dX = dY . Wcls of a small batch:
+// 6 tiles, K = 32000): split K over enough blocks to fill the chip.
+static int generic_tile(int64_t M, int64_t N) {          // block tile edge: 64 while 128 would leave most CUs idle
+  return ((M + 127) / 128) * ((N + 127) / 128) < 64 ? 64 : 128;
+}
+static int generic_splits(int64_t M, int64_t N, int64_t K) {
+  const int t = generic_tile(M, N);
+  const int64_t tiles = ((M + t - 1) / t) * ((N + t - 1) / t);
+  if (tiles >= 128 || K < 2048) return 1;
+  int64_t s = (t == 64 ? 1024 : 512) / tiles;          // about four (two) resident blocks per CU
+  if (s > K / 256) s = K / 256;
+  return (int)(s < 2 ? 1 : (s > 256 ? 256 : s));
 }
 
 template <int BM, int BN, int BK, int NSTAGE, int WM, int WN, bool AK, bool BKM>
@@ -941,11 +979,34 @@ static int launch_bf16_layout(hipStream_t st, const void* A, const void* B, cons
 
 template <typename T>
 static int launch_generic(hipStream_t st, const void* A, const void* B, const void* R, void* C, int M, int N, int K,
-                          int64_t lda, int64_t ldb, int64_t ldr, int64_t ldc, int trans_a, int trans_b) {
-  dim3 grid((N + 127) / 128, (M + 127) / 128);
+                          int64_t lda, int64_t ldb, int64_t ldr, int64_t ldc, int trans_a, int trans_b, void* workspace, size_t workspace_bytes) {
+  const int tile = generic_tile(M, N);
+  dim3 grid((N + tile - 1) / tile, (M + tile - 1) / tile);
   if (grid.y > 65535) return emi_fail(EMI_INVALID_ARGUMENT, "emi_gemm: M=%d too large for the generic path", M);
-  hipLaunchKernelGGL(gemm_generic_kernel<T>, grid, dim3(256), 0, st, static_cast<const T*>(A), static_cast<const T*>(B),
-                     static_cast<const T*>(R), static_cast<T*>(C), M, N, K, lda, ldb, ldr, ldc, trans_a, trans_b);
+  const int splits = generic_splits(M, N, K);
+#define EMI_GENERIC(PART, KPS)                                                                                          \
+  do {                                                                                                                   \
+    if (tile == 64)                                                                                                      \
+      hipLaunchKernelGGL((gemm_generic_kernel<T, 1>), grid, dim3(256), 0, st, static_cast<const T*>(A), static_cast<const T*>(B), \
+                         static_cast<const T*>(R), static_cast<T*>(C), M, N, K, lda, ldb, ldr, ldc, trans_a, trans_b, PART, KPS); \
+    else                                                                                                                 \
+      hipLaunchKernelGGL((gemm_generic_kernel<T, 2>), grid, dim3(256), 0, st, static_cast<const T*>(A), static_cast<const T*>(B), \
+                         static_cast<const T*>(R), static_cast<T*>(C), M, N, K, lda, ldb, ldr, ldc, trans_a, trans_b, PART, KPS); \
+  } while (0)
+  if (splits > 1 && workspace != nullptr && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0 &&
+      workspace_bytes >= (size_t)splits * M * N * sizeof(float)) {
+    const int kps = (((K + splits - 1) / splits) + 15) / 16 * 16;
+    grid.z = (K + kps - 1) / kps;
+    float* part = static_cast<float*>(workspace);
+    EMI_GENERIC(part, kps);
+    EMI_CHECK_LAUNCH("emi_gemm(generic split-K)");
+    hipLaunchKernelGGL(gemm_splitk_reduce_kernel<T>, dim3((unsigned)(((int64_t)M * N + 255) / 256)), dim3(256), 0, st, part,
+                       static_cast<const T*>(R), static_cast<T*>(C), M, N, (int)grid.z, ldr, ldc);
+    EMI_CHECK_LAUNCH("emi_gemm(generic split-K reduce)");
+    return EMI_OK;
+  }
+  EMI_GENERIC(static_cast<float*>(nullptr), 0);
+#undef EMI_GENERIC
   EMI_CHECK_LAUNCH("emi_gemm(generic)");
   return EMI_OK;
 }
@@ -962,7 +1023,12 @@ using namespace emi;
 
 
 extern "C" size_t emi_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int trans_a, int trans_b, int dtype) {
-  return skinny_workspace_bytes(M, N, K, trans_a, trans_b, dtype);
+  const size_t skinny = skinny_workspace_bytes(M, N, K, trans_a, trans_b, dtype);
+  if (skinny) return skinny;
+  if (M <= 0 || N <= 0 || K <= 0) return 0;
+  // fp32 (and bf16 shapes the fast path does not take) with few tiles and a long contraction: split-K partials
+  const int splits = generic_splits(M, N, K);
+  return splits > 1 ? (size_t)splits * M * N * sizeof(float) : 0;
 }
 
 extern "C" int emi_gemm(emi_stream_t stream, const void* A, const void* B, const void* R, void* C, int64_t M, int64_t N,
@@ -1010,7 +1076,7 @@ extern "C" int emi_gemm_ws(emi_stream_t stream, const void* A, const void* B, co
         return launch_bf16_layout<true, true>(st, A, B, R, C, m, n, k, (int)lda, (int)ldb, (int)ldr, (int)ldc, ab, bb);
       return launch_bf16_layout<true, false>(st, A, B, R, C, m, n, k, (int)lda, (int)ldb, (int)ldr, (int)ldc, ab, bb);
     }
-    return launch_generic<bf16>(st, A, B, R, C, (int)M, (int)N, (int)K, lda, ldb, ldr, ldc, trans_a, trans_b);
+    return launch_generic<bf16>(st, A, B, R, C, (int)M, (int)N, (int)K, lda, ldb, ldr, ldc, trans_a, trans_b, workspace, workspace_bytes);
   }
-  return launch_generic<float>(st, A, B, R, C, (int)M, (int)N, (int)K, lda, ldb, ldr, ldc, trans_a, trans_b);
+  return launch_generic<float>(st, A, B, R, C, (int)M, (int)N, (int)K, lda, ldb, ldr, ldc, trans_a, trans_b, workspace, workspace_bytes);
 }
