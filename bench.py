@@ -203,6 +203,19 @@ def bench_kernels(cfg, iters):
     hbm("swiglu_jvp_bf16", lambda: N.check(lib.emi_swiglu_jvp(st, P(a), P(b), P(dg), P(db), P(da), n, N.EMI_BF16)), 5 * n * 2)
     hbm("swiglu_bwd_bf16", lambda: N.check(lib.emi_swiglu_bwd(st, P(a), P(b), P(dg), P(da), P(db), n, N.EMI_BF16)), 5 * n * 2)
     del a, b, dg, da, db
+    # C4 logits: cross-entropy over [8 x 1024 tokens, 32000], bf16 and fp32 (algorithmic bytes: the logits read
+    # once forward, read and written once in the adjoint, logits and tangent read once in forward mode)
+    Tk, V = 8 * 1024, 32000
+    for dt, s, code in ((bf, 2, N.EMI_BF16), (torch.float32, 4, N.EMI_F32)):
+        tag = "bf16" if dt == bf else "f32"
+        z = (torch.randn((Tk, V), device="cuda") * 3).to(dt)
+        tz, dz = torch.randn((Tk, V), device="cuda").to(dt), torch.empty((Tk, V), device="cuda", dtype=dt)
+        tgt = torch.randint(0, V, (Tk,), device="cuda", dtype=torch.int32)
+        loss, lse_t, dl = (torch.ones(Tk, device="cuda") for _ in range(3))
+        hbm("cross_entropy_fwd_" + tag, lambda: N.check(lib.emi_cross_entropy_fwd(st, P(z), P(tgt), P(loss), P(lse_t), Tk, V, code)), Tk * V * s)
+        hbm("cross_entropy_bwd_" + tag, lambda: N.check(lib.emi_cross_entropy_bwd(st, P(z), P(tgt), P(lse_t), P(dl), P(dz), Tk, V, code)), 2 * Tk * V * s)
+        hbm("cross_entropy_jvp_" + tag, lambda: N.check(lib.emi_cross_entropy_jvp(st, P(z), P(tgt), P(lse_t), P(tz), P(loss), Tk, V, code)), 2 * Tk * V * s)
+        del z, tz, dz
     # C3: attention [8, 32, 2048, 128] bf16 causal
     B, h, S, d = 8, 32, 2048, 128
     q, k, v, do = (torch.randn((B, h, S, d), device="cuda").to(bf) for _ in range(4))

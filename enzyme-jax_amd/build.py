@@ -17,7 +17,7 @@ LIB = os.path.join(LIBDIR, "libemi_hip.so")
 OBJDIR = os.path.join(LIBDIR, "obj")
 
 HIP_SOURCES = ["elementwise.hip", "gemm.hip", "gemm_skinny.hip", "attention.hip", "attention_step.hip", "forward_mode.hip",
-               "tensor_ops.hip"]
+               "tensor_ops.hip", "cross_entropy.hip"]
 CXX_SOURCES = ["status.cc", "ffi_handlers.cc"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")

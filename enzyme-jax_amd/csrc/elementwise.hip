@@ -242,41 +242,46 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_generic_kernel(const T* __res
 }
 
 // Column sums of partial[nparts][dim]: block (cb, rc) adds rows [CS_ROWS*rc, CS_ROWS*rc +
-// CS_ROWS) of 64 columns (16 float4 columns x 16 row lanes, so a wavefront reads 256
-// contiguous bytes of four rows) into row rc of `out`.  The launcher applies it
-// until one row is left (one pass for the grids the adjoint uses); the last pass
-// writes type T.
+// CS_ROWS) of 64 columns into row rc of `out`.  1024 threads = 16 float4 columns x 64 row
+// lanes (a wavefront reads 256 contiguous bytes of four rows), eight loads in flight per
+// lane, so the 512 partial rows of the adjoint's grid are one round of loads.  The
+// launcher applies it until one row is left (one pass for the grids the adjoint uses);
+// the last pass writes type T.
 constexpr int CS_ROWS = 512;
 template <typename TO>
-__global__ __launch_bounds__(256) void colsum_kernel(const float* __restrict__ partial, int nparts, int64_t dim,
-                                                     TO* __restrict__ out) {
-  __shared__ float red[16][64 + 4];
+__global__ __launch_bounds__(1024) void colsum_kernel(const float* __restrict__ partial, int nparts, int64_t dim,
+                                                      TO* __restrict__ out) {
+  __shared__ float red[64][64 + 4];
   const int cq = threadIdx.x & 15, rl = threadIdx.x >> 4;
   const int64_t col = (int64_t)blockIdx.x * 64 + cq * 4;
   const int r0 = blockIdx.y * CS_ROWS;
   const int r1 = r0 + CS_ROWS < nparts ? r0 + CS_ROWS : nparts;
   float s[4] = {0.f, 0.f, 0.f, 0.f};
   if ((dim & 3) == 0 && col + 4 <= dim) {
-    float4 v[4];
-    int p = r0 + rl;
-    for (; p + 48 < r1; p += 64) {           // four independent loads in flight
+    float4 v[8];
 #pragma unroll
-      for (int u = 0; u < 4; u++) v[u] = *reinterpret_cast<const float4*>(partial + (int64_t)(p + 16 * u) * dim + col);
+    for (int u = 0; u < 8; u++) {
+      const int p = r0 + rl + 64 * u;
+      v[u] = p < r1 ? *reinterpret_cast<const float4*>(partial + (int64_t)p * dim + col) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
 #pragma unroll
-      for (int u = 0; u < 4; u++) { s[0] += v[u].x; s[1] += v[u].y; s[2] += v[u].z; s[3] += v[u].w; }
-    }
-    for (; p < r1; p += 16) {
-      const float4 w = *reinterpret_cast<const float4*>(partial + (int64_t)p * dim + col);
-      s[0] += w.x; s[1] += w.y; s[2] += w.z; s[3] += w.w;
-    }
+    for (int u = 0; u < 8; u++) { s[0] += v[u].x; s[1] += v[u].y; s[2] += v[u].z; s[3] += v[u].w; }
   } else {
-    for (int p = r0 + rl; p < r1; p += 16)
+    for (int p = r0 + rl; p < r1; p += 64)
 #pragma unroll
       for (int e = 0; e < 4; e++)
         if (col + e < dim) s[e] += partial[(int64_t)p * dim + col + e];
   }
 #pragma unroll
   for (int e = 0; e < 4; e++) red[rl][cq * 4 + e] = s[e];
+  __syncthreads();
+  // 64 columns x 16 row groups of four, then the 16 partial sums of a column
+  {
+    const int c = threadIdx.x & 63, g = threadIdx.x >> 6;
+    const float t = red[4 * g][c] + red[4 * g + 1][c] + red[4 * g + 2][c] + red[4 * g + 3][c];
+    __syncthreads();
+    red[g][c] = t;
+  }
   __syncthreads();
   if (threadIdx.x < 64) {
     const int64_t c = (int64_t)blockIdx.x * 64 + threadIdx.x;
@@ -583,14 +588,14 @@ static int rmsnorm_bwd_launch(hipStream_t st, const void* x, const void* gamma, 
   int64_t n = nparts;
   while (n > CS_ROWS) {
     const int64_t m = (n + CS_ROWS - 1) / CS_ROWS;
-    hipLaunchKernelGGL(colsum_kernel<float>, dim3(blocks_for(dim, 64), (unsigned)m), dim3(256), 0, st, cur, (int)n, dim, nxt);
+    hipLaunchKernelGGL(colsum_kernel<float>, dim3(blocks_for(dim, 64), (unsigned)m), dim3(1024), 0, st, cur, (int)n, dim, nxt);
     EMI_CHECK_LAUNCH("emi_rmsnorm_bwd(colsum)");
     float* t = cur;
     cur = nxt;
     nxt = t;
     n = m;
   }
-  hipLaunchKernelGGL(colsum_kernel<T>, dim3(blocks_for(dim, 64), 1), dim3(256), 0, st, cur, (int)n, dim,
+  hipLaunchKernelGGL(colsum_kernel<T>, dim3(blocks_for(dim, 64), 1), dim3(1024), 0, st, cur, (int)n, dim,
                      static_cast<T*>(dgamma));
   EMI_CHECK_LAUNCH("emi_rmsnorm_bwd(colsum)");
   return EMI_OK;

@@ -500,6 +500,58 @@ extern "C" XLA_FFI_Error* emi_embedding_bwd_ffi(XLA_FFI_CallFrame* cf) {
 }
 
 namespace {
+// logits[.., V] with per-token buffers shaped like its leading dimensions
+const char* xent_shapes(const XLA_FFI_Buffer* z, const XLA_FFI_Buffer* tgt, const XLA_FFI_Buffer* const* per_token, int n) {
+  if (!is_float(z) || z->rank < 1) return "logits must be f32 or bf16 of rank >= 1";
+  if (tgt->dtype != XLA_FFI_DataType_S32) return "targets must be s32";
+  const int64_t V = z->dims[z->rank - 1];
+  const int64_t T = V ? numel(z) / V : 0;
+  if (numel(tgt) != T) return "targets must have one entry per token";
+  for (int i = 0; i < n; i++)
+    if (per_token[i]->dtype != XLA_FFI_DataType_F32 || numel(per_token[i]) != T) return "loss, lse, dloss and tloss are f32 with one entry per token";
+  return nullptr;
+}
+}  // namespace
+
+extern "C" XLA_FFI_Error* emi_cross_entropy_fwd_ffi(XLA_FFI_CallFrame* cf) {
+  EMI_FFI_BEGIN("emi_cross_entropy_fwd", 2, 2, 2, 2)
+  const XLA_FFI_Buffer *z = f.arg(0), *tgt = f.arg(1), *loss = f.ret(0), *lse = f.ret(1);
+  const XLA_FFI_Buffer* pt[] = {loss, lse};
+  if (const char* why = xent_shapes(z, tgt, pt, 2)) return f.invalid(why);
+  EMI_FFI_STREAM()
+  const int64_t V = z->dims[z->rank - 1];
+  return f.from_status(emi_cross_entropy_fwd(stream, z->data, static_cast<const int32_t*>(tgt->data),
+                                             static_cast<float*>(loss->data), static_cast<float*>(lse->data),
+                                             V ? numel(z) / V : 0, V, z->dtype));
+}
+
+extern "C" XLA_FFI_Error* emi_cross_entropy_bwd_ffi(XLA_FFI_CallFrame* cf) {
+  EMI_FFI_BEGIN("emi_cross_entropy_bwd", 4, 4, 1, 1)
+  const XLA_FFI_Buffer *z = f.arg(0), *tgt = f.arg(1), *lse = f.arg(2), *dl = f.arg(3), *dz = f.ret(0);
+  const XLA_FFI_Buffer* pt[] = {lse, dl};
+  if (const char* why = xent_shapes(z, tgt, pt, 2)) return f.invalid(why);
+  if (dz->dtype != z->dtype || !same_shape(z, dz)) return f.invalid("dlogits must have the shape and dtype of logits");
+  EMI_FFI_STREAM()
+  const int64_t V = z->dims[z->rank - 1];
+  return f.from_status(emi_cross_entropy_bwd(stream, z->data, static_cast<const int32_t*>(tgt->data),
+                                             static_cast<const float*>(lse->data), static_cast<const float*>(dl->data),
+                                             dz->data, V ? numel(z) / V : 0, V, z->dtype));
+}
+
+extern "C" XLA_FFI_Error* emi_cross_entropy_jvp_ffi(XLA_FFI_CallFrame* cf) {
+  EMI_FFI_BEGIN("emi_cross_entropy_jvp", 4, 4, 1, 1)
+  const XLA_FFI_Buffer *z = f.arg(0), *tgt = f.arg(1), *lse = f.arg(2), *tz = f.arg(3), *tl = f.ret(0);
+  const XLA_FFI_Buffer* pt[] = {lse, tl};
+  if (const char* why = xent_shapes(z, tgt, pt, 2)) return f.invalid(why);
+  if (tz->dtype != z->dtype || !same_shape(z, tz)) return f.invalid("tlogits must have the shape and dtype of logits");
+  EMI_FFI_STREAM()
+  const int64_t V = z->dims[z->rank - 1];
+  return f.from_status(emi_cross_entropy_jvp(stream, z->data, static_cast<const int32_t*>(tgt->data),
+                                             static_cast<const float*>(lse->data), tz->data,
+                                             static_cast<float*>(tl->data), V ? numel(z) / V : 0, V, z->dtype));
+}
+
+namespace {
 struct Target {
   const char* name;
   XLA_FFI_Handler* handler;
@@ -514,6 +566,8 @@ const Target kTargets[] = {
     {"emi_rmsnorm_jvp", emi_rmsnorm_jvp_ffi}, {"emi_swiglu_jvp", emi_swiglu_jvp_ffi}, {"emi_attn_jvp", emi_attn_jvp_ffi},
     {"emi_attn_step_jvp", emi_attn_step_jvp_ffi},
     {"emi_embedding_fwd", emi_embedding_fwd_ffi}, {"emi_embedding_bwd", emi_embedding_bwd_ffi},
+    {"emi_cross_entropy_fwd", emi_cross_entropy_fwd_ffi}, {"emi_cross_entropy_bwd", emi_cross_entropy_bwd_ffi},
+    {"emi_cross_entropy_jvp", emi_cross_entropy_jvp_ffi},
 };
 constexpr int kNumTargets = sizeof(kTargets) / sizeof(kTargets[0]);
 XLA_FFI_Error* noop_stage(XLA_FFI_CallFrame*) { return nullptr; }

@@ -64,6 +64,9 @@ SIGNATURES = {
     "emi_embedding_bwd_workspace_bytes": (c_size_t, [c_i64, c_i64, c_int]),
     "emi_embedding_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_i64, c_i64, c_i64,
                                   c_int]),
+    "emi_cross_entropy_fwd": (c_int, [c_void_p] * 5 + [c_i64, c_i64, c_int]),
+    "emi_cross_entropy_bwd": (c_int, [c_void_p] * 6 + [c_i64, c_i64, c_int]),
+    "emi_cross_entropy_jvp": (c_int, [c_void_p] * 6 + [c_i64, c_i64, c_int]),
 }
 
 _lib = None

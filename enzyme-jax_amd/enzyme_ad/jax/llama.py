@@ -47,6 +47,19 @@ def forward(x, config, weights, logits=False, eps=1e-5, theta=10000.0):
     return x
 
 
+def loss(x, targets, config, weights, eps=1e-5, theta=10000.0):
+    """Mean over all tokens of the softmax cross-entropy of `forward(..., logits=True)` against int32 `targets`
+    `[B, S]`: a scalar fp32 tensor.  What a training step differentiates once the classifier commented out at
+    test/llama.py:236 is switched on."""
+    import torch
+
+    from . import hlo_ops as H
+
+    per_token = ops.cross_entropy(forward(x, config, weights, logits=True, eps=eps, theta=theta), targets)
+    total = H.reduce("add", per_token, range(per_token.dim()))
+    return H.binary("multiply", total, torch.full((), 1.0 / targets.numel(), dtype=torch.float32, device=total.device))
+
+
 def forward_step(x, config, weights, key_cache, value_cache, eps=1e-5, theta=10000.0):
     """The reference's own single-token form, argument for argument
     (test/llama.py:35-238): x is the residual stream of one token [dim];

@@ -32,13 +32,14 @@ FFI_TARGETS = {
     "attention_step": ("emi_attn_step_fwd", ("emi_attn_step_bwd",)),
     "add":       ("emi_add", ()),
     "embedding": ("emi_embedding_fwd", ("emi_embedding_bwd",)),
+    "cross_entropy": ("emi_cross_entropy_fwd", ("emi_cross_entropy_bwd",)),
 }
 
 # operator -> tangent target(s); linear operators push tangents through their forward target
 FFI_TANGENT_TARGETS = {
     "rmsnorm": ("emi_rmsnorm_jvp",), "rope": ("emi_rope",), "matmul_nt": ("emi_gemm", "emi_gemm"),
     "swiglu": ("emi_swiglu_jvp",), "attention": ("emi_attn_jvp",), "attention_step": ("emi_attn_step_jvp",),
-    "add": ("emi_add",), "embedding": ("emi_embedding_fwd",),
+    "add": ("emi_add",), "embedding": ("emi_embedding_fwd",), "cross_entropy": ("emi_cross_entropy_jvp",),
 }
 
 _DTYPES = {torch.float32: N.EMI_F32, torch.bfloat16: N.EMI_BF16}
@@ -591,6 +592,40 @@ def embedding(tokens, table):
         tt = tans[0]
         _set_tan(x, _quiet(lambda: embedding(tokens, tt)))                 # linear in the table
     return x
+
+
+def cross_entropy(logits, targets):
+    """Per-token softmax cross-entropy `logsumexp(z) - z[target]` of logits `[..., vocab]` against int32 targets
+    `[...]`; the losses are fp32 whatever the logits' dtype.  The loss that follows the classifier commented out at
+    test/llama.py:236.  Adjoint: `(softmax(z) - onehot) * dloss` from the saved logsumexp; a target outside
+    `[0, vocab)` masks its token (zero loss and gradient)."""
+    _dev(logits, targets)
+    if targets.dtype != torch.int32:
+        raise TypeError("cross_entropy: targets must be int32")
+    if tuple(targets.shape) != tuple(logits.shape[:-1]):
+        raise ValueError("cross_entropy: targets %s do not match logits %s" % (tuple(targets.shape), tuple(logits.shape)))
+    V = logits.shape[-1]
+    T = targets.numel()
+    loss = torch.empty(targets.shape, dtype=torch.float32, device=logits.device)
+    lse = torch.empty(targets.shape, dtype=torch.float32, device=logits.device)
+    N.check(N.lib().emi_cross_entropy_fwd(_stream(), _p(logits), _p(targets), _p(loss), _p(lse), T, V, _code(logits)))
+
+    def rule(c, acc):
+        if c.dtype != torch.float32 or not c.is_contiguous():
+            raise TypeError("cross_entropy: the cotangent of the losses must be contiguous float32")
+        dz = torch.empty_like(logits)
+        N.check(N.lib().emi_cross_entropy_bwd(_stream(), _p(logits), _p(targets), _p(lse), _p(c), _p(dz), T, V,
+                                              _code(logits)))
+        return _accumulate(acc[0], dz), None
+
+    Tape.record((logits, targets), loss, rule)
+    tans = _tan(logits)
+    if tans is not None and tans[0] is not None:
+        tl = torch.empty_like(loss)
+        N.check(N.lib().emi_cross_entropy_jvp(_stream(), _p(logits), _p(targets), _p(lse), _p(tans[0]), _p(tl), T, V,
+                                              _code(logits)))
+        _set_tan(loss, tl)
+    return loss
 
 
 def select(w, i):

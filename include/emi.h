@@ -276,6 +276,26 @@ int emi_embedding_bwd(emi_stream_t stream, const int32_t* tokens, const void* dx
                       void* workspace, size_t workspace_bytes, int64_t n_tokens, int64_t vocab,
                       int64_t dim, int dtype);
 
+/* Softmax cross-entropy of logits[tokens, vocab] against integer targets, the loss
+ * that follows the classifier (the classifier is commented out at test/llama.py:236;
+ * the reference's llama test stops at the final RMSNorm, so this operator has no
+ * reference call site: its definition is the standard one, per token
+ *   loss = logsumexp(z) - z[target]).
+ * fwd writes loss and lse (both f32[tokens]); bwd writes
+ *   dlogits = (exp(z - lse) - onehot(target)) * dloss      (dloss f32[tokens], dlogits in dtype);
+ * jvp writes tloss = sum_v exp(z_v - lse) tz_v - tz[target] (f32[tokens]).
+ * A token whose target lies outside [0, vocab) is masked: zero loss, gradient and
+ * tangent.  targets: int32[tokens]; vocab <= 2^24.  Rows that are not whole 16-byte
+ * chunks (vocab % 8 for bf16, % 4 for f32) take a scalar path. */
+int emi_cross_entropy_fwd(emi_stream_t stream, const void* logits, const int32_t* targets, float* loss,
+                          float* lse, int64_t tokens, int64_t vocab, int dtype);
+int emi_cross_entropy_bwd(emi_stream_t stream, const void* logits, const int32_t* targets,
+                          const float* lse, const float* dloss, void* dlogits, int64_t tokens,
+                          int64_t vocab, int dtype);
+int emi_cross_entropy_jvp(emi_stream_t stream, const void* logits, const int32_t* targets,
+                          const float* lse, const void* tlogits, float* tloss, int64_t tokens,
+                          int64_t vocab, int dtype);
+
 #ifdef __cplusplus
 }
 #endif

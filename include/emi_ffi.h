@@ -34,6 +34,9 @@
  *  emi_attn_step_jvp  q, k, v, o, lse, tq, tk, tv      to, workspace:u8[n]               scale:f32
  *  emi_embedding_fwd  tokens s32[..], table[V,D]       x[..,D]                           -
  *  emi_embedding_bwd  tokens s32[..], dx[..,D]         dtable[V,D] [, workspace:u8[n]]   -
+ *  emi_cross_entropy_fwd  logits[..,V], targets s32[..]  loss f32[..], lse f32[..]         -
+ *  emi_cross_entropy_bwd  logits, targets, lse, dloss f32[..]  dlogits[..,V]               -
+ *  emi_cross_entropy_jvp  logits, targets, lse, tlogits  tloss f32[..]                     -
  *
  * `bshd` true: rank-4 operands are [batch, seq, heads, head_dim]; false:
  * [batch, heads, seq, head_dim].  Workspace results must be at least as large as
@@ -68,6 +71,9 @@ struct XLA_FFI_Error* emi_attn_jvp_ffi(struct XLA_FFI_CallFrame*);
 struct XLA_FFI_Error* emi_attn_step_jvp_ffi(struct XLA_FFI_CallFrame*);
 struct XLA_FFI_Error* emi_embedding_fwd_ffi(struct XLA_FFI_CallFrame*);
 struct XLA_FFI_Error* emi_embedding_bwd_ffi(struct XLA_FFI_CallFrame*);
+struct XLA_FFI_Error* emi_cross_entropy_fwd_ffi(struct XLA_FFI_CallFrame*);
+struct XLA_FFI_Error* emi_cross_entropy_bwd_ffi(struct XLA_FFI_CallFrame*);
+struct XLA_FFI_Error* emi_cross_entropy_jvp_ffi(struct XLA_FFI_CallFrame*);
 
 /* Number of targets and the i-th (name, handler); for registration from Python
  * with jax.ffi.register_ffi_target(name, capsule(handler), platform="ROCM"). */

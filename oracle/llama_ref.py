@@ -428,6 +428,49 @@ def model_bwd(dout, weights, config, fcache, eps=EPS):
 
 
 # ---------------------------------------------------------------------------
+# 4b. Softmax cross-entropy on the logits.  The reference's llama test stops before
+#     the classifier (test/llama.py:236 is commented out), so there is no reference
+#     call site; the definition is the standard one (per token logsumexp(z) - z[t]),
+#     built from the same softmax as test/llama.py:13-18.  Pinned by closed forms
+#     (uniform logits give log V; shifting a row changes nothing; gradient rows sum
+#     to zero), by scipy's logsumexp, by torch's float64 cross_entropy + autograd and
+#     by central finite differences (tests/test_oracle_llama.py).
+# ---------------------------------------------------------------------------
+
+def cross_entropy_fwd(logits, targets):
+    """(loss[...], lse[...]) for logits [..., V] and integer targets [...]; a target outside [0, V) masks its token."""
+    z = np.asarray(logits, dtype=np.float64)
+    t = np.asarray(targets)
+    m = z.max(axis=-1, keepdims=True)                                     # test/llama.py:16 (max subtracted first)
+    lse = (m + np.log(np.exp(z - m).sum(axis=-1, keepdims=True)))[..., 0]
+    live = (t >= 0) & (t < z.shape[-1])
+    picked = np.take_along_axis(z, np.where(live, t, 0)[..., None].astype(np.int64), axis=-1)[..., 0]
+    return np.where(live, lse - picked, 0.0), lse
+
+
+def cross_entropy_bwd(logits, targets, dloss):
+    """dlogits = (softmax(z) - onehot(t)) * dloss."""
+    z = np.asarray(logits, dtype=np.float64)
+    t = np.asarray(targets)
+    _, lse = cross_entropy_fwd(z, t)
+    live = (t >= 0) & (t < z.shape[-1])
+    p = np.exp(z - lse[..., None])
+    onehot = (np.arange(z.shape[-1]) == np.where(live, t, -1)[..., None]).astype(np.float64)
+    return (p - onehot) * np.where(live, np.asarray(dloss, dtype=np.float64), 0.0)[..., None]
+
+
+def cross_entropy_jvp(logits, targets, tlogits):
+    """tloss = sum_v softmax(z)_v tz_v - tz[t]."""
+    z = np.asarray(logits, dtype=np.float64)
+    tz = np.asarray(tlogits, dtype=np.float64)
+    t = np.asarray(targets)
+    _, lse = cross_entropy_fwd(z, t)
+    live = (t >= 0) & (t < z.shape[-1])
+    picked = np.take_along_axis(tz, np.where(live, t, 0)[..., None].astype(np.int64), axis=-1)[..., 0]
+    return np.where(live, (np.exp(z - lse[..., None]) * tz).sum(axis=-1) - picked, 0.0)
+
+
+# ---------------------------------------------------------------------------
 # 5. Seeded synthetic inputs for the benchmark configurations
 # ---------------------------------------------------------------------------
 

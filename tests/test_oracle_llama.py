@@ -246,3 +246,49 @@ def test_forward_mode_matches_reverse_mode_and_finite_differences():
     up, _ = L.model_fwd(x + h * tx, {k: w[k] + h * tw[k] for k in w}, cfg)
     dn, _ = L.model_fwd(x - h * tx, {k: w[k] - h * tw[k] for k in w}, cfg)
     np.testing.assert_allclose(ty, (up - dn) / (2 * h), rtol=2e-5, atol=1e-6)
+
+
+def test_cross_entropy_oracle_is_pinned():
+    """The loss on the logits has no call site in the reference (the classifier is commented out at
+    test/llama.py:236), so the oracle's definition is pinned by what the mathematics fixes and by library
+    routines: uniform logits give log V, a shifted row gives the same loss, gradient rows sum to zero, scipy's
+    logsumexp, torch's float64 cross_entropy with autograd, central finite differences and the identity
+    <J v, w> = <v, J^T w>."""
+    from scipy.special import logsumexp
+
+    rng = np.random.default_rng(11)
+    T, V = 7, 53
+    z = rng.normal(size=(T, V)) * 3.0
+    t = rng.integers(0, V, size=(T,))
+    loss, lse = L.cross_entropy_fwd(z, t)
+    # closed forms
+    u_loss, u_lse = L.cross_entropy_fwd(np.full((2, V), 1.75), np.array([0, V - 1]))
+    np.testing.assert_allclose(u_loss, np.log(V), rtol=1e-14)
+    np.testing.assert_allclose(u_lse, 1.75 + np.log(V), rtol=1e-14)
+    np.testing.assert_allclose(L.cross_entropy_fwd(z + 100.0, t)[0], loss, rtol=1e-12)
+    big = np.zeros((1, 4)); big[0, 2] = 1000.0                      # no overflow; the hot class costs nothing
+    assert L.cross_entropy_fwd(big, np.array([2]))[0][0] == 0.0 and L.cross_entropy_fwd(big, np.array([0]))[0][0] == 1000.0
+    # library routines
+    np.testing.assert_allclose(lse, logsumexp(z, axis=-1), rtol=1e-14)
+    zt = torch.tensor(z, dtype=torch.float64, requires_grad=True)
+    lt = torch.nn.functional.cross_entropy(zt, torch.tensor(t), reduction="none")
+    np.testing.assert_allclose(loss, lt.detach().numpy(), rtol=1e-13)
+    dl = rng.normal(size=(T,))
+    (gt,) = torch.autograd.grad(lt, zt, torch.tensor(dl))
+    dz = L.cross_entropy_bwd(z, t, dl)
+    np.testing.assert_allclose(dz, gt.numpy(), rtol=1e-12, atol=1e-15)
+    np.testing.assert_allclose(L.cross_entropy_bwd(z, t, np.ones(T)).sum(axis=-1), 0.0, atol=1e-14)
+    # finite differences and forward / reverse agreement
+    tz = rng.normal(size=(T, V))
+    h = 1e-6
+    fd = (L.cross_entropy_fwd(z + h * tz, t)[0] - L.cross_entropy_fwd(z - h * tz, t)[0]) / (2 * h)
+    tl = L.cross_entropy_jvp(z, t, tz)
+    np.testing.assert_allclose(tl, fd, rtol=1e-7, atol=1e-9)
+    np.testing.assert_allclose((tl * dl).sum(), (tz * dz).sum(), rtol=1e-12)
+    # masked tokens
+    tm = t.copy(); tm[[1, 4]] = [-1, V]
+    lm, _ = L.cross_entropy_fwd(z, tm)
+    assert lm[1] == 0.0 and lm[4] == 0.0 and np.array_equal(np.delete(lm, [1, 4]), np.delete(loss, [1, 4]))
+    dm = L.cross_entropy_bwd(z, tm, dl)
+    assert not dm[1].any() and not dm[4].any()
+    assert not L.cross_entropy_jvp(z, tm, tz)[[1, 4]].any()
