@@ -787,7 +787,10 @@ __global__ __launch_bounds__(512) void gemm_bf16_pingpong_kernel(const uint16_t*
 
 // ---------------------------------------------------------------------------
 // Generic path: any dtype/shape/alignment, fp32 MFMA (v_mfma_f32_32x32x2_f32).
-// 256 threads, 128x128x16 tile, LDS tiles stored k-major as fp32.
+// 256 threads, LDS tiles stored k-major as fp32.  These problems are small, so a block's time is
+// the number of K-steps times the latency of one step: the steps are deep (64 for the 64x64 tile,
+// 32 for 128x128) and the next step's elements are loaded into registers while the matrix cores
+// work on the current one.
 // ---------------------------------------------------------------------------
 // WT: 32x32 MFMA tiles per wavefront and dimension: 2 -> 128x128 block tiles, 1 -> 64x64 (small problems: more
 // blocks, shorter iterations).
@@ -796,7 +799,8 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const T* __restrict__
                                                            T* C, int M, int N, int K, int64_t lda, int64_t ldb,
                                                            int64_t ldr, int64_t ldc, int trans_a, int trans_b,
                                                            float* __restrict__ part, int k_per_split) {
-  constexpr int BM = 64 * WT, BN = 64 * WT, BK = 16, PAD = 4;
+  constexpr int BM = 64 * WT, BN = 64 * WT, BK = 128 / (WT * WT > 1 ? 4 : 2), PAD = 1;
+  constexpr int NA = BM * BK / 256, NB = BN * BK / 256;      // elements per thread and step
   __shared__ float sA[BK][BM + PAD];
   __shared__ float sB[BK][BN + PAD];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -815,27 +819,48 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const T* __restrict__
   const int k_lo = part ? blockIdx.z * k_per_split : 0;
   const int k_hi = part ? (k_lo + k_per_split < K ? k_lo + k_per_split : K) : K;
   K = k_hi;
-  for (int k0 = k_lo; k0 < K; k0 += BK) {
-    // A tile: BM x 16 elements, BM / 16 per thread
+  // element `it` of this thread in a tile: (m, k) for A, (n, k) for B; the fast index follows memory
+  auto a_mk = [&](int it, int& m, int& k) {
+    if (trans_a) { m = tid & (BM - 1); k = tid / BM + it * (256 / BM); }     // A is [K,M]: m contiguous
+    else { k = tid & (BK - 1); m = tid / BK + it * (256 / BK); }             // A is [M,K]: k contiguous
+  };
+  auto b_nk = [&](int it, int& n, int& k) {
+    if (trans_b) { k = tid & (BK - 1); n = tid / BK + it * (256 / BK); }     // B is [N,K]
+    else { n = tid & (BN - 1); k = tid / BN + it * (256 / BN); }             // B is [K,N]
+  };
+  float ra[NA], rb[NB];
+  auto load_step = [&](int k0) {
 #pragma unroll
-    for (int it = 0; it < BM / 16; it++) {
+    for (int it = 0; it < NA; it++) {
       int m, k;
-      if (trans_a) { m = tid & (BM - 1); k = tid / BM + it * (256 / BM); }   // A is [K,M]: m contiguous
-      else { k = tid & 15; m = (tid >> 4) + it * 16; }                // A is [M,K]: k contiguous
-      float v = 0.f;
-      if (m0 + m < M && k0 + k < K) v = to_f32(trans_a ? A[(int64_t)(k0 + k) * lda + m0 + m] : A[(int64_t)(m0 + m) * lda + k0 + k]);
-      sA[k][m] = v;
+      a_mk(it, m, k);
+      ra[it] = (m0 + m < M && k0 + k < K)
+                   ? to_f32(trans_a ? A[(int64_t)(k0 + k) * lda + m0 + m] : A[(int64_t)(m0 + m) * lda + k0 + k]) : 0.f;
     }
 #pragma unroll
-    for (int it = 0; it < BN / 16; it++) {
+    for (int it = 0; it < NB; it++) {
       int n, k;
-      if (trans_b) { k = tid & 15; n = (tid >> 4) + it * 16; }        // B is [N,K]
-      else { n = tid & (BN - 1); k = tid / BN + it * (256 / BN); }    // B is [K,N]
-      float v = 0.f;
-      if (n0 + n < N && k0 + k < K) v = to_f32(trans_b ? B[(int64_t)(n0 + n) * ldb + k0 + k] : B[(int64_t)(k0 + k) * ldb + n0 + n]);
-      sB[k][n] = v;
+      b_nk(it, n, k);
+      rb[it] = (n0 + n < N && k0 + k < K)
+                   ? to_f32(trans_b ? B[(int64_t)(n0 + n) * ldb + k0 + k] : B[(int64_t)(k0 + k) * ldb + n0 + n]) : 0.f;
+    }
+  };
+  if (k_lo < K) load_step(k_lo);
+  for (int k0 = k_lo; k0 < K; k0 += BK) {
+#pragma unroll
+    for (int it = 0; it < NA; it++) {
+      int m, k;
+      a_mk(it, m, k);
+      sA[k][m] = ra[it];
+    }
+#pragma unroll
+    for (int it = 0; it < NB; it++) {
+      int n, k;
+      b_nk(it, n, k);
+      sB[k][n] = rb[it];
     }
     __syncthreads();
+    if (k0 + BK < K) load_step(k0 + BK);           // in flight while this step is multiplied
 #pragma unroll
     for (int kk = 0; kk < BK; kk += 2) {
       const int k = kk + (lane >> 5);
