@@ -245,7 +245,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_kernel(const uint16_t* 
                                                                  const uint16_t* __restrict__ B, const uint16_t* R,
                                                                  uint16_t* C, int M, int N, int K, int lda, int ldb,
                                                                  int ldr, int ldc, uint32_t a_bytes, uint32_t b_bytes,
-                                                                 int vec_ok) {
+                                                                 int vec_ok, float* __restrict__ part, int k_per_split) {
   constexpr int NW = WM * WN;
   constexpr int KS = BK / 16;
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
@@ -312,16 +312,20 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_kernel(const uint16_t* 
       for (int j = 0; j < TN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[j], a[i], acc[i][j], 0, 0, 0);
   };
 
-  const int nk = (K + BK - 1) / BK;
+  // split-K (part != nullptr): block z owns k in [z * k_per_split, ...) and leaves an fp32 partial
+  // tile in part[z][M][N]; gemm_splitk_reduce_kernel adds the partials (and R) in fixed order
+  const int k_lo = part ? blockIdx.z * k_per_split : 0;
+  if (part) K = k_lo + k_per_split < K ? k_lo + k_per_split : K;
+  const int nk = (K - k_lo + BK - 1) / BK;
   // Operand fragments are double buffered: the LDS reads of the next k-step are
   // issued before the MFMAs of the current one so their latency hides behind them.
   bf16x8_t fa[2][TM], fb[2][TN];
   if constexpr (NSTAGE == 2) {
-    issue_loads(0, 0);
+    issue_loads(0, k_lo);
     wait_vmcnt<0>();
     __syncthreads();
     for (int t = 0; t < nk; t++) {
-      if (t + 1 < nk) issue_loads((t + 1) & 1, (t + 1) * BK);
+      if (t + 1 < nk) issue_loads((t + 1) & 1, k_lo + (t + 1) * BK);
       load_frags(t & 1, 0, fa[0], fb[0]);
 #pragma unroll
       for (int kk = 0; kk < KS; kk++) {
@@ -335,14 +339,14 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_kernel(const uint16_t* 
     }
   } else {
     static_assert(KS % 2 == 0, "fragment double buffering assumes an even number of k-steps per tile");
-    issue_loads(0, 0);
-    issue_loads(1, BK);
-    issue_loads(2, 2 * BK);
+    issue_loads(0, k_lo);
+    issue_loads(1, k_lo + BK);
+    issue_loads(2, k_lo + 2 * BK);
     wait_vmcnt<LPT>();     // tiles 0 and 1 have landed
     __syncthreads();
     load_frags(0, 0, fa[0], fb[0]);
     for (int t = 0; t < nk; t++) {
-      issue_loads((t + 3) & 3, (t + 3) * BK);
+      issue_loads((t + 3) & 3, k_lo + (t + 3) * BK);
 #pragma unroll
       for (int kk = 0; kk < KS; kk++) {
         if (kk + 1 < KS) load_frags(t & 3, kk + 1, fa[(kk + 1) & 1], fb[(kk + 1) & 1]);
@@ -360,6 +364,31 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_kernel(const uint16_t* 
 
   constexpr int WR = BM / WM, WC = BN / WN;
   static_assert(NW * WR * WC * 2 <= NSTAGE * STAGE, "epilogue staging does not fit in the LDS allocation");
+  if (part != nullptr) {
+    // accumulator layout (swapped operands): register 4q+e of lane l holds row l%32, column 8q + 4(l/32) + e
+    float* pz = part + (int64_t)blockIdx.z * M * N;
+    const bool vec4 = (N & 3) == 0;
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int j = 0; j < TN; j++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          const int row = m0 + wm * WR + i * 32 + (lane & 31);
+          const int col = n0 + wn * WC + j * 32 + q * 8 + (lane >> 5) * 4;
+          if (row < M && col < N) {
+            float* dst = pz + (int64_t)row * N + col;
+            if (vec4 && col + 4 <= N) {
+              *reinterpret_cast<float4*>(dst) = make_float4(acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+            } else {
+#pragma unroll
+              for (int e = 0; e < 4; e++)
+                if (col + e < N) dst[e] = acc[i][j][4 * q + e];
+            }
+          }
+        }
+    return;
+  }
   epilogue_bf16<WR, WC, TM, TN>(acc, smem, wave, lane, m0 + wm * WR, n0 + wn * WC, R, C, M, N, ldr, ldc, vec_ok);
 }
 
@@ -926,7 +955,7 @@ static int generic_splits(int64_t M, int64_t N, int64_t K) {
 
 template <int BM, int BN, int BK, int NSTAGE, int WM, int WN, bool AK, bool BKM>
 static int launch_bf16(hipStream_t st, const void* A, const void* B, const void* R, void* C, int M, int N, int K, int lda,
-                       int ldb, int ldr, int ldc, uint32_t a_bytes, uint32_t b_bytes) {
+                       int ldb, int ldr, int ldc, uint32_t a_bytes, uint32_t b_bytes, float* part = nullptr, int splits = 1) {
   // 16-byte epilogue accesses need aligned rows of C (and R)
   const int vec_ok = ((reinterpret_cast<uintptr_t>(C) & 15) == 0 && ldc % 8 == 0 &&
                       (R == nullptr || ((reinterpret_cast<uintptr_t>(R) & 15) == 0 && ldr % 8 == 0)))
@@ -940,9 +969,21 @@ static int launch_bf16(hipStream_t st, const void* A, const void* B, const void*
     configured = true;
   }
   const int tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+  if (part != nullptr && splits > 1) {
+    const int kps = (((K + splits - 1) / splits) + BK - 1) / BK * BK;
+    const int nz = (K + kps - 1) / kps;
+    hipLaunchKernelGGL(kern, dim3(tiles, 1, nz), dim3(WM * WN * 64), smem, st, static_cast<const uint16_t*>(A),
+                       static_cast<const uint16_t*>(B), static_cast<const uint16_t*>(R), static_cast<uint16_t*>(C), M, N, K,
+                       lda, ldb, ldr, ldc, a_bytes, b_bytes, vec_ok, part, kps);
+    EMI_CHECK_LAUNCH("emi_gemm(split-K)");
+    hipLaunchKernelGGL(gemm_splitk_reduce_kernel<bf16>, dim3((unsigned)(((int64_t)M * N + 255) / 256)), dim3(256), 0, st, part,
+                       static_cast<const bf16*>(R), static_cast<bf16*>(C), M, N, nz, (int64_t)ldr, (int64_t)ldc);
+    EMI_CHECK_LAUNCH("emi_gemm(split-K reduce)");
+    return EMI_OK;
+  }
   hipLaunchKernelGGL(kern, dim3(tiles), dim3(WM * WN * 64), smem, st, static_cast<const uint16_t*>(A),
                      static_cast<const uint16_t*>(B), static_cast<const uint16_t*>(R), static_cast<uint16_t*>(C), M, N, K,
-                     lda, ldb, ldr, ldc, a_bytes, b_bytes, vec_ok);
+                     lda, ldb, ldr, ldc, a_bytes, b_bytes, vec_ok, static_cast<float*>(nullptr), 0);
   EMI_CHECK_LAUNCH("emi_gemm");
   return EMI_OK;
 }
@@ -982,10 +1023,29 @@ static int tile_override() {
   return v;
 }
 
+// The 128x128 bf16 kernel on few tiles and a long contraction (the weight gradients of a small model:
+// dW[768, 768] over 8192 tokens is 36 tiles): one block per CU, at least 512 of K per block.
+static int bf16_splits(int64_t M, int64_t N, int64_t K) {
+  if (((M + 255) / 256) * ((N + 255) / 256) >= 192) return 1;         // the 256x256 ping-pong kernel takes these
+  const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
+  if (tiles > 128 || K < 2048) return 1;
+  int64_t s = 256 / tiles;
+  if (s > K / 512) s = K / 512;
+  return (int)(s < 2 ? 1 : (s > 64 ? 64 : s));
+}
+
 template <bool AK, bool BKM>
 static int launch_bf16_layout(hipStream_t st, const void* A, const void* B, const void* R, void* C, int M, int N, int K,
-                              int lda, int ldb, int ldr, int ldc, uint32_t a_bytes, uint32_t b_bytes) {
+                              int lda, int ldb, int ldr, int ldc, uint32_t a_bytes, uint32_t b_bytes, void* workspace,
+                              size_t workspace_bytes) {
   int cfg = tile_override();
+  if (cfg == 0) {
+    const int splits = bf16_splits(M, N, K);
+    if (splits > 1 && workspace != nullptr && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0 &&
+        workspace_bytes >= (size_t)splits * M * N * sizeof(float))
+      return launch_bf16<128, 128, 64, 2, 2, 2, AK, BKM>(st, A, B, R, C, M, N, K, lda, ldb, ldr, ldc, a_bytes, b_bytes,
+                                                        static_cast<float*>(workspace), splits);
+  }
   if (cfg == 0) {
     // 256x256 tiles when they fill the chip (the ping-pong kernel for two
     // k-contiguous operands), else 128x128.
@@ -1051,8 +1111,10 @@ extern "C" size_t emi_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int 
   const size_t skinny = skinny_workspace_bytes(M, N, K, trans_a, trans_b, dtype);
   if (skinny) return skinny;
   if (M <= 0 || N <= 0 || K <= 0) return 0;
-  // fp32 (and bf16 shapes the fast path does not take) with few tiles and a long contraction: split-K partials
-  const int splits = generic_splits(M, N, K);
+  // few tiles and a long contraction: split-K partials (the larger of what the fp32 / odd-shape path and the
+  // 128x128 bf16 kernel would use, since alignment decides between them at launch time)
+  int splits = generic_splits(M, N, K);
+  if (dtype == EMI_BF16 && bf16_splits(M, N, K) > splits) splits = bf16_splits(M, N, K);
   return splits > 1 ? (size_t)splits * M * N * sizeof(float) : 0;
 }
 
@@ -1094,12 +1156,12 @@ extern "C" int emi_gemm_ws(emi_stream_t stream, const void* A, const void* B, co
       const int m = (int)M, n = (int)N, k = (int)K;
       const uint32_t ab = (uint32_t)a_bytes, bb = (uint32_t)b_bytes;
       if (!trans_a && trans_b)
-        return launch_bf16_layout<false, false>(st, A, B, R, C, m, n, k, (int)lda, (int)ldb, (int)ldr, (int)ldc, ab, bb);
+        return launch_bf16_layout<false, false>(st, A, B, R, C, m, n, k, (int)lda, (int)ldb, (int)ldr, (int)ldc, ab, bb, workspace, workspace_bytes);
       if (!trans_a && !trans_b)
-        return launch_bf16_layout<false, true>(st, A, B, R, C, m, n, k, (int)lda, (int)ldb, (int)ldr, (int)ldc, ab, bb);
+        return launch_bf16_layout<false, true>(st, A, B, R, C, m, n, k, (int)lda, (int)ldb, (int)ldr, (int)ldc, ab, bb, workspace, workspace_bytes);
       if (trans_a && !trans_b)
-        return launch_bf16_layout<true, true>(st, A, B, R, C, m, n, k, (int)lda, (int)ldb, (int)ldr, (int)ldc, ab, bb);
-      return launch_bf16_layout<true, false>(st, A, B, R, C, m, n, k, (int)lda, (int)ldb, (int)ldr, (int)ldc, ab, bb);
+        return launch_bf16_layout<true, true>(st, A, B, R, C, m, n, k, (int)lda, (int)ldb, (int)ldr, (int)ldc, ab, bb, workspace, workspace_bytes);
+      return launch_bf16_layout<true, false>(st, A, B, R, C, m, n, k, (int)lda, (int)ldb, (int)ldr, (int)ldc, ab, bb, workspace, workspace_bytes);
     }
     return launch_generic<bf16>(st, A, B, R, C, (int)M, (int)N, (int)K, lda, ldb, ldr, ldc, trans_a, trans_b, workspace, workspace_bytes);
   }

@@ -103,6 +103,8 @@ GEMM_SHAPES = [
     (64, 288, 288),      # C1 projection
     (4096, 3072, 264),   # fast path, 256-tiles (192 tiles)
     (4000, 3080, 128),   # 256-tiles, ragged M and N
+    (264, 136, 4104),    # few tiles, long contraction: split-K with fp32 partials (bf16 128-tile kernel and fp32 kernel)
+    (100, 200, 2600),    # split-K on the generic kernel for both dtypes where M is not a multiple of 8
 ]
 
 
