@@ -1024,13 +1024,13 @@ static int tile_override() {
 }
 
 // The 128x128 bf16 kernel on few tiles and a long contraction (the weight gradients of a small model:
-// dW[768, 768] over 8192 tokens is 36 tiles): one block per CU, at least 512 of K per block.
+// dW[768, 768] over 8192 tokens is 36 tiles): two blocks per CU, at least 1024 of K per block.
 static int bf16_splits(int64_t M, int64_t N, int64_t K) {
   if (((M + 255) / 256) * ((N + 255) / 256) >= 192) return 1;         // the 256x256 ping-pong kernel takes these
   const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
   if (tiles > 128 || K < 2048) return 1;
-  int64_t s = 256 / tiles;
-  if (s > K / 512) s = K / 512;
+  int64_t s = 512 / tiles;
+  if (s > K / 1024) s = K / 1024;
   return (int)(s < 2 ? 1 : (s > 64 ? 64 : s));
 }
 
