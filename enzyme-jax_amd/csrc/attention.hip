@@ -70,13 +70,53 @@ __device__ __forceinline__ void attn_block_coords(int* blk, int* bh) {
 // Generic path
 // ===========================================================================
 
+// Four consecutive elements as fp32 (8- or 16-byte load; the caller guarantees the alignment).
+__device__ __forceinline__ void load4(const float* p, float (&v)[4]) {
+  const float4 a = *reinterpret_cast<const float4*>(p);
+  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+}
+__device__ __forceinline__ void load4(const bf16* p, float (&v)[4]) {
+  const uint2 a = *reinterpret_cast<const uint2*>(p);
+  v[0] = __uint_as_float(a.x << 16); v[1] = __uint_as_float(a.x & 0xffff0000u);
+  v[2] = __uint_as_float(a.y << 16); v[3] = __uint_as_float(a.y & 0xffff0000u);
+}
+
+// a . b and c . e over d elements (rows of two operand pairs that are always needed together); vec4: rows
+// start on 4-element boundaries and d is a multiple of 4, so the loads are 4 elements wide.
+template <typename T, bool TWO>
+__device__ __forceinline__ void row_dots(const T* a, const T* b, const T* c, const T* e, int d, bool vec4, float* ab,
+                                         float* ce) {
+  float s0 = 0.f, s1 = 0.f;
+  int i = 0;
+  if (vec4) {
+#pragma unroll 4
+    for (; i + 4 <= d; i += 4) {
+      float x[4], y[4];
+      load4(a + i, x);
+      load4(b + i, y);
+      s0 += x[0] * y[0] + x[1] * y[1] + x[2] * y[2] + x[3] * y[3];
+      if constexpr (TWO) {
+        load4(c + i, x);
+        load4(e + i, y);
+        s1 += x[0] * y[0] + x[1] * y[1] + x[2] * y[2] + x[3] * y[3];
+      }
+    }
+  }
+  for (; i < d; i++) {
+    s0 += to_f32(a[i]) * to_f32(b[i]);
+    if constexpr (TWO) s1 += to_f32(c[i]) * to_f32(e[i]);
+  }
+  *ab = s0;
+  if constexpr (TWO) *ce = s1;
+}
+
 // One wavefront per query.  Lanes split the keys of a 64-key chunk for the
-// scores and split head_dim for the output.
+// scores and split head_dim for the output (four rows of V in flight at a time).
 template <typename T>
 __global__ __launch_bounds__(256) void attn_fwd_generic_kernel(const T* __restrict__ q, const T* __restrict__ k,
                                                                const T* __restrict__ v, T* __restrict__ o,
                                                                float* __restrict__ lse, AttnShape sh, int d, float scale,
-                                                               int causal) {
+                                                               int causal, int vec4) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int qi = blockIdx.x * 4 + wave;
   const int bh = blockIdx.y;
@@ -90,9 +130,8 @@ __global__ __launch_bounds__(256) void attn_fwd_generic_kernel(const T* __restri
     const int key = k0 + lane;
     float s = kNegBig;
     if (key < nkeys) {
-      const T* kr = k + base + (int64_t)key * sh.ss;
-      float dot = 0.f;
-      for (int i = 0; i < d; i++) dot += to_f32(qr[i]) * to_f32(kr[i]);
+      float dot;
+      row_dots<T, false>(qr, k + base + (int64_t)key * sh.ss, qr, qr, d, vec4 != 0, &dot, nullptr);
       s = dot * scale;
     }
     const float m_new = fmaxf(m, wave_max(s));
@@ -102,13 +141,25 @@ __global__ __launch_bounds__(256) void attn_fwd_generic_kernel(const T* __restri
 #pragma unroll
     for (int c = 0; c < 4; c++) acc[c] *= alpha;
     const int cnt = nkeys - k0 < 64 ? nkeys - k0 : 64;
-    for (int j = 0; j < cnt; j++) {
-      const float pj = __shfl(p, j, 64);
-      const T* vr = v + base + (int64_t)(k0 + j) * sh.ss;
+    for (int j = 0; j < cnt; j += 4) {
+      float pj[4];
+      const T* vr[4];
+#pragma unroll
+      for (int u = 0; u < 4; u++) {                      // rows past the last key: weight 0, row clamped
+        pj[u] = __shfl(p, (j + u) & 63, 64);
+        const int row = k0 + j + u < nkeys ? k0 + j + u : nkeys - 1;
+        vr[u] = v + base + (int64_t)row * sh.ss;
+      }
 #pragma unroll
       for (int c = 0; c < 4; c++) {
         const int i = lane + c * 64;
-        if (i < d) acc[c] += pj * to_f32(vr[i]);
+        if (i < d) {
+          float x[4];
+#pragma unroll
+          for (int u = 0; u < 4; u++) x[u] = to_f32(vr[u][i]);
+#pragma unroll
+          for (int u = 0; u < 4; u++) acc[c] += pj[u] * x[u];
+        }
       }
     }
     m = m_new;
@@ -143,7 +194,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_generic_kernel(const T* __res
                                                                   const T* __restrict__ v, const T* __restrict__ d_o,
                                                                   const float* __restrict__ lse,
                                                                   const float* __restrict__ delta, T* __restrict__ dq,
-                                                                  AttnShape sh, int d, float scale, int causal) {
+                                                                  AttnShape sh, int d, float scale, int causal, int vec4) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int qi = blockIdx.x * 4 + wave;
   const int bh = blockIdx.y;
@@ -158,24 +209,31 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_generic_kernel(const T* __res
     const int key = k0 + lane;
     float ds = 0.f;
     if (key < nkeys) {
-      const T* kr = k + base + (int64_t)key * sh.ss;
-      const T* vr = v + base + (int64_t)key * sh.ss;
-      float dot = 0.f, dp = 0.f;
-      for (int i = 0; i < d; i++) {
-        dot += to_f32(qr[i]) * to_f32(kr[i]);
-        dp += to_f32(dor[i]) * to_f32(vr[i]);
-      }
+      float dot, dp;
+      row_dots<T, true>(qr, k + base + (int64_t)key * sh.ss, dor, v + base + (int64_t)key * sh.ss, d, vec4 != 0, &dot, &dp);
       const float p = expf(dot * scale - L);
       ds = p * (dp - dl) * scale;
     }
     const int cnt = nkeys - k0 < 64 ? nkeys - k0 : 64;
-    for (int j = 0; j < cnt; j++) {
-      const float dsj = __shfl(ds, j, 64);
-      const T* kr = k + base + (int64_t)(k0 + j) * sh.ss;
+    for (int j = 0; j < cnt; j += 4) {
+      float dsj[4];
+      const T* kr[4];
+#pragma unroll
+      for (int u = 0; u < 4; u++) {                      // rows past the last key: weight 0, row clamped
+        dsj[u] = __shfl(ds, (j + u) & 63, 64);
+        const int row = k0 + j + u < nkeys ? k0 + j + u : nkeys - 1;
+        kr[u] = k + base + (int64_t)row * sh.ss;
+      }
 #pragma unroll
       for (int c = 0; c < 4; c++) {
         const int i = lane + c * 64;
-        if (i < d) acc[c] += dsj * to_f32(kr[i]);
+        if (i < d) {
+          float x[4];
+#pragma unroll
+          for (int u = 0; u < 4; u++) x[u] = to_f32(kr[u][i]);
+#pragma unroll
+          for (int u = 0; u < 4; u++) acc[c] += dsj[u] * x[u];
+        }
       }
     }
   }
@@ -194,7 +252,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_generic_kernel(const T* __re
                                                                    const float* __restrict__ lse,
                                                                    const float* __restrict__ delta, T* __restrict__ dk,
                                                                    T* __restrict__ dv, AttnShape sh, int d, float scale,
-                                                                   int causal) {
+                                                                   int causal, int vec4) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int ki = blockIdx.x * 4 + wave;
   const int bh = blockIdx.y;
@@ -208,27 +266,33 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_generic_kernel(const T* __re
     const int qi = q0 + lane;
     float p = 0.f, ds = 0.f;
     if (qi < sh.seq) {
-      const T* qr = q + base + (int64_t)qi * sh.ss;
-      const T* dor = d_o + base + (int64_t)qi * sh.ss;
-      float dot = 0.f, dp = 0.f;
-      for (int i = 0; i < d; i++) {
-        dot += to_f32(qr[i]) * to_f32(kr[i]);
-        dp += to_f32(dor[i]) * to_f32(vr[i]);
-      }
+      float dot, dp;
+      row_dots<T, true>(q + base + (int64_t)qi * sh.ss, kr, d_o + base + (int64_t)qi * sh.ss, vr, d, vec4 != 0, &dot, &dp);
       p = expf(dot * scale - lse[(int64_t)bh * sh.seq + qi]);
       ds = p * (dp - delta[(int64_t)bh * sh.seq + qi]) * scale;
     }
     const int cnt = sh.seq - q0 < 64 ? sh.seq - q0 : 64;
-    for (int j = 0; j < cnt; j++) {
-      const float pj = __shfl(p, j, 64), dsj = __shfl(ds, j, 64);
-      const T* qr = q + base + (int64_t)(q0 + j) * sh.ss;
-      const T* dor = d_o + base + (int64_t)(q0 + j) * sh.ss;
+    for (int j = 0; j < cnt; j += 2) {
+      float pj[2], dsj[2];
+      const T* qr[2];
+      const T* dor[2];
+#pragma unroll
+      for (int u = 0; u < 2; u++) {                      // rows past the last query: weight 0, row clamped
+        pj[u] = __shfl(p, (j + u) & 63, 64);
+        dsj[u] = __shfl(ds, (j + u) & 63, 64);
+        const int row = q0 + j + u < sh.seq ? q0 + j + u : sh.seq - 1;
+        qr[u] = q + base + (int64_t)row * sh.ss;
+        dor[u] = d_o + base + (int64_t)row * sh.ss;
+      }
 #pragma unroll
       for (int c = 0; c < 4; c++) {
         const int i = lane + c * 64;
         if (i < d) {
-          accv[c] += pj * to_f32(dor[i]);
-          acck[c] += dsj * to_f32(qr[i]);
+          float x[2], y[2];
+#pragma unroll
+          for (int u = 0; u < 2; u++) x[u] = to_f32(dor[u][i]), y[u] = to_f32(qr[u][i]);
+#pragma unroll
+          for (int u = 0; u < 2; u++) accv[c] += pj[u] * x[u], acck[c] += dsj[u] * y[u];
         }
       }
     }
@@ -1532,6 +1596,16 @@ extern "C" int emi_debug_attn_trace(unsigned long long* out) {
 }
 #endif
 
+// The generic kernels read four elements per load when every row starts on a 4-element boundary (8 bytes of bf16,
+// 16 of fp32) and head_dim is a multiple of 4.
+static inline int rows_vec4(int dtype, int64_t head_dim, int64_t sb, int64_t sh, int64_t ss, std::initializer_list<const void*> ptrs) {
+  const uintptr_t mask = dtype == EMI_BF16 ? 7 : 15;
+  if ((head_dim | sb | sh | ss) & 3) return 0;
+  for (const void* p : ptrs)
+    if (reinterpret_cast<uintptr_t>(p) & mask) return 0;
+  return 1;
+}
+
 extern "C" size_t emi_attn_fwd_workspace_bytes(int64_t batch, int64_t heads, int64_t seq, int64_t head_dim) {
   if (batch <= 0 || heads <= 0 || seq <= 0 || (head_dim != 64 && head_dim != 128)) return 0;
   const int64_t s_pad = (seq + 63) / 64 * 64;
@@ -1601,12 +1675,13 @@ extern "C" int emi_attn_fwd_ws(emi_stream_t stream, const void* q, const void* k
     return EMI_OK;
   }
   const dim3 grid((unsigned)((seq + 3) / 4), bh);
+  const int vec4 = rows_vec4(dtype, head_dim, shp.sb, shp.sh, shp.ss, {q, k});
   if (dtype == EMI_BF16)
     hipLaunchKernelGGL(attn_fwd_generic_kernel<bf16>, grid, dim3(256), 0, st, (const bf16*)q, (const bf16*)k,
-                       (const bf16*)v, (bf16*)o, lse, shp, (int)head_dim, scale, causal);
+                       (const bf16*)v, (bf16*)o, lse, shp, (int)head_dim, scale, causal, vec4);
   else
     hipLaunchKernelGGL(attn_fwd_generic_kernel<float>, grid, dim3(256), 0, st, (const float*)q, (const float*)k,
-                       (const float*)v, (float*)o, lse, shp, (int)head_dim, scale, causal);
+                       (const float*)v, (float*)o, lse, shp, (int)head_dim, scale, causal, vec4);
   EMI_CHECK_LAUNCH("emi_attn_fwd(generic)");
   return EMI_OK;
 }
@@ -1690,18 +1765,19 @@ extern "C" int emi_attn_bwd(emi_stream_t stream, const void* q, const void* k, c
     EMI_CHECK_LAUNCH("emi_attn_bwd(dq)");
     return EMI_OK;
   }
+  const int vec4 = rows_vec4(dtype, head_dim, shp.sb, shp.sh, shp.ss, {q, k, v, d_o});
   if (dtype == EMI_BF16) {
     hipLaunchKernelGGL(attn_bwd_dq_generic_kernel<bf16>, grid4, dim3(256), 0, st, (const bf16*)q, (const bf16*)k,
-                       (const bf16*)v, (const bf16*)d_o, lse, delta, (bf16*)dq, shp, (int)head_dim, scale, causal);
+                       (const bf16*)v, (const bf16*)d_o, lse, delta, (bf16*)dq, shp, (int)head_dim, scale, causal, vec4);
     hipLaunchKernelGGL(attn_bwd_dkv_generic_kernel<bf16>, grid4, dim3(256), 0, st, (const bf16*)q, (const bf16*)k,
                        (const bf16*)v, (const bf16*)d_o, lse, delta, (bf16*)dk, (bf16*)dv, shp, (int)head_dim, scale,
-                       causal);
+                       causal, vec4);
   } else {
     hipLaunchKernelGGL(attn_bwd_dq_generic_kernel<float>, grid4, dim3(256), 0, st, (const float*)q, (const float*)k,
-                       (const float*)v, (const float*)d_o, lse, delta, (float*)dq, shp, (int)head_dim, scale, causal);
+                       (const float*)v, (const float*)d_o, lse, delta, (float*)dq, shp, (int)head_dim, scale, causal, vec4);
     hipLaunchKernelGGL(attn_bwd_dkv_generic_kernel<float>, grid4, dim3(256), 0, st, (const float*)q, (const float*)k,
                        (const float*)v, (const float*)d_o, lse, delta, (float*)dk, (float*)dv, shp, (int)head_dim, scale,
-                       causal);
+                       causal, vec4);
   }
   EMI_CHECK_LAUNCH("emi_attn_bwd(generic)");
   return EMI_OK;
