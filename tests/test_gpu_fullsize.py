@@ -166,3 +166,44 @@ def test_c4_stories110m_full_size():
     rhs = sum(_dot(gw[k_], tw[k_]) for k_ in gw)
     print("C4 model <J v, w> = %.6g, <v, J^T w> = %.6g" % (lhs, rhs), flush=True)
     assert abs(lhs - rhs) <= 3e-2 * max(abs(lhs), abs(rhs))
+
+
+@pytest.mark.parametrize("dt", ["bf16", "f32"])
+def test_c4_logits_cross_entropy_full_size(dt):
+    """Logits [8 x 1024, 32000] of the 110M configuration: sampled tokens against the oracle (loss, adjoint row,
+    tangent), and over the whole tensor: every gradient row sums to zero and is linear in its loss cotangent, a
+    constant shift of a row leaves its loss unchanged, and <J v, w> = <v, J^T w> between the tangent and adjoint
+    kernels."""
+    from enzyme_ad.jax import ops, jvp, vjp
+
+    T, V = 8 * 1024, 32000
+    z = _randn((8, 1024, V), dt, 41, 3.0)
+    tz = _randn((8, 1024, V), dt, 42)
+    g = torch.Generator(device="cuda").manual_seed(43)
+    tgt = torch.randint(0, V, (8, 1024), device="cuda", generator=g, dtype=torch.int32)
+    dl = torch.randn((8, 1024), device="cuda", generator=g)
+    fn = lambda logits: ops.cross_entropy(logits, tgt)
+    loss, tl = jvp(fn, (z,), (tz,))
+    _, f_vjp = vjp(fn, z)
+    (dz,) = f_vjp(dl)
+    rows = [(0, 0), (3, 517), (7, 1023)]
+    for b, s_ in rows:
+        zr, tzr, t1 = host(z[b, s_]), host(tz[b, s_]), int(tgt[b, s_])
+        ref_loss, _ = L.cross_entropy_fwd(zr[None], np.array([t1]))
+        assert abs(float(loss[b, s_]) - ref_loss[0]) <= 1e-5 * max(1.0, abs(ref_loss[0]))
+        check(dz[b, s_], L.cross_entropy_bwd(zr[None], np.array([t1]), np.array([float(dl[b, s_])]))[0], dt, "dlogits row")
+        ref_tl = L.cross_entropy_jvp(zr[None], np.array([t1]), tzr[None])[0]
+        assert abs(float(tl[b, s_]) - ref_tl) <= 1e-4 * max(1.0, abs(ref_tl))
+    # rows of softmax - onehot sum to zero (up to the rounding of 32000 stored elements)
+    row_sum = dz.float().sum(dim=-1)
+    bound = (2e-2 if dt == "bf16" else 1e-4) * dl.abs().clamp_min(1e-3)
+    assert bool((row_sum.abs() <= bound).all()), float((row_sum.abs() / bound).max())
+    # exact linearity in the cotangent under a power-of-two scale
+    (dz4,) = f_vjp(dl * 4.0)
+    assert torch.equal(dz4, dz * 4.0)
+    # a shifted row has the same loss (fp32 logits; in bf16 the shift would round the logits)
+    if dt == "f32":
+        shifted = ops.cross_entropy(z[:1] + 8.0, tgt[:1])
+        assert float((shifted - loss[:1]).abs().max()) <= 2e-5
+    lhs, rhs = _dot(tl, dl), _dot(tz, dz)
+    assert abs(lhs - rhs) <= (2e-2 if dt == "bf16" else 1e-4) * max(abs(lhs), abs(rhs), 1.0), (lhs, rhs)
