@@ -358,7 +358,7 @@ def bench_frontend(iters):
 
 def bench_models(iters):
     """The two whole-model configurations: tokens in, logits out, fwd + VJP with a cotangent on the
-    logits.  C4 stories110M (dim 768, hidden 2048, 12 layers, 12 heads x 64, vocab 32000, seq 1024,
+    logits (and, as `loss_*`, tokens in, mean cross-entropy out, fwd + VJP).  C4 stories110M (dim 768, hidden 2048, 12 layers, 12 heads x 64, vocab 32000, seq 1024,
     batch 8, bf16) and C1 stories15M (dim 288, hidden 768, 6 layers, 6 heads x 48, seq 256, batch 1,
     fp32)."""
     import torch
@@ -387,6 +387,21 @@ def bench_models(iters):
 
         t = event_time(step, iters, warmup=2)
         out[name] = dict(ms_per_step=round(t * 1e3, 3), tokens_per_s=round(B * S / t, 1), tokens_per_step=B * S)
+        # the same model as a training step: mean cross-entropy against random targets, all weight gradients
+        tgt = torch.randint(0, V, (B, S), generator=g, device="cuda", dtype=torch.int32)
+        one = torch.ones((), device="cuda")
+
+        @enzyme_jax_ir(pipeline_options=JaXPipeline(), inner_jit=False)
+        def loss_fn(weights):
+            return llama.loss(tok, tgt, cfg, weights)
+
+        def loss_step():
+            y, f_vjp = vjp(loss_fn, w)
+            return f_vjp(one)
+
+        tl = event_time(loss_step, iters, warmup=2)
+        out[name]["loss_ms_per_step"] = round(tl * 1e3, 3)
+        out[name]["loss_tokens_per_s"] = round(B * S / tl, 1)
         if B * S <= 1024:
             # small enough to be bound by launches and host code: the same step replayed from a HIP graph
             from enzyme_ad.jax.graph import capture
