@@ -47,6 +47,10 @@ template <int OP> __device__ __forceinline__ float apply_binary(float a, float b
     case EMI_OP_D_COS: return -a * sinf(b);                                // b = x
     case EMI_OP_D_POW_A: return b * powf(a, b - 1.0f);
     case EMI_OP_D_POW_B: return powf(a, b) * logf(a);
+    case EMI_OP_D_ABS: return b >= 0.0f ? a : -a;                           // b = x
+    case EMI_OP_D_LOG1P: return a / (b + 1.0f);                            // b = x
+    case EMI_OP_D_EXPM1: return a * expf(b);                               // b = x
+    case EMI_OP_D_CBRT: return a / (3.0f * b * b);                         // b = cbrt(x)
     default: return 0.0f;
   }
 }
@@ -64,6 +68,9 @@ template <int OP> __device__ __forceinline__ float apply_unary(float a) {
     case EMI_OP_COS: return cosf(a);
     case EMI_OP_ABS: return fabsf(a);
     case EMI_OP_COPY: return a;
+    case EMI_OP_LOG1P: return log1pf(a);
+    case EMI_OP_EXPM1: return expm1f(a);
+    case EMI_OP_CBRT: return cbrtf(a);
     default: return 0.0f;
   }
 }
@@ -627,6 +634,7 @@ int launch_binary_op(hipStream_t st, int op, unsigned grid, const T* a, const T*
     EMI_BIN(EMI_OP_MIN) EMI_BIN(EMI_OP_GE) EMI_BIN(EMI_OP_EQ) EMI_BIN(EMI_OP_NMUL) EMI_BIN(EMI_OP_POW)
     EMI_BIN(EMI_OP_D_SQRT) EMI_BIN(EMI_OP_D_RSQRT) EMI_BIN(EMI_OP_D_LOGISTIC) EMI_BIN(EMI_OP_D_TANH)
     EMI_BIN(EMI_OP_D_SIN) EMI_BIN(EMI_OP_D_COS) EMI_BIN(EMI_OP_D_POW_A) EMI_BIN(EMI_OP_D_POW_B)
+    EMI_BIN(EMI_OP_D_ABS) EMI_BIN(EMI_OP_D_LOG1P) EMI_BIN(EMI_OP_D_EXPM1) EMI_BIN(EMI_OP_D_CBRT)
     default: return emi_fail(EMI_INVALID_ARGUMENT, "emi_map_binary: unknown operator code %d", op);
   }
 #undef EMI_BIN
@@ -654,7 +662,7 @@ int launch_unary_op(hipStream_t st, int op, unsigned grid, const T* x, T* y, int
   switch (op) {
     EMI_UN(EMI_OP_NEG) EMI_UN(EMI_OP_EXP) EMI_UN(EMI_OP_LOG) EMI_UN(EMI_OP_SQRT) EMI_UN(EMI_OP_RSQRT)
     EMI_UN(EMI_OP_LOGISTIC) EMI_UN(EMI_OP_TANH) EMI_UN(EMI_OP_SIN) EMI_UN(EMI_OP_COS) EMI_UN(EMI_OP_ABS)
-    EMI_UN(EMI_OP_COPY)
+    EMI_UN(EMI_OP_COPY) EMI_UN(EMI_OP_LOG1P) EMI_UN(EMI_OP_EXPM1) EMI_UN(EMI_OP_CBRT)
     default: return emi_fail(EMI_INVALID_ARGUMENT, "emi_map_unary: unknown operator code %d", op);
   }
 #undef EMI_UN
@@ -692,7 +700,7 @@ using namespace emi;
 
 extern "C" int emi_map_binary(emi_stream_t stream, int op, const void* a, const void* b, void* y, int64_t n,
                               int a_is_scalar, int b_is_scalar, int dtype) {
-  EMI_REQUIRE(op >= EMI_OP_ADD && op <= EMI_OP_D_POW_B, "emi_map_binary: unknown operator code %d", op);
+  EMI_REQUIRE(op >= EMI_OP_ADD && op <= EMI_OP_D_CBRT, "emi_map_binary: unknown operator code %d", op);
   EMI_REQUIRE(n >= 0 && n < (int64_t)1 << 39, "emi_map_binary: size out of range");
   if (n == 0) return EMI_OK;
   EMI_REQUIRE(a && b && y, "emi_map_binary: null buffer");
@@ -706,7 +714,7 @@ extern "C" int emi_map_binary(emi_stream_t stream, int op, const void* a, const 
 }
 
 extern "C" int emi_map_unary(emi_stream_t stream, int op, const void* x, void* y, int64_t n, int dtype) {
-  EMI_REQUIRE(op >= EMI_OP_NEG && op <= EMI_OP_COPY, "emi_map_unary: unknown operator code %d", op);
+  EMI_REQUIRE(op >= EMI_OP_NEG && op <= EMI_OP_CBRT, "emi_map_unary: unknown operator code %d", op);
   EMI_REQUIRE(n >= 0 && n < (int64_t)1 << 39, "emi_map_unary: size out of range");
   if (n == 0) return EMI_OK;
   EMI_REQUIRE(x && y, "emi_map_unary: null buffer");

@@ -20,9 +20,9 @@ from .ops import Tape, _accumulate, _code, _p, _quiet, _set_tan, _stream, _tan
 
 BINARY = {"add": 0, "subtract": 1, "multiply": 2, "divide": 3, "maximum": 4, "minimum": 5, "ge": 6, "eq": 7,
           "nmul": 8, "power": 9, "d_sqrt": 10, "d_rsqrt": 11, "d_logistic": 12, "d_tanh": 13, "d_sin": 14,
-          "d_cos": 15, "d_pow_a": 16, "d_pow_b": 17}
+          "d_cos": 15, "d_pow_a": 16, "d_pow_b": 17, "d_abs": 18, "d_log1p": 19, "d_expm1": 20, "d_cbrt": 21}
 UNARY = {"negate": 32, "exponential": 33, "log": 34, "sqrt": 35, "rsqrt": 36, "logistic": 37, "tanh": 38,
-         "sine": 39, "cosine": 40, "abs": 41, "copy": 42}
+         "sine": 39, "cosine": 40, "abs": 41, "copy": 42, "log_plus_one": 43, "exponential_minus_one": 44, "cbrt": 45}
 REDUCE = {"add": 0, "maximum": 4}
 
 
@@ -376,6 +376,7 @@ def binary(name, a, b):
 _D_UNARY = {   # operator -> (derivative kernel, which saved value it reads)
     "exponential": ("multiply", "y"), "log": ("divide", "x"), "sqrt": ("d_sqrt", "y"), "rsqrt": ("d_rsqrt", "y"),
     "logistic": ("d_logistic", "y"), "tanh": ("d_tanh", "y"), "sine": ("d_sin", "x"), "cosine": ("d_cos", "x"),
+    "abs": ("d_abs", "x"), "log_plus_one": ("d_log1p", "x"), "exponential_minus_one": ("d_expm1", "x"), "cbrt": ("d_cbrt", "y"),
 }
 
 

@@ -11,7 +11,8 @@ function that calls `hlo_call` differentiate through the parsed graph.
 
 The accepted text is MLIR's printed form of the operators JAX emits for such functions
 (pretty or quoted-generic operator names): constant, add, subtract, multiply, divide, maximum,
-minimum, power, negate, exponential, log, sqrt, rsqrt, logistic, tanh, sine, cosine, convert, reshape,
+minimum, power, negate, exponential, log, sqrt, rsqrt, logistic, tanh, sine, cosine, abs, log_plus_one,
+exponential_minus_one, cbrt, convert, reshape,
 transpose, broadcast_in_dim, reduce (add / maximum), dot_general, slice, pad, concatenate, compare,
 select, call,
 custom_call (this library's targets), return.  Anything else raises `NotImplementedError` naming the operator.
@@ -65,7 +66,8 @@ NUMPY_DTYPES = {"f32": np.float32, "f64": np.float64, "f16": np.float16, "i32": 
                 "i1": np.bool_, "ui32": np.uint32, "i8": np.int8}
 
 BINARY_OPS = {"add", "subtract", "multiply", "divide", "maximum", "minimum", "power"}
-UNARY_OPS = {"negate", "exponential", "log", "sqrt", "rsqrt", "logistic", "tanh", "sine", "cosine"}
+UNARY_OPS = {"negate", "exponential", "log", "sqrt", "rsqrt", "logistic", "tanh", "sine", "cosine", "abs", "log_plus_one",
+             "exponential_minus_one", "cbrt"}
 
 
 # ---------------------------------------------------------------------------
@@ -606,7 +608,8 @@ def _splat(op):
 
 _FOLD_UNARY = {"negate": np.negative, "exponential": np.exp, "log": np.log, "sqrt": np.sqrt,
                "rsqrt": lambda v: 1.0 / np.sqrt(v), "tanh": np.tanh, "sine": np.sin, "cosine": np.cos,
-               "logistic": lambda v: 1.0 / (1.0 + np.exp(-v))}
+               "logistic": lambda v: 1.0 / (1.0 + np.exp(-v)), "abs": np.abs, "log_plus_one": np.log1p,
+               "exponential_minus_one": np.expm1, "cbrt": np.cbrt}
 _FOLD_BINARY = {"add": np.add, "subtract": np.subtract, "multiply": np.multiply, "divide": np.divide,
                 "maximum": np.maximum, "minimum": np.minimum, "power": np.power}
 

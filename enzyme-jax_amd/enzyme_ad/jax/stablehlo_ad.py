@@ -265,6 +265,16 @@ def reverse_function(func, name=None, arg_active=None, ret_active=None):
             accum(xs[0], b.binary("multiply", b.binary("multiply", c, r), b.binary("subtract", splat_like(r, 1.0), r)))
         elif n == "tanh":
             accum(xs[0], b.binary("multiply", c, b.binary("subtract", splat_like(r, 1.0), b.binary("multiply", r, r))))
+        elif n == "abs":
+            # select(x >= 0, c, -c)  (Abs rule :1244, abs.mlir:21-27)
+            accum(xs[0], b.emit("select", [b.compare("GE", xs[0], splat_like(r, 0.0)), c, b.unary("negate", c)], {}, T[r]))
+        elif n == "log_plus_one":
+            accum(xs[0], b.binary("divide", c, b.binary("add", xs[0], splat_like(r, 1.0))))          # Log1p rule :1201
+        elif n == "exponential_minus_one":
+            accum(xs[0], b.binary("multiply", c, b.unary("exponential", xs[0])))                     # Expm1 rule :1184
+        elif n == "cbrt":
+            # c / (3 cbrt(x)^2), finite for negative x (Cbrt rule :1085, cbrt.mlir:19-26)
+            accum(xs[0], b.binary("divide", c, b.binary("multiply", splat_like(r, 3.0), b.binary("multiply", r, r))))
         elif n == "sine":
             accum(xs[0], b.binary("multiply", c, b.unary("cosine", xs[0])))
         elif n == "cosine":
@@ -436,6 +446,14 @@ def forward_function(func, name=None, arg_active=None):
             tan[r] = b.binary("multiply", b.binary("multiply", t, r), b.binary("subtract", b.const(1.0, T[r]), r))
         elif n == "tanh":
             tan[r] = b.binary("multiply", t, b.binary("subtract", b.const(1.0, T[r]), b.binary("multiply", r, r)))
+        elif n == "abs":
+            tan[r] = b.emit("select", [b.compare("GE", xs[0], b.const(0.0, T[r])), t, b.unary("negate", t)], {}, T[r])
+        elif n == "log_plus_one":
+            tan[r] = b.binary("divide", t, b.binary("add", xs[0], b.const(1.0, T[r])))
+        elif n == "exponential_minus_one":
+            tan[r] = b.binary("multiply", t, b.unary("exponential", xs[0]))
+        elif n == "cbrt":
+            tan[r] = b.binary("divide", t, b.binary("multiply", b.const(3.0, T[r]), b.binary("multiply", r, r)))
         elif n == "sine":
             tan[r] = b.binary("multiply", t, b.unary("cosine", xs[0]))
         elif n == "cosine":

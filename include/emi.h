@@ -220,9 +220,14 @@ enum {
   /* factors of the Pow rule (HLODerivatives.td:1237-1242) on the operands themselves */
   EMI_OP_D_POW_A,    /* b pow(a, b - 1) */
   EMI_OP_D_POW_B,    /* pow(a, b) log(a) */
+  /* further derivative factors (HLODerivatives.td: Abs :1244, Log1p :1201, Expm1 :1184, Cbrt :1085) */
+  EMI_OP_D_ABS,      /* b = x:           b >= 0 ? a : -a */
+  EMI_OP_D_LOG1P,    /* b = x:           a / (b + 1) */
+  EMI_OP_D_EXPM1,    /* b = x:           a exp(b) */
+  EMI_OP_D_CBRT,     /* b = cbrt(x):     a / (3 b^2) */
   /* unary: y = op(x) */
   EMI_OP_NEG = 32, EMI_OP_EXP, EMI_OP_LOG, EMI_OP_SQRT, EMI_OP_RSQRT, EMI_OP_LOGISTIC, EMI_OP_TANH,
-  EMI_OP_SIN, EMI_OP_COS, EMI_OP_ABS, EMI_OP_COPY
+  EMI_OP_SIN, EMI_OP_COS, EMI_OP_ABS, EMI_OP_COPY, EMI_OP_LOG1P, EMI_OP_EXPM1, EMI_OP_CBRT
 };
 
 /* y[i] = op(a[i], b[i]) for i < n, computed in fp32.  An operand flagged

@@ -103,6 +103,45 @@ def vjp_power(x, y, d):
             _checked_mul(d, np.power(x, y) * np.log(x)))
 
 
+def vjp_minimum(x, y, d):
+    """HLODerivatives.td:1213-1219 MinOp: y < x sends the cotangent to y, ties go to the first operand."""
+    lt = y < x
+    z = np.zeros_like(d)
+    return np.where(lt, z, d), np.where(lt, d, z)
+
+
+def vjp_abs(x, d):
+    """HLODerivatives.td:1244 AbsOp, real operands: select(x >= 0, d, -d) (abs.mlir:21-27)."""
+    return (np.where(x >= 0, d, -d),)
+
+
+def vjp_log(x, d):
+    """HLODerivatives.td:1199 LogOp."""
+    return (_checked_div(d, x),)
+
+
+def vjp_log_plus_one(x, d):
+    """HLODerivatives.td:1201 Log1pOp."""
+    return (_checked_div(d, x + 1.0),)
+
+
+def vjp_exponential_minus_one(x, d):
+    """HLODerivatives.td:1184 Expm1Op."""
+    return (_checked_mul(d, np.exp(x)),)
+
+
+def vjp_cbrt(x, d):
+    """HLODerivatives.td:1085-1087 CbrtOp: d / (3 cbrt(x)^2), real for negative x too."""
+    c = np.cbrt(x)
+    return (_checked_div(d, 3.0 * (c * c)),)
+
+
+def vjp_tanh(x, d):
+    """HLODerivatives.td:1326-1330 TanhOp."""
+    t = np.tanh(x)
+    return (_checked_mul(d, 1.0 - t * t),)
+
+
 def vjp_cosine(x, d):
     """HLODerivatives.td:1129 CosineOp."""
     return (_checked_mul(d, -np.sin(x)),)

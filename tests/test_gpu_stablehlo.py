@@ -37,11 +37,14 @@ NP_BINARY = {"add": np.add, "subtract": np.subtract, "multiply": np.multiply, "d
              "d_rsqrt": lambda a, b: -0.5 * a * b ** 3, "d_logistic": lambda a, b: a * b * (1 - b),
              "d_tanh": lambda a, b: a * (1 - b * b), "d_sin": lambda a, b: a * np.cos(b),
              "d_cos": lambda a, b: -a * np.sin(b), "d_pow_a": lambda a, b: b * np.power(a, b - 1),
-             "d_pow_b": lambda a, b: np.power(a, b) * np.log(a)}
+             "d_pow_b": lambda a, b: np.power(a, b) * np.log(a), "d_abs": lambda a, b: np.where(b >= 0, a, -a),
+             "d_log1p": lambda a, b: a / (b + 1), "d_expm1": lambda a, b: a * np.exp(b),
+             "d_cbrt": lambda a, b: a / (3 * b * b)}
 NP_UNARY = {"negate": np.negative, "exponential": np.exp, "log": np.log, "sqrt": np.sqrt,
             "rsqrt": lambda x: 1 / np.sqrt(x), "logistic": lambda x: 1 / (1 + np.exp(-x)), "tanh": np.tanh,
-            "sine": np.sin, "cosine": np.cos, "abs": np.abs, "copy": lambda x: x}
-POSITIVE = {"log", "sqrt", "rsqrt", "power", "d_pow_a", "d_pow_b"}
+            "sine": np.sin, "cosine": np.cos, "abs": np.abs, "copy": lambda x: x, "log_plus_one": np.log1p,
+            "exponential_minus_one": np.expm1, "cbrt": np.cbrt}
+POSITIVE = {"log", "sqrt", "rsqrt", "power", "d_pow_a", "d_pow_b", "log_plus_one", "d_log1p", "d_cbrt"}
 
 
 @pytest.mark.parametrize("dt", ["f32", "bf16"])
@@ -219,7 +222,7 @@ def test_hlo_call_rejects_wrong_arguments():
     with pytest.raises(AssertionError):
         hlo_call(f32(1.0), source="func.func @f(%a: tensor<f32>) -> tensor<f32> {\n return %a : tensor<f32>\n}")
     with pytest.raises(NotImplementedError):
-        hlo_call(f32(1.0), source="func.func @main(%a: tensor<f32>) -> tensor<f32> {\n %b = stablehlo.cbrt %a : tensor<f32>\n"
+        hlo_call(f32(1.0), source="func.func @main(%a: tensor<f32>) -> tensor<f32> {\n %b = stablehlo.erf_inv %a : tensor<f32>\n"
                                   " return %b : tensor<f32>\n}")
 
 

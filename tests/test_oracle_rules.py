@@ -15,6 +15,8 @@ FWD = {
     "subtract": lambda a, b: a - b, "negate": lambda a: -a, "exponential": np.exp,
     "sqrt": np.sqrt, "rsqrt": lambda a: 1 / np.sqrt(a), "logistic": R.logistic,
     "maximum": np.maximum, "power": np.power, "cosine": np.cos, "sine": np.sin,
+    "minimum": np.minimum, "abs": np.abs, "log": np.log, "log_plus_one": np.log1p, "exponential_minus_one": np.expm1,
+    "cbrt": np.cbrt, "tanh": np.tanh,
 }
 
 

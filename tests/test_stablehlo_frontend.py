@@ -59,8 +59,8 @@ def test_parser_errors_name_the_line_and_the_operator():
 
     with pytest.raises(S.ParseError, match="line 2"):
         S.parse_module("func.func @main(%a: tensor<2xf32>) -> tensor<2xf32> {\n  %b = stablehlo.add %a %a : tensor<2xf32>\n}")
-    with pytest.raises(NotImplementedError, match="stablehlo.cbrt"):
-        S.parse_module("func.func @main(%a: tensor<f32>) -> tensor<f32> {\n %b = stablehlo.cbrt %a : tensor<f32>\n return %b : tensor<f32>\n}")
+    with pytest.raises(NotImplementedError, match="stablehlo.erf_inv"):
+        S.parse_module("func.func @main(%a: tensor<f32>) -> tensor<f32> {\n %b = stablehlo.erf_inv %a : tensor<f32>\n return %b : tensor<f32>\n}")
     with pytest.raises(S.ParseError):
         S.parse_module("func.func @main(%a: tensor<?xf32>) -> tensor<2xf32> {\n return %a : tensor<2xf32>\n}")
     with pytest.raises(S.ParseError):
