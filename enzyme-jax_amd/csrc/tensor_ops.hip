@@ -51,6 +51,7 @@ template <int OP> __device__ __forceinline__ float apply_binary(float a, float b
     case EMI_OP_D_LOG1P: return a / (b + 1.0f);                            // b = x
     case EMI_OP_D_EXPM1: return a * expf(b);                               // b = x
     case EMI_OP_D_CBRT: return a / (3.0f * b * b);                         // b = cbrt(x)
+    case EMI_OP_ATAN2: return atan2f(a, b);
     default: return 0.0f;
   }
 }
@@ -634,7 +635,7 @@ int launch_binary_op(hipStream_t st, int op, unsigned grid, const T* a, const T*
     EMI_BIN(EMI_OP_MIN) EMI_BIN(EMI_OP_GE) EMI_BIN(EMI_OP_EQ) EMI_BIN(EMI_OP_NMUL) EMI_BIN(EMI_OP_POW)
     EMI_BIN(EMI_OP_D_SQRT) EMI_BIN(EMI_OP_D_RSQRT) EMI_BIN(EMI_OP_D_LOGISTIC) EMI_BIN(EMI_OP_D_TANH)
     EMI_BIN(EMI_OP_D_SIN) EMI_BIN(EMI_OP_D_COS) EMI_BIN(EMI_OP_D_POW_A) EMI_BIN(EMI_OP_D_POW_B)
-    EMI_BIN(EMI_OP_D_ABS) EMI_BIN(EMI_OP_D_LOG1P) EMI_BIN(EMI_OP_D_EXPM1) EMI_BIN(EMI_OP_D_CBRT)
+    EMI_BIN(EMI_OP_D_ABS) EMI_BIN(EMI_OP_D_LOG1P) EMI_BIN(EMI_OP_D_EXPM1) EMI_BIN(EMI_OP_D_CBRT) EMI_BIN(EMI_OP_ATAN2)
     default: return emi_fail(EMI_INVALID_ARGUMENT, "emi_map_binary: unknown operator code %d", op);
   }
 #undef EMI_BIN
@@ -700,7 +701,7 @@ using namespace emi;
 
 extern "C" int emi_map_binary(emi_stream_t stream, int op, const void* a, const void* b, void* y, int64_t n,
                               int a_is_scalar, int b_is_scalar, int dtype) {
-  EMI_REQUIRE(op >= EMI_OP_ADD && op <= EMI_OP_D_CBRT, "emi_map_binary: unknown operator code %d", op);
+  EMI_REQUIRE(op >= EMI_OP_ADD && op <= EMI_OP_ATAN2, "emi_map_binary: unknown operator code %d", op);
   EMI_REQUIRE(n >= 0 && n < (int64_t)1 << 39, "emi_map_binary: size out of range");
   if (n == 0) return EMI_OK;
   EMI_REQUIRE(a && b && y, "emi_map_binary: null buffer");

@@ -20,7 +20,7 @@ from .ops import Tape, _accumulate, _code, _p, _quiet, _set_tan, _stream, _tan
 
 BINARY = {"add": 0, "subtract": 1, "multiply": 2, "divide": 3, "maximum": 4, "minimum": 5, "ge": 6, "eq": 7,
           "nmul": 8, "power": 9, "d_sqrt": 10, "d_rsqrt": 11, "d_logistic": 12, "d_tanh": 13, "d_sin": 14,
-          "d_cos": 15, "d_pow_a": 16, "d_pow_b": 17, "d_abs": 18, "d_log1p": 19, "d_expm1": 20, "d_cbrt": 21}
+          "d_cos": 15, "d_pow_a": 16, "d_pow_b": 17, "d_abs": 18, "d_log1p": 19, "d_expm1": 20, "d_cbrt": 21, "atan2": 22}
 UNARY = {"negate": 32, "exponential": 33, "log": 34, "sqrt": 35, "rsqrt": 36, "logistic": 37, "tanh": 38,
          "sine": 39, "cosine": 40, "abs": 41, "copy": 42, "log_plus_one": 43, "exponential_minus_one": 44, "cbrt": 45}
 REDUCE = {"add": 0, "maximum": 4}
@@ -358,6 +358,21 @@ def binary(name, a, b):
         def tangent(ta, tb):
             pa = None if ta is None else _bin("multiply", ta, _bin("d_pow_a", a, b))
             pb = None if tb is None else _bin("multiply", tb, _bin("d_pow_b", a, b))
+            return pb if pa is None else pa if pb is None else _bin("add", pa, pb)
+    elif name == "atan2":
+        # y = atan2(a, b): da = c b / (a^2 + b^2), db = -c a / (a^2 + b^2)  (Atan2 rule, HLODerivatives.td:972-978)
+        def factors():
+            den = _bin("add", _bin("multiply", a, a), _bin("multiply", b, b))
+            return _bin("divide", b, den), _un("negate", _bin("divide", a, den))
+
+        def rule(c, acc):
+            fa, fb = factors()
+            return (_accumulate(acc[0], _fit(_bin("multiply", c, fa), a)), _accumulate(acc[1], _fit(_bin("multiply", c, fb), b)))
+
+        def tangent(ta, tb):
+            fa, fb = factors()
+            pa = None if ta is None else _bin("multiply", ta, fa)
+            pb = None if tb is None else _bin("multiply", tb, fb)
             return pb if pa is None else pa if pb is None else _bin("add", pa, pb)
     else:
         raise NotImplementedError("no differentiation rule for stablehlo.%s" % name)

@@ -11,7 +11,7 @@ function that calls `hlo_call` differentiate through the parsed graph.
 
 The accepted text is MLIR's printed form of the operators JAX emits for such functions
 (pretty or quoted-generic operator names): constant, add, subtract, multiply, divide, maximum,
-minimum, power, negate, exponential, log, sqrt, rsqrt, logistic, tanh, sine, cosine, abs, log_plus_one,
+minimum, power, atan2, clamp (as maximum + minimum), negate, exponential, log, sqrt, rsqrt, logistic, tanh, sine, cosine, abs, log_plus_one,
 exponential_minus_one, cbrt, convert, reshape,
 transpose, broadcast_in_dim, reduce (add / maximum), dot_general, slice, pad, concatenate, compare,
 select, call,
@@ -65,7 +65,7 @@ TORCH_DTYPES = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float
 NUMPY_DTYPES = {"f32": np.float32, "f64": np.float64, "f16": np.float16, "i32": np.int32, "i64": np.int64,
                 "i1": np.bool_, "ui32": np.uint32, "i8": np.int8}
 
-BINARY_OPS = {"add", "subtract", "multiply", "divide", "maximum", "minimum", "power"}
+BINARY_OPS = {"add", "subtract", "multiply", "divide", "maximum", "minimum", "power", "atan2"}
 UNARY_OPS = {"negate", "exponential", "log", "sqrt", "rsqrt", "logistic", "tanh", "sine", "cosine", "abs", "log_plus_one",
              "exponential_minus_one", "cbrt"}
 
@@ -436,6 +436,26 @@ def _parse_op(sc):
         operands = operand_list()
         _, types = sc.signature()
         return Op("select", results, operands, {}, types[-1:])
+    if short == "clamp":
+        # clamp(min, x, max) = minimum(maximum(x, min), max): two operators, so that every rule and rewrite of
+        # those applies (an operand at a bound keeps its cotangent, outside it gets none: clamp.mlir:14-26)
+        operands = operand_list()
+        in_types, types = sc.signature()
+        in_types = in_types or []
+        if len(operands) != 3:
+            sc.fail("clamp takes (min, operand, max)")
+        out, seq = types[-1], []
+        bounds = []
+        for tag, v, ty in (("lo", operands[0], in_types[0] if len(in_types) == 3 else out),
+                           ("hi", operands[2], in_types[2] if len(in_types) == 3 else out)):
+            if ty.shape == () and out.shape != ():          # rank-0 bounds are allowed: broadcast them
+                wide = "%s__clamp_%s" % (results[0], tag)
+                seq.append(Op("broadcast_in_dim", [wide], [v], {"dims": []}, [out]))
+                v = wide
+            bounds.append(v)
+        inner = results[0] + "__clamp_max"
+        return seq + [Op("maximum", [inner], [operands[1], bounds[0]], {}, [out]),
+                      Op("minimum", results, [inner, bounds[1]], {}, [out])]
     if short == "call":
         callee = sc.need(_SYM, "callee")
         sc.expect("(")
@@ -520,7 +540,8 @@ def _parse_func(sc):
     sc.expect("{")
     body = []
     while not sc.accept("}"):
-        body.append(_parse_op(sc))
+        op = _parse_op(sc)
+        body.extend(op if isinstance(op, list) else [op])
     return Func(name, args, result_types, body)
 
 
@@ -611,7 +632,7 @@ _FOLD_UNARY = {"negate": np.negative, "exponential": np.exp, "log": np.log, "sqr
                "logistic": lambda v: 1.0 / (1.0 + np.exp(-v)), "abs": np.abs, "log_plus_one": np.log1p,
                "exponential_minus_one": np.expm1, "cbrt": np.cbrt}
 _FOLD_BINARY = {"add": np.add, "subtract": np.subtract, "multiply": np.multiply, "divide": np.divide,
-                "maximum": np.maximum, "minimum": np.minimum, "power": np.power}
+                "maximum": np.maximum, "minimum": np.minimum, "power": np.power, "atan2": np.arctan2}
 
 
 _FOLD_COMPARE = {"EQ": np.equal, "NE": np.not_equal, "GE": np.greater_equal, "GT": np.greater, "LE": np.less_equal,

@@ -252,6 +252,11 @@ def reverse_function(func, name=None, arg_active=None, ret_active=None):
             ym1 = b.binary("subtract", xs[1], splat_like(r, 1.0))
             accum(xs[0], b.binary("multiply", c, b.binary("multiply", xs[1], b.binary("power", xs[0], ym1))))
             accum(xs[1], b.binary("multiply", c, b.binary("multiply", r, b.unary("log", xs[0]))))
+        elif n == "atan2":
+            # c x / (x^2 + y^2) and -c y / (x^2 + y^2) for atan2(y, x)  (Atan2 rule :972-978)
+            den = b.binary("add", b.binary("multiply", xs[1], xs[1]), b.binary("multiply", xs[0], xs[0]))
+            accum(xs[0], b.binary("multiply", c, b.binary("divide", xs[1], den)))
+            accum(xs[1], b.binary("multiply", c, b.binary("divide", b.unary("negate", xs[0]), den)))
         elif n == "compare":
             continue
         elif n == "select":
@@ -435,6 +440,14 @@ def forward_function(func, name=None, arg_active=None):
             ym1 = b.binary("subtract", xs[1], b.const(1.0, T[r]))
             tan[r] = add(None if ts[0] is None else b.binary("multiply", ts[0], b.binary("multiply", xs[1], b.binary("power", xs[0], ym1))),
                          None if ts[1] is None else b.binary("multiply", ts[1], b.binary("multiply", r, b.unary("log", xs[0]))))
+        elif n == "atan2":
+            # (x ty - y tx) / (x^2 + y^2), the reference's forward form
+            den = b.binary("add", b.binary("multiply", xs[1], xs[1]), b.binary("multiply", xs[0], xs[0]))
+            num = None if ts[0] is None else b.binary("multiply", xs[1], ts[0])
+            if ts[1] is not None:
+                sub = b.binary("multiply", xs[0], ts[1])
+                num = b.unary("negate", sub) if num is None else b.binary("subtract", num, sub)
+            tan[r] = b.binary("divide", num, den)
         elif n == "compare":
             continue
         elif n == "select":

@@ -225,6 +225,7 @@ enum {
   EMI_OP_D_LOG1P,    /* b = x:           a / (b + 1) */
   EMI_OP_D_EXPM1,    /* b = x:           a exp(b) */
   EMI_OP_D_CBRT,     /* b = cbrt(x):     a / (3 b^2) */
+  EMI_OP_ATAN2,      /* atan2(a, b): the angle of the point (b, a) */
   /* unary: y = op(x) */
   EMI_OP_NEG = 32, EMI_OP_EXP, EMI_OP_LOG, EMI_OP_SQRT, EMI_OP_RSQRT, EMI_OP_LOGISTIC, EMI_OP_TANH,
   EMI_OP_SIN, EMI_OP_COS, EMI_OP_ABS, EMI_OP_COPY, EMI_OP_LOG1P, EMI_OP_EXPM1, EMI_OP_CBRT

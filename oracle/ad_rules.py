@@ -142,6 +142,17 @@ def vjp_tanh(x, d):
     return (_checked_mul(d, 1.0 - t * t),)
 
 
+def vjp_atan2(y, x, d):
+    """HLODerivatives.td:972-978 Atan2Op (operands in the order y, x)."""
+    den = x * x + y * y
+    return _checked_mul(d, x / den), _checked_mul(d, -y / den)
+
+
+def vjp_clamp_operand(lo, x, hi, d):
+    """HLODerivatives.td:1050-1066 ClampOp, cotangent of the clamped operand: none outside [lo, hi]."""
+    return (np.where((x < lo) | (x > hi), 0.0, d),)
+
+
 def vjp_cosine(x, d):
     """HLODerivatives.td:1129 CosineOp."""
     return (_checked_mul(d, -np.sin(x)),)

@@ -39,7 +39,7 @@ NP_BINARY = {"add": np.add, "subtract": np.subtract, "multiply": np.multiply, "d
              "d_cos": lambda a, b: -a * np.sin(b), "d_pow_a": lambda a, b: b * np.power(a, b - 1),
              "d_pow_b": lambda a, b: np.power(a, b) * np.log(a), "d_abs": lambda a, b: np.where(b >= 0, a, -a),
              "d_log1p": lambda a, b: a / (b + 1), "d_expm1": lambda a, b: a * np.exp(b),
-             "d_cbrt": lambda a, b: a / (3 * b * b)}
+             "d_cbrt": lambda a, b: a / (3 * b * b), "atan2": np.arctan2}
 NP_UNARY = {"negate": np.negative, "exponential": np.exp, "log": np.log, "sqrt": np.sqrt,
             "rsqrt": lambda x: 1 / np.sqrt(x), "logistic": lambda x: 1 / (1 + np.exp(-x)), "tanh": np.tanh,
             "sine": np.sin, "cosine": np.cos, "abs": np.abs, "copy": lambda x: x, "log_plus_one": np.log1p,
@@ -264,6 +264,29 @@ def test_rule_matches_reference_vector_through_text(name):
         tans = [f32(np.ones(n)) if j == i else None for j in range(len(args))]
         _, t = jvp(fn, tuple(args), tuple(tans))
         np.testing.assert_allclose(host(t), want, rtol=3e-6, atol=1e-7)
+
+
+def test_clamp_rule_through_text():
+    """clamp.mlir:14-34: scalar bounds, the operand's cotangent vanishes outside them (reverse and forward mode)."""
+    from enzyme_ad.jax import hlo_call, jvp, vjp, stablehlo_ad
+
+    g = GOLDEN["clamp_operand"]
+    text = ("func.func @main(%x: tensor<10xf32>) -> tensor<10xf32> {\n"
+            "  %lo = stablehlo.constant dense<1.000000e+00> : tensor<f32>\n"
+            "  %hi = stablehlo.constant dense<2.000000e+00> : tensor<f32>\n"
+            "  %r = stablehlo.clamp %lo, %x, %hi : (tensor<f32>, tensor<10xf32>, tensor<f32>) -> tensor<10xf32>\n"
+            "  return %r : tensor<10xf32>\n}\n")
+    x, one = f32(g["operand"]), f32(np.ones(10))
+    fn = lambda a: hlo_call(a, source=text)[0]
+    out, f_vjp = vjp(fn, x)
+    assert np.array_equal(host(out), np.asarray(g["out"]))
+    assert np.array_equal(host(f_vjp(one)[0]), np.asarray(g["grad_operand"]))
+    _, t = jvp(fn, (x,), (one,))
+    assert np.array_equal(host(t), np.asarray(g["grad_operand"]))
+    (sym,) = hlo_call(x, one, source=stablehlo_ad.reverse_module_text(text))
+    assert np.array_equal(host(sym), np.asarray(g["grad_operand"]))
+    out2, tan2 = hlo_call(x, one, source=stablehlo_ad.forward_module_text(text))
+    assert np.array_equal(host(out2), np.asarray(g["out"])) and np.array_equal(host(tan2), np.asarray(g["grad_operand"]))
 
 
 def test_transpose_and_dot_general_rules_through_text():

@@ -16,7 +16,7 @@ FWD = {
     "sqrt": np.sqrt, "rsqrt": lambda a: 1 / np.sqrt(a), "logistic": R.logistic,
     "maximum": np.maximum, "power": np.power, "cosine": np.cos, "sine": np.sin,
     "minimum": np.minimum, "abs": np.abs, "log": np.log, "log_plus_one": np.log1p, "exponential_minus_one": np.expm1,
-    "cbrt": np.cbrt, "tanh": np.tanh,
+    "cbrt": np.cbrt, "tanh": np.tanh, "atan2": np.arctan2,
 }
 
 
@@ -85,3 +85,11 @@ def test_reduce_and_broadcast_rules_are_adjoint():
     assert parts[0].shape == (2, 4) and parts[1][0, 0] == 8.0
     (gs,) = R.vjp_slice(np.zeros((4,)), (1,), (3,), np.array([5.0, 6.0]))
     np.testing.assert_array_equal(gs, [0, 5, 6, 0])
+
+
+def test_clamp_rule_matches_reference_vector():
+    g = GOLD["clamp_operand"]
+    x = np.array(g["operand"])
+    np.testing.assert_array_equal(np.clip(x, g["min"], g["max"]), g["out"])
+    (dx,) = R.vjp_clamp_operand(g["min"], x, g["max"], np.ones_like(x))
+    np.testing.assert_array_equal(dx, g["grad_operand"])
