@@ -50,31 +50,64 @@ __global__ __launch_bounds__(256) void xent_fwd_kernel(const T* __restrict__ log
   const int64_t nchunk = (vocab + N - 1) / N;
   float m = -INFINITY, s = 0.f;
   for (int64_t c0 = threadIdx.x; c0 < nchunk; c0 += 256 * UN) {
-    float v[UN][N];
+    if constexpr (VEC) {
+      // chunks stay in storage format (16 bytes each) and are unpacked for the maximum and again for the sum
+      typename Chunk<T>::Raw raw[UN];
 #pragma unroll
-    for (int u = 0; u < UN; u++) {
-      const int64_t c = c0 + 256 * u;
-      if (c < nchunk) {
-        load_row_chunk<T, VEC>(z, c, vocab, -INFINITY, v[u]);
-      } else {
-#pragma unroll
-        for (int e = 0; e < N; e++) v[u][e] = -INFINITY;
+      for (int u = 0; u < UN; u++) {
+        const int64_t c = c0 + 256 * u;
+        raw[u] = Chunk<T>::load_raw(z + (c < nchunk ? c : c0) * N);      // past the end: this thread's first chunk again
       }
-    }
-    float top = -INFINITY;
+      float top = -INFINITY;
 #pragma unroll
-    for (int u = 0; u < UN; u++)
+      for (int u = 0; u < UN; u++) {
+        float v[N];
+        Chunk<T>::unpack(raw[u], v);
 #pragma unroll
-      for (int e = 0; e < N; e++) top = fmaxf(top, v[u][e]);
-    const float mx = fmaxf(m, top * kLog2e);
-    if (mx > -INFINITY) {                       // at least one finite logit so far
-      float t = 0.f;
+        for (int e = 0; e < N; e++) top = fmaxf(top, v[e]);
+      }
+      const float mx = fmaxf(m, top * kLog2e);
+      if (mx > -INFINITY) {                       // at least one finite logit so far
+        float t = 0.f;
+#pragma unroll
+        for (int u = 0; u < UN; u++) {
+          if (c0 + 256 * u < nchunk) {
+            float v[N];
+            Chunk<T>::unpack(raw[u], v);
+#pragma unroll
+            for (int e = 0; e < N; e++) t += __builtin_amdgcn_exp2f(fmaf(v[e], kLog2e, -mx));
+          }
+        }
+        s = s * __builtin_amdgcn_exp2f(m - mx) + t;
+        m = mx;
+      }
+    } else {
+      float v[UN][N];
+#pragma unroll
+      for (int u = 0; u < UN; u++) {
+        const int64_t c = c0 + 256 * u;
+        if (c < nchunk) {
+          load_row_chunk<T, VEC>(z, c, vocab, -INFINITY, v[u]);
+        } else {
+#pragma unroll
+          for (int e = 0; e < N; e++) v[u][e] = -INFINITY;
+        }
+      }
+      float top = -INFINITY;
 #pragma unroll
       for (int u = 0; u < UN; u++)
 #pragma unroll
-        for (int e = 0; e < N; e++) t += __builtin_amdgcn_exp2f(fmaf(v[u][e], kLog2e, -mx));
-      s = s * __builtin_amdgcn_exp2f(m - mx) + t;
-      m = mx;
+        for (int e = 0; e < N; e++) top = fmaxf(top, v[u][e]);
+      const float mx = fmaxf(m, top * kLog2e);
+      if (mx > -INFINITY) {                       // at least one finite logit so far
+        float t = 0.f;
+#pragma unroll
+        for (int u = 0; u < UN; u++)
+#pragma unroll
+          for (int e = 0; e < N; e++) t += __builtin_amdgcn_exp2f(fmaf(v[u][e], kLog2e, -mx));
+        s = s * __builtin_amdgcn_exp2f(m - mx) + t;
+        m = mx;
+      }
     }
   }
   // block reduction of (m, s)
@@ -190,7 +223,7 @@ static int xent_fwd_launch(hipStream_t st, const void* logits, const int32_t* ta
                            int64_t tokens, int64_t vocab) {
   const T* z = static_cast<const T*>(logits);
   if (row_chunks<T>(vocab, logits, nullptr))
-    hipLaunchKernelGGL((xent_fwd_kernel<T, true, 8>), dim3((unsigned)tokens), dim3(256), 0, st, z, targets, loss, lse, vocab);
+    hipLaunchKernelGGL((xent_fwd_kernel<T, true, 16>), dim3((unsigned)tokens), dim3(256), 0, st, z, targets, loss, lse, vocab);
   else
     hipLaunchKernelGGL((xent_fwd_kernel<T, false, 2>), dim3((unsigned)tokens), dim3(256), 0, st, z, targets, loss, lse, vocab);
   EMI_CHECK_LAUNCH("emi_cross_entropy_fwd");
