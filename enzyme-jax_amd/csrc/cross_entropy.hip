@@ -187,22 +187,44 @@ __global__ __launch_bounds__(256) void xent_jvp_kernel(const T* __restrict__ log
   const float l2 = lse[row] * kLog2e;
   float acc = 0.f;
   for (int64_t c0 = threadIdx.x; c0 < nchunk; c0 += 256 * UN) {
-    float v[UN][N], w[UN][N];
+    if constexpr (VEC) {
+      typename Chunk<T>::Raw rz[UN], rt[UN];                 // storage format until used
 #pragma unroll
-    for (int u = 0; u < UN; u++) {
-      const int64_t c = c0 + 256 * u;
-      if (c < nchunk) {
-        load_row_chunk<T, VEC>(z, c, vocab, -INFINITY, v[u]);
-        load_row_chunk<T, VEC>(tz, c, vocab, 0.f, w[u]);
-      } else {
-#pragma unroll
-        for (int e = 0; e < N; e++) v[u][e] = -INFINITY, w[u][e] = 0.f;
+      for (int u = 0; u < UN; u++) {
+        const int64_t c = c0 + 256 * u;
+        if (c < nchunk) {
+          rz[u] = Chunk<T>::load_raw(z + c * N);
+          rt[u] = Chunk<T>::load_raw(tz + c * N);
+        }
       }
+#pragma unroll
+      for (int u = 0; u < UN; u++) {
+        if (c0 + 256 * u < nchunk) {
+          float v[N], w[N];
+          Chunk<T>::unpack(rz[u], v);
+          Chunk<T>::unpack(rt[u], w);
+#pragma unroll
+          for (int e = 0; e < N; e++) acc += __builtin_amdgcn_exp2f(fmaf(v[e], kLog2e, -l2)) * w[e];
+        }
+      }
+    } else {
+      float v[UN][N], w[UN][N];
+#pragma unroll
+      for (int u = 0; u < UN; u++) {
+        const int64_t c = c0 + 256 * u;
+        if (c < nchunk) {
+          load_row_chunk<T, VEC>(z, c, vocab, -INFINITY, v[u]);
+          load_row_chunk<T, VEC>(tz, c, vocab, 0.f, w[u]);
+        } else {
+#pragma unroll
+          for (int e = 0; e < N; e++) v[u][e] = -INFINITY, w[u][e] = 0.f;
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < UN; u++)
+#pragma unroll
+        for (int e = 0; e < N; e++) acc += __builtin_amdgcn_exp2f(fmaf(v[u][e], kLog2e, -l2)) * w[u][e];
     }
-#pragma unroll
-    for (int u = 0; u < UN; u++)
-#pragma unroll
-      for (int e = 0; e < N; e++) acc += __builtin_amdgcn_exp2f(fmaf(v[u][e], kLog2e, -l2)) * w[u][e];
   }
   const float tot = block_sum(acc, red);
   if (threadIdx.x == 0) {
@@ -257,7 +279,7 @@ static int xent_jvp_launch(hipStream_t st, const void* logits, const int32_t* ta
   const T* z = static_cast<const T*>(logits);
   const T* tz = static_cast<const T*>(tlogits);
   if (row_chunks<T>(vocab, logits, tlogits))
-    hipLaunchKernelGGL((xent_jvp_kernel<T, true, 4>), dim3((unsigned)tokens), dim3(256), 0, st, z, targets, lse, tz, tloss, vocab);
+    hipLaunchKernelGGL((xent_jvp_kernel<T, true, 8>), dim3((unsigned)tokens), dim3(256), 0, st, z, targets, lse, tz, tloss, vocab);
   else
     hipLaunchKernelGGL((xent_jvp_kernel<T, false, 2>), dim3((unsigned)tokens), dim3(256), 0, st, z, targets, lse, tz, tloss, vocab);
   EMI_CHECK_LAUNCH("emi_cross_entropy_jvp");
