@@ -118,6 +118,13 @@ def test_model_mean_loss_and_gradients(dt):
     ref_grads = L.model_bwd(dlogits, wr, cfg, cache)[1]
     for k, g in zip(names, grads):
         check(g, ref_grads[k], dt, "d loss / d " + k, factor=1.0 if dt == "f32" else 2.0)
+    # forward mode through the same graph: d loss along a random direction = <gradient, direction>
+    from enzyme_ad.jax import jvp
+    tw = [dev(rng.standard_normal(w[k].shape) * 0.02, dt)[0] for k in names]
+    _, tl = jvp(mean_loss, tuple(dw[k] for k in names), tuple(tw))
+    parts = [float((g.double() * t.double()).sum()) for g, t in zip(grads, tw)]
+    want, scale = sum(parts), sum(abs(p_) for p_ in parts)          # the parts cancel: bound the error by their size
+    assert abs(float(tl) - want) <= (1e-3 if dt == "f32" else 5e-2) * scale, (float(tl), want, scale)
 
 
 def _call(name, xla, args, rets):
