@@ -21,7 +21,9 @@ Three layers of restatement, each checked against the one before it:
 
 Parity status: every function here is pinned by at least one of: the step-form
 replay, the rule-chained adjoint, finite differences, torch.autograd, or a
-closed-form special case (tests/test_oracle_*.py).  What cannot be pinned
+closed-form special case (tests/test_oracle_*.py).  The cross-entropy functions
+(section 4b) have no call site in the reference; they are pinned by closed forms,
+scipy's logsumexp, torch's float64 cross_entropy and finite differences.  What cannot be pinned
 without running the reference: the bit pattern of XLA-CPU's compiled result
 (summation order, 1/sqrt -> rsqrt rewrite); the reference's own test tolerates
 atol = rtol = 1e-3 there (test/llama.py:318-319) - "parity unpinned" below
