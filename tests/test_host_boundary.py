@@ -262,3 +262,19 @@ def test_vjp_and_jvp_record_the_reference_pipeline():
     g = ej.enzyme_jax_ir(pipeline_options=ej.XLAPipeline(), inner_jit=False)(lambda a: a)     # no MLIR AD: nothing recorded
     ej.jvp(g, (3,), (None,))
     assert not hasattr(g, "last_pipeline")
+
+
+def test_bench_refuses_more_than_one_gpu_and_entry_points_exist():
+    """bench.py is a one-GPU program: asked for more it exits with a message instead of launching anything;
+    the repository entry module exposes build() and smoke()."""
+    import importlib.util
+    import subprocess
+    import sys as _sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([_sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0 and "ONE GPU" in (r.stderr + r.stdout)
+    spec = importlib.util.spec_from_file_location("graft_entry", os.path.join(root, "__graft_entry__.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    assert callable(mod.build) and callable(mod.smoke)
