@@ -509,15 +509,26 @@ def main():
     # the other two programs the reference's harness times next to reverse mode (test/test_utils.py:626-735):
     # the primal alone, and forward mode with a tangent on the input and on every weight
     from enzyme_ad.jax import jvp
-    modes = None
-    if not args.no_kernels:
+
+    def optional(what, fn):
+        """The sections after the headline measurement must not cost the JSON line: a failure is reported in it."""
+        try:
+            return fn()
+        except Exception as e:                                   # noqa: BLE001
+            log("bench.py: section '%s' failed: %s: %s" % (what, type(e).__name__, e))
+            return {"error": "%s: %s" % (type(e).__name__, str(e)[:300])}
+
+    def programs():
         tx = torch.randn_like(x)
         tlw = {k: torch.randn_like(v) * 0.02 for k, v in lw.items()}
         t_primal = event_time(lambda: layer_fn(x, lw), 5)
         t_forward = event_time(lambda: jvp(layer_fn, (x, lw), (tx, tlw)), 5)
-        modes = {"Primal_ms": round(t_primal * 1e3, 3), "Forward_ms": round(t_forward * 1e3, 3), "BothRev_ms": round(dt * 1e3, 3)}
+        return {"Primal_ms": round(t_primal * 1e3, 3), "Forward_ms": round(t_forward * 1e3, 3), "BothRev_ms": round(dt * 1e3, 3)}
+
+    modes = None
+    if not args.no_kernels:
+        modes = optional("programs", programs)
         log("layer programs:", modes)
-        del tx, tlw
 
     t_gemm, gemm_fl, n_gemm, per_layout = bench_gemms(cfg, max(5, min(args.steps, 20)))
     roofline = dict(bound="mfma", kernel="gemm_bf16_pingpong_kernel (256x256x64 tiles; %d launches per step: Y, dX in the NT form, dW in the TN form, 7 weights)" % n_gemm,
@@ -529,29 +540,30 @@ def main():
                                 for k, v in per_layout.items()})
     log("GEMM: %.1f TFLOP/s (%.1f%% of bf16 MFMA peak); per role %s" % (roofline["achieved"], 100 * roofline["frac"], roofline["per_role"]))
 
-    kernels = None
-    if not args.no_kernels:
-        kernels = bench_kernels(cfg, 5)
-        for k, v in kernels.items():
+    def kernel_table():
+        table = bench_kernels(cfg, 5)
+        for k, v in table.items():
             log("%-20s %8.1f %s  %5.1f%% of peak  (%.0f us)" % (k, v["achieved"], v["unit"], 100 * v["frac"], v["us"]))
-        kernels = {k: dict(bound=v["bound"], achieved=round(v["achieved"], 1), unit=v["unit"], frac=round(v["frac"], 4))
-                   for k, v in kernels.items()}
+        return {k: dict(bound=v["bound"], achieved=round(v["achieved"], 1), unit=v["unit"], frac=round(v["frac"], 4))
+                for k, v in table.items()}
+
+    kernels = optional("kernels", kernel_table) if not args.no_kernels else None
 
     frontend = None
     if not args.no_kernels and not args.no_frontend:
-        frontend = bench_frontend(5)
+        frontend = optional("stablehlo_frontend", lambda: bench_frontend(5))
         for k, v in frontend.items():
-            log("%-28s %s" % (k, {a: b for a, b in v.items() if a != "clusters"}))
+            log("%-28s %s" % (k, {a: b for a, b in v.items() if a != "clusters"} if isinstance(v, dict) else v))
 
     models = None
     if not args.no_kernels and not args.no_frontend:
-        models = bench_models(5)
+        models = optional("whole_models", lambda: bench_models(5))
         for k, v in models.items():
             log("%-24s %s" % (k, v))
 
     cpu = None
     if not args.no_cpu_baseline:
-        cpu = cpu_baseline(cfg)
+        cpu = optional("cpu_baseline", lambda: cpu_baseline(cfg))
         log("cpu baseline:", cpu)
 
     print(json.dumps({
