@@ -606,18 +606,6 @@ __device__ __forceinline__ int perm_key(int m) { return (m & ~12) | ((m & 4) << 
 // than 8 (in log2 units), so the rescaling of O runs on a few early tiles only; P then
 // stays below 2^8 and the final O/l and log-sum-exp are exact for whatever m was used.
 // ---------------------------------------------------------------------------
-#ifdef EMI_ATTN_BLOCKLOG
-__device__ unsigned long long emi_attn_blocklog[4096 * 4];
-extern "C" int emi_debug_attn_blocklog(unsigned long long* out) {
-  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(emi_attn_blocklog), sizeof(unsigned long long) * 4096 * 4);
-}
-#endif
-#ifdef EMI_ATTN_TRACE
-__device__ unsigned long long emi_attn_trace_buf[8 * 40];
-#define EMI_ATRACE() do { if (tracing && nts < 40) ts[nts++] = __builtin_readcyclecounter(); } while (0)
-#else
-#define EMI_ATRACE() do { } while (0)
-#endif
 template <int D, bool VT>
 __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ k,
                                                           const uint16_t* __restrict__ v, uint16_t* __restrict__ o,
@@ -633,9 +621,6 @@ __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(const uint16_t* __rest
   int blk, bh;
   attn_block_coords(&blk, &bh);
   const int qblk = gridDim.x - 1 - blk;              // longest rows first
-#ifdef EMI_ATTN_BLOCKLOG
-  const unsigned long long log_w0 = wall_clock64(), log_c0 = __builtin_readcyclecounter();
-#endif
   const int64_t base = (int64_t)(bh / sh.heads) * sh.sb + (int64_t)(bh % sh.heads) * sh.sh;
   const int seq = sh.seq;
   const int q0 = qblk * BQ + wave * 32;
@@ -661,16 +646,9 @@ __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(const uint16_t* __rest
   f32x16_t s[2];
   bf16x8_t pf[2][2];
 
-#ifdef EMI_ATTN_TRACE
-  unsigned long long ts[40];
-  int nts = 0;
-  bool tracing = false;
-#endif
   auto phase_end = [&]() __attribute__((always_inline)) {
     __builtin_amdgcn_sched_barrier(0);
-    EMI_ATRACE();
     __builtin_amdgcn_s_barrier();
-    EMI_ATRACE();
     __builtin_amdgcn_sched_barrier(0);
   };
   auto issue_bundle = [&](int jb, int slot) __attribute__((always_inline)) {
@@ -786,40 +764,23 @@ __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(const uint16_t* __rest
     phase_end();
   };
 
-#ifdef EMI_ATTN_BLOCKLOG
-  const unsigned long long log_c1 = __builtin_readcyclecounter();
-#endif
   issue_bundle(-1, 0);
   issue_bundle(0, 1);
   __builtin_amdgcn_s_waitcnt(0x0f70);                 // vmcnt(0)
   issue_bundle(1, 2);
   phase_end();
-#ifdef EMI_ATTN_BLOCKLOG
-  const unsigned long long log_c2 = __builtin_readcyclecounter();
-#endif
   if (wave >= 4) phase_end();                         // second group runs one phase behind
   __builtin_amdgcn_s_setprio(1);
   mfma_phase(std::true_type{}, std::false_type{}, 0);      // MFMA phase -1
   __builtin_amdgcn_s_setprio(0);
   phase_end();
   for (int j = 0; j < nt; j += 3) {
-#ifdef EMI_ATTN_TRACE
-    tracing = (blockIdx.x == 0 && blockIdx.y == 5 && j >= 9 && j < 18);
-#endif
     step(std::integral_constant<int, 1>{}, j);
     if (j + 1 < nt) step(std::integral_constant<int, 2>{}, j + 1);
     if (j + 2 < nt) step(std::integral_constant<int, 0>{}, j + 2);
   }
-#ifdef EMI_ATTN_TRACE
-  tracing = false;
-  if (blockIdx.x == 0 && blockIdx.y == 5 && lane == 0)
-    for (int i = 0; i < 40; i++) emi_attn_trace_buf[wave * 40 + i] = i < nts ? ts[i] : 0ull;
-#endif
   if (wave < 4) phase_end();
   __builtin_amdgcn_s_waitcnt(0x0f70);                 // loads past the last tile
-#ifdef EMI_ATTN_BLOCKLOG
-  const unsigned long long log_c3 = __builtin_readcyclecounter();
-#endif
 
   // Epilogue.  A lane owns one query and, per register quad, four consecutive d: written
   // straight to HBM that is 8 bytes per lane to 32 different rows.  Instead each wavefront
@@ -852,20 +813,6 @@ __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(const uint16_t* __rest
       if (q0 + row < seq) *reinterpret_cast<u32x4_t*>(o + base + (int64_t)(q0 + row) * sh.ss + c * 8) = v4;
     }
   }
-#ifdef EMI_ATTN_BLOCKLOG
-  if (threadIdx.x == 0) {
-    const int lin = blockIdx.y * gridDim.x + blockIdx.x;
-    if (lin < 4096) {
-      emi_attn_blocklog[lin * 4 + 0] = log_w0;
-      emi_attn_blocklog[lin * 4 + 1] = wall_clock64();
-      const unsigned long long log_c4 = __builtin_readcyclecounter();
-      // packed: total cycles (24 bits) | q load (12, /16) | prologue (12, /16) | epilogue (12, /16)
-      emi_attn_blocklog[lin * 4 + 2] = (log_c4 - log_c0) | (((log_c1 - log_c0) >> 4) << 24) | (((log_c2 - log_c1) >> 4) << 36) |
-                                       (((log_c4 - log_c3) >> 4) << 48);
-      emi_attn_blocklog[lin * 4 + 3] = ((unsigned long long)qblk << 32) | (unsigned)bh;
-    }
-  }
-#endif
 }
 
 // ---------------------------------------------------------------------------
@@ -973,136 +920,6 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_bf16_kernel(const uint16_t
         w.x = pack_bf16x2(acc[dt][4 * jj] * scale, acc[dt][4 * jj + 1] * scale);
         w.y = pack_bf16x2(acc[dt][4 * jj + 2] * scale, acc[dt][4 * jj + 3] * scale);
         *reinterpret_cast<uint2*>(out + dcol) = w;
-      }
-  }
-}
-
-// ---------------------------------------------------------------------------
-// dK, dV: block = 4 waves x 32 keys; Q and dO tiles of 64 queries through LDS.
-//   S = Q K^T, dP = dO V^T (lane = key, registers = queries)
-//   dV^T = dO^T P, dK^T = Q^T dS
-// ---------------------------------------------------------------------------
-template <int D>
-__global__ __launch_bounds__(256) void attn_bwd_dkv_bf16_kernel(const uint16_t* __restrict__ q,
-                                                                const uint16_t* __restrict__ k,
-                                                                const uint16_t* __restrict__ v,
-                                                                const uint16_t* __restrict__ d_o,
-                                                                const float* __restrict__ lse,
-                                                                const float* __restrict__ delta,
-                                                                uint16_t* __restrict__ dk, uint16_t* __restrict__ dv,
-                                                                AttnShape sh, uint32_t head_bytes, float scale,
-                                                                int causal) {
-  constexpr int BKEY = 128, BQT = 64, NW = 4;
-  constexpr int TILE = BQT * D * 2, STAGE = 2 * TILE + 2 * BQT * 4;   // Q, dO, lse, delta
-  extern __shared__ __attribute__((aligned(1024))) uint8_t smem_raw[];
-  EMI_LDS uint8_t* smem = (EMI_LDS uint8_t*)smem_raw;
-  const int lane = threadIdx.x & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  int kblk, bh;                                        // early key blocks see the most queries: first
-  attn_block_coords(&kblk, &bh);
-  const int64_t base = (int64_t)(bh / sh.heads) * sh.sb + (int64_t)(bh % sh.heads) * sh.sh;
-  const int seq = sh.seq;
-  const int k0 = kblk * BKEY + wave * 32;
-  const int krow = k0 + (lane & 31);
-  const float scale_log2e = scale * kLog2e;
-
-  bf16x8_t kf[D / 16], vf[D / 16];
-  load_reg_rows<D>(k + base, krow, seq, sh.ss, lane, kf);
-  load_reg_rows<D>(v + base, krow, seq, sh.ss, lane, vf);
-
-  const __amdgpu_buffer_rsrc_t rQ = attn_rsrc(q + base, head_bytes);
-  const __amdgpu_buffer_rsrc_t rDO = attn_rsrc(d_o + base, head_bytes);
-  const float* lse_h = lse + (int64_t)bh * seq;
-  const float* delta_h = delta + (int64_t)bh * seq;
-  const int qt0 = causal ? (kblk * BKEY) / BQT : 0;     // first query tile that can see this key block
-  const int nqt = (seq + BQT - 1) / BQT;
-
-  f32x16_t acc_k[D / 32], acc_v[D / 32];
-#pragma unroll
-  for (int dt = 0; dt < D / 32; dt++)
-#pragma unroll
-    for (int r = 0; r < 16; r++) acc_k[dt][r] = 0.f, acc_v[dt][r] = 0.f;
-
-  auto issue = [&](int stage, int qt) {
-    EMI_LDS uint8_t* s0 = smem + stage * STAGE;
-    load_rows_tile<D, BQT, NW>(rQ, s0, wave, lane, qt * BQT, seq, sh.ss);
-    load_rows_tile<D, BQT, NW>(rDO, s0 + TILE, wave, lane, qt * BQT, seq, sh.ss);
-    if (threadIdx.x < BQT) {
-      const int qi = qt * BQT + threadIdx.x;
-      EMI_LDS float* st = (EMI_LDS float*)(s0 + 2 * TILE);
-      st[threadIdx.x] = qi < seq ? lse_h[qi] * kLog2e : 0.f;
-      st[BQT + threadIdx.x] = qi < seq ? delta_h[qi] : 0.f;
-    }
-  };
-
-  if (qt0 < nqt) issue(0, qt0);
-  __builtin_amdgcn_s_waitcnt(0x0070);   // vmcnt(0) and lgkmcnt(0)
-  __syncthreads();
-
-  for (int qt = qt0; qt < nqt; qt++) {
-    const int it = qt - qt0;
-    if (qt + 1 < nqt) issue((it + 1) & 1, qt + 1);
-    const EMI_LDS uint8_t* sQ = smem + (it & 1) * STAGE;
-    const EMI_LDS uint8_t* sDO = sQ + TILE;
-    const EMI_LDS float* sL = (const EMI_LDS float*)(sQ + 2 * TILE);
-    const EMI_LDS float* sDl = sL + BQT;
-    const int qbase = qt * BQT;
-    if (!(causal && qbase + BQT - 1 < k0)) {          // some query of the tile can see some key of this wave
-      const bool need_mask = (causal && qbase < k0 + 31) || qbase + BQT > seq || k0 + 32 > seq;
-#pragma unroll 1
-      for (int T = 0; T < 2; T++) {
-        f32x16_t s, dp;
-#pragma unroll
-        for (int r = 0; r < 16; r++) s[r] = 0.f, dp[r] = 0.f;
-#pragma unroll
-        for (int t = 0; t < D / 16; t++) {
-          s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(row_frag<D>(sQ, T * 32, t, lane), kf[t], s, 0, 0, 0);
-          dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(row_frag<D>(sDO, T * 32, t, lane), vf[t], dp, 0, 0, 0);
-        }
-        f32x16_t ds;
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-          const int ql = T * 32 + acc_row(r, lane);     // query inside the tile
-          float p = fast_exp2(s[r] * scale_log2e - sL[ql]);
-          if (need_mask) {
-            const int qi = qbase + ql;
-            if ((causal && krow > qi) || qi >= seq || krow >= seq) p = 0.f;
-          }
-          s[r] = p;
-          ds[r] = p * (dp[r] - sDl[ql]);
-        }
-#pragma unroll
-        for (int sI = 0; sI < 2; sI++) {
-          const bf16x8_t pf = acc_to_frag(s, sI);
-          const bf16x8_t dsf = acc_to_frag(ds, sI);
-#pragma unroll
-          for (int dt = 0; dt < D / 32; dt++) {
-            acc_v[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(col_frag<D>(sDO, T * 32 + sI * 16, dt * 32, lane), pf,
-                                                                acc_v[dt], 0, 0, 0);
-            acc_k[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(col_frag<D>(sQ, T * 32 + sI * 16, dt * 32, lane), dsf,
-                                                                acc_k[dt], 0, 0, 0);
-          }
-        }
-      }
-    }
-    __builtin_amdgcn_s_waitcnt(0x0070);
-    __syncthreads();
-  }
-  if (krow < seq) {
-    uint16_t* outk = dk + base + (int64_t)krow * sh.ss;
-    uint16_t* outv = dv + base + (int64_t)krow * sh.ss;
-#pragma unroll
-    for (int dt = 0; dt < D / 32; dt++)
-#pragma unroll
-      for (int jj = 0; jj < 4; jj++) {
-        const int dcol = dt * 32 + 8 * jj + 4 * (lane >> 5);
-        uint2 w;
-        w.x = pack_bf16x2(acc_k[dt][4 * jj] * scale, acc_k[dt][4 * jj + 1] * scale);
-        w.y = pack_bf16x2(acc_k[dt][4 * jj + 2] * scale, acc_k[dt][4 * jj + 3] * scale);
-        *reinterpret_cast<uint2*>(outk + dcol) = w;
-        w.x = pack_bf16x2(acc_v[dt][4 * jj], acc_v[dt][4 * jj + 1]);
-        w.y = pack_bf16x2(acc_v[dt][4 * jj + 2], acc_v[dt][4 * jj + 3]);
-        *reinterpret_cast<uint2*>(outv + dcol) = w;
       }
   }
 }
@@ -1590,11 +1407,6 @@ int launch_attn_jvp_mfma(hipStream_t st, const void* q, const void* k, const voi
 
 using namespace emi;
 
-#ifdef EMI_ATTN_TRACE
-extern "C" int emi_debug_attn_trace(unsigned long long* out) {
-  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(emi_attn_trace_buf), sizeof(unsigned long long) * 8 * 40);
-}
-#endif
 
 // The generic kernels read four elements per load when every row starts on a 4-element boundary (8 bytes of bf16,
 // 16 of fp32) and head_dim is a multiple of 4.
@@ -1626,14 +1438,13 @@ extern "C" int emi_attn_fwd_ws(emi_stream_t stream, const void* q, const void* k
   if (mfma_ok(a, dtype, {q, k, v, o})) {
     const uint32_t head_bytes = (uint32_t)(((seq - 1) * stride_s + head_dim) * 2);
     const float sl2 = scale * kLog2e;
-    static const int fwd_variant = getenv("EMI_ATTN_FWD") ? atoi(getenv("EMI_ATTN_FWD")) : 1;
-    if (fwd_variant >= 1 && seq >= 256) {
+    if (seq >= 256) {
       const dim3 gridp((unsigned)((seq + 255) / 256), bh);
       const int s_pad = (int)((seq + 63) / 64 * 64);
       const size_t need = emi_attn_fwd_workspace_bytes(batch, heads, seq, head_dim);
       // With a workspace V is transposed once (keys contiguous); without one the kernel
       // falls back to transposing LDS reads of V.
-      const bool vt = fwd_variant == 1 && workspace != nullptr && workspace_bytes >= need && aligned16(workspace) &&
+      const bool vt = workspace != nullptr && workspace_bytes >= need && aligned16(workspace) &&
                       (int64_t)head_dim * s_pad * 2 < 0x7fffff00LL && bh <= 65535;
 #define EMI_ATTN_FWD_PP(DD)                                                                                          \
   do {                                                                                                               \
@@ -1717,10 +1528,7 @@ extern "C" int emi_attn_bwd(emi_stream_t stream, const void* q, const void* k, c
   float* lse2 = delta + (size_t)batch * heads * seq;
   const dim3 grid4((unsigned)((seq + 3) / 4), bh);
   const bool fast = mfma_ok(a, dtype, {q, k, v, o, d_o, dq, dk, dv});
-  // EMI_ATTN_BWD=0 selects the plain dK/dV kernel (for comparison); the software-pipelined
-  // one wants -delta in the workspace.
-  static const int bwd_variant = getenv("EMI_ATTN_BWD") ? atoi(getenv("EMI_ATTN_BWD")) : 1;
-  const float delta_sign = bwd_variant == 1 ? -1.0f : 1.0f;
+  const float delta_sign = -1.0f;          // the MFMA kernels accumulate dP onto -delta
   if (fast) {
     if (head_dim == 128)
       hipLaunchKernelGGL(attn_prep_kernel<128>, dim3((unsigned)((seq + 15) / 16), bh), dim3(256), 0, st, (const uint16_t*)o,
@@ -1740,19 +1548,12 @@ extern "C" int emi_attn_bwd(emi_stream_t stream, const void* q, const void* k, c
     const dim3 grid((unsigned)((seq + 127) / 128), bh);
 #define EMI_ATTN_BWD_LAUNCH(DD)                                                                                          \
   do {                                                                                                                   \
-    constexpr int smem_q = 2 * 2 * 64 * DD * 2, smem_kv = 2 * (2 * 64 * DD * 2 + 2 * 64 * 4);                            \
+    constexpr int smem_q = 2 * 2 * 64 * DD * 2;                                                                          \
     constexpr int smem_sp = 6 * 64 * DD * 2 + 3 * 512;                                                                   \
-    if (bwd_variant == 1) {                                                                                              \
-      if (int rc = reserve_lds(attn_bwd_dkv_sp_kernel<DD>, smem_sp, "emi_attn_bwd")) return rc;                          \
-      hipLaunchKernelGGL(attn_bwd_dkv_sp_kernel<DD>, grid, dim3(256), smem_sp, st, (const uint16_t*)q,                   \
-                         (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse2, delta, (uint16_t*)dk,       \
-                         (uint16_t*)dv, shp, head_bytes, scale, causal);                                                 \
-    } else {                                                                                                             \
-      if (int rc = reserve_lds(attn_bwd_dkv_bf16_kernel<DD>, smem_kv, "emi_attn_bwd")) return rc;                        \
-      hipLaunchKernelGGL(attn_bwd_dkv_bf16_kernel<DD>, grid, dim3(256), smem_kv, st, (const uint16_t*)q,                 \
-                         (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, (uint16_t*)dk,        \
-                         (uint16_t*)dv, shp, head_bytes, scale, causal);                                                 \
-    }                                                                                                                    \
+    if (int rc = reserve_lds(attn_bwd_dkv_sp_kernel<DD>, smem_sp, "emi_attn_bwd")) return rc;                            \
+    hipLaunchKernelGGL(attn_bwd_dkv_sp_kernel<DD>, grid, dim3(256), smem_sp, st, (const uint16_t*)q,                     \
+                       (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse2, delta, (uint16_t*)dk,         \
+                       (uint16_t*)dv, shp, head_bytes, scale, causal);                                                   \
     EMI_CHECK_LAUNCH("emi_attn_bwd(dkv)");                                                                               \
     if (int rc = reserve_lds(attn_bwd_dq_bf16_kernel<DD>, smem_q, "emi_attn_bwd")) return rc;                            \
     hipLaunchKernelGGL(attn_bwd_dq_bf16_kernel<DD>, grid, dim3(256), smem_q, st, (const uint16_t*)q, (const uint16_t*)k, \

@@ -438,7 +438,9 @@ __global__ __launch_bounds__(256) void embedding_bwd_kernel(const int32_t* __res
                                                             int64_t n_tokens, int64_t vocab, int64_t dim) {
   const int64_t t = blockIdx.x;
   int64_t tok = tokens[t];
-  if (tok < 0 || tok >= vocab) return;                     // out-of-range updates are dropped (scatter)
+  // Out-of-range updates are dropped while the forward clamps: this pair is what the reference's program does
+  // (gather clamps its start indices, the scatter-add its adjoint rule emits drops updates that fall outside).
+  if (tok < 0 || tok >= vocab) return;
   for (int64_t c = threadIdx.x; c < dim; c += 256) atomicAdd(acc + tok * dim + c, to_f32(dx[t * dim + c]));
 }
 

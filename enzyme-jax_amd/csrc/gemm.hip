@@ -1010,19 +1010,6 @@ static int launch_bf16_pingpong(hipStream_t st, const void* A, const void* B, co
   return EMI_OK;
 }
 
-// Tile configuration.  EMI_GEMM_TILE (read once) overrides the choice for tuning:
-//   0 = automatic, 1 = 256x256x64 2-stage 8 waves, 2 = 256x256x32 4-stage 8 waves
-//   (slower: 64-byte rows double the cache-line requests per byte), 4 = 128x128x64,
-//   5 = 256x256x64 ping-pong (NT layout only).
-static int tile_override() {
-  static int v = -1;
-  if (v < 0) {
-    const char* e = getenv("EMI_GEMM_TILE");
-    v = e ? atoi(e) : 0;
-  }
-  return v;
-}
-
 // The 128x128 bf16 kernel on few tiles and a long contraction (the weight gradients of a small model:
 // dW[768, 768] over 8192 tokens is 36 tiles): two blocks per CU, at least 1024 of K per block.
 static int bf16_splits(int64_t M, int64_t N, int64_t K) {
@@ -1038,28 +1025,15 @@ template <bool AK, bool BKM>
 static int launch_bf16_layout(hipStream_t st, const void* A, const void* B, const void* R, void* C, int M, int N, int K,
                               int lda, int ldb, int ldr, int ldc, uint32_t a_bytes, uint32_t b_bytes, void* workspace,
                               size_t workspace_bytes) {
-  int cfg = tile_override();
-  if (cfg == 0) {
-    const int splits = bf16_splits(M, N, K);
-    if (splits > 1 && workspace != nullptr && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0 &&
-        workspace_bytes >= (size_t)splits * M * N * sizeof(float))
-      return launch_bf16<128, 128, 64, 2, 2, 2, AK, BKM>(st, A, B, R, C, M, N, K, lda, ldb, ldr, ldc, a_bytes, b_bytes,
-                                                        static_cast<float*>(workspace), splits);
-  }
-  if (cfg == 0) {
-    // 256x256 tiles when they fill the chip (the ping-pong kernel for two
-    // k-contiguous operands), else 128x128.
-    const int64_t big_tiles = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
-    cfg = big_tiles >= 192 ? 5 : 4;
-  }
-#define EMI_GEMM_ARGS st, A, B, R, C, M, N, K, lda, ldb, ldr, ldc, a_bytes, b_bytes
-  switch (cfg) {
-    case 1: return launch_bf16<256, 256, 64, 2, 2, 4, AK, BKM>(EMI_GEMM_ARGS);
-    case 5: return launch_bf16_pingpong<AK, BKM>(EMI_GEMM_ARGS);
-    case 2: return launch_bf16<256, 256, 32, 4, 2, 4, AK, BKM>(EMI_GEMM_ARGS);
-    default: return launch_bf16<128, 128, 64, 2, 2, 2, AK, BKM>(EMI_GEMM_ARGS);
-  }
-#undef EMI_GEMM_ARGS
+  const int splits = bf16_splits(M, N, K);
+  if (splits > 1 && workspace != nullptr && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0 &&
+      workspace_bytes >= (size_t)splits * M * N * sizeof(float))
+    return launch_bf16<128, 128, 64, 2, 2, 2, AK, BKM>(st, A, B, R, C, M, N, K, lda, ldb, ldr, ldc, a_bytes, b_bytes,
+                                                      static_cast<float*>(workspace), splits);
+  // 256x256 tiles (the ping-pong kernel) when they fill the chip, else 128x128.
+  const int64_t big_tiles = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
+  if (big_tiles >= 192) return launch_bf16_pingpong<AK, BKM>(st, A, B, R, C, M, N, K, lda, ldb, ldr, ldc, a_bytes, b_bytes);
+  return launch_bf16<128, 128, 64, 2, 2, 2, AK, BKM>(st, A, B, R, C, M, N, K, lda, ldb, ldr, ldc, a_bytes, b_bytes);
 }
 
 template <typename T>

@@ -576,7 +576,7 @@ def concatenate(xs, dim):
             hi = list(c.shape)
             lo[dim], hi[dim] = at, at + x.shape[dim]
             at += x.shape[dim]
-            out.append(_accumulate(acc[i], _slice(c, lo, hi, [1] * c.dim())))
+            out.append(_accumulate(acc[i], _contig(_slice(c, lo, hi, [1] * c.dim()))))
         return out
 
     Tape.record(tuple(xs), y, rule)

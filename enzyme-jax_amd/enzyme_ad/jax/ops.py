@@ -344,6 +344,9 @@ def transpose(a):
     out = torch.empty((cols, rows), dtype=a.dtype, device=a.device)
     N.check(N.lib().emi_transpose(_stream(), _p(a), _p(out), rows, cols, _code(a)))
     Tape.record((a,), out, lambda c, acc: (_accumulate(acc[0], transpose(c)),))
+    tans = _tan(a)
+    if tans is not None and tans[0] is not None:
+        _set_tan(out, _quiet(lambda: transpose(tans[0])))      # linear: the tangent is transposed
     return out
 
 
@@ -637,12 +640,18 @@ def select(w, i):
 
     def rule(c, acc):
         g = acc[0]
-        if g is None:
-            g = torch.zeros_like(w)          # device memset
-            g[i].copy_(c)                    # device-to-device copy
-        else:
+        if g is not None and getattr(g, "_emi_select_owned", False):
+            # a buffer an earlier select rule zero-filled and nobody else holds: add slice i in place
             N.check(N.lib().emi_add(_stream(), _p(g[i]), _p(c), _p(g[i]), c.numel(), _code(c)))
-        return (g,)
+            return (g,)
+        fresh = torch.zeros_like(w)          # device memset
+        fresh[i].copy_(c)                    # device-to-device copy
+        if g is None:
+            fresh._emi_select_owned = True
+            return (fresh,)
+        # the accumulated cotangent came from another rule (it may be shared with another operand or be the
+        # caller's own tensor): never written in place
+        return (add(g, fresh),)
 
     Tape.record((w,), y, rule)
     tans = _tan(w)

@@ -16,8 +16,12 @@ Pinning status:
   maximum, power, cosine, sine, transpose ... pinned by the lit vectors.
   dot_general ... pinned by the IR form in dot_general.mlir (operand order and
       transposition) plus the <Jv,w> = <v,J^T w> identity against numpy matmul.
-  reduce(add), broadcast_in_dim, convert, reshape, select ... pinned by
-      the same adjoint identity and by finite differences (tests).
+  reduce(add), broadcast_in_dim, concatenate, slice ... pinned by the adjoint
+      identity and hand-worked index cases (tests/test_oracle_rules.py).
+  select ... pinned by the REVERSE / FORWARD check lines of select.mlir
+      evaluated by hand on a vector, plus the adjoint identity.
+  reshape ... pinned by a hand-worked row-major index case + adjoint identity.
+  convert ... pinned by the result element type and its rounding.
   reduce(max) ... no numeric vector in the reference; pinned by the closed form
       stated in the C++ (cotangent to every element equal to the max) and by
       the softmax shift-invariance test (its contribution cancels).

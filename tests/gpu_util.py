@@ -29,3 +29,17 @@ def check(got, ref, dt, what, factor=1.0):
     assert np.all(np.isfinite(host(got) if isinstance(got, torch.Tensor) else got)), what + ": non-finite values"
     assert e <= TOL[dt] * factor, "%s: max rel err %.3e > %.1e" % (what, e, TOL[dt] * factor)
     return e
+
+
+def check_rows(got, ref, dt, what, factor=1.0, floor=1e-3):
+    """Row-wise companion of `check`: every row's error is bounded relative to that row's own largest reference
+    entry (rows much smaller than the tensor's maximum are invisible to the max-norm metric).  `floor` (relative to
+    the tensor's maximum) keeps rows that are zero up to cancellation from demanding more than the arithmetic has."""
+    got = host(got) if isinstance(got, torch.Tensor) else np.asarray(got, dtype=np.float64)
+    ref = np.asarray(ref, dtype=np.float64)
+    got, ref = got.reshape(-1, got.shape[-1]), ref.reshape(-1, ref.shape[-1])
+    den = np.maximum(np.max(np.abs(ref), axis=1), floor * float(np.max(np.abs(ref))) or 1.0)
+    e = np.max(np.abs(got - ref), axis=1) / den
+    worst = int(np.argmax(e))
+    assert e[worst] <= TOL[dt] * factor, "%s: row %d rel err %.3e > %.1e" % (what, worst, e[worst], TOL[dt] * factor)
+    return float(e[worst])

@@ -159,7 +159,9 @@ def test_c4_stories110m_full_size():
     dout = _randn(tuple(out.shape), "bf16", 90)
     (gw,) = f_vjp(dout)
     (gw2,) = f_vjp(dout * 2)
-    assert all(torch.equal(gw2[k_], gw[k_] * 2) for k_ in gw)
+    # bit for bit, except the embedding table: its scatter-add uses fp32 atomics, whose order is not fixed
+    assert all(torch.equal(gw2[k_], gw[k_] * 2) for k_ in gw if k_ != "token_embedding_table")
+    assert rel_err(host(gw2["token_embedding_table"]), 2 * host(gw["token_embedding_table"])) <= 2 ** -7
     tw = {k_: _randn(v_.shape, "bf16", 100 + i, 0.02) for i, (k_, v_) in enumerate(wd.items())}
     _, tout = jvp(fn, (wd,), (tw,))
     lhs = _dot(tout, dout)

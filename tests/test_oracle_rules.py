@@ -93,3 +93,61 @@ def test_clamp_rule_matches_reference_vector():
     np.testing.assert_array_equal(np.clip(x, g["min"], g["max"]), g["out"])
     (dx,) = R.vjp_clamp_operand(g["min"], x, g["max"], np.ones_like(x))
     np.testing.assert_array_equal(dx, g["grad_operand"])
+
+
+def test_select_rule_has_reference_ir_form():
+    """select.mlir REVERSE check lines, evaluated by hand on a vector: the cotangent d goes to
+    on_true where pred holds and to on_false elsewhere (`select %pred, %d, %zero` /
+    `select %pred, %zero, %d`); the predicate is inactive (HLODerivatives.td:1297-1304)."""
+    pred = np.array([True, False, True, False])
+    a = np.array([1.0, 2.0, 3.0, 4.0])
+    b = np.array([-1.0, -2.0, -3.0, -4.0])
+    d = np.array([3.0, 5.0, 7.0, 11.0])
+    da, db = R.vjp_select(pred, a, b, d)
+    np.testing.assert_array_equal(da, [3.0, 0.0, 7.0, 0.0])
+    np.testing.assert_array_equal(db, [0.0, 5.0, 0.0, 11.0])
+    # the two cotangents partition d, and J^T is the transpose of the forward's linear map
+    np.testing.assert_array_equal(da + db, d)
+    rng = np.random.default_rng(2)
+    va, vb = rng.standard_normal(4), rng.standard_normal(4)
+    assert np.isclose(np.sum(np.where(pred, va, vb) * d), np.sum(va * da) + np.sum(vb * db))
+    # FORWARD check lines: the tangent is select(pred, ta, tb)
+    eps = 1e-6
+    fd = (np.where(pred, a + eps * va, b + eps * vb) - np.where(pred, a - eps * va, b - eps * vb)) / (2 * eps)
+    np.testing.assert_allclose(np.sum(fd * d), np.sum(va * da) + np.sum(vb * db), rtol=1e-9)
+
+
+def test_reshape_rule_is_row_major_inverse():
+    """HLODerivatives.td:1271: the cotangent is reshaped to the operand's type. Element k of the
+    flattened cotangent must land on element k of the flattened operand (row-major both ways)."""
+    x = np.zeros((2, 3))
+    d = np.array([[0.0, 1.0], [2.0, 3.0], [4.0, 5.0]])            # cotangent of reshape(x, (3, 2))
+    (dx,) = R.vjp_reshape(x, d)
+    np.testing.assert_array_equal(dx, [[0.0, 1.0, 2.0], [3.0, 4.0, 5.0]])
+    rng = np.random.default_rng(3)
+    v = rng.standard_normal((2, 3, 4))
+    w = rng.standard_normal((6, 4))
+    (g,) = R.vjp_reshape(v, w)
+    assert g.shape == v.shape
+    assert np.isclose(np.sum(np.reshape(v, (6, 4)) * w), np.sum(v * g))
+    # a transposing "reshape" (the plausible mistake) fails the index check above: (2,3)->(3,2) via .T
+    assert not np.array_equal(d.T, dx)
+
+
+def test_convert_rule_returns_operand_type():
+    """HLODerivatives.td:1290-1295: `Convert (TypeOf $x), (DiffeRet)`: the cotangent takes the operand's
+    element type, with that type's rounding (a float64 cotangent of a float32 operand loses its low bits;
+    float16 likewise)."""
+    x32 = np.array([1.0, 2.0], dtype=np.float32)
+    d64 = np.array([1.0 + 2.0 ** -30, 3.0], dtype=np.float64)
+    (g,) = R.vjp_convert(x32, d64)
+    assert g.dtype == np.float32
+    np.testing.assert_array_equal(g, np.array([1.0, 3.0], dtype=np.float32))
+    x16 = np.array([1.0], dtype=np.float16)
+    (g16,) = R.vjp_convert(x16, np.array([1.0 + 2.0 ** -12], dtype=np.float32))
+    assert g16.dtype == np.float16 and g16[0] == np.float16(1.0)
+    # widening is exact, so <convert(v), w> = <v, convert^T(w)> holds bit for bit for representable values
+    v = np.array([0.5, -1.25], dtype=np.float32)
+    w = np.array([2.0, 4.0], dtype=np.float64)
+    (gt,) = R.vjp_convert(v, w)
+    assert float(np.sum(v.astype(np.float64) * w)) == float(np.sum(v * gt))
