@@ -145,7 +145,10 @@ def test_attention_whole_heads_full_size(cfg):
         for name, got, ref in (("o", o, ro), ("dq", dq, rdq), ("dk", dk, rdk), ("dv", dv, rdv)):
             g = host(pick(got, b, hh))
             check(g, ref[0, 0], "bf16", "%s of (batch %d, head %d)" % (name, b, hh))
-            check_rows(g, ref[0, 0], "bf16", "%s rows of (batch %d, head %d)" % (name, b, hh))
+            # row by row the gradients are held to 4x the bound: with few keys dS = P (dP - delta) cancels
+            # (delta is built from the rounded O), so a row's own error is not bounded by one bf16 rounding;
+            # a misplaced or missing row is off by ~100 %
+            check_rows(g, ref[0, 0], "bf16", "%s rows of (batch %d, head %d)" % (name, b, hh), factor=1.0 if name == "o" else 4.0)
 
 
 def _layer_weights(D, H, dt, seed):
