@@ -4,6 +4,8 @@
 // All of them stream 16-byte vectors per lane, keep a row in registers where a
 // reduction is needed, reduce across the 64-lane wavefront with DPP shuffles
 // and compute in fp32 whatever the storage type is.
+#include <mutex>
+
 #include "emi_device.h"
 
 namespace emi {
@@ -650,6 +652,50 @@ extern "C" int emi_rmsnorm_bwd(emi_stream_t stream, const void* x, const void* g
   EMI_DISPATCH_DTYPE("emi_rmsnorm_bwd", dtype,
                      rmsnorm_bwd_launch<float>(st, x, gamma, dy, dx_add, dx, dgamma, workspace, rows, dim, eps),
                      rmsnorm_bwd_launch<bf16>(st, x, gamma, dy, dx_add, dx, dgamma, workspace, rows, dim, eps));
+}
+
+// ---------------------------------------------------------------------------
+// Allocation-free variant of emi_rmsnorm_bwd for callers that cannot allocate (HIP graph capture, serving loops):
+// the fp32 partial rows of dgamma live in a file-scope device array instead of a caller workspace.  The array's
+// name is a host-side stand-in, not a device address; its address on each device is looked up once, with that
+// device current, and only that pointer is ever handed to a kernel.  Every call on a device shares the device's
+// array (overlapping calls on one device race); the kernels write every partial row they later read, so nothing
+// needs clearing between calls.
+// ---------------------------------------------------------------------------
+constexpr size_t kRmsScratchBytes = EMI_RMSNORM_BWD_NOALLOC_MAX_BYTES;      // (512 + 1) partial rows of 8192 floats
+static __device__ __align__(256) unsigned char emi_rms_scratch[kRmsScratchBytes];
+constexpr int kMaxDevices = 64;
+static void* g_rms_scratch_ptr[kMaxDevices];
+static std::mutex g_rms_scratch_mu;
+
+static int rms_scratch_for_current_device(void** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+    return emi_fail(EMI_INTERNAL, "emi_rmsnorm_bwd_noalloc: cannot identify the current device");
+  std::lock_guard<std::mutex> lock(g_rms_scratch_mu);
+  if (g_rms_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(emi_rms_scratch));
+    if (e != hipSuccess || p == nullptr)
+      return emi_fail(EMI_INTERNAL, "emi_rmsnorm_bwd_noalloc: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+    g_rms_scratch_ptr[dev] = p;
+  }
+  *out = g_rms_scratch_ptr[dev];
+  return EMI_OK;
+}
+
+extern "C" int emi_rmsnorm_bwd_noalloc(emi_stream_t stream, const void* x, const void* gamma, const void* dy,
+                                       const void* dx_add, void* dx, void* dgamma, int64_t rows, int64_t dim, float eps,
+                                       int dtype) {
+  EMI_REQUIRE(rows > 0 && dim > 0, "emi_rmsnorm_bwd_noalloc: bad shape rows=%lld dim=%lld", (long long)rows, (long long)dim);
+  const size_t need = emi_rmsnorm_bwd_workspace_bytes(rows, dim);
+  EMI_REQUIRE(need <= kRmsScratchBytes,
+              "emi_rmsnorm_bwd_noalloc: rows=%lld dim=%lld needs %zu bytes of scratch, the built-in array holds %zu "
+              "(dim <= 8192 and a multiple of 8 always fits); use emi_rmsnorm_bwd with a workspace",
+              (long long)rows, (long long)dim, need, kRmsScratchBytes);
+  void* scratch = nullptr;
+  if (int rc = rms_scratch_for_current_device(&scratch)) return rc;
+  return emi_rmsnorm_bwd(stream, x, gamma, dy, dx_add, dx, dgamma, scratch, kRmsScratchBytes, rows, dim, eps, dtype);
 }
 
 extern "C" int emi_rope_table(emi_stream_t stream, float* table, int64_t seq, int64_t head_dim, double theta,

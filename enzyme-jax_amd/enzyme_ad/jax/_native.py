@@ -23,6 +23,8 @@ SIGNATURES = {
     "emi_rmsnorm_bwd_workspace_bytes": (c_size_t, [c_i64, c_i64]),
     "emi_rmsnorm_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                 c_size_t, c_i64, c_i64, c_float, c_int]),
+    "emi_rmsnorm_bwd_noalloc": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_i64,
+                                        c_float, c_int]),
     "emi_rope_table": (c_int, [c_void_p, c_void_p, c_i64, c_i64, c_double, c_i64]),
     "emi_rope": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_i64, c_i64, c_i64, c_int, c_int]),
     "emi_swiglu_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_int]),

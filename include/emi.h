@@ -60,6 +60,18 @@ int emi_rmsnorm_bwd(emi_stream_t stream, const void* x, const void* gamma, const
                     const void* dx_add, void* dx, void* dgamma, void* workspace,
                     size_t workspace_bytes, int64_t rows, int64_t dim, float eps, int dtype);
 
+/* emi_rmsnorm_bwd without a workspace argument, for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid it).  No counterpart in the reference.  The dgamma
+ * partial rows go to an array of EMI_RMSNORM_BWD_NOALLOC_MAX_BYTES that the library holds on every device it
+ * has been called on, until the process ends; the call allocates and frees nothing (its first call on a device
+ * looks the array's address up).  Fails with EMI_INVALID_ARGUMENT when emi_rmsnorm_bwd_workspace_bytes(rows, dim)
+ * exceeds the array (any row count with dim <= 8192 and a multiple of 8 fits).  All calls on one device share
+ * the array: calls that overlap on one device (two streams, two threads) race; serialise them. */
+#define EMI_RMSNORM_BWD_NOALLOC_MAX_BYTES ((size_t)(512 + 1) * 8192 * 4)
+int emi_rmsnorm_bwd_noalloc(emi_stream_t stream, const void* x, const void* gamma, const void* dy,
+                            const void* dx_add, void* dx, void* dgamma, int64_t rows, int64_t dim,
+                            float eps, int dtype);
+
 /* RoPE angle table: table[s][j] = (cos, sin)(pos * theta^(-2j/head_dim)),
  * pos = pos0 + s, computed in float64 and rounded to fp32.  In the reference
  * these are trace-time constants (test/llama.py:127-140).
