@@ -419,37 +419,95 @@ def bench_models(iters):
     return out
 
 
-def cpu_baseline(cfg, seconds_hint=20):
-    """The numpy oracle of the same layer (fwd + bwd) on a bounded sample."""
-    import numpy as np
-    from oracle import llama_ref as L
+def _host_threads():
+    """Threads for the CPU baseline: the host cores this process may use (the scheduler affinity and an
+    OMP_NUM_THREADS limit both bound it)."""
+    n = os.cpu_count() or 1
     try:
-        from threadpoolctl import threadpool_info
-        threads = max([p.get("num_threads", 1) for p in threadpool_info()] or [1])
+        n = min(n, len(os.sched_getaffinity(0)))
     except Exception:
-        threads = os.cpu_count() or 1
+        pass
+    try:
+        n = min(n, int(os.environ.get("OMP_NUM_THREADS", n)))
+    except ValueError:
+        pass
+    return max(n, 1)
+
+
+def _cpu_model_name():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_baseline(cfg, repeats=5, budget_s=25.0):
+    """PyTorch-CPU restatement of test/llama.py (oracle/llama_torch.py), forward + autograd VJP in fp32 on all host
+    cores this process may use; warm-up 1, then the minimum over up to `repeats` runs (the reference harness reports
+    the minimum step time).  Always the 15M whole model (the configuration the reference's CPU path is quoted on); the
+    headline `value` is the same 7B layer as the GPU figure on a bounded sample of one 512-token sequence."""
+    import torch
+    from oracle import llama_torch as LT
+    threads = _host_threads()
+    torch.set_num_threads(threads)
+
+    def min_time(fn, budget):
+        fn()                                            # warm-up
+        best, t_start = None, time.perf_counter()
+        for _ in range(repeats):
+            t0 = time.perf_counter()
+            fn()
+            dt = time.perf_counter() - t0
+            best = dt if best is None else min(best, dt)
+            if time.perf_counter() - t_start > budget:
+                break
+        return best
+
+    g = torch.Generator().manual_seed(1)
+    # C1: dim 288, hidden 768, 6 layers, 6 heads, vocab 32000, batch 1 x seq 256, fp32, cotangent on the logits
+    c1 = dict(dim=288, hidden_dim=768, n_layers=6, n_heads=6, vocab_size=32000)
+    L_, D1, H1, V1 = c1["n_layers"], c1["dim"], c1["hidden_dim"], c1["vocab_size"]
+    shapes = dict(token_embedding_table=(V1, D1), rms_att_weight=(L_, D1), wq=(L_, D1, D1), wk=(L_, D1, D1), wv=(L_, D1, D1),
+                  wo=(L_, D1, D1), rms_ffn_weight=(L_, D1), w1=(L_, H1, D1), w2=(L_, D1, H1), w3=(L_, H1, D1),
+                  rms_final_weight=(D1,), wcls=(V1, D1))
+    w1 = {k: (torch.randn(shp, generator=g) * 0.02).requires_grad_(True) for k, shp in shapes.items()}
+    tok = torch.randint(0, V1, (1, 256), generator=g)
+    dlogits = torch.randn((1, 256, V1), generator=g)
+
+    def c1_step():
+        for t in w1.values():
+            t.grad = None
+        LT.model(tok, w1, c1, True).backward(dlogits)
+
+    t_c1 = min_time(c1_step, 6.0)
+    del w1, dlogits
+
+    # the headline layer (dim 4096, hidden 11008, 32 heads) on one sequence of 512 tokens
     D, H, nh = cfg["dim"], cfg["hidden_dim"], cfg["n_heads"]
     B, S = 1, 512
-    rng = np.random.Generator(np.random.PCG64(5))
-    f32 = np.float32
-    lw = {k: (rng.standard_normal(s, dtype=f32) * f32(0.02)) for k, s in
+    lw = {k: (torch.randn(shp, generator=g) * 0.02).requires_grad_(True) for k, shp in
           [("rms_att_weight", (D,)), ("wq", (D, D)), ("wk", (D, D)), ("wv", (D, D)), ("wo", (D, D)),
            ("rms_ffn_weight", (D,)), ("w1", (H, D)), ("w2", (D, H)), ("w3", (H, D))]}
-    x = rng.standard_normal((B, S, D), dtype=f32)
-    dy = rng.standard_normal((B, S, D), dtype=f32)
-    best = None
-    t_start = time.perf_counter()
-    for rep in range(3):
-        t0 = time.perf_counter()
-        y, cache = L.layer_fwd(x, lw, nh)
-        L.layer_bwd(dy, lw, cache, nh)
-        dt = time.perf_counter() - t0
-        best = dt if best is None else min(best, dt)
-        if time.perf_counter() - t_start > seconds_hint:
-            break
-    return dict(value=B * S / best, unit="tokens/s", cores=threads, kind="port",
-                sample="numpy fp32 oracle (oracle/llama_ref.py layer_fwd+layer_bwd), same 7B layer shape, "
-                       "batch 1 x seq 512 = 512 tokens, min of up to 3 runs (%.2f s each)" % best)
+    x = torch.randn((B, S, D), generator=g).requires_grad_(True)
+    dy = torch.randn((B, S, D), generator=g)
+
+    def layer_step():
+        x.grad = None
+        for t in lw.values():
+            t.grad = None
+        LT.layer(x, lw, nh).backward(dy)
+
+    t_layer = min_time(layer_step, budget_s - 8.0)
+    return dict(value=round(B * S / t_layer, 1), unit="tokens/s", cores=threads, kind="port", cpu=_cpu_model_name(),
+                sample="PyTorch-CPU fp32 restatement of test/llama.py (oracle/llama_torch.py), forward + autograd VJP, "
+                       "torch.set_num_threads(%d), warm-up 1, min of up to %d runs: the 7B layer of the GPU figure on "
+                       "batch 1 x seq 512 = 512 tokens (%.3f s per step)" % (threads, repeats, t_layer),
+                c1_stories15m=dict(tokens_per_s=round(256 / t_c1, 1), seconds_per_step=round(t_c1, 4),
+                                   sample="whole 15M model (dim 288, hidden 768, 6 layers, 6 heads, vocab 32000), "
+                                          "batch 1 x seq 256 tokens -> logits, cotangent on the logits, fp32"))
 
 
 def main():

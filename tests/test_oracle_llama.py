@@ -130,33 +130,8 @@ def test_layer_backward_matches_finite_differences():
 # ---- independent torch restatement (written against test/llama.py, not the oracle)
 
 def _torch_model(tokens, w, cfg, logits):
-    D, nh = cfg["dim"], cfg["n_heads"]
-    d = D // nh
-    x = w["token_embedding_table"][tokens]
-    B, S, _ = x.shape
-    pos = torch.arange(S, dtype=torch.float64)
-    freq = 1.0 / torch.pow(torch.tensor(10000.0, dtype=torch.float64), torch.arange(0, d, 2, dtype=torch.float64) / d)
-    ang = pos[:, None] * freq[None]
-    rot = torch.polar(torch.ones_like(ang), ang)      # complex rotation e^{i angle}
-
-    def norm(t, g):
-        return g * t * torch.rsqrt((t * t).mean(-1, keepdim=True) + 1e-5)
-
-    def rope(t):
-        tc = torch.view_as_complex(t.reshape(B, S, nh, d // 2, 2).contiguous())
-        return torch.view_as_real(tc * rot[None, :, None, :]).reshape(B, S, nh, d)
-
-    for i in range(cfg["n_layers"]):
-        xb = norm(x, w["rms_att_weight"][i])
-        q = rope((xb @ w["wq"][i].T).reshape(B, S, nh, d)).transpose(1, 2)
-        k = rope((xb @ w["wk"][i].T).reshape(B, S, nh, d)).transpose(1, 2)
-        v = (xb @ w["wv"][i].T).reshape(B, S, nh, d).transpose(1, 2)
-        o = torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True)
-        x = x + o.transpose(1, 2).reshape(B, S, D) @ w["wo"][i].T
-        xb = norm(x, w["rms_ffn_weight"][i])
-        x = x + (torch.nn.functional.silu(xb @ w["w1"][i].T) * (xb @ w["w3"][i].T)) @ w["w2"][i].T
-    x = norm(x, w["rms_final_weight"])
-    return x @ w["wcls"].T if logits else x
+    from oracle import llama_torch
+    return llama_torch.model(tokens, w, cfg, logits)
 
 
 @pytest.mark.parametrize("logits", [False, True])
