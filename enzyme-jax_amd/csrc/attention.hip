@@ -746,16 +746,17 @@ __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(const uint16_t* __rest
     }
     l += rs;
   };
-  // One tile step; bundle b(j) sits in slot (j + 1) % 3 = SLOT.  Every wavefront runs
-  // every step of its block (the barriers keep the eight in lockstep anyway); tiles in a
-  // wavefront's future are fully masked and contribute exact zeros, and the scores
-  // computed past the last tile are never used.
+  // One tile step; bundle b(j) sits in slot (j + 1) % 3 = SLOT.  Every wavefront meets every barrier and issues its
+  // share of every bundle, but a tile that lies wholly in the causal future of the wavefront's 32 queries (the
+  // last tiles of the block's diagonal, for the wavefronts with the lower queries) costs it neither softmax nor
+  // matrix work: nt_w is the number of tiles that hold a key this wavefront can see.
+  const int nt_w = causal ? ((q0 + 31) / BKV + 1 < nt ? (q0 + 31) / BKV + 1 : nt) : nt;
   auto step = [&](auto slot_c, int j) __attribute__((always_inline)) {
     constexpr int SLOT = decltype(slot_c)::value;
-    softmax(j);                                       // VALU phase
+    if (j < nt_w) softmax(j);                         // VALU phase
     phase_end();
     __builtin_amdgcn_s_setprio(1);                    // MFMA phase
-    mfma_phase(std::true_type{}, std::true_type{}, SLOT);
+    if (j < nt_w) mfma_phase(std::true_type{}, std::true_type{}, SLOT);    // (its last scores are never used)
     __builtin_amdgcn_s_setprio(0);
     // After the LDS reads of this phase: the compiler orders every LDS read behind all
     // outstanding direct-to-LDS loads, so loads issued earlier would be waited for here.
