@@ -17,6 +17,7 @@
 // (or key) row, plain fp32 FMA, same maths.
 #include <initializer_list>
 #include <type_traits>
+#include <utility>
 #include <stdlib.h>
 
 #include "emi_device.h"
@@ -538,60 +539,26 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_kernel(const uint16_t* _
   }
 }
 
-// V^T for the forward pass: vt[bh][d][s_pad] = v[b][s][h][d] (keys contiguous, rows
-// padded with zeros to a multiple of 64 keys), so that the P.V product can fetch its
-// V operand with plain 16-byte LDS reads instead of the slow transposing ones.
-template <int D>
-__global__ __launch_bounds__(256) void attn_vt_kernel(const uint16_t* __restrict__ v, uint16_t* __restrict__ vt,
-                                                      AttnShape sh, int s_pad) {
-  __shared__ uint16_t tile[64][66];
-  const int k0 = blockIdx.x * 64, d0 = blockIdx.y * 64, bh = blockIdx.z;
-  const int64_t base = (int64_t)(bh / sh.heads) * sh.sb + (int64_t)(bh % sh.heads) * sh.sh;
-#pragma unroll
-  for (int i = 0; i < 2; i++) {
-    const int idx = threadIdx.x + i * 256, r = idx >> 3, c = idx & 7;
-    uint4 w = make_uint4(0, 0, 0, 0);
-    if (k0 + r < sh.seq) w = *reinterpret_cast<const uint4*>(v + base + (int64_t)(k0 + r) * sh.ss + d0 + c * 8);
-    const uint32_t u[4] = {w.x, w.y, w.z, w.w};
-#pragma unroll
-    for (int e = 0; e < 8; e++) tile[r][c * 8 + e] = (uint16_t)(u[e >> 1] >> ((e & 1) * 16));
-  }
-  __syncthreads();
-#pragma unroll
-  for (int i = 0; i < 2; i++) {
-    const int idx = threadIdx.x + i * 256, dd = idx >> 3, c = idx & 7;
-    uint32_t u[4];
-#pragma unroll
-    for (int e = 0; e < 4; e++) u[e] = (uint32_t)tile[c * 8 + 2 * e][dd] | ((uint32_t)tile[c * 8 + 2 * e + 1][dd] << 16);
-    *reinterpret_cast<uint4*>(vt + ((int64_t)bh * D + d0 + dd) * s_pad + k0 + c * 8) = make_uint4(u[0], u[1], u[2], u[3]);
-  }
+// Transposing LDS read as inline assembly (the result is valid after an attn_tr_wait that covers it), and the wait:
+// at most N LDS operations issued after the two reads may still be outstanding.
+template <int OFF> __device__ __forceinline__ u32x2_t attn_tr_read(uint32_t addr) {
+  static_assert(OFF >= 0 && OFF < 65536, "ds offset field");
+  u32x2_t r;
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF));
+  return r;
+}
+template <int N> __device__ __forceinline__ void attn_tr_wait(u32x2_t& lo, u32x2_t& hi) {
+  static_assert(N >= 0 && N < 16, "lgkmcnt field");
+  asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(lo), "+v"(hi) : "n"(N));
 }
 
-// LDS tile [D][64 keys] of V^T: 128-byte rows, 16-byte chunk c of row r at chunk
-// c ^ ((r >> 1) & 7) (16 consecutive rows at one logical chunk cover all 64 banks).
-template <int D, int NW>
-__device__ __forceinline__ void load_vt_tile(__amdgpu_buffer_rsrc_t rsrc, EMI_LDS uint8_t* lds, int wave, int lane,
-                                             int key0, int s_pad) {
-  constexpr int NLOAD = D * 128 / 1024 / NW;       // wave-loads of 8 rows x 128 bytes
-  static_assert(NLOAD >= 1, "V^T tile smaller than one pass of the block");
-#pragma unroll
-  for (int it = 0; it < NLOAD; it++) {
-    const int r = (it * NW + wave) * 8 + (lane >> 3);
-    const int lc = (lane & 7) ^ ((r >> 1) & 7);
-    const uint32_t voff = (uint32_t)(r * s_pad + key0 + lc * 8) * 2u;      // key0 < s_pad always
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, lds + (it * NW + wave) * 1024, 16, voff, 0, 0, 0);
-  }
+template <typename F, int... Is>
+__device__ __forceinline__ void attn_static_for_impl(F&& f, std::integer_sequence<int, Is...>) {
+  (f(std::integral_constant<int, Is>{}), ...);
 }
-// Operand fragment "32 of D x 8 keys per lane": lane l holds D-index row_base + (l & 31),
-// keys 8*chunk .. +7 of the tile.
-__device__ __forceinline__ bf16x8_t vt_frag(const EMI_LDS uint8_t* tile, int row_base, int chunk, int lane) {
-  const int row = row_base + (lane & 31);
-  return *reinterpret_cast<const EMI_LDS bf16x8_t*>(tile + row * 128 + ((chunk ^ ((row >> 1) & 7)) << 4));
+template <int N, typename F> __device__ __forceinline__ void attn_static_for(F&& f) {
+  attn_static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
-// Key permutation inside a 32-row score tile (swaps bits 2 and 3): MFMA row m holds key
-// perm_key(m), which makes registers 8s..8s+7 of a lane's accumulator eight consecutive
-// keys, the order a 16-byte read of a V^T row delivers.
-__device__ __forceinline__ int perm_key(int m) { return (m & ~12) | ((m & 4) << 1) | ((m & 8) >> 1); }
 
 // ---------------------------------------------------------------------------
 // Forward, ping-pong form: block = 8 waves x 32 queries in two groups of four, one
@@ -606,11 +573,11 @@ __device__ __forceinline__ int perm_key(int m) { return (m & ~12) | ((m & 4) << 
 // than 8 (in log2 units), so the rescaling of O runs on a few early tiles only; P then
 // stays below 2^8 and the final O/l and log-sum-exp are exact for whatever m was used.
 // ---------------------------------------------------------------------------
-template <int D, bool VT>
+template <int D>
 __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ k,
                                                           const uint16_t* __restrict__ v, uint16_t* __restrict__ o,
                                                           float* __restrict__ lse, AttnShape sh, uint32_t head_bytes,
-                                                          float scale_log2e, int causal, int s_pad) {
+                                                          float scale_log2e, int causal) {
   constexpr int BQ = 256, BKV = 64, NW = 8;
   constexpr int TILE = BKV * D * 2, BUNDLE = 2 * TILE;
   constexpr int LPB = 2 * (BKV * D * 2 / 1024 / NW);       // loads per wave per bundle
@@ -630,12 +597,10 @@ __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(const uint16_t* __rest
   load_reg_rows<D>(q + base, qrow, seq, sh.ss, lane, qf);
 
   const __amdgpu_buffer_rsrc_t rK = attn_rsrc(k + base, head_bytes);
-  // VT: v is the transposed copy [bh][D][s_pad]
-  const __amdgpu_buffer_rsrc_t rV = VT ? attn_rsrc(v + (int64_t)bh * D * s_pad, (uint32_t)(D * s_pad * 2))
-                                       : attn_rsrc(v + base, head_bytes);
+  const __amdgpu_buffer_rsrc_t rV = attn_rsrc(v + base, head_bytes);
   const int kv_end = causal ? (qblk * BQ + BQ < seq ? qblk * BQ + BQ : seq) : seq;
   const int nt = (kv_end + BKV - 1) / BKV;
-  const int krow_l = VT ? perm_key(lane & 31) : (lane & 31);      // K row this lane feeds into the score MFMAs
+  const int krow_l = lane & 31;                      // K row this lane feeds into the score MFMAs
 
   f32x16_t acc_o[D / 32];
 #pragma unroll
@@ -656,30 +621,51 @@ __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(const uint16_t* __rest
     EMI_LDS uint8_t* sV = smem + 3 * TILE + slot * TILE;
     load_rows_tile<D, BKV, NW>(rK, sK, wave, lane, (jb + 1) * BKV, seq, sh.ss);
     const int vrow0 = jb < 0 ? 0 : jb * BKV;
-    if constexpr (VT) load_vt_tile<D, NW>(rV, sV, wave, lane, vrow0 < s_pad ? vrow0 : 0, s_pad);
-    else load_rows_tile<D, BKV, NW>(rV, sV, wave, lane, vrow0, seq, sh.ss);
+    load_rows_tile<D, BKV, NW>(rV, sV, wave, lane, vrow0, seq, sh.ss);
   };
-  // MFMA phase: scores of tile j+1 (DO_S) and P.V of tile j (DO_PV) out of bundle `slot`.
+  // MFMA phase: scores of tile j+1 (DO_S) and P.V of tile j (DO_PV) out of bundle SLOT.
   // The operand fragments go through a ring of DEPTH registers sets: the LDS read of
   // operation i + DEPTH is issued right after the MFMA of operation i, so the LDS latency
   // hides behind DEPTH MFMAs.
-  auto mfma_phase = [&](auto do_s_c, auto do_pv_c, int slot) __attribute__((always_inline)) {
+  // The V operand (V^T fragments of a row-major V tile) comes through transposing LDS reads, two 8-byte reads per
+  // fragment with the lane mapping of col_frag.  They are written as inline assembly with their own lgkmcnt waits: the compiler
+  // puts a wait for every outstanding direct-to-LDS load in front of a transposing read it knows of, which would
+  // make every MFMA phase wait for the bundle issued one step earlier.  vadr[dt][h]: LDS address of this lane's 8
+  // bytes for d-block dt, key rows h*8 + ..., key block 0, ring slot 0.
+  uint32_t vadr[D / 32][2];
+  {
+    const int i16 = lane & 15;
+#pragma unroll
+    for (int dt = 0; dt < D / 32; dt++)
+#pragma unroll
+      for (int h = 0; h < 2; h++) {
+        const int r = (lane >> 5) * 4 + (i16 >> 2) + 8 * h;
+        const int col = dt * 32 + ((lane >> 4) & 1) * 16 + (i16 & 3) * 4;
+        vadr[dt][h] = (uint32_t)(uintptr_t)(smem + 3 * TILE) + (uint32_t)(r * (D * 2) + (((col >> 3) ^ swz<D>(r)) << 4) + (col & 7) * 2);
+      }
+  }
+  auto mfma_phase = [&](auto do_s_c, auto do_pv_c, auto slot_c) __attribute__((always_inline)) {
     constexpr bool DO_S = decltype(do_s_c)::value, DO_PV = decltype(do_pv_c)::value;
+    constexpr int SLOT = decltype(slot_c)::value;
     constexpr int NS = DO_S ? 2 * (D / 16) : 0, NPV = DO_PV ? 4 * (D / 32) : 0, NOP = NS + NPV, DEPTH = 6;
     // K tiles of the three bundles first, then the V tiles: every fragment address is
     // one of a few per-lane bases plus an immediate offset below 64 KiB
-    const EMI_LDS uint8_t* sK = smem + slot * TILE;
-    const EMI_LDS uint8_t* sV = smem + 3 * TILE + slot * TILE;
-    auto fetch = [&](int i) __attribute__((always_inline)) -> bf16x8_t {
-      if (i < NS) {
-        const int t = i >> 1, T = i & 1;
+    const EMI_LDS uint8_t* sK = smem + SLOT * TILE;
+    bf16x8_t ring[DEPTH];
+    u32x2_t tlo[DEPTH], thi[DEPTH];            // halves of V fragments in flight (asm path)
+    auto fetch = [&](auto ic) __attribute__((always_inline)) {
+      constexpr int i = decltype(ic)::value;
+      if constexpr (i < NS) {
+        constexpr int t = i >> 1, T = i & 1;
         const int row = T * 32 + krow_l;
         const int chunk = (t * 2 + (lane >> 5)) ^ swz<D>(row);
-        return *reinterpret_cast<const EMI_LDS bf16x8_t*>(sK + row * (D * 2) + chunk * 16);
+        ring[i % DEPTH] = *reinterpret_cast<const EMI_LDS bf16x8_t*>(sK + row * (D * 2) + chunk * 16);
+      } else {
+        constexpr int x = i - NS, dt = x % (D / 32), sI = (x / (D / 32)) & 1, T = x / (2 * (D / 32));
+        constexpr int OFF = SLOT * TILE + (T * 32 + sI * 16) * (D * 2);
+        tlo[i % DEPTH] = attn_tr_read<OFF>(vadr[dt][0]);
+        thi[i % DEPTH] = attn_tr_read<OFF>(vadr[dt][1]);
       }
-      const int x = i - NS, dt = x % (D / 32), sI = (x / (D / 32)) & 1, T = x / (2 * (D / 32));
-      if constexpr (VT) return vt_frag(sV, dt * 32, 4 * T + 2 * sI + (lane >> 5), lane);
-      else return col_frag<D>(sV, T * 32 + sI * 16, dt * 32, lane);
     };
     if constexpr (DO_S) {
 #pragma unroll
@@ -687,21 +673,24 @@ __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(const uint16_t* __rest
 #pragma unroll
         for (int r = 0; r < 16; r++) s[T][r] = 0.f;
     }
-    bf16x8_t ring[DEPTH];
-#pragma unroll
-    for (int i = 0; i < DEPTH && i < NOP; i++) ring[i] = fetch(i);
+    attn_static_for<(DEPTH < NOP ? DEPTH : NOP)>([&](auto ic) __attribute__((always_inline)) { fetch(ic); });
     __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int i = 0; i < NOP; i++) {
-      if (i < NS) {
+    attn_static_for<NOP>([&](auto ic) __attribute__((always_inline)) {
+      constexpr int i = decltype(ic)::value;
+      if constexpr (i < NS) {
         s[i & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[i % DEPTH], qf[i >> 1], s[i & 1], 0, 0, 0);
       } else {
-        const int x = i - NS, dt = x % (D / 32), sI = (x / (D / 32)) & 1, T = x / (2 * (D / 32));
+        constexpr int x = i - NS, dt = x % (D / 32), sI = (x / (D / 32)) & 1, T = x / (2 * (D / 32));
+        // the reads of the fragments behind this one (all of them V fragments) may still be in flight
+        constexpr int AFTER = 2 * ((NOP - 1 - i) < (DEPTH - 1) ? (NOP - 1 - i) : (DEPTH - 1));
+        attn_tr_wait<AFTER>(tlo[i % DEPTH], thi[i % DEPTH]);
+        const u32x4_t w = {tlo[i % DEPTH][0], tlo[i % DEPTH][1], thi[i % DEPTH][0], thi[i % DEPTH][1]};
+        ring[i % DEPTH] = __builtin_bit_cast(bf16x8_t, w);
         acc_o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[i % DEPTH], pf[T][sI], acc_o[dt], 0, 0, 0);
       }
-      if (i + DEPTH < NOP) ring[i % DEPTH] = fetch(i + DEPTH);
+      if constexpr (i + DEPTH < NOP) fetch(std::integral_constant<int, i + DEPTH>{});
       __builtin_amdgcn_sched_barrier(0);
-    }
+    });
   };
   auto softmax = [&](int j) __attribute__((always_inline)) {
     const int key0 = j * BKV;
@@ -712,7 +701,7 @@ __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(const uint16_t* __rest
 #pragma unroll
         for (int r = 0; r < 16; r++) {
           const int mrow = acc_row(r, lane);
-          const int key = key0 + T * 32 + (VT ? perm_key(mrow) : mrow);
+          const int key = key0 + T * 32 + mrow;
           if ((causal && key > qrow) || key >= seq) s[T][r] = kNegBig;
         }
     }
@@ -756,7 +745,7 @@ __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(const uint16_t* __rest
     if (j < nt_w) softmax(j);                         // VALU phase
     phase_end();
     __builtin_amdgcn_s_setprio(1);                    // MFMA phase
-    if (j < nt_w) mfma_phase(std::true_type{}, std::true_type{}, SLOT);    // (its last scores are never used)
+    if (j < nt_w) mfma_phase(std::true_type{}, std::true_type{}, slot_c);    // (its last scores are never used)
     __builtin_amdgcn_s_setprio(0);
     // After the LDS reads of this phase: the compiler orders every LDS read behind all
     // outstanding direct-to-LDS loads, so loads issued earlier would be waited for here.
@@ -772,7 +761,7 @@ __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(const uint16_t* __rest
   phase_end();
   if (wave >= 4) phase_end();                         // second group runs one phase behind
   __builtin_amdgcn_s_setprio(1);
-  mfma_phase(std::true_type{}, std::false_type{}, 0);      // MFMA phase -1
+  mfma_phase(std::true_type{}, std::false_type{}, std::integral_constant<int, 0>{});      // MFMA phase -1
   __builtin_amdgcn_s_setprio(0);
   phase_end();
   for (int j = 0; j < nt; j += 3) {
@@ -1420,9 +1409,8 @@ static inline int rows_vec4(int dtype, int64_t head_dim, int64_t sb, int64_t sh,
 }
 
 extern "C" size_t emi_attn_fwd_workspace_bytes(int64_t batch, int64_t heads, int64_t seq, int64_t head_dim) {
-  if (batch <= 0 || heads <= 0 || seq <= 0 || (head_dim != 64 && head_dim != 128)) return 0;
-  const int64_t s_pad = (seq + 63) / 64 * 64;
-  return (size_t)batch * (size_t)heads * (size_t)head_dim * (size_t)s_pad * 2;     // V^T, bf16
+  (void)batch; (void)heads; (void)seq; (void)head_dim;
+  return 0;          // the forward kernels need no scratch (V is transposed by the LDS reads)
 }
 
 extern "C" int emi_attn_fwd_ws(emi_stream_t stream, const void* q, const void* k, const void* v, void* o, float* lse,
@@ -1433,6 +1421,7 @@ extern "C" int emi_attn_fwd_ws(emi_stream_t stream, const void* q, const void* k
   if (int rc = check_common("emi_attn_fwd", a, dtype)) return rc;
   if (batch == 0) return EMI_OK;
   EMI_REQUIRE(q && k && v && o && lse, "emi_attn_fwd: null buffer");
+  (void)workspace; (void)workspace_bytes;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const AttnShape shp{(int)seq, (int)heads, stride_b, stride_h, stride_s};
   const unsigned bh = (unsigned)(batch * heads);
@@ -1441,29 +1430,12 @@ extern "C" int emi_attn_fwd_ws(emi_stream_t stream, const void* q, const void* k
     const float sl2 = scale * kLog2e;
     if (seq >= 256) {
       const dim3 gridp((unsigned)((seq + 255) / 256), bh);
-      const int s_pad = (int)((seq + 63) / 64 * 64);
-      const size_t need = emi_attn_fwd_workspace_bytes(batch, heads, seq, head_dim);
-      // With a workspace V is transposed once (keys contiguous); without one the kernel
-      // falls back to transposing LDS reads of V.
-      const bool vt = workspace != nullptr && workspace_bytes >= need && aligned16(workspace) &&
-                      (int64_t)head_dim * s_pad * 2 < 0x7fffff00LL && bh <= 65535;
 #define EMI_ATTN_FWD_PP(DD)                                                                                          \
   do {                                                                                                               \
     constexpr int smem = 3 * 2 * 64 * DD * 2;                                                                        \
-    if (vt) {                                                                                                        \
-      hipLaunchKernelGGL(attn_vt_kernel<DD>, dim3((unsigned)(s_pad / 64), DD / 64, bh), dim3(256), 0, st,            \
-                         (const uint16_t*)v, (uint16_t*)workspace, shp, s_pad);                                      \
-      EMI_CHECK_LAUNCH("emi_attn_fwd(vt)");                                                                          \
-      if (int rc = reserve_lds(attn_fwd_pp_kernel<DD, true>, smem, "emi_attn_fwd")) return rc;                       \
-      hipLaunchKernelGGL((attn_fwd_pp_kernel<DD, true>), gridp, dim3(512), smem, st, (const uint16_t*)q,             \
-                         (const uint16_t*)k, (const uint16_t*)workspace, (uint16_t*)o, lse, shp, head_bytes, sl2,    \
-                         causal, s_pad);                                                                             \
-    } else {                                                                                                         \
-      if (int rc = reserve_lds(attn_fwd_pp_kernel<DD, false>, smem, "emi_attn_fwd")) return rc;                      \
-      hipLaunchKernelGGL((attn_fwd_pp_kernel<DD, false>), gridp, dim3(512), smem, st, (const uint16_t*)q,            \
-                         (const uint16_t*)k, (const uint16_t*)v, (uint16_t*)o, lse, shp, head_bytes, sl2, causal,    \
-                         s_pad);                                                                                     \
-    }                                                                                                                \
+    if (int rc = reserve_lds(attn_fwd_pp_kernel<DD>, smem, "emi_attn_fwd")) return rc;                               \
+    hipLaunchKernelGGL(attn_fwd_pp_kernel<DD>, gridp, dim3(512), smem, st, (const uint16_t*)q, (const uint16_t*)k,   \
+                       (const uint16_t*)v, (uint16_t*)o, lse, shp, head_bytes, sl2, causal);                         \
   } while (0)
       if (head_dim == 128) EMI_ATTN_FWD_PP(128);
       else EMI_ATTN_FWD_PP(64);

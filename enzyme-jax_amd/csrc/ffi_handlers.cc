@@ -300,16 +300,12 @@ extern "C" XLA_FFI_Error* emi_attn_fwd_ffi(XLA_FFI_CallFrame* cf) {
     return f.invalid("q, k, v, o must be rank 4 with one shape (q rank %lld)", q->rank);
   if (lse->dtype != XLA_FFI_DataType_F32 || lse->rank != 3 || lse->dims[0] != d.B || lse->dims[1] != d.H || lse->dims[2] != d.S)
     return f.invalid("lse must be f32[batch, heads, seq] = [%lld, %lld, %lld]", d.B, d.H, d.S);
-  // The optional workspace result holds the transposed copy of V; a buffer smaller than the query is an error,
-  // not a silent fall back to the slower path.
-  if (ws != nullptr) {
-    const size_t need = emi_attn_fwd_workspace_bytes(d.B, d.H, d.S, d.D);
-    if (byte_size(ws) < need) return f.invalid("workspace result has %lld bytes, %lld needed", (long long)byte_size(ws), (long long)need);
-  }
+  // An optional third result (scratch of earlier versions of this target) is accepted and left untouched.
+  (void)ws;
   EMI_FFI_STREAM()
   return f.from_status(emi_attn_fwd_ws(stream, q->data, k->data, v->data, o->data, static_cast<float*>(lse->data),
-                                       ws ? ws->data : nullptr, ws ? byte_size(ws) : 0, d.B, d.H, d.S, d.D, d.sb, d.sh, d.ss,
-                                       (float)scale, (int)causal, q->dtype));
+                                       nullptr, 0, d.B, d.H, d.S, d.D, d.sb, d.sh, d.ss, (float)scale, (int)causal,
+                                       q->dtype));
 }
 
 extern "C" XLA_FFI_Error* emi_attn_bwd_ffi(XLA_FFI_CallFrame* cf) {

@@ -136,10 +136,10 @@ int emi_attn_fwd(emi_stream_t stream, const void* q, const void* k, const void* 
                  int64_t stride_b, int64_t stride_h, int64_t stride_s, float scale, int causal,
                  int dtype);
 
-/* The same with a scratch buffer of emi_attn_fwd_workspace_bytes() bytes: the bf16
- * MFMA kernel then transposes V once so that the P.V product reads keys
- * contiguously (faster); a null or too small workspace selects the in-kernel
- * transposing reads.  Results are identical up to rounding of P. */
+/* The same with a scratch argument, kept for callers that pass one: the forward
+ * kernels need no scratch (V is transposed by the LDS reads inside the kernel; a
+ * separate V^T pass cost more than it saved), emi_attn_fwd_workspace_bytes() returns 0
+ * and `workspace` may be null. */
 size_t emi_attn_fwd_workspace_bytes(int64_t batch, int64_t heads, int64_t seq, int64_t head_dim);
 int emi_attn_fwd_ws(emi_stream_t stream, const void* q, const void* k, const void* v, void* o,
                     float* lse, void* workspace, size_t workspace_bytes, int64_t batch,

@@ -24,7 +24,7 @@
  *  emi_swiglu_bwd     a, b, dg                         da, db                            -
  *  emi_add            a, b                             y                                 -
  *  emi_gemm           A[.,.], B[.,.] [, R[M,N]]        C[M,N] [, workspace:u8[n]]        trans_a:pred, trans_b:pred
- *  emi_attn_fwd       q, k, v  (rank 4)                o, lse f32[B,h,S] [, workspace:u8[n]]  scale:f32, causal:pred, bshd:pred
+ *  emi_attn_fwd       q, k, v  (rank 4)                o, lse f32[B,h,S] [, unused:u8[n]]     scale:f32, causal:pred, bshd:pred
  *  emi_attn_bwd       q, k, v, o, lse, do              dq, dk, dv, workspace:u8[n]       scale:f32, causal:pred, bshd:pred
  *  emi_attn_step_fwd  q[B,h,d], k, v [B,S,h,d]         o[B,h,d], lse f32[B,h], workspace:u8[n]  scale:f32
  *  emi_attn_step_bwd  q, k, v, o, lse, do              dq, dk, dv, workspace:u8[n]       scale:f32

@@ -104,8 +104,6 @@ def test_ffi_metadata_probe_and_stages():
      {"scale": (F.F32, 0.1), "causal": (F.PRED, 1)}, "lse"),
     ("emi_attn_fwd_ffi", [(F.BF16, [1, 2, 64, 128])] * 3, [(F.BF16, [1, 2, 64, 128]), (F.F32, [1, 2, 64])],
      {"causal": (F.PRED, 1)}, "scale"),
-    ("emi_attn_fwd_ffi", [(F.BF16, [1, 2, 512, 128])] * 3, [(F.BF16, [1, 2, 512, 128]), (F.F32, [1, 2, 512]), (F.U8, [64])],
-     {"scale": (F.F32, 0.1), "causal": (F.PRED, 1)}, "workspace"),
     ("emi_attn_bwd_ffi", [(F.BF16, [1, 2, 64, 128])] * 4 + [(F.F32, [1, 2, 64]), (F.BF16, [1, 2, 64, 128])],
      [(F.BF16, [1, 2, 64, 128])] * 3 + [(F.U8, [8])], {"scale": (F.F32, 0.1)}, "workspace"),
     ("emi_attn_step_fwd_ffi", [(F.F32, [1, 6, 48]), (F.F32, [1, 9, 6, 48]), (F.F32, [1, 9, 6, 48])],
