@@ -372,6 +372,8 @@ def _parse_op(sc):
                 sc.fail("constant without a dense value")
             sub = _Scanner(text[m.end() - 1:])
             attrs = {"value": _dense(sub.balanced()[1:-1], types[0])}
+        elif short == "gather":
+            attrs = _gather_attrs(text)
         elif short in BINARY_OPS or short in UNARY_OPS or short in ("reshape", "convert"):
             pass
         else:
@@ -515,10 +517,41 @@ def _parse_op(sc):
     return Op(short, results, operands, attrs, types)
 
 
+def _gather_attrs(text):
+    """Attributes of a quoted `stablehlo.gather`; only the row lookup `table[indices]` an embedding traces to is
+    accepted (checked against the operand types by `check_gather`): whole rows of a rank-2 operand selected by one
+    index each."""
+    def ints(key):
+        m = re.search(key + r"\s*=\s*\[([^\]]*)\]", text)
+        return [int(v) for v in m.group(1).split(",") if v.strip()] if m else []
+    m = re.search(r"index_vector_dim\s*=\s*(\d+)", text)
+    ss = re.search(r"slice_sizes\s*=\s*(?:array<i64:\s*([^>]*)>|dense<\[([^\]]*)\]>)", text)
+    if m is None or ss is None:
+        raise ParseError("stablehlo.gather without index_vector_dim / slice_sizes")
+    return {"offset_dims": ints("offset_dims"), "collapsed_slice_dims": ints("collapsed_slice_dims"),
+            "operand_batching_dims": ints("operand_batching_dims"), "start_index_map": ints("start_index_map"),
+            "index_vector_dim": int(m.group(1)),
+            "slice_sizes": [int(v) for v in (ss.group(1) or ss.group(2)).split(",") if v.strip()]}
+
+
+def check_gather(attrs, table_t, idx_t, out_t):
+    """Raises NotImplementedError unless the gather is `table[indices]`: operand [V, D], indices [..., 1] (the index
+    vector last), one collapsed dimension 0, slices of one whole row, result [..., D]."""
+    lead = tuple(idx_t.shape[:-1])
+    ok = (len(table_t.shape) == 2 and len(idx_t.shape) >= 1 and idx_t.shape[-1] == 1
+          and attrs["index_vector_dim"] == len(idx_t.shape) - 1 and attrs["collapsed_slice_dims"] == [0]
+          and attrs["start_index_map"] == [0] and not attrs["operand_batching_dims"]
+          and attrs["offset_dims"] == [len(lead)] and attrs["slice_sizes"] == [1, table_t.shape[1]]
+          and tuple(out_t.shape) == lead + (table_t.shape[1],) and idx_t.dtype in ("i32", "i64"))
+    if not ok:
+        raise NotImplementedError("stablehlo.gather other than a row lookup table[indices] (operand %r, indices %r, %s)" %
+                                  (table_t, idx_t, attrs))
+
+
 def _parse_func(sc):
     for vis in ("public", "private", "nested"):
         sc.accept(vis)
-    name = sc.need(_SYM, "function name")[1:]
+    name = sc.need(_SYM, "function name")[1:].strip('"')
     sc.expect("(")
     args = []
     if not sc.accept(")"):
@@ -1363,6 +1396,13 @@ class Executable:
             return [H.slice_(xs[0], op.attrs["start"], op.attrs["limit"], op.attrs["stride"])]
         if n == "concatenate":
             return [H.concatenate(xs, op.attrs["dim"])]
+        if n == "gather":
+            names = {v: k for k, v in TORCH_DTYPES.items() if k != "ui32"}
+            check_gather(op.attrs, TensorType(xs[0].shape, names[xs[0].dtype]), TensorType(xs[1].shape, names[xs[1].dtype]),
+                         op.types[0])
+            if xs[1].dtype != torch.int32:
+                raise NotImplementedError("stablehlo.gather with %s indices (s32 wanted)" % xs[1].dtype)
+            return [ops.embedding(xs[1].reshape(xs[1].shape[:-1]), xs[0])]
         if n == "iota":
             raise NotImplementedError("stablehlo.iota of type %r (integer iotas feeding masks are folded at parse time)" % op.types[0])
         if n == "compare":
@@ -1536,6 +1576,20 @@ def _custom_call_impl(self, op, xs):
         N.check(lib.emi_attn_step_bwd(st, P(q), P(k), P(v), P(o), P(lse), P(do), P(dq), P(dk), P(dv), P(ws), nbytes, 1, h, S, d,
                                       h * d, d, S * h * d, d, h * d, float(cfg["scale"]), ops._code(q)))
         return [dq, dk, dv, None][:len(op.results)]
+    if target == "emi_embedding_fwd":
+        tok, table = _packed(xs[0]), _packed(xs[1])
+        return [ops.embedding(tok, table)]
+    if target == "emi_embedding_bwd":
+        tok, dx = _packed(xs[0]), _packed(xs[1])
+        V, D = op.types[0].shape
+        if tok.dtype != torch.int32 or tuple(dx.shape) != tuple(tok.shape) + (D,):
+            raise ValueError("custom call emi_embedding_bwd: tokens %s %s, dx %s, table [%d, %d]" %
+                             (tok.dtype, tuple(tok.shape), tuple(dx.shape), V, D))
+        dt = torch.empty((V, D), dtype=dx.dtype, device=dx.device)
+        nbytes = lib.emi_embedding_bwd_workspace_bytes(V, D, ops._code(dx))
+        ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=dx.device)
+        N.check(lib.emi_embedding_bwd(st, P(tok), P(dx), P(dt), P(ws), nbytes, tok.numel(), V, D, ops._code(dx)))
+        return [dt, None][:len(op.results)]
     raise NotImplementedError("custom call target '%s' is not one of this library's" % target)
 
 
@@ -1662,10 +1716,17 @@ class _Printer:
         elif n == "concatenate":
             self.emit("%s = stablehlo.concatenate %s, dim = %d : (%s) -> %r" % (r, ", ".join(op.operands), op.attrs["dim"],
                                                                                 ", ".join(repr(T[o]) for o in op.operands), ty))
+        elif n == "gather":
+            a = op.attrs
+            self.emit('%s = "stablehlo.gather"(%s, %s) <{dimension_numbers = #stablehlo.gather<offset_dims = %s, '
+                      'collapsed_slice_dims = %s, start_index_map = %s, index_vector_dim = %d>, indices_are_sorted = false, '
+                      'slice_sizes = array<i64: %s>}> : (%r, %r) -> %r' % (
+                          r, op.operands[0], op.operands[1], a["offset_dims"], a["collapsed_slice_dims"], a["start_index_map"],
+                          a["index_vector_dim"], ", ".join(str(v) for v in a["slice_sizes"]), T[op.operands[0]], T[op.operands[1]], ty))
         elif n == "call":
             lhs = r if len(op.results) == 1 else "%s:%d" % (op.results[0].split("#")[0], len(op.results))
             outs = repr(ty) if len(op.types) == 1 else "(" + ", ".join(repr(t) for t in op.types) + ")"
-            self.emit("%s = call @%s(%s) : (%s) -> %s" % (lhs, op.attrs["callee"], ", ".join(op.operands),
+            self.emit("%s = call @%s(%s) : (%s) -> %s" % (lhs, _sym(op.attrs["callee"]), ", ".join(op.operands),
                                                          ", ".join(repr(T[o]) for o in op.operands), outs))
         elif n == "custom_call":
             self.custom_call(op.results, op.attrs["target"], op.operands, op.attrs["config"], op.types)
@@ -1684,6 +1745,11 @@ class _Printer:
             raise NotImplementedError("cannot print operator '%s'" % n)
 
 
+def _sym(name):
+    """A symbol name as MLIR prints it: quoted unless it is a plain identifier."""
+    return name if re.fullmatch(r"[A-Za-z0-9_.$-]+", name) else '"%s"' % name
+
+
 def print_module(funcs):
     """StableHLO text of parsed (and possibly rewritten) functions; fused clusters are printed
     as `stablehlo.custom_call @emi_*` with `api_version = 4` and their scalars in
@@ -1698,7 +1764,7 @@ def print_module(funcs):
         for op in f.ops:
             p.op(op)
         rets = [o for op in f.ops if op.name == "return" for o in op.operands]
-        out.append("  func.func %s@%s(%s) -> (%s) {" % ("public " if f.name == "main" else "private ", f.name,
+        out.append("  func.func %s@%s(%s) -> (%s) {" % ("public " if f.name == "main" else "private ", _sym(f.name),
                                                       ", ".join("%s: %r" % (a, t) for a, t in f.args),
                                                       ", ".join(repr(p.types[o]) for o in rets)))
         out += p.lines

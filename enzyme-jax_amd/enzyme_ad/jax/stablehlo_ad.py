@@ -17,7 +17,7 @@ import re
 
 import numpy as np
 
-from .stablehlo import Func, Op, TensorType, _drop_dead
+from .stablehlo import Func, Op, TensorType, _drop_dead, check_gather
 
 FLOAT = ("f32", "bf16", "f16", "f64")
 
@@ -342,6 +342,12 @@ def reverse_function(func, name=None, arg_active=None, ret_active=None):
                 start[dim], limit[dim] = at, at + xt.shape[dim]
                 at += xt.shape[dim]
                 accum(x, b.emit("slice", [c], {"start": start, "limit": limit, "stride": [1] * len(start)}, xt))
+        elif n == "gather":
+            # the adjoint of the row lookup table[indices] is a scatter-add of the cotangent rows into a zero table
+            # (reference rule: HLODerivatives.td:1022-1046): the emi_embedding_bwd target; the indices are inactive
+            check_gather(op.attrs, T[xs[0]], T[xs[1]], T[r])
+            idx = b.emit("reshape", [xs[1]], {}, TensorType(T[xs[1]].shape[:-1], T[xs[1]].dtype))
+            accum(xs[0], b.emit("custom_call", [idx, c], {"target": "emi_embedding_bwd", "config": {}}, T[xs[0]]))
         elif n == "custom_call":
             _reverse_custom_call(b, op, cs, accum)
         elif n == "call":
@@ -493,6 +499,9 @@ def forward_function(func, name=None, arg_active=None):
                 tan[r] = b.emit("pad", [t, zero(TensorType((), T[r].dtype))], op.attrs, T[r])
         elif n == "concatenate":
             tan[r] = b.emit("concatenate", [tz(x) for x in xs], op.attrs, T[r])
+        elif n == "gather":
+            if ts[0] is not None:              # linear in the table; the indices carry no tangent
+                tan[r] = b.emit("gather", [ts[0], xs[1]], op.attrs, T[r])
         elif n == "dot_general":
             tan[r] = add(None if ts[0] is None else b.emit("dot_general", [ts[0], xs[1]], op.attrs, T[r]),
                          None if ts[1] is None else b.emit("dot_general", [xs[0], ts[1]], op.attrs, T[r]))

@@ -22,6 +22,8 @@ Pinning status:
       evaluated by hand on a vector, plus the adjoint identity.
   reshape ... pinned by a hand-worked row-major index case + adjoint identity.
   convert ... pinned by the result element type and its rounding.
+  gather (row lookup) ... pinned by a hand-worked case with a repeated index and the
+      adjoint identity against numpy indexing; its IR forms by gather.mlir's check lines.
   reduce(max) ... no numeric vector in the reference; pinned by the closed form
       stated in the C++ (cotangent to every element equal to the max) and by
       the softmax shift-invariance test (its contribution cancels).
@@ -188,6 +190,26 @@ def vjp_select(cond, a, b, d):
     """HLODerivatives.td:1297-1304 SelectOp."""
     z = np.zeros_like(d)
     return np.where(cond, d, z), np.where(cond, z, d)
+
+
+def gather_rows(table, indices):
+    """stablehlo.gather in the form an embedding lookup traces to (gather.mlir:4-7): indices [..., 1] select whole
+    rows of table [V, D]; out-of-range indices are clamped (the gather semantics)."""
+    idx = np.clip(np.asarray(indices)[..., 0], 0, table.shape[0] - 1)
+    return table[idx]
+
+
+def vjp_gather_rows(table, indices, d):
+    """HLODerivatives.td:1022-1046 GatherOp: scatter-add of the cotangent rows into a zero tensor shaped like the
+    operand (REVERSE check lines of gather.mlir: `stablehlo.scatter` with an add region on a zero constant, repeated
+    indices accumulate); the indices are inactive.  Updates whose index falls outside the operand are dropped (the
+    scatter semantics)."""
+    idx = np.asarray(indices)[..., 0].reshape(-1)
+    g = np.zeros_like(table)
+    rows = np.asarray(d).reshape(-1, table.shape[1])
+    live = (idx >= 0) & (idx < table.shape[0])
+    np.add.at(g, idx[live], rows[live])
+    return (g,)
 
 
 def vjp_matmul_nt(x, w, d):

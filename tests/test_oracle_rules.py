@@ -151,3 +151,20 @@ def test_convert_rule_returns_operand_type():
     w = np.array([2.0, 4.0], dtype=np.float64)
     (gt,) = R.vjp_convert(v, w)
     assert float(np.sum(v.astype(np.float64) * w)) == float(np.sum(v * gt))
+
+
+def test_gather_rows_rule_scatter_adds_repeated_indices():
+    """gather.mlir REVERSE check lines: the cotangent rows are scatter-added into a zero table, so an index that
+    occurs twice receives the sum of both rows and rows nobody looked up stay zero."""
+    table = np.arange(12.0).reshape(4, 3)
+    idx = np.array([[2], [0], [2]])
+    np.testing.assert_array_equal(R.gather_rows(table, idx), table[[2, 0, 2]])
+    d = np.array([[1.0, 2.0, 3.0], [10.0, 20.0, 30.0], [100.0, 200.0, 300.0]])
+    (g,) = R.vjp_gather_rows(table, idx, d)
+    np.testing.assert_array_equal(g, [[10.0, 20.0, 30.0], [0.0, 0.0, 0.0], [101.0, 202.0, 303.0], [0.0, 0.0, 0.0]])
+    rng = np.random.default_rng(5)
+    v = rng.standard_normal(table.shape)
+    assert np.isclose(np.sum(R.gather_rows(v, idx) * d), np.sum(v * g))     # <J v, w> = <v, J^T w>
+    # out of range: the lookup clamps, the scatter drops
+    np.testing.assert_array_equal(R.gather_rows(table, np.array([[7]])), table[[3]])
+    np.testing.assert_array_equal(R.vjp_gather_rows(table, np.array([[7]]), np.ones((1, 3)))[0], np.zeros((4, 3)))

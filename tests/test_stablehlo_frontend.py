@@ -262,3 +262,76 @@ module @jit_f attributes {mhlo.num_partitions = 1 : i32, mhlo.num_replicas = 1 :
     funcs = S.parse_module(text)
     assert [o.name for o in funcs["main"].ops] == ["multiply", "call", "return"]
     assert [o.name for o in funcs["inner"].ops] == ["negate", "return"]
+
+
+# ---- the reference's own differentiation test inputs -------------------------------------------------------------
+
+import json
+import os
+
+LIT = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "lit_primal_functions.json")))
+
+# Files of test/lit_tests/diffrules/stablehlo/ whose operators are on the llama path or next to it: every primal
+# function in them must parse, print and parse again to the same operator list.
+LIT_IN_SCOPE = ["add", "atan2", "broadcastindim", "broadcastindim2", "cbrt", "checked_mul", "clamp", "cosine", "divide",
+                "dot_general_2", "dot_general_3", "dotgeneral_vectormode", "exponential", "exponential_minus_one",
+                "gather", "log", "log_plus_one", "logistic", "maximum", "minimum", "negate", "pad", "power", "reduce",
+                "reduceactivity", "rsqrt", "select", "sine", "sqrt", "subtract", "tanh", "transpose",
+                "transpose_elem_batch_autodiff"]
+# Files that hold a complex-valued variant next to the real one: the real functions must parse.
+LIT_REAL_PART = ["abs", "dot_general", "multiply"]
+
+
+@pytest.mark.parametrize("name", LIT_IN_SCOPE + LIT_REAL_PART)
+def test_reference_lit_inputs_parse_and_print_to_a_fixed_point(name):
+    from enzyme_ad.jax import stablehlo as H
+    fns = LIT[name + ".mlir"]
+    if name in LIT_REAL_PART:
+        fns = [f for f in fns if "complex<" not in f]
+    assert fns
+    for fn in fns:
+        m = H.parse_module("module {\n" + fn + "\n}")
+        (f,) = m.values()
+        assert f.ops and f.ops[-1].name == "return"
+        again = H.parse_module(H.print_module(m))
+        (g,) = again.values()
+        assert [(o.name, len(o.operands), [repr(t) for t in o.types]) for o in f.ops] == \
+               [(o.name, len(o.operands), [repr(t) for t in o.types]) for o in g.ops]
+
+
+def test_reference_lit_inputs_out_of_scope_fail_cleanly():
+    """Everything else in that directory (control flow, scatter, sort, convolution, FFT, complex numbers, dynamic
+    slices, batch norm, einsum) is outside the llama path: the parser must say so by name, not crash."""
+    from enzyme_ad.jax import stablehlo as H
+    seen = 0
+    for fname, fns in LIT.items():
+        if fname[:-5] in LIT_IN_SCOPE + LIT_REAL_PART:
+            continue
+        for fn in fns:
+            try:
+                H.parse_module("module {\n" + fn + "\n}")
+            except (NotImplementedError, H.ParseError) as e:
+                assert str(e)
+                seen += 1
+    assert seen >= 30
+
+
+def test_gather_rule_has_the_reference_ir_form():
+    """gather.mlir: FORWARD = gather of the tangent table with the primal indices, next to the primal gather;
+    REVERSE = one scatter-add of the cotangent rows into a zero table, here the emi_embedding_bwd target; the
+    indices get no cotangent."""
+    from enzyme_ad.jax import stablehlo as H, stablehlo_ad as AD
+    (fn,) = LIT["gather.mlir"]
+    f = H.parse_module("module {\n" + fn + "\n}")["main"]
+    fwd = AD.forward_function(f, arg_active=[True, False])
+    assert [o.name for o in fwd.ops] == ["gather", "gather", "return"]
+    assert fwd.ops[0].operands[1] == fwd.ops[1].operands[1] and fwd.ops[1].operands[0].startswith("%t_")
+    rev = AD.reverse_function(f, arg_active=[True, False])
+    assert [o.name for o in rev.ops] == ["reshape", "custom_call", "return"]
+    assert rev.ops[1].attrs["target"] == "emi_embedding_bwd" and repr(rev.result_types[0]) == "tensor<64x3xf32>"
+    text = H.print_module({"main": rev})
+    assert "@emi_embedding_bwd" in text and "api_version = 4" in text
+    with pytest.raises(NotImplementedError):          # a gather that is not a row lookup is refused by name
+        H.Executable  # noqa: B018  (the class exists)
+        bad = fn.replace("slice_sizes = array<i64: 1, 3>", "slice_sizes = array<i64: 1, 2>")
+        AD.reverse_function(H.parse_module("module {\n" + bad + "\n}")["main"], arg_active=[True, False])
