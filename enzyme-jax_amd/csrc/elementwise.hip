@@ -36,37 +36,39 @@ template <int TPR> __device__ __forceinline__ void row_reduce2(float& a, float& 
 template <typename T, int TPR, int NCH>
 __global__ __launch_bounds__(256) void rmsnorm_fwd_kernel(const T* __restrict__ x, const T* __restrict__ gamma,
                                                           T* __restrict__ y, int64_t rows, int dim, float eps) {
-  constexpr int RPB = 256 / TPR;
+  // NCH groups of 8 elements per thread, held as 16-byte pieces (8 bf16 or 4 floats): consecutive lanes cover
+  // consecutive 16 bytes, the access shape the streaming loads and stores want.
+  constexpr int RPB = 256 / TPR, N = Chunk<T>::N, NC = NCH * 8 / N;
   __shared__ float red[2][4][2];
   const int tir = threadIdx.x % TPR;
   const int rib = threadIdx.x / TPR;
   const int64_t row = (int64_t)blockIdx.x * RPB + rib;
   const bool active = row < rows;
-  const int nchunk = dim >> 3;
+  const int nchunk = dim / N;
   const T* xr = x + row * dim;
-  float v[NCH][8];
+  float v[NC][N];
   float ss = 0.f, dummy = 0.f;
 #pragma unroll
-  for (int j = 0; j < NCH; j++) {
+  for (int j = 0; j < NC; j++) {
     const int c = tir + j * TPR;
     if (active && c < nchunk) {
-      Vec8<T>::load(xr + c * 8, v[j]);
+      Chunk<T>::load(xr + c * N, v[j]);
 #pragma unroll
-      for (int e = 0; e < 8; e++) ss += v[j][e] * v[j][e];
+      for (int e = 0; e < N; e++) ss += v[j][e] * v[j][e];
     }
   }
   row_reduce2<TPR>(ss, dummy, red, 0);
   const float r = 1.0f / sqrtf(ss / (float)dim + eps);
   T* yr = y + row * dim;
 #pragma unroll
-  for (int j = 0; j < NCH; j++) {
+  for (int j = 0; j < NC; j++) {
     const int c = tir + j * TPR;
     if (active && c < nchunk) {
-      float g[8], o[8];
-      Vec8<T>::load(gamma + c * 8, g);
+      float g[N], o[N];
+      ChunkCached<T>::load(gamma + c * N, g);
 #pragma unroll
-      for (int e = 0; e < 8; e++) o[e] = g[e] * v[j][e] * r;
-      Vec8<T>::store(yr + c * 8, o);
+      for (int e = 0; e < N; e++) o[e] = g[e] * v[j][e] * r;
+      Chunk<T>::store(yr + c * N, o);
     }
   }
 }
@@ -324,14 +326,14 @@ __global__ __launch_bounds__(256) void rope_kernel(const T* x, const float2* __r
   const float cs[4] = {t0.x, t0.z, t1.x, t1.z};
   float sn[4] = {t0.y, t0.w, t1.y, t1.w};
   float v[8], o[8];
-  Vec8<T>::load(x + e, v);
+  Vec8<T>::load_cached(x + e, v);              // (streaming accesses measured slower here)
 #pragma unroll
   for (int p = 0; p < 4; p++) {
     const float sp = inverse ? -sn[p] : sn[p];
     o[2 * p] = cs[p] * v[2 * p] - sp * v[2 * p + 1];
     o[2 * p + 1] = sp * v[2 * p] + cs[p] * v[2 * p + 1];
   }
-  Vec8<T>::store(y + e, o);
+  Vec8<T>::store_cached(y + e, o);
 }
 
 template <typename T>

@@ -18,7 +18,7 @@ namespace {
 template <typename T, int MT>
 __global__ __launch_bounds__(256) void gemv_nt_kernel(const T* __restrict__ A, const T* __restrict__ B, const T* R, T* C, int M,
                                                       int N, int K, int64_t lda, int64_t ldb, int64_t ldr, int64_t ldc) {
-  constexpr int V = Chunk<T>::N;
+  constexpr int V = ChunkCached<T>::N;
   const int lane = threadIdx.x & 63;
   const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (n >= N) return;
@@ -28,23 +28,23 @@ __global__ __launch_bounds__(256) void gemv_nt_kernel(const T* __restrict__ A, c
   for (int m = 0; m < MT; m++) acc[m] = 0.f;
   constexpr int UN = 8;                      // 16-byte loads of the row in flight per lane
   for (int k0 = lane * V; k0 < K; k0 += 64 * V * UN) {
-    typename Chunk<T>::Raw raw[UN];
+    typename ChunkCached<T>::Raw raw[UN];
 #pragma unroll
     for (int u = 0; u < UN; u++) {
       const int k = k0 + u * 64 * V;
-      if (k < K) raw[u] = Chunk<T>::load_raw(brow + k);
+      if (k < K) raw[u] = ChunkCached<T>::load_raw(brow + k);
     }
 #pragma unroll
     for (int u = 0; u < UN; u++) {
       const int k = k0 + u * 64 * V;
       if (k < K) {
         float b[V];
-        Chunk<T>::unpack(raw[u], b);
+        ChunkCached<T>::unpack(raw[u], b);
 #pragma unroll
         for (int m = 0; m < MT; m++) {
           if (m < M) {
             float a[V];
-            Chunk<T>::load(A + (int64_t)m * lda + k, a);
+            ChunkCached<T>::load(A + (int64_t)m * lda + k, a);
 #pragma unroll
             for (int e = 0; e < V; e++) acc[m] = fmaf(a[e], b[e], acc[m]);
           }
@@ -73,7 +73,7 @@ __global__ __launch_bounds__(256) void gemv_nt_kernel(const T* __restrict__ A, c
 template <typename T, int MT>
 __global__ __launch_bounds__(1024) void gemv_nn_kernel(const T* __restrict__ A, const T* __restrict__ B, const T* R, T* C, int M,
                                                        int N, int K, int64_t lda, int64_t ldb, int64_t ldr, int64_t ldc) {
-  constexpr int V = Chunk<T>::N, UN = MT * V > 32 ? 4 : 8, ROWS = 128;
+  constexpr int V = ChunkCached<T>::N, UN = MT * V > 32 ? 4 : 8, ROWS = 128;
   __shared__ float part[16][MT][8 * V];
   const int cl = threadIdx.x & 7, rl = threadIdx.x >> 3;           // chunk lane, row lane (0..127)
   const int n = (blockIdx.x * 8 + cl) * V;
@@ -88,7 +88,7 @@ __global__ __launch_bounds__(1024) void gemv_nn_kernel(const T* __restrict__ A, 
 #pragma unroll
       for (int u = 0; u < UN; u++) {
         const int k = k0 + u * ROWS;
-        if (k < K) Chunk<T>::load(B + (int64_t)k * ldb + n, b[u]);
+        if (k < K) ChunkCached<T>::load(B + (int64_t)k * ldb + n, b[u]);
       }
 #pragma unroll
       for (int u = 0; u < UN; u++) {
@@ -139,7 +139,7 @@ template <typename T, int MT>
 __global__ __launch_bounds__(256) void gemv_nn_bands_kernel(const T* __restrict__ A, const T* __restrict__ B,
                                                             float* __restrict__ part, int M, int N, int K, int64_t lda,
                                                             int64_t ldb, int rows_per_band) {
-  constexpr int V = Chunk<T>::N, UN = 16, AR = 256;
+  constexpr int V = ChunkCached<T>::N, UN = 16, AR = 256;
   __shared__ float sa[MT][AR];                                    // A values of the rows being processed
   const int n = (blockIdx.x * 256 + threadIdx.x) * V;
   const int k_begin = blockIdx.y * rows_per_band;
@@ -159,15 +159,15 @@ __global__ __launch_bounds__(256) void gemv_nn_bands_kernel(const T* __restrict_
     const int kce = kc + AR < k_end ? kc + AR : k_end;
     if (live) {
       for (int k0 = kc; k0 < kce; k0 += UN) {
-        typename Chunk<T>::Raw b[UN];
+        typename ChunkCached<T>::Raw b[UN];
 #pragma unroll
         for (int u = 0; u < UN; u++)
-          if (k0 + u < kce) b[u] = Chunk<T>::load_raw(B + (int64_t)(k0 + u) * ldb + n);
+          if (k0 + u < kce) b[u] = ChunkCached<T>::load_raw(B + (int64_t)(k0 + u) * ldb + n);
 #pragma unroll
         for (int u = 0; u < UN; u++)
           if (k0 + u < kce) {
             float bf[V];
-            Chunk<T>::unpack(b[u], bf);
+            ChunkCached<T>::unpack(b[u], bf);
 #pragma unroll
             for (int m = 0; m < MT; m++)
               if (m < M) {
@@ -235,13 +235,13 @@ int nn_bands(int64_t N, int64_t K, int V) {
 template <typename T>
 __global__ __launch_bounds__(256) void outer_tn_kernel(const T* __restrict__ A, const T* __restrict__ B, const T* R, T* C, int M,
                                                        int N, int K, int64_t lda, int64_t ldb, int64_t ldr, int64_t ldc) {
-  constexpr int V = Chunk<T>::N;
+  constexpr int V = ChunkCached<T>::N;
   const int chunks = N / V;
   const int64_t total = (int64_t)M * chunks;
   for (int64_t i = blockIdx.x * (int64_t)256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
     const int m = (int)(i / chunks), n = (int)(i % chunks) * V;
     float acc[V];
-    if (R != nullptr) Chunk<T>::load(R + (int64_t)m * ldr + n, acc);
+    if (R != nullptr) ChunkCached<T>::load(R + (int64_t)m * ldr + n, acc);
     else {
 #pragma unroll
       for (int e = 0; e < V; e++) acc[e] = 0.f;
@@ -249,11 +249,11 @@ __global__ __launch_bounds__(256) void outer_tn_kernel(const T* __restrict__ A, 
     for (int k = 0; k < K; k++) {
       const float a = to_f32(A[(int64_t)k * lda + m]);
       float b[V];
-      Chunk<T>::load(B + (int64_t)k * ldb + n, b);
+      ChunkCached<T>::load(B + (int64_t)k * ldb + n, b);
 #pragma unroll
       for (int e = 0; e < V; e++) acc[e] = fmaf(a, b[e], acc[e]);
     }
-    Chunk<T>::store(C + (int64_t)m * ldc + n, acc);
+    ChunkCached<T>::store(C + (int64_t)m * ldc + n, acc);
   }
 }
 
@@ -263,7 +263,7 @@ template <typename T>
 int launch_skinny_t(hipStream_t st, const void* A_, const void* B_, const void* R_, void* C_, void* workspace,
                     size_t workspace_bytes, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldr, int64_t ldc,
                     int trans_a, int trans_b) {
-  constexpr int V = Chunk<T>::N;
+  constexpr int V = ChunkCached<T>::N;
   const T* A = static_cast<const T*>(A_);
   const T* B = static_cast<const T*>(B_);
   const T* R = static_cast<const T*>(R_);
