@@ -356,7 +356,7 @@ def bench_frontend(iters):
     return out
 
 
-def bench_models(iters):
+def bench_models(iters, only=None):
     """The two whole-model configurations: tokens in, logits out, fwd + VJP with a cotangent on the
     logits (and, as `loss_*`, tokens in, mean cross-entropy out, fwd + VJP).  C4 stories110M (dim 768, hidden 2048, 12 layers, 12 heads x 64, vocab 32000, seq 1024,
     batch 8, bf16) and C1 stories15M (dim 288, hidden 768, 6 layers, 6 heads x 48, seq 256, batch 1,
@@ -368,6 +368,8 @@ def bench_models(iters):
                                                             vocab_size=32000, seq_len=1024), 8, 1024, torch.bfloat16),
                                 ("c1_stories15m_f32", dict(dim=288, hidden_dim=768, n_layers=6, n_heads=6, n_kv_heads=6,
                                                           vocab_size=32000, seq_len=256), 1, 256, torch.float32)):
+        if only is not None and not name.startswith(only):
+            continue
         g = torch.Generator(device="cuda").manual_seed(4)
         L_, D, H, V = cfg["n_layers"], cfg["dim"], cfg["hidden_dim"], cfg["vocab_size"]
         n = lambda *shape: (torch.randn(shape, generator=g, device="cuda") * 0.02).to(dt)
@@ -387,6 +389,8 @@ def bench_models(iters):
 
         t = event_time(step, iters, warmup=2)
         out[name] = dict(ms_per_step=round(t * 1e3, 3), tokens_per_s=round(B * S / t, 1), tokens_per_step=B * S)
+        if only is not None:            # profiling run: the logits step alone
+            continue
         # the same model as a training step: mean cross-entropy against random targets, all weight gradients
         tgt = torch.randint(0, V, (B, S), generator=g, device="cuda", dtype=torch.int32)
         one = torch.ones((), device="cuda")
@@ -521,15 +525,20 @@ def main():
     ap.add_argument("--calibrate", action="store_true",
                     help="also run one emi_add over 3 x 512 MiB (reads 1 GiB, writes 512 MiB): the known-size kernel "
                          "that FETCH_SIZE / WRITE_SIZE counter runs are scaled by")
+    ap.add_argument("--only-model", choices=["c1", "c4"], default=None,
+                    help="run only the fwd + VJP steps of one whole-model configuration (c1 = stories15M fp32, c4 = "
+                         "stories110M bf16) and print its timing: the command kernel traces of those models are taken from")
     ap.add_argument("--seq", type=int, default=C5["seq"])
     ap.add_argument("--batch", type=int, default=C5["batch"])
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (the path shards by batch; no multi-GPU code here); use --gpus 1")
-
     import torch
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible; the HIP path has no CPU fallback")
+    if args.only_model:
+        print(json.dumps({"whole_models": bench_models(max(args.steps, 5), only=args.only_model)}))
+        return
     from enzyme_ad.jax import enzyme_jax_ir, JaXPipeline, vjp, llama
 
     if args.calibrate:

@@ -523,8 +523,9 @@ static inline void rms_bwd_shape(int64_t rows, int64_t dim, int* tpr, int* nch, 
     const int rpb = 256 / *tpr;
     const int64_t groups = (rows + rpb - 1) / rpb;
     // Two resident blocks per CU: more blocks add partial rows (written here, read
-    // again by the column sum) without adding bandwidth.
-    const int64_t cap = (*tpr == 64) ? 128 : 512;
+    // again by the column sum) without adding bandwidth.  (Narrow rows, four per block: the same 512 blocks;
+    // 128 left half of the CUs idle on the 768-wide model.)
+    const int64_t cap = 512;
     *grid = groups < cap ? (groups > 0 ? groups : 1) : cap;
     *nparts = *grid * rpb;
   } else {
