@@ -16,7 +16,7 @@ LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libemi_hip.so")
 OBJDIR = os.path.join(LIBDIR, "obj")
 
-HIP_SOURCES = ["elementwise.hip", "gemm.hip", "gemm_skinny.hip", "attention.hip", "attention_step.hip", "forward_mode.hip",
+HIP_SOURCES = ["elementwise.hip", "gemm.hip", "gemm_skinny.hip", "attention.hip", "attention_f32.hip", "attention_step.hip", "forward_mode.hip",
                "tensor_ops.hip", "cross_entropy.hip"]
 CXX_SOURCES = ["status.cc", "ffi_handlers.cc"]
 

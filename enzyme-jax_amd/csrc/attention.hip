@@ -13,7 +13,8 @@
 // and produces dQ, another owns key blocks and produces dK and dV; both
 // recompute P from q, k and the saved log-sum-exp.
 //
-// Generic path (fp32 or any other head_dim <= 256): one wavefront per query
+// fp32 with head_dim a multiple of 16 (up to 128): attention_f32.hip, the same scheme on the fp32 matrix
+// instruction.  Generic path (any other head_dim <= 256 or unaligned rows): one wavefront per query
 // (or key) row, plain fp32 FMA, same maths.
 #include <initializer_list>
 #include <type_traits>
@@ -1393,6 +1394,14 @@ int launch_attn_jvp_mfma(hipStream_t st, const void* q, const void* k, const voi
   return EMI_OK;
 }
 
+// attention_f32.hip: the fp32 matrix-core kernels (head_dim a multiple of 16, 16-byte aligned rows); -1 = not applicable
+int launch_attn_fwd_f32_mfma(hipStream_t st, const void* q, const void* k, const void* v, void* o, float* lse, int64_t batch,
+                             int64_t heads, int64_t seq, int64_t head_dim, int64_t sb, int64_t shh, int64_t ss, float scale,
+                             int causal);
+int launch_attn_bwd_f32_mfma(hipStream_t st, const void* q, const void* k, const void* v, const void* d_o, const float* lse,
+                             const float* delta, void* dq, void* dk, void* dv, int64_t batch, int64_t heads, int64_t seq,
+                             int64_t head_dim, int64_t sb, int64_t shh, int64_t ss, float scale, int causal);
+
 }  // namespace emi
 
 using namespace emi;
@@ -1457,6 +1466,11 @@ extern "C" int emi_attn_fwd_ws(emi_stream_t stream, const void* q, const void* k
     }
     EMI_CHECK_LAUNCH("emi_attn_fwd");
     return EMI_OK;
+  }
+  if (dtype == EMI_F32) {
+    const int rc = launch_attn_fwd_f32_mfma(st, q, k, v, o, lse, batch, heads, seq, head_dim, stride_b, stride_h, stride_s,
+                                            scale, causal);
+    if (rc >= 0) return rc;
   }
   const dim3 grid((unsigned)((seq + 3) / 4), bh);
   const int vec4 = rows_vec4(dtype, head_dim, shp.sb, shp.sh, shp.ss, {q, k});
@@ -1538,6 +1552,11 @@ extern "C" int emi_attn_bwd(emi_stream_t stream, const void* q, const void* k, c
 #undef EMI_ATTN_BWD_LAUNCH
     EMI_CHECK_LAUNCH("emi_attn_bwd(dq)");
     return EMI_OK;
+  }
+  if (dtype == EMI_F32) {
+    const int rc = launch_attn_bwd_f32_mfma(st, q, k, v, d_o, lse, delta, dq, dk, dv, batch, heads, seq, head_dim, stride_b,
+                                            stride_h, stride_s, scale, causal);
+    if (rc >= 0) return rc;
   }
   const int vec4 = rows_vec4(dtype, head_dim, shp.sb, shp.sh, shp.ss, {q, k, v, d_o});
   if (dtype == EMI_BF16) {

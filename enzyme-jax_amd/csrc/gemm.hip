@@ -40,11 +40,14 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint3
 // (8 of them, each with its own L2), so give every XCD a contiguous run of
 // tiles, and walk tiles in groups of GROUP_M tile-rows so that the A and B
 // panels a XCD touches stay in its L2.
-__device__ __forceinline__ void tile_coords(int tiles_m, int tiles_n, int* tm, int* tn) {
+__device__ __forceinline__ int xcd_contiguous_id() {
   const int nb = gridDim.x, bid = blockIdx.x;
   const int per = nb >> 3, rem = nb & 7;
   const int xcd = bid & 7, idx = bid >> 3;
-  const int pid = xcd * per + (xcd < rem ? xcd : rem) + idx;
+  return xcd * per + (xcd < rem ? xcd : rem) + idx;
+}
+
+__device__ __forceinline__ void tile_coords(int pid, int tiles_m, int tiles_n, int* tm, int* tn) {
   constexpr int GROUP_M = 8;
   const int group_size = GROUP_M * tiles_n;
   const int group = pid / group_size;
@@ -261,7 +264,11 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_kernel(const uint16_t* 
 
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
   int tile_m, tile_n;
-  tile_coords(tiles_m, tiles_n, &tile_m, &tile_n);
+  // split-K: the grid is one run of tiles x splits blocks, split-major, so that the blocks of one XCD work on
+  // the same slab of K and that slab of A and B is fetched into one L2 rather than into all eight
+  const int pid = xcd_contiguous_id();
+  const int split = part ? pid / (tiles_m * tiles_n) : 0;
+  tile_coords(part ? pid - split * tiles_m * tiles_n : pid, tiles_m, tiles_n, &tile_m, &tile_n);
   const int m0 = tile_m * BM, n0 = tile_n * BN;
 
   const __amdgpu_buffer_rsrc_t rA = make_rsrc(A, a_bytes);
@@ -312,9 +319,9 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_kernel(const uint16_t* 
       for (int j = 0; j < TN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[j], a[i], acc[i][j], 0, 0, 0);
   };
 
-  // split-K (part != nullptr): block z owns k in [z * k_per_split, ...) and leaves an fp32 partial
+  // split-K (part != nullptr): split z owns k in [z * k_per_split, ...) and leaves an fp32 partial
   // tile in part[z][M][N]; gemm_splitk_reduce_kernel adds the partials (and R) in fixed order
-  const int k_lo = part ? blockIdx.z * k_per_split : 0;
+  const int k_lo = split * k_per_split;
   if (part) K = k_lo + k_per_split < K ? k_lo + k_per_split : K;
   const int nk = (K - k_lo + BK - 1) / BK;
   // Operand fragments are double buffered: the LDS reads of the next k-step are
@@ -366,7 +373,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_kernel(const uint16_t* 
   static_assert(NW * WR * WC * 2 <= NSTAGE * STAGE, "epilogue staging does not fit in the LDS allocation");
   if (part != nullptr) {
     // accumulator layout (swapped operands): register 4q+e of lane l holds row l%32, column 8q + 4(l/32) + e
-    float* pz = part + (int64_t)blockIdx.z * M * N;
+    float* pz = part + (int64_t)split * M * N;
     const bool vec4 = (N & 3) == 0;
 #pragma unroll
     for (int i = 0; i < TM; i++)
@@ -594,7 +601,7 @@ __global__ __launch_bounds__(512) void gemm_bf16_pingpong_kernel(const uint16_t*
 
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
   int tile_m, tile_n;
-  tile_coords(tiles_m, tiles_n, &tile_m, &tile_n);
+  tile_coords(xcd_contiguous_id(), tiles_m, tiles_n, &tile_m, &tile_n);
   const int m0 = tile_m * BM, n0 = tile_n * BN;
 
   const __amdgpu_buffer_rsrc_t rA = make_rsrc(A, a_bytes);
@@ -972,7 +979,7 @@ static int launch_bf16(hipStream_t st, const void* A, const void* B, const void*
   if (part != nullptr && splits > 1) {
     const int kps = (((K + splits - 1) / splits) + BK - 1) / BK * BK;
     const int nz = (K + kps - 1) / kps;
-    hipLaunchKernelGGL(kern, dim3(tiles, 1, nz), dim3(WM * WN * 64), smem, st, static_cast<const uint16_t*>(A),
+    hipLaunchKernelGGL(kern, dim3(tiles * nz), dim3(WM * WN * 64), smem, st, static_cast<const uint16_t*>(A),
                        static_cast<const uint16_t*>(B), static_cast<const uint16_t*>(R), static_cast<uint16_t*>(C), M, N, K,
                        lda, ldb, ldr, ldc, a_bytes, b_bytes, vec_ok, part, kps);
     EMI_CHECK_LAUNCH("emi_gemm(split-K)");

@@ -142,8 +142,13 @@ def test_matmul_nt_vjp(ops, dt):
 
 
 ATTN_CASES = [
-    ("f32", 2, 6, 100, 48, "bshd"),     # C1 head shape, generic path
-    ("f32", 1, 2, 64, 128, "bhsd"),
+    ("f32", 2, 6, 100, 48, "bshd"),     # C1 head shape, ragged sequence: fp32 matrix-core path
+    ("f32", 1, 6, 256, 48, "bshd"),     # C1 (stories15M) attention at its own size
+    ("f32", 1, 2, 64, 128, "bhsd"),     # fp32 matrix-core path, widest head
+    ("f32", 2, 3, 333, 64, "bhsd"),     # several 64-key steps, ragged
+    ("f32", 1, 1, 1, 16, "bhsd"),       # single position: out = v
+    ("f32", 1, 2, 77, 40, "bshd"),      # head_dim not a multiple of 16: generic path
+    ("f32", 2, 2, 50, 6, "bhsd"),       # generic path, rows not 16-byte aligned
     ("bf16", 1, 3, 70, 48, "bshd"),     # bf16 on the generic path
     ("bf16", 2, 2, 256, 128, "bhsd"),   # MFMA path
     ("bf16", 1, 2, 200, 128, "bshd"),   # MFMA, ragged sequence, token-major strides
@@ -212,6 +217,18 @@ def test_attention_forward_entry_points_agree(ops):
         check(o, ro, "bf16", "attention out")
         assert np.max(np.abs(lse - rlse)) < 2e-2
     assert np.array_equal(outs[0][0], outs[1][0]) and np.array_equal(outs[0][1], outs[1][1])
+
+
+def test_attention_lse_fp32_matrix_core_path(ops):
+    """The saved log-sum-exp of the fp32 kernels, ragged sequence (test/llama.py:13-18: max-subtracted softmax)."""
+    B, h, S, d = 2, 6, 201, 48
+    rng = np.random.default_rng(2)
+    (q, qr), (k, kr), (v, vr) = (dev(rng.standard_normal((B, h, S, d)), "f32") for _ in range(3))
+    for causal in (True, False):
+        o, lse, _ = ops.attention_raw(q, k, v, h, 1.0 / np.sqrt(d), causal, "bhsd")
+        ro, rlse = L.attention_fwd(qr, kr, vr, causal=causal)
+        assert np.max(np.abs(host(lse) - rlse)) < 1e-5
+        check(host(o), ro, "f32", "attention out")
 
 
 def test_attention_lse(ops):
