@@ -399,8 +399,9 @@ def matmul_nt(x, w, residual=None):
         # dX = dY . W: W is transposed first (2|W| bytes of HBM traffic, shared by nothing
         # else) so that the contraction index is innermost in both operands: the
         # k-contiguous kernel beats the k-major one by more than the transpose costs.
-        # With a handful of tokens (the single-token step) W is read in place, once.
-        if c2.shape[0] <= 8:
+        # With a handful of tokens (the single-token step) W is read in place, once; so it is in fp32, whose
+        # kernels read either layout at the same speed.
+        if c2.shape[0] <= 8 or c2.dtype == torch.float32:
             dx = gemm(c2, w, False, False, ax).reshape(x.shape)
         else:
             dx = gemm(c2, _transpose_shared(w), False, True, ax).reshape(x.shape)
