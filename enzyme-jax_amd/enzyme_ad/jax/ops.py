@@ -598,7 +598,7 @@ def embedding(tokens, table):
     return x
 
 
-def cross_entropy(logits, targets):
+def cross_entropy(logits, targets, return_lse=False):
     """Per-token softmax cross-entropy `logsumexp(z) - z[target]` of logits `[..., vocab]` against int32 targets
     `[...]`; the losses are fp32 whatever the logits' dtype.  The loss that follows the classifier commented out at
     test/llama.py:236.  Adjoint: `(softmax(z) - onehot) * dloss` from the saved logsumexp; a target outside
@@ -629,7 +629,7 @@ def cross_entropy(logits, targets):
         N.check(N.lib().emi_cross_entropy_jvp(_stream(), _p(logits), _p(targets), _p(lse), _p(tans[0]), _p(tl), T, V,
                                               _code(logits)))
         _set_tan(loss, tl)
-    return loss
+    return (loss, lse) if return_lse else loss
 
 
 def select(w, i):

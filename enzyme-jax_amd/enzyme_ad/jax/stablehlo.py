@@ -742,7 +742,8 @@ def _drop_dead(func):
     func.ops = list(reversed(kept))
 
 
-ALL_KINDS = ("rmsnorm", "swiglu", "rope", "softmax_dot", "attention_step", "rmsnorm_rows", "rope_rows", "attention", "linear")
+ALL_KINDS = ("rmsnorm", "swiglu", "rope", "softmax_dot", "attention_step", "rmsnorm_rows", "rope_rows", "attention", "cross_entropy",
+             "linear")
 
 
 def fuse_clusters(func, kinds=ALL_KINDS):
@@ -756,15 +757,18 @@ def fuse_clusters(func, kinds=ALL_KINDS):
       emi.softmax_dot  softmax(dot(K, q) / c) followed by the dot with V  (llama.py:13-18,193-204)
       emi.attention_step  the concatenation of emi.softmax_dot over consecutive head slices of
                    one query and one pair of caches (llama.py:178-209)
+      emi.cross_entropy  sum(onehot(targets) * log_softmax(logits)) over the vocabulary, the one-hot built at run
+                   time from integer targets (iota, compare EQ, convert or select): the loss after the classifier
+                   of llama.py:236
 
     A cluster is fused only when none of its interior values is used outside it.  Returns
     the number of clusters fused per kind."""
     counts = {"rmsnorm": 0, "swiglu": 0, "rope": 0, "softmax_dot": 0, "attention_step": 0, "rmsnorm_rows": 0, "rope_rows": 0,
-              "attention": 0, "linear": 0}
+              "attention": 0, "cross_entropy": 0, "linear": 0}
     matchers = [m for k, m in (("rmsnorm", _match_rmsnorm), ("swiglu", _match_swiglu), ("rope", _match_rope),
                                ("softmax_dot", _match_softmax_dot), ("attention_step", _match_heads),
                                ("rmsnorm_rows", _match_rmsnorm_rows), ("rope_rows", _match_rope_rows),
-                               ("attention", _match_attention)) if k in kinds]
+                               ("attention", _match_attention), ("cross_entropy", _match_cross_entropy)) if k in kinds]
     want_linear = "linear" in kinds
     changed = True
     while changed:
@@ -775,6 +779,11 @@ def fuse_clusters(func, kinds=ALL_KINDS):
 
         def d(name):
             return defs.get(name)
+
+        d.types = {a: t for a, t in func.args}            # for matchers that need the type of a function argument
+        for o_ in func.ops:
+            for r_, t_ in zip(o_.results, o_.types):
+                d.types[r_] = t_
 
         def through_broadcast(name):
             """The rank-0 value behind a broadcast_in_dim (or the name itself)."""
@@ -990,6 +999,137 @@ def _match_softmax_dot(op, d, tb):
         interior = [op, att, e, sbc, sm, sub, mbc, mx, s, sdot] + ([cbc] if cbc is not None else [])
         return ("softmax_dot", Op("emi.softmax_dot", op.results, [q, k, v], {"scale": scale}, op.types), interior)
     return None
+
+
+def _per_row_source(name, d, through=()):
+    """Follows `name`, a value of shape rows + (V,), back through the broadcast_in_dim / reshape operators that only
+    spread a per-row value along the last axis (shapes rows, rows + (1,), rows + (V,)) and through the unary
+    operators named in `through`.  Returns (source name, operators passed, unary names passed) or None."""
+    ty = d.types.get(name)
+    if ty is None or not ty.shape:
+        return None
+    rows = tuple(ty.shape[:-1])
+    passed, unary = [], []
+    while True:
+        op = d(name)
+        if op is None:
+            break
+        if op.name in through:
+            passed.append(op)
+            unary.append(op.name)
+            name = op.operands[0]
+            continue
+        if op.name not in ("broadcast_in_dim", "reshape"):
+            break
+        src = d.types.get(op.operands[0])
+        if src is None or tuple(src.shape) not in (rows, rows + (1,)):
+            break
+        if op.name == "broadcast_in_dim" and list(op.attrs["dims"]) != list(range(len(src.shape))):
+            break
+        passed.append(op)
+        name = op.operands[0]
+    if not passed or tuple(d.types[name].shape) not in (rows, rows + (1,)):
+        return None
+    return name, passed, unary
+
+
+def _is_class_index(name, d):
+    """True (with the operators passed) when `name` holds, at every position, its index along the last axis: an iota
+    over that axis, or the constant it folds to, possibly broadcast over the leading axes."""
+    ty = d.types.get(name)
+    passed = []
+    while True:
+        op = d(name)
+        if op is None or ty is None:
+            return None
+        V = ty.shape[-1]
+        if op.name == "iota":
+            return passed + [op] if op.attrs["dim"] == len(op.types[0].shape) - 1 and op.types[0].shape[-1] == V else None
+        if op.name == "constant":
+            v = np.asarray(op.attrs["value"])
+            if v.dtype.kind not in "iu" or v.shape[-1:] != (V,):
+                return None
+            return passed if np.array_equal(v.reshape(-1, V), np.broadcast_to(np.arange(V), (v.size // V, V))) else None
+        if op.name not in ("broadcast_in_dim", "reshape"):
+            return None
+        src = d.types.get(op.operands[0])
+        if src is None or not src.shape or src.shape[-1] != V or any(x != 1 for x in src.shape[:-1]):
+            return None
+        if op.name == "broadcast_in_dim":
+            dims = list(op.attrs["dims"])
+            if dims[-1] != len(op.types[0].shape) - 1:
+                return None
+        passed.append(op)
+        name = op.operands[0]
+
+
+def _match_cross_entropy(op, d, tb):
+    # root: reduce-add over the last axis of onehot * logp (either order) or select(eq, logp, 0), with
+    #   eq     = compare EQ of the targets spread along the last axis and the class index along it
+    #   onehot = convert(eq)
+    #   logp   = shifted - spread(log(reduce-add(exp(shifted)))),  shifted = logits - spread(reduce-max(logits))
+    # (jax.nn.log_softmax and jax.nn.one_hot).  The root equals minus the per-row cross-entropy; a target outside
+    # [0, V) matches no class and gives 0, as the kernel does.
+    if op.name != "reduce" or op.attrs["body"] != "add" or _splat(d(op.operands[1])) != 0.0:
+        return None
+    prod = d(op.operands[0])
+    if prod is None or not prod.types[0].shape or list(op.attrs["dims"]) != [len(prod.types[0].shape) - 1]:
+        return None
+    interior = [op, prod]
+    if prod.name == "multiply":
+        for oi in (0, 1):
+            cv = d(prod.operands[oi])
+            if cv is not None and cv.name == "convert" and d(cv.operands[0]) is not None and d(cv.operands[0]).name == "compare":
+                eq, logp_name = d(cv.operands[0]), prod.operands[1 - oi]
+                interior.append(cv)
+                break
+        else:
+            return None
+    elif prod.name == "select":
+        eq, logp_name = d(prod.operands[0]), prod.operands[1]
+        if eq is None or eq.name != "compare" or _splat(d(prod.operands[2])) != 0.0:
+            return None
+    else:
+        return None
+    if eq.attrs["direction"] != "EQ":
+        return None
+    interior.append(eq)
+    targets = None
+    for ti in (0, 1):
+        src = _per_row_source(eq.operands[ti], d)
+        idx = _is_class_index(eq.operands[1 - ti], d)
+        if src is not None and idx is not None and d.types[src[0]].dtype == "i32":
+            targets = src[0]
+            interior += src[1] + idx
+            break
+    if targets is None:
+        return None
+    logp = d(logp_name)
+    if logp is None or logp.name != "subtract":
+        return None
+    shifted = d(logp.operands[0])
+    norm = _per_row_source(logp.operands[1], d, through=("log",))
+    if shifted is None or shifted.name != "subtract" or norm is None or norm[2] != ["log"]:
+        return None
+    sm = d(norm[0])
+    if sm is None or sm.name != "reduce" or sm.attrs["body"] != "add" or _splat(d(sm.operands[1])) != 0.0:
+        return None
+    ex = d(sm.operands[0])
+    rank = len(shifted.types[0].shape)
+    if ex is None or ex.name != "exponential" or ex.operands[0] != logp.operands[0] or list(sm.attrs["dims"]) != [rank - 1]:
+        return None
+    logits = shifted.operands[0]
+    top = _per_row_source(shifted.operands[1], d)
+    if top is None:
+        return None
+    mx = d(top[0])
+    if mx is None or mx.name != "reduce" or mx.attrs["body"] != "maximum" or mx.operands[0] != logits or \
+            list(mx.attrs["dims"]) != [rank - 1] or _splat(d(mx.operands[1])) != -math.inf:
+        return None
+    if d.types[logits].dtype not in ("f32", "bf16"):
+        return None
+    interior += [logp, shifted, sm, ex, mx] + norm[1] + top[1]
+    return ("cross_entropy", Op("emi.cross_entropy", op.results, [logits, targets], {"negated": True}, op.types), interior)
 
 
 def _bcast(name, d, dims=None):
@@ -1435,6 +1575,15 @@ class Executable:
         if n == "emi.attention":
             q, k, v = (_packed(t) for t in xs)
             return [ops.attention(q, k, v, op.attrs["heads"], op.attrs["scale"], causal=op.attrs["causal"], layout="bshd")]
+        if n == "emi.cross_entropy":
+            z = _packed(xs[0])
+            loss = ops.cross_entropy(z, xs[1].reshape(z.shape[:-1]).contiguous())          # fp32 per-row losses
+            if op.attrs.get("negated"):
+                loss = H.unary("negate", loss)
+            dt = TORCH_DTYPES[op.types[0].dtype]
+            if loss.dtype != dt:
+                loss = H.convert(loss, dt)
+            return [ops.reshape(loss, op.types[0].shape)]
         if n == "emi.rmsnorm":
             x, w = _packed(xs[0]), _packed(xs[1])
             return [ops.reshape(ops.rmsnorm(ops.reshape(x, (1, x.shape[0])), w, op.attrs["eps"]), tuple(x.shape))]
@@ -1576,6 +1725,27 @@ def _custom_call_impl(self, op, xs):
         N.check(lib.emi_attn_step_bwd(st, P(q), P(k), P(v), P(o), P(lse), P(do), P(dq), P(dk), P(dv), P(ws), nbytes, 1, h, S, d,
                                       h * d, d, S * h * d, d, h * d, float(cfg["scale"]), ops._code(q)))
         return [dq, dk, dv, None][:len(op.results)]
+    if target == "emi_cross_entropy_fwd":
+        z, t = _packed(xs[0]), xs[1].contiguous()
+        loss, lse = ops.cross_entropy(z, t, return_lse=True)
+        return [loss, lse][:len(op.results)]
+    if target in ("emi_cross_entropy_bwd", "emi_cross_entropy_jvp"):
+        z, t, lse, w = (_packed(x) for x in xs)
+        rows, V = z.numel() // z.shape[-1], z.shape[-1]
+        if t.dtype != torch.int32 or lse.dtype != torch.float32 or t.numel() != rows or lse.numel() != rows:
+            raise ValueError("custom call %s: logits %s, targets %s %s, lse %s %s" %
+                             (target, tuple(z.shape), t.dtype, tuple(t.shape), lse.dtype, tuple(lse.shape)))
+        if target == "emi_cross_entropy_bwd":
+            if w.dtype != torch.float32 or w.numel() != rows:
+                raise ValueError("custom call emi_cross_entropy_bwd: the cotangent of the losses must be f32[%d]" % rows)
+            dz = torch.empty_like(z)
+            N.check(lib.emi_cross_entropy_bwd(st, P(z), P(t), P(lse), P(w), P(dz), rows, V, ops._code(z)))
+            return [dz]
+        if w.dtype != z.dtype or tuple(w.shape) != tuple(z.shape):
+            raise ValueError("custom call emi_cross_entropy_jvp: the tangent must have the logits' type")
+        tl = torch.empty(t.shape, dtype=torch.float32, device=z.device)
+        N.check(lib.emi_cross_entropy_jvp(st, P(z), P(t), P(lse), P(w), P(tl), rows, V, ops._code(z)))
+        return [tl]
     if target == "emi_embedding_fwd":
         tok, table = _packed(xs[0]), _packed(xs[1])
         return [ops.embedding(tok, table)]

@@ -126,6 +126,17 @@ def lower_fused(func):
             o4, _ = b.custom_call("emi_attn_fwd", [q4, k4, v4], {"scale": op.attrs["scale"], "causal": bool(op.attrs["causal"]), "bshd": True},
                                   [T[q4], TensorType((B_, h, S_), "f32")])
             b.ops.append(Op("reshape", op.results, [o4], {}, op.types))
+        elif n == "emi.cross_entropy":
+            z, t = op.operands
+            V = T[z].shape[-1]
+            rows = int(np.prod(T[z].shape[:-1])) if len(T[z].shape) > 1 else 1
+            loss, _ = b.custom_call("emi_cross_entropy_fwd", [b.reshape(z, (rows, V)), b.reshape(t, (rows,))], {},
+                                    [TensorType((rows,), "f32"), TensorType((rows,), "f32")])
+            if op.attrs.get("negated"):
+                loss = b.emit("negate", [loss], {}, T[loss])
+            if ty.dtype != "f32":
+                loss = b.emit("convert", [loss], {}, TensorType((rows,), ty.dtype))
+            b.ops.append(Op("reshape", op.results, [loss], {}, op.types))
         elif n in ("emi.softmax_dot", "emi.attention_step"):
             q, k, v = op.operands
             h = op.attrs.get("heads", 1)
@@ -530,6 +541,10 @@ def forward_function(func, name=None, arg_active=None):
                 tan[o], = b.custom_call("emi_attn_jvp", [xs[0], xs[1], xs[2], lse, tz(xs[0]), tz(xs[1]), tz(xs[2])],
                                         {"scale": cfg["scale"], "causal": bool(cfg.get("causal", True)), "bshd": bool(cfg.get("bshd", False))},
                                         [T[o]])
+            elif target == "emi_cross_entropy_fwd":
+                if ts[0] is not None:          # the targets carry no tangent
+                    loss, lse = op.results
+                    tan[loss], = b.custom_call("emi_cross_entropy_jvp", [xs[0], xs[1], lse, ts[0]], {}, [T[loss]])
             elif target == "emi_attn_step_fwd":
                 o, lse, ws = op.results
                 tan[o], _ = b.custom_call("emi_attn_step_jvp", [xs[0], xs[1], xs[2], o, lse, tz(xs[0]), tz(xs[1]), tz(xs[2])],
@@ -643,6 +658,15 @@ def _reverse_custom_call(b, op, cs, accum):
         accum(q, dq)
         accum(k, dk)
         accum(v, dv)
+    elif target == "emi_cross_entropy_fwd":
+        if len(cs) > 1 and cs[1] is not None:
+            raise NotImplementedError("cotangent of the log-sum-exp result of emi_cross_entropy_fwd")
+        if c is None:
+            return
+        z, t = xs
+        lse = op.results[1]
+        dz, = b.custom_call("emi_cross_entropy_bwd", [z, t, lse, c], {}, [T[z]])       # the targets are inactive
+        accum(z, dz)
     else:
         raise NotImplementedError("symbolic reverse mode of custom call '%s'" % target)
 

@@ -445,3 +445,43 @@ def test_gather_row_lookup_through_text_in_all_three_modes(dt):
     assert np.max(np.abs(host(rev[0]) - rg)) <= (1e-6 if dt == "f32" else 2e-2) * np.max(np.abs(rg))
     fwd = hlo_call(table, ttab, idx, source=stablehlo_ad.forward_module_text(text, arg_active=[True, False]))
     assert np.array_equal(host(fwd[0]), host(out)) and np.array_equal(host(fwd[1]), host(t))
+
+
+@pytest.mark.parametrize("dt,rows,V,select_form", [("f32", (64,), 1000, False), ("f32", (3, 21), 517, True), ("bf16", (40,), 4096, False)])
+def test_traced_cross_entropy_through_text_in_all_three_modes(dt, rows, V, select_form):
+    """A traced mean softmax cross-entropy (log_softmax, one-hot from run-time integer targets, sum, mean) run from
+    its text: the cluster is matched onto the cross-entropy kernels; value, gradient and tangent against the
+    oracle (logsumexp(z) - z[target], (softmax - onehot) / n, targets outside [0, V) contributing nothing), and the
+    symbolic reverse and forward programs through hlo_call against the same figures."""
+    from enzyme_ad.jax import hlo_call, jvp, stablehlo, stablehlo_ad, vjp
+    from oracle import llama_ref as L
+    from test_stablehlo_frontend import traced_cross_entropy_text
+    text = traced_cross_entropy_text(rows, V, dt=dt, select_form=select_form)
+    assert stablehlo.Executable(text).fused == {"cross_entropy": 1}
+    n = int(np.prod(rows))
+    rng = np.random.default_rng(23)
+    z, zr = dev(3.0 * rng.standard_normal(rows + (V,)), dt)
+    tz, tzr = dev(rng.standard_normal(rows + (V,)), dt)
+    tgt_np = rng.integers(0, V, size=rows).astype(np.int32)
+    tgt_np.reshape(-1)[1] = -1                       # masked rows: no class matches
+    tgt_np.reshape(-1)[5] = V
+    tgt = torch.from_numpy(tgt_np).cuda()
+    loss_rows, _ = L.cross_entropy_fwd(zr.reshape(n, V), tgt_np.reshape(n))
+    want = float(np.sum(loss_rows) / n)
+    tol = 1e-5 if dt == "f32" else 2e-2
+    fn = lambda a: hlo_call(a, tgt, source=text)[0]
+    out, f_vjp = vjp(fn, z)
+    assert abs(float(host(out)) - want) <= tol * abs(want)
+    one = torch.ones((), device="cuda", dtype=torch.float32 if dt == "f32" else torch.bfloat16)
+    (g,) = f_vjp(one)
+    rg = L.cross_entropy_bwd(zr.reshape(n, V), tgt_np.reshape(n), np.full(n, 1.0 / n)).reshape(rows + (V,))
+    assert np.max(np.abs(host(g) - rg)) <= (2e-6 if dt == "f32" else 2e-2) * np.max(np.abs(rg))
+    assert not host(g).reshape(n, V)[1].any() and not host(g).reshape(n, V)[5].any()
+    _, t = jvp(fn, (z,), (tz,))
+    rt = float(np.sum(L.cross_entropy_jvp(zr.reshape(n, V), tgt_np.reshape(n), tzr.reshape(n, V))) / n)
+    assert abs(float(host(t)) - rt) <= (1e-4 if dt == "f32" else 3e-2) * max(abs(rt), 0.05)
+    rev = hlo_call(z, tgt, one, source=stablehlo_ad.reverse_module_text(text))
+    assert np.max(np.abs(host(rev[0]) - rg)) <= (2e-6 if dt == "f32" else 2e-2) * np.max(np.abs(rg))
+    fwd = hlo_call(z, tz, tgt, source=stablehlo_ad.forward_module_text(text))
+    assert abs(float(host(fwd[0])) - want) <= tol * abs(want)
+    assert abs(float(host(fwd[1])) - rt) <= (1e-4 if dt == "f32" else 3e-2) * max(abs(rt), 0.05)

@@ -335,3 +335,101 @@ def test_gather_rule_has_the_reference_ir_form():
         H.Executable  # noqa: B018  (the class exists)
         bad = fn.replace("slice_sizes = array<i64: 1, 3>", "slice_sizes = array<i64: 1, 2>")
         AD.reverse_function(H.parse_module("module {\n" + bad + "\n}")["main"], arg_active=[True, False])
+
+
+# The mean softmax cross-entropy of integer targets in the form `jax.jit(f).lower(...).as_text()` prints for
+#   f = lambda z, t: -jnp.mean(jnp.sum(jax.nn.one_hot(t, V) * jax.nn.log_softmax(z), axis=-1))
+# (log_softmax: reduce max, subtract, exp, reduce add, log, subtract with keep-dims broadcasts; one_hot: targets
+# spread along a new last axis compared with an iota over it).  Written by hand to that form: no JAX here.
+def traced_cross_entropy_text(rows, V, dt="f32", select_form=False):
+    lead = "x".join(str(r) for r in rows)
+    R, n = len(rows), int(np.prod(rows))
+    full, keep, flat = "tensor<%sx%dx%s>" % (lead, V, dt), "tensor<%sx1x%s>" % (lead, dt), "tensor<%sx%s>" % (lead, dt)
+    ifull, ikeep, iflat = "tensor<%sx%dxi32>" % (lead, V), "tensor<%sx1xi32>" % lead, "tensor<%sxi32>" % lead
+    iota = "tensor<%sx%dxi32>" % ("x".join("1" for _ in rows), V)
+    d_flat, d_keep = list(range(R)), list(range(R + 1))
+    onehot = ("%%15 = stablehlo.convert %%14 : (%s) -> %s\n      %%16 = stablehlo.multiply %%15, %%9 : %s" %
+              (full.replace(dt + ">", "i1>"), full, full))
+    if select_form:
+        onehot = ("%%z = stablehlo.constant dense<0.000000e+00> : %s\n      %%16 = stablehlo.select %%14, %%9, %%z : %s, %s" %
+                  (full, full.replace(dt + ">", "i1>"), full))
+    return """
+module @jit_loss {
+  func.func public @main(%%arg0: %(full)s, %%arg1: %(iflat)s) -> (tensor<%(dt)s>) {
+      %%cst = stablehlo.constant dense<%(ninf)s> : tensor<%(dt)s>
+      %%0 = stablehlo.reduce(%%arg0 init: %%cst) applies stablehlo.maximum across dimensions = [%(R)d] : (%(full)s, tensor<%(dt)s>) -> %(flat)s
+      %%1 = stablehlo.broadcast_in_dim %%0, dims = %(d_flat)s : (%(flat)s) -> %(keep)s
+      %%2 = stablehlo.broadcast_in_dim %%1, dims = %(d_keep)s : (%(keep)s) -> %(full)s
+      %%3 = stablehlo.subtract %%arg0, %%2 : %(full)s
+      %%4 = stablehlo.exponential %%3 : %(full)s
+      %%cst_0 = stablehlo.constant dense<0.000000e+00> : tensor<%(dt)s>
+      %%5 = stablehlo.reduce(%%4 init: %%cst_0) applies stablehlo.add across dimensions = [%(R)d] : (%(full)s, tensor<%(dt)s>) -> %(flat)s
+      %%6 = stablehlo.broadcast_in_dim %%5, dims = %(d_flat)s : (%(flat)s) -> %(keep)s
+      %%7 = stablehlo.log %%6 : %(keep)s
+      %%8 = stablehlo.broadcast_in_dim %%7, dims = %(d_keep)s : (%(keep)s) -> %(full)s
+      %%9 = stablehlo.subtract %%3, %%8 : %(full)s
+      %%10 = stablehlo.broadcast_in_dim %%arg1, dims = %(d_flat)s : (%(iflat)s) -> %(ikeep)s
+      %%11 = stablehlo.iota dim = %(R)d : %(iota)s
+      %%12 = stablehlo.broadcast_in_dim %%10, dims = %(d_keep)s : (%(ikeep)s) -> %(ifull)s
+      %%13 = stablehlo.broadcast_in_dim %%11, dims = %(d_keep)s : (%(iota)s) -> %(ifull)s
+      %%14 = stablehlo.compare  EQ, %%12, %%13,  SIGNED : (%(ifull)s, %(ifull)s) -> %(mask)s
+      %(onehot)s
+      %%17 = stablehlo.reduce(%%16 init: %%cst_0) applies stablehlo.add across dimensions = [%(R)d] : (%(full)s, tensor<%(dt)s>) -> %(flat)s
+      %%18 = stablehlo.reduce(%%17 init: %%cst_0) applies stablehlo.add across dimensions = %(d_flat)s : (%(flat)s, tensor<%(dt)s>) -> tensor<%(dt)s>
+      %%cst_1 = stablehlo.constant dense<%(n)d.0> : tensor<%(dt)s>
+      %%19 = stablehlo.divide %%18, %%cst_1 : tensor<%(dt)s>
+      %%20 = stablehlo.negate %%19 : tensor<%(dt)s>
+      return %%20 : tensor<%(dt)s>
+  }
+}""" % dict(full=full, keep=keep, flat=flat, ifull=ifull, ikeep=ikeep, iflat=iflat, iota=iota, d_flat=d_flat, d_keep=d_keep, R=R,
+           dt=dt, n=n, onehot=onehot, mask=full.replace(dt + ">", "i1>"), ninf="0xFF800000" if dt == "f32" else "0xFF80")
+
+
+@pytest.mark.parametrize("rows,select_form", [((8,), False), ((2, 5), False), ((8,), True)])
+def test_traced_cross_entropy_is_matched_and_lowered(rows, select_form):
+    """The whole softmax / one-hot cluster becomes one emi.cross_entropy (printed as emi_cross_entropy_fwd); what is
+    left is the mean.  Reverse mode calls emi_cross_entropy_bwd on the saved log-sum-exp with the targets inactive,
+    forward mode emi_cross_entropy_jvp."""
+    import enzyme_ad.jax as ej
+    from enzyme_ad.jax import stablehlo as S
+    from enzyme_ad.jax import stablehlo_ad as AD
+    text = traced_cross_entropy_text(rows, 16, select_form=select_form)
+    exe = S.Executable(text)
+    assert exe.fused == {"cross_entropy": 1}
+    names = [o.name for o in exe.funcs["main"].ops]
+    for gone in ("exponential", "log", "compare", "iota", "convert", "select", "multiply", "subtract"):
+        assert gone not in names, names
+    ce = [o for o in exe.funcs["main"].ops if o.name == "emi.cross_entropy"][0]
+    assert ce.operands == ["%arg0", "%arg1"] and ce.attrs == {"negated": True}
+    n = int(np.prod(rows))
+    low = ej.optimize_module(text)
+    call = [l for l in low.splitlines() if "stablehlo.custom_call" in l]
+    assert len(call) == 1 and "@emi_cross_entropy_fwd(" in call[0]
+    assert ": (tensor<%dx16xf32>, tensor<%dxi32>) -> (tensor<%dxf32>, tensor<%dxf32>)" % (n, n, n, n) in call[0]
+    assert S.print_module(S.parse_module(low)) == low
+    rev = AD.reverse_module_text(text)
+    rcalls = [l.split("@")[1].split("(")[0] for l in rev.splitlines() if "stablehlo.custom_call" in l]
+    assert rcalls == ["emi_cross_entropy_fwd", "emi_cross_entropy_bwd"]
+    bwd = [l for l in rev.splitlines() if "@emi_cross_entropy_bwd" in l][0]
+    assert ": (tensor<%dx16xf32>, tensor<%dxi32>, tensor<%dxf32>, tensor<%dxf32>) -> tensor<%dx16xf32>" % (n, n, n, n, n) in bwd
+    sig = S.parse_module(rev)["main"]
+    assert [repr(t) for _, t in sig.args][-1] == "tensor<f32>" and len(sig.result_types) == 1        # d logits only
+    fwd = AD.forward_module_text(text)
+    assert [l.split("@")[1].split("(")[0] for l in fwd.splitlines() if "stablehlo.custom_call" in l] == \
+        ["emi_cross_entropy_fwd", "emi_cross_entropy_jvp"]
+
+
+def test_cross_entropy_cluster_is_left_alone_when_it_is_not_one():
+    from enzyme_ad.jax import stablehlo as S
+    text = traced_cross_entropy_text((8,), 16)
+    # the log-probabilities are also returned: interior value used outside
+    leaky = text.replace("-> (tensor<f32>)", "-> (tensor<f32>, tensor<8x16xf32>)").replace(
+        "return %20 : tensor<f32>", "return %20, %9 : tensor<f32>, tensor<8x16xf32>")
+    assert S.Executable(leaky).fused.get("cross_entropy", 0) == 0
+    # compared with NE, or against an index that is not the class index: not a one-hot
+    assert S.Executable(text.replace("compare  EQ", "compare  NE")).fused.get("cross_entropy", 0) == 0
+    shifted = text.replace("%11 = stablehlo.iota dim = 1 : tensor<1x16xi32>",
+                           "%11 = stablehlo.constant dense<[[1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16]]> : tensor<1x16xi32>")
+    assert S.Executable(shifted).fused.get("cross_entropy", 0) == 0
+    # the normaliser is the sum of exp of something else
+    assert S.Executable(text.replace("%4 = stablehlo.exponential %3", "%4 = stablehlo.exponential %arg0")).fused.get("cross_entropy", 0) == 0
