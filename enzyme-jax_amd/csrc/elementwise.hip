@@ -505,6 +505,44 @@ __global__ __launch_bounds__(256) void transpose_kernel(const T* __restrict__ in
   }
 }
 
+// The same for whole 16-byte pieces (rows and cols multiples of V = 16 / sizeof(T), aligned buffers) without LDS:
+// a thread owns a V x V block, reads its V rows as one 16-byte piece each, transposes the block in registers and
+// writes V pieces.  The lanes of a wavefront form an 8 x 8 grid of such blocks, so that every read and every write
+// instruction covers whole 128-byte lines (8 lanes x 16 bytes per row).
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_blocks_kernel(const T* __restrict__ in, T* __restrict__ out, int64_t rows,
+                                                               int64_t cols) {
+  constexpr int V = 16 / sizeof(T);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t r = ((int64_t)blockIdx.y * 2 + (wave >> 1)) * 8 * V + (lane >> 3) * V;
+  const int64_t c = ((int64_t)blockIdx.x * 2 + (wave & 1)) * 8 * V + (lane & 7) * V;
+  if (r >= rows || c >= cols) return;
+  uint32_t x[V][4], y[V][4];
+#pragma unroll
+  for (int i = 0; i < V; i++) {
+    const uint4 v = *reinterpret_cast<const uint4*>(in + (r + i) * cols + c);       // cached: weights are re-read soon
+    x[i][0] = v.x; x[i][1] = v.y; x[i][2] = v.z; x[i][3] = v.w;
+  }
+  if constexpr (V == 4) {
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+#pragma unroll
+      for (int i = 0; i < 4; i++) y[j][i] = x[i][j];
+  } else {
+    // 16-bit elements: dword k of output row j holds input rows 2k and 2k + 1 at column j
+#pragma unroll
+    for (int j = 0; j < 8; j++)
+#pragma unroll
+      for (int k = 0; k < 4; k++) {
+        const uint32_t a = x[2 * k][j >> 1], b = x[2 * k + 1][j >> 1];
+        y[j][k] = (j & 1) ? ((a >> 16) | (b & 0xffff0000u)) : ((a & 0xffffu) | (b << 16));
+      }
+  }
+#pragma unroll
+  for (int j = 0; j < V; j++)
+    *reinterpret_cast<uint4*>(out + (c + j) * rows + r) = make_uint4(y[j][0], y[j][1], y[j][2], y[j][3]);
+}
+
 // ---------------------------------------------------------------------------
 // launch helpers
 // ---------------------------------------------------------------------------
@@ -856,6 +894,14 @@ extern "C" int emi_embedding_bwd(emi_stream_t stream, const int32_t* tokens, con
 
 template <typename T> static int transpose_launch(hipStream_t st, const void* in, void* out, int64_t rows, int64_t cols) {
   const int vec_ok = (aligned16(in) && aligned16(out) && rows % 8 == 0 && cols % 8 == 0) ? 1 : 0;
+  constexpr int V = 16 / sizeof(T);
+  if (vec_ok && (rows + 16 * V - 1) / (16 * V) <= 65535) {
+    const dim3 gridb(blocks_for(cols, 16 * V), blocks_for(rows, 16 * V));
+    hipLaunchKernelGGL(transpose_blocks_kernel<T>, gridb, dim3(256), 0, st, static_cast<const T*>(in), static_cast<T*>(out),
+                       rows, cols);
+    EMI_CHECK_LAUNCH("emi_transpose");
+    return EMI_OK;
+  }
   const dim3 grid(blocks_for(cols, 64), blocks_for(rows, 64));
   hipLaunchKernelGGL(transpose_kernel<T>, grid, dim3(256), 0, st, static_cast<const T*>(in), static_cast<T*>(out), rows, cols,
                      vec_ok);

@@ -333,6 +333,56 @@ __global__ void __launch_bounds__(kBlock) tiled_permute_kernel(const E* __restri
   }
 }
 
+// The same permutation on whole 16-byte pieces (2- and 4-byte elements, n_dt and n_last multiples of V = 16 /
+// sizeof(E)) without LDS: a thread owns a V x V block over (last, dt), reads V pieces, transposes the block in
+// registers and writes V pieces; the lanes of a wavefront form an 8 x 8 grid of blocks, so every access
+// instruction covers whole 128-byte lines.
+template <typename E>
+__global__ void __launch_bounds__(kBlock) block_permute_kernel(const E* __restrict__ in, E* __restrict__ out, TilePlan p) {
+  constexpr int V = 16 / sizeof(E);
+  static_assert(V == 4 || V == 8, "2- or 4-byte elements");
+  int64_t rem = blockIdx.z, ib = 0, ob = 0;
+#pragma unroll
+  for (int d = kMaxRank - 1; d >= 0; d--) {
+    if (d < p.nouter) {
+      const int64_t q = rem / p.dims[d], r = rem - q * p.dims[d];
+      ib += r * p.is[d];
+      ob += r * p.os[d];
+      rem = q;
+    }
+  }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t r = ((int64_t)blockIdx.y * 2 + (wave >> 1)) * 8 * V + (lane >> 3) * V;      // r: last index, c: dt index
+  const int64_t c = ((int64_t)blockIdx.x * 2 + (wave & 1)) * 8 * V + (lane & 7) * V;
+  if (r >= p.n_last || c >= p.n_dt) return;
+  in += ib;
+  out += ob;
+  uint32_t x[V][4], y[V][4];
+#pragma unroll
+  for (int i = 0; i < V; i++) {
+    const uint4 v = *reinterpret_cast<const uint4*>(in + (r + i) * p.is_last + c);
+    x[i][0] = v.x; x[i][1] = v.y; x[i][2] = v.z; x[i][3] = v.w;
+  }
+  if constexpr (V == 4) {
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+#pragma unroll
+      for (int i = 0; i < 4; i++) y[j][i] = x[i][j];
+  } else {
+    // 16-bit elements: dword k of output row j holds source rows 2k and 2k + 1 at column j
+#pragma unroll
+    for (int j = 0; j < 8; j++)
+#pragma unroll
+      for (int k = 0; k < 4; k++) {
+        const uint32_t a = x[2 * k][j >> 1], b = x[2 * k + 1][j >> 1];
+        y[j][k] = (j & 1) ? ((a >> 16) | (b & 0xffff0000u)) : ((a & 0xffffu) | (b << 16));
+      }
+  }
+#pragma unroll
+  for (int j = 0; j < V; j++)
+    *reinterpret_cast<uint4*>(out + (c + j) * p.os_dt + r) = make_uint4(y[j][0], y[j][1], y[j][2], y[j][3]);
+}
+
 // Tries the tiled form; returns false when the plan does not have it (then the generic
 // kernel runs).
 template <typename E>
@@ -364,6 +414,16 @@ bool launch_tiled(hipStream_t st, const void* in, void* out, const CopyPlan& p, 
   constexpr int V = 16 / sizeof(E);
   int vec_ok = sizeof(E) <= 4 && al16(in) && al16(out) && t.is_last % V == 0 && t.os_dt % V == 0;
   for (int d = 0; d < t.nouter && vec_ok; d++) vec_ok = t.is[d] % V == 0 && t.os[d] % V == 0;
+  if constexpr (sizeof(E) == 2 || sizeof(E) == 4) {
+    if (vec_ok && t.n_dt % V == 0 && t.n_last % V == 0 && kBlock == 256) {
+      const int64_t bx = (t.n_dt + 16 * V - 1) / (16 * V), by = (t.n_last + 16 * V - 1) / (16 * V);
+      hipLaunchKernelGGL(block_permute_kernel<E>, dim3((unsigned)bx, (unsigned)by, (unsigned)nz), dim3(kBlock), 0, st,
+                         static_cast<const E*>(in), static_cast<E*>(out), t);
+      hipError_t eb = hipGetLastError();
+      *status = eb == hipSuccess ? EMI_OK : emi_fail(EMI_INTERNAL, "emi_strided_copy: launch failed: %s", hipGetErrorString(eb));
+      return true;
+    }
+  }
   hipLaunchKernelGGL(tiled_permute_kernel<E>, dim3((unsigned)gx, (unsigned)gy, (unsigned)nz), dim3(kBlock), 0, st,
                      static_cast<const E*>(in), static_cast<E*>(out), t, vec_ok);
   hipError_t e = hipGetLastError();
