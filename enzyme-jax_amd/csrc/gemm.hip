@@ -40,6 +40,17 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint3
 // (8 of them, each with its own L2), so give every XCD a contiguous run of
 // tiles, and walk tiles in groups of GROUP_M tile-rows so that the A and B
 // panels a XCD touches stay in its L2.
+// Up to four products of one shape in one launch of the 128x128 kernel (emi_gemm_grouped).  count == 0: the plain
+// single product.  sum == 0: independent results C[i] = op(A[i]) . op(B[i]) [+ R[i]], the grid holds count times the
+// tiles; sum == 1: every product is accumulated into the tile of C[0] (+ R[0]), pair after pair.
+struct GemmGroup {
+  const uint16_t* A[4];
+  const uint16_t* B[4];
+  const uint16_t* R[4];
+  uint16_t* C[4];
+  int count, sum;
+};
+
 __device__ __forceinline__ int xcd_contiguous_id() {
   const int nb = gridDim.x, bid = blockIdx.x;
   const int per = nb >> 3, rem = nb & 7;
@@ -248,7 +259,8 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_kernel(const uint16_t* 
                                                                  const uint16_t* __restrict__ B, const uint16_t* R,
                                                                  uint16_t* C, int M, int N, int K, int lda, int ldb,
                                                                  int ldr, int ldc, uint32_t a_bytes, uint32_t b_bytes,
-                                                                 int vec_ok, float* __restrict__ part, int k_per_split) {
+                                                                 int vec_ok, float* __restrict__ part, int k_per_split,
+                                                                 GemmGroup grp) {
   constexpr int NW = WM * WN;
   constexpr int KS = BK / 16;
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
@@ -266,13 +278,26 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_kernel(const uint16_t* 
   int tile_m, tile_n;
   // split-K: the grid is one run of tiles x splits blocks, split-major, so that the blocks of one XCD work on
   // the same slab of K and that slab of A and B is fetched into one L2 rather than into all eight
+  // (a group of independent products: split-major, then product, then tile)
   const int pid = xcd_contiguous_id();
-  const int split = part ? pid / (tiles_m * tiles_n) : 0;
-  tile_coords(part ? pid - split * tiles_m * tiles_n : pid, tiles_m, tiles_n, &tile_m, &tile_n);
+  const int tiles = tiles_m * tiles_n;
+  const int nprod = (grp.count > 0 && !grp.sum) ? grp.count : 1;
+  const int split = part ? pid / (tiles * nprod) : 0;
+  const int in_split = pid - split * tiles * nprod;
+  const int prod = in_split / tiles;
+  tile_coords(in_split - prod * tiles, tiles_m, tiles_n, &tile_m, &tile_n);
   const int m0 = tile_m * BM, n0 = tile_n * BN;
+  if (grp.count > 0 && !grp.sum) {
+    A = grp.A[prod];
+    B = grp.B[prod];
+    R = grp.R[prod];
+    C = grp.C[prod];
+    if (part) part += (int64_t)prod * (gridDim.x / (tiles * nprod)) * M * N;
+  }
+  const int npairs = (grp.count > 0 && grp.sum) ? grp.count : 1;
 
-  const __amdgpu_buffer_rsrc_t rA = make_rsrc(A, a_bytes);
-  const __amdgpu_buffer_rsrc_t rB = make_rsrc(B, b_bytes);
+  __amdgpu_buffer_rsrc_t rA = make_rsrc(A, a_bytes);
+  __amdgpu_buffer_rsrc_t rB = make_rsrc(B, b_bytes);
 
   auto issue_loads = [&](int stage, int k0) {
     EMI_LDS uint8_t* sA = smem + stage * STAGE;
@@ -328,21 +353,27 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_kernel(const uint16_t* 
   // issued before the MFMAs of the current one so their latency hides behind them.
   bf16x8_t fa[2][TM], fb[2][TN];
   if constexpr (NSTAGE == 2) {
-    issue_loads(0, k_lo);
-    wait_vmcnt<0>();
-    __syncthreads();
-    for (int t = 0; t < nk; t++) {
-      if (t + 1 < nk) issue_loads((t + 1) & 1, k_lo + (t + 1) * BK);
-      load_frags(t & 1, 0, fa[0], fb[0]);
-#pragma unroll
-      for (int kk = 0; kk < KS; kk++) {
-        if (kk + 1 < KS) load_frags(t & 1, kk + 1, fa[(kk + 1) & 1], fb[(kk + 1) & 1]);
-        __builtin_amdgcn_sched_barrier(0);
-        mfma_step(fa[kk & 1], fb[kk & 1]);
-        __builtin_amdgcn_sched_barrier(0);
+    for (int pair = 0; pair < npairs; pair++) {        // one pass unless several products are summed into this tile
+      if (npairs > 1) {
+        rA = make_rsrc(grp.A[pair], a_bytes);
+        rB = make_rsrc(grp.B[pair], b_bytes);
       }
-      wait_vmcnt<0>();     // next stage has landed
-      __syncthreads();     // and everyone is done reading this one
+      issue_loads(0, k_lo);
+      wait_vmcnt<0>();
+      __syncthreads();
+      for (int t = 0; t < nk; t++) {
+        if (t + 1 < nk) issue_loads((t + 1) & 1, k_lo + (t + 1) * BK);
+        load_frags(t & 1, 0, fa[0], fb[0]);
+#pragma unroll
+        for (int kk = 0; kk < KS; kk++) {
+          if (kk + 1 < KS) load_frags(t & 1, kk + 1, fa[(kk + 1) & 1], fb[(kk + 1) & 1]);
+          __builtin_amdgcn_sched_barrier(0);
+          mfma_step(fa[kk & 1], fb[kk & 1]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        wait_vmcnt<0>();     // next stage has landed
+        __syncthreads();     // and everyone is done reading this one
+      }
     }
   } else {
     static_assert(KS % 2 == 0, "fragment double buffering assumes an even number of k-steps per tile");
@@ -1069,7 +1100,7 @@ static int launch_bf16(hipStream_t st, const void* A, const void* B, const void*
     const int nz = (K + kps - 1) / kps;
     hipLaunchKernelGGL(kern, dim3(tiles * nz), dim3(WM * WN * 64), smem, st, static_cast<const uint16_t*>(A),
                        static_cast<const uint16_t*>(B), static_cast<const uint16_t*>(R), static_cast<uint16_t*>(C), M, N, K,
-                       lda, ldb, ldr, ldc, a_bytes, b_bytes, vec_ok, part, kps);
+                       lda, ldb, ldr, ldc, a_bytes, b_bytes, vec_ok, part, kps, GemmGroup{});
     EMI_CHECK_LAUNCH("emi_gemm(split-K)");
     hipLaunchKernelGGL(gemm_splitk_reduce_kernel<bf16>, dim3((unsigned)(((int64_t)M * N + 255) / 256)), dim3(256), 0, st, part,
                        static_cast<const bf16*>(R), static_cast<bf16*>(C), M, N, nz, (int64_t)ldr, (int64_t)ldc);
@@ -1078,8 +1109,59 @@ static int launch_bf16(hipStream_t st, const void* A, const void* B, const void*
   }
   hipLaunchKernelGGL(kern, dim3(tiles), dim3(WM * WN * 64), smem, st, static_cast<const uint16_t*>(A),
                      static_cast<const uint16_t*>(B), static_cast<const uint16_t*>(R), static_cast<uint16_t*>(C), M, N, K,
-                     lda, ldb, ldr, ldc, a_bytes, b_bytes, vec_ok, static_cast<float*>(nullptr), 0);
+                     lda, ldb, ldr, ldc, a_bytes, b_bytes, vec_ok, static_cast<float*>(nullptr), 0, GemmGroup{});
   EMI_CHECK_LAUNCH("emi_gemm");
+  return EMI_OK;
+}
+
+// Splits of K for `count` independent products of one shape in one launch (see bf16_splits).
+static int grouped_splits(int64_t M, int64_t N, int64_t K, int count) {
+  const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128) * count;
+  if (tiles > 128 || K < 2048) return 1;
+  int64_t s = 512 / tiles;
+  if (s > K / 1024) s = K / 1024;
+  return (int)(s < 2 ? 1 : (s > 64 ? 64 : s));
+}
+
+// The 128x128 kernel on a group of products (GemmGroup): one launch, count times the tiles (or, summed, count times
+// the contraction).
+template <bool AK, bool BKM>
+static int launch_bf16_grouped(hipStream_t st, const GemmGroup& g, int M, int N, int K, int lda, int ldb, int ldr, int ldc,
+                               uint32_t a_bytes, uint32_t b_bytes, void* workspace, size_t workspace_bytes) {
+  constexpr int BM = 128, BN = 128, BK = 64;
+  int vec_ok = (ldc % 8 == 0 && ldr % 8 == 0) ? 1 : 0;
+  const int nout = g.sum ? 1 : g.count;
+  for (int i = 0; i < nout; i++)
+    if ((reinterpret_cast<uintptr_t>(g.C[i]) & 15) || (g.R[i] != nullptr && (reinterpret_cast<uintptr_t>(g.R[i]) & 15))) vec_ok = 0;
+  auto kern = gemm_bf16_kernel<BM, BN, BK, 2, 2, 2, AK, BKM>;
+  constexpr int smem = 2 * (BM + BN) * BK * 2;
+  static bool configured = false;   // idempotent; a race only repeats the call
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return emi_fail(EMI_INTERNAL, "emi_gemm_grouped: cannot reserve %d bytes of LDS: %s", smem, hipGetErrorString(e));
+    configured = true;
+  }
+  const int tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+  const int splits = g.sum ? 1 : grouped_splits(M, N, K, g.count);
+  if (splits > 1 && workspace != nullptr && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0 &&
+      workspace_bytes >= (size_t)g.count * splits * M * N * sizeof(float)) {
+    float* part = static_cast<float*>(workspace);
+    const int kps = (((K + splits - 1) / splits) + BK - 1) / BK * BK;
+    const int nz = (K + kps - 1) / kps;
+    hipLaunchKernelGGL(kern, dim3(tiles * g.count * nz), dim3(256), smem, st, g.A[0], g.B[0], g.R[0], g.C[0], M, N, K, lda, ldb,
+                       ldr, ldc, a_bytes, b_bytes, vec_ok, part, kps, g);
+    EMI_CHECK_LAUNCH("emi_gemm_grouped(split-K)");
+    for (int i = 0; i < g.count; i++) {
+      hipLaunchKernelGGL(gemm_splitk_reduce_kernel<bf16>, dim3((unsigned)(((int64_t)M * N + 255) / 256)), dim3(256), 0, st,
+                         part + (int64_t)i * nz * M * N, reinterpret_cast<const bf16*>(g.R[i]), reinterpret_cast<bf16*>(g.C[i]), M, N,
+                         nz, (int64_t)ldr, (int64_t)ldc);
+      EMI_CHECK_LAUNCH("emi_gemm_grouped(split-K reduce)");
+    }
+    return EMI_OK;
+  }
+  hipLaunchKernelGGL(kern, dim3(tiles * nout), dim3(256), smem, st, g.A[0], g.B[0], g.R[0], g.C[0], M, N, K, lda, ldb, ldr, ldc,
+                     a_bytes, b_bytes, vec_ok, static_cast<float*>(nullptr), 0, g);
+  EMI_CHECK_LAUNCH("emi_gemm_grouped");
   return EMI_OK;
 }
 
@@ -1255,4 +1337,80 @@ extern "C" int emi_gemm_ws(emi_stream_t stream, const void* A, const void* B, co
     return EMI_OK;
   }
   return launch_generic<float>(st, A, B, R, C, (int)M, (int)N, (int)K, lda, ldb, ldr, ldc, trans_a, trans_b, workspace, workspace_bytes);
+}
+
+extern "C" size_t emi_gemm_grouped_workspace_bytes(int count, int64_t M, int64_t N, int64_t K, int trans_a, int trans_b, int sum,
+                                                    int dtype) {
+  size_t need = emi_gemm_workspace_bytes(M, N, K, trans_a, trans_b, dtype);          // the one-by-one fallback
+  if (count >= 2 && count <= 4 && !sum && dtype == EMI_BF16 && M > 0 && N > 0 && K > 0) {
+    const int splits = grouped_splits(M, N, K, count);
+    const size_t grouped = splits > 1 ? (size_t)count * splits * M * N * sizeof(float) : 0;
+    if (grouped > need) need = grouped;
+  }
+  return need;
+}
+
+extern "C" int emi_gemm_grouped(emi_stream_t stream, int count, const void* const* A, const void* const* B, const void* const* R,
+                                void* const* C, void* workspace, size_t workspace_bytes, int64_t M, int64_t N, int64_t K,
+                                int64_t lda, int64_t ldb, int64_t ldr, int64_t ldc, int trans_a, int trans_b, int sum, int dtype) {
+  EMI_REQUIRE(count >= 1 && count <= 4, "emi_gemm_grouped: count %d not in 1..4", count);
+  EMI_REQUIRE(A && B && C, "emi_gemm_grouped: null pointer table");
+  EMI_REQUIRE(M >= 0 && N >= 0 && K >= 0 && M <= 0x7fffffff && N <= 0x7fffffff && K <= 0x7fffffff,
+              "emi_gemm_grouped: bad dimensions M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
+  EMI_REQUIRE(dtype == EMI_F32 || dtype == EMI_BF16, "emi_gemm_grouped: unsupported dtype code %d (want 11=f32 or 16=bf16)", dtype);
+  const int nout = sum ? 1 : count;
+  for (int i = 0; i < count; i++) EMI_REQUIRE(A[i] && B[i], "emi_gemm_grouped: null operand %d", i);
+  for (int i = 0; i < nout; i++) EMI_REQUIRE(C[i], "emi_gemm_grouped: null result %d", i);
+  if (M == 0 || N == 0) return EMI_OK;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  bool fast = dtype == EMI_BF16 && count >= 2 && K > 0 && M > 8;
+  if (fast) {
+    const int64_t a_rows = trans_a ? K : M, b_rows = trans_b ? N : K;
+    const int64_t a_bytes = ((a_rows - 1) * lda + (trans_a ? M : K)) * 2;
+    const int64_t b_bytes = ((b_rows - 1) * ldb + (trans_b ? K : N)) * 2;
+    auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+    fast = lda >= (trans_a ? M : K) && ldb >= (trans_b ? K : N) && ldc >= N && (lda % 8 == 0) && (ldb % 8 == 0) && (K % 8 == 0) &&
+           (!trans_a || M % 8 == 0) && (trans_b || N % 8 == 0) && a_bytes < 0x7fffff00LL && b_bytes < 0x7fffff00LL &&
+           ldr <= 0x7fffffff && ldc <= 0x7fffffff && ((M + 255) / 256) * ((N + 255) / 256) < 192;
+    for (int i = 0; i < count && fast; i++) fast = al16(A[i]) && al16(B[i]);
+    // a residual on some results only would need a null check per product: all or none
+    bool any_r = false, all_r = true;
+    for (int i = 0; i < nout; i++) {
+      const bool has = R != nullptr && R[i] != nullptr;
+      any_r = any_r || has;
+      all_r = all_r && has;
+    }
+    if (any_r && (!all_r || ldr < N)) fast = false;
+    if (fast) {
+      GemmGroup g{};
+      g.count = count;
+      g.sum = sum ? 1 : 0;
+      for (int i = 0; i < count; i++) {
+        g.A[i] = static_cast<const uint16_t*>(A[i]);
+        g.B[i] = static_cast<const uint16_t*>(B[i]);
+      }
+      for (int i = 0; i < nout; i++) {
+        g.R[i] = any_r ? static_cast<const uint16_t*>(R[i]) : nullptr;
+        g.C[i] = static_cast<uint16_t*>(C[i]);
+      }
+      const int m = (int)M, n = (int)N, k = (int)K;
+      const uint32_t ab = (uint32_t)a_bytes, bb = (uint32_t)b_bytes;
+      if (!trans_a && trans_b)
+        return launch_bf16_grouped<false, false>(st, g, m, n, k, (int)lda, (int)ldb, (int)ldr, (int)ldc, ab, bb, workspace, workspace_bytes);
+      if (!trans_a && !trans_b)
+        return launch_bf16_grouped<false, true>(st, g, m, n, k, (int)lda, (int)ldb, (int)ldr, (int)ldc, ab, bb, workspace, workspace_bytes);
+      if (trans_a && !trans_b)
+        return launch_bf16_grouped<true, true>(st, g, m, n, k, (int)lda, (int)ldb, (int)ldr, (int)ldc, ab, bb, workspace, workspace_bytes);
+      return launch_bf16_grouped<true, false>(st, g, m, n, k, (int)lda, (int)ldb, (int)ldr, (int)ldc, ab, bb, workspace, workspace_bytes);
+    }
+  }
+  // one product after the other; summed: each launch adds onto the result of the one before
+  for (int i = 0; i < count; i++) {
+    const void* r = sum ? (i == 0 ? (R ? R[0] : nullptr) : C[0]) : (R ? R[i] : nullptr);
+    void* c = sum ? C[0] : C[i];
+    const int rc = emi_gemm_ws(stream, A[i], B[i], r, c, workspace, workspace_bytes, M, N, K, lda, ldb, (sum && i > 0) ? ldc : ldr, ldc,
+                               trans_a, trans_b, dtype);
+    if (rc != EMI_OK) return rc;
+  }
+  return EMI_OK;
 }

@@ -45,6 +45,10 @@ SIGNATURES = {
     "emi_gemm_workspace_bytes": (c_size_t, [c_i64, c_i64, c_i64, c_int, c_int, c_int]),
     "emi_gemm_ws": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_i64, c_i64, c_i64, c_i64,
                             c_i64, c_i64, c_i64, c_int, c_int, c_int]),
+    "emi_gemm_grouped_workspace_bytes": (c_size_t, [c_int, c_i64, c_i64, c_i64, c_int, c_int, c_int, c_int]),
+    "emi_gemm_grouped": (c_int, [c_void_p, c_int, ctypes.POINTER(c_void_p), ctypes.POINTER(c_void_p), ctypes.POINTER(c_void_p),
+                                 ctypes.POINTER(c_void_p), c_void_p, c_size_t, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64,
+                                 c_int, c_int, c_int, c_int]),
     "emi_attn_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_i64, c_i64, c_i64,
                              c_i64, c_i64, c_i64, c_float, c_int, c_int]),
     "emi_attn_fwd_workspace_bytes": (c_size_t, [c_i64, c_i64, c_i64, c_i64]),

@@ -16,16 +16,13 @@ LAYER_KEYS = ("rms_att_weight", "wq", "wk", "wv", "wo", "rms_ffn_weight", "w1", 
 def layer(x, lw, n_heads, eps=1e-5, theta=10000.0):
     """One decoder layer (test/llama.py:144-233).  x: [B, S, dim]."""
     xb = ops.rmsnorm(x, lw["rms_att_weight"], eps)                 # :145
-    q = ops.matmul_nt(xb, lw["wq"])                                # :149-157
-    k = ops.matmul_nt(xb, lw["wk"])
-    v = ops.matmul_nt(xb, lw["wv"])
+    q, k, v = ops.matmul_nt_group(xb, (lw["wq"], lw["wk"], lw["wv"]))      # :149-157, one launch when the shapes agree
     q = ops.rope(q, n_heads, theta)                                # :161-168
     k = ops.rope(k, n_heads, theta)
     att = ops.attention(q, k, v, n_heads, causal=True)             # :178-209
     x = ops.matmul_nt(att, lw["wo"], residual=x)                   # :211-215
     xb = ops.rmsnorm(x, lw["rms_ffn_weight"], eps)                 # :219
-    h1 = ops.matmul_nt(xb, lw["w1"])                               # :224-225
-    h3 = ops.matmul_nt(xb, lw["w3"])
+    h1, h3 = ops.matmul_nt_group(xb, (lw["w1"], lw["w3"]))         # :224-227
     g = ops.swiglu(h1, h3)                                         # :227-229
     return ops.matmul_nt(g, lw["w2"], residual=x)                  # :231-233
 

@@ -18,6 +18,8 @@ instead of costing an extra pass over HBM.
 """
 import math
 
+import ctypes
+
 import torch
 
 from . import _native as N
@@ -103,8 +105,9 @@ class Tape:
     def record(inputs, output, rule):
         t = Tape._active
         if t is not None:
-            t.nodes.append((inputs, output, rule))
-            t.produced.add(id(output))
+            t.nodes.append((inputs, output, rule))       # output: a tensor, or a tuple of tensors (one rule for all of them)
+            for o in (output if isinstance(output, tuple) else (output,)):
+                t.produced.add(id(o))
 
     def backward(self, outputs, cotangents, wrt):
         """Cotangents of `wrt` (list of tensors) given cotangents of `outputs`."""
@@ -117,9 +120,14 @@ class Tape:
                 raise ValueError("cotangent %s/%s does not match output %s/%s" % (tuple(c.shape), c.dtype, tuple(o.shape), o.dtype))
             ct[id(o)] = c if id(o) not in ct else add(ct[id(o)], c)
         for inputs, output, rule in reversed(self.nodes):
-            c = ct.pop(id(output), None)
-            if c is None:
-                continue
+            if isinstance(output, tuple):                # the rule takes the tuple of cotangents (None = zero)
+                c = tuple(ct.pop(id(o), None) for o in output)
+                if all(x is None for x in c):
+                    continue
+            else:
+                c = ct.pop(id(output), None)
+                if c is None:
+                    continue
             first, acc = set(), []
             for i in inputs:          # an operand that appears twice gets its fan-in summed afterwards
                 fresh = isinstance(i, torch.Tensor) and id(i) not in first
@@ -383,6 +391,89 @@ def gemm(a, b, trans_a=False, trans_b=False, residual=None):
     return c
 
 
+def _weight_in_place(rows2d, w):
+    """dX = dY . W reads W as stored (k-major) rather than through a transposed copy."""
+    return rows2d.shape[0] <= 8 or rows2d.dtype == torch.float32
+
+
+def _ptr_table(ts):
+    return (ctypes.c_void_p * len(ts))(*[None if t is None else t.data_ptr() for t in ts])
+
+
+def gemm_grouped(As, Bs, trans_a=False, trans_b=False, residuals=None, sum_into_one=False):
+    """Up to four products of one shape in one launch (emi_gemm_grouped): the list of op(a_i) . op(b_i) [+ r_i], or, with
+    sum_into_one, the single tensor sum_i op(a_i) . op(b_i) [+ r_0]."""
+    n = len(As)
+    if n != len(Bs) or not 1 <= n <= 4:
+        raise ValueError("gemm_grouped: %d / %d operands (1 to 4 pairs wanted)" % (len(As), len(Bs)))
+    rs = list(residuals) if residuals is not None else [None] * (1 if sum_into_one else n)
+    _dev(*As, *Bs, *rs)
+    _same_dtype(*As, *Bs, *rs)
+    a, b = As[0], Bs[0]
+    if any(t.shape != a.shape for t in As) or any(t.shape != b.shape for t in Bs):
+        raise ValueError("gemm_grouped: the products must have one shape")
+    M, K = (a.shape[1], a.shape[0]) if trans_a else a.shape
+    Kb, Nn = (b.shape[1], b.shape[0]) if trans_b else b.shape
+    if K != Kb:
+        raise ValueError("gemm_grouped: contraction mismatch %d vs %d" % (K, Kb))
+    if any(r is not None and r.shape != (M, Nn) for r in rs):
+        raise ValueError("gemm_grouped: residual shape")
+    if any(r is None for r in rs) and any(r is not None for r in rs):
+        raise ValueError("gemm_grouped: residuals for all results or for none")
+    outs = [torch.empty((M, Nn), dtype=a.dtype, device=a.device) for _ in rs]
+    lib = N.lib()
+    nbytes = lib.emi_gemm_grouped_workspace_bytes(n, M, Nn, K, int(trans_a), int(trans_b), int(sum_into_one), _code(a))
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=a.device) if nbytes else None
+    N.check(lib.emi_gemm_grouped(_stream(), n, _ptr_table(As), _ptr_table(Bs), _ptr_table(rs) if rs[0] is not None else None,
+                                 _ptr_table(outs), _p(ws), nbytes, M, Nn, K, a.shape[1], b.shape[1], Nn, Nn, int(trans_a),
+                                 int(trans_b), int(sum_into_one), _code(a)))
+    return outs[0] if sum_into_one else outs
+
+
+def matmul_nt_group(x, ws):
+    """(x . w^T for w in ws) for two to four weights of one shape applied to the same activation: q, k, v of
+    test/llama.py:149-157 and w1, w3 of :224-227 as one launch.  Reverse mode is one rule for the group: the weight
+    gradients dW_i = dY_i^T . X as one launch and dX = sum_i dY_i . W_i as one accumulation (the fan-in the Add rule
+    would build from three separate adjoints)."""
+    ws = list(ws)
+    if not 2 <= len(ws) <= 4 or any(w.shape != ws[0].shape or w.dtype != x.dtype for w in ws):
+        return tuple(matmul_nt(x, w) for w in ws)
+    lead, K, Nout = x.shape[:-1], x.shape[-1], ws[0].shape[0]
+    x2 = x.reshape(-1, K)
+    ys = tuple(y.reshape(*lead, Nout) for y in gemm_grouped([x2] * len(ws), ws, False, True))
+
+    def rule(cs, acc):
+        live = [i for i, c in enumerate(cs) if c is not None]
+        c2 = [cs[i].reshape(-1, Nout) for i in live]
+        ax = None if acc[0] is None else acc[0].reshape(-1, K)
+        few = _weight_in_place(x2, ws[0])                              # as in matmul_nt
+        wb = [ws[i] if few else _transpose_shared(ws[i]) for i in live]
+        dx = gemm_grouped(c2, wb, False, not few, None if ax is None else [ax], sum_into_one=True).reshape(x.shape)
+        racc = [acc[1 + i] for i in live]
+        if any(r is None for r in racc) and any(r is not None for r in racc):
+            dws = [gemm(c, x2, True, False, r) for c, r in zip(c2, racc)]
+        else:
+            dws = gemm_grouped(c2, [x2] * len(live), True, False, None if racc[0] is None else racc)
+        out = [dx] + [None] * len(ws)
+        for i, dw in zip(live, dws):
+            out[1 + i] = dw
+        return out
+
+    Tape.record((x, *ws), ys, rule)
+    tans = _tan(x, *ws)
+    if tans is not None and any(t is not None for t in tans):
+        tx = tans[0]
+        for y, w, tw in zip(ys, ws, tans[1:]):                  # ty = tx W^T + x tW^T
+            t = None
+            if tx is not None:
+                t = gemm(tx.reshape(-1, K), w, False, True, t)
+            if tw is not None:
+                t = gemm(x2, tw, False, True, t)
+            if t is not None:
+                _set_tan(y, t.reshape(*lead, Nout))
+    return ys
+
+
 def matmul_nt(x, w, residual=None):
     """Y[..., out] = X[..., in] . W[out, in]^T [+ residual]  (`w @ x` of
     test/llama.py:149-157,211,224-233, batched over tokens)."""
@@ -400,8 +491,9 @@ def matmul_nt(x, w, residual=None):
         # else) so that the contraction index is innermost in both operands: the
         # k-contiguous kernel beats the k-major one by more than the transpose costs.
         # With a handful of tokens (the single-token step) W is read in place, once; so it is in fp32, whose
-        # kernels read either layout at the same speed.
-        if c2.shape[0] <= 8 or c2.dtype == torch.float32:
+        # kernels read either layout at the same speed.  (Reading small bf16 weights in place was tried for the
+        # 768-wide model: the whole step came out 1.4 % slower than with the transposes.)
+        if _weight_in_place(c2, w):
             dx = gemm(c2, w, False, False, ax).reshape(x.shape)
         else:
             dx = gemm(c2, _transpose_shared(w), False, True, ax).reshape(x.shape)

@@ -126,6 +126,22 @@ int emi_gemm_ws(emi_stream_t stream, const void* A, const void* B, const void* R
                 int64_t lda, int64_t ldb, int64_t ldr, int64_t ldc, int trans_a, int trans_b,
                 int dtype);
 
+/* Up to four products of one shape in one launch: the q, k and v projections of one activation (test/llama.py:149-157),
+ * w1 and w3 (:224-227), the weight gradients of such a group, and -- with `sum` -- the fan-in of their input gradients,
+ * dX = sum_i dY_i . W_i (the DotGeneral rule HLODerivatives.td:1166-1178 followed by the additions of the Add rule :964).
+ * A, B, R, C: tables of `count` pointers (R null, or one entry per result, all set or all null).
+ *   sum == 0:  C[i] = op(A[i]) . op(B[i]) [+ R[i]]            (entries may repeat: one X against three weights)
+ *   sum == 1:  C[0] = sum_i op(A[i]) . op(B[i]) [+ R[0]]      (products added in index order)
+ * Shapes, leading dimensions and flags as for emi_gemm, the same for every product.  Small aligned bf16 products run
+ * as one launch of the 128x128 kernel; anything else runs as `count` emi_gemm_ws calls with the same results up to the
+ * rounding of the intermediate sums (sum == 1 then rounds C[0] to its type between products).  The workspace (size
+ * from emi_gemm_grouped_workspace_bytes, may be null) holds split-K partials. */
+size_t emi_gemm_grouped_workspace_bytes(int count, int64_t M, int64_t N, int64_t K, int trans_a, int trans_b, int sum,
+                                        int dtype);
+int emi_gemm_grouped(emi_stream_t stream, int count, const void* const* A, const void* const* B, const void* const* R,
+                     void* const* C, void* workspace, size_t workspace_bytes, int64_t M, int64_t N, int64_t K, int64_t lda,
+                     int64_t ldb, int64_t ldr, int64_t ldc, int trans_a, int trans_b, int sum, int dtype);
+
 /* Causal softmax attention, forward.  Replaces the per-head loop of
  * test/llama.py:178-206 with softmax of :13-18 (scale applied after the dot,
  * max-subtracted, fp32 statistics).  Element (b, h, s, i) of q/k/v/o lives at

@@ -126,6 +126,80 @@ def test_gemm_layouts(ops, dt, ta, tb, M, N, K):
     check(ops.gemm(a, b, bool(ta), bool(tb), r), ref + rr, dt, "gemm + residual")
 
 
+GROUPED_SHAPES = [
+    (256, 384, 320),     # one launch of the 128-tile kernel, K not a multiple of 64
+    (200, 136, 72),      # ragged tiles
+    (264, 136, 4104),    # few tiles, long contraction: split-K partials per product
+    (37, 29, 19),        # nothing aligned: product after product
+    (4096, 3072, 264),   # each product fills the chip with 256-tiles on its own: product after product
+]
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("ta,tb", [(0, 1), (0, 0), (1, 0), (1, 1)])
+@pytest.mark.parametrize("M,N,K", GROUPED_SHAPES)
+def test_gemm_grouped(ops, dt, ta, tb, M, N, K):
+    """emi_gemm_grouped: three products of one shape, independent (with a shared A, as q/k/v share the activation)
+    and summed into one result, with and without residuals, against fp64 matmul."""
+    _say("gemm_grouped", dt, ta, tb, M, N, K)
+    rng = np.random.default_rng(M + 3 * N + K + ta * 2 + tb)
+    a0, a0r = dev(rng.standard_normal((K, M) if ta else (M, K)), dt)
+    As, Ars = [a0, a0], [a0r, a0r]                                     # two products share their A operand
+    a2, a2r = dev(rng.standard_normal((K, M) if ta else (M, K)), dt)
+    As.append(a2)
+    Ars.append(a2r)
+    Bs, Brs = zip(*[dev(rng.standard_normal((N, K) if tb else (K, N)), dt) for _ in range(3)])
+    Rs, Rrs = zip(*[dev(rng.standard_normal((M, N)), dt) for _ in range(3)])
+    prods = [(ar.T if ta else ar) @ (br.T if tb else br) for ar, br in zip(Ars, Brs)]
+    outs = ops.gemm_grouped(As, list(Bs), bool(ta), bool(tb))
+    for o, ref in zip(outs, prods):
+        check(o, ref, dt, "grouped")
+    outs = ops.gemm_grouped(As, list(Bs), bool(ta), bool(tb), list(Rs))
+    for o, ref, rr in zip(outs, prods, Rrs):
+        check(o, ref + rr, dt, "grouped + residual")
+    total = sum(prods)
+    check(ops.gemm_grouped(As, list(Bs), bool(ta), bool(tb), sum_into_one=True), total, dt, "grouped sum", factor=2.0)
+    check(ops.gemm_grouped(As, list(Bs), bool(ta), bool(tb), [Rs[0]], sum_into_one=True), total + Rrs[0], dt, "grouped sum + residual",
+          factor=2.0)
+    # run-to-run identical bits (fixed summation order)
+    again = ops.gemm_grouped(As, list(Bs), bool(ta), bool(tb), sum_into_one=True)
+    assert torch.equal(again, ops.gemm_grouped(As, list(Bs), bool(ta), bool(tb), sum_into_one=True))
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+def test_matmul_nt_group_matches_separate_projections(ops, dt):
+    """q, k, v = x W^T for three weights of one shape: values, the gradients of x and of every weight, with one of the
+    three cotangents missing, and the tangent, against the oracle's linear rule applied three times."""
+    rng = np.random.default_rng(8)
+    x, xr = dev(rng.standard_normal((2, 130, 136)), dt)
+    ws, wrs = zip(*[dev(rng.standard_normal((200, 136)) * 0.1, dt) for _ in range(3)])
+    dys, dyrs = zip(*[dev(rng.standard_normal((2, 130, 200)), dt) for _ in range(3)])
+    with ops.Tape() as tape:
+        ys = ops.matmul_nt_group(x, ws)
+    for y, wr in zip(ys, wrs):
+        check(y, L.linear_fwd(xr, wr), dt, "group fwd")
+    grads = tape.backward(list(ys), list(dys), [x, *ws])
+    rdx = sum(L.linear_bwd(xr, wr, dyr)[0] for wr, dyr in zip(wrs, dyrs))
+    check(grads[0], rdx, dt, "group dX", factor=2.0)
+    for g, wr, dyr in zip(grads[1:], wrs, dyrs):
+        check(g, L.linear_bwd(xr, wr, dyr)[1], dt, "group dW")
+    # the cotangent of k missing: its weight gets no gradient, dX is the sum of the other two
+    with ops.Tape() as tape:
+        ys = ops.matmul_nt_group(x, ws)
+    grads = tape.backward([ys[0], ys[2]], [dys[0], dys[2]], [x, *ws])
+    check(grads[0], L.linear_bwd(xr, wrs[0], dyrs[0])[0] + L.linear_bwd(xr, wrs[2], dyrs[2])[0], dt, "group dX, two of three", factor=2.0)
+    assert grads[2] is None
+    check(grads[3], L.linear_bwd(xr, wrs[2], dyrs[2])[1], dt, "group dW, two of three")
+    # forward mode
+    from enzyme_ad.jax import jvp
+    tx, txr = dev(rng.standard_normal((2, 130, 136)), dt)
+    tw, twr = dev(rng.standard_normal((200, 136)) * 0.1, dt)
+    zero = torch.zeros_like(ws[0])
+    _, tans = jvp(lambda a, b, c, d: ops.matmul_nt_group(a, (b, c, d)), (x, *ws), (tx, tw, zero, zero))
+    check(tans[0], L.linear_fwd(txr, wrs[0]) + L.linear_fwd(xr, twr), dt, "group tangent q", factor=2.0)
+    check(tans[1], L.linear_fwd(txr, wrs[1]), dt, "group tangent k")
+
+
 @pytest.mark.parametrize("dt", ["f32", "bf16"])
 def test_matmul_nt_vjp(ops, dt):
     rng = np.random.default_rng(3)
