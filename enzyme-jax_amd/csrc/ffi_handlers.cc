@@ -265,6 +265,51 @@ extern "C" XLA_FFI_Error* emi_gemm_ffi(XLA_FFI_CallFrame* cf) {
                                    ws ? byte_size(ws) : 0, M, N, K, A->dims[1], B->dims[1], N, N, (int)ta, (int)tb, A->dtype));
 }
 
+// count A operands, count B operands, then no residual or one per result; count results (one when `sum`), then an
+// optional scratch result for split-K partials.
+extern "C" XLA_FFI_Error* emi_gemm_grouped_ffi(XLA_FFI_CallFrame* cf) {
+  EMI_FFI_BEGIN("emi_gemm_grouped", 4, 12, 1, 5)
+  int64_t count = 0, sum = 0, ta = 0, tb = 0;
+  if (!f.get_i("count", &count) || count < 2 || count > 4) return f.invalid("attribute 'count' must be 2, 3 or 4 (got %lld)", count);
+  f.get_i("sum", &sum);
+  f.get_i("trans_a", &ta);
+  f.get_i("trans_b", &tb);
+  const int64_t nout = sum ? 1 : count;
+  const int64_t nargs = cf->args.size, nrets = cf->rets.size;
+  if (nargs != 2 * count && nargs != 2 * count + nout)
+    return f.invalid("expected %lld operands (A..., B...) or %lld (with residuals), got %lld", 2 * count, 2 * count + nout, nargs);
+  if (nrets != nout && nrets != nout + 1) return f.invalid("expected %lld result(s) plus an optional workspace, got %lld", nout, nrets);
+  const bool has_r = nargs == 2 * count + nout;
+  const XLA_FFI_Buffer* A0 = f.arg(0);
+  const XLA_FFI_Buffer* B0 = f.arg((int)count);
+  if (!is_float(A0) || A0->rank != 2 || B0->rank != 2) return f.invalid("operands must be rank-2 f32 or bf16 (A rank %lld, B rank %lld)", A0->rank, B0->rank);
+  const int64_t M = ta ? A0->dims[1] : A0->dims[0], K = ta ? A0->dims[0] : A0->dims[1];
+  const int64_t Kb = tb ? B0->dims[1] : B0->dims[0], N = tb ? B0->dims[0] : B0->dims[1];
+  if (K != Kb) return f.invalid("contraction sizes differ: %lld vs %lld", K, Kb);
+  const void *a[4], *b[4], *r[4] = {nullptr, nullptr, nullptr, nullptr};
+  void* c[4];
+  for (int64_t i = 0; i < count; i++) {
+    const XLA_FFI_Buffer *Ai = f.arg((int)i), *Bi = f.arg((int)(count + i));
+    if (Ai->dtype != A0->dtype || Bi->dtype != A0->dtype || !same_shape(Ai, A0) || !same_shape(Bi, B0))
+      return f.invalid("product %lld: operands must have the dtype and shapes of product 0", i);
+    a[i] = Ai->data;
+    b[i] = Bi->data;
+  }
+  for (int64_t i = 0; i < nout; i++) {
+    const XLA_FFI_Buffer* Ci = f.ret((int)i);
+    const XLA_FFI_Buffer* Ri = has_r ? f.arg((int)(2 * count + i)) : nullptr;
+    if (Ci->dtype != A0->dtype || Ci->rank != 2 || Ci->dims[0] != M || Ci->dims[1] != N || (Ri && (Ri->dtype != A0->dtype || !same_shape(Ri, Ci))))
+      return f.invalid("result %lld (and its residual) must be [%lld, %lld] of the operands' dtype", i, M, N);
+    c[i] = Ci->data;
+    r[i] = Ri ? Ri->data : nullptr;
+  }
+  const XLA_FFI_Buffer* ws = nrets == nout + 1 ? f.ret((int)nout) : nullptr;
+  EMI_FFI_STREAM()
+  return f.from_status(emi_gemm_grouped(stream, (int)count, a, b, has_r ? r : nullptr, c, ws ? ws->data : nullptr,
+                                        ws ? byte_size(ws) : 0, M, N, K, A0->dims[1], B0->dims[1], N, N, (int)ta, (int)tb,
+                                        sum ? 1 : 0, A0->dtype));
+}
+
 namespace {
 struct AttnDims {
   int64_t B, H, S, D, sb, sh, ss;
@@ -557,6 +602,7 @@ const Target kTargets[] = {
     {"emi_rope_table", emi_rope_table_ffi},   {"emi_rope", emi_rope_ffi},
     {"emi_swiglu_fwd", emi_swiglu_fwd_ffi},   {"emi_swiglu_bwd", emi_swiglu_bwd_ffi},
     {"emi_add", emi_add_ffi},                 {"emi_gemm", emi_gemm_ffi},
+    {"emi_gemm_grouped", emi_gemm_grouped_ffi},
     {"emi_attn_fwd", emi_attn_fwd_ffi},       {"emi_attn_bwd", emi_attn_bwd_ffi},
     {"emi_attn_step_fwd", emi_attn_step_fwd_ffi}, {"emi_attn_step_bwd", emi_attn_step_bwd_ffi},
     {"emi_rmsnorm_jvp", emi_rmsnorm_jvp_ffi}, {"emi_swiglu_jvp", emi_swiglu_jvp_ffi}, {"emi_attn_jvp", emi_attn_jvp_ffi},

@@ -67,6 +67,17 @@ def test_ffi_handlers_launch_on_the_frame_stream():
               {"trans_a": (F.PRED, 0), "trans_b": (F.PRED, 1)})
         assert torch.equal(c, ops.gemm(a, w, False, True, r))
         check(c, ar @ wr.T + rr, "bf16", "ffi gemm")
+        # grouped gemm: three weights against one activation, then the three adjoints summed into one dX
+        ws3 = [dev(rng.standard_normal((192, 256)) * 0.1, "bf16") for _ in range(3)]
+        cs3 = [torch.empty((128, 192), dtype=torch.bfloat16, device="cuda") for _ in range(3)]
+        _call("emi_gemm_grouped_ffi", xla, [_buf(xla, a)] * 3 + [_buf(xla, w_) for w_, _ in ws3], [_buf(xla, c_) for c_ in cs3],
+              {"count": (F.S64, 3), "sum": (F.PRED, 0), "trans_a": (F.PRED, 0), "trans_b": (F.PRED, 1)})
+        for c_, (w_, wr_) in zip(cs3, ws3):
+            check(c_, ar @ wr_.T, "bf16", "ffi grouped gemm")
+        dx = torch.empty((128, 256), dtype=torch.bfloat16, device="cuda")
+        _call("emi_gemm_grouped_ffi", xla, [_buf(xla, c_) for c_ in cs3] + [_buf(xla, w_) for w_, _ in ws3], [_buf(xla, dx)],
+              {"count": (F.S64, 3), "sum": (F.PRED, 1), "trans_a": (F.PRED, 0), "trans_b": (F.PRED, 0)})
+        check(dx, sum(host(c_) @ wr_ for c_, (_, wr_) in zip(cs3, ws3)), "bf16", "ffi grouped gemm, summed", factor=2.0)
         # attention fwd + bwd, [B, S, h, d] layout
         B, S, h, d = 1, 96, 2, 128
         (q, qr), (k, kr), (v, vr), (do, dor) = (dev(rng.standard_normal((B, S, h, d)), "bf16") for _ in range(4))
