@@ -113,6 +113,7 @@ class Tape:
         """Cotangents of `wrt` (list of tensors) given cotangents of `outputs`."""
         ct = {}
         _transposed.clear()
+        _stack_reset(self.nodes)
         for o, c in zip(outputs, cotangents):
             if c is None:
                 continue
@@ -141,6 +142,7 @@ class Tape:
                 ct[id(i)] = g if id(i) not in done else add(ct[id(i)], g)
                 done.add(id(i))
         _transposed.clear()
+        _stack_reset(())
         return [ct.get(id(w)) for w in wrt]
 
 
@@ -237,7 +239,9 @@ def rmsnorm(x, gamma, eps=1e-5):
 
     def rule(c, acc):
         dx = torch.empty_like(x)
-        dgamma = torch.empty_like(gamma)
+        dgamma = _grad_target(gamma, acc[1])
+        if dgamma is None:
+            dgamma = torch.empty_like(gamma)
         nbytes = N.lib().emi_rmsnorm_bwd_workspace_bytes(rows, D)
         ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
         N.check(N.lib().emi_rmsnorm_bwd(_stream(), _p(x), _p(gamma), _p(c), _p(acc[0]), _p(dx), _p(dgamma), _p(ws),
@@ -358,6 +362,47 @@ def transpose(a):
     return out
 
 
+# Gradients of the slices of a stacked per-layer weight (`wq[l]`): when every use of the stacked tensor on the tape is
+# a `select` and no slice is selected twice, the kernel that produces a slice's gradient writes it straight into
+# slice l of one zero-filled buffer shaped like the stacked tensor, instead of into a temporary that the select rule
+# then adds in.  Valid for the duration of one Tape.backward.
+_stack = {"ok": set(), "buf": {}, "handed": set()}
+
+
+def _stack_reset(nodes):
+    ok, other, seen, twice = set(), set(), set(), set()
+    for inputs, _, rule in nodes:
+        sel = getattr(rule, "_emi_select", None)
+        for t in inputs:
+            if isinstance(t, torch.Tensor):
+                if sel is None:
+                    other.add(id(t))
+                else:
+                    ok.add(id(t))
+                    if (id(t), sel) in seen:
+                        twice.add(id(t))
+                    seen.add((id(t), sel))
+    _stack["ok"] = ok - other - twice
+    _stack["buf"] = {}
+    _stack["handed"] = set()
+
+
+def _stack_buffer(w):
+    buf = _stack["buf"].get(id(w))
+    if buf is None:
+        buf = _stack["buf"][id(w)] = torch.zeros_like(w)        # device memset
+    return buf
+
+
+def _grad_target(t, acc):
+    """The place the gradient of `t` is to be written to directly, or None (then the producer allocates)."""
+    st = getattr(t, "_emi_stack", None)
+    if acc is not None or st is None or id(st[0]) not in _stack["ok"] or id(t) in _stack["handed"]:
+        return None
+    _stack["handed"].add(id(t))
+    return _stack_buffer(st[0])[st[1]]
+
+
 _transposed = {}      # (data_ptr, shape) -> a^T, valid for the duration of one Tape.backward
 
 
@@ -373,8 +418,8 @@ def _transpose_shared(a):
     return hit[0]
 
 
-def gemm(a, b, trans_a=False, trans_b=False, residual=None):
-    """op(a) . op(b) [+ residual] on 2-D operands; fp32 accumulate."""
+def gemm(a, b, trans_a=False, trans_b=False, residual=None, out=None):
+    """op(a) . op(b) [+ residual] on 2-D operands; fp32 accumulate.  out: a contiguous [M, N] tensor to write to."""
     _dev(a, b, residual)
     _same_dtype(a, b, residual)
     M, K = (a.shape[1], a.shape[0]) if trans_a else a.shape
@@ -383,7 +428,9 @@ def gemm(a, b, trans_a=False, trans_b=False, residual=None):
         raise ValueError("gemm: contraction mismatch %d vs %d" % (K, Kb))
     if residual is not None and residual.shape != (M, Nn):
         raise ValueError("gemm: residual shape %s != (%d, %d)" % (tuple(residual.shape), M, Nn))
-    c = torch.empty((M, Nn), dtype=a.dtype, device=a.device)
+    if out is not None and (tuple(out.shape) != (M, Nn) or out.dtype != a.dtype or not out.is_contiguous()):
+        raise ValueError("gemm: out must be a contiguous [%d, %d] tensor of the operands' dtype" % (M, Nn))
+    c = torch.empty((M, Nn), dtype=a.dtype, device=a.device) if out is None else out
     nbytes = N.lib().emi_gemm_workspace_bytes(M, Nn, K, int(trans_a), int(trans_b), _code(a))
     ws = torch.empty(nbytes, dtype=torch.uint8, device=a.device) if nbytes else None
     N.check(N.lib().emi_gemm_ws(_stream(), _p(a), _p(b), _p(residual), _p(c), _p(ws), nbytes, M, Nn, K, a.shape[1],
@@ -400,7 +447,7 @@ def _ptr_table(ts):
     return (ctypes.c_void_p * len(ts))(*[None if t is None else t.data_ptr() for t in ts])
 
 
-def gemm_grouped(As, Bs, trans_a=False, trans_b=False, residuals=None, sum_into_one=False):
+def gemm_grouped(As, Bs, trans_a=False, trans_b=False, residuals=None, sum_into_one=False, outs=None):
     """Up to four products of one shape in one launch (emi_gemm_grouped): the list of op(a_i) . op(b_i) [+ r_i], or, with
     sum_into_one, the single tensor sum_i op(a_i) . op(b_i) [+ r_0]."""
     n = len(As)
@@ -420,7 +467,11 @@ def gemm_grouped(As, Bs, trans_a=False, trans_b=False, residuals=None, sum_into_
         raise ValueError("gemm_grouped: residual shape")
     if any(r is None for r in rs) and any(r is not None for r in rs):
         raise ValueError("gemm_grouped: residuals for all results or for none")
-    outs = [torch.empty((M, Nn), dtype=a.dtype, device=a.device) for _ in rs]
+    given = list(outs) if outs is not None else [None] * len(rs)
+    if len(given) != len(rs) or any(o is not None and (tuple(o.shape) != (M, Nn) or o.dtype != a.dtype or not o.is_contiguous())
+                                    for o in given):
+        raise ValueError("gemm_grouped: outs must be contiguous [%d, %d] tensors of the operands' dtype, one per result" % (M, Nn))
+    outs = [torch.empty((M, Nn), dtype=a.dtype, device=a.device) if o is None else o for o in given]
     lib = N.lib()
     nbytes = lib.emi_gemm_grouped_workspace_bytes(n, M, Nn, K, int(trans_a), int(trans_b), int(sum_into_one), _code(a))
     ws = torch.empty(nbytes, dtype=torch.uint8, device=a.device) if nbytes else None
@@ -453,7 +504,8 @@ def matmul_nt_group(x, ws):
         if any(r is None for r in racc) and any(r is not None for r in racc):
             dws = [gemm(c, x2, True, False, r) for c, r in zip(c2, racc)]
         else:
-            dws = gemm_grouped(c2, [x2] * len(live), True, False, None if racc[0] is None else racc)
+            dws = gemm_grouped(c2, [x2] * len(live), True, False, None if racc[0] is None else racc,
+                               outs=[_grad_target(ws[i], acc[1 + i]) for i in live])
         out = [dx] + [None] * len(ws)
         for i, dw in zip(live, dws):
             out[1 + i] = dw
@@ -501,7 +553,7 @@ def matmul_nt(x, w, residual=None):
         # k-major form of the GEMM kernel reads them in place (transposing LDS loads),
         # 3-7% slower than the k-contiguous form but without two activation-sized
         # transposes per projection.
-        dw = gemm(c2, x2, True, False, acc[1])
+        dw = gemm(c2, x2, True, False, acc[1], out=_grad_target(w, acc[1]))
         out = [dx, dw]
         if residual is not None:
             out.append(_accumulate(acc[2], c))
@@ -730,9 +782,17 @@ def select(w, i):
     cotangent is placed into slice i of a zero tensor shaped like w."""
     _dev(w)
     y = w[i]
+    y._emi_stack = (w, i)
 
     def rule(c, acc):
         g = acc[0]
+        if id(w) in _stack["ok"]:
+            # every cotangent of w comes from select rules, one per slice: slice i of the shared buffer is either
+            # already written (the producer was handed it) or still zero
+            buf = _stack_buffer(w)
+            if c.data_ptr() != buf[i].data_ptr():
+                buf[i].copy_(c)              # device-to-device copy
+            return (buf,)
         if g is not None and getattr(g, "_emi_select_owned", False):
             # a buffer an earlier select rule zero-filled and nobody else holds: add slice i in place
             N.check(N.lib().emi_add(_stream(), _p(g[i]), _p(c), _p(g[i]), c.numel(), _code(c)))
@@ -746,6 +806,7 @@ def select(w, i):
         # caller's own tensor): never written in place
         return (add(g, fresh),)
 
+    rule._emi_select = i
     Tape.record((w,), y, rule)
     tans = _tan(w)
     if tans is not None and tans[0] is not None:

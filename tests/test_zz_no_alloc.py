@@ -1,6 +1,8 @@
 """The allocation-free RMSNorm adjoint entry point against the workspace one, through the C ABI: two calls in a row on
 the same device, the second with a smaller input (the built-in scratch array keeps the first call's contents), plus
 the size limit."""
+import gc
+
 import numpy as np
 import pytest
 import torch
@@ -22,10 +24,15 @@ def _run_pair(lib, N, rows, dim, dt, code, seed):
     N.check(lib.emi_rmsnorm_bwd(st, p(x), p(gamma), p(dy), p(add), p(dx_ref), p(dg_ref), p(ws), nbytes, rows, dim, 1e-5, code))
     dx, dg = torch.full_like(x, float("nan")), torch.full_like(gamma, float("nan"))
     torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated()
-    N.check(lib.emi_rmsnorm_bwd_noalloc(st, p(x), p(gamma), p(dy), p(add), p(dx), p(dg), rows, dim, 1e-5, code))
-    torch.cuda.synchronize()
-    assert torch.cuda.memory_allocated() == before
+    gc.collect()                  # tensors that earlier tests left in reference cycles must not be freed inside the window
+    gc.disable()
+    try:
+        before = torch.cuda.memory_allocated()
+        N.check(lib.emi_rmsnorm_bwd_noalloc(st, p(x), p(gamma), p(dy), p(add), p(dx), p(dg), rows, dim, 1e-5, code))
+        torch.cuda.synchronize()
+        assert torch.cuda.memory_allocated() == before
+    finally:
+        gc.enable()
     assert torch.equal(dx, dx_ref), "dx differs (rows %d, dim %d)" % (rows, dim)
     assert torch.equal(dg, dg_ref), "dgamma differs (rows %d, dim %d)" % (rows, dim)
 
