@@ -40,14 +40,15 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint3
 // (8 of them, each with its own L2), so give every XCD a contiguous run of
 // tiles, and walk tiles in groups of GROUP_M tile-rows so that the A and B
 // panels a XCD touches stay in its L2.
-// Up to four products of one shape in one launch of the 128x128 kernel (emi_gemm_grouped).  count == 0: the plain
+// Several products of one shape in one launch of the 128x128 kernel (emi_gemm_grouped).  count == 0: the plain
 // single product.  sum == 0: independent results C[i] = op(A[i]) . op(B[i]) [+ R[i]], the grid holds count times the
 // tiles; sum == 1: every product is accumulated into the tile of C[0] (+ R[0]), pair after pair.
+constexpr int kMaxGroup = 48;      // products per launch (the argument block stays under 2 KB)
 struct GemmGroup {
-  const uint16_t* A[4];
-  const uint16_t* B[4];
-  const uint16_t* R[4];
-  uint16_t* C[4];
+  const uint16_t* A[kMaxGroup];
+  const uint16_t* B[kMaxGroup];
+  const uint16_t* R[kMaxGroup];
+  uint16_t* C[kMaxGroup];
   int count, sum;
 };
 
@@ -1342,7 +1343,7 @@ extern "C" int emi_gemm_ws(emi_stream_t stream, const void* A, const void* B, co
 extern "C" size_t emi_gemm_grouped_workspace_bytes(int count, int64_t M, int64_t N, int64_t K, int trans_a, int trans_b, int sum,
                                                     int dtype) {
   size_t need = emi_gemm_workspace_bytes(M, N, K, trans_a, trans_b, dtype);          // the one-by-one fallback
-  if (count >= 2 && count <= 4 && !sum && dtype == EMI_BF16 && M > 0 && N > 0 && K > 0) {
+  if (count >= 2 && count <= kMaxGroup && !sum && dtype == EMI_BF16 && M > 0 && N > 0 && K > 0) {
     const int splits = grouped_splits(M, N, K, count);
     const size_t grouped = splits > 1 ? (size_t)count * splits * M * N * sizeof(float) : 0;
     if (grouped > need) need = grouped;
@@ -1353,7 +1354,7 @@ extern "C" size_t emi_gemm_grouped_workspace_bytes(int count, int64_t M, int64_t
 extern "C" int emi_gemm_grouped(emi_stream_t stream, int count, const void* const* A, const void* const* B, const void* const* R,
                                 void* const* C, void* workspace, size_t workspace_bytes, int64_t M, int64_t N, int64_t K,
                                 int64_t lda, int64_t ldb, int64_t ldr, int64_t ldc, int trans_a, int trans_b, int sum, int dtype) {
-  EMI_REQUIRE(count >= 1 && count <= 4, "emi_gemm_grouped: count %d not in 1..4", count);
+  EMI_REQUIRE(count >= 1 && count <= kMaxGroup, "emi_gemm_grouped: count %d not in 1..%d", count, kMaxGroup);
   EMI_REQUIRE(A && B && C, "emi_gemm_grouped: null pointer table");
   EMI_REQUIRE(M >= 0 && N >= 0 && K >= 0 && M <= 0x7fffffff && N <= 0x7fffffff && K <= 0x7fffffff,
               "emi_gemm_grouped: bad dimensions M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);

@@ -126,7 +126,7 @@ int emi_gemm_ws(emi_stream_t stream, const void* A, const void* B, const void* R
                 int64_t lda, int64_t ldb, int64_t ldr, int64_t ldc, int trans_a, int trans_b,
                 int dtype);
 
-/* Up to four products of one shape in one launch: the q, k and v projections of one activation (test/llama.py:149-157),
+/* Up to EMI_GEMM_GROUP_MAX products of one shape in one launch: the q, k and v projections of one activation (test/llama.py:149-157),
  * w1 and w3 (:224-227), the weight gradients of such a group, and -- with `sum` -- the fan-in of their input gradients,
  * dX = sum_i dY_i . W_i (the DotGeneral rule HLODerivatives.td:1166-1178 followed by the additions of the Add rule :964).
  * A, B, R, C: tables of `count` pointers (R null, or one entry per result, all set or all null).
@@ -136,6 +136,7 @@ int emi_gemm_ws(emi_stream_t stream, const void* A, const void* B, const void* R
  * as one launch of the 128x128 kernel; anything else runs as `count` emi_gemm_ws calls with the same results up to the
  * rounding of the intermediate sums (sum == 1 then rounds C[0] to its type between products).  The workspace (size
  * from emi_gemm_grouped_workspace_bytes, may be null) holds split-K partials. */
+#define EMI_GEMM_GROUP_MAX 48
 size_t emi_gemm_grouped_workspace_bytes(int count, int64_t M, int64_t N, int64_t K, int trans_a, int trans_b, int sum,
                                         int dtype);
 int emi_gemm_grouped(emi_stream_t stream, int count, const void* const* A, const void* const* B, const void* const* R,
