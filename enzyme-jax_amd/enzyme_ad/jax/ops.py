@@ -367,15 +367,16 @@ def transpose(a):
 # a `select` and no slice is selected twice, the kernel that produces a slice's gradient writes it straight into
 # slice l of one zero-filled buffer shaped like the stacked tensor, instead of into a temporary that the select rule
 # then adds in.  Valid for the duration of one Tape.backward.
-_stack = {"ok": set(), "buf": {}, "handed": set()}
+_stack = {"ok": set(), "buf": {}, "handed": set(), "uses": {}}
 
 
 def _stack_reset(nodes):
-    ok, other, seen, twice = set(), set(), set(), set()
+    ok, other, seen, twice, uses = set(), set(), set(), set(), {}
     for inputs, _, rule in nodes:
         sel = getattr(rule, "_emi_select", None)
         for t in inputs:
             if isinstance(t, torch.Tensor):
+                uses[id(t)] = uses.get(id(t), 0) + 1
                 if sel is None:
                     other.add(id(t))
                 else:
@@ -386,6 +387,7 @@ def _stack_reset(nodes):
     _stack["ok"] = ok - other - twice
     _stack["buf"] = {}
     _stack["handed"] = set()
+    _stack["uses"] = uses
     _pending_dw[:] = []
 
 
@@ -421,9 +423,12 @@ def _stack_buffer(w):
 
 
 def _grad_target(t, acc):
-    """The place the gradient of `t` is to be written to directly, or None (then the producer allocates)."""
+    """The place the gradient of `t` is to be written to directly, or None (then the producer allocates): `t` is a
+    slice of an eligible stacked tensor and the caller is its only consumer (with two, the second would read the first
+    one's gradient as its residual before a deferred product has written it)."""
     st = getattr(t, "_emi_stack", None)
-    if acc is not None or st is None or id(st[0]) not in _stack["ok"] or id(t) in _stack["handed"]:
+    if acc is not None or st is None or id(st[0]) not in _stack["ok"] or id(t) in _stack["handed"] or \
+            _stack["uses"].get(id(t), 0) != 1:
         return None
     _stack["handed"].add(id(t))
     return _stack_buffer(st[0])[st[1]]

@@ -65,3 +65,61 @@ def test_concatenate_inner_dim_with_operand_fan_in():
     assert ga.is_contiguous() and gb.is_contiguous()
     assert np.max(np.abs(host(ga) - (host(cy)[:, :10] + 2 * host(ca)))) <= 1e-5
     assert torch.equal(gb, cy[:, 10:].contiguous())
+
+
+@pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
+def test_stacked_weight_gradients_written_in_place_and_deferred(dt):
+    """A stacked weight that is only ever sliced, one select per layer: the weight-gradient products are written
+    straight into the slices of one buffer and run grouped at the end of the backward pass.  Layers that are never
+    selected keep a zero gradient; the RMSNorm gain of a stacked gain tensor takes the same route."""
+    from enzyme_ad.jax import ops, vjp
+    L, T, D, H = 4, 136, 64, 96
+    w = (_randn((L, H, D), 20) * 0.1).to(dt)
+    gam = (_randn((L, D), 21) * 0.1 + 1).to(dt)
+    x = _randn((T, D), 22).to(dt)
+
+    def fn(w, gam):
+        ys = []
+        for l in (0, 1, 3):                                  # layer 2 is never used
+            ys.append(ops.matmul_nt(ops.rmsnorm(x, ops.select(gam, l)), ops.select(w, l)))
+        return ops.add(ops.add(ys[0], ys[1]), ys[2])
+
+    out, f_vjp = vjp(fn, w, gam)
+    c = _randn((T, H), 23).to(dt)
+    gw, gg = f_vjp(c)
+    w64, g64, x64, c64 = (t.double().requires_grad_(t is not x and t is not c) for t in (w, gam, x, c))
+    ref = 0
+    for l in (0, 1, 3):
+        xn = x64 * torch.rsqrt((x64 * x64).mean(-1, keepdim=True) + 1e-5) * g64[l]
+        ref = ref + xn @ w64[l].T
+    ref.backward(c64)
+    tol = 1e-4 if dt == torch.float32 else 3e-2
+    assert float((gw.double() - w64.grad).abs().max()) <= tol * float(w64.grad.abs().max())
+    assert float((gg.double() - g64.grad).abs().max()) <= tol * float(g64.grad.abs().max())
+    assert not gw[2].any() and not gg[2].any()
+    # twice in a row: the buffers of the first call are not reused
+    gw2, _ = f_vjp(c)
+    assert torch.equal(gw, gw2) and gw2.data_ptr() != gw.data_ptr()
+
+
+def test_stacked_weight_slice_selected_twice_or_used_twice():
+    """The cases the in-place route must stay away from: one slice selected by two select calls, and one selected
+    slice feeding two products (its cotangent is a sum that the select rule stores)."""
+    from enzyme_ad.jax import ops, vjp
+    w = _randn((2, 24, 40), 30)
+    x1, x2 = _randn((16, 40), 31), _randn((16, 40), 32)
+
+    def twice_selected(w):
+        return ops.add(ops.matmul_nt(x1, ops.select(w, 1)), ops.matmul_nt(x2, ops.select(w, 1)))
+
+    def twice_used(w):
+        s = ops.select(w, 1)
+        return ops.add(ops.matmul_nt(x1, s), ops.matmul_nt(x2, s))
+
+    c = _randn((16, 24), 33)
+    ref = np.zeros((2, 24, 40))
+    ref[1] = host(c).T @ host(x1) + host(c).T @ host(x2)
+    for fn in (twice_selected, twice_used):
+        _, f_vjp = vjp(fn, w)
+        (gw,) = f_vjp(c)
+        assert np.max(np.abs(host(gw) - ref)) <= 1e-4 * np.max(np.abs(ref)), fn.__name__
