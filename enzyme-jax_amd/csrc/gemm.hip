@@ -613,12 +613,16 @@ template <int N, typename F> __device__ __forceinline__ void static_for(F&& f) {
 // read with two transposing loads per fragment: the 32 lanes that are served
 // together address k-rows {0..3} and {8..11} (+4 for the second load), 32 bytes
 // each, which the swizzle spreads over all 64 banks.
-template <bool AKM, bool BKM>
+// GROUPED: the grid holds the tiles of grp.count independent products of one shape, product-major (GemmGroup with
+// sum == 0); otherwise the last argument is an empty placeholder.
+struct NoGroup {};
+template <bool AKM, bool BKM, bool GROUPED = false>
 __global__ __launch_bounds__(512) void gemm_bf16_pingpong_kernel(const uint16_t* __restrict__ A,
                                                                   const uint16_t* __restrict__ B, const uint16_t* R,
                                                                   uint16_t* C, int M, int N, int K, int lda, int ldb,
                                                                   int ldr, int ldc, uint32_t a_bytes, uint32_t b_bytes,
-                                                                  int vec_ok) {
+                                                                  int vec_ok,
+                                                                  std::conditional_t<GROUPED, GemmGroup, NoGroup> grp) {
   constexpr int BM = 256, BN = 256, BK = 64;
   constexpr int REGION = 128 * BK * 2;                          // 16 KiB
   // LDS map: A_h of stage s at (2s + h) regions, B_j of stage s at 64 KiB + (2s + j) regions, so that
@@ -633,7 +637,17 @@ __global__ __launch_bounds__(512) void gemm_bf16_pingpong_kernel(const uint16_t*
 
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
   int tile_m, tile_n;
-  tile_coords(xcd_contiguous_id(), tiles_m, tiles_n, &tile_m, &tile_n);
+  if constexpr (GROUPED) {
+    const int pid = xcd_contiguous_id(), tiles = tiles_m * tiles_n;
+    const int prod = pid / tiles;
+    tile_coords(pid - prod * tiles, tiles_m, tiles_n, &tile_m, &tile_n);
+    A = grp.A[prod];
+    B = grp.B[prod];
+    R = grp.R[prod];
+    C = grp.C[prod];
+  } else {
+    tile_coords(xcd_contiguous_id(), tiles_m, tiles_n, &tile_m, &tile_n);
+  }
   const int m0 = tile_m * BM, n0 = tile_n * BN;
 
   const __amdgpu_buffer_rsrc_t rA = make_rsrc(A, a_bytes);
@@ -1142,6 +1156,22 @@ static int launch_bf16_grouped(hipStream_t st, const GemmGroup& g, int M, int N,
     if (e != hipSuccess) return emi_fail(EMI_INTERNAL, "emi_gemm_grouped: cannot reserve %d bytes of LDS: %s", smem, hipGetErrorString(e));
     configured = true;
   }
+  const int big_tiles = ((M + 255) / 256) * ((N + 255) / 256);
+  if (!g.sum && (int64_t)big_tiles * g.count >= 192) {
+    // enough 256x256 tiles over the whole group to fill the chip: the ping-pong kernel, product-major
+    constexpr int smem_pp = 2 * 65536;
+    static bool configured_pp = false;
+    if (!configured_pp) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_pingpong_kernel<AK, BKM, true>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, smem_pp);
+      if (e != hipSuccess) return emi_fail(EMI_INTERNAL, "emi_gemm_grouped: cannot reserve %d bytes of LDS: %s", smem_pp, hipGetErrorString(e));
+      configured_pp = true;
+    }
+    hipLaunchKernelGGL((gemm_bf16_pingpong_kernel<AK, BKM, true>), dim3(big_tiles * g.count), dim3(512), smem_pp, st, g.A[0], g.B[0],
+                       g.R[0], g.C[0], M, N, K, lda, ldb, ldr, ldc, a_bytes, b_bytes, vec_ok, g);
+    EMI_CHECK_LAUNCH("emi_gemm_grouped(256-tiles)");
+    return EMI_OK;
+  }
   const int tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
   const int splits = g.sum ? 1 : grouped_splits(M, N, K, g.count);
   if (splits > 1 && workspace != nullptr && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0 &&
@@ -1183,7 +1213,7 @@ static int launch_bf16_pingpong(hipStream_t st, const void* A, const void* B, co
   const int tiles = ((M + 255) / 256) * ((N + 255) / 256);
   hipLaunchKernelGGL((gemm_bf16_pingpong_kernel<AKM, BKM>), dim3(tiles), dim3(512), smem, st, static_cast<const uint16_t*>(A),
                      static_cast<const uint16_t*>(B), static_cast<const uint16_t*>(R), static_cast<uint16_t*>(C), M, N, K,
-                     lda, ldb, ldr, ldc, a_bytes, b_bytes, vec_ok);
+                     lda, ldb, ldr, ldc, a_bytes, b_bytes, vec_ok, NoGroup{});
   EMI_CHECK_LAUNCH("emi_gemm");
   return EMI_OK;
 }

@@ -166,6 +166,23 @@ def test_gemm_grouped(ops, dt, ta, tb, M, N, K):
     assert torch.equal(again, ops.gemm_grouped(As, list(Bs), bool(ta), bool(tb), sum_into_one=True))
 
 
+@pytest.mark.parametrize("ta,tb", [(0, 1), (0, 0), (1, 0), (1, 1)])
+@pytest.mark.parametrize("count,M,N,K", [(24, 520, 768, 136), (48, 256, 256, 72), (12, 768, 768, 1032)])
+def test_gemm_grouped_many_products(ops, ta, tb, count, M, N, K):
+    """Groups large enough to fill the chip with 256 x 256 tiles (the same weight gradient of every layer of a model):
+    every product against fp64 matmul, with and without residuals, ragged M."""
+    _say("gemm_grouped_many", ta, tb, count, M, N, K)
+    rng = np.random.default_rng(count + M + ta * 2 + tb)
+    As, Ars = zip(*[dev(rng.standard_normal((K, M) if ta else (M, K)), "bf16") for _ in range(count)])
+    Bs, Brs = zip(*[dev(rng.standard_normal((N, K) if tb else (K, N)), "bf16") for _ in range(count)])
+    Rs, Rrs = zip(*[dev(rng.standard_normal((M, N)), "bf16") for _ in range(count)])
+    prods = [(ar.T if ta else ar) @ (br.T if tb else br) for ar, br in zip(Ars, Brs)]
+    for o, ref in zip(ops.gemm_grouped(list(As), list(Bs), bool(ta), bool(tb)), prods):
+        check(o, ref, "bf16", "grouped (many)")
+    for o, ref, rr in zip(ops.gemm_grouped(list(As), list(Bs), bool(ta), bool(tb), list(Rs)), prods, Rrs):
+        check(o, ref + rr, "bf16", "grouped (many) + residual")
+
+
 @pytest.mark.parametrize("dt", ["f32", "bf16"])
 def test_matmul_nt_group_matches_separate_projections(ops, dt):
     """q, k, v = x W^T for three weights of one shape: values, the gradients of x and of every weight, with one of the
