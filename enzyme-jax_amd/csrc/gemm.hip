@@ -51,6 +51,7 @@ struct GemmGroup {
   uint16_t* C[kMaxGroup];
   int count, sum;
 };
+struct NoGroup {};       // placeholder argument of the kernels' ungrouped instantiations
 
 __device__ __forceinline__ int xcd_contiguous_id() {
   const int nb = gridDim.x, bid = blockIdx.x;
@@ -615,7 +616,6 @@ template <int N, typename F> __device__ __forceinline__ void static_for(F&& f) {
 // each, which the swizzle spreads over all 64 banks.
 // GROUPED: the grid holds the tiles of grp.count independent products of one shape, product-major (GemmGroup with
 // sum == 0); otherwise the last argument is an empty placeholder.
-struct NoGroup {};
 template <bool AKM, bool BKM, bool GROUPED = false>
 __global__ __launch_bounds__(512) void gemm_bf16_pingpong_kernel(const uint16_t* __restrict__ A,
                                                                   const uint16_t* __restrict__ B, const uint16_t* R,
@@ -989,12 +989,21 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const T* __restrict__
 // 16-byte pieces and a k-major one in 128-byte rows.  The four partial tiles are added in wavefront order through
 // LDS (fixed order: run-to-run identical bits).
 // ---------------------------------------------------------------------------
-template <bool A_KMAJOR, bool B_KMAJOR>
+// GROUPED: blockIdx.z picks one of grp.count independent products of one shape (GemmGroup with sum == 0, its pointers
+// read as float).
+template <bool A_KMAJOR, bool B_KMAJOR, bool GROUPED = false>
 __global__ __launch_bounds__(256) void gemm_f32_small_kernel(const float* __restrict__ A, const float* __restrict__ B,
                                                              const float* R, float* C, int M, int N, int K, int64_t lda,
-                                                             int64_t ldb, int64_t ldr, int64_t ldc) {
+                                                             int64_t ldb, int64_t ldr, int64_t ldc,
+                                                             std::conditional_t<GROUPED, GemmGroup, NoGroup> grp) {
   constexpr int U = 4;                                   // 8-wide chunks in flight per step
   __shared__ float red[3][16][64];
+  if constexpr (GROUPED) {
+    A = reinterpret_cast<const float*>(grp.A[blockIdx.z]);
+    B = reinterpret_cast<const float*>(grp.B[blockIdx.z]);
+    R = reinterpret_cast<const float*>(grp.R[blockIdx.z]);
+    C = reinterpret_cast<float*>(grp.C[blockIdx.z]);
+  }
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int i = lane & 31, g = lane >> 5;
   const int m0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
@@ -1358,7 +1367,7 @@ extern "C" int emi_gemm_ws(emi_stream_t stream, const void* A, const void* B, co
 #define EMI_F32_SMALL(AKM, BKM)                                                                                       \
   hipLaunchKernelGGL((gemm_f32_small_kernel<AKM, BKM>), grid, dim3(256), 0, st, static_cast<const float*>(A),         \
                      static_cast<const float*>(B), static_cast<const float*>(R), static_cast<float*>(C), (int)M, (int)N, \
-                     (int)K, lda, ldb, ldr, ldc)
+                     (int)K, lda, ldb, ldr, ldc, NoGroup{})
     if (!trans_a && trans_b) EMI_F32_SMALL(false, false);
     else if (!trans_a && !trans_b) EMI_F32_SMALL(false, true);
     else if (trans_a && !trans_b) EMI_F32_SMALL(true, true);
@@ -1433,6 +1442,41 @@ extern "C" int emi_gemm_grouped(emi_stream_t stream, int count, const void* cons
       if (trans_a && !trans_b)
         return launch_bf16_grouped<true, true>(st, g, m, n, k, (int)lda, (int)ldb, (int)ldr, (int)ldc, ab, bb, workspace, workspace_bytes);
       return launch_bf16_grouped<true, false>(st, g, m, n, k, (int)lda, (int)ldb, (int)ldr, (int)ldc, ab, bb, workspace, workspace_bytes);
+    }
+  }
+  if (dtype == EMI_F32 && count >= 2 && !sum && K > 0 && M > 8 && (M + 31) / 32 <= 65535 && lda >= (trans_a ? M : K) &&
+      ldb >= (trans_b ? K : N) && ldc >= N && (trans_a || lda % 4 == 0) && (!trans_b || ldb % 4 == 0) &&
+      !(generic_splits(M, N, K) > 1 && (int64_t)count * ((M + 63) / 64) * ((N + 63) / 64) < 128)) {
+    bool ok = true, any_r = false, all_r = true;
+    for (int i = 0; i < count && ok; i++)
+      ok = (trans_a || (reinterpret_cast<uintptr_t>(A[i]) & 15) == 0) && (!trans_b || (reinterpret_cast<uintptr_t>(B[i]) & 15) == 0);
+    for (int i = 0; i < count; i++) {
+      const bool has = R != nullptr && R[i] != nullptr;
+      any_r = any_r || has;
+      all_r = all_r && has;
+    }
+    if (ok && (!any_r || (all_r && ldr >= N))) {
+      // the fp32 kernel, one grid plane per product
+      GemmGroup g{};
+      g.count = count;
+      for (int i = 0; i < count; i++) {
+        g.A[i] = static_cast<const uint16_t*>(A[i]);
+        g.B[i] = static_cast<const uint16_t*>(B[i]);
+        g.R[i] = any_r ? static_cast<const uint16_t*>(R[i]) : nullptr;
+        g.C[i] = static_cast<uint16_t*>(C[i]);
+      }
+      const dim3 grid((unsigned)((N + 31) / 32), (unsigned)((M + 31) / 32), (unsigned)count);
+#define EMI_F32_GROUPED(AKM, BKM)                                                                                          \
+  hipLaunchKernelGGL((gemm_f32_small_kernel<AKM, BKM, true>), grid, dim3(256), 0, st, static_cast<const float*>(A[0]),     \
+                     static_cast<const float*>(B[0]), static_cast<const float*>(nullptr), static_cast<float*>(C[0]), (int)M, \
+                     (int)N, (int)K, lda, ldb, ldr, ldc, g)
+      if (!trans_a && trans_b) EMI_F32_GROUPED(false, false);
+      else if (!trans_a && !trans_b) EMI_F32_GROUPED(false, true);
+      else if (trans_a && !trans_b) EMI_F32_GROUPED(true, true);
+      else EMI_F32_GROUPED(true, false);
+#undef EMI_F32_GROUPED
+      EMI_CHECK_LAUNCH("emi_gemm_grouped(fp32)");
+      return EMI_OK;
     }
   }
   // one product after the other; summed: each launch adds onto the result of the one before
