@@ -1166,8 +1166,11 @@ static int launch_bf16_grouped(hipStream_t st, const GemmGroup& g, int M, int N,
     configured = true;
   }
   const int big_tiles = ((M + 255) / 256) * ((N + 255) / 256);
-  if (!g.sum && (int64_t)big_tiles * g.count >= 192) {
-    // enough 256x256 tiles over the whole group to fill the chip: the ping-pong kernel, product-major
+  const int64_t group_tiles = (int64_t)big_tiles * g.count, rounds = (group_tiles + 255) / 256;
+  if (!g.sum && group_tiles >= 192 && (4 * group_tiles >= 3 * rounds * 256 || K >= 4096)) {
+    // enough 256x256 tiles over the whole group to fill the chip: the ping-pong kernel, product-major.  With a short
+    // contraction a last round that leaves most CUs idle costs more than the larger tile gains (3 x [8192, 768] x 768:
+    // 288 tiles, 48 us against 43 us on 128x128 tiles); with a long one it does not (12 x [768, 2048] x 8192: 351 vs 462 us).
     constexpr int smem_pp = 2 * 65536;
     static bool configured_pp = false;
     if (!configured_pp) {
