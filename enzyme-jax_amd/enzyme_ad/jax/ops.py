@@ -438,7 +438,21 @@ _transposed = {}      # (data_ptr, shape) -> a^T, valid for the duration of one 
 
 
 def _transpose_shared(a):
-    """a^T, computed once per reverse pass however many adjoint GEMMs read it."""
+    """a^T, computed once per reverse pass however many adjoint GEMMs read it.  A slice of a stacked per-layer
+    weight takes its transpose from one batched transpose of the whole stack (one launch for all layers)."""
+    st = getattr(a, "_emi_stack", None)
+    if st is not None and st[0].dim() == 3 and st[0].is_contiguous():
+        w, i = st
+        skey = ("stack", w.data_ptr(), tuple(w.shape), w.dtype)
+        hit = _transposed.get(skey)
+        if hit is None:
+            L_, rows, cols = w.shape
+            out = torch.empty((L_, cols, rows), dtype=w.dtype, device=w.device)
+            i64 = lambda v: (ctypes.c_int64 * len(v))(*v)
+            N.check(N.lib().emi_strided_copy(_stream(), _p(w), _p(out), 3, i64([L_, cols, rows]), i64([rows * cols, 1, cols]), 0,
+                                             i64([rows * cols, rows, 1]), 0, w.element_size()))
+            hit = _transposed[skey] = (out, w)
+        return hit[0][i]
     key = (a.data_ptr(), tuple(a.shape), a.dtype)
     hit = _transposed.get(key)
     if hit is None:
