@@ -188,7 +188,25 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const T* __restrict__ 
       }
     }
   }
-  float* prow = partial + ((int64_t)blockIdx.x * RPB + rib) * dim;
+  if constexpr (RPB > 1) {
+    // the rows-in-block of a narrow-row block add their partial sums in index order: one partial row per block
+    __shared__ float comb[(RPB - 1) * TPR * NCH * 8];
+    if (rib > 0) {
+#pragma unroll
+      for (int j = 0; j < NCH; j++)
+#pragma unroll
+        for (int e = 0; e < 8; e++) comb[(((rib - 1) * NCH + j) * 8 + e) * TPR + tir] = acc[j][e];
+    }
+    __syncthreads();
+    if (rib > 0) return;
+#pragma unroll
+    for (int r = 0; r < RPB - 1; r++)
+#pragma unroll
+      for (int j = 0; j < NCH; j++)
+#pragma unroll
+        for (int e = 0; e < 8; e++) acc[j][e] += comb[((r * NCH + j) * 8 + e) * TPR + tir];
+  }
+  float* prow = partial + (int64_t)blockIdx.x * dim;
 #pragma unroll
   for (int j = 0; j < NCH; j++) {
     const int c = tir + j * TPR;
@@ -551,7 +569,7 @@ static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t
 static inline unsigned blocks_for(int64_t n, int per) { return (unsigned)((n + per - 1) / per); }
 
 // grid used by the RMSNorm adjoint; the workspace holds one fp32 partial row
-// of dgamma per (block, row-in-block).
+// of dgamma per block.
 static inline void rms_bwd_shape(int64_t rows, int64_t dim, int* tpr, int* nch, int64_t* grid, int64_t* nparts) {
   if ((dim & 7) == 0 && dim <= 8192) {
     const int64_t chunks = dim >> 3;
@@ -565,7 +583,7 @@ static inline void rms_bwd_shape(int64_t rows, int64_t dim, int* tpr, int* nch, 
     // 128 left half of the CUs idle on the 768-wide model.)
     const int64_t cap = 512;
     *grid = groups < cap ? (groups > 0 ? groups : 1) : cap;
-    *nparts = *grid * rpb;
+    *nparts = *grid;
   } else {
     *tpr = 0;
     *nch = 0;
