@@ -98,37 +98,39 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const T* __restrict__ 
                                                           const T* __restrict__ dy, const T* dx_add, T* dx,
                                                           float* __restrict__ partial, int64_t rows, int dim,
                                                           float eps) {
-  constexpr int RPB = 256 / TPR;
+  // NCH groups of 8 elements per thread, held as 16-byte pieces (8 bf16 or 4 floats) so that consecutive lanes cover
+  // consecutive 16 bytes (the access shape of the streaming loads and stores)
+  constexpr int RPB = 256 / TPR, N = Chunk<T>::N, NC = NCH * 8 / N;
   __shared__ float red[2][4][2 * NR];
   const int tir = threadIdx.x % TPR;
   const int rib = threadIdx.x / TPR;
-  const int nchunk = dim >> 3;
-  float gm[NCH][8], acc[NCH][8];
+  const int nchunk = dim / N;
+  float gm[NC][N], acc[NC][N];
 #pragma unroll
-  for (int j = 0; j < NCH; j++) {
+  for (int j = 0; j < NC; j++) {
     const int c = tir + j * TPR;
 #pragma unroll
-    for (int e = 0; e < 8; e++) acc[j][e] = 0.f, gm[j][e] = 0.f;
-    if (c < nchunk) Vec8<T>::load(gamma + c * 8, gm[j]);
+    for (int e = 0; e < N; e++) acc[j][e] = 0.f, gm[j][e] = 0.f;
+    if (c < nchunk) ChunkCached<T>::load(gamma + c * N, gm[j]);
   }
   const int64_t nstep = (rows + RPB * NR - 1) / (RPB * NR);   // steps of RPB*NR rows
   // Steps are software pipelined: the loads of the next step are issued before the
   // reduction (shuffles, LDS, barrier) of the current one, which keeps twice the
   // bytes in flight per block.
-  typename Vec8<T>::Raw xn[NR][NCH], gn[NR][NCH];      // kept in storage format to save registers
+  typename Chunk<T>::Raw xn[NR][NC], gn[NR][NC];      // kept in storage format to save registers
   auto load_step = [&](int64_t sg) {
 #pragma unroll
     for (int u = 0; u < NR; u++) {
       const int64_t row = (sg * NR + u) * RPB + rib;
 #pragma unroll
-      for (int j = 0; j < NCH; j++) {
+      for (int j = 0; j < NC; j++) {
         const int c = tir + j * TPR;
         if (sg < nstep && row < rows && c < nchunk) {
-          xn[u][j] = Vec8<T>::load_raw(x + row * dim + c * 8);
-          gn[u][j] = Vec8<T>::load_raw(dy + row * dim + c * 8);
+          xn[u][j] = Chunk<T>::load_raw(x + row * dim + c * N);
+          gn[u][j] = Chunk<T>::load_raw(dy + row * dim + c * N);
         } else {
-          xn[u][j] = Vec8<T>::zero_raw();
-          gn[u][j] = Vec8<T>::zero_raw();
+          xn[u][j] = typename Chunk<T>::Raw{};
+          gn[u][j] = typename Chunk<T>::Raw{};
         }
       }
     }
@@ -136,20 +138,20 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const T* __restrict__ 
   load_step(blockIdx.x);
   int it = 0;
   for (int64_t sg = blockIdx.x; sg < nstep; sg += gridDim.x, ++it) {
-    typename Vec8<T>::Raw xc[NR][NCH], gc[NR][NCH];
+    typename Chunk<T>::Raw xc[NR][NC], gc[NR][NC];
     float red_v[2 * NR];
 #pragma unroll
     for (int u = 0; u < NR; u++) {
       float ss = 0.f, gx = 0.f;
 #pragma unroll
-      for (int j = 0; j < NCH; j++) {
+      for (int j = 0; j < NC; j++) {
         xc[u][j] = xn[u][j];
         gc[u][j] = gn[u][j];
-        float xv[8], gv[8];
-        Vec8<T>::unpack(xc[u][j], xv);
-        Vec8<T>::unpack(gc[u][j], gv);
+        float xv[N], gv[N];
+        Chunk<T>::unpack(xc[u][j], xv);
+        Chunk<T>::unpack(gc[u][j], gv);
 #pragma unroll
-        for (int e = 0; e < 8; e++) {
+        for (int e = 0; e < N; e++) {
           ss += xv[e] * xv[e];
           gx += gv[e] * gm[j][e] * xv[e];
         }
@@ -166,51 +168,55 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const T* __restrict__ 
       const float r = 1.0f / sqrtf(red_v[2 * u] / (float)dim + eps);
       const float coef = r * r * r * (red_v[2 * u + 1] / (float)dim);
 #pragma unroll
-      for (int j = 0; j < NCH; j++) {
+      for (int j = 0; j < NC; j++) {
         const int c = tir + j * TPR;
         if (active && c < nchunk) {
-          float xv[8], gv[8], o[8];
-          Vec8<T>::unpack(xc[u][j], xv);
-          Vec8<T>::unpack(gc[u][j], gv);
+          float xv[N], gv[N], o[N];
+          Chunk<T>::unpack(xc[u][j], xv);
+          Chunk<T>::unpack(gc[u][j], gv);
 #pragma unroll
-          for (int e = 0; e < 8; e++) {
+          for (int e = 0; e < N; e++) {
             acc[j][e] += gv[e] * xv[e] * r;
             o[e] = r * gv[e] * gm[j][e] - xv[e] * coef;
           }
           if (dx_add != nullptr) {
-            float a[8];
-            Vec8<T>::load(dx_add + row * dim + c * 8, a);
+            float a[N];
+            Chunk<T>::load(dx_add + row * dim + c * N, a);
 #pragma unroll
-            for (int e = 0; e < 8; e++) o[e] += a[e];
+            for (int e = 0; e < N; e++) o[e] += a[e];
           }
-          Vec8<T>::store(dx + row * dim + c * 8, o);
+          Chunk<T>::store(dx + row * dim + c * N, o);
         }
       }
     }
   }
   if constexpr (RPB > 1) {
     // the rows-in-block of a narrow-row block add their partial sums in index order: one partial row per block
-    __shared__ float comb[(RPB - 1) * TPR * NCH * 8];
+    __shared__ float comb[(RPB - 1) * TPR * NC * N];
     if (rib > 0) {
 #pragma unroll
-      for (int j = 0; j < NCH; j++)
+      for (int j = 0; j < NC; j++)
 #pragma unroll
-        for (int e = 0; e < 8; e++) comb[(((rib - 1) * NCH + j) * 8 + e) * TPR + tir] = acc[j][e];
+        for (int e = 0; e < N; e++) comb[(((rib - 1) * NC + j) * N + e) * TPR + tir] = acc[j][e];
     }
     __syncthreads();
     if (rib > 0) return;
 #pragma unroll
     for (int r = 0; r < RPB - 1; r++)
 #pragma unroll
-      for (int j = 0; j < NCH; j++)
+      for (int j = 0; j < NC; j++)
 #pragma unroll
-        for (int e = 0; e < 8; e++) acc[j][e] += comb[((r * NCH + j) * 8 + e) * TPR + tir];
+        for (int e = 0; e < N; e++) acc[j][e] += comb[((r * NC + j) * N + e) * TPR + tir];
   }
   float* prow = partial + (int64_t)blockIdx.x * dim;
 #pragma unroll
-  for (int j = 0; j < NCH; j++) {
+  for (int j = 0; j < NC; j++) {
     const int c = tir + j * TPR;
-    if (c < nchunk) Vec8<float>::store(prow + c * 8, acc[j]);
+    if (c < nchunk) {
+#pragma unroll
+      for (int q = 0; q < N / 4; q++)
+        *reinterpret_cast<float4*>(prow + c * N + 4 * q) = make_float4(acc[j][4 * q], acc[j][4 * q + 1], acc[j][4 * q + 2], acc[j][4 * q + 3]);
+    }
   }
 }
 
