@@ -358,7 +358,14 @@ def reverse_function(func, name=None, arg_active=None, ret_active=None):
             # (reference rule: HLODerivatives.td:1022-1046): the emi_embedding_bwd target; the indices are inactive
             check_gather(op.attrs, T[xs[0]], T[xs[1]], T[r])
             idx = b.emit("reshape", [xs[1]], {}, TensorType(T[xs[1]].shape[:-1], T[xs[1]].dtype))
-            accum(xs[0], b.emit("custom_call", [idx, c], {"target": "emi_embedding_bwd", "config": {}}, T[xs[0]]))
+            from . import _native as N
+            tt = T[xs[0]]
+            nbytes = int(N.lib().emi_embedding_bwd_workspace_bytes(tt.shape[0], tt.shape[1], 16 if tt.dtype == "bf16" else 11))
+            if nbytes:         # bf16: the rows are summed in an fp32 table that the handler takes as an extra result
+                dt_, _ = b.custom_call("emi_embedding_bwd", [idx, c], {}, [tt, TensorType((nbytes,), "i8")])
+            else:
+                dt_, = b.custom_call("emi_embedding_bwd", [idx, c], {}, [tt])
+            accum(xs[0], dt_)
         elif n == "custom_call":
             _reverse_custom_call(b, op, cs, accum)
         elif n == "call":

@@ -102,3 +102,52 @@ def test_layer_modules_through_the_ffi_handlers():
         assert len(calls) == low.count("stablehlo.custom_call") and set(calls) >= {"emi_gemm", "emi_attn_fwd", "emi_rope"}, name
         for a, b in zip(got, want):
             assert torch.equal(a, b) if name == "primal" else _close(a, b, 2e-2), name
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+def test_cross_entropy_and_gather_modules_through_the_ffi_handlers(dt):
+    """The printed programs of a traced mean softmax cross-entropy and of a row lookup (the reference's gather.mlir
+    input), primal, reverse and forward, with every custom call served by the library's FFI handler: the s32 operands
+    (targets, indices), the f32 loss / log-sum-exp results and the scatter-add's table-shaped result are laid out as
+    the handlers expect."""
+    import json
+    import os
+    from enzyme_ad.jax import hlo_call, stablehlo_ad
+    from enzyme_ad.jax import optimize_module
+    from test_stablehlo_frontend import traced_cross_entropy_text
+
+    rng = np.random.Generator(np.random.PCG64(12))
+    tdt = torch.float32 if dt == "f32" else torch.bfloat16
+    # cross-entropy
+    rows, V = (6, 9), 520
+    text = traced_cross_entropy_text(rows, V, dt=dt)
+    z = dev(2.0 * rng.standard_normal(rows + (V,)), dt)[0]
+    tz = dev(rng.standard_normal(rows + (V,)), dt)[0]
+    tgt = torch.from_numpy(rng.integers(0, V, size=rows).astype(np.int32)).cuda()
+    one = torch.ones((), device="cuda", dtype=tdt)
+    programs = (("primal", optimize_module(text), [z, tgt], {"emi_cross_entropy_fwd"}),
+                ("reverse", stablehlo_ad.reverse_module_text(text), [z, tgt, one], {"emi_cross_entropy_fwd", "emi_cross_entropy_bwd"}),
+                ("forward", stablehlo_ad.forward_module_text(text), [z, tz, tgt], {"emi_cross_entropy_fwd", "emi_cross_entropy_jvp"}))
+    for name, low, ins, targets in programs:
+        exe, calls = _ffi_executable(low)
+        got = exe.run(ins)
+        torch.cuda.synchronize()
+        want = hlo_call(*ins, source=low)
+        assert set(calls) == targets and len(calls) == low.count("stablehlo.custom_call"), (name, calls)
+        for a, b in zip(got, want):
+            assert torch.equal(a, b), name
+    # gather
+    fixture = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "lit_primal_functions.json")))
+    (fn_text,) = fixture["gather.mlir"]
+    gtext = "module {\n" + fn_text.replace("f32", "f32" if dt == "f32" else "bf16") + "\n}"
+    table = dev(rng.standard_normal((64, 3)), dt)[0]
+    ttab = dev(rng.standard_normal((64, 3)), dt)[0]
+    c = dev(rng.standard_normal((45, 3)), dt)[0]
+    idx = torch.from_numpy(rng.integers(0, 64, size=(45, 1)).astype(np.int32)).cuda()
+    rev = stablehlo_ad.reverse_module_text(gtext, arg_active=[True, False])
+    exe, calls = _ffi_executable(rev)
+    got = exe.run([table, idx, c])
+    torch.cuda.synchronize()
+    want = hlo_call(table, idx, c, source=rev)
+    assert "emi_embedding_bwd" in calls
+    assert _close(got[0], want[0], 1e-6 if dt == "f32" else 2e-2)          # fp32 atomics: the order of repeated rows differs
