@@ -82,6 +82,27 @@ __device__ __forceinline__ void add_cols(const float* __restrict__ head, int64_t
   }
 }
 
+// The two halves of add_cols, for callers that issue the loads well before the weights exist.
+template <int NT>
+__device__ __forceinline__ void load_cols(const float* __restrict__ head, int64_t ss, int row0, int last, int lane,
+                                          float (&x)[4][NT]) {
+#pragma unroll
+  for (int t = 0; t < 4; t++) {
+    int r = row0 + 4 * (lane >> 4) + t;
+    r = r < last ? r : last;
+    const float* p = head + (int64_t)r * ss + NT * (lane & 15);
+#pragma unroll
+    for (int n = 0; n < NT; n++) x[t][n] = p[n];
+  }
+}
+template <int NT>
+__device__ __forceinline__ void mma_cols(const float (&x)[4][NT], const f32q_t w, f32q_t (&acc)[NT]) {
+#pragma unroll
+  for (int t = 0; t < 4; t++)
+#pragma unroll
+    for (int n = 0; n < NT; n++) acc[n] = mfma_f32(x[t][n], w[t], acc[n]);
+}
+
 template <int NT>
 __device__ __forceinline__ void store_cols(float* __restrict__ row, int lane, const f32q_t (&acc)[NT], float mul) {
 #pragma unroll
@@ -119,16 +140,31 @@ __global__ __launch_bounds__(64) void attn_fwd_f32_kernel(const float* __restric
   f32q_t acc[NT];
 #pragma unroll
   for (int n = 0; n < NT; n++) acc[n] = f32q_t{0.f, 0.f, 0.f, 0.f};
+  constexpr bool AHEAD = NT <= 4;      // head_dim <= 64: all K and V operands of a 64-key step fit in registers, so
+                                       // their loads are issued together and the step waits for memory once
   for (int k0 = 0; k0 < nkeys; k0 += 64) {
     f32q_t s[4];
     float mx = kMasked;
+    float kfa[AHEAD ? 4 : 1][NT][4], vxa[AHEAD ? 4 : 1][4][NT];
+    if constexpr (AHEAD) {
+#pragma unroll
+      for (int kt = 0; kt < 4; kt++)
+        if (k0 + 16 * kt < nkeys) load_rows<NT>(k + base, sh.ss, k0 + 16 * kt, last, lane, kfa[kt]);
+#pragma unroll
+      for (int kt = 0; kt < 4; kt++)
+        if (k0 + 16 * kt < nkeys) load_cols<NT>(v + base, sh.ss, k0 + 16 * kt, last, lane, vxa[kt]);
+    }
 #pragma unroll
     for (int kt = 0; kt < 4; kt++) {
       const int kb = k0 + 16 * kt;
       if (kb < nkeys) {
-        float kf[NT][4];
-        load_rows<NT>(k + base, sh.ss, kb, last, lane, kf);
-        s[kt] = rows_dot<NT>(kf, qf);
+        if constexpr (AHEAD) {
+          s[kt] = rows_dot<NT>(kfa[kt], qf);
+        } else {
+          float kf[NT][4];
+          load_rows<NT>(k + base, sh.ss, kb, last, lane, kf);
+          s[kt] = rows_dot<NT>(kf, qf);
+        }
       } else {
         s[kt] = f32q_t{0.f, 0.f, 0.f, 0.f};
       }
@@ -156,7 +192,10 @@ __global__ __launch_bounds__(64) void attn_fwd_f32_kernel(const float* __restric
     for (int n = 0; n < NT; n++) acc[n] *= alpha;
 #pragma unroll
     for (int kt = 0; kt < 4; kt++)
-      if (k0 + 16 * kt < nkeys) add_cols<NT>(v + base, sh.ss, k0 + 16 * kt, last, lane, s[kt], acc);
+      if (k0 + 16 * kt < nkeys) {
+        if constexpr (AHEAD) mma_cols<NT>(vxa[kt], s[kt], acc);
+        else add_cols<NT>(v + base, sh.ss, k0 + 16 * kt, last, lane, s[kt], acc);
+      }
     m = m_new;
   }
   lsum = groups_sum(lsum);
@@ -189,9 +228,10 @@ __global__ __launch_bounds__(64) void attn_bwd_dq_f32_kernel(const float* __rest
 #pragma unroll
   for (int n = 0; n < NT; n++) acc[n] = f32q_t{0.f, 0.f, 0.f, 0.f};
   for (int kb = 0; kb < nkeys; kb += 16) {
-    float kf[NT][4], vf[NT][4];
+    float kf[NT][4], vf[NT][4], kx[4][NT];
     load_rows<NT>(k + base, sh.ss, kb, last, lane, kf);
     load_rows<NT>(v + base, sh.ss, kb, last, lane, vf);
+    load_cols<NT>(k + base, sh.ss, kb, last, lane, kx);        // for dQ += dS . K below: issued with the others
     f32q_t s = rows_dot<NT>(kf, qf);
     const f32q_t dp = rows_dot<NT>(vf, dof);
 #pragma unroll
@@ -201,7 +241,7 @@ __global__ __launch_bounds__(64) void attn_bwd_dq_f32_kernel(const float* __rest
       const float p = valid ? expf(s[r] * scale - L) : 0.f;
       s[r] = p * (dp[r] - dl) * scale;
     }
-    add_cols<NT>(k + base, sh.ss, kb, last, lane, s, acc);
+    mma_cols<NT>(kx, s, acc);
   }
   if (myq < sh.seq) store_cols<NT>(dq + base + (int64_t)myq * sh.ss, lane, acc, 1.f);
 }
@@ -228,9 +268,11 @@ __global__ __launch_bounds__(64) void attn_bwd_dkv_f32_kernel(const float* __res
 #pragma unroll
   for (int n = 0; n < NT; n++) acck[n] = accv[n] = f32q_t{0.f, 0.f, 0.f, 0.f};
   for (int qb = causal ? key0 : 0; qb < sh.seq; qb += 16) {
-    float qf[NT][4], dof[NT][4];
+    float qf[NT][4], dof[NT][4], qx[4][NT], dox[4][NT];
     load_rows<NT>(q + base, sh.ss, qb, last, lane, qf);
     load_rows<NT>(d_o + base, sh.ss, qb, last, lane, dof);
+    load_cols<NT>(d_o + base, sh.ss, qb, last, lane, dox);    // for dV += P^T . dO and dK += dS^T . Q below
+    load_cols<NT>(q + base, sh.ss, qb, last, lane, qx);
     f32q_t s = rows_dot<NT>(qf, kf);               // register r: query qb + 4 G + r, key mykey
     f32q_t dp = rows_dot<NT>(dof, vf);
 #pragma unroll
@@ -242,8 +284,8 @@ __global__ __launch_bounds__(64) void attn_bwd_dkv_f32_kernel(const float* __res
       s[r] = p;
       dp[r] = p * (dp[r] - drow[qc]) * scale;
     }
-    add_cols<NT>(d_o + base, sh.ss, qb, last, lane, s, accv);
-    add_cols<NT>(q + base, sh.ss, qb, last, lane, dp, acck);
+    mma_cols<NT>(dox, s, accv);
+    mma_cols<NT>(qx, dp, acck);
   }
   if (mykey < sh.seq) {
     store_cols<NT>(dk + base + (int64_t)mykey * sh.ss, lane, acck, 1.f);
