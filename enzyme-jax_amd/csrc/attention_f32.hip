@@ -227,21 +227,32 @@ __global__ __launch_bounds__(64) void attn_bwd_dq_f32_kernel(const float* __rest
   f32q_t acc[NT];
 #pragma unroll
   for (int n = 0; n < NT; n++) acc[n] = f32q_t{0.f, 0.f, 0.f, 0.f};
-  for (int kb = 0; kb < nkeys; kb += 16) {
-    float kf[NT][4], vf[NT][4], kx[4][NT];
-    load_rows<NT>(k + base, sh.ss, kb, last, lane, kf);
-    load_rows<NT>(v + base, sh.ss, kb, last, lane, vf);
-    load_cols<NT>(k + base, sh.ss, kb, last, lane, kx);        // for dQ += dS . K below: issued with the others
-    f32q_t s = rows_dot<NT>(kf, qf);
-    const f32q_t dp = rows_dot<NT>(vf, dof);
+  // U key tiles per step, all their operands requested before the first product (one wait for memory per step)
+  constexpr int U = NT <= 3 ? 4 : (NT <= 4 ? 2 : 1);      // (166 registers at NT = 4: three wavefronts per SIMD)
+  for (int kb0 = 0; kb0 < nkeys; kb0 += 16 * U) {
+    float kf[U][NT][4], vf[U][NT][4], kx[U][4][NT];
 #pragma unroll
-    for (int r = 0; r < 4; r++) {
-      const int key = kb + 4 * G + r;
-      const bool valid = key < nkeys && (!causal || key <= myq);
-      const float p = valid ? expf(s[r] * scale - L) : 0.f;
-      s[r] = p * (dp[r] - dl) * scale;
+    for (int u = 0; u < U; u++)
+      if (kb0 + 16 * u < nkeys) {
+        load_rows<NT>(k + base, sh.ss, kb0 + 16 * u, last, lane, kf[u]);
+        load_rows<NT>(v + base, sh.ss, kb0 + 16 * u, last, lane, vf[u]);
+        load_cols<NT>(k + base, sh.ss, kb0 + 16 * u, last, lane, kx[u]);        // for dQ += dS . K
+      }
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const int kb = kb0 + 16 * u;
+      if (kb >= nkeys) break;
+      f32q_t s = rows_dot<NT>(kf[u], qf);
+      const f32q_t dp = rows_dot<NT>(vf[u], dof);
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const int key = kb + 4 * G + r;
+        const bool valid = key < nkeys && (!causal || key <= myq);
+        const float p = valid ? expf(s[r] * scale - L) : 0.f;
+        s[r] = p * (dp[r] - dl) * scale;
+      }
+      mma_cols<NT>(kx[u], s, acc);
     }
-    mma_cols<NT>(kx, s, acc);
   }
   if (myq < sh.seq) store_cols<NT>(dq + base + (int64_t)myq * sh.ss, lane, acc, 1.f);
 }
@@ -267,25 +278,43 @@ __global__ __launch_bounds__(64) void attn_bwd_dkv_f32_kernel(const float* __res
   f32q_t acck[NT], accv[NT];
 #pragma unroll
   for (int n = 0; n < NT; n++) acck[n] = accv[n] = f32q_t{0.f, 0.f, 0.f, 0.f};
-  for (int qb = causal ? key0 : 0; qb < sh.seq; qb += 16) {
-    float qf[NT][4], dof[NT][4], qx[4][NT], dox[4][NT];
-    load_rows<NT>(q + base, sh.ss, qb, last, lane, qf);
-    load_rows<NT>(d_o + base, sh.ss, qb, last, lane, dof);
-    load_cols<NT>(d_o + base, sh.ss, qb, last, lane, dox);    // for dV += P^T . dO and dK += dS^T . Q below
-    load_cols<NT>(q + base, sh.ss, qb, last, lane, qx);
-    f32q_t s = rows_dot<NT>(qf, kf);               // register r: query qb + 4 G + r, key mykey
-    f32q_t dp = rows_dot<NT>(dof, vf);
+  // U query tiles per step, operands (and the rows' lse / delta) requested together; two tiles only while the
+  // registers allow three wavefronts per SIMD to stay resident
+  constexpr int U = NT <= 3 ? 2 : 1;
+  for (int qb0 = causal ? key0 : 0; qb0 < sh.seq; qb0 += 16 * U) {
+    float qf[U][NT][4], dof[U][NT][4], qx[U][4][NT], dox[U][4][NT], lq[U][4], dq_[U][4];
 #pragma unroll
-    for (int r = 0; r < 4; r++) {
-      const int qi = qb + 4 * G + r;
-      const int qc = qi < last ? qi : last;
-      const bool valid = qi < sh.seq && (!causal || mykey <= qi);
-      const float p = valid ? expf(s[r] * scale - lrow[qc]) : 0.f;
-      s[r] = p;
-      dp[r] = p * (dp[r] - drow[qc]) * scale;
+    for (int u = 0; u < U; u++)
+      if (qb0 + 16 * u < sh.seq) {
+        load_rows<NT>(q + base, sh.ss, qb0 + 16 * u, last, lane, qf[u]);
+        load_rows<NT>(d_o + base, sh.ss, qb0 + 16 * u, last, lane, dof[u]);
+        load_cols<NT>(d_o + base, sh.ss, qb0 + 16 * u, last, lane, dox[u]);    // for dV += P^T . dO
+        load_cols<NT>(q + base, sh.ss, qb0 + 16 * u, last, lane, qx[u]);       // for dK += dS^T . Q
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          const int qi = qb0 + 16 * u + 4 * G + r;
+          const int qc = qi < last ? qi : last;
+          lq[u][r] = lrow[qc];
+          dq_[u][r] = drow[qc];
+        }
+      }
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const int qb = qb0 + 16 * u;
+      if (qb >= sh.seq) break;
+      f32q_t s = rows_dot<NT>(qf[u], kf);               // register r: query qb + 4 G + r, key mykey
+      f32q_t dp = rows_dot<NT>(dof[u], vf);
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const int qi = qb + 4 * G + r;
+        const bool valid = qi < sh.seq && (!causal || mykey <= qi);
+        const float p = valid ? expf(s[r] * scale - lq[u][r]) : 0.f;
+        s[r] = p;
+        dp[r] = p * (dp[r] - dq_[u][r]) * scale;
+      }
+      mma_cols<NT>(dox[u], s, accv);
+      mma_cols<NT>(qx[u], dp, acck);
     }
-    mma_cols<NT>(dox, s, accv);
-    mma_cols<NT>(qx, dp, acck);
   }
   if (mykey < sh.seq) {
     store_cols<NT>(dk + base + (int64_t)mykey * sh.ss, lane, acck, 1.f);
