@@ -991,13 +991,15 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const T* __restrict__
 // ---------------------------------------------------------------------------
 // GROUPED: blockIdx.z picks one of grp.count independent products of one shape (GemmGroup with sum == 0, its pointers
 // read as float).
-template <bool A_KMAJOR, bool B_KMAJOR, bool GROUPED = false>
-__global__ __launch_bounds__(256) void gemm_f32_small_kernel(const float* __restrict__ A, const float* __restrict__ B,
-                                                             const float* R, float* C, int M, int N, int K, int64_t lda,
-                                                             int64_t ldb, int64_t ldr, int64_t ldc,
-                                                             std::conditional_t<GROUPED, GemmGroup, NoGroup> grp) {
-  constexpr int U = 4;                                   // 8-wide chunks in flight per step
-  __shared__ float red[3][16][64];
+// NW wavefronts share K; U 8-wide chunks are in flight per step.  ONCE: a wavefront's share of K is at most U chunks
+// (K <= 96 NW), so everything is requested up front and the block waits for memory once: a short contraction is a
+// chain of load latencies otherwise (256 x 288 x 288: 10 us in three steps).
+template <bool A_KMAJOR, bool B_KMAJOR, bool GROUPED = false, int NW = 4, int U = 4, bool ONCE = false>
+__global__ __launch_bounds__(NW * 64) void gemm_f32_small_kernel(const float* __restrict__ A, const float* __restrict__ B,
+                                                                 const float* R, float* C, int M, int N, int K, int64_t lda,
+                                                                 int64_t ldb, int64_t ldr, int64_t ldc,
+                                                                 std::conditional_t<GROUPED, GemmGroup, NoGroup> grp) {
+  __shared__ float red[NW - 1][16][64];
   if constexpr (GROUPED) {
     A = reinterpret_cast<const float*>(grp.A[blockIdx.z]);
     B = reinterpret_cast<const float*>(grp.B[blockIdx.z]);
@@ -1008,7 +1010,7 @@ __global__ __launch_bounds__(256) void gemm_f32_small_kernel(const float* __rest
   const int i = lane & 31, g = lane >> 5;
   const int m0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
   const int mi = m0 + i < M ? m0 + i : M - 1, ni = n0 + i < N ? n0 + i : N - 1;      // clamped: those results are not stored
-  const int kper = ((K + 31) / 32) * 8;                  // a quarter of K, rounded up to whole chunks
+  const int kper = ((K + 8 * NW - 1) / (8 * NW)) * 8;    // this wavefront's share of K, rounded up to whole chunks
   const int ks = wave * kper, ke = ks + kper < K ? ks + kper : K;
   const float* pa = A_KMAJOR ? A + mi : A + (int64_t)mi * lda;
   const float* pb = B_KMAJOR ? B + ni : B + (int64_t)ni * ldb;
@@ -1031,7 +1033,7 @@ __global__ __launch_bounds__(256) void gemm_f32_small_kernel(const float* __rest
   f32x16_t acc;
 #pragma unroll
   for (int r = 0; r < 16; r++) acc[r] = 0.f;
-  float a[U][4], b[U][4], an[U][4], bn[U][4];
+  float a[U][4], b[U][4];
   auto load = [&](int k0, float (&fa)[U][4], float (&fb)[U][4]) {
 #pragma unroll
     for (int u = 0; u < U; u++) {
@@ -1040,18 +1042,28 @@ __global__ __launch_bounds__(256) void gemm_f32_small_kernel(const float* __rest
     }
   };
   if (ks < ke) load(ks, a, b);
-  for (int k0 = ks; k0 < ke; k0 += 8 * U) {
-    const bool more = k0 + 8 * U < ke;
-    if (more) load(k0 + 8 * U, an, bn);            // in flight while this step is multiplied
-#pragma unroll
-    for (int u = 0; u < U; u++)
-#pragma unroll
-      for (int t = 0; t < 4; t++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u][t], b[u][t], acc, 0, 0, 0);
-    if (more) {
+  if constexpr (ONCE) {
+    if (ks < ke) {
 #pragma unroll
       for (int u = 0; u < U; u++)
 #pragma unroll
-        for (int t = 0; t < 4; t++) { a[u][t] = an[u][t]; b[u][t] = bn[u][t]; }
+        for (int t = 0; t < 4; t++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u][t], b[u][t], acc, 0, 0, 0);
+    }
+  } else {
+    float an[U][4], bn[U][4];
+    for (int k0 = ks; k0 < ke; k0 += 8 * U) {
+      const bool more = k0 + 8 * U < ke;
+      if (more) load(k0 + 8 * U, an, bn);            // in flight while this step is multiplied
+#pragma unroll
+      for (int u = 0; u < U; u++)
+#pragma unroll
+        for (int t = 0; t < 4; t++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u][t], b[u][t], acc, 0, 0, 0);
+      if (more) {
+#pragma unroll
+        for (int u = 0; u < U; u++)
+#pragma unroll
+          for (int t = 0; t < 4; t++) { a[u][t] = an[u][t]; b[u][t] = bn[u][t]; }
+      }
     }
   }
   if (wave > 0) {
@@ -1061,7 +1073,7 @@ __global__ __launch_bounds__(256) void gemm_f32_small_kernel(const float* __rest
   __syncthreads();
   if (wave > 0) return;
 #pragma unroll
-  for (int w = 0; w < 3; w++)
+  for (int w = 0; w < NW - 1; w++)
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[r] += red[w][r][lane];
   // register r of lane l: row 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32
@@ -1367,15 +1379,25 @@ extern "C" int emi_gemm_ws(emi_stream_t stream, const void* A, const void* B, co
       (trans_a || ((reinterpret_cast<uintptr_t>(A) & 15) == 0 && lda % 4 == 0)) &&
       (!trans_b || ((reinterpret_cast<uintptr_t>(B) & 15) == 0 && ldb % 4 == 0))) {
     const dim3 grid((unsigned)((N + 31) / 32), (unsigned)((M + 31) / 32));
-#define EMI_F32_SMALL(AKM, BKM)                                                                                       \
-  hipLaunchKernelGGL((gemm_f32_small_kernel<AKM, BKM>), grid, dim3(256), 0, st, static_cast<const float*>(A),         \
-                     static_cast<const float*>(B), static_cast<const float*>(R), static_cast<float*>(C), (int)M, (int)N, \
-                     (int)K, lda, ldb, ldr, ldc, NoGroup{})
+#define EMI_F32_SMALL_V(AKM, BKM, NWV, UV, ONCEV)                                                                          \
+  hipLaunchKernelGGL((gemm_f32_small_kernel<AKM, BKM, false, NWV, UV, ONCEV>), grid, dim3(NWV * 64), 0, st,                \
+                     static_cast<const float*>(A), static_cast<const float*>(B), static_cast<const float*>(R),             \
+                     static_cast<float*>(C), (int)M, (int)N, (int)K, lda, ldb, ldr, ldc, NoGroup{})
+    // few blocks: latency decides, everything is requested at once; many blocks: the stepped form, whose smaller
+    // register footprint keeps more wavefronts resident
+    const bool few = (int64_t)grid.x * grid.y <= 1024;
+#define EMI_F32_SMALL(AKM, BKM)                                            \
+  do {                                                                     \
+    if (few && K <= 384) EMI_F32_SMALL_V(AKM, BKM, 4, 12, true);           \
+    else if (few && K <= 768) EMI_F32_SMALL_V(AKM, BKM, 8, 12, true);      \
+    else EMI_F32_SMALL_V(AKM, BKM, 4, 4, false);                           \
+  } while (0)
     if (!trans_a && trans_b) EMI_F32_SMALL(false, false);
     else if (!trans_a && !trans_b) EMI_F32_SMALL(false, true);
     else if (trans_a && !trans_b) EMI_F32_SMALL(true, true);
     else EMI_F32_SMALL(true, false);
 #undef EMI_F32_SMALL
+#undef EMI_F32_SMALL_V
     EMI_CHECK_LAUNCH("emi_gemm(fp32 small)");
     return EMI_OK;
   }
@@ -1469,15 +1491,23 @@ extern "C" int emi_gemm_grouped(emi_stream_t stream, int count, const void* cons
         g.C[i] = static_cast<uint16_t*>(C[i]);
       }
       const dim3 grid((unsigned)((N + 31) / 32), (unsigned)((M + 31) / 32), (unsigned)count);
-#define EMI_F32_GROUPED(AKM, BKM)                                                                                          \
-  hipLaunchKernelGGL((gemm_f32_small_kernel<AKM, BKM, true>), grid, dim3(256), 0, st, static_cast<const float*>(A[0]),     \
-                     static_cast<const float*>(B[0]), static_cast<const float*>(nullptr), static_cast<float*>(C[0]), (int)M, \
-                     (int)N, (int)K, lda, ldb, ldr, ldc, g)
+#define EMI_F32_GROUPED_V(AKM, BKM, NWV, UV, ONCEV)                                                                        \
+  hipLaunchKernelGGL((gemm_f32_small_kernel<AKM, BKM, true, NWV, UV, ONCEV>), grid, dim3(NWV * 64), 0, st,                 \
+                     static_cast<const float*>(A[0]), static_cast<const float*>(B[0]), static_cast<const float*>(nullptr), \
+                     static_cast<float*>(C[0]), (int)M, (int)N, (int)K, lda, ldb, ldr, ldc, g)
+      const bool few = (int64_t)grid.x * grid.y * grid.z <= 1024;
+#define EMI_F32_GROUPED(AKM, BKM)                                          \
+  do {                                                                     \
+    if (few && K <= 384) EMI_F32_GROUPED_V(AKM, BKM, 4, 12, true);         \
+    else if (few && K <= 768) EMI_F32_GROUPED_V(AKM, BKM, 8, 12, true);    \
+    else EMI_F32_GROUPED_V(AKM, BKM, 4, 4, false);                         \
+  } while (0)
       if (!trans_a && trans_b) EMI_F32_GROUPED(false, false);
       else if (!trans_a && !trans_b) EMI_F32_GROUPED(false, true);
       else if (trans_a && !trans_b) EMI_F32_GROUPED(true, true);
       else EMI_F32_GROUPED(true, false);
 #undef EMI_F32_GROUPED
+#undef EMI_F32_GROUPED_V
       EMI_CHECK_LAUNCH("emi_gemm_grouped(fp32)");
       return EMI_OK;
     }
