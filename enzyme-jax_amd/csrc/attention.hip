@@ -345,6 +345,30 @@ __device__ __forceinline__ void load_rows_tile(__amdgpu_buffer_rsrc_t rsrc, EMI_
   }
 }
 
+// One of those loads on its own, for a kernel that spreads them between its MFMAs.  off[it] is the per-lane part
+// of load it's byte offset (tile row 0), computed once per kernel.  No bounds test: a row past the end of the
+// sequence lies past the end of the buffer descriptor (which ends with the last row of the head) and reads as zero.
+template <int D, int ROWS, int NW> struct TileLaneOffsets { uint32_t off[ROWS / (64 / (D / 8)) / NW]; };
+template <int D, int ROWS, int NW>
+__device__ __forceinline__ TileLaneOffsets<D, ROWS, NW> tile_lane_offsets(int wave, int lane, int64_t ss) {
+  constexpr int CPR = D / 8, RPL = 64 / CPR, NLOAD = ROWS / RPL / NW;
+  TileLaneOffsets<D, ROWS, NW> t;
+#pragma unroll
+  for (int it = 0; it < NLOAD; it++) {
+    const int r = (it * NW + wave) * RPL + lane / CPR;
+    const int lc = (lane % CPR) ^ swz<D>(r);
+    t.off[it] = (uint32_t)((int64_t)r * ss + lc * 8) * 2u;
+  }
+  return t;
+}
+template <int D, int ROWS, int NW>
+__device__ __forceinline__ void load_rows_one(__amdgpu_buffer_rsrc_t rsrc, EMI_LDS uint8_t* lds, int wave,
+                                              const TileLaneOffsets<D, ROWS, NW>& t, const int it, int row0,
+                                              uint32_t row_bytes) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, lds + (it * NW + wave) * 1024, 16, t.off[it] + (uint32_t)row0 * row_bytes,
+                                           0, 0, 0);
+}
+
 // Operand fragment "32 tile rows x 16 of D": lane l holds row row_base + (l & 31),
 // D-index 16*step + 8*(l >> 5) + 0..7.
 template <int D>
@@ -568,8 +592,9 @@ template <int N, typename F> __device__ __forceinline__ void attn_static_for(F&&
 // of the next tile, then P.V of this one).  The groups run one phase apart, so on every
 // SIMD the softmax of one wavefront overlaps the matrix work of the other.
 //   bundle b(j) = {K tile j+1, V tile j}: what MFMA phase j reads; three bundles in LDS.
-//   MFMA phase j ends by issuing the loads of b(j+2) (its slot was last read two phases
-//   ago by both groups) and waiting for its own part of b(j+1) before the barrier.
+//   MFMA phase j issues the loads of b(j+2) between its P.V MFMAs (the slot was last read
+//   by the MFMA phases j-1 of both groups, which ended before this phase began) and ends
+//   by waiting for its own part of b(j+1) before the barrier.
 // The running maximum is only raised when some row's tile maximum exceeds it by more
 // than 8 (in log2 units), so the rescaling of O runs on a few early tiles only; P then
 // stays below 2^8 and the final O/l and log-sum-exp are exact for whatever m was used.
@@ -645,7 +670,16 @@ __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(const uint16_t* __rest
         vadr[dt][h] = (uint32_t)(uintptr_t)(smem + 3 * TILE) + (uint32_t)(r * (D * 2) + (((col >> 3) ^ swz<D>(r)) << 4) + (col & 7) * 2);
       }
   }
-  auto mfma_phase = [&](auto do_s_c, auto do_pv_c, auto slot_c) __attribute__((always_inline)) {
+  // Load n (0 .. LPB-1; K loads first, then V loads) of bundle jb into ring slot slot2.
+  const TileLaneOffsets<D, BKV, NW> lane_off = tile_lane_offsets<D, BKV, NW>(wave, lane, sh.ss);
+  const uint32_t row_bytes = (uint32_t)sh.ss * 2u;
+  auto issue_one = [&](const int n, const int slot2, int jb) __attribute__((always_inline)) {
+    constexpr int NL = LPB / 2;
+    if (n < NL) load_rows_one<D, BKV, NW>(rK, smem + slot2 * TILE, wave, lane_off, n, (jb + 1) * BKV, row_bytes);
+    else load_rows_one<D, BKV, NW>(rV, smem + 3 * TILE + slot2 * TILE, wave, lane_off, n - NL, jb * BKV, row_bytes);
+  };
+  // jb_issue: the bundle whose loads this phase issues (phases that compute both products only)
+  auto mfma_phase = [&](auto do_s_c, auto do_pv_c, auto slot_c, int jb_issue) __attribute__((always_inline)) {
     constexpr bool DO_S = decltype(do_s_c)::value, DO_PV = decltype(do_pv_c)::value;
     constexpr int SLOT = decltype(slot_c)::value;
     constexpr int NS = DO_S ? 2 * (D / 16) : 0, NPV = DO_PV ? 4 * (D / 32) : 0, NOP = NS + NPV, DEPTH = 6;
@@ -690,6 +724,14 @@ __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(const uint16_t* __rest
         acc_o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[i % DEPTH], pf[T][sI], acc_o[dt], 0, 0, 0);
       }
       if constexpr (i + DEPTH < NOP) fetch(std::integral_constant<int, i + DEPTH>{});
+      // The loads of the bundle two steps ahead go out one at a time between the P.V MFMAs (no K read, before
+      // which the compiler would wait for them, follows).  Issued together at the end of the phase, the 16 loads
+      // of a group queue up in the memory pipeline and hold every wavefront for 300-400 cycles with its matrix
+      // core idle (4096 keys x 128: 629 -> 590 us).
+      if constexpr (DO_S && DO_PV) {
+        constexpr int GAP = NPV / LPB;
+        if constexpr (i >= NS && (i - NS) % GAP == 0 && (i - NS) / GAP < LPB) issue_one((i - NS) / GAP, (SLOT + 2) % 3, jb_issue);
+      }
       __builtin_amdgcn_sched_barrier(0);
     });
   };
@@ -746,11 +788,9 @@ __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(const uint16_t* __rest
     if (j < nt_w) softmax(j);                         // VALU phase
     phase_end();
     __builtin_amdgcn_s_setprio(1);                    // MFMA phase
-    if (j < nt_w) mfma_phase(std::true_type{}, std::true_type{}, slot_c);    // (its last scores are never used)
+    if (j < nt_w) mfma_phase(std::true_type{}, std::true_type{}, slot_c, j + 2);    // (its last scores are never used)
+    else issue_bundle(j + 2, (SLOT + 2) % 3);
     __builtin_amdgcn_s_setprio(0);
-    // After the LDS reads of this phase: the compiler orders every LDS read behind all
-    // outstanding direct-to-LDS loads, so loads issued earlier would be waited for here.
-    issue_bundle(j + 2, (SLOT + 2) % 3);
     __builtin_amdgcn_s_waitcnt(0x0f70 | (LPB & 15));  // vmcnt(LPB): own part of b(j+1) has landed
     phase_end();
   };
@@ -762,7 +802,7 @@ __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(const uint16_t* __rest
   phase_end();
   if (wave >= 4) phase_end();                         // second group runs one phase behind
   __builtin_amdgcn_s_setprio(1);
-  mfma_phase(std::true_type{}, std::false_type{}, std::integral_constant<int, 0>{});      // MFMA phase -1
+  mfma_phase(std::true_type{}, std::false_type{}, std::integral_constant<int, 0>{}, 0);      // MFMA phase -1
   __builtin_amdgcn_s_setprio(0);
   phase_end();
   for (int j = 0; j < nt; j += 3) {
@@ -954,7 +994,8 @@ __global__ __launch_bounds__(256) void attn_prep_kernel(const uint16_t* __restri
 // Iteration H runs A(H+1) interleaved with B(H), so the softmax arithmetic of one half
 // issues in the shadow of the MFMAs of the next, then C(H).  Tiles sit in a ring of
 // three LDS slots; once per tile the wavefronts meet at a barrier, after which the loads
-// of tile t+3 may overwrite tile t.  The column fragments are fetched with
+// of tile t+3 may overwrite tile t: they go out one by one between the MFMAs of the first
+// half of tile t+1.  The column fragments are fetched with
 // ds_read_b64_tr_b16 through inline asm: the compiler orders every LDS read it knows of
 // behind all outstanding direct-to-LDS loads, which would serialise loading and compute.
 // ---------------------------------------------------------------------------
@@ -1013,23 +1054,40 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_sp_kernel(const uint16_t* __
   bf16x8_t pf[2], dsf[2];
 
   // tile ti (query tile qt0 + ti) -> slot; rows >= seq read as zeros
-  auto issue_tile = [&](int ti, int slot) __attribute__((always_inline)) {
-    const int row0 = (qt0 + ti) * BQT;
-    load_rows_tile<D, BQT, NW>(rQ, smem + slot * TILE, wave, lane, row0, seq, sh.ss);
-    load_rows_tile<D, BQT, NW>(rDO, smem + NSLOT * TILE + slot * TILE, wave, lane, row0, seq, sh.ss);
+  auto issue_stats = [&](int row0, int slot) __attribute__((always_inline)) {
     // one 256-byte load of lse2 (even wavefronts) or delta (odd ones); the copies are identical
     const uint32_t voff = row0 + lane < seq ? (uint32_t)(row0 + lane) * 4u : kOobA;
     __builtin_amdgcn_raw_ptr_buffer_load_lds((wave & 1) ? rDl : rL, smem + STATS + slot * 512 + (wave & 1) * 256, 4, voff, 0, 0,
                                              0);
   };
+  auto issue_tile = [&](int ti, int slot) __attribute__((always_inline)) {
+    const int row0 = (qt0 + ti) * BQT;
+    load_rows_tile<D, BQT, NW>(rQ, smem + slot * TILE, wave, lane, row0, seq, sh.ss);
+    load_rows_tile<D, BQT, NW>(rDO, smem + NSLOT * TILE + slot * TILE, wave, lane, row0, seq, sh.ss);
+    issue_stats(row0, slot);
+  };
+  // The same loads one at a time (n = 0 .. LPB-1: Q rows, dO rows, statistics), for the steady state, where they
+  // go out between MFMAs: issued together after the barrier, the 36 loads of a block queue up in the memory
+  // pipeline and every wavefront, alone on its SIMD, waits for its last one with the matrix core idle.
+  const TileLaneOffsets<D, BQT, NW> lane_off = tile_lane_offsets<D, BQT, NW>(wave, lane, sh.ss);
+  const uint32_t row_bytes = (uint32_t)sh.ss * 2u;
+  auto issue_part = [&](const int n, int ti, int slot) __attribute__((always_inline)) {
+    constexpr int NLQ = (LPB - 1) / 2;
+    const int row0 = (qt0 + ti) * BQT;
+    if (n < NLQ) load_rows_one<D, BQT, NW>(rQ, smem + slot * TILE, wave, lane_off, n, row0, row_bytes);
+    else if (n < 2 * NLQ) load_rows_one<D, BQT, NW>(rDO, smem + NSLOT * TILE + slot * TILE, wave, lane_off, n - NLQ, row0, row_bytes);
+    else issue_stats(row0, slot);
+  };
+  constexpr int LA = (LPB + 1) / 2, LC = LPB - LA;        // loads issued inside stage A/B and inside stage C
   // A(H+1) with B(H), interleaved by hand: after each of the 16 MFMAs of A (S and dP - delta
   // of half (slot_n, Tn) into sn, dpn; the dP accumulator starts from the -delta of its rows,
   // read from LDS, which saves a subtraction per score) comes the softmax arithmetic of one
   // score of half (ti, slot_p, Tp) held in sp, dpp.  The scheduler is fenced after every
   // step: left alone it issues all MFMAs first and the VALU work after them.
-  auto stage_ab = [&](auto masked_c, auto do_b_c, int slot_n, int Tn, f32x16_t& sn, f32x16_t& dpn, int ti, int slot_p,
-                      int Tp, f32x16_t& sp, f32x16_t& dpp) __attribute__((always_inline)) {
-    constexpr bool MASKED = decltype(masked_c)::value, DO_B = decltype(do_b_c)::value;
+  auto stage_ab = [&](auto masked_c, auto do_b_c, auto issue_c, int slot_n, int Tn, f32x16_t& sn, f32x16_t& dpn, int ti,
+                      int slot_p, int Tp, f32x16_t& sp, f32x16_t& dpp, int ti_issue, int slot_issue)
+                      __attribute__((always_inline)) {
+    constexpr bool MASKED = decltype(masked_c)::value, DO_B = decltype(do_b_c)::value, ISSUE = decltype(issue_c)::value;
     const EMI_LDS uint8_t* sQ = smem + slot_n * TILE;
     const EMI_LDS uint8_t* sDO = smem + NSLOT * TILE + slot_n * TILE;
     const EMI_LDS float* sNd = (const EMI_LDS float*)(smem + STATS + slot_n * 512) + 64 + Tn * 32 + 4 * (lane >> 5);
@@ -1060,6 +1118,10 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_sp_kernel(const uint16_t* __
       if (i & 1) dpn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[i % DEPTH], vf[i >> 1], dpn, 0, 0, 0);
       else sn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[i % DEPTH], kf[i >> 1], i == 0 ? zero16 : sn, 0, 0, 0);
       if (i + DEPTH < NOP) ring[i % DEPTH] = fetch(i + DEPTH);
+      if constexpr (ISSUE) {
+        constexpr int SP = NOP / LA;
+        if (i % SP == 1 && i / SP < LA) issue_part(i / SP, ti_issue, slot_issue);
+      }
       if constexpr (DO_B) {
 #pragma unroll
         for (int u = 0; u < EPM; u++) {
@@ -1082,7 +1144,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_sp_kernel(const uint16_t* __
   // C: dV, dK contributions of half (slot, T).  16 column fragments, two asm reads each,
   // ring of 4 fragments: after the reads of fragment i+4 are issued, fragments i..i+4 (10
   // reads) are outstanding and lgkmcnt(8) means fragment i has arrived.
-  auto stage_c = [&](int slot, int T) __attribute__((always_inline)) {
+  auto stage_c = [&](auto issue_c, int slot, int T, int ti_issue, int slot_issue) __attribute__((always_inline)) {
+    constexpr bool ISSUE = decltype(issue_c)::value;
     const uint32_t aQ = (uint32_t)(uintptr_t)(smem + slot * TILE);
     const uint32_t aDO = (uint32_t)(uintptr_t)(smem + NSLOT * TILE + slot * TILE);
     // per-lane address of the first read of col_frag<D>(tile, row_base, col_base): see col_frag
@@ -1116,6 +1179,10 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_sp_kernel(const uint16_t* __
       if (which) acc_k[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, dsf[sI], acc_k[dt], 0, 0, 0);
       else acc_v[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, pf[sI], acc_v[dt], 0, 0, 0);
       if (i + DEPTH < NF) fetch(i + DEPTH, i % DEPTH);
+      if constexpr (ISSUE) {
+        constexpr int SP = NF / LC;
+        if (i % SP == 1 && i / SP < LC) issue_part(LA + i / SP, ti_issue, slot_issue);
+      }
     }
   };
 
@@ -1123,25 +1190,25 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_sp_kernel(const uint16_t* __
   issue_tile(1, 1);
   __builtin_amdgcn_s_waitcnt(0x0f70);                 // vmcnt(0)
   __syncthreads();
-  issue_tile(2, 2);
 
   f32x16_t sA, dpA, sB, dpB;                          // scores of even / odd halves
-  stage_ab(std::false_type{}, std::false_type{}, 0, 0, sA, dpA, 0, 0, 0, sB, dpB);
+  stage_ab(std::false_type{}, std::false_type{}, std::false_type{}, 0, 0, sA, dpA, 0, 0, 0, sB, dpB, 0, 0);
   int slot = 0;                                       // slot of tile ti
   auto tile_step = [&](auto masked_c, int ti) __attribute__((always_inline)) {
     const int nslot = slot == NSLOT - 1 ? 0 : slot + 1;
-    // iteration 2*ti: A(half 1 of this tile) with B(half 0), then C(half 0)
-    stage_ab(masked_c, std::true_type{}, slot, 1, sB, dpB, ti, slot, 0, sA, dpA);
-    stage_c(slot, 0);
+    const int pslot = slot == 0 ? NSLOT - 1 : slot - 1;   // slot of tile ti-1 = slot of tile ti+2
+    // iteration 2*ti: A(half 1 of this tile) with B(half 0), then C(half 0).  The loads of tile ti+2 go out
+    // between the MFMAs of this iteration: every wavefront has passed the barrier that ended tile ti-1, whose
+    // slot they fill, and they have the second iteration to land.
+    stage_ab(masked_c, std::true_type{}, std::true_type{}, slot, 1, sB, dpB, ti, slot, 0, sA, dpA, ti + 2, pslot);
+    stage_c(std::true_type{}, slot, 0, ti + 2, pslot);
     // iteration 2*ti+1: A(half 0 of the next tile) with B(half 1), then C(half 1)
-    stage_ab(masked_c, std::true_type{}, nslot, 0, sA, dpA, ti, slot, 1, sB, dpB);
-    stage_c(slot, 1);
-    // Tile ti is finished.  Own part of tile ti+2 (issued one tile ago) must have landed;
-    // after the barrier every wavefront is done with tile ti and sees tile ti+2, and the
-    // loads of tile ti+3 may go into the slot of tile ti.
-    __builtin_amdgcn_s_waitcnt(0x0f70);               // vmcnt(0): only tile ti+2 is outstanding
+    stage_ab(masked_c, std::true_type{}, std::false_type{}, nslot, 0, sA, dpA, ti, slot, 1, sB, dpB, 0, 0);
+    stage_c(std::false_type{}, slot, 1, 0, 0);
+    // Tile ti is finished.  Own part of tile ti+2 must have landed; after the barrier every wavefront is done
+    // with tile ti and sees tile ti+2.
+    __builtin_amdgcn_s_waitcnt(0x0f70);               // vmcnt(0)
     __builtin_amdgcn_s_barrier();
-    issue_tile(ti + 3, slot);
     slot = nslot;
   };
   // Only the first two query tiles of a key block can hold queries that precede its keys.
@@ -1358,6 +1425,7 @@ static bool mfma_ok(const AttnArgs& a, int dtype, std::initializer_list<const vo
   if (dtype != EMI_BF16 || (a.d != 64 && a.d != 128)) return false;
   if ((a.sb % 8) || (a.sh % 8) || (a.ss % 8)) return false;
   if ((a.seq - 1) * a.ss + a.d >= (int64_t)0x3fffff00) return false;
+  if ((a.seq + 256) * a.ss >= (int64_t)0x7fffff00) return false;    // tiles addressed past the last row: 32-bit byte offsets
   for (const void* p : ptrs)
     if (!aligned16(p)) return false;
   return true;
@@ -1437,7 +1505,8 @@ extern "C" int emi_attn_fwd_ws(emi_stream_t stream, const void* q, const void* k
   if (mfma_ok(a, dtype, {q, k, v, o})) {
     const uint32_t head_bytes = (uint32_t)(((seq - 1) * stride_s + head_dim) * 2);
     const float sl2 = scale * kLog2e;
-    if (seq > 512) {        // 256-query blocks; at 512 keys and fewer the 128-query kernel below is faster (25 vs 31 us at 16 x 12 x 512 x 64)
+    // 256-query blocks; at 512 keys and fewer the 128-query kernel below is faster (25 vs 31 us at 16 x 12 x 512 x 64)
+    if (seq > 512) {
       const dim3 gridp((unsigned)((seq + 255) / 256), bh);
 #define EMI_ATTN_FWD_PP(DD)                                                                                          \
   do {                                                                                                               \
