@@ -304,24 +304,44 @@ __global__ __launch_bounds__(256) void attn_step_fwd1_kernel(const T* __restrict
   }
 }
 
-// o = sum_i w_i o_i / sum_i w_i l_i with w_i = exp(m_i - max m); lse = max m + log(sum).
+// o = sum_i w_i o_i / sum_i w_i l_i with w_i = exp(m_i - max m); lse = max m + log(sum).  One wavefront per
+// (batch, head): lane i holds the statistics and the weight of split c + i and hands the weight round by lane
+// index, so the partial rows stream in with independent loads instead of one dependent chain per pass.
 template <typename T>
 __global__ __launch_bounds__(64) void attn_step_combine_kernel(const float* __restrict__ part, T* __restrict__ o,
                                                                float* __restrict__ lse, StepShape sh, int nsplit) {
   const int bh = blockIdx.x, b = bh / sh.heads, h = bh % sh.heads;
-  const float* p0 = part + (int64_t)bh * nsplit * (sh.head_dim + 2);
+  const int lane = threadIdx.x, hd = sh.head_dim, stride = sh.head_dim + 2;
+  const float* p0 = part + (int64_t)bh * nsplit * stride;
   float mx = -INFINITY;
-  for (int i = 0; i < nsplit; i++) mx = fmaxf(mx, p0[i * (sh.head_dim + 2) + sh.head_dim]);
+  for (int i = lane; i < nsplit; i += 64) mx = fmaxf(mx, p0[i * stride + hd]);
+  mx = wave_max(mx);
   float l = 0.f;
-  for (int i = 0; i < nsplit; i++) l += p0[i * (sh.head_dim + 2) + sh.head_dim + 1] * __expf(p0[i * (sh.head_dim + 2) + sh.head_dim] - mx);
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};                         // head_dim <= 256: up to four columns per lane
+  for (int c = 0; c < nsplit; c += 64) {
+    const int i = c + lane;
+    float w = 0.f;
+    if (i < nsplit) {
+      w = __expf(p0[i * stride + hd] - mx);
+      l += p0[i * stride + hd + 1] * w;
+    }
+    const int cnt = nsplit - c < 64 ? nsplit - c : 64;
+#pragma unroll 4
+    for (int ii = 0; ii < cnt; ii++) {
+      const float wi = __shfl(w, ii, kWave);
+      const float* row = p0 + (int64_t)(c + ii) * stride;
+#pragma unroll
+      for (int q = 0; q < 4; q++)
+        if (lane + 64 * q < hd) acc[q] = fmaf(row[lane + 64 * q], wi, acc[q]);
+    }
+  }
+  l = wave_sum(l);
   const float inv = 1.0f / l;
   T* orow = o + b * sh.q_sb + h * sh.q_sh;
-  for (int e = threadIdx.x; e < sh.head_dim; e += 64) {
-    float acc = 0.f;
-    for (int i = 0; i < nsplit; i++) acc += p0[i * (sh.head_dim + 2) + e] * __expf(p0[i * (sh.head_dim + 2) + sh.head_dim] - mx);
-    orow[e] = from_f32<T>(acc * inv);
-  }
-  if (threadIdx.x == 0) lse[bh] = mx + __logf(l);
+#pragma unroll
+  for (int q = 0; q < 4; q++)
+    if (lane + 64 * q < hd) orow[lane + 64 * q] = from_f32<T>(acc[q] * inv);
+  if (lane == 0) lse[bh] = mx + __logf(l);
 }
 
 // dV_s = p_s dO; dP_s = dO . V_s; dS_s = p_s (dP_s - dO . O); dQ = scale sum_s dS_s K_s;

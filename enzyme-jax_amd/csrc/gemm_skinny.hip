@@ -189,33 +189,35 @@ __global__ __launch_bounds__(256) void gemv_nn_bands_kernel(const T* __restrict_
     }
 }
 
-// C[m][n] = sum over bands (in a fixed order) + R: 64 columns per block, 4 band lanes each
-// with 8 loads in flight, met through LDS.
+// C[m][n] = sum over bands (in a fixed order) + R: 16 columns (64 bytes of a partial row) per block, 16 band
+// lanes with up to 16 loads in flight each, so 256 bands are one round trip; the lanes meet through LDS.
 template <typename T>
 __global__ __launch_bounds__(256) void gemv_bands_reduce_kernel(const float* __restrict__ part, const T* R, T* C, int M, int N,
                                                                 int bands, int64_t ldr, int64_t ldc) {
-  __shared__ float red[4][64];
-  const int col = threadIdx.x & 63, bl = threadIdx.x >> 6;
-  const int64_t i = blockIdx.x * (int64_t)64 + col;               // index into [M][N]
+  constexpr int BL = 16, UN = 16;
+  __shared__ float red[BL][16];
+  const int col = threadIdx.x & 15, bl = threadIdx.x >> 4;
+  const int64_t i = blockIdx.x * (int64_t)16 + col;               // index into [M][N]
   const bool live = i < (int64_t)M * N;
   float v = 0.f;
   if (live) {
-    const int m = (int)(i / N), n = (int)(i % N);
-    const float* p = part + (int64_t)m * N + n;
+    const float* p = part + i;
     const int64_t bstride = (int64_t)M * N;
-    for (int b0 = bl; b0 < bands; b0 += 4 * 8) {
-      float t[8];
+    for (int b0 = bl; b0 < bands; b0 += BL * UN) {
+      float t[UN];
 #pragma unroll
-      for (int u = 0; u < 8; u++) t[u] = b0 + 4 * u < bands ? p[(int64_t)(b0 + 4 * u) * bstride] : 0.f;
+      for (int u = 0; u < UN; u++) t[u] = b0 + BL * u < bands ? p[(int64_t)(b0 + BL * u) * bstride] : 0.f;
 #pragma unroll
-      for (int u = 0; u < 8; u++) v += t[u];
+      for (int u = 0; u < UN; u++) v += t[u];
     }
   }
   red[bl][col] = v;
   __syncthreads();
   if (bl == 0 && live) {
     const int m = (int)(i / N), n = (int)(i % N);
-    v = red[0][col] + red[1][col] + red[2][col] + red[3][col];
+    v = 0.f;
+#pragma unroll
+    for (int b = 0; b < BL; b++) v += red[b][col];
     if (R != nullptr) v += to_f32(R[(int64_t)m * ldr + n]);
     C[(int64_t)m * ldc + n] = from_f32<T>(v);
   }
@@ -293,7 +295,7 @@ int launch_skinny_t(hipStream_t st, const void* A_, const void* B_, const void* 
       else EMI_BANDS(8);
 #undef EMI_BANDS
       EMI_CHECK_LAUNCH("emi_gemm(skinny bands)");
-      hipLaunchKernelGGL(gemv_bands_reduce_kernel<T>, dim3((unsigned)((M * N + 63) / 64)), dim3(256), 0, st, part, R, C, (int)M,
+      hipLaunchKernelGGL(gemv_bands_reduce_kernel<T>, dim3((unsigned)((M * N + 15) / 16)), dim3(256), 0, st, part, R, C, (int)M,
                          (int)N, bands, ldr, ldc);
     } else {
       EMI_SKINNY_MT(gemv_nn_kernel, dim3((unsigned)((N / V + 7) / 8)), 1024);
