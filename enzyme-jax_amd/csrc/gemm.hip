@@ -998,7 +998,8 @@ template <bool A_KMAJOR, bool B_KMAJOR, bool GROUPED = false, int NW = 4, int U 
 __global__ __launch_bounds__(NW * 64) void gemm_f32_small_kernel(const float* __restrict__ A, const float* __restrict__ B,
                                                                  const float* R, float* C, int M, int N, int K, int64_t lda,
                                                                  int64_t ldb, int64_t ldr, int64_t ldc,
-                                                                 std::conditional_t<GROUPED, GemmGroup, NoGroup> grp) {
+                                                                 std::conditional_t<GROUPED, GemmGroup, NoGroup> grp,
+                                                                 float* __restrict__ part = nullptr, int kps = 0) {
   __shared__ float red[NW - 1][16][64];
   if constexpr (GROUPED) {
     A = reinterpret_cast<const float*>(grp.A[blockIdx.z]);
@@ -1010,8 +1011,12 @@ __global__ __launch_bounds__(NW * 64) void gemm_f32_small_kernel(const float* __
   const int i = lane & 31, g = lane >> 5;
   const int m0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
   const int mi = m0 + i < M ? m0 + i : M - 1, ni = n0 + i < N ? n0 + i : N - 1;      // clamped: those results are not stored
-  const int kper = ((K + 8 * NW - 1) / (8 * NW)) * 8;    // this wavefront's share of K, rounded up to whole chunks
-  const int ks = wave * kper, ke = ks + kper < K ? ks + kper : K;
+  // split-K (part != nullptr, not GROUPED): plane blockIdx.z takes kps (a multiple of 8 NW) of K and leaves its
+  // 32 x 32 partial in part[z][M][N] for gemm_splitk_reduce_kernel
+  const int kb = part != nullptr ? (int)blockIdx.z * kps : 0;
+  const int kend = part != nullptr && kb + kps < K ? kb + kps : K;
+  const int kper = ((kend - kb + 8 * NW - 1) / (8 * NW)) * 8;    // this wavefront's share of K, rounded up to whole chunks
+  const int ks = kb + wave * kper, ke = ks + kper < kend ? ks + kper : kend;
   const float* pa = A_KMAJOR ? A + mi : A + (int64_t)mi * lda;
   const float* pb = B_KMAJOR ? B + ni : B + (int64_t)ni * ldb;
   // elements k0 + 4 g + t, t = 0..3, of this lane's row (column) of an operand; zero past the wavefront's share of K
@@ -1083,8 +1088,12 @@ __global__ __launch_bounds__(NW * 64) void gemm_f32_small_kernel(const float* __
     const int row = m0 + (r >> 2) * 8 + g * 4 + (r & 3);
     if (row < M && col < N) {
       float v = acc[r];
-      if (R != nullptr) v += R[(int64_t)row * ldr + col];
-      C[(int64_t)row * ldc + col] = v;
+      if (part != nullptr) {
+        part[((int64_t)blockIdx.z * M + row) * N + col] = v;
+      } else {
+        if (R != nullptr) v += R[(int64_t)row * ldr + col];
+        C[(int64_t)row * ldc + col] = v;
+      }
     }
   }
 }
@@ -1371,14 +1380,35 @@ extern "C" int emi_gemm_ws(emi_stream_t stream, const void* A, const void* B, co
     }
     return launch_generic<bf16>(st, A, B, R, C, (int)M, (int)N, (int)K, lda, ldb, ldr, ldc, trans_a, trans_b, workspace, workspace_bytes);
   }
-  // fp32 on 16-byte aligned k-contiguous rows, unless few tiles and a long contraction call for split-K partials:
-  // 32x32 tiles, K split over the block's wavefronts, operands straight from global memory (at every size measured
+  // fp32 on 16-byte aligned k-contiguous rows: 32x32 tiles, K split over the block's wavefronts, operands straight from global memory (at every size measured
   // this beats the LDS-staged kernel, whose loads are element-wise: 1024^3 45 vs 3 TFLOP/s, 2048^3 55 vs 13)
   if (K > 0 && (M + 31) / 32 <= 65535 &&
-      !(generic_splits(M, N, K) > 1 && workspace != nullptr) &&
       (trans_a || ((reinterpret_cast<uintptr_t>(A) & 15) == 0 && lda % 4 == 0)) &&
       (!trans_b || ((reinterpret_cast<uintptr_t>(B) & 15) == 0 && ldb % 4 == 0))) {
-    const dim3 grid((unsigned)((N + 31) / 32), (unsigned)((M + 31) / 32));
+    dim3 grid((unsigned)((N + 31) / 32), (unsigned)((M + 31) / 32));
+    const int splits = generic_splits(M, N, K);
+    if (splits > 1 && workspace != nullptr && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0 &&
+        workspace_bytes >= (size_t)splits * M * N * sizeof(float)) {
+      // few tiles and a long contraction (dX = dY . Wcls of a small batch): planes of K on the same kernel, partials
+      // added in fixed order by the reduce kernel (256 x 288 x 32000: 130 us on the LDS-staged kernel)
+      const int kps = (int)((((K + splits - 1) / splits) + 31) / 32 * 32);
+      grid.z = (unsigned)((K + kps - 1) / kps);
+      float* part = static_cast<float*>(workspace);
+#define EMI_F32_SPLIT(AKM, BKM)                                                                                            \
+  hipLaunchKernelGGL((gemm_f32_small_kernel<AKM, BKM, false, 4, 4, false>), grid, dim3(256), 0, st,                        \
+                     static_cast<const float*>(A), static_cast<const float*>(B), static_cast<const float*>(nullptr),       \
+                     static_cast<float*>(C), (int)M, (int)N, (int)K, lda, ldb, ldr, ldc, NoGroup{}, part, kps)
+      if (!trans_a && trans_b) EMI_F32_SPLIT(false, false);
+      else if (!trans_a && !trans_b) EMI_F32_SPLIT(false, true);
+      else if (trans_a && !trans_b) EMI_F32_SPLIT(true, true);
+      else EMI_F32_SPLIT(true, false);
+#undef EMI_F32_SPLIT
+      EMI_CHECK_LAUNCH("emi_gemm(fp32 split-K)");
+      hipLaunchKernelGGL(gemm_splitk_reduce_kernel<float>, dim3((unsigned)(((int64_t)M * N + 255) / 256)), dim3(256), 0, st, part,
+                         static_cast<const float*>(R), static_cast<float*>(C), (int)M, (int)N, (int)grid.z, ldr, ldc);
+      EMI_CHECK_LAUNCH("emi_gemm(fp32 split-K reduce)");
+      return EMI_OK;
+    }
 #define EMI_F32_SMALL_V(AKM, BKM, NWV, UV, ONCEV)                                                                          \
   hipLaunchKernelGGL((gemm_f32_small_kernel<AKM, BKM, false, NWV, UV, ONCEV>), grid, dim3(NWV * 64), 0, st,                \
                      static_cast<const float*>(A), static_cast<const float*>(B), static_cast<const float*>(R),             \

@@ -106,6 +106,7 @@ GEMM_SHAPES = [
     (264, 136, 4104),    # few tiles, long contraction: split-K with fp32 partials (bf16 128-tile kernel and fp32 kernel)
     (100, 200, 2600),    # split-K on the generic kernel for both dtypes where M is not a multiple of 8
     (64, 101, 4096),     # split-K with rows of the partials that are not 16-byte aligned (scalar partial stores)
+    (256, 288, 32000),   # the logits adjoint dX = dY . Wcls of the 15M model: 50 planes of K
 ]
 
 
