@@ -326,7 +326,6 @@ __global__ __launch_bounds__(64) void attn_step_combine_kernel(const float* __re
       l += p0[i * stride + hd + 1] * w;
     }
     const int cnt = nsplit - c < 64 ? nsplit - c : 64;
-#pragma unroll 4
     for (int ii = 0; ii < cnt; ii++) {
       const float wi = __shfl(w, ii, kWave);
       const float* row = p0 + (int64_t)(c + ii) * stride;

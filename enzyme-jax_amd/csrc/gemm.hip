@@ -1098,6 +1098,140 @@ __global__ __launch_bounds__(NW * 64) void gemm_f32_small_kernel(const float* __
   }
 }
 
+// ---------------------------------------------------------------------------
+// fp32 products that fill the chip with 128 x 128 tiles (the logits and their adjoints: 256 x 32000 x 288 and its
+// two transposes): the same matrix instruction fed from LDS.  The K-split kernel above has every 32 x 32 tile read
+// its own 64 operand rows from the L2 (8 flop per byte), which bounds it at 35-55 TFLOP/s.  Here a block of four
+// wavefronts (2 x 2, 64 x 64 each = four 32 x 32 accumulators) stages 128 x 32 pieces of both operands per step:
+// a k-contiguous operand as [row][32 + 4] (a lane reads its 4 consecutive k as one 16-byte piece), a k-major one as
+// [k][128] (four 4-byte reads, lanes along the rows).  Global loads of step s+1 are in flight while step s is
+// multiplied (held in registers, written to LDS between two barriers).  part / kps as in the kernel above (planes of K).
+// Needs 16-byte aligned bases and leading dimensions that are multiples of 4.
+// ---------------------------------------------------------------------------
+template <bool A_KMAJOR, bool B_KMAJOR>
+__global__ __launch_bounds__(256) void gemm_f32_tiled_kernel(const float* __restrict__ A, const float* __restrict__ B,
+                                                             const float* R, float* C, int M, int N, int K, int64_t lda,
+                                                             int64_t ldb, int64_t ldr, int64_t ldc, float* __restrict__ part,
+                                                             int kps) {
+  constexpr int BT = 128, BK = 32, KC_LD = BK + 4;
+  constexpr int A_FLOATS = A_KMAJOR ? BK * BT : BT * KC_LD, B_FLOATS = B_KMAJOR ? BK * BT : BT * KC_LD;
+  __shared__ __attribute__((aligned(16))) float sA[A_FLOATS];
+  __shared__ __attribute__((aligned(16))) float sB[B_FLOATS];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int i = lane & 31, g = lane >> 5;
+  const int m0 = blockIdx.y * BT, n0 = blockIdx.x * BT;
+  const int kb = part != nullptr ? (int)blockIdx.z * kps : 0;
+  const int kend = part != nullptr && kb + kps < K ? kb + kps : K;
+  const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+
+  // global -> registers: four 16-byte pieces of each operand per thread and step; zero outside the operand
+  auto gload = [&](const float* X, int64_t ld, bool kmajor, int row0, int rows, int k0, float4 (&v)[4]) {
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      const int idx = tid + 256 * q;
+      float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (!kmajor) {
+        const int row = row0 + (idx >> 3), k = k0 + (idx & 7) * 4;
+        if (row < rows) {
+          const float* p = X + (int64_t)row * ld + k;
+          if (k + 4 <= kend) x = *reinterpret_cast<const float4*>(p);
+          else {
+            if (k < kend) x.x = p[0];
+            if (k + 1 < kend) x.y = p[1];
+            if (k + 2 < kend) x.z = p[2];
+          }
+        }
+      } else {
+        const int k = k0 + (idx >> 5), row = row0 + (idx & 31) * 4;
+        if (k < kend) {
+          const float* p = X + (int64_t)k * ld + row;
+          if (row + 4 <= rows) x = *reinterpret_cast<const float4*>(p);
+          else {
+            if (row < rows) x.x = p[0];
+            if (row + 1 < rows) x.y = p[1];
+            if (row + 2 < rows) x.z = p[2];
+          }
+        }
+      }
+      v[q] = x;
+    }
+  };
+  auto sstore = [&](float* sX, bool kmajor, const float4 (&v)[4]) {
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      const int idx = tid + 256 * q;
+      if (!kmajor) *reinterpret_cast<float4*>(sX + (idx >> 3) * KC_LD + (idx & 7) * 4) = v[q];
+      else *reinterpret_cast<float4*>(sX + (idx >> 5) * BT + (idx & 31) * 4) = v[q];
+    }
+  };
+  // the four k of chunk j (8 wide) that this lane contracts, for tile row r of an operand
+  auto frag = [&](const float* sX, bool kmajor, int r, int j, float (&f)[4]) {
+    if (!kmajor) {
+      const float4 x = *reinterpret_cast<const float4*>(sX + r * KC_LD + 8 * j + 4 * g);
+      f[0] = x.x; f[1] = x.y; f[2] = x.z; f[3] = x.w;
+    } else {
+#pragma unroll
+      for (int t = 0; t < 4; t++) f[t] = sX[(8 * j + 4 * g + t) * BT + r];
+    }
+  };
+
+  f32x16_t acc[2][2];
+#pragma unroll
+  for (int a = 0; a < 2; a++)
+#pragma unroll
+    for (int b = 0; b < 2; b++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[a][b][r] = 0.f;
+
+  float4 va[4], vb[4];
+  gload(A, lda, A_KMAJOR, m0, M, kb, va);
+  gload(B, ldb, B_KMAJOR, n0, N, kb, vb);
+  for (int k0 = kb; k0 < kend; k0 += BK) {
+    sstore(sA, A_KMAJOR, va);
+    sstore(sB, B_KMAJOR, vb);
+    __syncthreads();
+    if (k0 + BK < kend) {                                // in flight while this step is multiplied
+      gload(A, lda, A_KMAJOR, m0, M, k0 + BK, va);
+      gload(B, ldb, B_KMAJOR, n0, N, k0 + BK, vb);
+    }
+#pragma unroll
+    for (int j = 0; j < BK / 8; j++) {
+      float fa[2][4], fb[2][4];
+#pragma unroll
+      for (int a = 0; a < 2; a++) frag(sA, A_KMAJOR, wm + a * 32 + i, j, fa[a]);
+#pragma unroll
+      for (int b = 0; b < 2; b++) frag(sB, B_KMAJOR, wn + b * 32 + i, j, fb[b]);
+#pragma unroll
+      for (int t = 0; t < 4; t++)
+#pragma unroll
+        for (int a = 0; a < 2; a++)
+#pragma unroll
+          for (int b = 0; b < 2; b++) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[a][t], fb[b][t], acc[a][b], 0, 0, 0);
+    }
+    __syncthreads();                                     // every wavefront is done with this step's tiles
+  }
+  // register r of lane l: row 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32 of its 32 x 32 tile
+#pragma unroll
+  for (int a = 0; a < 2; a++)
+#pragma unroll
+    for (int b = 0; b < 2; b++) {
+      const int col = n0 + wn + b * 32 + i;
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int row = m0 + wm + a * 32 + (r >> 2) * 8 + g * 4 + (r & 3);
+        if (row < M && col < N) {
+          float v = acc[a][b][r];
+          if (part != nullptr) {
+            part[((int64_t)blockIdx.z * M + row) * N + col] = v;
+          } else {
+            if (R != nullptr) v += R[(int64_t)row * ldr + col];
+            C[(int64_t)row * ldc + col] = v;
+          }
+        }
+      }
+    }
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __restrict__ part, const T* R, T* C, int M, int N,
                                                                  int splits, int64_t ldr, int64_t ldc) {
@@ -1105,7 +1239,15 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __
   if (i >= (int64_t)M * N) return;
   const int row = (int)(i / N), col = (int)(i - (int64_t)row * N);
   float v = 0.f;
-  for (int z = 0; z < splits; z++) v += part[(int64_t)z * M * N + i];
+  int z = 0;
+  for (; z + 8 <= splits; z += 8) {                       // eight loads in flight, added in plane order
+    float t[8];
+#pragma unroll
+    for (int u = 0; u < 8; u++) t[u] = part[(int64_t)(z + u) * M * N + i];
+#pragma unroll
+    for (int u = 0; u < 8; u++) v += t[u];
+  }
+  for (; z < splits; z++) v += part[(int64_t)z * M * N + i];
   if (R != nullptr) v += to_f32(R[(int64_t)row * ldr + col]);
   C[(int64_t)row * ldc + col] = from_f32<T>(v);
 }
@@ -1387,13 +1529,38 @@ extern "C" int emi_gemm_ws(emi_stream_t stream, const void* A, const void* B, co
       (!trans_b || ((reinterpret_cast<uintptr_t>(B) & 15) == 0 && ldb % 4 == 0))) {
     dim3 grid((unsigned)((N + 31) / 32), (unsigned)((M + 31) / 32));
     const int splits = generic_splits(M, N, K);
+    // 128 x 128 tiles staged through LDS once they fill the chip (alone or as planes of K)
+    const bool tiled_ok = (reinterpret_cast<uintptr_t>(A) & 15) == 0 && (reinterpret_cast<uintptr_t>(B) & 15) == 0 &&
+                          lda % 4 == 0 && ldb % 4 == 0;
+    const int64_t tiles128 = ((M + 127) / 128) * ((N + 127) / 128);
     if (splits > 1 && workspace != nullptr && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0 &&
         workspace_bytes >= (size_t)splits * M * N * sizeof(float)) {
       // few tiles and a long contraction (dX = dY . Wcls of a small batch): planes of K on the same kernel, partials
       // added in fixed order by the reduce kernel (256 x 288 x 32000: 130 us on the LDS-staged kernel)
-      const int kps = (int)((((K + splits - 1) / splits) + 31) / 32 * 32);
+      int kps = (int)((((K + splits - 1) / splits) + 31) / 32 * 32);
       grid.z = (unsigned)((K + kps - 1) / kps);
       float* part = static_cast<float*>(workspace);
+      if (tiled_ok && tiles128 * grid.z >= 192) {
+        // one block per CU and no second round: at most 256 / tiles planes (never more than the workspace holds)
+        const int64_t want = 256 / tiles128 < splits ? 256 / tiles128 : splits;
+        kps = (int)((((K + want - 1) / want) + 31) / 32 * 32);
+        grid.z = (unsigned)((K + kps - 1) / kps);
+        const dim3 gridt((unsigned)((N + 127) / 128), (unsigned)((M + 127) / 128), grid.z);
+#define EMI_F32_TILED_SPLIT(AKM, BKM)                                                                                      \
+  hipLaunchKernelGGL((gemm_f32_tiled_kernel<AKM, BKM>), gridt, dim3(256), 0, st, static_cast<const float*>(A),             \
+                     static_cast<const float*>(B), static_cast<const float*>(nullptr), static_cast<float*>(C), (int)M,     \
+                     (int)N, (int)K, lda, ldb, ldr, ldc, part, kps)
+        if (!trans_a && trans_b) EMI_F32_TILED_SPLIT(false, false);
+        else if (!trans_a && !trans_b) EMI_F32_TILED_SPLIT(false, true);
+        else if (trans_a && !trans_b) EMI_F32_TILED_SPLIT(true, true);
+        else EMI_F32_TILED_SPLIT(true, false);
+#undef EMI_F32_TILED_SPLIT
+        EMI_CHECK_LAUNCH("emi_gemm(fp32 tiled split-K)");
+        hipLaunchKernelGGL(gemm_splitk_reduce_kernel<float>, dim3((unsigned)(((int64_t)M * N + 255) / 256)), dim3(256), 0, st, part,
+                           static_cast<const float*>(R), static_cast<float*>(C), (int)M, (int)N, (int)grid.z, ldr, ldc);
+        EMI_CHECK_LAUNCH("emi_gemm(fp32 split-K reduce)");
+        return EMI_OK;
+      }
 #define EMI_F32_SPLIT(AKM, BKM)                                                                                            \
   hipLaunchKernelGGL((gemm_f32_small_kernel<AKM, BKM, false, 4, 4, false>), grid, dim3(256), 0, st,                        \
                      static_cast<const float*>(A), static_cast<const float*>(B), static_cast<const float*>(nullptr),       \
@@ -1413,6 +1580,20 @@ extern "C" int emi_gemm_ws(emi_stream_t stream, const void* A, const void* B, co
   hipLaunchKernelGGL((gemm_f32_small_kernel<AKM, BKM, false, NWV, UV, ONCEV>), grid, dim3(NWV * 64), 0, st,                \
                      static_cast<const float*>(A), static_cast<const float*>(B), static_cast<const float*>(R),             \
                      static_cast<float*>(C), (int)M, (int)N, (int)K, lda, ldb, ldr, ldc, NoGroup{})
+    if (tiled_ok && tiles128 >= 192) {
+      const dim3 gridt((unsigned)((N + 127) / 128), (unsigned)((M + 127) / 128));
+#define EMI_F32_TILED(AKM, BKM)                                                                                            \
+  hipLaunchKernelGGL((gemm_f32_tiled_kernel<AKM, BKM>), gridt, dim3(256), 0, st, static_cast<const float*>(A),             \
+                     static_cast<const float*>(B), static_cast<const float*>(R), static_cast<float*>(C), (int)M, (int)N,   \
+                     (int)K, lda, ldb, ldr, ldc, static_cast<float*>(nullptr), 0)
+      if (!trans_a && trans_b) EMI_F32_TILED(false, false);
+      else if (!trans_a && !trans_b) EMI_F32_TILED(false, true);
+      else if (trans_a && !trans_b) EMI_F32_TILED(true, true);
+      else EMI_F32_TILED(true, false);
+#undef EMI_F32_TILED
+      EMI_CHECK_LAUNCH("emi_gemm(fp32 tiled)");
+      return EMI_OK;
+    }
     // few blocks: latency decides, everything is requested at once; many blocks: the stepped form, whose smaller
     // register footprint keeps more wavefronts resident
     const bool few = (int64_t)grid.x * grid.y <= 1024;

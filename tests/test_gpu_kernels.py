@@ -127,6 +127,35 @@ def test_gemm_layouts(ops, dt, ta, tb, M, N, K):
     check(ops.gemm(a, b, bool(ta), bool(tb), r), ref + rr, dt, "gemm + residual")
 
 
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("ta,tb", [(0, 1), (0, 0), (1, 0), (1, 1)])
+@pytest.mark.parametrize("M,N,K,pad", [(2049, 1537, 262, 8), (259, 290, 20011, 8)])
+def test_gemm_padded_leading_dimensions(ops, dt, ta, tb, M, N, K, pad):
+    """emi_gemm_ws through the C ABI on operands that are windows of larger buffers: leading dimensions longer than
+    the rows (16-byte aligned rows, so the chunked kernels are taken), sizes that are multiples of nothing: the tiled
+    kernels' edge handling in every layout (many tiles; few tiles with planes of K)."""
+    import torch
+    from enzyme_ad.jax import _native as nat
+    _say("gemm padded", dt, ta, tb, M, N, K)
+    rng = np.random.default_rng(M + N + K + 5 * ta + 3 * tb)
+    ar, ac = (K, M) if ta else (M, K)
+    br, bc = (N, K) if tb else (K, N)
+    A, Ar = dev(rng.standard_normal((ar, ac + pad)), dt)
+    B, Br = dev(rng.standard_normal((br, bc + pad)), dt)
+    R, Rr = dev(rng.standard_normal((M, N + pad)), dt)
+    C = torch.full((M, N + pad), 7.0, dtype=A.dtype, device="cuda")
+    a2, b2 = Ar[:, :ac], Br[:, :bc]
+    ref = (a2.T if ta else a2) @ (b2.T if tb else b2) + Rr[:, :N]
+    lib = nat.lib()
+    code = nat.EMI_F32 if dt == "f32" else nat.EMI_BF16
+    nbytes = lib.emi_gemm_workspace_bytes(M, N, K, ta, tb, code)
+    ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device="cuda")
+    nat.check(lib.emi_gemm_ws(torch.cuda.current_stream().cuda_stream, A.data_ptr(), B.data_ptr(), R.data_ptr(), C.data_ptr(),
+                            ws.data_ptr(), nbytes, M, N, K, ac + pad, bc + pad, N + pad, N + pad, ta, tb, code))
+    check(C[:, :N], ref, dt, "gemm on windows")
+    assert bool((C[:, N:] == 7.0).all()), "wrote outside the window"
+
+
 GROUPED_SHAPES = [
     (256, 384, 320),     # one launch of the 128-tile kernel, K not a multiple of 64
     (200, 136, 72),      # ragged tiles
