@@ -278,6 +278,12 @@ ATTN_CASES = [
     ("bf16", 1, 2, 130, 64, "bhsd"),
     ("bf16", 1, 2, 600, 128, "bshd"),   # ping-pong forward, several 256-query blocks, ragged
     ("bf16", 1, 2, 1030, 64, "bhsd"),   # ping-pong forward, head_dim 64
+    # tile loads that run past the last row of a head (they rely on the buffer descriptor's bounds) with live data
+    # of the next head / sequence right behind it
+    ("bf16", 2, 2, 513, 128, "bhsd"),   # ping-pong forward just above its threshold: a last key tile of one row
+    ("bf16", 2, 2, 577, 64, "bshd"),
+    ("bf16", 2, 3, 65, 128, "bhsd"),    # dK/dV with two query tiles, the second of one row
+    ("bf16", 2, 2, 191, 64, "bshd"),
 ]
 
 
