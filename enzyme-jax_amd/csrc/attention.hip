@@ -345,28 +345,28 @@ __device__ __forceinline__ void load_rows_tile(__amdgpu_buffer_rsrc_t rsrc, EMI_
   }
 }
 
-// One of those loads on its own, for a kernel that spreads them between its MFMAs.  off[it] is the per-lane part
-// of load it's byte offset (tile row 0), computed once per kernel.  No bounds test: a row past the end of the
-// sequence lies past the end of the buffer descriptor (which ends with the last row of the head) and reads as zero.
-template <int D, int ROWS, int NW> struct TileLaneOffsets { uint32_t off[ROWS / (64 / (D / 8)) / NW]; };
-template <int D, int ROWS, int NW>
-__device__ __forceinline__ TileLaneOffsets<D, ROWS, NW> tile_lane_offsets(int wave, int lane, int64_t ss) {
-  constexpr int CPR = D / 8, RPL = 64 / CPR, NLOAD = ROWS / RPL / NW;
-  TileLaneOffsets<D, ROWS, NW> t;
-#pragma unroll
-  for (int it = 0; it < NLOAD; it++) {
-    const int r = (it * NW + wave) * RPL + lane / CPR;
-    const int lc = (lane % CPR) ^ swz<D>(r);
-    t.off[it] = (uint32_t)((int64_t)r * ss + lc * 8) * 2u;
-  }
-  return t;
+// One of those loads on its own, for a kernel that spreads them between its MFMAs: lane_off is the per-lane part of
+// the byte offset of load 0 at tile row 0, computed once per kernel; load `it` lies it * NW * (64 / (D / 8)) rows
+// further (a multiple of 16 rows: the swizzle does not change), which together with the tile's first row is a
+// wave-uniform term.  No bounds test: a row past the end of the sequence lies past the end of the buffer descriptor
+// (which ends with the last row of the head) and reads as zero.
+template <int D, int NW> __device__ __forceinline__ uint32_t tile_lane_offset(int wave, int lane, int64_t ss) {
+  constexpr int CPR = D / 8, RPL = 64 / CPR;
+  static_assert((NW * RPL) % 16 == 0, "swizzle period");
+  const int r = wave * RPL + lane / CPR;
+  const int lc = (lane % CPR) ^ swz<D>(r);
+  return (uint32_t)((int64_t)r * ss + lc * 8) * 2u;
 }
-template <int D, int ROWS, int NW>
-__device__ __forceinline__ void load_rows_one(__amdgpu_buffer_rsrc_t rsrc, EMI_LDS uint8_t* lds, int wave,
-                                              const TileLaneOffsets<D, ROWS, NW>& t, const int it, int row0,
-                                              uint32_t row_bytes) {
-  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, lds + (it * NW + wave) * 1024, 16, t.off[it] + (uint32_t)row0 * row_bytes,
-                                           0, 0, 0);
+template <int D, int NW>
+__device__ __forceinline__ uint32_t tile_piece_offset(uint32_t lane_off, int it, int row0, uint32_t row_bytes) {
+  return lane_off + (uint32_t)(row0 + it * NW * (64 / (D / 8))) * row_bytes;
+}
+// load `it` of wavefront `wave` into its 1 KB piece of the LDS tile
+template <int D, int NW>
+__device__ __forceinline__ void load_tile_piece(__amdgpu_buffer_rsrc_t rsrc, EMI_LDS uint8_t* tile, int wave, uint32_t lane_off,
+                                                int it, int row0, uint32_t row_bytes) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, tile + (it * NW + wave) * 1024, 16,
+                                           tile_piece_offset<D, NW>(lane_off, it, row0, row_bytes), 0, 0, 0);
 }
 
 // Operand fragment "32 tile rows x 16 of D": lane l holds row row_base + (l & 31),
@@ -671,12 +671,12 @@ __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(const uint16_t* __rest
       }
   }
   // Load n (0 .. LPB-1; K loads first, then V loads) of bundle jb into ring slot slot2.
-  const TileLaneOffsets<D, BKV, NW> lane_off = tile_lane_offsets<D, BKV, NW>(wave, lane, sh.ss);
+  const uint32_t lane_off = tile_lane_offset<D, NW>(wave, lane, sh.ss);
   const uint32_t row_bytes = (uint32_t)sh.ss * 2u;
   auto issue_one = [&](const int n, const int slot2, int jb) __attribute__((always_inline)) {
     constexpr int NL = LPB / 2;
-    if (n < NL) load_rows_one<D, BKV, NW>(rK, smem + slot2 * TILE, wave, lane_off, n, (jb + 1) * BKV, row_bytes);
-    else load_rows_one<D, BKV, NW>(rV, smem + 3 * TILE + slot2 * TILE, wave, lane_off, n - NL, jb * BKV, row_bytes);
+    if (n < NL) load_tile_piece<D, NW>(rK, smem + slot2 * TILE, wave, lane_off, n, (jb + 1) * BKV, row_bytes);
+    else load_tile_piece<D, NW>(rV, smem + 3 * TILE + slot2 * TILE, wave, lane_off, n - NL, jb * BKV, row_bytes);
   };
   // jb_issue: the bundle whose loads this phase issues (phases that compute both products only)
   auto mfma_phase = [&](auto do_s_c, auto do_pv_c, auto slot_c, int jb_issue) __attribute__((always_inline)) {
@@ -1069,13 +1069,13 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_sp_kernel(const uint16_t* __
   // The same loads one at a time (n = 0 .. LPB-1: Q rows, dO rows, statistics), for the steady state, where they
   // go out between MFMAs: issued together after the barrier, the 36 loads of a block queue up in the memory
   // pipeline and every wavefront, alone on its SIMD, waits for its last one with the matrix core idle.
-  const TileLaneOffsets<D, BQT, NW> lane_off = tile_lane_offsets<D, BQT, NW>(wave, lane, sh.ss);
+  const uint32_t lane_off = tile_lane_offset<D, NW>(wave, lane, sh.ss);
   const uint32_t row_bytes = (uint32_t)sh.ss * 2u;
   auto issue_part = [&](const int n, int ti, int slot) __attribute__((always_inline)) {
     constexpr int NLQ = (LPB - 1) / 2;
     const int row0 = (qt0 + ti) * BQT;
-    if (n < NLQ) load_rows_one<D, BQT, NW>(rQ, smem + slot * TILE, wave, lane_off, n, row0, row_bytes);
-    else if (n < 2 * NLQ) load_rows_one<D, BQT, NW>(rDO, smem + NSLOT * TILE + slot * TILE, wave, lane_off, n - NLQ, row0, row_bytes);
+    if (n < NLQ) load_tile_piece<D, NW>(rQ, smem + slot * TILE, wave, lane_off, n, row0, row_bytes);
+    else if (n < 2 * NLQ) load_tile_piece<D, NW>(rDO, smem + NSLOT * TILE + slot * TILE, wave, lane_off, n - NLQ, row0, row_bytes);
     else issue_stats(row0, slot);
   };
   constexpr int LA = (LPB + 1) / 2, LC = LPB - LA;        // loads issued inside stage A/B and inside stage C
