@@ -261,19 +261,6 @@ def bench_kernels(cfg, iters):
     # Single-token (decode) step at the 7B layer's widths: mat-vec over W [11008, 4096] and its
     # adjoints (weight read or written once), attention of one query per head over a
     # 4096-row cache for 8 sequences (cache rows read once; the adjoint also writes dK, dV).
-    D = cfg["dim"]
-    w = (torch.randn((H, D), device="cuda") * 0.02).to(bf)
-    xv, yv, dyv, dxv = (torch.randn(n_, device="cuda").to(bf) for n_ in (D, H, H, D))
-    dw = torch.empty_like(w)
-    gm = lambda A, Bm, C, M_, N_, K_, lda, ldb, ta, tb: N.check(lib.emi_gemm(st, P(A), P(Bm), None, P(C), M_, N_, K_, lda, ldb,
-                                                                             N_, N_, ta, tb, N.EMI_BF16))
-    hbm("step_matvec_bf16", lambda: gm(xv, w, yv, 1, H, D, D, D, 0, 1), w.numel() * 2, in_graph=True)
-    gwb = lib.emi_gemm_workspace_bytes(1, D, H, 0, 0, N.EMI_BF16)
-    gws = torch.empty(gwb, dtype=torch.uint8, device="cuda")
-    hbm("step_matvec_dx_bf16", lambda: N.check(lib.emi_gemm_ws(st, P(dyv), P(w), None, P(dxv), P(gws), gwb, 1, D, H, H, D, D, D, 0, 0,
-                                                               N.EMI_BF16)), w.numel() * 2, in_graph=True)
-    hbm("step_matvec_dw_bf16", lambda: gm(dyv, xv, dw, H, D, 1, H, D, 1, 0), w.numel() * 2, in_graph=True)
-    del w, dw, gws
     Bq, hq, Sk, dd = 8, 32, 4096, 128
     Dq = hq * dd
     qs, dos = (torch.randn((Bq, Dq), device="cuda").to(bf) for _ in range(2))
@@ -295,6 +282,21 @@ def bench_kernels(cfg, iters):
     hbm("step_attn_jvp_bf16", lambda: N.check(lib.emi_attn_step_jvp(st, P(qs), P(kc), P(vc), P(os_), P(lses), P(tqs), P(tkc), P(tvc),
                                                                     P(dqs), P(sws), swb, Bq, hq, Sk, dd, *strides, dd ** -0.5,
                                                                     N.EMI_BF16)), 4 * kc.numel() * 2)
+    del qs, dos, kc, vc, os_, dqs, lses, sws, tqs, tkc, tvc
+    # (the graph-timed entries last: stream-launch timings taken after a graph capture came out 10 % lower)
+    D = cfg["dim"]
+    w = (torch.randn((H, D), device="cuda") * 0.02).to(bf)
+    xv, yv, dyv, dxv = (torch.randn(n_, device="cuda").to(bf) for n_ in (D, H, H, D))
+    dw = torch.empty_like(w)
+    gm = lambda A, Bm, C, M_, N_, K_, lda, ldb, ta, tb: N.check(lib.emi_gemm(st, P(A), P(Bm), None, P(C), M_, N_, K_, lda, ldb,
+                                                                             N_, N_, ta, tb, N.EMI_BF16))
+    hbm("step_matvec_bf16", lambda: gm(xv, w, yv, 1, H, D, D, D, 0, 1), w.numel() * 2, in_graph=True)
+    gwb = lib.emi_gemm_workspace_bytes(1, D, H, 0, 0, N.EMI_BF16)
+    gws = torch.empty(gwb, dtype=torch.uint8, device="cuda")
+    hbm("step_matvec_dx_bf16", lambda: N.check(lib.emi_gemm_ws(st, P(dyv), P(w), None, P(dxv), P(gws), gwb, 1, D, H, H, D, D, D, 0, 0,
+                                                               N.EMI_BF16)), w.numel() * 2, in_graph=True)
+    hbm("step_matvec_dw_bf16", lambda: gm(dyv, xv, dw, H, D, 1, H, D, 1, 0), w.numel() * 2, in_graph=True)
+    del w, dw, gws
     return out
 
 
