@@ -17,8 +17,7 @@ def layer(x, lw, n_heads, eps=1e-5, theta=10000.0):
     """One decoder layer (test/llama.py:144-233).  x: [B, S, dim]."""
     xb = ops.rmsnorm(x, lw["rms_att_weight"], eps)                 # :145
     q, k, v = ops.matmul_nt_group(xb, (lw["wq"], lw["wk"], lw["wv"]))      # :149-157, one launch when the shapes agree
-    q = ops.rope(q, n_heads, theta)                                # :161-168
-    k = ops.rope(k, n_heads, theta)
+    q, k = ops.rope_pair(q, k, n_heads, theta)                     # :161-168
     att = ops.attention(q, k, v, n_heads, causal=True)             # :178-209
     x = ops.matmul_nt(att, lw["wo"], residual=x)                   # :211-215
     xb = ops.rmsnorm(x, lw["rms_ffn_weight"], eps)                 # :219

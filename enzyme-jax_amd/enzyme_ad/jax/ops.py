@@ -301,6 +301,57 @@ def rope(x, n_heads, theta=10000.0, pos0=0, inverse=False):
     return y
 
 
+_STACK_SMALL = 1 << 25        # elements: groups of results up to this size are laid out side by side so that a pair can share a launch
+
+
+def _adjacent(a, b):
+    """b starts where a ends (same shape, dtype, both contiguous): the two are one [2, ...] tensor in memory."""
+    return (a.shape == b.shape and a.dtype == b.dtype and a.is_contiguous() and b.is_contiguous()
+            and b.data_ptr() == a.data_ptr() + a.numel() * a.element_size())
+
+
+def rope_pair(q, k, n_heads, theta=10000.0, pos0=0):
+    """(rope(q), rope(k)) of test/llama.py:161-168.  When k lies right behind q in memory (the grouped projection lays
+    small results out that way) both are rotated by one launch, and so are their cotangents when the attention
+    adjoint hands them over the same way: for a small model a launch costs more than the rotation."""
+    if not _adjacent(q, k) or q.dim() != 3:
+        return rope(q, n_heads, theta, pos0), rope(k, n_heads, theta, pos0)
+    _dev(q, k)
+    B, S, D = q.shape
+    d = D // n_heads
+    if d * n_heads != D or d % 2:
+        raise ValueError("rope: dim %d is not n_heads=%d x even head_dim" % (D, n_heads))
+    table = rope_table(S, d, theta, pos0, q.device)
+    ybuf = torch.empty((2, B, S, D), dtype=q.dtype, device=q.device)
+    N.check(N.lib().emi_rope(_stream(), _p(q), _p(table), _p(ybuf), 2 * B, S, n_heads, d, 0, _code(q)))
+    yq, yk = ybuf[0], ybuf[1]
+
+    def rule(cs, acc):
+        cq, ck = cs
+        if cq is not None and ck is not None and _adjacent(cq, ck):
+            gbuf = torch.empty((2, B, S, D), dtype=cq.dtype, device=cq.device)
+            N.check(N.lib().emi_rope(_stream(), _p(cq), _p(table), _p(gbuf), 2 * B, S, n_heads, d, 1, _code(cq)))
+            gs = [gbuf[0], gbuf[1]]
+        else:
+            gs = []
+            for c in (cq, ck):
+                g = None
+                if c is not None:
+                    c = c.contiguous()
+                    g = torch.empty_like(c)
+                    N.check(N.lib().emi_rope(_stream(), _p(c), _p(table), _p(g), B, S, n_heads, d, 1, _code(c)))
+                gs.append(g)
+        return [None if g is None else _accumulate(a, g) for g, a in zip(gs, acc)]
+
+    Tape.record((q, k), (yq, yk), rule)
+    tans = _tan(q, k)
+    if tans is not None:
+        for y, t in zip((yq, yk), tans):
+            if t is not None:
+                _set_tan(y, _quiet(lambda t=t: rope(t, n_heads, theta, pos0)))          # linear
+    return yq, yk
+
+
 def rotate_pairs(x, table, inverse=False):
     """Rotate the adjacent pairs (2p, 2p+1) of the last dimension of x by the angles of an
     explicit fp32 (cos, sin) table [pairs, 2]: the batched 2x2 products of
@@ -522,6 +573,8 @@ def gemm_grouped(As, Bs, trans_a=False, trans_b=False, residuals=None, sum_into_
     if len(given) != len(rs) or any(o is not None and (tuple(o.shape) != (M, Nn) or o.dtype != a.dtype or not o.is_contiguous())
                                     for o in given):
         raise ValueError("gemm_grouped: outs must be contiguous [%d, %d] tensors of the operands' dtype, one per result" % (M, Nn))
+    if all(o is None for o in given) and 1 < len(given) and len(given) * M * Nn <= _STACK_SMALL:
+        given = list(torch.empty((len(given), M, Nn), dtype=a.dtype, device=a.device).unbind(0))     # side by side: see rope_pair
     outs = [torch.empty((M, Nn), dtype=a.dtype, device=a.device) if o is None else o for o in given]
     lib = N.lib()
     nbytes = lib.emi_gemm_grouped_workspace_bytes(n, M, Nn, K, int(trans_a), int(trans_b), int(sum_into_one), _code(a))
@@ -685,7 +738,10 @@ def attention(q, k, v, n_heads, scale=None, causal=True, layout="bshd", return_l
     o, lse, (B, S, d, sb, sh, ss) = attention_raw(q, k, v, n_heads, scale, causal, layout)
 
     def rule(c, acc):
-        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        if 3 * q.numel() <= _STACK_SMALL and q.is_contiguous():
+            dq, dk, dv = torch.empty((3,) + tuple(q.shape), dtype=q.dtype, device=q.device).unbind(0)   # side by side: see rope_pair
+        else:
+            dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
         nbytes = N.lib().emi_attn_bwd_workspace_bytes(B, n_heads, S, d)
         ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
         N.check(N.lib().emi_attn_bwd(_stream(), _p(q), _p(k), _p(v), _p(o), _p(lse), _p(c), _p(dq), _p(dk), _p(dv),

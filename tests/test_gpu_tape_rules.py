@@ -123,3 +123,34 @@ def test_stacked_weight_slice_selected_twice_or_used_twice():
         _, f_vjp = vjp(fn, w)
         (gw,) = f_vjp(c)
         assert np.max(np.abs(host(gw) - ref)) <= 1e-4 * np.max(np.abs(ref)), fn.__name__
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rope_pair_shares_a_launch_and_matches_two_ropes(dtype):
+    """rope_pair on operands that lie side by side (as the grouped projection returns them) and on operands that do
+    not: outputs and both cotangents equal those of two separate rope calls, bit for bit."""
+    from enzyme_ad.jax import ops
+    B, S, H, d = 2, 37, 3, 16
+    buf = _randn((2, B, S, H * d), 11).to(dtype)
+    cot = _randn((2, B, S, H * d), 12).to(dtype)
+    for side_by_side in (True, False):
+        q, k = (buf[0], buf[1]) if side_by_side else (buf[0].clone(), buf[1].clone())
+        cq, ck = (cot[0], cot[1]) if side_by_side else (cot[0].clone(), cot[1].clone())
+        with ops.Tape() as tape:
+            yq, yk = ops.rope_pair(q, k, H)
+        gq, gk = tape.backward([yq, yk], [cq, ck], [q, k])
+        with ops.Tape() as tape2:
+            rq, rk = ops.rope(q, H), ops.rope(k, H)
+        hq, hk = tape2.backward([rq, rk], [cq, ck], [q, k])
+        for a, b in ((yq, rq), (yk, rk), (gq, hq), (gk, hk)):
+            assert torch.equal(a, b)
+    # a cotangent on one of the two results only
+    q, k = buf[0], buf[1]
+    with ops.Tape() as tape:
+        yq, yk = ops.rope_pair(q, k, H)
+    gq, gk = tape.backward([yk], [cot[1]], [q, k])
+    with ops.Tape() as tape2:
+        rk = ops.rope(k, H)
+    (hk,) = tape2.backward([rk], [cot[1]], [k])
+    assert gq is None or not bool(gq.any())
+    assert torch.equal(gk, hk)
