@@ -747,9 +747,9 @@ __global__ __launch_bounds__(512) void gemm_bf16_pingpong_kernel(const uint16_t*
 #pragma unroll
     for (int ks = 0; ks < 2; ks++)
 #pragma unroll
-      for (int i = 0; i < 4; i++)
+      for (int j = 0; j < 4; j++)
 #pragma unroll
-        for (int j = 0; j < 4; j++)
+        for (int i = 0; i < 4; i++)
           acc[h * 4 + i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb[j][ks], fa[i][ks], acc[h * 4 + i][j], 0, 0, 0);
     __builtin_amdgcn_s_setprio(0);
     slot_end();
