@@ -19,6 +19,7 @@ instead of costing an extra pass over HBM.
 import math
 
 import ctypes
+import threading
 
 import torch
 
@@ -85,10 +86,62 @@ def _same_dtype(*ts):
 # tape
 # ---------------------------------------------------------------------------
 
-class Tape:
-    """Linear record of operator applications for reverse mode."""
+_tls = threading.local()      # the active Tape / Forward context and the running reverse passes of this thread
 
-    _active = None
+
+class _PerThread(type):
+    """`Tape._active` / `Forward._active` are per thread: executor threads that differentiate different functions at
+    the same time (the reference guards its registries for the same reason, enzyme_call.cc:173,263) never see each
+    other's context."""
+
+    @property
+    def _active(cls):
+        return getattr(_tls, cls.__name__, None)
+
+    @_active.setter
+    def _active(cls, value):
+        setattr(_tls, cls.__name__, value)
+
+
+class _Pass:
+    """What one Tape.backward call shares between its rules: the in-place gradient buffers of stacked weights, the
+    deferred weight-gradient products and the weight transposes.  One object per call, kept on a per-thread stack, so
+    that a reverse pass started inside a rule of another one (or on another thread) has its own."""
+
+    def __init__(self, tape):
+        ok, other, seen, twice, uses, selects = set(), set(), set(), set(), {}, {}
+        for inputs, _, rule in tape.nodes:
+            sel = getattr(rule, "_emi_select", None)
+            for t in inputs:
+                if isinstance(t, torch.Tensor):
+                    uses[id(t)] = uses.get(id(t), 0) + 1
+                    if sel is None:
+                        other.add(id(t))
+                    else:
+                        ok.add(id(t))
+                        selects[id(t)] = selects.get(id(t), 0) + 1
+                        if (id(t), sel) in seen:
+                            twice.add(id(t))
+                        seen.add((id(t), sel))
+        # a stacked tensor that an operator on this tape produced (a converted or scaled copy of master weights) is
+        # not eligible: its producer's rule runs before the deferred products have written the buffer
+        self.ok = ok - other - twice - tape.produced
+        self.buf = {}
+        self.handed = set()
+        self.uses = uses
+        self.selects = selects           # id(stack) -> number of slices selected on this tape
+        self.pending_dw = []
+        self.pending_dw_bytes = 0
+        self.transposed = {}             # (data_ptr, shape, dtype) -> (a^T, a)
+
+
+def _pass():
+    stack = getattr(_tls, "passes", None)
+    return stack[-1] if stack else None
+
+
+class Tape(metaclass=_PerThread):
+    """Linear record of operator applications for reverse mode."""
 
     def __init__(self):
         self.nodes = []          # (inputs, output, rule)
@@ -113,9 +166,16 @@ class Tape:
 
     def backward(self, outputs, cotangents, wrt):
         """Cotangents of `wrt` (list of tensors) given cotangents of `outputs`."""
+        if not hasattr(_tls, "passes"):
+            _tls.passes = []
+        _tls.passes.append(_Pass(self))
+        try:
+            return self._backward(outputs, cotangents, wrt)
+        finally:
+            _tls.passes.pop()            # also on an exception: nothing of the pass outlives it
+
+    def _backward(self, outputs, cotangents, wrt):
         ct = {}
-        _transposed.clear()
-        _stack_reset(self.nodes)
         for o, c in zip(outputs, cotangents):
             if c is None:
                 continue
@@ -144,18 +204,14 @@ class Tape:
                 ct[id(i)] = g if id(i) not in done else add(ct[id(i)], g)
                 done.add(id(i))
         _flush_dw()
-        _transposed.clear()
-        _stack_reset(())
         return [ct.get(id(w)) for w in wrt]
 
 
-class Forward:
+class Forward(metaclass=_PerThread):
     """Forward mode: tangents travel with the primal values.  While a Forward context is
     active every operator also computes the tangent of its result from the tangents of
     its operands (None = zero) with the forward kernels; linear operators reuse their own
     kernel on the tangent."""
-
-    _active = None
 
     def __init__(self):
         self.tan = {}            # id(primal tensor) -> tangent tensor
@@ -261,6 +317,7 @@ def rmsnorm(x, gamma, eps=1e-5):
 
 
 _rope_tables = {}
+_rope_tables_lock = threading.Lock()
 
 
 def rope_table(seq, head_dim, theta=10000.0, pos0=0, device=None):
@@ -270,9 +327,17 @@ def rope_table(seq, head_dim, theta=10000.0, pos0=0, device=None):
     key = (str(device), seq, head_dim, float(theta), pos0)
     t = _rope_tables.get(key)
     if t is None:
-        t = torch.empty((seq, head_dim // 2, 2), dtype=torch.float32, device=device)
-        N.check(N.lib().emi_rope_table(_stream(), _p(t), seq, head_dim, float(theta), pos0))
-        _rope_tables[key] = t
+        with _rope_tables_lock:
+            t = _rope_tables.get(key)
+            if t is None:
+                t = torch.empty((seq, head_dim // 2, 2), dtype=torch.float32, device=device)
+                N.check(N.lib().emi_rope_table(_stream(), _p(t), seq, head_dim, float(theta), pos0))
+                # the table is shared by every stream of the process: it is complete before anyone else can find it
+                # (a one-time wait at what is trace time in the reference; never reached under graph capture, whose
+                # eager warm-up run has filled the cache)
+                if not torch.cuda.is_current_stream_capturing():
+                    torch.cuda.current_stream().synchronize()
+                _rope_tables[key] = t
     return t
 
 
@@ -417,52 +482,28 @@ def transpose(a):
 
 
 # Gradients of the slices of a stacked per-layer weight (`wq[l]`): when every use of the stacked tensor on the tape is
-# a `select` and no slice is selected twice, the kernel that produces a slice's gradient writes it straight into
-# slice l of one zero-filled buffer shaped like the stacked tensor, instead of into a temporary that the select rule
-# then adds in.  Valid for the duration of one Tape.backward.
-_stack = {"ok": set(), "buf": {}, "handed": set(), "uses": {}}
-
-
-def _stack_reset(nodes):
-    ok, other, seen, twice, uses = set(), set(), set(), set(), {}
-    for inputs, _, rule in nodes:
-        sel = getattr(rule, "_emi_select", None)
-        for t in inputs:
-            if isinstance(t, torch.Tensor):
-                uses[id(t)] = uses.get(id(t), 0) + 1
-                if sel is None:
-                    other.add(id(t))
-                else:
-                    ok.add(id(t))
-                    if (id(t), sel) in seen:
-                        twice.add(id(t))
-                    seen.add((id(t), sel))
-    _stack["ok"] = ok - other - twice
-    _stack["buf"] = {}
-    _stack["handed"] = set()
-    _stack["uses"] = uses
-    _pending_dw[:] = []
-    _pending_dw_bytes[0] = 0
-
-
+# a `select`, no slice is selected twice and the stack is a leaf, the kernel that produces a slice's gradient writes it
+# straight into slice l of one zero-filled buffer shaped like the stacked tensor, instead of into a temporary that the
+# select rule then adds in.  The buffers belong to the running reverse pass (`_Pass`).
+#
 # Weight gradients dW = dY^T . X whose destination is a slice of such a buffer feed nothing else in the backward
 # pass, so they wait: at the end of Tape.backward the products of one shape (the same weight of every layer) run as
 # one grouped launch, which fills the chip without split-K partials (12 x [768, 768] over 8192 tokens: 446 -> 173 us).
-_pending_dw = []
-_pending_dw_bytes = [0]
 _PENDING_DW_BYTES = 6 << 30          # cotangents kept alive for the deferred products, at most
 
 
 def _defer_dw(c2, x2, target):
-    _pending_dw.append((c2, x2, target))
-    _pending_dw_bytes[0] += c2.numel() * c2.element_size()
-    if _pending_dw_bytes[0] > _PENDING_DW_BYTES:
+    ps = _pass()
+    ps.pending_dw.append((c2, x2, target))
+    ps.pending_dw_bytes += c2.numel() * c2.element_size()
+    if ps.pending_dw_bytes > _PENDING_DW_BYTES:
         _flush_dw()
 
 
 def _flush_dw():
-    todo, _pending_dw[:] = list(_pending_dw), []
-    _pending_dw_bytes[0] = 0
+    ps = _pass()
+    todo, ps.pending_dw = ps.pending_dw, []
+    ps.pending_dw_bytes = 0
     by_shape = {}
     for c2, x2, target in todo:
         by_shape.setdefault((tuple(c2.shape), tuple(x2.shape), c2.dtype), []).append((c2, x2, target))
@@ -472,10 +513,10 @@ def _flush_dw():
             gemm_grouped([c for c, _, _ in part], [x for _, x, _ in part], True, False, outs=[t for _, _, t in part])
 
 
-def _stack_buffer(w):
-    buf = _stack["buf"].get(id(w))
+def _stack_buffer(ps, w):
+    buf = ps.buf.get(id(w))
     if buf is None:
-        buf = _stack["buf"][id(w)] = torch.zeros_like(w)        # device memset
+        buf = ps.buf[id(w)] = torch.zeros_like(w)        # device memset
     return buf
 
 
@@ -484,39 +525,42 @@ def _grad_target(t, acc):
     slice of an eligible stacked tensor and the caller is its only consumer (with two, the second would read the first
     one's gradient as its residual before a deferred product has written it)."""
     st = getattr(t, "_emi_stack", None)
-    if acc is not None or st is None or id(st[0]) not in _stack["ok"] or id(t) in _stack["handed"] or \
-            _stack["uses"].get(id(t), 0) != 1:
+    ps = _pass()
+    if acc is not None or st is None or ps is None or id(st[0]) not in ps.ok or id(t) in ps.handed or \
+            ps.uses.get(id(t), 0) != 1:
         return None
-    _stack["handed"].add(id(t))
-    return _stack_buffer(st[0])[st[1]]
-
-
-_transposed = {}      # (data_ptr, shape) -> a^T, valid for the duration of one Tape.backward
+    ps.handed.add(id(t))
+    return _stack_buffer(ps, st[0])[st[1]]
 
 
 def _transpose_shared(a):
     """a^T, computed once per reverse pass however many adjoint GEMMs read it.  A slice of a stacked per-layer
-    weight takes its transpose from one batched transpose of the whole stack (one launch for all layers)."""
+    weight takes its transpose from one batched transpose of the whole stack (one launch for all layers) when at
+    least half of the stack's slices are selected on the tape; a pass over one layer of a deep stack transposes
+    that slice alone."""
+    ps = _pass()
+    cache = ps.transposed if ps is not None else {}
     st = getattr(a, "_emi_stack", None)
-    if st is not None and st[0].dim() == 3 and st[0].is_contiguous():
+    if st is not None and st[0].dim() == 3 and st[0].is_contiguous() and ps is not None and \
+            2 * ps.selects.get(id(st[0]), 0) >= st[0].shape[0]:
         w, i = st
         skey = ("stack", w.data_ptr(), tuple(w.shape), w.dtype)
-        hit = _transposed.get(skey)
+        hit = cache.get(skey)
         if hit is None:
             L_, rows, cols = w.shape
             out = torch.empty((L_, cols, rows), dtype=w.dtype, device=w.device)
             i64 = lambda v: (ctypes.c_int64 * len(v))(*v)
             N.check(N.lib().emi_strided_copy(_stream(), _p(w), _p(out), 3, i64([L_, cols, rows]), i64([rows * cols, 1, cols]), 0,
                                              i64([rows * cols, rows, 1]), 0, w.element_size()))
-            hit = _transposed[skey] = (out, w)
+            hit = cache[skey] = (out, w)
         return hit[0][i]
     key = (a.data_ptr(), tuple(a.shape), a.dtype)
-    hit = _transposed.get(key)
+    hit = cache.get(key)
     if hit is None:
         rows, cols = a.shape
         out = torch.empty((cols, rows), dtype=a.dtype, device=a.device)
         N.check(N.lib().emi_transpose(_stream(), _p(a), _p(out), rows, cols, _code(a)))
-        hit = _transposed[key] = (out, a)       # keeps `a` alive so the pointer cannot be reused
+        hit = cache[key] = (out, a)       # keeps `a` alive so the pointer cannot be reused
     return hit[0]
 
 
@@ -897,15 +941,17 @@ def select(w, i):
     Adjoint (Slice rule, StableHLOAutoDiffOpInterfaceImpl.cpp:1586-1620): the
     cotangent is placed into slice i of a zero tensor shaped like w."""
     _dev(w)
+    i = int(i) % w.shape[0]             # w[-1] and w[L-1] are one slice
     y = w[i]
     y._emi_stack = (w, i)
 
     def rule(c, acc):
         g = acc[0]
-        if id(w) in _stack["ok"]:
+        ps = _pass()
+        if ps is not None and id(w) in ps.ok:
             # every cotangent of w comes from select rules, one per slice: slice i of the shared buffer is either
             # already written (the producer was handed it) or still zero
-            buf = _stack_buffer(w)
+            buf = _stack_buffer(ps, w)
             if c.data_ptr() != buf[i].data_ptr():
                 buf[i].copy_(c)              # device-to-device copy
             return (buf,)

@@ -77,7 +77,7 @@ def test_ffi_handlers_launch_on_the_frame_stream():
         dx = torch.empty((128, 256), dtype=torch.bfloat16, device="cuda")
         _call("emi_gemm_grouped_ffi", xla, [_buf(xla, c_) for c_ in cs3] + [_buf(xla, w_) for w_, _ in ws3], [_buf(xla, dx)],
               {"count": (F.S64, 3), "sum": (F.PRED, 1), "trans_a": (F.PRED, 0), "trans_b": (F.PRED, 0)})
-        check(dx, sum(host(c_) @ wr_ for c_, (_, wr_) in zip(cs3, ws3)), "bf16", "ffi grouped gemm, summed", factor=2.0)
+        check(dx, sum(host(c_) @ wr_ for c_, (_, wr_) in zip(cs3, ws3)), "bf16", "ffi grouped gemm, summed")
         # attention fwd + bwd, [B, S, h, d] layout
         B, S, h, d = 1, 96, 2, 128
         (q, qr), (k, kr), (v, vr), (do, dor) = (dev(rng.standard_normal((B, S, h, d)), "bf16") for _ in range(4))

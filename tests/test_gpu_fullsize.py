@@ -41,7 +41,7 @@ def test_c2_rmsnorm_rope_full_size(dt):
     check(dx.reshape(-1, D)[rows], L.rmsnorm_bwd(xs, gr, dys)[0], dt, "rmsnorm dx rows")
     x64, dy64 = x.reshape(-1, D).double(), dy.reshape(-1, D).double()
     r = torch.rsqrt((x64 * x64).mean(dim=1, keepdim=True) + 1e-5)
-    check(dg, (dy64 * x64 * r).sum(dim=0).cpu().numpy(), dt, "dgamma over 32768 rows", factor=2.0 if dt == "bf16" else 1.0)
+    check(dg, (dy64 * x64 * r).sum(dim=0).cpu().numpy(), dt, "dgamma over 32768 rows")
     with ops.Tape() as tape:
         z = ops.rope(x, h)
     back = ops.rope(z, h, inverse=True)

@@ -125,6 +125,8 @@ def test_c4_gemm_shapes_sampled(shape):
     # (B, h, S, d, layout, heads checked): C3 and the attention of C5
     (8, 32, 2048, 128, "bhsd", [(0, 0), (5, 17), (7, 31)]),
     (4, 32, 4096, 128, "bshd", [(0, 0), (3, 31)]),
+    # the attention of C4 (stories110M: 12 heads of 64, seq 1024, batch 8) at its own grid
+    (8, 12, 1024, 64, "bshd", [(0, 0), (7, 11)]),
 ])
 def test_attention_whole_heads_full_size(cfg):
     """Every row of o, lse, dQ, dK and dV of a few (batch, head) pairs against the oracle, with the kernels running
@@ -145,10 +147,15 @@ def test_attention_whole_heads_full_size(cfg):
         for name, got, ref in (("o", o, ro), ("dq", dq, rdq), ("dk", dk, rdk), ("dv", dv, rdv)):
             g = host(pick(got, b, hh))
             check(g, ref[0, 0], "bf16", "%s of (batch %d, head %d)" % (name, b, hh))
-            # row by row the gradients are held to 4x the bound: with few keys dS = P (dP - delta) cancels
-            # (delta is built from the rounded O), so a row's own error is not bounded by one bf16 rounding;
-            # a misplaced or missing row is off by ~100 %
-            check_rows(g, ref[0, 0], "bf16", "%s rows of (batch %d, head %d)" % (name, b, hh), factor=1.0 if name == "o" else 4.0)
+            # Beyond the contract's per-tensor bound: every row against its own maximum.  Outputs hold 2e-2 row by
+            # row.  Gradient rows are held to 4x that: where a query sees few keys, dS = P (dP - delta) cancels to a
+            # small difference while delta = rowsum(dO . O) carries the rounding of the stored bf16 O (|error| about
+            # 2^-9 |dO| |O| sqrt(d)), so a row's own error is not bounded by one bf16 rounding of its largest entry
+            # (measured worst rows: dq 2.3e-2 at query 1 of a head, dk / dv below 1e-2); a misplaced or missing row
+            # would be off by ~100 %.
+            worst = check_rows(g, ref[0, 0], "bf16", "%s rows of (batch %d, head %d)" % (name, b, hh),
+                               factor=1.0 if name == "o" else 4.0)
+            print("attention %s (batch %d, head %d) of %s: worst row-relative error %.3e" % (name, b, hh, cfg[:4], worst), flush=True)
 
 
 def _layer_weights(D, H, dt, seed):
@@ -217,3 +224,46 @@ def test_c5_width_short_sequence_every_gradient():
         check(gw[k_], rgw[k_], "bf16", "d" + k_)
         if rgw[k_].ndim == 2:
             check_rows(host(gw[k_]), rgw[k_], "bf16", "rows of d" + k_)
+
+
+def test_c4_model_every_gradient_from_prefix_cotangent():
+    """The 110M configuration at its own size (12 layers, dim 768, hidden 2048, 12 heads of 64, vocabulary 32000,
+    batch 8 x seq 1024, bf16, tokens in, logits out) with a logits cotangent that is non-zero on the first 32
+    positions of every sequence only.  By causality the reverse pass depends on those positions alone, so the oracle
+    redoes it whole: the logits on the prefixes and every weight gradient (per layer, `wcls`, the final gain, the
+    embedding table) at the contract's bound, while the kernels run their full-size launches (the deferred weight
+    gradients contract over all 8192 tokens, the head_dim-64 attention kernels run the 8 x 12 x 1024 grid)."""
+    from enzyme_ad.jax import enzyme_jax_ir, JaXPipeline, vjp, llama
+    from gpu_util import dev
+    cfg = {"dim": 768, "hidden_dim": 2048, "n_layers": 12, "n_heads": 12, "n_kv_heads": 12, "vocab_size": 32000, "seq_len": 1024}
+    B, S, P = 8, 1024, 32
+    w = L.make_weights(cfg, 4, std=0.02, norm_gain="uniform")
+    wd, wr = {}, {}
+    for k_, a in w.items():
+        wd[k_], wr[k_] = dev(a, "bf16")
+    rng = np.random.Generator(np.random.PCG64(1004))
+    tok = rng.integers(0, cfg["vocab_size"], size=(B, S))
+    tokd = torch.from_numpy(tok.astype(np.int32)).cuda()
+
+    @enzyme_jax_ir(pipeline_options=JaXPipeline(), inner_jit=False)
+    def fn(weights):
+        return llama.forward(tokd, cfg, weights, logits=True)
+
+    out, f_vjp = vjp(fn, wd)
+    dout = _randn(tuple(out.shape), "bf16", 91)
+    dout[:, P:] = 0
+    (gw,) = f_vjp(dout)
+    ref, fcache = L.model_fwd(tok[:, :P], wr, cfg, logits=True)
+    check(out[:, :P], ref, "bf16", "logits on the prefixes")
+    _, rgw = L.model_bwd(host(dout[:, :P]), wr, cfg, fcache)
+    assert set(rgw) == set(gw)
+    for k_ in sorted(rgw):
+        e = check(gw[k_], rgw[k_], "bf16", "d" + k_)
+        print("C4 prefix cotangent: d%s max relative error %.3e" % (k_, e), flush=True)
+        if rgw[k_].ndim == 3:
+            # per layer, for the record (beyond the contract, which bounds each gradient tensor as a whole): twelve
+            # layers of bf16 activations separate the last layer's cotangent from the first layer's weights, and a
+            # layer's own maximum can be far below the stack's (measured worst: dwk[6] 2.6e-2 of that layer's maximum)
+            per = [rel_err(host(gw[k_][l]), rgw[k_][l]) for l in range(cfg["n_layers"])]
+            print("    per layer: worst %.3e (layer %d)" % (max(per), int(np.argmax(per))), flush=True)
+            assert max(per) <= 4e-2

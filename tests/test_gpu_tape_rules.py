@@ -154,3 +154,116 @@ def test_rope_pair_shares_a_launch_and_matches_two_ropes(dtype):
     (hk,) = tape2.backward([rk], [cot[1]], [k])
     assert gq is None or not bool(gq.any())
     assert torch.equal(gk, hk)
+
+
+def test_stack_produced_on_the_tape_takes_the_general_slice_rule():
+    """A stacked weight that an operator on the tape produced (bf16 copy of fp32 master weights) is sliced and
+    multiplied: its producer's rule runs before any deferred product could have filled an in-place buffer, so such a
+    stack must take the general Slice rule.  Also `w[-1]` and `w[L-1]` are one slice (its two cotangents add)."""
+    from enzyme_ad.jax import ops, hlo_ops as H, vjp
+    L_, T, D, Hd = 3, 72, 64, 96
+    w32 = _randn((L_, Hd, D), 40) * 0.1
+    x = _randn((T, D), 41).to(torch.bfloat16)
+
+    def fn(w32):
+        w = H.convert(w32, torch.bfloat16)
+        y0 = ops.matmul_nt(x, ops.select(w, 0))
+        y2 = ops.matmul_nt(x, ops.select(w, 2))
+        y2b = ops.matmul_nt(x, ops.select(w, -1))
+        return y0, y2, y2b
+
+    ys, f_vjp = vjp(fn, w32)
+    cs = [_randn((T, Hd), 42 + i).to(torch.bfloat16) for i in range(3)]
+    (g,) = f_vjp(tuple(cs))
+    assert g.dtype == torch.float32
+    xr = host(x)
+    ref = np.zeros((L_, Hd, D))
+    ref[0] = host(cs[0]).T @ xr
+    ref[2] = host(cs[1]).T @ xr + host(cs[2]).T @ xr
+    assert float(g[1].abs().max()) == 0.0
+    assert np.max(np.abs(host(g) - ref)) <= 2e-2 * np.max(np.abs(ref))
+
+
+def _small_model(seed):
+    cfg = {"dim": 64, "hidden_dim": 96, "n_layers": 2, "n_heads": 2, "n_kv_heads": 2, "vocab_size": 50, "seq_len": 48}
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    r = lambda *s: torch.randn(s, device="cuda", generator=g) * 0.1
+    Lc, D, Hd = cfg["n_layers"], cfg["dim"], cfg["hidden_dim"]
+    w = {"rms_att_weight": r(Lc, D) + 1, "rms_ffn_weight": r(Lc, D) + 1, "rms_final_weight": r(D) + 1,
+         "wq": r(Lc, D, D), "wk": r(Lc, D, D), "wv": r(Lc, D, D), "wo": r(Lc, D, D),
+         "w1": r(Lc, Hd, D), "w3": r(Lc, Hd, D), "w2": r(Lc, D, Hd)}
+    x = torch.randn((2, 48, D), device="cuda", generator=g)
+    dy = torch.randn((2, 48, D), device="cuda", generator=g)
+    return cfg, w, x, dy
+
+
+def test_reverse_passes_on_two_threads_match_the_serial_run():
+    """The active tape and everything a reverse pass shares between its rules (in-place gradient buffers of stacked
+    weights, deferred weight-gradient products, weight transposes) are per thread and per pass: two threads that each
+    differentiate their own model on their own stream, many times over, get the bits of the serial run (handlers run
+    on executor threads in the reference, enzyme_call.cc:173,263)."""
+    import threading
+    from enzyme_ad.jax import vjp, llama
+
+    def run(seed):
+        cfg, w, x, dy = _small_model(seed)
+        y, f_vjp = vjp(lambda x, w: llama.forward(x, cfg, w), x, w)
+        gx, gw = f_vjp(dy)
+        return [y, gx] + [gw[k] for k in sorted(gw)]
+
+    serial = {seed: [t.clone() for t in run(seed)] for seed in (1, 2)}
+    torch.cuda.synchronize()
+    results, errors = {}, []
+
+    def worker(seed):
+        try:
+            stream = torch.cuda.Stream()                       # default priority
+            with torch.cuda.stream(stream):
+                for _ in range(6):
+                    out = run(seed)
+                stream.synchronize()
+            results[seed] = out
+        except Exception as e:                                 # surfaced in the main thread
+            errors.append(e)
+
+    threads = [threading.Thread(target=worker, args=(seed,)) for seed in (1, 2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for seed in (1, 2):
+        for a, b in zip(results[seed], serial[seed]):
+            assert torch.equal(a, b)
+
+
+def test_vjp_inside_a_rule_of_another_reverse_pass():
+    """A reverse pass started while another one is running (a rule that itself differentiates a function) has its own
+    buffers: the outer pass's in-place stacked gradients and deferred products are untouched by it."""
+    from enzyme_ad.jax import ops, vjp, llama
+    cfg, w, x, dy = _small_model(3)
+    cfg2, w2, x2, dy2 = _small_model(4)
+    y, f_vjp = vjp(lambda x, w: llama.forward(x, cfg, w), x, w)
+    gx_ref, gw_ref = f_vjp(dy)
+    y2, f_vjp2 = vjp(lambda x, w: llama.forward(x, cfg2, w), x2, w2)
+    gx2_ref, gw2_ref = f_vjp2(dy2)
+    inner = {}
+
+    def fn(x, w):
+        h = llama.forward(x, cfg, w)
+        out = ops.add(h, h)
+
+        def rule(c, acc):
+            # runs in the middle of the outer pass, before the layers' rules
+            _, g = vjp(lambda x, w: llama.forward(x, cfg2, w), x2, w2)
+            inner["g"] = g(dy2)
+            return (ops._accumulate(acc[0], c), ops._accumulate(acc[1], c))
+
+        ops.Tape._active.nodes[-1] = (ops.Tape._active.nodes[-1][0], out, rule)
+        return out
+
+    out, f = vjp(fn, x, w)
+    gx, gw = f(dy)
+    gx_in, gw_in = inner["g"]
+    assert torch.equal(gx_in, gx2_ref) and all(torch.equal(gw_in[k], gw2_ref[k]) for k in gw2_ref)
+    assert torch.equal(gx, gx_ref * 2) and all(torch.equal(gw[k], gw_ref[k] * 2) for k in gw_ref)
