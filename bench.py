@@ -13,8 +13,11 @@ Prints ONE JSON line on stdout (everything else goes to stderr):
             algorithmic flops / HIP-event time of exactly those launches
   kernels   the same figure for every other kernel of the path at its
             configuration-C2/C3/C5 shape (HBM GB/s or MFMA TFLOP/s)
-  cpu_baseline  the numpy oracle of the same layer timed on the host cores on
-            a bounded sample (reported next to the GPU number, not a target)
+            (`vendor`: torch.matmul = hipBLASLt timed on the same launches in the same
+            run, a yardstick only: the library is never on the product path)
+  cpu_baseline  a PyTorch-CPU fp32 restatement of test/llama.py (oracle/llama_torch.py,
+            autograd as the VJP) timed on the host cores on a bounded sample
+            (reported next to the GPU number, not a target)
 """
 import argparse
 import json
@@ -114,7 +117,22 @@ def bench_gemms(cfg, iters):
         fl = sum(c[3] for c in mine)
         per_role[role] = dict(launches=len(mine), seconds=t, tflops=fl / t / 1e12)
     t_all = event_time(lambda: [ops.gemm(a, b, r == "dW", r != "dW") for (r, a, b, _) in calls], iters)
-    return t_all, sum(c[3] for c in calls), len(calls), per_role
+    # per distinct shape of the forward (NT) products, this library and the vendor library side by side
+    per_shape = {}
+    for (role, a, b, fl) in calls:
+        key = "%s_%dx%dx%d" % (role, a.shape[1] if role == "dW" else a.shape[0], b.shape[1] if role == "dW" else b.shape[0],
+                               a.shape[0] if role == "dW" else a.shape[1])
+        if key in per_shape:
+            continue
+        ta, tb = (True, False) if role == "dW" else (False, True)
+        t_own = event_time(lambda: ops.gemm(a, b, ta, tb), iters)
+        t_ven = event_time((lambda: torch.matmul(a.t(), b)) if role == "dW" else (lambda: torch.matmul(a, b.t())), iters)
+        per_shape[key] = dict(tflops=round(fl / t_own / 1e12, 1), vendor_tflops=round(fl / t_ven / 1e12, 1))
+    t_vendor = event_time(lambda: [torch.matmul(a.t(), b) if r == "dW" else torch.matmul(a, b.t()) for (r, a, b, _) in calls], iters)
+    vendor = dict(library="torch.matmul (hipBLASLt), same operands, same run; yardstick only",
+                  tflops=round(sum(c[3] for c in calls) / t_vendor / 1e12, 1), avg_launch_us=round(t_vendor / len(calls) * 1e6, 1),
+                  per_shape=per_shape)
+    return t_all, sum(c[3] for c in calls), len(calls), per_role, vendor
 
 
 def bench_kernels(cfg, iters):
@@ -485,15 +503,16 @@ def cpu_baseline(cfg, repeats=5, budget_s=25.0):
 
     def min_time(fn, budget):
         fn()                                            # warm-up
-        best, t_start = None, time.perf_counter()
+        best, taken, t_start = None, 0, time.perf_counter()
         for _ in range(repeats):
             t0 = time.perf_counter()
             fn()
             dt = time.perf_counter() - t0
             best = dt if best is None else min(best, dt)
+            taken += 1
             if time.perf_counter() - t_start > budget:
                 break
-        return best
+        return best, taken
 
     g = torch.Generator().manual_seed(1)
     # C1: dim 288, hidden 768, 6 layers, 6 heads, vocab 32000, batch 1 x seq 256, fp32, cotangent on the logits
@@ -511,7 +530,7 @@ def cpu_baseline(cfg, repeats=5, budget_s=25.0):
             t.grad = None
         LT.model(tok, w1, c1, True).backward(dlogits)
 
-    t_c1 = min_time(c1_step, 6.0)
+    t_c1, n_c1 = min_time(c1_step, 6.0)
     del w1, dlogits
 
     # the headline layer (dim 4096, hidden 11008, 32 heads) on one sequence of 512 tokens
@@ -529,12 +548,12 @@ def cpu_baseline(cfg, repeats=5, budget_s=25.0):
             t.grad = None
         LT.layer(x, lw, nh).backward(dy)
 
-    t_layer = min_time(layer_step, budget_s - 8.0)
+    t_layer, n_layer = min_time(layer_step, budget_s - 8.0)
     return dict(value=round(B * S / t_layer, 1), unit="tokens/s", cores=threads, kind="port", cpu=_cpu_model_name(),
                 sample="PyTorch-CPU fp32 restatement of test/llama.py (oracle/llama_torch.py), forward + autograd VJP, "
-                       "torch.set_num_threads(%d), warm-up 1, min of up to %d runs: the 7B layer of the GPU figure on "
-                       "batch 1 x seq 512 = 512 tokens (%.3f s per step)" % (threads, repeats, t_layer),
-                c1_stories15m=dict(tokens_per_s=round(256 / t_c1, 1), seconds_per_step=round(t_c1, 4),
+                       "torch.set_num_threads(%d), warm-up 1, min of %d timed runs (at most %d within the time budget): the 7B "
+                       "layer of the GPU figure on batch 1 x seq 512 = 512 tokens (%.3f s per step)" % (threads, n_layer, repeats, t_layer),
+                c1_stories15m=dict(tokens_per_s=round(256 / t_c1, 1), seconds_per_step=round(t_c1, 4), timed_runs=n_c1,
                                    sample="whole 15M model (dim 288, hidden 768, 6 layers, 6 heads, vocab 32000), "
                                           "batch 1 x seq 256 tokens -> logits, cotangent on the logits, fp32"))
 
@@ -622,15 +641,17 @@ def main():
         modes = optional("programs", programs)
         log("layer programs:", modes)
 
-    t_gemm, gemm_fl, n_gemm, per_layout = bench_gemms(cfg, max(5, min(args.steps, 20)))
+    t_gemm, gemm_fl, n_gemm, per_layout, vendor = bench_gemms(cfg, max(5, min(args.steps, 20)))
     roofline = dict(bound="mfma", kernel="gemm_bf16_pingpong_kernel (256x256x64 tiles; %d launches per step: Y, dX in the NT form, dW in the TN form, 7 weights)" % n_gemm,
                     achieved=gemm_fl / t_gemm / 1e12, peak=PEAK_BF16_TFLOPS, unit="TFLOP/s",
                     frac=gemm_fl / t_gemm / 1e12 / PEAK_BF16_TFLOPS,
                     traffic=GEMM_TRAFFIC_BYTES_PER_LAUNCH if (args.seq, args.batch) == (C5["seq"], C5["batch"]) else None,
                     avg_launch_us=t_gemm / n_gemm * 1e6, flops_per_launch=gemm_fl / n_gemm,
                     per_role={k: dict(tflops=round(v["tflops"], 1), avg_launch_us=round(v["seconds"] / v["launches"] * 1e6, 1))
-                                for k, v in per_layout.items()})
+                                for k, v in per_layout.items()},
+                    vendor=vendor)
     log("GEMM: %.1f TFLOP/s (%.1f%% of bf16 MFMA peak); per role %s" % (roofline["achieved"], 100 * roofline["frac"], roofline["per_role"]))
+    log("vendor yardstick:", vendor)
 
     def kernel_table():
         table = bench_kernels(cfg, 5)
