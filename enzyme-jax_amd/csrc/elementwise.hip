@@ -537,18 +537,24 @@ __global__ __launch_bounds__(256) void transpose_kernel(const T* __restrict__ in
 // a thread owns a V x V block, reads its V rows as one 16-byte piece each, transposes the block in registers and
 // writes V pieces.  The lanes of a wavefront form an 8 x 8 grid of such blocks, so that every read and every write
 // instruction covers whole 128-byte lines (8 lanes x 16 bytes per row).
-template <typename T>
+template <typename T, bool STREAM>
 __global__ __launch_bounds__(256) void transpose_blocks_kernel(const T* __restrict__ in, T* __restrict__ out, int64_t rows,
                                                                int64_t cols) {
   constexpr int V = 16 / sizeof(T);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int64_t r = ((int64_t)blockIdx.y * 2 + (wave >> 1)) * 8 * V + (lane >> 3) * V;
+  // Blocks that run at the same time differ in both block coordinates (block row (y + x) mod rows of blocks): with
+  // power-of-two row lengths, blocks of one block row write pieces that lie a multiple of 64 KiB apart, and those
+  // of one block column read such pieces: either way a few memory channels would take all the traffic.
+  const unsigned by = (blockIdx.y + blockIdx.x) % gridDim.y;
+  const int64_t r = ((int64_t)by * 2 + (wave >> 1)) * 8 * V + (lane >> 3) * V;
   const int64_t c = ((int64_t)blockIdx.x * 2 + (wave & 1)) * 8 * V + (lane & 7) * V;
   if (r >= rows || c >= cols) return;
   uint32_t x[V][4], y[V][4];
 #pragma unroll
   for (int i = 0; i < V; i++) {
-    const uint4 v = *reinterpret_cast<const uint4*>(in + (r + i) * cols + c);       // cached: weights are re-read soon
+    // weight-sized operands are read again soon (cached loads); activation-sized ones stream through
+    const uint4 v = STREAM ? stream_load(reinterpret_cast<const uint4*>(in + (r + i) * cols + c))
+                           : *reinterpret_cast<const uint4*>(in + (r + i) * cols + c);
     x[i][0] = v.x; x[i][1] = v.y; x[i][2] = v.z; x[i][3] = v.w;
   }
   if constexpr (V == 4) {
@@ -567,8 +573,10 @@ __global__ __launch_bounds__(256) void transpose_blocks_kernel(const T* __restri
       }
   }
 #pragma unroll
-  for (int j = 0; j < V; j++)
-    *reinterpret_cast<uint4*>(out + (c + j) * rows + r) = make_uint4(y[j][0], y[j][1], y[j][2], y[j][3]);
+  for (int j = 0; j < V; j++) {
+    if (STREAM) stream_store(reinterpret_cast<uint4*>(out + (c + j) * rows + r), make_uint4(y[j][0], y[j][1], y[j][2], y[j][3]));
+    else *reinterpret_cast<uint4*>(out + (c + j) * rows + r) = make_uint4(y[j][0], y[j][1], y[j][2], y[j][3]);
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -930,8 +938,12 @@ template <typename T> static int transpose_launch(hipStream_t st, const void* in
   constexpr int V = 16 / sizeof(T);
   if (vec_ok && (rows + 16 * V - 1) / (16 * V) <= 65535) {
     const dim3 gridb(blocks_for(cols, 16 * V), blocks_for(rows, 16 * V));
-    hipLaunchKernelGGL(transpose_blocks_kernel<T>, gridb, dim3(256), 0, st, static_cast<const T*>(in), static_cast<T*>(out),
-                       rows, cols);
+    if (rows * cols * (int64_t)sizeof(T) > (int64_t)(128 << 20))
+      hipLaunchKernelGGL((transpose_blocks_kernel<T, true>), gridb, dim3(256), 0, st, static_cast<const T*>(in), static_cast<T*>(out),
+                         rows, cols);
+    else
+      hipLaunchKernelGGL((transpose_blocks_kernel<T, false>), gridb, dim3(256), 0, st, static_cast<const T*>(in), static_cast<T*>(out),
+                         rows, cols);
     EMI_CHECK_LAUNCH("emi_transpose");
     return EMI_OK;
   }

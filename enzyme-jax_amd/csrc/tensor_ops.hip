@@ -337,7 +337,7 @@ __global__ void __launch_bounds__(kBlock) tiled_permute_kernel(const E* __restri
 // sizeof(E)) without LDS: a thread owns a V x V block over (last, dt), reads V pieces, transposes the block in
 // registers and writes V pieces; the lanes of a wavefront form an 8 x 8 grid of blocks, so every access
 // instruction covers whole 128-byte lines.
-template <typename E>
+template <typename E, bool STREAM>
 __global__ void __launch_bounds__(kBlock) block_permute_kernel(const E* __restrict__ in, E* __restrict__ out, TilePlan p) {
   constexpr int V = 16 / sizeof(E);
   static_assert(V == 4 || V == 8, "2- or 4-byte elements");
@@ -352,7 +352,10 @@ __global__ void __launch_bounds__(kBlock) block_permute_kernel(const E* __restri
     }
   }
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int64_t r = ((int64_t)blockIdx.y * 2 + (wave >> 1)) * 8 * V + (lane >> 3) * V;      // r: last index, c: dt index
+  // blocks that run at the same time differ in both block coordinates, so that with power-of-two row lengths their
+  // reads and their writes do not all fall on the same few memory channels
+  const unsigned by = (blockIdx.y + blockIdx.x) % gridDim.y;
+  const int64_t r = ((int64_t)by * 2 + (wave >> 1)) * 8 * V + (lane >> 3) * V;      // r: last index, c: dt index
   const int64_t c = ((int64_t)blockIdx.x * 2 + (wave & 1)) * 8 * V + (lane & 7) * V;
   if (r >= p.n_last || c >= p.n_dt) return;
   in += ib;
@@ -360,7 +363,8 @@ __global__ void __launch_bounds__(kBlock) block_permute_kernel(const E* __restri
   uint32_t x[V][4], y[V][4];
 #pragma unroll
   for (int i = 0; i < V; i++) {
-    const uint4 v = *reinterpret_cast<const uint4*>(in + (r + i) * p.is_last + c);
+    const uint4 v = STREAM ? stream_load(reinterpret_cast<const uint4*>(in + (r + i) * p.is_last + c))
+                           : *reinterpret_cast<const uint4*>(in + (r + i) * p.is_last + c);
     x[i][0] = v.x; x[i][1] = v.y; x[i][2] = v.z; x[i][3] = v.w;
   }
   if constexpr (V == 4) {
@@ -379,8 +383,10 @@ __global__ void __launch_bounds__(kBlock) block_permute_kernel(const E* __restri
       }
   }
 #pragma unroll
-  for (int j = 0; j < V; j++)
-    *reinterpret_cast<uint4*>(out + (c + j) * p.os_dt + r) = make_uint4(y[j][0], y[j][1], y[j][2], y[j][3]);
+  for (int j = 0; j < V; j++) {
+    if (STREAM) stream_store(reinterpret_cast<uint4*>(out + (c + j) * p.os_dt + r), make_uint4(y[j][0], y[j][1], y[j][2], y[j][3]));
+    else *reinterpret_cast<uint4*>(out + (c + j) * p.os_dt + r) = make_uint4(y[j][0], y[j][1], y[j][2], y[j][3]);
+  }
 }
 
 // Tries the tiled form; returns false when the plan does not have it (then the generic
@@ -417,8 +423,13 @@ bool launch_tiled(hipStream_t st, const void* in, void* out, const CopyPlan& p, 
   if constexpr (sizeof(E) == 2 || sizeof(E) == 4) {
     if (vec_ok && t.n_dt % V == 0 && t.n_last % V == 0 && kBlock == 256) {
       const int64_t bx = (t.n_dt + 16 * V - 1) / (16 * V), by = (t.n_last + 16 * V - 1) / (16 * V);
-      hipLaunchKernelGGL(block_permute_kernel<E>, dim3((unsigned)bx, (unsigned)by, (unsigned)nz), dim3(kBlock), 0, st,
-                         static_cast<const E*>(in), static_cast<E*>(out), t);
+      // operands beyond 128 MiB stream through (non-temporal accesses); smaller ones (weights) are read again soon
+      if (p.total * (int64_t)sizeof(E) > (int64_t)(128 << 20))
+        hipLaunchKernelGGL((block_permute_kernel<E, true>), dim3((unsigned)bx, (unsigned)by, (unsigned)nz), dim3(kBlock), 0, st,
+                           static_cast<const E*>(in), static_cast<E*>(out), t);
+      else
+        hipLaunchKernelGGL((block_permute_kernel<E, false>), dim3((unsigned)bx, (unsigned)by, (unsigned)nz), dim3(kBlock), 0, st,
+                           static_cast<const E*>(in), static_cast<E*>(out), t);
       hipError_t eb = hipGetLastError();
       *status = eb == hipSuccess ? EMI_OK : emi_fail(EMI_INTERNAL, "emi_strided_copy: launch failed: %s", hipGetErrorString(eb));
       return true;
@@ -431,9 +442,29 @@ bool launch_tiled(hipStream_t st, const void* in, void* out, const CopyPlan& p, 
   return true;
 }
 
+// Rows of whole 16-byte chunks, contiguous on both sides (row broadcast: source row stride 0; slices and
+// concatenations along the slow index): one chunk per thread, blockIdx.y = row, no index divisions.  The result
+// is written with streaming stores; a broadcast source is read through the cache (every row reads it again).
+__global__ void __launch_bounds__(kBlock) row_copy_kernel(const uint4* __restrict__ in, uint4* __restrict__ out, int64_t chunks,
+                                                          int64_t is_row, int64_t os_row) {
+  const int64_t c = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (c >= chunks) return;
+  const uint4* src = in + (int64_t)blockIdx.y * is_row + c;
+  const uint4 v = is_row == 0 ? *src : stream_load(src);
+  stream_store(out + (int64_t)blockIdx.y * os_row + c, v);
+}
+
 template <typename E>
 int launch_copy(hipStream_t st, const void* in, void* out, const CopyPlan& p) {
   int status = EMI_OK;
+  if constexpr (sizeof(E) == 16) {
+    if (p.rank == 2 && p.is[1] == 1 && p.os[1] == 1 && p.dims[1] >= 64 && p.dims[0] <= 65535) {
+      hipLaunchKernelGGL(row_copy_kernel, dim3((unsigned)((p.dims[1] + kBlock - 1) / kBlock), (unsigned)p.dims[0]), dim3(kBlock), 0, st,
+                         static_cast<const uint4*>(in), static_cast<uint4*>(out), p.dims[1], p.is[0], p.os[0]);
+      EMI_CHECK_LAUNCH("emi_strided_copy");
+      return EMI_OK;
+    }
+  }
   if constexpr (sizeof(E) <= 8) {
     if (launch_tiled<E>(st, in, out, p, &status)) return status;
   }
