@@ -449,6 +449,25 @@ def bench_models(iters, only=None):
         tl = event_time(loss_step, iters, warmup=2)
         out[name]["loss_ms_per_step"] = round(tl * 1e3, 3)
         out[name]["loss_tokens_per_s"] = round(B * S / tl, 1)
+        # the same training step handed over as StableHLO text (tokens -> gather -> layers sliced out of the stacked
+        # weights -> wcls -> mean softmax cross-entropy in the one-hot spelling), matched onto the same kernels
+        from enzyme_ad.jax import stablehlo
+        from enzyme_ad.jax.llama_text import MODEL_ORDER, llama_model_text
+        mtext, _ = llama_model_text(cfg, B, S, "bf16" if dt == torch.bfloat16 else "f32", "onehot")
+        mexe = stablehlo.compile_text(mtext, fuse=True)
+        margs = [tok] + [w[k] for k in MODEL_ORDER] + [tgt]
+        one_t = torch.ones((), device="cuda", dtype=dt)
+
+        def text_step():
+            y, f_vjp = vjp(lambda *a: mexe.run(list(a))[0], *margs)
+            return f_vjp(one_t)
+
+        tt = event_time(text_step, iters, warmup=2)
+        out[name]["text_fused_loss_ms_per_step"] = round(tt * 1e3, 3)
+        out[name]["text_fused_loss_tokens_per_s"] = round(B * S / tt, 1)
+        out[name]["text_fused_clusters"] = {k: v for k, v in mexe.fused.items() if v}
+        out[name]["text_bytes"] = len(mtext)
+        del mexe, margs
         if B * S <= 1024:
             # small enough to be bound by launches and host code: the same step replayed from a HIP graph
             from enzyme_ad.jax.graph import capture

@@ -224,39 +224,35 @@ def llama_step_text(config, pos, dtype="f32"):
 LAYER_ORDER = ["rms_att_weight", "wq", "wk", "wv", "wo", "rms_ffn_weight", "w1", "w2", "w3"]
 
 
-def llama_layer_text(config, batch, seq, dtype="f32", eps=1e-5, theta=10000.0):
-    """(text, argument names): one decoder layer of test/llama.py:144-233 over a whole batch of
-    sequences, main(x [B, S, dim], <weights in LAYER_ORDER>) -> x, written the way the batched
-    form of that function traces: RMSNorm as sum(x*x) / dim over the last index, projections as
-    dot_general against [out, in] weights, the pair rotation with cos / sin tables [S, hs/2]
-    (constants: positions are static), scores per head from a batched dot_general, a causal mask
-    from two iotas and a compare, softmax over the keys, and the SwiGLU FFN."""
-    dim, hidden, H = config["dim"], config["hidden_dim"], config["n_heads"]
-    hs = dim // H
-    B, S = batch, seq
-    b = Builder(dtype)
-    shapes = {"x": (B, S, dim), "rms_att_weight": (dim,), "wq": (dim, dim), "wk": (dim, dim), "wv": (dim, dim), "wo": (dim, dim),
-              "rms_ffn_weight": (dim,), "w1": (hidden, dim), "w2": (dim, hidden), "w3": (hidden, dim)}
-    order = ["x"] + LAYER_ORDER
-    a = {n: b.arg("%" + n, shapes[n]) for n in order}
-
-    def rmsnorm(x, w):
-        ss = b.reduce(b.binary("multiply", x, x), "add", [2])                          # [B, S]
-        ss = b.binary("divide", ss, b.bcast(b.const(float(dim)), (B, S)))
-        ss = b.binary("add", ss, b.bcast(b.const(eps), (B, S)))
-        ss = b.binary("divide", b.bcast(b.const(1.0), (B, S)), b.unary("sqrt", ss))
-        xn = b.binary("multiply", x, b.bcast(ss, (B, S, dim), (0, 1)))
-        return b.binary("multiply", xn, b.bcast(w, (B, S, dim), (2,)))
-
-    def linear(x, w):
-        return b.dot(x, w, contract=((len(b.types[x]) - 1,), (1,)))
-
+def _rope_tables(b, S, hs, theta, dtype):
     pos = np.arange(S, dtype=np.float64)[:, None]
     freq = 1.0 / np.power(theta, (2.0 * np.arange(hs // 2, dtype=np.float64)) / hs)[None, :]
     cos_c, sin_c = b.blob(np.cos(pos * freq), "f32"), b.blob(np.sin(pos * freq), "f32")
     if dtype != "f32":
         cos_c = b.emit((S, hs // 2), "stablehlo.convert %s : (tensor<%dx%dxf32>) -> %s" % (cos_c, S, hs // 2, b.ty((S, hs // 2))))
         sin_c = b.emit((S, hs // 2), "stablehlo.convert %s : (tensor<%dx%dxf32>) -> %s" % (sin_c, S, hs // 2, b.ty((S, hs // 2))))
+    return cos_c, sin_c
+
+
+def _rmsnorm_rows(b, x, w, eps):
+    B, S, dim = b.types[x]
+    ss = b.reduce(b.binary("multiply", x, x), "add", [2])                          # [B, S]
+    ss = b.binary("divide", ss, b.bcast(b.const(float(dim)), (B, S)))
+    ss = b.binary("add", ss, b.bcast(b.const(eps), (B, S)))
+    ss = b.binary("divide", b.bcast(b.const(1.0), (B, S)), b.unary("sqrt", ss))
+    xn = b.binary("multiply", x, b.bcast(ss, (B, S, dim), (0, 1)))
+    return b.binary("multiply", xn, b.bcast(w, (B, S, dim), (2,)))
+
+
+def _linear_rows(b, x, w):
+    return b.dot(x, w, contract=((len(b.types[x]) - 1,), (1,)))
+
+
+def _layer_rows(b, x, a, H, hidden, tables, eps):
+    """One decoder layer of test/llama.py:144-233 over x [B, S, dim]; a: weight name -> value name."""
+    B, S, dim = b.types[x]
+    hs = dim // H
+    cos_c, sin_c = tables
 
     def rope(x):
         xr = b.reshape(x, (B, S, H, hs // 2, 2))
@@ -269,9 +265,8 @@ def llama_layer_text(config, batch, seq, dtype="f32", eps=1e-5, theta=10000.0):
         both = b.concat([b.reshape(o0, half + (1,)), b.reshape(o1, half + (1,))], 4)
         return b.reshape(both, (B, S, dim))
 
-    x = a["x"]
-    xb = rmsnorm(x, a["rms_att_weight"])
-    q, k, v = rope(linear(xb, a["wq"])), rope(linear(xb, a["wk"])), linear(xb, a["wv"])
+    xb = _rmsnorm_rows(b, x, a["rms_att_weight"], eps)
+    q, k, v = rope(_linear_rows(b, xb, a["wq"])), rope(_linear_rows(b, xb, a["wk"])), _linear_rows(b, xb, a["wv"])
     heads = lambda t: b.transpose(b.reshape(t, (B, S, H, hs)), [0, 2, 1, 3])                 # [B, H, S, hs]
     qh, kh, vh = heads(q), heads(k), heads(v)
     att = b.dot(qh, kh, batch=((0, 1), (0, 1)), contract=((3,), (3,)))                      # [B, H, S, S]
@@ -283,12 +278,109 @@ def llama_layer_text(config, batch, seq, dtype="f32", eps=1e-5, theta=10000.0):
     p = b.binary("divide", e, b.bcast(b.reduce(e, "add", [3]), (B, H, S, S), (0, 1, 2)))
     o = b.dot(p, vh, batch=((0, 1), (0, 1)), contract=((3,), (2,)))                         # [B, H, S, hs]
     o = b.reshape(b.transpose(o, [0, 2, 1, 3]), (B, S, dim))
-    x = b.binary("add", x, linear(o, a["wo"]))
-    xb = rmsnorm(x, a["rms_ffn_weight"])
-    hb, hb2 = linear(xb, a["w1"]), linear(xb, a["w3"])
+    x = b.binary("add", x, _linear_rows(b, o, a["wo"]))
+    xb = _rmsnorm_rows(b, x, a["rms_ffn_weight"], eps)
+    hb, hb2 = _linear_rows(b, xb, a["w1"]), _linear_rows(b, xb, a["w3"])
     one = b.bcast(b.const(1.0), (B, S, hidden))
     sig = b.binary("divide", one, b.binary("add", one, b.unary("exponential", b.unary("negate", hb))))
-    x = b.binary("add", x, linear(b.binary("multiply", b.binary("multiply", hb, sig), hb2), a["w2"]))
+    return b.binary("add", x, _linear_rows(b, b.binary("multiply", b.binary("multiply", hb, sig), hb2), a["w2"]))
+
+
+def llama_layer_text(config, batch, seq, dtype="f32", eps=1e-5, theta=10000.0):
+    """(text, argument names): one decoder layer of test/llama.py:144-233 over a whole batch of
+    sequences, main(x [B, S, dim], <weights in LAYER_ORDER>) -> x, written the way the batched
+    form of that function traces: RMSNorm as sum(x*x) / dim over the last index, projections as
+    dot_general against [out, in] weights, the pair rotation with cos / sin tables [S, hs/2]
+    (constants: positions are static), scores per head from a batched dot_general, a causal mask
+    from two iotas and a compare, softmax over the keys, and the SwiGLU FFN."""
+    dim, hidden, H = config["dim"], config["hidden_dim"], config["n_heads"]
+    B, S = batch, seq
+    b = Builder(dtype)
+    shapes = {"x": (B, S, dim), "rms_att_weight": (dim,), "wq": (dim, dim), "wk": (dim, dim), "wv": (dim, dim), "wo": (dim, dim),
+              "rms_ffn_weight": (dim,), "w1": (hidden, dim), "w2": (dim, hidden), "w3": (hidden, dim)}
+    order = ["x"] + LAYER_ORDER
+    a = {n: b.arg("%" + n, shapes[n]) for n in order}
+    x = _layer_rows(b, a["x"], a, H, hidden, _rope_tables(b, S, dim // H, theta, dtype), eps)
     head = "module @jit_layer {\n  func.func public @main(%s) -> (%s {jax.result_info = \"\"}) {\n" % (
         ", ".join("%s: %s" % (a[n], b.ty(shapes[n])) for n in order), b.ty((B, S, dim)))
     return head + "\n".join(b.lines) + "\n    return %s : %s\n  }\n}\n" % (x, b.ty((B, S, dim))), order
+
+
+MODEL_ORDER = ["token_embedding_table"] + WEIGHT_ORDER + ["wcls"]
+
+
+def llama_model_text(config, batch, seq, dtype="f32", loss=None, eps=1e-5, theta=10000.0):
+    """(text, argument names): the whole model over a batch of token sequences, the pieces test/llama.py comments out
+    (:109-113, :236) switched on: main(tokens [B, S] i32, <weights in MODEL_ORDER, per-layer ones stacked [L, ...]>
+    [, targets [B, S] i32]) -> logits [B, S, vocab], or with `loss` the mean softmax cross-entropy (a scalar) in one
+    of the two spellings JAX users write:
+      loss="onehot":  -mean(sum(one_hot(targets) * log_softmax(logits), -1))
+      loss="gather":  -mean(take_along_axis(log_softmax(logits), targets[..., None], -1))
+    The embedding is the row lookup `table[tokens]` (a gather), every layer slices its weights out of the stacks
+    (`wq[l, :, :]`, :149) and is written as in `llama_layer_text`."""
+    dim, hidden, H, L, V = config["dim"], config["hidden_dim"], config["n_heads"], config["n_layers"], config["vocab_size"]
+    B, S, T = batch, seq, batch * seq
+    if loss not in (None, "onehot", "gather"):
+        raise ValueError("loss must be None, 'onehot' or 'gather'")
+    b = Builder(dtype)
+    shapes = {"token_embedding_table": (V, dim), "rms_att_weight": (L, dim), "wq": (L, dim, dim), "wk": (L, dim, dim), "wv": (L, dim, dim),
+              "wo": (L, dim, dim), "rms_ffn_weight": (L, dim), "w1": (L, hidden, dim), "w2": (L, dim, hidden), "w3": (L, hidden, dim),
+              "rms_final_weight": (dim,), "wcls": (V, dim)}
+    a = {n: b.arg("%" + n, shapes[n]) for n in MODEL_ORDER}
+    i32 = lambda shape: "tensor<%s>" % "x".join([str(s) for s in shape] + ["i32"])
+
+    def raw(shape, text):               # an operator whose result the float-typed helpers do not describe
+        r = b.new(shape)
+        b.lines.append("    %s = %s" % (r, text))
+        return r
+
+    idx = raw((T, 1), "stablehlo.reshape %%tokens : (%s) -> %s" % (i32((B, S)), i32((T, 1))))
+    rows = b.emit((T, dim), '"stablehlo.gather"(%s, %s) <{dimension_numbers = #stablehlo.gather<offset_dims = [1], '
+                            'collapsed_slice_dims = [0], start_index_map = [0], index_vector_dim = 1>, indices_are_sorted = false, '
+                            'slice_sizes = array<i64: 1, %d>}> : (%s, %s) -> %s' % (
+                                a["token_embedding_table"], idx, dim, b.ty((V, dim)), i32((T, 1)), b.ty((T, dim))))
+    x = b.reshape(rows, (B, S, dim))
+    tables = _rope_tables(b, S, dim // H, theta, dtype)
+
+    def layer_slice(w, i):
+        shape = b.types[w]
+        s = b.slice(w, [i] + [0] * (len(shape) - 1), [i + 1] + list(shape[1:]))
+        return b.reshape(s, shape[1:])
+
+    for l in range(L):
+        x = _layer_rows(b, x, {k: layer_slice(a[k], l) for k in LAYER_ORDER}, H, hidden, tables, eps)
+    x = _rmsnorm_rows(b, x, a["rms_final_weight"], eps)
+    logits = _linear_rows(b, x, a["wcls"])                                    # [B, S, V]
+    order = ["tokens"] + MODEL_ORDER
+    sig = ["%%tokens: %s" % i32((B, S))] + ["%s: %s" % (a[n], b.ty(shapes[n])) for n in MODEL_ORDER]
+    if loss is None:
+        out, out_shape = logits, (B, S, V)
+    else:
+        order.append("targets")
+        sig.append("%%targets: %s" % i32((B, S)))
+        full = (B, S, V)
+        mx = b.reduce(logits, "maximum", [2])
+        shifted = b.binary("subtract", logits, b.bcast(b.bcast(mx, (B, S, 1), (0, 1)), full, (0, 1, 2)))
+        se = b.reduce(b.unary("exponential", shifted), "add", [2])
+        lg = b.unary("log", b.bcast(se, (B, S, 1), (0, 1)))
+        logp = b.binary("subtract", shifted, b.bcast(lg, full, (0, 1, 2)))
+        if loss == "onehot":
+            t1 = raw((B, S, 1), "stablehlo.broadcast_in_dim %%targets, dims = [0, 1] : (%s) -> %s" % (i32((B, S)), i32((B, S, 1))))
+            t2 = raw(full, "stablehlo.broadcast_in_dim %s, dims = [0, 1, 2] : (%s) -> %s" % (t1, i32((B, S, 1)), i32(full)))
+            io = raw((1, 1, V), "stablehlo.iota dim = 2 : %s" % i32((1, 1, V)))
+            io2 = raw(full, "stablehlo.broadcast_in_dim %s, dims = [0, 1, 2] : (%s) -> %s" % (io, i32((1, 1, V)), i32(full)))
+            i1 = "tensor<%s>" % "x".join([str(s_) for s_ in full] + ["i1"])
+            eq = raw(full, "stablehlo.compare  EQ, %s, %s,  SIGNED : (%s, %s) -> %s" % (t2, io2, i32(full), i32(full), i1))
+            oh = b.emit(full, "stablehlo.convert %s : (%s) -> %s" % (eq, i1, b.ty(full)))
+            picked = b.reduce(b.binary("multiply", oh, logp), "add", [2])                     # [B, S]
+        else:
+            t1 = raw((B, S, 1), "stablehlo.reshape %%targets : (%s) -> %s" % (i32((B, S)), i32((B, S, 1))))
+            picked = b.emit((B, S), '"stablehlo.gather"(%s, %s) <{dimension_numbers = #stablehlo.gather<collapsed_slice_dims = [2], '
+                                    'operand_batching_dims = [0, 1], start_indices_batching_dims = [0, 1], start_index_map = [2], '
+                                    'index_vector_dim = 2>, indices_are_sorted = false, slice_sizes = array<i64: 1, 1, 1>}> : (%s, %s) -> %s' % (
+                                        logp, t1, b.ty(full), i32((B, S, 1)), b.ty((B, S))))
+        total = b.reduce(picked, "add", [0, 1])
+        out = b.unary("negate", b.binary("divide", total, b.const(float(T))))
+        out_shape = ()
+    head = "module @jit_model {\n  func.func public @main(%s) -> (%s {jax.result_info = \"\"}) {\n" % (", ".join(sig), b.ty(out_shape))
+    return head + "\n".join(b.lines) + "\n    return %s : %s\n  }\n}\n" % (out, b.ty(out_shape)), order

@@ -529,7 +529,8 @@ def _gather_attrs(text):
     if m is None or ss is None:
         raise ParseError("stablehlo.gather without index_vector_dim / slice_sizes")
     return {"offset_dims": ints("offset_dims"), "collapsed_slice_dims": ints("collapsed_slice_dims"),
-            "operand_batching_dims": ints("operand_batching_dims"), "start_index_map": ints("start_index_map"),
+            "operand_batching_dims": ints("operand_batching_dims"),
+            "start_indices_batching_dims": ints("start_indices_batching_dims"), "start_index_map": ints("start_index_map"),
             "index_vector_dim": int(m.group(1)),
             "slice_sizes": [int(v) for v in (ss.group(1) or ss.group(2)).split(",") if v.strip()]}
 
@@ -743,7 +744,7 @@ def _drop_dead(func):
 
 
 ALL_KINDS = ("rmsnorm", "swiglu", "rope", "softmax_dot", "attention_step", "rmsnorm_rows", "rope_rows", "attention", "cross_entropy",
-             "linear")
+             "linear", "linear_group")
 
 
 def fuse_clusters(func, kinds=ALL_KINDS):
@@ -764,7 +765,7 @@ def fuse_clusters(func, kinds=ALL_KINDS):
     A cluster is fused only when none of its interior values is used outside it.  Returns
     the number of clusters fused per kind."""
     counts = {"rmsnorm": 0, "swiglu": 0, "rope": 0, "softmax_dot": 0, "attention_step": 0, "rmsnorm_rows": 0, "rope_rows": 0,
-              "attention": 0, "cross_entropy": 0, "linear": 0}
+              "attention": 0, "cross_entropy": 0, "linear": 0, "linear_group": 0}
     matchers = [m for k, m in (("rmsnorm", _match_rmsnorm), ("swiglu", _match_swiglu), ("rope", _match_rope),
                                ("softmax_dot", _match_softmax_dot), ("attention_step", _match_heads),
                                ("rmsnorm_rows", _match_rmsnorm_rows), ("rope_rows", _match_rope_rows),
@@ -846,8 +847,99 @@ def fuse_clusters(func, kinds=ALL_KINDS):
                     counts["linear"] += 1
                 changed = True
                 break
+    if want_linear and "linear_group" in kinds:
+        counts["linear_group"] = _group_linears(func)
     _drop_dead(func)
     return counts
+
+
+def _group_linears(func):
+    """Sibling projections of one activation against weights of one shape (q, k, v of test/llama.py:149-157; w1, w3 of
+    :224-227) become one `emi.linear_group` (operands x, w_1 .. w_n; results y_1 .. y_n; at most four): one grouped
+    launch forward, one for the weight gradients and one summed launch for dX.  A member's weight must be a function
+    argument or a slice / reshape chain of one, so that the operators that produce it can move in front of the
+    group.  Returns the number of groups formed."""
+    args = set(a for a, _ in func.args)
+    types = {a: t for a, t in func.args}
+    defs = {}
+    for op in func.ops:
+        for r, t in zip(op.results, op.types):
+            defs[r] = op
+            types[r] = t
+    pos = {id(op): i for i, op in enumerate(func.ops)}
+
+    def chain(name):
+        out = []
+        while name not in args:
+            op = defs.get(name)
+            if op is None or op.name not in ("slice", "reshape"):
+                return None
+            out.append(op)
+            name = op.operands[0]
+        return out[::-1]
+
+    groups = {}
+    for op in func.ops:
+        if op.name == "emi.linear" and len(op.operands) == 2 and chain(op.operands[1]) is not None:
+            xt = types[op.operands[0]]
+            if len(xt.shape) < 2 or int(np.prod(xt.shape[:-1])) < 16:
+                continue                 # the single-token step: each mat-vec streams its weight through its own kernel
+            wt = types[op.operands[1]]
+            groups.setdefault((op.operands[0], tuple(wt.shape), wt.dtype), []).append(op)
+    formed = 0
+    for members in groups.values():
+        for k in range(0, len(members) - 1, 4):
+            part = members[k:k + 4]
+            if len(part) < 2:
+                continue
+            first = part[0]
+            hoist, seen = [], set()
+            for m in part[1:]:
+                for c in chain(m.operands[1]):
+                    if pos[id(c)] > pos[id(first)] and id(c) not in seen:
+                        seen.add(id(c))
+                        hoist.append(c)
+            new = Op("emi.linear_group", [r for m in part for r in m.results], [first.operands[0]] + [m.operands[1] for m in part], {},
+                     [t for m in part for t in m.types])
+            drop = set(id(m) for m in part[1:]) | seen
+            out = []
+            for o in func.ops:
+                if o is first:
+                    out.extend(hoist)
+                    out.append(new)
+                elif id(o) not in drop:
+                    out.append(o)
+            func.ops = out
+            pos = {id(op): i for i, op in enumerate(func.ops)}
+            formed += 1
+    return formed
+
+
+def _fold_selects(func):
+    """The operator list `Executable.run` walks: `reshape(slice(w, [i:i+1, 0:, ...]))` of a stacked function argument
+    (`wq[i, :, :]`, test/llama.py:149) becomes `emi.select` {index}, which the tape differentiates in place (the
+    slice's gradient is written straight into slice i of one buffer shaped like the stack).  The printed and the
+    symbolic forms keep slice + reshape."""
+    arg_t = {a: t for a, t in func.args}
+    use = _users(func)
+    rets = set(o for op in func.ops if op.name == "return" for o in op.operands)
+    out, dropped = [], {}
+    for op in func.ops:
+        if op.name == "slice" and op.operands[0] in arg_t and op.results[0] not in rets:
+            t = arg_t[op.operands[0]]
+            a = op.attrs
+            users = use.get(op.results[0], [])
+            if (len(t.shape) >= 2 and len(users) == 1 and users[0].name == "reshape" and all(st == 1 for st in a["stride"])
+                    and a["limit"][0] == a["start"][0] + 1 and list(a["start"][1:]) == [0] * (len(t.shape) - 1)
+                    and list(a["limit"][1:]) == list(t.shape[1:]) and tuple(users[0].types[0].shape) == tuple(t.shape[1:])):
+                dropped[op.results[0]] = (op.operands[0], a["start"][0])
+                continue
+        if op.name == "reshape" and op.operands[0] in dropped:
+            w, i = dropped[op.operands[0]]
+            out.append(Op("emi.select", op.results, [w], {"index": i}, op.types))
+            continue
+        out.append(op)
+    return out
 
 
 def _match_rmsnorm(op, d, tb):
@@ -1063,13 +1155,68 @@ def _is_class_index(name, d):
         name = op.operands[0]
 
 
+def _log_softmax(logp_name, d):
+    """(logits, interior operators) when `logp_name` is jax.nn.log_softmax over the last axis:
+    shifted - spread(log(reduce-add(exp(shifted)))) with shifted = logits - spread(reduce-max(logits))."""
+    logp = d(logp_name)
+    if logp is None or logp.name != "subtract":
+        return None
+    shifted = d(logp.operands[0])
+    norm = _per_row_source(logp.operands[1], d, through=("log",))
+    if shifted is None or shifted.name != "subtract" or norm is None or norm[2] != ["log"]:
+        return None
+    sm = d(norm[0])
+    if sm is None or sm.name != "reduce" or sm.attrs["body"] != "add" or _splat(d(sm.operands[1])) != 0.0:
+        return None
+    ex = d(sm.operands[0])
+    rank = len(shifted.types[0].shape)
+    if ex is None or ex.name != "exponential" or ex.operands[0] != logp.operands[0] or list(sm.attrs["dims"]) != [rank - 1]:
+        return None
+    logits = shifted.operands[0]
+    top = _per_row_source(shifted.operands[1], d)
+    if top is None:
+        return None
+    mx = d(top[0])
+    if mx is None or mx.name != "reduce" or mx.attrs["body"] != "maximum" or mx.operands[0] != logits or \
+            list(mx.attrs["dims"]) != [rank - 1] or _splat(d(mx.operands[1])) != -math.inf:
+        return None
+    if d.types[logits].dtype not in ("f32", "bf16"):
+        return None
+    return logits, [logp, shifted, sm, ex, mx] + norm[1] + top[1]
+
+
 def _match_cross_entropy(op, d, tb):
-    # root: reduce-add over the last axis of onehot * logp (either order) or select(eq, logp, 0), with
-    #   eq     = compare EQ of the targets spread along the last axis and the class index along it
-    #   onehot = convert(eq)
-    #   logp   = shifted - spread(log(reduce-add(exp(shifted)))),  shifted = logits - spread(reduce-max(logits))
-    # (jax.nn.log_softmax and jax.nn.one_hot).  The root equals minus the per-row cross-entropy; a target outside
-    # [0, V) matches no class and gives 0, as the kernel does.
+    # Two spellings of minus the per-row cross-entropy of jax.nn.log_softmax(logits) against run-time integer targets:
+    # (1) root: reduce-add over the last axis of onehot * logp (either order) or select(eq, logp, 0), with
+    #       eq     = compare EQ of the targets spread along the last axis and the class index along it
+    #       onehot = convert(eq)                                     (jax.nn.one_hot)
+    # (2) root: gather(logp, targets[..., None]) picking one class per row (jnp.take_along_axis): every leading index a
+    #     batching index of operand and indices, the last one collapsed, slices of one element.
+    # A target outside [0, V) gives 0, as the kernel does.
+    if op.name == "gather":
+        a = op.attrs
+        logp_name, idx_name = op.operands
+        lt, it = d.types.get(logp_name), d.types.get(idx_name)
+        if lt is None or it is None or len(lt.shape) < 2 or it.dtype != "i32":
+            return None
+        R = len(lt.shape) - 1
+        rows = tuple(lt.shape[:-1])
+        lead = list(range(R))
+        if not (tuple(it.shape) == rows + (1,) and a["index_vector_dim"] == R and a["collapsed_slice_dims"] == [R]
+                and a["operand_batching_dims"] == lead and a.get("start_indices_batching_dims", []) == lead
+                and a["start_index_map"] == [R] and a["offset_dims"] == [] and a["slice_sizes"] == [1] * (R + 1)
+                and tuple(op.types[0].shape) == rows):
+            return None
+        ls = _log_softmax(logp_name, d)
+        if ls is None:
+            return None
+        src = d(idx_name)                       # targets[..., None]: a reshape or broadcast of the [rows] targets
+        passed = []
+        targets = idx_name
+        if src is not None and src.name in ("reshape", "broadcast_in_dim") and tuple(d.types[src.operands[0]].shape) == rows:
+            targets, passed = src.operands[0], [src]
+        return ("cross_entropy", Op("emi.cross_entropy", op.results, [ls[0], targets], {"negated": True}, op.types),
+                [op] + passed + ls[1])
     if op.name != "reduce" or op.attrs["body"] != "add" or _splat(d(op.operands[1])) != 0.0:
         return None
     prod = d(op.operands[0])
@@ -1104,32 +1251,10 @@ def _match_cross_entropy(op, d, tb):
             break
     if targets is None:
         return None
-    logp = d(logp_name)
-    if logp is None or logp.name != "subtract":
+    ls = _log_softmax(logp_name, d)
+    if ls is None:
         return None
-    shifted = d(logp.operands[0])
-    norm = _per_row_source(logp.operands[1], d, through=("log",))
-    if shifted is None or shifted.name != "subtract" or norm is None or norm[2] != ["log"]:
-        return None
-    sm = d(norm[0])
-    if sm is None or sm.name != "reduce" or sm.attrs["body"] != "add" or _splat(d(sm.operands[1])) != 0.0:
-        return None
-    ex = d(sm.operands[0])
-    rank = len(shifted.types[0].shape)
-    if ex is None or ex.name != "exponential" or ex.operands[0] != logp.operands[0] or list(sm.attrs["dims"]) != [rank - 1]:
-        return None
-    logits = shifted.operands[0]
-    top = _per_row_source(shifted.operands[1], d)
-    if top is None:
-        return None
-    mx = d(top[0])
-    if mx is None or mx.name != "reduce" or mx.attrs["body"] != "maximum" or mx.operands[0] != logits or \
-            list(mx.attrs["dims"]) != [rank - 1] or _splat(d(mx.operands[1])) != -math.inf:
-        return None
-    if d.types[logits].dtype not in ("f32", "bf16"):
-        return None
-    interior += [logp, shifted, sm, ex, mx] + norm[1] + top[1]
-    return ("cross_entropy", Op("emi.cross_entropy", op.results, [logits, targets], {"negated": True}, op.types), interior)
+    return ("cross_entropy", Op("emi.cross_entropy", op.results, [ls[0], targets], {"negated": True}, op.types), interior + ls[1])
 
 
 def _bcast(name, d, dims=None):
@@ -1454,6 +1579,8 @@ class Executable:
                     if v:
                         self.fused[k] = self.fused.get(k, 0) + v
         self._consts = {}
+        for f in self.funcs.values():
+            f.run_ops = _fold_selects(f) if fuse else f.ops
 
     def signature(self, fn="main"):
         f = self._func(fn)
@@ -1492,7 +1619,7 @@ class Executable:
             env[name] = a
         if device is None:
             device = torch.device("cuda", torch.cuda.current_device())
-        for op in f.ops:
+        for op in getattr(f, "run_ops", f.ops):
             if op.name == "return":
                 return [env[o] for o in op.operands]
             outs = self._apply(f, op, [env[o] for o in op.operands], device)
@@ -1563,6 +1690,10 @@ class Executable:
             x, w = _packed(xs[0]), _packed(xs[1])
             r = _packed(xs[2]) if len(xs) > 2 else None
             return [ops.matmul_nt(x, w, residual=r)]
+        if n == "emi.linear_group":
+            return list(ops.matmul_nt_group(_packed(xs[0]), [_packed(w) for w in xs[1:]]))
+        if n == "emi.select":
+            return [ops.select(xs[0], op.attrs["index"])]
         if n == "emi.rmsnorm_rows":
             x, w = _packed(xs[0]), _packed(xs[1])
             return [ops.rmsnorm(x, w, op.attrs["eps"])]
@@ -1625,6 +1756,15 @@ def _custom_call_impl(self, op, xs):
         if not ta and tb_:
             return [ops.matmul_nt(a, b_, residual=r)]                   # the projection form: differentiable on the tape
         return [ops.gemm(a, b_, ta, tb_, r)]                            # the forms derivative programs use
+    if target == "emi_gemm_grouped":
+        n_, sum_ = int(cfg["count"]), bool(cfg.get("sum", False))
+        ta, tb_ = bool(cfg.get("trans_a", False)), bool(cfg.get("trans_b", False))
+        As, Bs = [_packed(t) for t in xs[:n_]], [_packed(t) for t in xs[n_:2 * n_]]
+        rs = [_packed(t) for t in xs[2 * n_:]] or None
+        if not ta and tb_ and not sum_ and rs is None and all(a is As[0] for a in As):
+            return list(ops.matmul_nt_group(As[0], Bs))                  # sibling projections: differentiable on the tape
+        out = ops.gemm_grouped(As, Bs, ta, tb_, rs, sum_into_one=sum_)   # the forms derivative programs use
+        return ([out] if sum_ else list(out)) + [None] * (len(op.results) - (1 if sum_ else n_))
     if target == "emi_add":
         return [ops.add(_packed(xs[0]), _packed(xs[1]))]
     if target == "emi_rope":

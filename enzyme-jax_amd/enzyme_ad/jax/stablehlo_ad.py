@@ -108,6 +108,15 @@ def lower_fused(func):
             operands = [b.reshape(x, (rows, K)), w] + [b.reshape(r_, (rows, Nn)) for r_ in op.operands[2:]]
             c2, = b.custom_call("emi_gemm", operands, {"trans_a": False, "trans_b": True}, [TensorType((rows, Nn), ty.dtype)])
             b.ops.append(Op("reshape", op.results, [c2], {}, op.types))
+        elif n == "emi.linear_group":
+            x, ws = op.operands[0], list(op.operands[1:])
+            K, Nn = T[x].shape[-1], T[ws[0]].shape[0]
+            rows = int(np.prod(T[x].shape[:-1])) if len(T[x].shape) > 1 else 1
+            x2 = b.reshape(x, (rows, K))
+            outs = b.custom_call("emi_gemm_grouped", [x2] * len(ws) + ws, {"count": len(ws), "sum": False, "trans_a": False, "trans_b": True},
+                                 [TensorType((rows, Nn), ty.dtype)] * len(ws))
+            for r_, c2, t_ in zip(op.results, outs, op.types):
+                b.ops.append(Op("reshape", [r_], [c2], {}, [t_]))
         elif n == "emi.rmsnorm_rows":
             b.ops.append(Op("custom_call", op.results, list(op.operands), {"target": "emi_rmsnorm_fwd", "config": {"eps": op.attrs["eps"]}},
                             op.types))
@@ -543,6 +552,21 @@ def forward_function(func, name=None, arg_active=None):
                     acc_t, = b.custom_call("emi_gemm", [xs[0], ts[1]] + ([acc_t] if acc_t is not None else []), flags, [T[r]])
                 if acc_t is not None:
                     tan[r] = acc_t
+            elif target == "emi_gemm_grouped":
+                # sibling projections y_i = x . w_i^T: ty_i = tx . w_i^T + x . tw_i^T, product after product
+                n_ = int(cfg["count"])
+                if cfg.get("sum", False) or cfg.get("trans_a", False) or not cfg.get("trans_b", False) or len(xs) != 2 * n_:
+                    raise NotImplementedError("symbolic forward mode of emi_gemm_grouped other than sibling projections")
+                flags = {"trans_a": False, "trans_b": True}
+                for i in range(n_):
+                    acc_t = None
+                    if ts[i] is not None:
+                        acc_t, = b.custom_call("emi_gemm", [ts[i], xs[n_ + i]], flags, [T[op.results[i]]])
+                    if ts[n_ + i] is not None:
+                        acc_t, = b.custom_call("emi_gemm", [xs[i], ts[n_ + i]] + ([acc_t] if acc_t is not None else []), flags,
+                                               [T[op.results[i]]])
+                    if acc_t is not None:
+                        tan[op.results[i]] = acc_t
             elif target == "emi_attn_fwd":
                 o, lse = op.results[:2]
                 tan[o], = b.custom_call("emi_attn_jvp", [xs[0], xs[1], xs[2], lse, tz(xs[0]), tz(xs[1]), tz(xs[2])],
@@ -636,6 +660,27 @@ def _reverse_custom_call(b, op, cs, accum):
         accum(Bm, gemm(A, c, not ta, False, T[Bm]) if not tb_ else gemm(c, A, True, ta, T[Bm]))
         if len(xs) > 2:
             accum(xs[2], c)
+    elif target == "emi_gemm_grouped":
+        # sibling projections y_i = x . w_i^T (DotGeneral rule per product): dX = sum_i dY_i . w_i as one summed
+        # launch, dW_i = dY_i^T . x as one grouped launch; a result without a cotangent contributes nothing
+        n_ = int(cfg["count"])
+        if cfg.get("sum", False) or cfg.get("trans_a", False) or not cfg.get("trans_b", False) or len(xs) != 2 * n_ or \
+                any(x != xs[0] for x in xs[:n_]):
+            raise NotImplementedError("symbolic reverse mode of emi_gemm_grouped other than sibling projections of one operand")
+        live = [i for i in range(n_) if cs[i] is not None]
+        x = xs[0]
+        if len(live) >= 2:
+            dx, = b.custom_call("emi_gemm_grouped", [cs[i] for i in live] + [xs[n_ + i] for i in live],
+                                {"count": len(live), "sum": True, "trans_a": False, "trans_b": False}, [T[x]])
+            accum(x, dx)
+            dws = b.custom_call("emi_gemm_grouped", [cs[i] for i in live] + [x] * len(live),
+                                {"count": len(live), "sum": False, "trans_a": True, "trans_b": False}, [T[xs[n_ + i]] for i in live])
+            for i, dw in zip(live, dws):
+                accum(xs[n_ + i], dw)
+        else:
+            for i in live:
+                accum(x, b.custom_call("emi_gemm", [cs[i], xs[n_ + i]], {"trans_a": False, "trans_b": False}, [T[x]])[0])
+                accum(xs[n_ + i], b.custom_call("emi_gemm", [cs[i], x], {"trans_a": True, "trans_b": False}, [T[xs[n_ + i]]])[0])
     elif target == "emi_attn_fwd":
         if any(x is not None for x in cs[1:]):
             raise NotImplementedError("cotangents of the log-sum-exp or workspace results of emi_attn_fwd")

@@ -43,9 +43,10 @@ def test_layer_text_fp32(fuse):
     cfg = {"dim": 128, "hidden_dim": 352, "n_heads": 2}
     exe, errs = _case(cfg, 2, 40, "f32", 5, fuse)
     if fuse:
-        assert exe.fused == {"rmsnorm_rows": 2, "rope_rows": 2, "attention": 1, "swiglu": 1, "linear": 7}
+        assert exe.fused == {"rmsnorm_rows": 2, "rope_rows": 2, "attention": 1, "swiglu": 1, "linear": 7, "linear_group": 2}
         names = sorted(o.name for o in exe.funcs["main"].ops)                 # the hand-wired llama.layer, operator for operator
-        assert names == sorted(["emi.linear"] * 7 + ["emi.rmsnorm_rows"] * 2 + ["emi.rope_rows"] * 2 + ["emi.attention", "emi.swiglu", "return"])
+        assert names == sorted(["emi.linear"] * 2 + ["emi.linear_group"] * 2 + ["emi.rmsnorm_rows"] * 2 + ["emi.rope_rows"] * 2 +
+                               ["emi.attention", "emi.swiglu", "return"])      # q, k, v and w1, w3 as grouped launches
     print("layer text fuse=%s max rel errors" % fuse, {k: "%.2e" % v for k, v in errs.items()}, flush=True)
 
 
@@ -93,7 +94,8 @@ def test_layer_text_lowered_and_symbolic_programs():
         y, f_vjp = vjp(fn, *args)
         grads = f_vjp(dy)
         low = optimize_module(text)
-        assert low.count("stablehlo.custom_call") == 13 and "stablehlo.exponential" not in low and "stablehlo.dot_general" not in low
+        assert low.count("stablehlo.custom_call") == 10 and low.count("@emi_gemm_grouped") == 2
+        assert "stablehlo.exponential" not in low and "stablehlo.dot_general" not in low
         y_low = hlo_call(*args, source=low)[0]
         assert torch.equal(y_low, y)
         fwd_pipe = P.forward_mode_pipeline(P.JaXPipeline(), [True] * len(args), 1)
