@@ -577,6 +577,176 @@ def cpu_baseline(cfg, repeats=5, budget_s=25.0):
                                           "batch 1 x seq 256 tokens -> logits, cotangent on the logits, fp32"))
 
 
+def gemm_replay(cfg, reps):
+    """Child mode of `measure_gemm_traffic`: the known-size calibration kernel, then the step's 21 GEMM launches."""
+    import torch
+    from enzyme_ad.jax import ops
+    ca = torch.ones(1 << 28, dtype=torch.bfloat16, device="cuda")
+    cb = torch.ones(1 << 28, dtype=torch.bfloat16, device="cuda")
+    ops.add(ca, cb)                       # emi::add_kernel: reads 2 x 512 MiB, writes 512 MiB
+    torch.cuda.synchronize()
+    del ca, cb
+    D, H, T = cfg["dim"], cfg["hidden_dim"], cfg["batch"] * cfg["seq"]
+    big = max(D, H)
+    flat_a = torch.randn((T * big,), device="cuda").to(torch.bfloat16)
+    flat_b = (torch.randn((T * big,), device="cuda") * 0.02).to(torch.bfloat16)
+    for _ in range(reps):
+        for (role, M, N, K) in gemm_launches(cfg):
+            if role == "dW":
+                ops.gemm(flat_a[:M * K].view(K, M), flat_b[:N * K].view(K, N), True, False)
+            else:
+                ops.gemm(flat_a[:M * K].view(M, K), flat_b[:N * K].view(N, K), False, True)
+    torch.cuda.synchronize()
+
+
+def measure_gemm_traffic(cfg):
+    """HBM-side bytes per GEMM launch, measured now: two child runs of this file under `rocprofv3 --pmc` (FETCH_SIZE,
+    then WRITE_SIZE; one counter per run), each replaying the step's 21 GEMM launches after a copy-like kernel of known
+    size (emi::add_kernel over 2^28 bf16: reads 1 GiB, writes 512 MiB) whose reading scales the counter.  Returns
+    (bytes per launch, note); (None, reason) when the profiler is not available or a run fails."""
+    import csv
+    import glob
+    import shutil
+    import subprocess
+    import tempfile
+    if shutil.which("rocprofv3") is None:
+        return None, "rocprofv3 not found"
+    known = {"FETCH_SIZE": 2.0 * (1 << 29) / 1024.0, "WRITE_SIZE": 1.0 * (1 << 29) / 1024.0}       # KiB
+    per_launch, scales = 0.0, {}
+    env = dict(os.environ, TMPDIR="/tmp")
+    for ctr in ("FETCH_SIZE", "WRITE_SIZE"):
+        out = tempfile.mkdtemp(prefix="emi_pmc_", dir="/tmp")
+        try:
+            cmd = ["timeout", "-s", "KILL", "120", "rocprofv3", "--pmc", ctr, "--output-format", "csv", "-d", out, "-o", "t", "--",
+                   "python3", os.path.abspath(__file__), "--gemm-replay", "1", "--seq", str(cfg["seq"]), "--batch", str(cfg["batch"])]
+            r = subprocess.run(cmd, cwd="/tmp", env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+            files = glob.glob(os.path.join(out, "**", "*counter_collection.csv"), recursive=True)
+            if r.returncode != 0 or not files:
+                return None, "rocprofv3 --pmc %s failed (rc %d)" % (ctr, r.returncode)
+            cal, gemm = [], []
+            for row in csv.DictReader(open(files[0])):
+                if row.get("Counter_Name") != ctr:
+                    continue
+                name, v = row["Kernel_Name"], float(row["Counter_Value"])
+                if "add_kernel" in name:
+                    cal.append(v)
+                elif "gemm_bf16_pingpong_kernel" in name:
+                    gemm.append(v)
+            if not cal or not gemm or sum(cal) <= 0:
+                return None, "no %s rows for the calibration or GEMM kernels" % ctr
+            scales[ctr] = known[ctr] / (sum(cal) / len(cal))
+            per_launch += scales[ctr] * (sum(gemm) / len(gemm)) * 1024.0
+        finally:
+            shutil.rmtree(out, ignore_errors=True)
+    return per_launch, ("measured in this run: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (one counter per child run of "
+                        "`bench.py --gemm-replay 1`), scaled by the same counter's reading for emi::add_kernel over 2^28 bf16 "
+                        "(factors %.3f / %.3f)" % (scales["FETCH_SIZE"], scales["WRITE_SIZE"]))
+
+
+def power_probe(cfg, seconds=4.0):
+    """Shader clock and socket power (amd-smi, sampled from a side thread) while one kernel family runs back to back,
+    with the rate it achieves: the step's 21 GEMM launches on N(0,1) x N(0,0.02) operands, the same on all-zero
+    operands (same binary, no switching in the data paths), causal attention forward and backward at the step's shape,
+    and the whole step.  Prints a text table (the content of profiles/power_clock_summary.txt)."""
+    import statistics
+    import subprocess
+    import threading
+    import torch
+    from enzyme_ad.jax import ops, enzyme_jax_ir, JaXPipeline, vjp, llama
+
+    def sample():
+        try:
+            r = subprocess.run(["amd-smi", "metric", "-p", "-c", "--json"], stdout=subprocess.PIPE, stderr=subprocess.DEVNULL, text=True, timeout=5)
+            g = json.loads(r.stdout)
+            g = g["gpu_data"][0] if isinstance(g, dict) else g[0]
+            clk = [v["clk"]["value"] for k, v in g["clock"].items() if k.startswith("gfx_") and isinstance(v["clk"], dict)]
+            return float(g["power"]["socket_power"]["value"]), float(sum(clk)) / len(clk)
+        except Exception:                                        # noqa: BLE001
+            return None
+
+    def run(name, fn, flops_per_call):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        samples, stop = [], threading.Event()
+
+        def poll():
+            time.sleep(0.8)                                      # past the clock ramp from idle
+            while not stop.is_set():
+                s_ = sample()
+                if s_ is not None:
+                    samples.append(s_)
+                time.sleep(0.1)
+
+        th = threading.Thread(target=poll)
+        th.start()
+        calls, t0 = 0, time.perf_counter()
+        while time.perf_counter() - t0 < seconds:
+            for _ in range(4):
+                fn()
+                calls += 1
+            torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        stop.set()
+        th.join()
+        pw = [s_[0] for s_ in samples]
+        ck = [s_[1] for s_ in samples]
+        row = dict(name=name, tflops=flops_per_call * calls / dt / 1e12, samples=len(samples),
+                   power_w=(statistics.median(pw), min(pw), max(pw)) if pw else None,
+                   clock_mhz=(statistics.median(ck), min(ck), max(ck)) if ck else None)
+        print("%-58s %8.1f TFLOP/s  %s  %s  (%d samples)" % (
+            name, row["tflops"],
+            "power %4.0f W (%4.0f-%4.0f)" % row["power_w"] if pw else "power n/a",
+            "shader clock %4.0f MHz (%4.0f-%4.0f)" % row["clock_mhz"] if ck else "clock n/a", len(samples)), flush=True)
+        return row
+
+    D, H, T = cfg["dim"], cfg["hidden_dim"], cfg["batch"] * cfg["seq"]
+    big = max(D, H)
+    launches = gemm_launches(cfg)
+    gfl = sum(2.0 * M * N * K for (_, M, N, K) in launches)
+    rows = []
+    for tag, zero in (("N(0,1) x N(0,0.02) operands", False), ("all-zero operands (same binary)", True)):
+        fa = torch.randn((T * big,), device="cuda").to(torch.bfloat16)
+        fb = (torch.randn((T * big,), device="cuda") * 0.02).to(torch.bfloat16)
+        if zero:
+            fa.zero_()
+            fb.zero_()
+
+        def gemms():
+            for (role, M, N, K) in launches:
+                if role == "dW":
+                    ops.gemm(fa[:M * K].view(K, M), fb[:N * K].view(K, N), True, False)
+                else:
+                    ops.gemm(fa[:M * K].view(M, K), fb[:N * K].view(N, K), False, True)
+
+        rows.append(run("GEMM, the step's 21 launches, " + tag, gemms, gfl))
+        del fa, fb
+    B, S, nh = cfg["batch"], cfg["seq"], cfg["n_heads"]
+    fl = layer_flops(cfg)
+    for tag, zero in (("N(0,1) operands", False), ("all-zero operands", True)):
+        q, k, v, do = (torch.randn((B, S, D), device="cuda").to(torch.bfloat16) for _ in range(4))
+        if zero:
+            for t_ in (q, k, v, do):
+                t_.zero_()
+        rows.append(run("attention forward [%d, %d, %d x %d], " % (B, S, nh, D // nh) + tag, lambda: ops.attention(q, k, v, nh), fl["attn_fwd"]))
+        with ops.Tape() as tape:
+            o = ops.attention(q, k, v, nh)
+        rows.append(run("attention adjoint (dQ, dK, dV), " + tag, lambda: tape.backward([o], [do], [q, k, v]), fl["attn_bwd"]))
+        del q, k, v, do, o, tape
+    x, lw, dy = make_layer_inputs(cfg)
+
+    @enzyme_jax_ir(pipeline_options=JaXPipeline(), inner_jit=False)
+    def layer_fn(x, lw):
+        return llama.layer(x, lw, nh)
+
+    def step():
+        out, f_vjp = vjp(layer_fn, x, lw)
+        return f_vjp(dy)
+
+    rows.append(run("whole step (forward + VJP of the layer)", step, fl["total"]))
+    return rows
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -591,6 +761,13 @@ def main():
     ap.add_argument("--only-model", choices=["c1", "c4"], default=None,
                     help="run only the fwd + VJP steps of one whole-model configuration (c1 = stories15M fp32, c4 = "
                          "stories110M bf16) and print its timing: the command kernel traces of those models are taken from")
+    ap.add_argument("--gemm-replay", type=int, default=0, metavar="REPS",
+                    help="child mode of the traffic measurement: the calibration kernel and REPS replays of the step's 21 "
+                         "GEMM launches, nothing else")
+    ap.add_argument("--power-probe", action="store_true",
+                    help="sample shader clock and socket power (amd-smi) while GEMM, attention and the whole step run back "
+                         "to back, on random and on all-zero operands; prints a table")
+    ap.add_argument("--no-traffic", action="store_true", help="skip the rocprofv3 child runs that measure roofline.traffic")
     ap.add_argument("--seq", type=int, default=C5["seq"])
     ap.add_argument("--batch", type=int, default=C5["batch"])
     args = ap.parse_args()
@@ -601,6 +778,12 @@ def main():
         sys.exit("bench.py: no GPU visible; the HIP path has no CPU fallback")
     if args.only_model:
         print(json.dumps({"whole_models": bench_models(max(args.steps, 5), only=args.only_model)}))
+        return
+    if args.gemm_replay:
+        gemm_replay(dict(C5, seq=args.seq, batch=args.batch), args.gemm_replay)
+        return
+    if args.power_probe:
+        power_probe(dict(C5, seq=args.seq, batch=args.batch))
         return
     from enzyme_ad.jax import enzyme_jax_ir, JaXPipeline, vjp, llama
 
@@ -664,12 +847,24 @@ def main():
     roofline = dict(bound="mfma", kernel="gemm_bf16_pingpong_kernel (256x256x64 tiles; %d launches per step: Y, dX in the NT form, dW in the TN form, 7 weights)" % n_gemm,
                     achieved=gemm_fl / t_gemm / 1e12, peak=PEAK_BF16_TFLOPS, unit="TFLOP/s",
                     frac=gemm_fl / t_gemm / 1e12 / PEAK_BF16_TFLOPS,
-                    traffic=GEMM_TRAFFIC_BYTES_PER_LAUNCH if (args.seq, args.batch) == (C5["seq"], C5["batch"]) else None,
+                    traffic=None, traffic_source=None,
                     avg_launch_us=t_gemm / n_gemm * 1e6, flops_per_launch=gemm_fl / n_gemm,
                     per_role={k: dict(tflops=round(v["tflops"], 1), avg_launch_us=round(v["seconds"] / v["launches"] * 1e6, 1))
                                 for k, v in per_layout.items()},
                     vendor=vendor)
     log("GEMM: %.1f TFLOP/s (%.1f%% of bf16 MFMA peak); per role %s" % (roofline["achieved"], 100 * roofline["frac"], roofline["per_role"]))
+    if not args.no_traffic:
+        # the operand buffers of this process stay allocated meanwhile (a few GiB of 288); the child runs alone on the GPU
+        torch.cuda.synchronize()
+        try:
+            traffic, note = measure_gemm_traffic(cfg)
+        except Exception as e:                                   # noqa: BLE001
+            traffic, note = None, "%s: %s" % (type(e).__name__, str(e)[:200])
+        if traffic is None and (args.seq, args.batch) == (C5["seq"], C5["batch"]):
+            traffic, note = GEMM_TRAFFIC_BYTES_PER_LAUNCH, ("not measured in this run (%s); figure of "
+                                                            "profiles/gemm_bf16_llama7b_layer_hbm_traffic.txt" % note)
+        roofline["traffic"], roofline["traffic_source"] = traffic, note
+        log("GEMM traffic per launch: %s (%s)" % (traffic, note))
     log("vendor yardstick:", vendor)
 
     def kernel_table():
