@@ -384,7 +384,7 @@ __global__ __launch_bounds__(256) void rope_pair_kernel(const T* x, const float2
 // SwiGLU (test/llama.py:21-28,229-231) and elementwise add
 // ---------------------------------------------------------------------------
 
-__device__ __forceinline__ float sigmoidf(float a) { return 1.0f / (1.0f + expf(-a)); }
+__device__ __forceinline__ float sigmoidf(float a) { return emi_sigmoid(a); }
 
 template <typename T>
 __global__ __launch_bounds__(256) void swiglu_fwd_kernel(const T* __restrict__ a, const T* __restrict__ b,

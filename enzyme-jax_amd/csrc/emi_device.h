@@ -58,6 +58,22 @@ __device__ __forceinline__ void stream_store(uint4* p, uint4 a) {
   __builtin_nontemporal_store(v, reinterpret_cast<emi_u32x4_t*>(p));
 }
 
+// SwiGLU of test/llama.py:21-28,229-231 and its adjoint, shared by the elementwise kernels and the GEMM epilogues
+// that apply them to a tile: g = a sigmoid(a) b;  da = dg b s (1 + a (1 - s)),  db = dg a s  with s = sigmoid(a).
+// The sigmoid costs one hardware exponential and one hardware reciprocal (each good to about one unit in the last
+// place; 2^x overflows to inf and underflows to 0 exactly where the sigmoid saturates): an epilogue that applies it
+// to a whole tile holds up its CU's matrix cores for as long as its arithmetic lasts, and with the library's expf and
+// an IEEE division that was three times longer.
+__device__ __forceinline__ float emi_sigmoid(float a) {
+  return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(a * -1.44269504088896340736f));
+}
+__device__ __forceinline__ float emi_swiglu(float a, float b) { return a * emi_sigmoid(a) * b; }
+__device__ __forceinline__ void emi_swiglu_adjoint(float a, float b, float dg, float* da, float* db) {
+  const float s = emi_sigmoid(a);
+  *da = dg * b * s * (1.0f + a * (1.0f - s));
+  *db = dg * a * s;
+}
+
 // Eight consecutive elements as fp32 (one 16-byte load for bf16, two for fp32).
 template <typename T> struct Vec8;
 template <> struct Vec8<float> {

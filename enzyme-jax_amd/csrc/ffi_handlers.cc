@@ -265,6 +265,37 @@ extern "C" XLA_FFI_Error* emi_gemm_ffi(XLA_FFI_CallFrame* cf) {
                                    ws ? byte_size(ws) : 0, M, N, K, A->dims[1], B->dims[1], N, N, (int)ta, (int)tb, A->dtype));
 }
 
+// x[M, K], w3[N, K], a[M, N] -> b[M, N], g[M, N]
+extern "C" XLA_FFI_Error* emi_gemm_swiglu_fwd_ffi(XLA_FFI_CallFrame* cf) {
+  EMI_FFI_BEGIN("emi_gemm_swiglu_fwd", 3, 3, 2, 2)
+  const XLA_FFI_Buffer *X = f.arg(0), *W = f.arg(1), *A = f.arg(2), *B = f.ret(0), *G = f.ret(1);
+  if (!is_float(X) || W->dtype != X->dtype || A->dtype != X->dtype || B->dtype != X->dtype || G->dtype != X->dtype)
+    return f.invalid("x, w3, a, b, g must share one dtype, f32 or bf16 (code %lld)", X->dtype);
+  if (X->rank != 2 || W->rank != 2 || A->rank != 2) return f.invalid("operands must be rank 2");
+  const int64_t M = X->dims[0], K = X->dims[1], N = W->dims[0];
+  if (W->dims[1] != K) return f.invalid("contraction sizes differ: %lld vs %lld", K, W->dims[1]);
+  if (A->dims[0] != M || A->dims[1] != N || !same_shape(A, B) || !same_shape(A, G)) return f.invalid("a, b, g must be [%lld, %lld]", M, N);
+  EMI_FFI_STREAM()
+  return f.from_status(emi_gemm_swiglu_fwd(stream, X->data, W->data, A->data, B->data, G->data, M, N, K, X->dtype));
+}
+
+// dy[M, K], w2t[N, K], a[M, N], b[M, N] -> da[M, N], db[M, N] [, workspace]
+extern "C" XLA_FFI_Error* emi_gemm_swiglu_bwd_ffi(XLA_FFI_CallFrame* cf) {
+  EMI_FFI_BEGIN("emi_gemm_swiglu_bwd", 4, 4, 2, 3)
+  const XLA_FFI_Buffer *dY = f.arg(0), *W = f.arg(1), *A = f.arg(2), *B = f.arg(3), *dA = f.ret(0), *dB = f.ret(1);
+  const XLA_FFI_Buffer* ws = cf->rets.size == 3 ? f.ret(2) : nullptr;
+  if (!is_float(dY) || W->dtype != dY->dtype || A->dtype != dY->dtype || B->dtype != dY->dtype || dA->dtype != dY->dtype || dB->dtype != dY->dtype)
+    return f.invalid("dy, w2t, a, b, da, db must share one dtype, f32 or bf16 (code %lld)", dY->dtype);
+  if (dY->rank != 2 || W->rank != 2 || A->rank != 2) return f.invalid("operands must be rank 2");
+  const int64_t M = dY->dims[0], K = dY->dims[1], N = W->dims[0];
+  if (W->dims[1] != K) return f.invalid("contraction sizes differ: %lld vs %lld", K, W->dims[1]);
+  if (A->dims[0] != M || A->dims[1] != N || !same_shape(A, B) || !same_shape(A, dA) || !same_shape(A, dB))
+    return f.invalid("a, b, da, db must be [%lld, %lld]", M, N);
+  EMI_FFI_STREAM()
+  return f.from_status(emi_gemm_swiglu_bwd(stream, dY->data, W->data, A->data, B->data, dA->data, dB->data, ws ? ws->data : nullptr,
+                                           ws ? byte_size(ws) : 0, M, N, K, dY->dtype));
+}
+
 // count A operands, count B operands, then no residual or one per result; count results (one when `sum`), then an
 // optional scratch result for split-K partials.
 extern "C" XLA_FFI_Error* emi_gemm_grouped_ffi(XLA_FFI_CallFrame* cf) {
@@ -603,6 +634,7 @@ const Target kTargets[] = {
     {"emi_swiglu_fwd", emi_swiglu_fwd_ffi},   {"emi_swiglu_bwd", emi_swiglu_bwd_ffi},
     {"emi_add", emi_add_ffi},                 {"emi_gemm", emi_gemm_ffi},
     {"emi_gemm_grouped", emi_gemm_grouped_ffi},
+    {"emi_gemm_swiglu_fwd", emi_gemm_swiglu_fwd_ffi}, {"emi_gemm_swiglu_bwd", emi_gemm_swiglu_bwd_ffi},
     {"emi_attn_fwd", emi_attn_fwd_ffi},       {"emi_attn_bwd", emi_attn_bwd_ffi},
     {"emi_attn_step_fwd", emi_attn_step_fwd_ffi}, {"emi_attn_step_bwd", emi_attn_step_bwd_ffi},
     {"emi_rmsnorm_jvp", emi_rmsnorm_jvp_ffi}, {"emi_swiglu_jvp", emi_swiglu_jvp_ffi}, {"emi_attn_jvp", emi_attn_jvp_ffi},

@@ -555,6 +555,130 @@ __device__ __forceinline__ void epilogue_bf16_t16(f32x4_t (&acc)[TM][TN], EMI_LD
   }
 }
 
+// Epilogues of the ping-pong kernel that apply the SwiGLU of the FFN (test/llama.py:224-231) to the tile instead of
+// leaving it to a pass of its own over [tokens, hidden]:
+//   MODE 1 (forward, the accumulators hold b = x . W3^T): P0 = a = x . W1^T is read, Q0 = b and Q1 = g = a sigmoid(a) b
+//          are written (the elementwise pass would read a and b again and write g);
+//   MODE 2 (adjoint, the accumulators hold dg = dy . W2): P0 = a and P1 = b are read, Q0 = da and Q1 = db are written;
+//          dg itself never reaches memory (the elementwise pass would read a, b and a stored dg).
+// The products are rounded to bf16 before the elementwise arithmetic, as they are when they go through memory.
+// Whole 128 x 64 wave tiles inside the matrices and 16-byte accesses only (the launcher checks).  All four matrices
+// are [M, N] with leading dimension ld.  Tiles travel through the wavefront's 16 KiB LDS slice as in
+// epilogue_bf16_t16: direct-to-LDS loads / 16-byte row stores on the memory side, 8-byte quads on the accumulator side.
+template <int MODE>
+__device__ __forceinline__ void epilogue_swiglu_t16(f32x4_t (&acc)[8][4], EMI_LDS uint8_t* smem, int wave, int lane, int rbase,
+                                                    int cbase, const uint16_t* P0, const uint16_t* P1, uint16_t* Q0,
+                                                    uint16_t* Q1, int ld) {
+  constexpr int RSB = 128;
+  EMI_LDS uint8_t* wl = smem + wave * (128 * RSB);
+  const int lrow = lane & 15, lq = lane >> 4;
+  auto quad_slot = [&](int row, int j) {      // 8-byte slot of columns 16*j + 4*lq .. +3 of LDS row `row`
+    const int chunk = 2 * j + (lq >> 1);
+    return row * RSB + ((chunk ^ ((row >> 1) & 7)) << 4) + ((lq & 1) << 3);
+  };
+  // wave-load / row-store number it covers LDS rows 8*it .. 8*it+7: lane l moves physical chunk (l & 7) of row
+  // 8*it + (l >> 3), i.e. logical chunk (l & 7) ^ swizzle(row), whose swizzle only depends on the parity of it
+  const int prow = lane >> 3, pc = lane & 7;
+  const uint32_t gE = (uint32_t)prow * (uint32_t)ld * 2u + ((pc ^ (prow >> 1)) << 4);
+  const uint32_t gO = (uint32_t)prow * (uint32_t)ld * 2u + ((pc ^ ((prow >> 1) + 4)) << 4);
+  const uint32_t gC = (uint32_t)prow * (uint32_t)ld * 2u + (pc << 4);
+  const uint32_t ldsE = prow * RSB + ((pc ^ (prow >> 1)) << 4), ldsO = prow * RSB + ((pc ^ ((prow >> 1) + 4)) << 4);
+  // tile rows t0 .. t0+8*n-1 of `src` into LDS rows l0 ..
+  auto load_rows = [&](const uint16_t* src, int t0, int l0, int n) __attribute__((always_inline)) {
+    const uint8_t* sb = reinterpret_cast<const uint8_t*>(src + (int64_t)(rbase + t0) * ld + cbase);       // wave-uniform
+#pragma unroll
+    for (int it = 0; it < 8; it++) {
+      if (it < n) {
+        const uint8_t* p = sb + (int64_t)it * 16 * ld + (((l0 >> 3) + it) & 1 ? gO : gE);
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)p,
+                                         (EMI_LDS void*)(wl + (l0 + 8 * it) * RSB), 16, 0, 0);
+      }
+    }
+  };
+  // LDS rows l0 .. l0+8*n-1 to tile rows t0 .. of `dst`
+  auto store_rows = [&](uint16_t* dst, int t0, int l0, int n) __attribute__((always_inline)) {
+    uint8_t* db = reinterpret_cast<uint8_t*>(dst + (int64_t)(rbase + t0) * ld + cbase);                    // wave-uniform
+#pragma unroll
+    for (int it = 0; it < 16; it++) {
+      if (it < n) {
+        const u32x4_t v = *reinterpret_cast<const EMI_LDS u32x4_t*>(wl + (l0 + 8 * it) * RSB + ((((l0 >> 3) + it) & 1) ? ldsO : ldsE));
+        *reinterpret_cast<u32x4_t*>(db + (int64_t)it * 16 * ld + gC) = v;
+      }
+    }
+  };
+  auto unpack = [](const u32x2_t w, float (&f)[4]) {
+    f[0] = __uint_as_float(w[0] << 16);
+    f[1] = __uint_as_float(w[0] & 0xffff0000u);
+    f[2] = __uint_as_float(w[1] << 16);
+    f[3] = __uint_as_float(w[1] & 0xffff0000u);
+  };
+  if constexpr (MODE == 1) {
+    load_rows(P0, 0, 0, 8);
+    load_rows(P0, 64, 64, 8);
+    wait_vmcnt<0>();
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        EMI_LDS u32x2_t* slot = reinterpret_cast<EMI_LDS u32x2_t*>(wl + quad_slot(i * 16 + lrow, j));
+        float a[4], b[4];
+        unpack(*slot, a);
+        u32x2_t bq;
+        bq[0] = pack_bf16x2(acc[i][j][0], acc[i][j][1]);
+        bq[1] = pack_bf16x2(acc[i][j][2], acc[i][j][3]);
+        unpack(bq, b);
+        *slot = bq;                               // b takes a's place in the slice; g stays in the registers
+#pragma unroll
+        for (int e = 0; e < 4; e++) acc[i][j][e] = emi_swiglu(a[e], b[e]);
+      }
+    store_rows(Q0, 0, 0, 16);
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        u32x2_t w;
+        w[0] = pack_bf16x2(acc[i][j][0], acc[i][j][1]);
+        w[1] = pack_bf16x2(acc[i][j][2], acc[i][j][3]);
+        *reinterpret_cast<EMI_LDS u32x2_t*>(wl + quad_slot(i * 16 + lrow, j)) = w;
+      }
+    store_rows(Q1, 0, 0, 16);
+  } else {
+    // two passes over 64 tile rows: a in LDS rows 0..63, b in LDS rows 64..127
+#pragma unroll
+    for (int p = 0; p < 2; p++) {
+      if (p) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");       // the first pass has read its rows out of the slice
+      load_rows(P0, 64 * p, 0, 8);
+      load_rows(P1, 64 * p, 64, 8);
+      wait_vmcnt<0>();
+#pragma unroll
+      for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          EMI_LDS u32x2_t* sa = reinterpret_cast<EMI_LDS u32x2_t*>(wl + quad_slot(i * 16 + lrow, j));
+          EMI_LDS u32x2_t* sb = reinterpret_cast<EMI_LDS u32x2_t*>(wl + quad_slot(64 + i * 16 + lrow, j));
+          float a[4], b[4], g[4], da[4], db[4];
+          unpack(*sa, a);
+          unpack(*sb, b);
+          u32x2_t gq;
+          gq[0] = pack_bf16x2(acc[4 * p + i][j][0], acc[4 * p + i][j][1]);
+          gq[1] = pack_bf16x2(acc[4 * p + i][j][2], acc[4 * p + i][j][3]);
+          unpack(gq, g);
+#pragma unroll
+          for (int e = 0; e < 4; e++) emi_swiglu_adjoint(a[e], b[e], g[e], &da[e], &db[e]);
+          u32x2_t wa, wb;
+          wa[0] = pack_bf16x2(da[0], da[1]);
+          wa[1] = pack_bf16x2(da[2], da[3]);
+          wb[0] = pack_bf16x2(db[0], db[1]);
+          wb[1] = pack_bf16x2(db[2], db[3]);
+          *sa = wa;
+          *sb = wb;
+        }
+      store_rows(Q0, 64 * p, 0, 8);
+      store_rows(Q1, 64 * p, 64, 8);
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------
 // Ping-pong kernel for two k-contiguous operands (the NT layout): 256x256x64 block
 // tile, 8 wavefronts = two groups of four, one wavefront of each group per SIMD.
@@ -616,13 +740,20 @@ template <int N, typename F> __device__ __forceinline__ void static_for(F&& f) {
 // each, which the swizzle spreads over all 64 banks.
 // GROUPED: the grid holds the tiles of grp.count independent products of one shape, product-major (GemmGroup with
 // sum == 0); otherwise the last argument is an empty placeholder.
-template <bool AKM, bool BKM, bool GROUPED = false>
+// EPI: 0 = the result [+ R]; 1 / 2 = the SwiGLU epilogues (epilogue_swiglu_t16; R is P0, C is Q0, plus P1 and Q1).
+struct NoEpi {};
+struct SwigluEpi {
+  const uint16_t* P1;
+  uint16_t* Q1;
+};
+template <bool AKM, bool BKM, bool GROUPED = false, int EPI = 0>
 __global__ __launch_bounds__(512) void gemm_bf16_pingpong_kernel(const uint16_t* __restrict__ A,
                                                                   const uint16_t* __restrict__ B, const uint16_t* R,
                                                                   uint16_t* C, int M, int N, int K, int lda, int ldb,
                                                                   int ldr, int ldc, uint32_t a_bytes, uint32_t b_bytes,
                                                                   int vec_ok,
-                                                                  std::conditional_t<GROUPED, GemmGroup, NoGroup> grp) {
+                                                                  std::conditional_t<GROUPED, GemmGroup, NoGroup> grp,
+                                                                  std::conditional_t<EPI != 0, SwigluEpi, NoEpi> epi = {}) {
   constexpr int BM = 256, BN = 256, BK = 64;
   constexpr int REGION = 128 * BK * 2;                          // 16 KiB
   // LDS map: A_h of stage s at (2s + h) regions, B_j of stage s at 64 KiB + (2s + j) regions, so that
@@ -867,8 +998,13 @@ __global__ __launch_bounds__(512) void gemm_bf16_pingpong_kernel(const uint16_t*
   wait_vmcnt<0>();                          // zero-filled loads past the end of K
   slot_end();
 
-  epilogue_bf16_t16<8, 4, (BKM ? 96 : 0)>(acc, smem, wave, lane, m0 + wm * 128, n0 + wn * (BKM ? 32 : 64), R, C, M, N, ldr,
-                                          ldc, vec_ok);
+  if constexpr (EPI != 0) {
+    static_assert(!AKM && !BKM && !GROUPED, "the SwiGLU epilogues belong to the k-contiguous single product");
+    epilogue_swiglu_t16<EPI>(acc, smem, wave, lane, m0 + wm * 128, n0 + wn * 64, R, epi.P1, C, epi.Q1, ldc);
+  } else {
+    epilogue_bf16_t16<8, 4, (BKM ? 96 : 0)>(acc, smem, wave, lane, m0 + wm * 128, n0 + wn * (BKM ? 32 : 64), R, C, M, N, ldr,
+                                            ldc, vec_ok);
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -1397,6 +1533,34 @@ static int launch_bf16_pingpong(hipStream_t st, const void* A, const void* B, co
   return EMI_OK;
 }
 
+// C = A . B^T with a SwiGLU epilogue (MODE 1: P0 = a in, Q0 = b, Q1 = g out; MODE 2: P0 = a, P1 = b in, Q0 = da, Q1 = db
+// out).  Returns -1 when the shape is not one the fused kernel serves (the caller then runs the two passes).
+template <int MODE>
+static int launch_bf16_swiglu(hipStream_t st, const void* A, const void* B, const void* P0, const void* P1, void* Q0, void* Q1,
+                              int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb) {
+  auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+  const int64_t a_bytes = ((M - 1) * lda + K) * 2, b_bytes = ((N - 1) * ldb + K) * 2;
+  if (M % 256 || N % 256 || K % 8 || K <= 0 || lda % 8 || ldb % 8 || (M / 256) * (N / 256) < 192 || !al16(A) || !al16(B) ||
+      !al16(P0) || (MODE == 2 && !al16(P1)) || !al16(Q0) || !al16(Q1) || a_bytes >= 0x7fffff00LL || b_bytes >= 0x7fffff00LL ||
+      M * N * 2 >= 0x7fffff00LL)
+    return -1;
+  constexpr int smem = 2 * 65536;
+  auto kern = gemm_bf16_pingpong_kernel<false, false, false, MODE>;
+  static bool configured = false;   // idempotent; a race only repeats the call
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return emi_fail(EMI_INTERNAL, "emi_gemm_swiglu: cannot reserve %d bytes of LDS: %s", smem, hipGetErrorString(e));
+    configured = true;
+  }
+  const int tiles = (int)((M / 256) * (N / 256));
+  hipLaunchKernelGGL(kern, dim3(tiles), dim3(512), smem, st, static_cast<const uint16_t*>(A), static_cast<const uint16_t*>(B),
+                     static_cast<const uint16_t*>(P0), static_cast<uint16_t*>(Q0), (int)M, (int)N, (int)K, (int)lda, (int)ldb, (int)N,
+                     (int)N, (uint32_t)a_bytes, (uint32_t)b_bytes, 1, NoGroup{},
+                     SwigluEpi{static_cast<const uint16_t*>(P1), static_cast<uint16_t*>(Q1)});
+  EMI_CHECK_LAUNCH("emi_gemm_swiglu");
+  return EMI_OK;
+}
+
 // The 128x128 bf16 kernel on few tiles and a long contraction (the weight gradients of a small model:
 // dW[768, 768] over 8192 tokens is 36 tiles): two blocks per CU, at least 1024 of K per block.
 static int bf16_splits(int64_t M, int64_t N, int64_t K) {
@@ -1617,6 +1781,51 @@ extern "C" int emi_gemm_ws(emi_stream_t stream, const void* A, const void* B, co
     return EMI_OK;
   }
   return launch_generic<float>(st, A, B, R, C, (int)M, (int)N, (int)K, lda, ldb, ldr, ldc, trans_a, trans_b, workspace, workspace_bytes);
+}
+
+extern "C" int emi_swiglu_fwd(emi_stream_t stream, const void* a, const void* b, void* g, int64_t n, int dtype);
+extern "C" int emi_swiglu_bwd(emi_stream_t stream, const void* a, const void* b, const void* dg, void* da, void* db, int64_t n,
+                              int dtype);
+
+extern "C" int emi_gemm_swiglu_fwd(emi_stream_t stream, const void* X, const void* W3, const void* A, void* B_out, void* G_out,
+                                   int64_t M, int64_t N, int64_t K, int dtype) {
+  EMI_REQUIRE(M >= 0 && N >= 0 && K >= 0, "emi_gemm_swiglu_fwd: negative dimension");
+  EMI_REQUIRE(dtype == EMI_F32 || dtype == EMI_BF16, "emi_gemm_swiglu_fwd: unsupported dtype code %d", dtype);
+  if (M == 0 || N == 0) return EMI_OK;
+  EMI_REQUIRE(X && W3 && A && B_out && G_out, "emi_gemm_swiglu_fwd: null buffer");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == EMI_BF16) {
+    const int rc = launch_bf16_swiglu<1>(st, X, W3, A, nullptr, B_out, G_out, M, N, K, K, K);
+    if (rc >= 0) return rc;
+  }
+  const int rc = emi_gemm(stream, X, W3, nullptr, B_out, M, N, K, K, K, N, N, 0, 1, dtype);
+  if (rc != EMI_OK) return rc;
+  return emi_swiglu_fwd(stream, A, B_out, G_out, M * N, dtype);
+}
+
+extern "C" size_t emi_gemm_swiglu_bwd_workspace_bytes(int64_t M, int64_t N, int64_t K, int dtype) {
+  if (M <= 0 || N <= 0) return 0;
+  return (size_t)M * N * (dtype == EMI_BF16 ? 2 : 4);           // dg, when the two passes run
+}
+
+extern "C" int emi_gemm_swiglu_bwd(emi_stream_t stream, const void* dY, const void* W2T, const void* A, const void* B, void* dA,
+                                   void* dB, void* workspace, size_t workspace_bytes, int64_t M, int64_t N, int64_t K, int dtype) {
+  EMI_REQUIRE(M >= 0 && N >= 0 && K >= 0, "emi_gemm_swiglu_bwd: negative dimension");
+  EMI_REQUIRE(dtype == EMI_F32 || dtype == EMI_BF16, "emi_gemm_swiglu_bwd: unsupported dtype code %d", dtype);
+  if (M == 0 || N == 0) return EMI_OK;
+  EMI_REQUIRE(dY && W2T && A && B && dA && dB, "emi_gemm_swiglu_bwd: null buffer");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == EMI_BF16) {
+    const int rc = launch_bf16_swiglu<2>(st, dY, W2T, A, B, dA, dB, M, N, K, K, K);
+    if (rc >= 0) return rc;
+  }
+  const size_t need = emi_gemm_swiglu_bwd_workspace_bytes(M, N, K, dtype);
+  EMI_REQUIRE(workspace != nullptr && workspace_bytes >= need && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0,
+              "emi_gemm_swiglu_bwd: this shape runs as two passes and needs a 16-byte aligned workspace of %zu bytes (got %zu)",
+              need, workspace_bytes);
+  const int rc = emi_gemm(stream, dY, W2T, nullptr, workspace, M, N, K, K, K, N, N, 0, 1, dtype);
+  if (rc != EMI_OK) return rc;
+  return emi_swiglu_bwd(stream, A, B, workspace, dA, dB, M * N, dtype);
 }
 
 extern "C" size_t emi_gemm_grouped_workspace_bytes(int count, int64_t M, int64_t N, int64_t K, int trans_a, int trans_b, int sum,

@@ -49,6 +49,9 @@ SIGNATURES = {
     "emi_gemm_grouped": (c_int, [c_void_p, c_int, ctypes.POINTER(c_void_p), ctypes.POINTER(c_void_p), ctypes.POINTER(c_void_p),
                                  ctypes.POINTER(c_void_p), c_void_p, c_size_t, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64,
                                  c_int, c_int, c_int, c_int]),
+    "emi_gemm_swiglu_fwd": (c_int, [c_void_p] * 6 + [c_i64, c_i64, c_i64, c_int]),
+    "emi_gemm_swiglu_bwd_workspace_bytes": (c_size_t, [c_i64, c_i64, c_i64, c_int]),
+    "emi_gemm_swiglu_bwd": (c_int, [c_void_p] * 8 + [c_size_t, c_i64, c_i64, c_i64, c_int]),
     "emi_attn_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_i64, c_i64, c_i64,
                              c_i64, c_i64, c_i64, c_float, c_int, c_int]),
     "emi_attn_fwd_workspace_bytes": (c_size_t, [c_i64, c_i64, c_i64, c_i64]),

@@ -21,9 +21,7 @@ def layer(x, lw, n_heads, eps=1e-5, theta=10000.0):
     att = ops.attention(q, k, v, n_heads, causal=True)             # :178-209
     x = ops.matmul_nt(att, lw["wo"], residual=x)                   # :211-215
     xb = ops.rmsnorm(x, lw["rms_ffn_weight"], eps)                 # :219
-    h1, h3 = ops.matmul_nt_group(xb, (lw["w1"], lw["w3"]))         # :224-227
-    g = ops.swiglu(h1, h3)                                         # :227-229
-    return ops.matmul_nt(g, lw["w2"], residual=x)                  # :231-233
+    return ops.ffn(xb, lw["w1"], lw["w3"], lw["w2"], residual=x)   # :224-233 (SwiGLU in the GEMM epilogues)
 
 
 def forward(x, config, weights, logits=False, eps=1e-5, theta=10000.0):

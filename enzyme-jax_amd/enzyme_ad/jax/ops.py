@@ -31,6 +31,7 @@ FFI_TARGETS = {
     "rope":      ("emi_rope", ("emi_rope",)),                    # adjoint = inverse rotation
     "matmul_nt": ("emi_gemm", ("emi_gemm", "emi_gemm")),         # dX (NN) and dW (TN)
     "swiglu":    ("emi_swiglu_fwd", ("emi_swiglu_bwd",)),
+    "ffn":       ("emi_gemm_swiglu_fwd", ("emi_gemm_swiglu_bwd", "emi_gemm_grouped", "emi_gemm")),   # between two emi_gemm
     "attention": ("emi_attn_fwd", ("emi_attn_bwd",)),
     "attention_step": ("emi_attn_step_fwd", ("emi_attn_step_bwd",)),
     "add":       ("emi_add", ()),
@@ -750,6 +751,71 @@ def swiglu(a, b):
         N.check(N.lib().emi_swiglu_jvp(_stream(), _p(a), _p(b), _p(tans[0]), _p(tans[1]), _p(tg), a.numel(), _code(a)))
         _set_tan(g, tg)
     return g
+
+
+def ffn(xb, w1, w3, w2, residual=None):
+    """The SwiGLU FFN of test/llama.py:224-233 as one operator: w2 @ (silu(w1 @ xb) * (w3 @ xb)) [+ residual], with the
+    elementwise part applied in GEMM epilogues (emi_gemm_swiglu_fwd / _bwd) instead of in passes of their own over
+    [tokens, hidden].  The same values and gradients as matmul_nt_group + swiglu + matmul_nt, whose rules it chains:
+    h1, h3 = x W1^T, x W3^T;  g = swiglu(h1, h3);  y = g W2^T + r.  Reverse: dW2 = dY^T g; (dh1, dh3) from dY . W2 through
+    the SwiGLU adjoint in the product's epilogue; dX = dh1 . W1 + dh3 . W3 as one summed launch; dW1, dW3 grouped.
+    Shapes the fused kernels do not serve, fp32, and forward mode take the three separate operators."""
+    lead, K = xb.shape[:-1], xb.shape[-1]
+    Hn = w1.shape[0]
+    fused = (xb.dtype == torch.bfloat16 and Forward._active is None and w1.shape == w3.shape and w2.shape == (K, Hn)
+             and w1.dtype == xb.dtype and w3.dtype == xb.dtype and w2.dtype == xb.dtype
+             and xb.numel() // K >= 256 and (residual is None or residual.shape == xb.shape))
+    if not fused:
+        h1, h3 = matmul_nt_group(xb, (w1, w3))
+        return matmul_nt(swiglu(h1, h3), w2, residual=residual)
+    _dev(xb, w1, w3, w2, residual)
+    x2 = xb.reshape(-1, K)
+    T = x2.shape[0]
+    lib = N.lib()
+    h1 = gemm(x2, w1, False, True)
+    h3 = torch.empty_like(h1)
+    g = torch.empty_like(h1)
+    N.check(lib.emi_gemm_swiglu_fwd(_stream(), _p(x2), _p(w3), _p(h1), _p(h3), _p(g), T, Hn, K, _code(x2)))
+    r2 = None if residual is None else residual.reshape(-1, K)
+    y = gemm(g, w2, False, True, r2).reshape(*lead, K)
+
+    def rule(c, acc):
+        c2 = c.reshape(-1, K)
+        # w2: dW2 = dY^T . g (deferred when its destination is a slice of a stacked gradient)
+        target = _grad_target(w2, acc[3])
+        if target is not None:
+            _defer_dw(c2, g, target)
+            dw2 = target
+        else:
+            dw2 = gemm(c2, g, True, False, acc[3])
+        # (dh1, dh3) = SwiGLU adjoint of dY . W2, in the epilogue of that product
+        dh1, dh3 = torch.empty_like(h1), torch.empty_like(h3)
+        nbytes = lib.emi_gemm_swiglu_bwd_workspace_bytes(T, Hn, K, _code(c2))
+        one_launch = T % 256 == 0 and Hn % 256 == 0 and (T // 256) * (Hn // 256) >= 192      # else dY . W2 goes through a workspace
+        ws = None if one_launch else torch.empty(nbytes, dtype=torch.uint8, device=c2.device)
+        N.check(lib.emi_gemm_swiglu_bwd(_stream(), _p(c2), _p(_transpose_shared(w2)), _p(h1), _p(h3), _p(dh1), _p(dh3), _p(ws),
+                                        nbytes if ws is not None else 0, T, Hn, K, _code(c2)))
+        # the group's rule: dX summed over the two branches, dW1 / dW3 grouped or deferred
+        ax = None if acc[0] is None else acc[0].reshape(-1, K)
+        dx = gemm_grouped([dh1, dh3], [_transpose_shared(w1), _transpose_shared(w3)], False, True, None if ax is None else [ax],
+                          sum_into_one=True).reshape(xb.shape)
+        t1, t3 = _grad_target(w1, acc[1]), _grad_target(w3, acc[2])
+        if t1 is not None and t3 is not None:
+            _defer_dw(dh1, x2, t1)
+            _defer_dw(dh3, x2, t3)
+            dw1, dw3 = t1, t3
+        elif t1 is not None or t3 is not None or (acc[1] is None) != (acc[2] is None):
+            dw1 = gemm(dh1, x2, True, False, acc[1], out=t1)
+            dw3 = gemm(dh3, x2, True, False, acc[2], out=t3)
+        else:
+            dw1, dw3 = gemm_grouped([dh1, dh3], [x2, x2], True, False, None if acc[1] is None else [acc[1], acc[2]])
+        out = [dx, dw1, dw3, dw2]
+        if residual is not None:
+            out.append(_accumulate(acc[4], c))
+        return out
+
+    Tape.record((xb, w1, w3, w2) if residual is None else (xb, w1, w3, w2, residual), y, rule)
+    return y
 
 
 def attention_raw(q, k, v, n_heads, scale, causal, strides):

@@ -143,6 +143,23 @@ int emi_gemm_grouped(emi_stream_t stream, int count, const void* const* A, const
                      void* const* C, void* workspace, size_t workspace_bytes, int64_t M, int64_t N, int64_t K, int64_t lda,
                      int64_t ldb, int64_t ldr, int64_t ldc, int trans_a, int trans_b, int sum, int dtype);
 
+/* The SwiGLU of the FFN (test/llama.py:224-231: hb = w1 @ xb; hb2 = w3 @ xb; hb = hb * sigmoid(hb) * hb2) applied in the
+ * epilogue of the product next to it, so that the elementwise pass over [tokens, hidden] disappears; same results as
+ * the product followed by emi_swiglu_fwd / emi_swiglu_bwd (the product is rounded to its type before the elementwise
+ * arithmetic, as it is when it goes through memory).  All matrices contiguous.
+ *   emi_gemm_swiglu_fwd:  B_out[M, N] = X[M, K] . W3[N, K]^T ;  G_out = A * sigmoid(A) * B_out   (A = X . W1^T, given)
+ *   emi_gemm_swiglu_bwd:  dG = dY[M, K] . W2T[N, K]^T (never stored) ;  (dA, dB) = adjoint of SwiGLU at (A, B) on dG
+ *                         (W2T = the transposed down projection, [hidden, dim]; Mul / Div / Exp rules
+ *                         HLODerivatives.td:1221,1133,1182 behind the DotGeneral rule :1166-1178)
+ * bf16 products of whole 256 x 256 tiles (M, N multiples of 256, at least 192 tiles, 16-byte aligned buffers) run as
+ * one launch; anything else as the product followed by the elementwise kernel, for which emi_gemm_swiglu_bwd needs a
+ * workspace of emi_gemm_swiglu_bwd_workspace_bytes (dG) and fails without it. */
+int emi_gemm_swiglu_fwd(emi_stream_t stream, const void* X, const void* W3, const void* A, void* B_out, void* G_out, int64_t M,
+                        int64_t N, int64_t K, int dtype);
+size_t emi_gemm_swiglu_bwd_workspace_bytes(int64_t M, int64_t N, int64_t K, int dtype);
+int emi_gemm_swiglu_bwd(emi_stream_t stream, const void* dY, const void* W2T, const void* A, const void* B, void* dA, void* dB,
+                        void* workspace, size_t workspace_bytes, int64_t M, int64_t N, int64_t K, int dtype);
+
 /* Causal softmax attention, forward.  Replaces the per-head loop of
  * test/llama.py:178-206 with softmax of :13-18 (scale applied after the dot,
  * max-subtracted, fp32 statistics).  Element (b, h, s, i) of q/k/v/o lives at

@@ -405,3 +405,70 @@ def test_transpose(ops, dt, rows, cols):
     rng = np.random.default_rng(rows + cols)
     a, ar = dev(rng.standard_normal((rows, cols)), dt)
     assert np.array_equal(host(ops.transpose(a)), ar.T)      # a pure permutation is exact
+
+
+@pytest.mark.parametrize("T,D,Hd,dt", [(2048, 512, 6144, "bf16"),      # one launch each way: 8 x 24 = 192 tiles of 256 x 256
+                                       (520, 256, 704, "bf16"),        # ragged: product followed by the elementwise kernel
+                                       (300, 128, 352, "f32")])
+def test_gemm_swiglu_epilogues(ops, T, D, Hd, dt):
+    """emi_gemm_swiglu_fwd / _bwd (the SwiGLU of test/llama.py:224-231 in the epilogue of the product next to it) through
+    the C ABI and through their XLA-FFI handlers, against the oracle's linear and SwiGLU rules; and the `ffn` operator
+    built on them (value and every gradient) against matmul_nt_group + swiglu + matmul_nt."""
+    import ctypes as C
+    import ffi_frames as F
+    from enzyme_ad.jax import _native as N, vjp
+    lib = N.lib()
+    st = torch.cuda.current_stream().cuda_stream
+    rng = np.random.default_rng(T + Hd)
+    x, xr = dev(rng.standard_normal((T, D)), dt)
+    w1, w1r = dev(rng.standard_normal((Hd, D)) * 0.1, dt)
+    w3, w3r = dev(rng.standard_normal((Hd, D)) * 0.1, dt)
+    w2, w2r = dev(rng.standard_normal((D, Hd)) * 0.1, dt)
+    dy, dyr = dev(rng.standard_normal((T, D)), dt)
+    code = N.EMI_BF16 if dt == "bf16" else N.EMI_F32
+    a = ops.gemm(x, w1, False, True)
+    b, g = torch.empty_like(a), torch.empty_like(a)
+    N.check(lib.emi_gemm_swiglu_fwd(st, x.data_ptr(), w3.data_ptr(), a.data_ptr(), b.data_ptr(), g.data_ptr(), T, Hd, D, code))
+    ar_, br_ = host(a), L.linear_fwd(xr, w3r)
+    check(b, br_, dt, "b = x w3^T")
+    check(g, L.swiglu_fwd(ar_, host(b)), dt, "g = swiglu(a, b)")
+    assert torch.equal(b, ops.gemm(x, w3, False, True)) and torch.equal(g, ops.swiglu(a, b))
+    w2t = w2.t().contiguous()
+    da, db = torch.empty_like(a), torch.empty_like(a)
+    nb = lib.emi_gemm_swiglu_bwd_workspace_bytes(T, Hd, D, code)
+    ws = torch.empty(nb, dtype=torch.uint8, device="cuda")
+    N.check(lib.emi_gemm_swiglu_bwd(st, dy.data_ptr(), w2t.data_ptr(), a.data_ptr(), b.data_ptr(), da.data_ptr(), db.data_ptr(),
+                                    ws.data_ptr(), nb, T, Hd, D, code))
+    dg = ops.gemm(dy, w2t, False, True)
+    rda, rdb = L.swiglu_bwd(host(a), host(b), host(dg))
+    check(da, rda, dt, "da")
+    check(db, rdb, dt, "db")
+    # the handlers
+    xla = F.FakeXla(stream=st)
+    codes = {torch.float32: F.F32, torch.bfloat16: F.BF16, torch.uint8: F.U8}
+    buf = lambda t: xla.buffer(codes[t.dtype], list(t.shape), t.data_ptr())
+
+    def call(name, args, rets):
+        fn = getattr(lib, name)
+        fn.restype, fn.argtypes = C.c_void_p, [C.POINTER(F.CallFrame)]
+        cf = xla.frame(args, rets, {})
+        assert fn(C.byref(cf)) is None, (name, xla.errors)
+
+    b2, g2, da2, db2 = (torch.empty_like(a) for _ in range(4))
+    call("emi_gemm_swiglu_fwd_ffi", [buf(x), buf(w3), buf(a)], [buf(b2), buf(g2)])
+    call("emi_gemm_swiglu_bwd_ffi", [buf(dy), buf(w2t), buf(a), buf(b)], [buf(da2), buf(db2), buf(ws)])
+    torch.cuda.synchronize()
+    assert torch.equal(b2, b) and torch.equal(g2, g) and torch.equal(da2, da) and torch.equal(db2, db)
+    # the operator
+    r, rr = dev(rng.standard_normal((T, D)), dt)
+
+    def unfused(x, w1, w3, w2, r):
+        h1, h3 = ops.matmul_nt_group(x, (w1, w3))
+        return ops.matmul_nt(ops.swiglu(h1, h3), w2, residual=r)
+
+    y0, f0 = vjp(unfused, x, w1, w3, w2, r)
+    y1, f1 = vjp(ops.ffn, x, w1, w3, w2, r)
+    h = L.swiglu_fwd(L.linear_fwd(xr, w1r), L.linear_fwd(xr, w3r))
+    check(y1, L.linear_fwd(h, w2r) + rr, dt, "ffn value")
+    for name, u, v in zip(("dx", "dw1", "dw3", "dw2", "dr"), f0(dy), f1(dy)):
+        check(v, host(u), dt, "ffn " + name + " against the separate operators", factor=0.5)
