@@ -846,6 +846,15 @@ __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(const uint16_t* __rest
   }
 }
 
+// The adjoint of RoPE (test/llama.py:161-168) on four consecutive elements of a head's row (two rotation pairs): the
+// cotangent of the rotated vector is turned back by the angle.  t points at the (cos, sin) entries of the two pairs.
+__device__ __forceinline__ void unrope_quad(const float* t, float& x0, float& x1, float& x2, float& x3) {
+  const float4 cs = *reinterpret_cast<const float4*>(t);
+  const float y0 = cs.x * x0 + cs.y * x1, y1 = cs.x * x1 - cs.y * x0;
+  const float y2 = cs.z * x2 + cs.w * x3, y3 = cs.z * x3 - cs.w * x2;
+  x0 = y0, x1 = y1, x2 = y2, x3 = y3;
+}
+
 // ---------------------------------------------------------------------------
 // dQ: block = 4 waves x 32 queries; K and V tiles of 64 keys through LDS.
 //   S^T = K Q^T, dP^T = V dO^T, dS^T = P^T (dP^T - delta), dQ^T = K^T dS^T
@@ -859,7 +868,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_bf16_kernel(const uint16_t
                                                                const float* __restrict__ delta,
                                                                uint16_t* __restrict__ dq, AttnShape sh,
                                                                uint32_t head_bytes, float scale, int causal,
-                                                               float delta_sign) {
+                                                               float delta_sign, const float* __restrict__ unrope) {
   constexpr int BQ = 128, BKV = 64, NW = 4;
   constexpr int TILE = BKV * D * 2, STAGE = 2 * TILE;
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem_raw[];
@@ -942,14 +951,18 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_bf16_kernel(const uint16_t
   }
   if (qrow < seq) {
     uint16_t* out = dq + base + (int64_t)qrow * sh.ss;
+    const float* trow = unrope ? unrope + (int64_t)qrow * D : nullptr;     // D/2 (cos, sin) pairs per position
 #pragma unroll
     for (int dt = 0; dt < D / 32; dt++)
 #pragma unroll
       for (int jj = 0; jj < 4; jj++) {
         const int dcol = dt * 32 + 8 * jj + 4 * (lane >> 5);
+        float x0 = acc[dt][4 * jj] * scale, x1 = acc[dt][4 * jj + 1] * scale, x2 = acc[dt][4 * jj + 2] * scale,
+              x3 = acc[dt][4 * jj + 3] * scale;
+        if (trow != nullptr) unrope_quad(trow + dcol, x0, x1, x2, x3);
         uint2 w;
-        w.x = pack_bf16x2(acc[dt][4 * jj] * scale, acc[dt][4 * jj + 1] * scale);
-        w.y = pack_bf16x2(acc[dt][4 * jj + 2] * scale, acc[dt][4 * jj + 3] * scale);
+        w.x = pack_bf16x2(x0, x1);
+        w.y = pack_bf16x2(x2, x3);
         *reinterpret_cast<uint2*>(out + dcol) = w;
       }
   }
@@ -1017,7 +1030,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_sp_kernel(const uint16_t* __
                                                               const float* __restrict__ lse2,
                                                               const float* __restrict__ delta, uint16_t* __restrict__ dk,
                                                               uint16_t* __restrict__ dv, AttnShape sh,
-                                                              uint32_t head_bytes, float scale, int causal) {
+                                                              uint32_t head_bytes, float scale, int causal,
+                                                              const float* __restrict__ unrope) {
   constexpr int BKEY = 128, BQT = 64, NW = 4, NSLOT = 3;
   constexpr int TILE = BQT * D * 2;
   constexpr int STATS = 2 * NSLOT * TILE;                 // lse2 and delta of each slot: 2 x 256 bytes
@@ -1224,6 +1238,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_sp_kernel(const uint16_t* __
     constexpr int CH = D / 8, RB = D * 2;
     EMI_LDS uint8_t* wl = smem + wave * (32 * RB);
     const int r = lane & 31, g = lane >> 5;
+    const float* trow = (unrope != nullptr && krow < seq) ? unrope + (int64_t)krow * D : nullptr;   // dK only
 #pragma unroll
     for (int which = 0; which < 2; which++) {
       const float mul = which ? 1.0f : scale;
@@ -1232,9 +1247,11 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_sp_kernel(const uint16_t* __
 #pragma unroll
         for (int jj = 0; jj < 4; jj++) {
           const f32x16_t& a = which ? acc_v[dt] : acc_k[dt];
+          float x0 = a[4 * jj] * mul, x1 = a[4 * jj + 1] * mul, x2 = a[4 * jj + 2] * mul, x3 = a[4 * jj + 3] * mul;
+          if (which == 0 && trow != nullptr) unrope_quad(trow + dt * 32 + 8 * jj + 4 * g, x0, x1, x2, x3);
           u32x2_t w;
-          w[0] = pack_bf16x2(a[4 * jj] * mul, a[4 * jj + 1] * mul);
-          w[1] = pack_bf16x2(a[4 * jj + 2] * mul, a[4 * jj + 3] * mul);
+          w[0] = pack_bf16x2(x0, x1);
+          w[1] = pack_bf16x2(x2, x3);
           const int c = dt * 4 + jj;
           *reinterpret_cast<EMI_LDS u32x2_t*>(wl + r * RB + ((c ^ (r & (CH - 1))) << 4) + ((g ^ ((r / CH) & 1)) << 3)) = w;
         }
@@ -1566,14 +1583,31 @@ extern "C" size_t emi_attn_bwd_workspace_bytes(int64_t batch, int64_t heads, int
   return 2 * (size_t)batch * (size_t)heads * (size_t)seq * sizeof(float);   // delta = rowsum(dO * O), lse * log2(e)
 }
 
-extern "C" int emi_attn_bwd(emi_stream_t stream, const void* q, const void* k, const void* v, const void* o,
-                            const float* lse, const void* d_o, void* dq, void* dk, void* dv, void* workspace,
-                            size_t workspace_bytes, int64_t batch, int64_t heads, int64_t seq, int64_t head_dim,
-                            int64_t stride_b, int64_t stride_h, int64_t stride_s, float scale, int causal, int dtype) {
+extern "C" int emi_rope(emi_stream_t stream, const void* x, const float* table, void* y, int64_t batch, int64_t seq,
+                        int64_t heads, int64_t head_dim, int inverse, int dtype);
+
+// unrope: null, or the RoPE angle table [seq, head_dim/2] of (cos, sin): dq and dk are then the cotangents of the
+// vectors before their rotation (the MFMA kernels turn them back as they store them; otherwise a pass over each).
+static int attn_bwd_impl(emi_stream_t stream, const void* q, const void* k, const void* v, const void* o, const float* lse,
+                         const void* d_o, void* dq, void* dk, void* dv, void* workspace, size_t workspace_bytes, int64_t batch,
+                         int64_t heads, int64_t seq, int64_t head_dim, int64_t stride_b, int64_t stride_h, int64_t stride_s,
+                         float scale, int causal, int dtype, const float* unrope) {
   const AttnArgs a{batch, heads, seq, head_dim, stride_b, stride_h, stride_s};
   if (int rc = check_common("emi_attn_bwd", a, dtype)) return rc;
   if (batch == 0) return EMI_OK;
   EMI_REQUIRE(q && k && v && o && lse && d_o && dq && dk && dv, "emi_attn_bwd: null buffer");
+  if (unrope != nullptr) {
+    EMI_REQUIRE((reinterpret_cast<uintptr_t>(unrope) & 15) == 0, "emi_attn_bwd_rope: the angle table must be 16-byte aligned");
+    if (!mfma_ok(a, dtype, {q, k, v, o, d_o, dq, dk, dv})) {
+      EMI_REQUIRE(stride_h == head_dim && stride_s == heads * head_dim && stride_b == seq * stride_s,
+                  "emi_attn_bwd_rope: this shape needs contiguous [batch, seq, heads, head_dim] operands");
+      int rc = attn_bwd_impl(stream, q, k, v, o, lse, d_o, dq, dk, dv, workspace, workspace_bytes, batch, heads, seq, head_dim,
+                             stride_b, stride_h, stride_s, scale, causal, dtype, nullptr);
+      if (rc == EMI_OK) rc = emi_rope(stream, dq, unrope, dq, batch, seq, heads, head_dim, 1, dtype);
+      if (rc == EMI_OK) rc = emi_rope(stream, dk, unrope, dk, batch, seq, heads, head_dim, 1, dtype);
+      return rc;
+    }
+  }
   const size_t need = emi_attn_bwd_workspace_bytes(batch, heads, seq, head_dim);
   EMI_REQUIRE(workspace != nullptr && workspace_bytes >= need, "emi_attn_bwd: workspace of %zu bytes needed, got %zu", need,
               workspace_bytes);
@@ -1609,12 +1643,12 @@ extern "C" int emi_attn_bwd(emi_stream_t stream, const void* q, const void* k, c
     if (int rc = reserve_lds(attn_bwd_dkv_sp_kernel<DD>, smem_sp, "emi_attn_bwd")) return rc;                            \
     hipLaunchKernelGGL(attn_bwd_dkv_sp_kernel<DD>, grid, dim3(256), smem_sp, st, (const uint16_t*)q,                     \
                        (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse2, delta, (uint16_t*)dk,         \
-                       (uint16_t*)dv, shp, head_bytes, scale, causal);                                                   \
+                       (uint16_t*)dv, shp, head_bytes, scale, causal, unrope);                                           \
     EMI_CHECK_LAUNCH("emi_attn_bwd(dkv)");                                                                               \
     if (int rc = reserve_lds(attn_bwd_dq_bf16_kernel<DD>, smem_q, "emi_attn_bwd")) return rc;                            \
     hipLaunchKernelGGL(attn_bwd_dq_bf16_kernel<DD>, grid, dim3(256), smem_q, st, (const uint16_t*)q, (const uint16_t*)k, \
                        (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, (uint16_t*)dq, shp, head_bytes, scale,      \
-                       causal, delta_sign);                                                                              \
+                       causal, delta_sign, unrope);                                                                      \
   } while (0)
     if (head_dim == 128) EMI_ATTN_BWD_LAUNCH(128);
     else EMI_ATTN_BWD_LAUNCH(64);
@@ -1643,4 +1677,22 @@ extern "C" int emi_attn_bwd(emi_stream_t stream, const void* q, const void* k, c
   }
   EMI_CHECK_LAUNCH("emi_attn_bwd(generic)");
   return EMI_OK;
+}
+
+extern "C" int emi_attn_bwd(emi_stream_t stream, const void* q, const void* k, const void* v, const void* o,
+                            const float* lse, const void* d_o, void* dq, void* dk, void* dv, void* workspace,
+                            size_t workspace_bytes, int64_t batch, int64_t heads, int64_t seq, int64_t head_dim,
+                            int64_t stride_b, int64_t stride_h, int64_t stride_s, float scale, int causal, int dtype) {
+  return attn_bwd_impl(stream, q, k, v, o, lse, d_o, dq, dk, dv, workspace, workspace_bytes, batch, heads, seq, head_dim,
+                       stride_b, stride_h, stride_s, scale, causal, dtype, nullptr);
+}
+
+extern "C" int emi_attn_bwd_rope(emi_stream_t stream, const void* q, const void* k, const void* v, const void* o,
+                                 const float* lse, const void* d_o, void* dq, void* dk, void* dv, const float* rope_table,
+                                 void* workspace, size_t workspace_bytes, int64_t batch, int64_t heads, int64_t seq,
+                                 int64_t head_dim, int64_t stride_b, int64_t stride_h, int64_t stride_s, float scale,
+                                 int causal, int dtype) {
+  EMI_REQUIRE(rope_table != nullptr || batch == 0, "emi_attn_bwd_rope: null angle table");
+  return attn_bwd_impl(stream, q, k, v, o, lse, d_o, dq, dk, dv, workspace, workspace_bytes, batch, heads, seq, head_dim,
+                       stride_b, stride_h, stride_s, scale, causal, dtype, rope_table);
 }

@@ -279,6 +279,23 @@ extern "C" XLA_FFI_Error* emi_gemm_swiglu_fwd_ffi(XLA_FFI_CallFrame* cf) {
   return f.from_status(emi_gemm_swiglu_fwd(stream, X->data, W->data, A->data, B->data, G->data, M, N, K, X->dtype));
 }
 
+// x[M, K], w[N, K], table[seq, head_dim/2, 2] -> y[M, N] = rope(x . w^T); rows are whole sequences of `seq` positions
+extern "C" XLA_FFI_Error* emi_gemm_rope_ffi(XLA_FFI_CallFrame* cf) {
+  EMI_FFI_BEGIN("emi_gemm_rope", 3, 3, 1, 1)
+  const XLA_FFI_Buffer *X = f.arg(0), *W = f.arg(1), *T = f.arg(2), *Y = f.ret(0);
+  if (!is_float(X) || W->dtype != X->dtype || Y->dtype != X->dtype)
+    return f.invalid("x, w, y must share one dtype, f32 or bf16 (code %lld)", X->dtype);
+  if (X->rank != 2 || W->rank != 2 || Y->rank != 2) return f.invalid("x, w, y must be rank 2");
+  const int64_t M = X->dims[0], K = X->dims[1], N = W->dims[0];
+  if (W->dims[1] != K) return f.invalid("contraction sizes differ: %lld vs %lld", K, W->dims[1]);
+  if (Y->dims[0] != M || Y->dims[1] != N) return f.invalid("y must be [%lld, %lld]", M, N);
+  if (T->dtype != XLA_FFI_DataType_F32 || T->rank != 3 || T->dims[2] != 2 || T->dims[0] <= 0 || T->dims[1] <= 0)
+    return f.invalid("the angle table must be f32[seq, head_dim/2, 2]");
+  EMI_FFI_STREAM()
+  return f.from_status(emi_gemm_rope(stream, X->data, W->data, Y->data, static_cast<const float*>(T->data), M, N, K, T->dims[0],
+                                     2 * T->dims[1], X->dtype));
+}
+
 // dy[M, K], w2t[N, K], a[M, N], b[M, N] -> da[M, N], db[M, N] [, workspace]
 extern "C" XLA_FFI_Error* emi_gemm_swiglu_bwd_ffi(XLA_FFI_CallFrame* cf) {
   EMI_FFI_BEGIN("emi_gemm_swiglu_bwd", 4, 4, 2, 3)
@@ -407,6 +424,35 @@ extern "C" XLA_FFI_Error* emi_attn_bwd_ffi(XLA_FFI_CallFrame* cf) {
   return f.from_status(emi_attn_bwd(stream, q->data, k->data, v->data, o->data, static_cast<const float*>(lse->data), d_o->data,
                                     dq->data, dk->data, dv->data, ws->data, byte_size(ws), d.B, d.H, d.S, d.D, d.sb, d.sh, d.ss,
                                     (float)scale, (int)causal, q->dtype));
+}
+
+// emi_attn_bwd with a seventh operand, the RoPE angle table f32[seq, head_dim/2, 2]: dq and dk come out as the
+// cotangents of q and k before their rotation.
+extern "C" XLA_FFI_Error* emi_attn_bwd_rope_ffi(XLA_FFI_CallFrame* cf) {
+  EMI_FFI_BEGIN("emi_attn_bwd_rope", 7, 7, 4, 4)
+  const XLA_FFI_Buffer *q = f.arg(0), *k = f.arg(1), *v = f.arg(2), *o = f.arg(3), *lse = f.arg(4), *d_o = f.arg(5), *T = f.arg(6);
+  const XLA_FFI_Buffer *dq = f.ret(0), *dk = f.ret(1), *dv = f.ret(2), *ws = f.ret(3);
+  const XLA_FFI_Buffer* same[] = {k, v, o, d_o, dq, dk, dv};
+  if (!is_float(q)) return f.invalid("q must be f32 or bf16 (code %lld)", q->dtype);
+  for (const XLA_FFI_Buffer* b : same)
+    if (b->dtype != q->dtype || !same_shape(q, b)) return f.invalid("q, k, v, o, do, dq, dk, dv must share dtype and shape");
+  int64_t causal = 1, bshd = 0;
+  double scale;
+  f.get_i("causal", &causal);
+  f.get_i("bshd", &bshd);
+  if (!f.get_f("scale", &scale)) return f.invalid("missing f32/f64 attribute 'scale'");
+  AttnDims d;
+  if (!attn_dims(q, bshd, &d)) return f.invalid("q must be rank 4 (rank %lld)", q->rank);
+  if (lse->dtype != XLA_FFI_DataType_F32 || lse->rank != 3 || lse->dims[0] != d.B || lse->dims[1] != d.H || lse->dims[2] != d.S)
+    return f.invalid("lse must be f32[batch, heads, seq] = [%lld, %lld, %lld]", d.B, d.H, d.S);
+  if (T->dtype != XLA_FFI_DataType_F32 || T->rank != 3 || T->dims[0] != d.S || 2 * T->dims[1] != d.D || T->dims[2] != 2)
+    return f.invalid("the angle table must be f32[seq, head_dim/2, 2] = [%lld, %lld, 2]", d.S, d.D / 2);
+  const size_t need = emi_attn_bwd_workspace_bytes(d.B, d.H, d.S, d.D);
+  if (byte_size(ws) < need) return f.invalid("workspace result has %lld bytes, %lld needed", (long long)byte_size(ws), (long long)need);
+  EMI_FFI_STREAM()
+  return f.from_status(emi_attn_bwd_rope(stream, q->data, k->data, v->data, o->data, static_cast<const float*>(lse->data),
+                                         d_o->data, dq->data, dk->data, dv->data, static_cast<const float*>(T->data), ws->data,
+                                         byte_size(ws), d.B, d.H, d.S, d.D, d.sb, d.sh, d.ss, (float)scale, (int)causal, q->dtype));
 }
 
 // Forward mode: tangents are ordinary operands (a zero tangent is passed as zeros).
@@ -635,6 +681,7 @@ const Target kTargets[] = {
     {"emi_add", emi_add_ffi},                 {"emi_gemm", emi_gemm_ffi},
     {"emi_gemm_grouped", emi_gemm_grouped_ffi},
     {"emi_gemm_swiglu_fwd", emi_gemm_swiglu_fwd_ffi}, {"emi_gemm_swiglu_bwd", emi_gemm_swiglu_bwd_ffi},
+    {"emi_gemm_rope", emi_gemm_rope_ffi},     {"emi_attn_bwd_rope", emi_attn_bwd_rope_ffi},
     {"emi_attn_fwd", emi_attn_fwd_ffi},       {"emi_attn_bwd", emi_attn_bwd_ffi},
     {"emi_attn_step_fwd", emi_attn_step_fwd_ffi}, {"emi_attn_step_bwd", emi_attn_step_bwd_ffi},
     {"emi_rmsnorm_jvp", emi_rmsnorm_jvp_ffi}, {"emi_swiglu_jvp", emi_swiglu_jvp_ffi}, {"emi_attn_jvp", emi_attn_jvp_ffi},

@@ -439,11 +439,16 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_kernel(const uint16_t* 
 // column-quad accesses of the accumulator layout and for the 16-byte row accesses
 // of the global loads and stores.  CSPLIT: the wave tile's columns 32..63 lie CSPLIT
 // columns further right in C (two 32-column strips instead of one 64-column strip).
-template <int TM, int TN, int CSPLIT = 0>
+// ROPE: the rows are token vectors of heads of `rope_hd` elements and the result is stored rotated (test/llama.py:161-168):
+// a lane's four consecutive columns are two rotation pairs, whose (cos, sin) entries are 16 bytes of the fp32 table
+// [rope_seq, rope_hd/2]; row r sits at position r % rope_seq.  Whole wave tiles only (the launcher checks).
+template <int TM, int TN, int CSPLIT = 0, bool ROPE = false, bool FULL = false>
 __device__ __forceinline__ void epilogue_bf16_t16(f32x4_t (&acc)[TM][TN], EMI_LDS uint8_t* smem, int wave, int lane,
                                                   int rbase, int cbase, const uint16_t* R, uint16_t* C, int M, int N,
-                                                  int ldr, int ldc, int vec_ok) {
+                                                  int ldr, int ldc, int vec_ok, const float* rope = nullptr,
+                                                  int rope_seq = 1, int rope_hd = 4) {
   static_assert(TN == 4, "64-column wave tile");
+  static_assert(!ROPE || CSPLIT == 0, "rotation pairs are adjacent columns");
   constexpr int WR = TM * 16, RSB = 128;
   EMI_LDS uint8_t* wl = smem + wave * (WR * RSB);
   const int lrow = lane & 15, lq = lane >> 4;
@@ -453,7 +458,7 @@ __device__ __forceinline__ void epilogue_bf16_t16(f32x4_t (&acc)[TM][TN], EMI_LD
   };
   // Whole wave tile inside C and 16-byte accesses allowed (wave-uniform): straight-line
   // code, the residual comes in with direct-to-LDS loads that are all in flight at once.
-  if (vec_ok && rbase + WR <= M && cbase + CSPLIT + 64 <= N) {
+  if (ROPE || FULL || (vec_ok && rbase + WR <= M && cbase + CSPLIT + 64 <= N)) {
     // Wave-load it covers rows 8*it .. 8*it+7: lane l moves physical chunk (l & 7) of row 8*it + (l >> 3),
     // whose swizzle term ((row >> 1) & 7) only depends on the parity of it.
     const int prow = lane >> 3, pc = lane & 7;
@@ -480,6 +485,56 @@ __device__ __forceinline__ void epilogue_bf16_t16(f32x4_t (&acc)[TM][TN], EMI_LD
           acc[i][j][2] += __uint_as_float(w[1] << 16);
           acc[i][j][3] += __uint_as_float(w[1] & 0xffff0000u);
         }
+    }
+    if constexpr (ROPE) {
+      const int hcol = (cbase + 4 * lq) % rope_hd;
+      auto rotate = [&](int i, int j, const float4& t) {
+        const float x0 = acc[i][j][0], x1 = acc[i][j][1], x2 = acc[i][j][2], x3 = acc[i][j][3];
+        acc[i][j][0] = t.x * x0 - t.y * x1;
+        acc[i][j][1] = t.y * x0 + t.x * x1;
+        acc[i][j][2] = t.z * x2 - t.w * x3;
+        acc[i][j][3] = t.w * x2 + t.z * x3;
+      };
+      const int p0 = rbase % rope_seq;                        // wave-uniform
+      if (p0 + WR <= rope_seq) {
+        // The wave tile's rows are consecutive positions of one sequence.  The table costs 4 bytes per element, twice
+        // what the result does: only the entries of rows p and p + 16 are read, and the angle is advanced from one
+        // 16-row block to the next by their difference (a rotation by 16 positions' worth of angle, the same for
+        // every block; seven fp32 steps).
+        const float* trow = rope + (int64_t)(p0 + lrow) * rope_hd;
+        float4 cs[TN], dl[TN];
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+          const int hc = (hcol + 16 * j) % rope_hd;
+          cs[j] = *reinterpret_cast<const float4*>(trow + hc);
+          const float4 nx = *reinterpret_cast<const float4*>(trow + 16 * rope_hd + hc);
+          dl[j].x = nx.x * cs[j].x + nx.y * cs[j].y;
+          dl[j].y = nx.y * cs[j].x - nx.x * cs[j].y;
+          dl[j].z = nx.z * cs[j].z + nx.w * cs[j].w;
+          dl[j].w = nx.w * cs[j].z - nx.z * cs[j].w;
+        }
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+          for (int j = 0; j < TN; j++) {
+            rotate(i, j, cs[j]);
+            if (i + 1 < TM) {
+              const float4 c = cs[j];
+              cs[j].x = c.x * dl[j].x - c.y * dl[j].y;
+              cs[j].y = c.y * dl[j].x + c.x * dl[j].y;
+              cs[j].z = c.z * dl[j].z - c.w * dl[j].w;
+              cs[j].w = c.w * dl[j].z + c.z * dl[j].w;
+            }
+          }
+      } else {
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+          const float* trow = rope + (int64_t)((rbase + i * 16 + lrow) % rope_seq) * rope_hd;
+#pragma unroll
+          for (int j = 0; j < TN; j++) rotate(i, j, *reinterpret_cast<const float4*>(trow + (hcol + 16 * j) % rope_hd));
+          __builtin_amdgcn_sched_barrier(0);      // one block's table entries in registers at a time
+        }
+      }
     }
 #pragma unroll
     for (int i = 0; i < TM; i++)
@@ -740,12 +795,22 @@ template <int N, typename F> __device__ __forceinline__ void static_for(F&& f) {
 // each, which the swizzle spreads over all 64 banks.
 // GROUPED: the grid holds the tiles of grp.count independent products of one shape, product-major (GemmGroup with
 // sum == 0); otherwise the last argument is an empty placeholder.
-// EPI: 0 = the result [+ R]; 1 / 2 = the SwiGLU epilogues (epilogue_swiglu_t16; R is P0, C is Q0, plus P1 and Q1).
+// EPI: 0 = the result [+ R]; 1 / 2 = the SwiGLU epilogues (epilogue_swiglu_t16; R is P0, C is Q0, plus P1 and Q1);
+// 3 = the result [+ R] with RoPE applied to it (epilogue_bf16_t16<..., ROPE>); 4 = as 0 for matrices of whole tiles and
+// 16-byte accesses (the launcher checks): without the code for ragged tiles the kernel needs no scratch memory.
 struct NoEpi {};
 struct SwigluEpi {
   const uint16_t* P1;
   uint16_t* Q1;
 };
+struct RopeEpi {
+  const float* table;      // [seq, head_dim / 2] of (cos, sin)
+  int seq, head_dim;
+};
+template <int EPI> struct EpiArg { using type = NoEpi; };
+template <> struct EpiArg<1> { using type = SwigluEpi; };
+template <> struct EpiArg<2> { using type = SwigluEpi; };
+template <> struct EpiArg<3> { using type = RopeEpi; };
 template <bool AKM, bool BKM, bool GROUPED = false, int EPI = 0>
 __global__ __launch_bounds__(512) void gemm_bf16_pingpong_kernel(const uint16_t* __restrict__ A,
                                                                   const uint16_t* __restrict__ B, const uint16_t* R,
@@ -753,7 +818,7 @@ __global__ __launch_bounds__(512) void gemm_bf16_pingpong_kernel(const uint16_t*
                                                                   int ldr, int ldc, uint32_t a_bytes, uint32_t b_bytes,
                                                                   int vec_ok,
                                                                   std::conditional_t<GROUPED, GemmGroup, NoGroup> grp,
-                                                                  std::conditional_t<EPI != 0, SwigluEpi, NoEpi> epi = {}) {
+                                                                  typename EpiArg<EPI>::type epi = {}) {
   constexpr int BM = 256, BN = 256, BK = 64;
   constexpr int REGION = 128 * BK * 2;                          // 16 KiB
   // LDS map: A_h of stage s at (2s + h) regions, B_j of stage s at 64 KiB + (2s + j) regions, so that
@@ -998,7 +1063,14 @@ __global__ __launch_bounds__(512) void gemm_bf16_pingpong_kernel(const uint16_t*
   wait_vmcnt<0>();                          // zero-filled loads past the end of K
   slot_end();
 
-  if constexpr (EPI != 0) {
+  if constexpr (EPI == 3) {
+    static_assert(!AKM && !BKM && !GROUPED, "the RoPE epilogue belongs to the k-contiguous single product");
+    epilogue_bf16_t16<8, 4, 0, true>(acc, smem, wave, lane, m0 + wm * 128, n0 + wn * 64, R, C, M, N, ldr, ldc, vec_ok, epi.table,
+                                     epi.seq, epi.head_dim);
+  } else if constexpr (EPI == 4) {
+    epilogue_bf16_t16<8, 4, (BKM ? 96 : 0), false, true>(acc, smem, wave, lane, m0 + wm * 128, n0 + wn * (BKM ? 32 : 64), R, C, M, N,
+                                                         ldr, ldc, vec_ok);
+  } else if constexpr (EPI != 0) {
     static_assert(!AKM && !BKM && !GROUPED, "the SwiGLU epilogues belong to the k-contiguous single product");
     epilogue_swiglu_t16<EPI>(acc, smem, wave, lane, m0 + wm * 128, n0 + wn * 64, R, epi.P1, C, epi.Q1, ldc);
   } else {
@@ -1526,6 +1598,20 @@ static int launch_bf16_pingpong(hipStream_t st, const void* A, const void* B, co
     configured = true;
   }
   const int tiles = ((M + 255) / 256) * ((N + 255) / 256);
+  if (vec_ok && M % 256 == 0 && N % 256 == 0) {
+    static bool configured_full = false;
+    if (!configured_full) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_pingpong_kernel<AKM, BKM, false, 4>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+      if (e != hipSuccess) return emi_fail(EMI_INTERNAL, "emi_gemm: cannot reserve %d bytes of LDS: %s", smem, hipGetErrorString(e));
+      configured_full = true;
+    }
+    hipLaunchKernelGGL((gemm_bf16_pingpong_kernel<AKM, BKM, false, 4>), dim3(tiles), dim3(512), smem, st,
+                       static_cast<const uint16_t*>(A), static_cast<const uint16_t*>(B), static_cast<const uint16_t*>(R),
+                       static_cast<uint16_t*>(C), M, N, K, lda, ldb, ldr, ldc, a_bytes, b_bytes, 1, NoGroup{}, NoEpi{});
+    EMI_CHECK_LAUNCH("emi_gemm");
+    return EMI_OK;
+  }
   hipLaunchKernelGGL((gemm_bf16_pingpong_kernel<AKM, BKM>), dim3(tiles), dim3(512), smem, st, static_cast<const uint16_t*>(A),
                      static_cast<const uint16_t*>(B), static_cast<const uint16_t*>(R), static_cast<uint16_t*>(C), M, N, K,
                      lda, ldb, ldr, ldc, a_bytes, b_bytes, vec_ok, NoGroup{});
@@ -1558,6 +1644,33 @@ static int launch_bf16_swiglu(hipStream_t st, const void* A, const void* B, cons
                      (int)N, (uint32_t)a_bytes, (uint32_t)b_bytes, 1, NoGroup{},
                      SwigluEpi{static_cast<const uint16_t*>(P1), static_cast<uint16_t*>(Q1)});
   EMI_CHECK_LAUNCH("emi_gemm_swiglu");
+  return EMI_OK;
+}
+
+// C = rope(A . B^T): returns -1 when the shape is not one the fused kernel serves (the caller then runs the two passes).
+static int launch_bf16_rope(hipStream_t st, const void* A, const void* B, void* C, const float* table, int64_t M, int64_t N,
+                            int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int64_t seq, int64_t head_dim) {
+  auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+  const int64_t a_bytes = ((M - 1) * lda + K) * 2, b_bytes = ((N - 1) * ldb + K) * 2;
+  // a head is a whole number of the lanes' 4-column quads
+  if (M % 256 || N % 256 || K % 8 || K <= 0 || lda % 8 || ldb % 8 || ldc % 8 || ldc < N || (M / 256) * (N / 256) < 192 ||
+      !al16(A) || !al16(B) || !al16(C) || !al16(table) || a_bytes >= 0x7fffff00LL || b_bytes >= 0x7fffff00LL ||
+      ((M - 1) * ldc + N) * 2 >= 0x7fffff00LL || head_dim % 4 || seq > 0x7fffffff)
+    return -1;
+  constexpr int smem = 2 * 65536;
+  auto kern = gemm_bf16_pingpong_kernel<false, false, false, 3>;
+  static bool configured = false;   // idempotent; a race only repeats the call
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return emi_fail(EMI_INTERNAL, "emi_gemm_rope: cannot reserve %d bytes of LDS: %s", smem, hipGetErrorString(e));
+    configured = true;
+  }
+  const int tiles = (int)((M / 256) * (N / 256));
+  hipLaunchKernelGGL(kern, dim3(tiles), dim3(512), smem, st, static_cast<const uint16_t*>(A), static_cast<const uint16_t*>(B),
+                     static_cast<const uint16_t*>(nullptr), static_cast<uint16_t*>(C), (int)M, (int)N, (int)K, (int)lda, (int)ldb,
+                     (int)ldc, (int)ldc, (uint32_t)a_bytes, (uint32_t)b_bytes, 1, NoGroup{},
+                     RopeEpi{table, (int)seq, (int)head_dim});
+  EMI_CHECK_LAUNCH("emi_gemm_rope");
   return EMI_OK;
 }
 
@@ -1826,6 +1939,25 @@ extern "C" int emi_gemm_swiglu_bwd(emi_stream_t stream, const void* dY, const vo
   const int rc = emi_gemm(stream, dY, W2T, nullptr, workspace, M, N, K, K, K, N, N, 0, 1, dtype);
   if (rc != EMI_OK) return rc;
   return emi_swiglu_bwd(stream, A, B, workspace, dA, dB, M * N, dtype);
+}
+
+extern "C" int emi_rope(emi_stream_t stream, const void* x, const float* table, void* y, int64_t batch, int64_t seq,
+                        int64_t heads, int64_t head_dim, int inverse, int dtype);
+
+extern "C" int emi_gemm_rope(emi_stream_t stream, const void* X, const void* W, void* Y, const float* rope_table, int64_t M,
+                             int64_t N, int64_t K, int64_t seq, int64_t head_dim, int dtype) {
+  EMI_REQUIRE(M >= 0 && N >= 0 && K >= 0 && seq > 0 && head_dim > 0 && head_dim % 2 == 0 && N % head_dim == 0 && M % seq == 0,
+              "emi_gemm_rope: bad shape M=%lld N=%lld K=%lld seq=%lld head_dim=%lld (rows are whole sequences, columns whole heads)",
+              (long long)M, (long long)N, (long long)K, (long long)seq, (long long)head_dim);
+  if (M == 0 || N == 0) return EMI_OK;
+  EMI_REQUIRE(X && W && Y && rope_table, "emi_gemm_rope: null buffer");
+  if (dtype == EMI_BF16) {
+    const int rc = launch_bf16_rope(static_cast<hipStream_t>(stream), X, W, Y, rope_table, M, N, K, K, K, N, seq, head_dim);
+    if (rc >= 0) return rc;
+  }
+  const int rc = emi_gemm(stream, X, W, nullptr, Y, M, N, K, K, K, N, N, 0, 1, dtype);
+  if (rc != EMI_OK) return rc;
+  return emi_rope(stream, Y, rope_table, Y, M / seq, seq, N / head_dim, head_dim, 0, dtype);
 }
 
 extern "C" size_t emi_gemm_grouped_workspace_bytes(int count, int64_t M, int64_t N, int64_t K, int trans_a, int trans_b, int sum,

@@ -60,6 +60,9 @@ SIGNATURES = {
     "emi_attn_bwd_workspace_bytes": (c_size_t, [c_i64, c_i64, c_i64, c_i64]),
     "emi_attn_bwd": (c_int, [c_void_p] * 10 + [c_void_p, c_size_t, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64,
                                                c_float, c_int, c_int]),
+    "emi_attn_bwd_rope": (c_int, [c_void_p] * 11 + [c_void_p, c_size_t, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64,
+                                                    c_float, c_int, c_int]),
+    "emi_gemm_rope": (c_int, [c_void_p] * 5 + [c_i64, c_i64, c_i64, c_i64, c_i64, c_int]),
     "emi_attn_step_workspace_bytes": (c_size_t, [c_i64, c_i64, c_i64, c_i64]),
     "emi_attn_step_fwd": (c_int, [c_void_p] * 7 + [c_size_t] + [c_i64] * 9 + [c_float, c_int]),
     "emi_attn_step_bwd": (c_int, [c_void_p] * 11 + [c_size_t] + [c_i64] * 9 + [c_float, c_int]),

@@ -16,9 +16,7 @@ LAYER_KEYS = ("rms_att_weight", "wq", "wk", "wv", "wo", "rms_ffn_weight", "w1", 
 def layer(x, lw, n_heads, eps=1e-5, theta=10000.0):
     """One decoder layer (test/llama.py:144-233).  x: [B, S, dim]."""
     xb = ops.rmsnorm(x, lw["rms_att_weight"], eps)                 # :145
-    q, k, v = ops.matmul_nt_group(xb, (lw["wq"], lw["wk"], lw["wv"]))      # :149-157, one launch when the shapes agree
-    q, k = ops.rope_pair(q, k, n_heads, theta)                     # :161-168
-    att = ops.attention(q, k, v, n_heads, causal=True)             # :178-209
+    att = ops.attention_block(xb, lw["wq"], lw["wk"], lw["wv"], n_heads, theta)     # :149-209 (RoPE in the epilogues)
     x = ops.matmul_nt(att, lw["wo"], residual=x)                   # :211-215
     xb = ops.rmsnorm(x, lw["rms_ffn_weight"], eps)                 # :219
     return ops.ffn(xb, lw["w1"], lw["w3"], lw["w2"], residual=x)   # :224-233 (SwiGLU in the GEMM epilogues)

@@ -33,6 +33,7 @@ FFI_TARGETS = {
     "swiglu":    ("emi_swiglu_fwd", ("emi_swiglu_bwd",)),
     "ffn":       ("emi_gemm_swiglu_fwd", ("emi_gemm_swiglu_bwd", "emi_gemm_grouped", "emi_gemm")),   # between two emi_gemm
     "attention": ("emi_attn_fwd", ("emi_attn_bwd",)),
+    "attention_block": ("emi_gemm_rope", ("emi_attn_bwd_rope", "emi_gemm_grouped", "emi_gemm")),  # + emi_gemm (v), emi_attn_fwd
     "attention_step": ("emi_attn_step_fwd", ("emi_attn_step_bwd",)),
     "add":       ("emi_add", ()),
     "embedding": ("emi_embedding_fwd", ("emi_embedding_bwd",)),
@@ -630,6 +631,33 @@ def gemm_grouped(As, Bs, trans_a=False, trans_b=False, residuals=None, sum_into_
     return outs[0] if sum_into_one else outs
 
 
+def _group_rule(x, ws, cs, acc):
+    """Reverse rule of (x . w^T for w in ws) for cotangents cs (None = zero) and accumulated cotangents acc of
+    (x, *ws): dX as one summed launch, the dW_i grouped, or deferred into their stacked gradients."""
+    K, Nout = x.shape[-1], ws[0].shape[0]
+    x2 = x.reshape(-1, K)
+    live = [i for i, c in enumerate(cs) if c is not None]
+    c2 = [cs[i].reshape(-1, Nout) for i in live]
+    ax = None if acc[0] is None else acc[0].reshape(-1, K)
+    few = _weight_in_place(x2, ws[0])                              # as in matmul_nt
+    wb = [ws[i] if few else _transpose_shared(ws[i]) for i in live]
+    dx = gemm_grouped(c2, wb, False, not few, None if ax is None else [ax], sum_into_one=True).reshape(x.shape)
+    racc = [acc[1 + i] for i in live]
+    targets = [_grad_target(ws[i], acc[1 + i]) for i in live]
+    if all(t is not None for t in targets):
+        for c, t in zip(c2, targets):
+            _defer_dw(c, x2, t)
+        dws = targets
+    elif any(t is not None for t in targets) or (any(r is None for r in racc) and any(r is not None for r in racc)):
+        dws = [gemm(c, x2, True, False, r, out=t) for c, r, t in zip(c2, racc, targets)]     # (a target implies r is None)
+    else:
+        dws = gemm_grouped(c2, [x2] * len(live), True, False, None if racc[0] is None else racc)
+    out = [dx] + [None] * len(ws)
+    for i, dw in zip(live, dws):
+        out[1 + i] = dw
+    return out
+
+
 def matmul_nt_group(x, ws):
     """(x . w^T for w in ws) for two to four weights of one shape applied to the same activation: q, k, v of
     test/llama.py:149-157 and w1, w3 of :224-227 as one launch.  Reverse mode is one rule for the group: the weight
@@ -643,26 +671,7 @@ def matmul_nt_group(x, ws):
     ys = tuple(y.reshape(*lead, Nout) for y in gemm_grouped([x2] * len(ws), ws, False, True))
 
     def rule(cs, acc):
-        live = [i for i, c in enumerate(cs) if c is not None]
-        c2 = [cs[i].reshape(-1, Nout) for i in live]
-        ax = None if acc[0] is None else acc[0].reshape(-1, K)
-        few = _weight_in_place(x2, ws[0])                              # as in matmul_nt
-        wb = [ws[i] if few else _transpose_shared(ws[i]) for i in live]
-        dx = gemm_grouped(c2, wb, False, not few, None if ax is None else [ax], sum_into_one=True).reshape(x.shape)
-        racc = [acc[1 + i] for i in live]
-        targets = [_grad_target(ws[i], acc[1 + i]) for i in live]
-        if all(t is not None for t in targets):
-            for c, t in zip(c2, targets):
-                _defer_dw(c, x2, t)
-            dws = targets
-        elif any(t is not None for t in targets) or (any(r is None for r in racc) and any(r is not None for r in racc)):
-            dws = [gemm(c, x2, True, False, r, out=t) for c, r, t in zip(c2, racc, targets)]     # (a target implies r is None)
-        else:
-            dws = gemm_grouped(c2, [x2] * len(live), True, False, None if racc[0] is None else racc)
-        out = [dx] + [None] * len(ws)
-        for i, dw in zip(live, dws):
-            out[1 + i] = dw
-        return out
+        return _group_rule(x, ws, cs, acc)
 
     Tape.record((x, *ws), ys, rule)
     tans = _tan(x, *ws)
@@ -866,6 +875,53 @@ def attention(q, k, v, n_heads, scale=None, causal=True, layout="bshd", return_l
                                      B, n_heads, S, d, sb, sh, ss, float(scale), int(causal), _code(q)))
         _set_tan(o, to)
     return (o, lse) if return_lse else o
+
+
+def attention_block(xb, wq, wk, wv, n_heads, theta=10000.0, scale=None, causal=True):
+    """The attention sub-block of test/llama.py:149-209 as one operator: q, k, v = xb Wq^T, xb Wk^T, xb Wv^T;
+    q, k = rope(q), rope(k); softmax attention.  xb: [B, S, dim]; returns [B, S, n_heads*head_dim].  The rotation of
+    q and k is applied in the epilogue of their projections (emi_gemm_rope) and its adjoint where the attention
+    adjoint stores dq and dk (emi_attn_bwd_rope), so that the four passes over [tokens, dim] that rope and its
+    adjoint would make disappear.  Same values and gradients as matmul_nt_group + rope_pair + attention up to the
+    rounding of the unrotated q, k, dq, dk, which here never exist in bf16.  Small shapes, fp32 and forward mode take
+    the three separate operators."""
+    D = wq.shape[0]
+    d = D // max(n_heads, 1)
+    fused = (xb.dim() == 3 and xb.dtype == torch.bfloat16 and Forward._active is None and wq.shape == wk.shape == wv.shape
+             and wq.dtype == wk.dtype == wv.dtype == xb.dtype and wq.dim() == 2 and wq.shape[1] == xb.shape[-1]
+             and d * n_heads == D and d in (64, 128))
+    if fused:
+        T = xb.shape[0] * xb.shape[1]
+        fused = T % 256 == 0 and D % 256 == 0 and (T // 256) * (D // 256) >= 192 and xb.shape[1] >= 128
+    if not fused:
+        q, k, v = matmul_nt_group(xb, (wq, wk, wv))
+        q, k = rope_pair(q, k, n_heads, theta)
+        return attention(q, k, v, n_heads, scale=scale, causal=causal)
+    _dev(xb, wq, wk, wv)
+    B, S, K = xb.shape
+    if scale is None:
+        scale = 1.0 / math.sqrt(d)
+    lib = N.lib()
+    x2 = xb.reshape(-1, K)
+    table = rope_table(S, d, theta, 0, xb.device)
+    q = torch.empty((B, S, D), dtype=xb.dtype, device=xb.device)
+    k = torch.empty_like(q)
+    N.check(lib.emi_gemm_rope(_stream(), _p(x2), _p(wq), _p(q), _p(table), T, D, K, S, d, _code(x2)))
+    N.check(lib.emi_gemm_rope(_stream(), _p(x2), _p(wk), _p(k), _p(table), T, D, K, S, d, _code(x2)))
+    v = gemm(x2, wv, False, True).reshape(B, S, D)
+    o, lse, (_, _, _, sb, sh, ss) = attention_raw(q, k, v, n_heads, scale, causal, "bshd")
+
+    def rule(c, acc):
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        nbytes = lib.emi_attn_bwd_workspace_bytes(B, n_heads, S, d)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
+        N.check(lib.emi_attn_bwd_rope(_stream(), _p(q), _p(k), _p(v), _p(o), _p(lse), _p(c.contiguous()), _p(dq), _p(dk), _p(dv),
+                                      _p(table), _p(ws), nbytes, B, n_heads, S, d, sb, sh, ss, float(scale), int(causal),
+                                      _code(q)))
+        return _group_rule(xb, (wq, wk, wv), (dq, dk, dv), acc)
+
+    Tape.record((xb, wq, wk, wv), o, rule)
+    return o
 
 
 def reshape(x, shape):

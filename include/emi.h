@@ -160,6 +160,15 @@ size_t emi_gemm_swiglu_bwd_workspace_bytes(int64_t M, int64_t N, int64_t K, int 
 int emi_gemm_swiglu_bwd(emi_stream_t stream, const void* dY, const void* W2T, const void* A, const void* B, void* dA, void* dB,
                         void* workspace, size_t workspace_bytes, int64_t M, int64_t N, int64_t K, int dtype);
 
+/* A projection with RoPE in its epilogue (test/llama.py:149-157 followed by :161-168 for q and k):
+ * Y[M, N] = rope(X[M, K] . W[N, K]^T), all contiguous.  Rows are tokens, `seq` consecutive rows one sequence (M a
+ * multiple of seq), columns are heads of `head_dim`; rope_table as emi_rope_table writes it ([seq, head_dim/2] of
+ * (cos, sin)).  The product is rotated in fp32 and rounded once.  bf16 products of whole 256 x 256 tiles (M, N
+ * multiples of 256, at least 192 tiles, head_dim a multiple of 4) run as one launch; anything else as emi_gemm
+ * followed by emi_rope in place. */
+int emi_gemm_rope(emi_stream_t stream, const void* X, const void* W, void* Y, const float* rope_table, int64_t M, int64_t N,
+                  int64_t K, int64_t seq, int64_t head_dim, int dtype);
+
 /* Causal softmax attention, forward.  Replaces the per-head loop of
  * test/llama.py:178-206 with softmax of :13-18 (scale applied after the dot,
  * max-subtracted, fp32 statistics).  Element (b, h, s, i) of q/k/v/o lives at
@@ -191,6 +200,16 @@ int emi_attn_bwd(emi_stream_t stream, const void* q, const void* k, const void* 
                  size_t workspace_bytes, int64_t batch, int64_t heads, int64_t seq,
                  int64_t head_dim, int64_t stride_b, int64_t stride_h, int64_t stride_s,
                  float scale, int causal, int dtype);
+
+/* emi_attn_bwd for q and k that are RoPE outputs (test/llama.py:161-168 in front of :178-206): dq and dk are the
+ * cotangents of the vectors BEFORE the rotation, i.e. emi_attn_bwd followed by emi_rope(inverse) on dq and dk, with
+ * the rotation applied as the MFMA kernels (bf16, head_dim 64 or 128) store their results, in fp32 before the one
+ * rounding.  Other shapes run emi_attn_bwd and two emi_rope passes in place and need contiguous
+ * [batch, seq, heads, head_dim] operands.  rope_table: [seq, head_dim/2] of (cos, sin), 16-byte aligned. */
+int emi_attn_bwd_rope(emi_stream_t stream, const void* q, const void* k, const void* v, const void* o, const float* lse,
+                      const void* d_o, void* dq, void* dk, void* dv, const float* rope_table, void* workspace,
+                      size_t workspace_bytes, int64_t batch, int64_t heads, int64_t seq, int64_t head_dim, int64_t stride_b,
+                      int64_t stride_h, int64_t stride_s, float scale, int causal, int dtype);
 
 /* Attention of the single-token step exactly as the reference writes it
  * (test/llama.py:178-206, softmax :13-18): one query per (batch, head) against

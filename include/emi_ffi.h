@@ -27,6 +27,8 @@
  *  emi_gemm_grouped   A0..An-1, B0..Bn-1 [, R...]      C0..Cn-1 (C0 alone if sum) [, workspace:u8[n]]  count:i64 (2-4), sum:pred, trans_a:pred, trans_b:pred
  *  emi_gemm_swiglu_fwd  x[M,K], w3[N,K], a[M,N]       b[M,N] = x.w3^T, g[M,N] = a*sigmoid(a)*b   -
  *  emi_gemm_swiglu_bwd  dy[M,K], w2t[N,K], a, b[M,N]  da, db[M,N] [, workspace:u8[n]]          -
+ *  emi_gemm_rope      x[M,K], w[N,K], table f32[S,d/2,2]  y[M,N] = rope(x.w^T)             -
+ *  emi_attn_bwd_rope  q, k, v, o, lse, do, table       dq, dk (before RoPE), dv, workspace:u8[n]  scale:f32, causal:pred, bshd:pred
  *  emi_attn_fwd       q, k, v  (rank 4)                o, lse f32[B,h,S] [, unused:u8[n]]     scale:f32, causal:pred, bshd:pred
  *  emi_attn_bwd       q, k, v, o, lse, do              dq, dk, dv, workspace:u8[n]       scale:f32, causal:pred, bshd:pred
  *  emi_attn_step_fwd  q[B,h,d], k, v [B,S,h,d]         o[B,h,d], lse f32[B,h], workspace:u8[n]  scale:f32
@@ -67,6 +69,8 @@ struct XLA_FFI_Error* emi_gemm_ffi(struct XLA_FFI_CallFrame*);
 struct XLA_FFI_Error* emi_gemm_grouped_ffi(struct XLA_FFI_CallFrame*);
 struct XLA_FFI_Error* emi_gemm_swiglu_fwd_ffi(struct XLA_FFI_CallFrame*);
 struct XLA_FFI_Error* emi_gemm_swiglu_bwd_ffi(struct XLA_FFI_CallFrame*);
+struct XLA_FFI_Error* emi_gemm_rope_ffi(struct XLA_FFI_CallFrame*);
+struct XLA_FFI_Error* emi_attn_bwd_rope_ffi(struct XLA_FFI_CallFrame*);
 struct XLA_FFI_Error* emi_attn_fwd_ffi(struct XLA_FFI_CallFrame*);
 struct XLA_FFI_Error* emi_attn_bwd_ffi(struct XLA_FFI_CallFrame*);
 struct XLA_FFI_Error* emi_attn_step_fwd_ffi(struct XLA_FFI_CallFrame*);

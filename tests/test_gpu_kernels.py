@@ -472,3 +472,85 @@ def test_gemm_swiglu_epilogues(ops, T, D, Hd, dt):
     check(y1, L.linear_fwd(h, w2r) + rr, dt, "ffn value")
     for name, u, v in zip(("dx", "dw1", "dw3", "dw2", "dr"), f0(dy), f1(dy)):
         check(v, host(u), dt, "ffn " + name + " against the separate operators", factor=0.5)
+
+
+@pytest.mark.parametrize("B,S,nh,d,D_in,dt", [(16, 256, 24, 128, 256, "bf16"),    # one launch: 16 x 12 tiles of 256 x 256, MFMA adjoint
+                                              (16, 256, 48, 64, 128, "bf16"),     # head_dim 64: a wave strip holds one whole head
+                                              (4, 192, 128, 128, 64, "bf16"),     # one launch; wave tiles that straddle two sequences
+                                              (2, 200, 4, 64, 96, "bf16"),        # ragged: product + rope pass; MFMA adjoint with a partial block
+                                              (2, 40, 3, 16, 48, "f32")])         # generic kernels, rope passes in place
+def test_rope_in_epilogues(ops, B, S, nh, d, D_in, dt):
+    """emi_gemm_rope (test/llama.py:149-168: a projection with the rotation in its epilogue) and emi_attn_bwd_rope (the
+    attention adjoint of :178-206 that hands back the cotangents of q and k before their rotation), through the C ABI and
+    their XLA-FFI handlers, against the oracle; and the `attention_block` operator built on them (value and every
+    gradient) against the oracle's chain."""
+    import ctypes as C
+    import ffi_frames as F
+    from enzyme_ad.jax import _native as N, vjp
+    _say("rope in epilogues", B, S, nh, d, D_in, dt)
+    lib = N.lib()
+    st = torch.cuda.current_stream().cuda_stream
+    rng = np.random.default_rng(B * S + d)
+    D, T = nh * d, B * S
+    code = N.EMI_BF16 if dt == "bf16" else N.EMI_F32
+    x, xr = dev(rng.standard_normal((B, S, D_in)), dt)
+    wq, wqr = dev(rng.standard_normal((D, D_in)) * 0.2, dt)
+    wk, wkr = dev(rng.standard_normal((D, D_in)) * 0.2, dt)
+    wv, wvr = dev(rng.standard_normal((D, D_in)) * 0.2, dt)
+    do, dor = dev(rng.standard_normal((B, S, D)), dt)
+    table = ops.rope_table(S, d, 10000.0, 0)
+    cos, sin = L.rope_angles(S, d)
+    # the projection
+    q = torch.empty((B, S, D), dtype=x.dtype, device="cuda")
+    N.check(lib.emi_gemm_rope(st, x.data_ptr(), wq.data_ptr(), q.data_ptr(), table.data_ptr(), T, D, D_in, S, d, code))
+    qr = L.rope_fwd(L.linear_fwd(xr, wqr).reshape(B, S, nh, d), cos, sin).reshape(B, S, D)
+    check(q, qr, dt, "rope(x wq^T)")
+    k = torch.empty_like(q)
+    N.check(lib.emi_gemm_rope(st, x.data_ptr(), wk.data_ptr(), k.data_ptr(), table.data_ptr(), T, D, D_in, S, d, code))
+    v = ops.gemm(x.reshape(T, D_in), wv, False, True).reshape(B, S, D)
+    # the adjoint: oracle operands are [B, h, S, d]
+    o, lse = ops.attention(q, k, v, nh, return_lse=True)
+    bhsd = lambda t: host(t).reshape(B, S, nh, d).transpose(0, 2, 1, 3)
+    rdq, rdk, rdv = L.attention_bwd(bhsd(q), bhsd(k), bhsd(v), bhsd(do))
+    back = lambda a: a.transpose(0, 2, 1, 3)
+    rdq = L.rope_bwd(back(rdq), cos, sin).reshape(B, S, D)
+    rdk = L.rope_bwd(back(rdk), cos, sin).reshape(B, S, D)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(q), torch.empty_like(q)
+    nb = lib.emi_attn_bwd_workspace_bytes(B, nh, S, d)
+    ws = torch.empty(nb, dtype=torch.uint8, device="cuda")
+    scale = 1.0 / np.sqrt(d)
+    N.check(lib.emi_attn_bwd_rope(st, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr(), do.data_ptr(),
+                                  dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), table.data_ptr(), ws.data_ptr(), nb, B, nh, S, d,
+                                  S * D, d, D, scale, 1, code))
+    check(dq, rdq, dt, "dq before the rotation")
+    check(dk, rdk, dt, "dk before the rotation")
+    check(dv, back(rdv).reshape(B, S, D), dt, "dv")
+    # the handlers
+    xla = F.FakeXla(stream=st)
+    codes = {torch.float32: F.F32, torch.bfloat16: F.BF16, torch.uint8: F.U8}
+    buf = lambda t, shape=None: xla.buffer(codes[t.dtype], list(t.shape if shape is None else shape), t.data_ptr())
+
+    def call(name, args, rets, attrs):
+        fn = getattr(lib, name)
+        fn.restype, fn.argtypes = C.c_void_p, [C.POINTER(F.CallFrame)]
+        cf = xla.frame(args, rets, attrs)
+        assert fn(C.byref(cf)) is None, (name, xla.errors)
+
+    q2 = torch.empty_like(q)
+    call("emi_gemm_rope_ffi", [buf(x, (T, D_in)), buf(wq), buf(table)], [buf(q2, (T, D))], {})
+    dq2, dk2, dv2 = torch.empty_like(q), torch.empty_like(q), torch.empty_like(q)
+    r4 = (B, S, nh, d)
+    call("emi_attn_bwd_rope_ffi", [buf(q, r4), buf(k, r4), buf(v, r4), buf(o, r4), buf(lse), buf(do, r4), buf(table)],
+         [buf(dq2, r4), buf(dk2, r4), buf(dv2, r4), buf(ws)], {"scale": (F.F32, scale), "causal": (F.PRED, 1), "bshd": (F.PRED, 1)})
+    torch.cuda.synchronize()
+    assert torch.equal(q2, q) and torch.equal(dq2, dq) and torch.equal(dk2, dk) and torch.equal(dv2, dv)
+    # the operator
+    y1, f1 = vjp(lambda *a: ops.attention_block(*a, nh), x, wq, wk, wv)
+    ro, _ = L.attention_fwd(bhsd(q), bhsd(k), bhsd(v))
+    check(y1, back(ro).reshape(B, S, D), dt, "attention_block value")
+    rdv = back(rdv).reshape(B, S, D)
+    x2r = xr.reshape(T, D_in)
+    want = {"dx": (rdq @ wqr + rdk @ wkr + rdv @ wvr), "dwq": rdq.reshape(T, D).T @ x2r, "dwk": rdk.reshape(T, D).T @ x2r,
+            "dwv": rdv.reshape(T, D).T @ x2r}
+    for name, w in zip(("dx", "dwq", "dwk", "dwv"), f1(do)):
+        check(w, want[name], dt, "attention_block " + name)

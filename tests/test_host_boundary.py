@@ -144,7 +144,7 @@ def test_ffi_registration_lists_all_targets_for_rocm():
     lib.emi_ffi_target_handler.restype = C.c_void_p
     n = lib.emi_ffi_target_count()
     names = [lib.emi_ffi_target_name(i).decode() for i in range(n)]
-    assert n == 24 and "emi_gemm_swiglu_bwd" in names and "emi_gemm_grouped" in names and "emi_cross_entropy_bwd" in names and "emi_attn_bwd" in names and "emi_attn_step_bwd" in names and "emi_attn_jvp" in names and all(lib.emi_ffi_target_handler(i) for i in range(n))
+    assert n == 26 and "emi_gemm_rope" in names and "emi_attn_bwd_rope" in names and "emi_gemm_swiglu_bwd" in names and "emi_gemm_grouped" in names and "emi_cross_entropy_bwd" in names and "emi_attn_bwd" in names and "emi_attn_step_bwd" in names and "emi_attn_jvp" in names and all(lib.emi_ffi_target_handler(i) for i in range(n))
     from enzyme_ad.jax import ops
     used = {t for fwd, bwd in ops.FFI_TARGETS.values() for t in (fwd,) + tuple(bwd)}
     used |= {t for ts in ops.FFI_TANGENT_TARGETS.values() for t in ts}
