@@ -8,59 +8,127 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "emi_device.h"
 
 namespace emi {
 namespace {
 
-// y[m][n] = sum_k A[m][k] B[n][k] (+ R[m][n]); one wavefront per row n of B, which streams
-// through in 16-byte chunks (eight in flight per lane); A (M x K, a few KB) comes from cache.
-template <typename T, int MT>
+// y[m][n] = sum_k A[m][k] B[n][k] (+ R[m][n]).  A row n of B streams through in batches of UN 16-byte chunks per lane
+// (8 KB of a bf16 row); SPLIT wavefronts of a block share a row (batch b goes to wavefront b mod SPLIT) and meet in LDS,
+// so that a matrix of few long rows still puts thousands of wavefronts' loads in flight.  A wavefront issues the loads
+// of its next batch before it sums the current one.  The loads are unconditional (a chunk past the end of the row is
+// read from the row's start and multiplied by zero): guarded loads made the compiler wait for all earlier ones before
+// each.  A (M x K, a few KB) comes from cache; AREG: one row of A and K of one batch, A stays in registers.
+// STREAM: B is read with streaming loads (a weight that is larger than the caches).
+template <typename T, int MT, int SPLIT, bool AREG, bool STREAM>
 __global__ __launch_bounds__(256) void gemv_nt_kernel(const T* __restrict__ A, const T* __restrict__ B, const T* R, T* C, int M,
                                                       int N, int K, int64_t lda, int64_t ldb, int64_t ldr, int64_t ldc) {
+  using BC = std::conditional_t<STREAM, Chunk<T>, ChunkCached<T>>;
+  using Raw = typename ChunkCached<T>::Raw;
   constexpr int V = ChunkCached<T>::N;
-  const int lane = threadIdx.x & 63;
-  const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (n >= N) return;
-  const T* brow = B + (int64_t)n * ldb;
+  constexpr int UN = 8;                      // 16-byte loads of a row in flight per lane and batch
+  constexpr int BATCH = 64 * V * UN;         // elements of a row per batch
+  static_assert(!AREG || (MT == 1 && SPLIT == 1), "A in registers: one row of A, one batch");
+  __shared__ float red[4][MT];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int sub = wave % SPLIT;
+  const int row = blockIdx.x * (4 / SPLIT) + wave / SPLIT;
+  const bool live = row < N;
+  const int nb = (K + BATCH - 1) / BATCH;
   float acc[MT];
 #pragma unroll
   for (int m = 0; m < MT; m++) acc[m] = 0.f;
-  constexpr int UN = 8;                      // 16-byte loads of the row in flight per lane
-  for (int k0 = lane * V; k0 < K; k0 += 64 * V * UN) {
-    typename ChunkCached<T>::Raw raw[UN];
+  if (live) {
+    const T* brow = B + (int64_t)row * ldb;
+    Raw areg[AREG ? UN : 1];
+    if constexpr (AREG) {
 #pragma unroll
-    for (int u = 0; u < UN; u++) {
-      const int k = k0 + u * 64 * V;
-      if (k < K) raw[u] = ChunkCached<T>::load_raw(brow + k);
+      for (int u = 0; u < UN; u++) {
+        const int k = lane * V + u * 64 * V;
+        areg[u] = ChunkCached<T>::load_raw(A + (k < K ? k : 0));
+      }
     }
+    auto issue = [&](int b, Raw(&r)[UN]) {
 #pragma unroll
-    for (int u = 0; u < UN; u++) {
-      const int k = k0 + u * 64 * V;
-      if (k < K) {
-        float b[V];
-        ChunkCached<T>::unpack(raw[u], b);
+      for (int u = 0; u < UN; u++) {
+        const int k = b * BATCH + lane * V + u * 64 * V;
+        r[u] = BC::load_raw(brow + (k < K ? k : 0));
+      }
+    };
+    // one row of A: its chunks of a batch are requested before the loads of the next batch of B, whose arrival
+    // (the memory counter is in order) the sum would otherwise wait for
+    auto load_a = [&](int b, Raw(&ra)[UN]) {
+#pragma unroll
+      for (int u = 0; u < UN; u++) {
+        const int k = b * BATCH + lane * V + u * 64 * V;
+        ra[u] = ChunkCached<T>::load_raw(A + (k < K ? k : 0));
+      }
+    };
+    constexpr bool APRE = MT == 1 && !AREG;
+    Raw ra[APRE ? UN : 1];
+    auto consume = [&](int b, const Raw(&r)[UN]) {
+#pragma unroll
+      for (int u = 0; u < UN; u++) {
+        const int k = b * BATCH + lane * V + u * 64 * V;
+        const bool ok = k < K;
+        float bv[V];
+        ChunkCached<T>::unpack(r[u], bv);
+#pragma unroll
+        for (int e = 0; e < V; e++) bv[e] = ok ? bv[e] : 0.f;
 #pragma unroll
         for (int m = 0; m < MT; m++) {
           if (m < M) {
             float a[V];
-            ChunkCached<T>::load(A + (int64_t)m * lda + k, a);
+            if constexpr (AREG) ChunkCached<T>::unpack(areg[u], a);
+            else if constexpr (APRE) ChunkCached<T>::unpack(ra[u], a);
+            else ChunkCached<T>::load(A + (int64_t)m * lda + (ok ? k : 0), a);
 #pragma unroll
-            for (int e = 0; e < V; e++) acc[m] = fmaf(a[e], b[e], acc[m]);
+            for (int e = 0; e < V; e++) acc[m] = fmaf(ok ? a[e] : 0.f, bv[e], acc[m]);
           }
         }
       }
+    };
+    Raw r0[UN], r1[UN];
+    int b = sub;
+    if (b < nb) issue(b, r0);
+    while (b < nb) {
+      const int b1 = b + SPLIT;
+      if constexpr (APRE) load_a(b, ra);
+      if (b1 < nb) issue(b1, r1);
+      consume(b, r0);
+      if (b1 >= nb) break;
+      b = b1 + SPLIT;
+      if constexpr (APRE) load_a(b1, ra);
+      if (b < nb) issue(b, r0);
+      consume(b1, r1);
+    }
+#pragma unroll
+    for (int m = 0; m < MT; m++) acc[m] = wave_sum(acc[m]);
+  }
+  if constexpr (SPLIT > 1) {
+    if (lane == 0) {
+#pragma unroll
+      for (int m = 0; m < MT; m++) red[wave][m] = acc[m];
+    }
+    __syncthreads();
+    if (sub == 0 && lane == 0) {
+#pragma unroll
+      for (int m = 0; m < MT; m++) {
+        acc[m] = 0.f;
+#pragma unroll
+        for (int w = 0; w < SPLIT; w++) acc[m] += red[wave + w][m];      // in wavefront order: the result does not depend on timing
+      }
     }
   }
-#pragma unroll
-  for (int m = 0; m < MT; m++) acc[m] = wave_sum(acc[m]);
-  if (lane == 0) {
+  if (live && sub == 0 && lane == 0) {
 #pragma unroll
     for (int m = 0; m < MT; m++)
       if (m < M) {
         float v = acc[m];
-        if (R != nullptr) v += to_f32(R[(int64_t)m * ldr + n]);
-        C[(int64_t)m * ldc + n] = from_f32<T>(v);
+        if (R != nullptr) v += to_f32(R[(int64_t)m * ldr + row]);
+        C[(int64_t)m * ldc + row] = from_f32<T>(v);
       }
   }
 }
@@ -139,44 +207,62 @@ template <typename T, int MT>
 __global__ __launch_bounds__(256) void gemv_nn_bands_kernel(const T* __restrict__ A, const T* __restrict__ B,
                                                             float* __restrict__ part, int M, int N, int K, int64_t lda,
                                                             int64_t ldb, int rows_per_band) {
-  constexpr int V = ChunkCached<T>::N, UN = 16, AR = 256;
-  __shared__ float sa[MT][AR];                                    // A values of the rows being processed
+  using Raw = typename ChunkCached<T>::Raw;
+  constexpr int V = ChunkCached<T>::N, UN = 8, AR = 256;
+  __shared__ float sa[MT][AR + 2 * UN];                           // A values of the rows being processed, then zeros
   const int n = (blockIdx.x * 256 + threadIdx.x) * V;
   const int k_begin = blockIdx.y * rows_per_band;
   const int k_end = k_begin + rows_per_band < K ? k_begin + rows_per_band : K;
   const bool live = n < N;
+  const T* bcol = B + (live ? n : 0);
   float acc[MT][V];
 #pragma unroll
   for (int m = 0; m < MT; m++)
 #pragma unroll
     for (int e = 0; e < V; e++) acc[m][e] = 0.f;
+  // Unconditional loads (a row past the band is read from the band's last row and meets a zero of A): guarded
+  // loads made the compiler wait for all earlier ones before each.  The next UN rows are requested before the
+  // current ones are summed.
+  auto issue = [&](int k0, Raw(&r)[UN]) {
+#pragma unroll
+    for (int u = 0; u < UN; u++) {
+      const int k = k0 + u < k_end ? k0 + u : k_end - 1;
+      r[u] = Chunk<T>::load_raw(bcol + (int64_t)k * ldb);
+    }
+  };
+  auto consume = [&](int j0, const Raw(&r)[UN]) {                 // j0: index of the first row within sa
+#pragma unroll
+    for (int u = 0; u < UN; u++) {
+      float bf[V];
+      ChunkCached<T>::unpack(r[u], bf);
+#pragma unroll
+      for (int m = 0; m < MT; m++)
+        if (m < M) {
+          const float a = sa[m][j0 + u];
+#pragma unroll
+          for (int e = 0; e < V; e++) acc[m][e] = fmaf(a, bf[e], acc[m][e]);
+        }
+    }
+  };
   for (int kc = k_begin; kc < k_end; kc += AR) {
     __syncthreads();
+    for (int j = threadIdx.x; j < AR + 2 * UN; j += 256)
 #pragma unroll
-    for (int m = 0; m < MT; m++)
-      if (m < M) sa[m][threadIdx.x] = kc + (int)threadIdx.x < k_end ? to_f32(A[(int64_t)m * lda + kc + threadIdx.x]) : 0.f;
+      for (int m = 0; m < MT; m++)
+        if (m < M) sa[m][j] = (j < AR && kc + j < k_end) ? to_f32(A[(int64_t)m * lda + kc + j]) : 0.f;
     __syncthreads();
     const int kce = kc + AR < k_end ? kc + AR : k_end;
-    if (live) {
-      for (int k0 = kc; k0 < kce; k0 += UN) {
-        typename ChunkCached<T>::Raw b[UN];
-#pragma unroll
-        for (int u = 0; u < UN; u++)
-          if (k0 + u < kce) b[u] = ChunkCached<T>::load_raw(B + (int64_t)(k0 + u) * ldb + n);
-#pragma unroll
-        for (int u = 0; u < UN; u++)
-          if (k0 + u < kce) {
-            float bf[V];
-            ChunkCached<T>::unpack(b[u], bf);
-#pragma unroll
-            for (int m = 0; m < MT; m++)
-              if (m < M) {
-                const float a = sa[m][k0 + u - kc];
-#pragma unroll
-                for (int e = 0; e < V; e++) acc[m][e] = fmaf(a, bf[e], acc[m][e]);
-              }
-          }
-      }
+    Raw r0[UN], r1[UN];
+    int k0 = kc;
+    issue(k0, r0);
+    while (k0 < kce) {
+      const int k1 = k0 + UN;
+      if (k1 < kce) issue(k1, r1);
+      consume(k0 - kc, r0);
+      if (k1 >= kce) break;
+      k0 = k1 + UN;
+      if (k0 < kce) issue(k0, r0);
+      consume(k1 - kc, r1);
     }
   }
   if (!live) return;
@@ -226,15 +312,15 @@ __global__ __launch_bounds__(256) void gemv_bands_reduce_kernel(const float* __r
 // Number of row bands for the workspace form (the same in the size query and the launch).
 int nn_bands(int64_t N, int64_t K, int V) {
   const int64_t colgroups = (N / V + 255) / 256;
-  int64_t bands = (1024 + colgroups - 1) / colgroups;
-  if (bands > 256) bands = 256;
+  int64_t bands = (256 + colgroups - 1) / colgroups;             // one block per CU measured best (19.5 us against 21.3 and 25.1
+  if (bands > 256) bands = 256;                                  // for two and four on [11008, 4096])
   if (bands > (K + 7) / 8) bands = (K + 7) / 8;
   return (int)(bands < 1 ? 1 : bands);
 }
 
 // C[m][n] = sum_{k < K <= 8} A[k][m] B[k][n] (+ R): a sum of K outer products, one 16-byte
 // store per thread; bound by the write of C.
-template <typename T>
+template <typename T, bool STREAM>
 __global__ __launch_bounds__(256) void outer_tn_kernel(const T* __restrict__ A, const T* __restrict__ B, const T* R, T* C, int M,
                                                        int N, int K, int64_t lda, int64_t ldb, int64_t ldr, int64_t ldc) {
   constexpr int V = ChunkCached<T>::N;
@@ -255,7 +341,8 @@ __global__ __launch_bounds__(256) void outer_tn_kernel(const T* __restrict__ A, 
 #pragma unroll
       for (int e = 0; e < V; e++) acc[e] = fmaf(a, b[e], acc[e]);
     }
-    ChunkCached<T>::store(C + (int64_t)m * ldc + n, acc);
+    if constexpr (STREAM) Chunk<T>::store(C + (int64_t)m * ldc + n, acc);
+    else ChunkCached<T>::store(C + (int64_t)m * ldc + n, acc);
   }
 }
 
@@ -279,7 +366,37 @@ int launch_skinny_t(hipStream_t st, const void* A_, const void* B_, const void* 
   } while (0)
   if (!trans_a && trans_b) {                 // mat-vec: 16-byte chunks along K of both operands
     if (M > 8 || K % V || lda % V || ldb % V || !al16(A) || !al16(B)) return -1;
-    EMI_SKINNY_MT(gemv_nt_kernel, dim3((unsigned)((N + 3) / 4)), 256);
+    // wavefronts per row: enough of them that about 8192 are in flight, at most one per batch of the row
+    constexpr int kBatch = 64 * V * 8;
+    const int64_t nbat = (K + kBatch - 1) / kBatch;
+    int split = 1;
+    while (split < 4 && N * split < 8192 && split < nbat) split *= 2;
+    const dim3 grid((unsigned)((N * split + 3) / 4));
+    const bool stream = (size_t)N * (size_t)K * sizeof(T) > ((size_t)32 << 20);
+#define EMI_GEMV_NT_L(MT, SPLIT, AREG)                                                                                         \
+  do {                                                                                                                         \
+    if (stream)                                                                                                                \
+      hipLaunchKernelGGL((gemv_nt_kernel<T, MT, SPLIT, AREG, true>), grid, dim3(256), 0, st, A, B, R, C, (int)M, (int)N, (int)K, lda, \
+                         ldb, ldr, ldc);                                                                                       \
+    else                                                                                                                       \
+      hipLaunchKernelGGL((gemv_nt_kernel<T, MT, SPLIT, AREG, false>), grid, dim3(256), 0, st, A, B, R, C, (int)M, (int)N, (int)K, lda, \
+                         ldb, ldr, ldc);                                                                                       \
+  } while (0)
+#define EMI_GEMV_NT(MT)                                    \
+  do {                                                     \
+    if (split == 4) EMI_GEMV_NT_L(MT, 4, false);           \
+    else if (split == 2) EMI_GEMV_NT_L(MT, 2, false);      \
+    else EMI_GEMV_NT_L(MT, 1, false);                      \
+  } while (0)
+    // (a variant that kept the vector in registers over several rows per wavefront measured the same: 17.5-18.8 us
+    // for 1 to 11 rows against 17.8 us on [11008, 4096])
+    if (M <= 1 && split == 1 && nbat == 1) EMI_GEMV_NT_L(1, 1, true);
+    else if (M <= 1) EMI_GEMV_NT(1);
+    else if (M <= 2) EMI_GEMV_NT(2);
+    else if (M <= 4) EMI_GEMV_NT(4);
+    else EMI_GEMV_NT(8);
+#undef EMI_GEMV_NT
+#undef EMI_GEMV_NT_L
   } else if (!trans_a && !trans_b) {         // 16-byte chunks along N of B
     if (M > 8 || N % V || ldb % V || !al16(B)) return -1;
     const int bands = nn_bands(N, K, V);
@@ -304,7 +421,10 @@ int launch_skinny_t(hipStream_t st, const void* A_, const void* B_, const void* 
     if (K > 8 || N % V || ldb % V || ldc % V || !al16(B) || !al16(C) || (R != nullptr && (ldr % V || !al16(R)))) return -1;
     const int64_t total = M * (N / V);
     const unsigned grid = (unsigned)((total + 255) / 256 < 16384 ? (total + 255) / 256 : 16384);
-    hipLaunchKernelGGL(outer_tn_kernel<T>, dim3(grid), dim3(256), 0, st, A, B, R, C, (int)M, (int)N, (int)K, lda, ldb, ldr, ldc);
+    if ((size_t)M * (size_t)N * sizeof(T) > ((size_t)32 << 20))       // a result larger than the caches: streaming stores
+      hipLaunchKernelGGL((outer_tn_kernel<T, true>), dim3(grid), dim3(256), 0, st, A, B, R, C, (int)M, (int)N, (int)K, lda, ldb, ldr, ldc);
+    else
+      hipLaunchKernelGGL((outer_tn_kernel<T, false>), dim3(grid), dim3(256), 0, st, A, B, R, C, (int)M, (int)N, (int)K, lda, ldb, ldr, ldc);
   } else {
     return -1;
   }
