@@ -251,8 +251,8 @@ __global__ __launch_bounds__(256) void attn_step_fwd1_kernel(const T* __restrict
       kr[u] = Vec16<T>::zero();
       vr[u] = Vec16<T>::zero();
       if (mine && s < sh.seq_kv) {
-        kr[u] = *reinterpret_cast<const raw_t*>(kbase + (int64_t)s * sh.kv_ss);
-        vr[u] = *reinterpret_cast<const raw_t*>(vbase + (int64_t)s * sh.kv_ss);
+        kr[u] = stream_load(reinterpret_cast<const raw_t*>(kbase + (int64_t)s * sh.kv_ss));     // the cache rows are read once
+        vr[u] = stream_load(reinterpret_cast<const raw_t*>(vbase + (int64_t)s * sh.kv_ss));
       }
     }
     float sc[KPS];
@@ -326,12 +326,23 @@ __global__ __launch_bounds__(64) void attn_step_combine_kernel(const float* __re
       l += p0[i * stride + hd + 1] * w;
     }
     const int cnt = nsplit - c < 64 ? nsplit - c : 64;
-    for (int ii = 0; ii < cnt; ii++) {
-      const float wi = __shfl(w, ii, kWave);
-      const float* row = p0 + (int64_t)(c + ii) * stride;
+    // eight partial rows requested together (a row past the last is the last again, with weight zero): one round
+    // trip to memory per eight splits instead of one per split
+    for (int i0 = 0; i0 < cnt; i0 += 8) {
+      float r[8][4];
 #pragma unroll
-      for (int q = 0; q < 4; q++)
-        if (lane + 64 * q < hd) acc[q] = fmaf(row[lane + 64 * q], wi, acc[q]);
+      for (int u = 0; u < 8; u++) {
+        const float* row = p0 + (int64_t)(c + (i0 + u < cnt ? i0 + u : cnt - 1)) * stride;
+#pragma unroll
+        for (int q = 0; q < 4; q++) r[u][q] = row[lane + 64 * q < hd ? lane + 64 * q : 0];
+      }
+#pragma unroll
+      for (int u = 0; u < 8; u++) {
+        const float ws = __shfl(w, (i0 + u) & 63, kWave);
+        const float wi = i0 + u < cnt ? ws : 0.f;
+#pragma unroll
+        for (int q = 0; q < 4; q++) acc[q] = fmaf(r[u][q], wi, acc[q]);
+      }
     }
   }
   l = wave_sum(l);
