@@ -877,14 +877,15 @@ def attention(q, k, v, n_heads, scale=None, causal=True, layout="bshd", return_l
     return (o, lse) if return_lse else o
 
 
-def attention_block(xb, wq, wk, wv, n_heads, theta=10000.0, scale=None, causal=True):
+def attention_block(xb, wq, wk, wv, n_heads, theta=10000.0, scale=None, causal=True, table=None):
     """The attention sub-block of test/llama.py:149-209 as one operator: q, k, v = xb Wq^T, xb Wk^T, xb Wv^T;
     q, k = rope(q), rope(k); softmax attention.  xb: [B, S, dim]; returns [B, S, n_heads*head_dim].  The rotation of
     q and k is applied in the epilogue of their projections (emi_gemm_rope) and its adjoint where the attention
     adjoint stores dq and dk (emi_attn_bwd_rope), so that the four passes over [tokens, dim] that rope and its
     adjoint would make disappear.  Same values and gradients as matmul_nt_group + rope_pair + attention up to the
     rounding of the unrotated q, k, dq, dk, which here never exist in bf16.  Small shapes, fp32 and forward mode take
-    the three separate operators."""
+    the three separate operators.  `table`: an explicit fp32 (cos, sin) table [S, head_dim/2, 2] instead of the angles
+    of `theta` (what the StableHLO front end recovers from a module's constants)."""
     D = wq.shape[0]
     d = D // max(n_heads, 1)
     fused = (xb.dim() == 3 and xb.dtype == torch.bfloat16 and Forward._active is None and wq.shape == wk.shape == wv.shape
@@ -893,17 +894,24 @@ def attention_block(xb, wq, wk, wv, n_heads, theta=10000.0, scale=None, causal=T
     if fused:
         T = xb.shape[0] * xb.shape[1]
         fused = T % 256 == 0 and D % 256 == 0 and (T // 256) * (D // 256) >= 192 and xb.shape[1] >= 128
+    if table is not None and (table.dtype != torch.float32 or xb.dim() != 3 or tuple(table.shape) != (xb.shape[1], d // 2, 2)
+                              or not table.is_contiguous()):
+        raise ValueError("attention_block: table %s for x %s with %d heads" % (tuple(table.shape), tuple(xb.shape), n_heads))
     if not fused:
         q, k, v = matmul_nt_group(xb, (wq, wk, wv))
-        q, k = rope_pair(q, k, n_heads, theta)
+        if table is None:
+            q, k = rope_pair(q, k, n_heads, theta)
+        else:
+            q, k = rope_rows(q, n_heads, table), rope_rows(k, n_heads, table)
         return attention(q, k, v, n_heads, scale=scale, causal=causal)
-    _dev(xb, wq, wk, wv)
+    _dev(xb, wq, wk, wv, table)
     B, S, K = xb.shape
     if scale is None:
         scale = 1.0 / math.sqrt(d)
     lib = N.lib()
     x2 = xb.reshape(-1, K)
-    table = rope_table(S, d, theta, 0, xb.device)
+    if table is None:
+        table = rope_table(S, d, theta, 0, xb.device)
     q = torch.empty((B, S, D), dtype=xb.dtype, device=xb.device)
     k = torch.empty_like(q)
     N.check(lib.emi_gemm_rope(_stream(), _p(x2), _p(wq), _p(q), _p(table), T, D, K, S, d, _code(x2)))

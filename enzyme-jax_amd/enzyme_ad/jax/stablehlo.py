@@ -942,6 +942,53 @@ def _fold_selects(func):
     return out
 
 
+def _fuse_blocks(run_ops, func):
+    """On the operator list `Executable.run` walks, the two sub-blocks of a decoder layer become the operators that apply
+    their elementwise parts in GEMM and attention epilogues (`ops.ffn`, `ops.attention_block`):
+      linear_group(x; w1, w3) -> swiglu -> linear(g, w2 [, r])               =>  emi.ffn
+      linear_group(x; wq, wk, wv) -> rope_rows(q), rope_rows(k) -> attention  =>  emi.attention_block
+    when every interior value has that one use (test/llama.py:149-209, 224-233).  The printed and the symbolic forms
+    keep the separate clusters."""
+    rets = set(o for op in func.ops if op.name == "return" for o in op.operands)
+    use = {}
+    for op in run_ops:
+        for o in op.operands:
+            use.setdefault(o, []).append(op)
+    producer = {r: op for op in run_ops for r in op.results}
+
+    def only_use(name, user):
+        return name not in rets and len(use.get(name, [])) == 1 and use[name][0] is user
+
+    drop, place = set(), {}
+    for op in run_ops:
+        if op.name == "emi.linear" and producer.get(op.operands[0]) is not None and producer[op.operands[0]].name == "emi.swiglu":
+            sg = producer[op.operands[0]]
+            ga, gb = producer.get(sg.operands[0]), producer.get(sg.operands[1])
+            if (ga is not None and ga is gb and ga.name == "emi.linear_group" and len(ga.results) == 2 and sg.operands[0] != sg.operands[1]
+                    and only_use(sg.results[0], op) and only_use(sg.operands[0], sg) and only_use(sg.operands[1], sg)
+                    and id(ga) not in drop):
+                ia, ib = ga.results.index(sg.operands[0]), ga.results.index(sg.operands[1])
+                operands = [ga.operands[0], ga.operands[1 + ia], ga.operands[1 + ib], op.operands[1]] + list(op.operands[2:])
+                place[id(op)] = Op("emi.ffn", op.results, operands, {}, op.types)
+                drop.update((id(ga), id(sg)))
+        if op.name == "emi.attention" and op.attrs.get("causal") is not None:
+            rq, rk, g = (producer.get(o) for o in op.operands)
+            if (rq is not None and rk is not None and g is not None and rq.name == "emi.rope_rows" and rk.name == "emi.rope_rows"
+                    and rq is not rk and g.name == "emi.linear_group" and len(g.results) == 3 and producer.get(rq.operands[0]) is g
+                    and producer.get(rk.operands[0]) is g and id(g) not in drop
+                    and g.results.index(rq.operands[0]) == 0 and g.results.index(rk.operands[0]) == 1 and op.operands[2] == g.results[2]
+                    and rq.attrs["heads"] == rk.attrs["heads"] == op.attrs["heads"]
+                    and np.array_equal(rq.attrs["table"], rk.attrs["table"])
+                    and only_use(rq.results[0], op) and only_use(rk.results[0], op) and only_use(g.results[0], rq)
+                    and only_use(g.results[1], rk) and only_use(g.results[2], op)):
+                attrs = {"table": rq.attrs["table"], "heads": op.attrs["heads"], "scale": op.attrs["scale"], "causal": op.attrs["causal"]}
+                place[id(op)] = Op("emi.attention_block", op.results, list(g.operands), attrs, op.types)
+                drop.update((id(g), id(rq), id(rk)))
+    if not place:
+        return run_ops
+    return [place.get(id(op), op) for op in run_ops if id(op) not in drop]
+
+
 def _match_rmsnorm(op, d, tb):
     # root: a product of three factors, (w * x) * bcast(ss) or w * (x * bcast(ss)) in any
     # operand order, ss = 1 / sqrt(dot(x, x) / n + eps) or rsqrt(...)
@@ -1580,7 +1627,7 @@ class Executable:
                         self.fused[k] = self.fused.get(k, 0) + v
         self._consts = {}
         for f in self.funcs.values():
-            f.run_ops = _fold_selects(f) if fuse else f.ops
+            f.run_ops = _fuse_blocks(_fold_selects(f), f) if fuse else f.ops
 
     def signature(self, fn="main"):
         f = self._func(fn)
@@ -1694,6 +1741,17 @@ class Executable:
             return list(ops.matmul_nt_group(_packed(xs[0]), [_packed(w) for w in xs[1:]]))
         if n == "emi.select":
             return [ops.select(xs[0], op.attrs["index"])]
+        if n == "emi.ffn":
+            x, w1, w3, w2 = (_packed(t) for t in xs[:4])
+            return [ops.ffn(x, w1, w3, w2, residual=_packed(xs[4]) if len(xs) > 4 else None)]
+        if n == "emi.attention_block":
+            key = (id(op), "table", str(device))
+            table = self._consts.get(key)
+            if table is None:
+                table = self._consts[key] = torch.from_numpy(op.attrs["table"]).to(device).contiguous()
+            x, wq, wk, wv = (_packed(t) for t in xs)
+            return [ops.attention_block(x, wq, wk, wv, op.attrs["heads"], scale=op.attrs["scale"], causal=op.attrs["causal"],
+                                        table=table)]
         if n == "emi.rmsnorm_rows":
             x, w = _packed(xs[0]), _packed(xs[1])
             return [ops.rmsnorm(x, w, op.attrs["eps"])]

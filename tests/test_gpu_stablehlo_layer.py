@@ -56,6 +56,37 @@ def test_layer_text_bf16_head_dim_128_runs_the_mfma_kernels():
     assert exe.fused["attention"] == 1 and exe.fused["rope_rows"] == 2
 
 
+def test_layer_text_at_a_size_the_fused_epilogues_serve():
+    """4096 tokens x dim 3072 (24 heads x 128): the run list's `emi.attention_block` and `emi.ffn` take the kernels with
+    RoPE and SwiGLU in their epilogues.  Value and every gradient against the hand-wired `llama.layer` on the same
+    operands (the same kernels; the angle table comes from the module's constants instead of the device kernel)."""
+    from enzyme_ad.jax import llama, stablehlo, vjp
+    cfg = {"dim": 3072, "hidden_dim": 3072, "n_heads": 24}
+    B, S, dt = 16, 256, "bf16"
+    text, order = llama_layer_text(cfg, B, S, dt)
+    exe = stablehlo.compile_text(text)
+    assert sorted(o.name for o in exe.funcs["main"].run_ops) == sorted(["emi.rmsnorm_rows"] * 2 + ["emi.attention_block", "emi.linear",
+                                                                        "emi.ffn", "return"])
+    rng = np.random.Generator(np.random.PCG64(11))
+    D, H = cfg["dim"], cfg["hidden_dim"]
+    shapes = {"rms_att_weight": (D,), "wq": (D, D), "wk": (D, D), "wv": (D, D), "wo": (D, D), "rms_ffn_weight": (D,), "w1": (H, D),
+              "w2": (D, H), "w3": (H, D)}
+    lw = {k: dev(rng.uniform(0.5, 1.5, shapes[k]) if k.startswith("rms") else rng.standard_normal(shapes[k]) * 0.02, dt)[0]
+          for k in LAYER_ORDER}
+    x = dev(rng.standard_normal((B, S, D)), dt)[0]
+    dy = dev(rng.standard_normal((B, S, D)), dt)[0]
+    y, f_vjp = vjp(lambda x, w: exe.run([x] + [w[k] for k in LAYER_ORDER])[0], x, lw)
+    gx, gw = f_vjp(dy)
+    y0, f0 = vjp(lambda x, w: llama.layer(x, w, cfg["n_heads"]), x, lw)
+    gx0, gw0 = f0(dy)
+    # the two tables differ in the last bit of an fp32 entry here and there, which flips bf16 roundings: agreement to
+    # about one bf16 unit of the largest element is what identical kernels give
+    check(y, host(y0), dt, "y")
+    check(gx, host(gx0), dt, "dx")
+    for k in LAYER_ORDER:
+        check(gw[k], host(gw0[k]), dt, "grad " + k)
+
+
 def test_layer_text_forward_mode_adjoint_identity():
     from enzyme_ad.jax import hlo_call, jvp, vjp
 

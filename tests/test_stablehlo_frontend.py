@@ -91,6 +91,30 @@ def test_llama_text_clusters_are_matched():
     assert plain.fused == {} and names["sqrt"] == 2 * L + 1 and names["exponential"] == 7 * L
 
 
+def test_run_list_joins_the_sub_blocks_of_a_layer():
+    """On the list the executable walks, projections + rotation + attention and projections + SwiGLU + projection of a
+    batched layer are the two operators that apply the elementwise parts in the epilogues; the function's own
+    operator list (what is printed and differentiated symbolically) keeps the separate clusters."""
+    from enzyme_ad.jax import stablehlo as S
+    from enzyme_ad.jax.llama_text import llama_layer_text, llama_model_text
+
+    text, _ = llama_layer_text({"dim": 128, "hidden_dim": 352, "n_heads": 2}, 2, 40, "bf16")
+    f = S.Executable(text).funcs["main"]
+    run = Counter(o.name for o in f.run_ops)
+    assert run == Counter({"emi.rmsnorm_rows": 2, "emi.attention_block": 1, "emi.linear": 1, "emi.ffn": 1, "return": 1})
+    own = Counter(o.name for o in f.ops)
+    assert own["emi.rope_rows"] == 2 and own["emi.swiglu"] == 1 and "emi.ffn" not in own
+    blk = [o for o in f.run_ops if o.name == "emi.attention_block"][0]
+    assert blk.attrs["heads"] == 2 and blk.attrs["causal"] and blk.attrs["table"].shape == (40, 32, 2) and len(blk.operands) == 4
+    ffn = [o for o in f.run_ops if o.name == "emi.ffn"][0]
+    assert len(ffn.operands) == 5                                      # x, w1, w3, w2 and the residual
+    # whole model: every layer's blocks, the weights as in-place selects of the stacked arguments
+    cfg = {"dim": 64, "hidden_dim": 176, "n_layers": 3, "n_heads": 2, "vocab_size": 100}
+    text, _ = llama_model_text(cfg, 2, 24, "bf16", loss="gather")
+    run = Counter(o.name for o in S.Executable(text).funcs["main"].run_ops)
+    assert run["emi.ffn"] == 3 and run["emi.attention_block"] == 3 and run["emi.select"] == 27 and "emi.swiglu" not in run
+
+
 def test_matcher_leaves_clusters_with_outside_uses_alone():
     from enzyme_ad.jax import stablehlo as S
 
