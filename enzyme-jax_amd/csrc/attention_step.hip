@@ -10,6 +10,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "emi_device.h"
 
 namespace emi {
@@ -17,18 +19,6 @@ namespace {
 
 constexpr int kRedFloats = 2048;                 // LDS floats for the reduction over key slots
 constexpr int kKeysPerBlock = 512;
-
-template <typename T, bool VEC> struct Elems {   // VEC: 16-byte chunks; else single elements (any head_dim / alignment)
-  static constexpr int N = VEC ? Chunk<T>::N : 1;
-  static __device__ __forceinline__ void load(const T* p, float (&v)[N]) {
-    if constexpr (VEC) Chunk<T>::load(p, v);
-    else v[0] = to_f32(p[0]);
-  }
-  static __device__ __forceinline__ void store(T* p, const float (&v)[N]) {
-    if constexpr (VEC) Chunk<T>::store(p, v);
-    else p[0] = from_f32<T>(v[0]);
-  }
-};
 
 template <typename T> struct Vec16;              // 16 raw bytes of T, unpacked on use
 template <> struct Vec16<float> {
@@ -40,6 +30,32 @@ template <> struct Vec16<bf16> {
   typedef uint4 type;
   static __device__ __forceinline__ uint4 zero() { return make_uint4(0, 0, 0, 0); }
   static __device__ __forceinline__ void unpack(const uint4& r, float (&v)[8]) { Vec8<bf16>::unpack(r, v); }
+};
+
+template <typename T, bool VEC> struct Elems {   // VEC: 16-byte chunks; else single elements (any head_dim / alignment)
+  static constexpr int N = VEC ? Chunk<T>::N : 1;
+  // the same piece as it sits in memory (a streaming load: the cache rows are read once), unpacked on use
+  typedef std::conditional_t<VEC, typename Vec16<T>::type, T> Raw;
+  static __device__ __forceinline__ Raw load_raw(const T* p) {
+    if constexpr (VEC) return stream_load(reinterpret_cast<const Raw*>(p));
+    else return p[0];
+  }
+  static __device__ __forceinline__ Raw zero_raw() {
+    if constexpr (VEC) return Vec16<T>::zero();
+    else return from_f32<T>(0.f);
+  }
+  static __device__ __forceinline__ void unpack(const Raw& r, float (&v)[N]) {
+    if constexpr (VEC) Vec16<T>::unpack(r, v);
+    else v[0] = to_f32(r);
+  }
+  static __device__ __forceinline__ void load(const T* p, float (&v)[N]) {
+    if constexpr (VEC) Chunk<T>::load(p, v);
+    else v[0] = to_f32(p[0]);
+  }
+  static __device__ __forceinline__ void store(T* p, const float (&v)[N]) {
+    if constexpr (VEC) Chunk<T>::store(p, v);
+    else p[0] = from_f32<T>(v[0]);
+  }
 };
 
 struct StepShape {
@@ -362,7 +378,9 @@ __global__ __launch_bounds__(256) void attn_step_bwd_kernel(const T* __restrict_
                                                             const float* __restrict__ lse, const T* __restrict__ d_o,
                                                             float* __restrict__ part, T* __restrict__ dk, T* __restrict__ dv,
                                                             StepShape sh, float scale) {
-  constexpr int NE = Elems<T, VEC>::N, MAXC = NCH, kUnroll = NCH >= 4 ? 2 : 8 / NCH;
+  using E = Elems<T, VEC>;
+  using Raw = typename E::Raw;
+  constexpr int NE = E::N, MAXC = NCH, U = NCH >= 4 ? 1 : 4 / NCH;      // keys per slot and batch
   __shared__ float red[kRedFloats];
   const int bh = blockIdx.y, b = bh / sh.heads, h = bh % sh.heads;
   const int s0 = blockIdx.x * kKeysPerBlock;
@@ -374,17 +392,22 @@ __global__ __launch_bounds__(256) void attn_step_bwd_kernel(const T* __restrict_
   const float L = lse[bh];
 
   float qf[MAXC][NE], dof[MAXC][NE];
+  int coff[MAXC];                                   // element offset of chunk c inside a row (a lane's idle chunks: 0)
   float delta = 0.f;
 #pragma unroll
-  for (int c = 0; c < MAXC; c++)
+  for (int c = 0; c < MAXC; c++) {
+    coff[c] = c < nch ? (l16 + 16 * c) * NE : 0;
+#pragma unroll
+    for (int e = 0; e < NE; e++) qf[c][e] = dof[c][e] = 0.f;
     if (c < nch) {
       float of[NE];
-      Elems<T, VEC>::load(q + qoff + (l16 + 16 * c) * NE, qf[c]);
-      Elems<T, VEC>::load(d_o + qoff + (l16 + 16 * c) * NE, dof[c]);
-      Elems<T, VEC>::load(o + qoff + (l16 + 16 * c) * NE, of);
+      E::load(q + qoff + coff[c], qf[c]);
+      E::load(d_o + qoff + coff[c], dof[c]);
+      E::load(o + qoff + coff[c], of);
 #pragma unroll
       for (int e = 0; e < NE; e++) delta = fmaf(dof[c][e], of[e], delta);
     }
+  }
   delta = sum16(delta);
 
   float acc[MAXC][NE];
@@ -392,34 +415,37 @@ __global__ __launch_bounds__(256) void attn_step_bwd_kernel(const T* __restrict_
   for (int c = 0; c < MAXC; c++)
 #pragma unroll
     for (int e = 0; e < NE; e++) acc[c][e] = 0.f;
-  for (int sb = s0 + slot; sb < s1; sb += 16 * kUnroll) {
-    float kf[kUnroll][MAXC][NE], vf[kUnroll][MAXC][NE];
+  // Two register sets of U keys: the next batch is requested before the current one is worked on.  The loads are
+  // unconditional (a key past the block's range re-reads the last key and gets weight zero; a lane's idle chunks
+  // re-read chunk 0 against zero q and dO): guarded loads make the compiler wait for all earlier ones before each.
+  auto issue = [&](int sb, Raw(&kr)[U][MAXC], Raw(&vr)[U][MAXC]) {
 #pragma unroll
-    for (int u = 0; u < kUnroll; u++) {
-      const int s = sb + 16 * u;
-      if (s < s1) {
+    for (int u = 0; u < U; u++) {
+      const int s = sb + 16 * u < s1 ? sb + 16 * u : s1 - 1;
+      const int64_t row = kvoff + (int64_t)s * sh.kv_ss;
 #pragma unroll
-        for (int c = 0; c < MAXC; c++)
-          if (c < nch) {
-            Elems<T, VEC>::load(k + kvoff + (int64_t)s * sh.kv_ss + (l16 + 16 * c) * NE, kf[u][c]);
-            Elems<T, VEC>::load(v + kvoff + (int64_t)s * sh.kv_ss + (l16 + 16 * c) * NE, vf[u][c]);
-          }
+      for (int c = 0; c < MAXC; c++) {
+        kr[u][c] = E::load_raw(k + row + coff[c]);
+        vr[u][c] = E::load_raw(v + row + coff[c]);
       }
     }
+  };
+  auto consume = [&](int sb, const Raw(&kr)[U][MAXC], const Raw(&vr)[U][MAXC]) {
 #pragma unroll
-    for (int u = 0; u < kUnroll; u++) {
+    for (int u = 0; u < U; u++) {
       const int s = sb + 16 * u;
+      float kf[MAXC][NE];
       float dot = 0.f, dp = 0.f;
-      if (s < s1) {
 #pragma unroll
-        for (int c = 0; c < MAXC; c++)
-          if (c < nch) {
+      for (int c = 0; c < MAXC; c++) {
+        float vf[NE];
+        E::unpack(kr[u][c], kf[c]);
+        E::unpack(vr[u][c], vf);
 #pragma unroll
-            for (int e = 0; e < NE; e++) {
-              dot = fmaf(qf[c][e], kf[u][c][e], dot);
-              dp = fmaf(dof[c][e], vf[u][c][e], dp);
-            }
-          }
+        for (int e = 0; e < NE; e++) {
+          dot = fmaf(qf[c][e], kf[c][e], dot);
+          dp = fmaf(dof[c][e], vf[e], dp);
+        }
       }
       dot = sum16(dot);
       dp = sum16(dp);
@@ -433,15 +459,29 @@ __global__ __launch_bounds__(256) void attn_step_bwd_kernel(const T* __restrict_
           if (c < nch) {
             float t[NE];
 #pragma unroll
-            for (int e = 0; e < NE; e++) acc[c][e] = fmaf(ds, kf[u][c][e], acc[c][e]);
+            for (int e = 0; e < NE; e++) acc[c][e] = fmaf(ds, kf[c][e], acc[c][e]);
 #pragma unroll
             for (int e = 0; e < NE; e++) t[e] = ds * qf[c][e];
-            Elems<T, VEC>::store(dkrow + (l16 + 16 * c) * NE, t);
+            E::store(dkrow + coff[c], t);
 #pragma unroll
             for (int e = 0; e < NE; e++) t[e] = p * dof[c][e];
-            Elems<T, VEC>::store(dvrow + (l16 + 16 * c) * NE, t);
+            E::store(dvrow + coff[c], t);
           }
       }
+    }
+  };
+  {
+    Raw k0[U][MAXC], v0[U][MAXC], k1[U][MAXC], v1[U][MAXC];
+    int sb = s0 + slot;
+    issue(sb, k0, v0);
+    while (sb < s1) {
+      const int sb1 = sb + 16 * U;
+      if (sb1 < s1) issue(sb1, k1, v1);
+      consume(sb, k0, v0);
+      if (sb1 >= s1) break;
+      sb = sb1 + 16 * U;
+      if (sb < s1) issue(sb, k0, v0);
+      consume(sb1, k1, v1);
     }
   }
   reduce_keys<MAXC, NE>(acc, nch, red);
@@ -481,7 +521,9 @@ __global__ __launch_bounds__(256) void attn_step_jvp_kernel(const T* __restrict_
                                                             const T* __restrict__ tq, const T* __restrict__ tk,
                                                             const T* __restrict__ tv, float* __restrict__ part, StepShape sh,
                                                             float scale) {
-  constexpr int NE = Elems<T, VEC>::N, MAXC = NCH, kUnroll = NCH >= 4 ? 1 : 4 / NCH;
+  using E = Elems<T, VEC>;
+  using Raw = typename E::Raw;
+  constexpr int NE = E::N, MAXC = NCH, U = NCH >= 2 ? 1 : 2;            // keys per slot and batch (four streams)
   __shared__ float red[kRedFloats];
   __shared__ float scratch[4];
   const int bh = blockIdx.y, b = bh / sh.heads, h = bh % sh.heads;
@@ -494,13 +536,15 @@ __global__ __launch_bounds__(256) void attn_step_jvp_kernel(const T* __restrict_
   const float L = lse[bh];
 
   float qf[MAXC][NE], tqf[MAXC][NE];
+  int coff[MAXC];
 #pragma unroll
   for (int c = 0; c < MAXC; c++) {
+    coff[c] = c < nch ? (l16 + 16 * c) * NE : 0;
 #pragma unroll
     for (int e = 0; e < NE; e++) qf[c][e] = tqf[c][e] = 0.f;
     if (c < nch) {
-      Elems<T, VEC>::load(q + qoff + (l16 + 16 * c) * NE, qf[c]);
-      if (tq) Elems<T, VEC>::load(tq + qoff + (l16 + 16 * c) * NE, tqf[c]);
+      E::load(q + qoff + coff[c], qf[c]);
+      if (tq) E::load(tq + qoff + coff[c], tqf[c]);
     }
   }
   float acc[MAXC][NE];
@@ -509,36 +553,42 @@ __global__ __launch_bounds__(256) void attn_step_jvp_kernel(const T* __restrict_
 #pragma unroll
     for (int e = 0; e < NE; e++) acc[c][e] = 0.f;
   float mu = 0.f;
-  for (int sb = s0 + slot; sb < s1; sb += 16 * kUnroll) {
-    float kf[kUnroll][MAXC][NE], vf[kUnroll][MAXC][NE], tkf[kUnroll][MAXC][NE], tvf[kUnroll][MAXC][NE];
+  // as in the adjoint kernel: two register sets, unconditional loads (clamped key, idle chunks against zero q, tq);
+  // a null tangent cache is a block-uniform branch around its loads
+  struct Set {
+    Raw k[U][MAXC], v[U][MAXC], tk[U][MAXC], tv[U][MAXC];
+  };
+  auto issue = [&](int sb, Set& r) {
 #pragma unroll
-    for (int u = 0; u < kUnroll; u++) {
-      const int s = sb + 16 * u;
+    for (int u = 0; u < U; u++) {
+      const int s = sb + 16 * u < s1 ? sb + 16 * u : s1 - 1;
+      const int64_t row = kvoff + (int64_t)s * sh.kv_ss;
 #pragma unroll
       for (int c = 0; c < MAXC; c++) {
-#pragma unroll
-        for (int e = 0; e < NE; e++) kf[u][c][e] = vf[u][c][e] = tkf[u][c][e] = tvf[u][c][e] = 0.f;
-        if (s < s1 && c < nch) {
-          const int64_t off = kvoff + (int64_t)s * sh.kv_ss + (l16 + 16 * c) * NE;
-          Elems<T, VEC>::load(k + off, kf[u][c]);
-          Elems<T, VEC>::load(v + off, vf[u][c]);
-          if (tk) Elems<T, VEC>::load(tk + off, tkf[u][c]);
-          if (tv) Elems<T, VEC>::load(tv + off, tvf[u][c]);
-        }
+        r.k[u][c] = E::load_raw(k + row + coff[c]);
+        r.v[u][c] = E::load_raw(v + row + coff[c]);
+        r.tk[u][c] = tk ? E::load_raw(tk + row + coff[c]) : E::zero_raw();
+        r.tv[u][c] = tv ? E::load_raw(tv + row + coff[c]) : E::zero_raw();
       }
     }
+  };
+  auto consume = [&](int sb, const Set& r) {
 #pragma unroll
-    for (int u = 0; u < kUnroll; u++) {
+    for (int u = 0; u < U; u++) {
       const int s = sb + 16 * u;
       float dot = 0.f, tdot = 0.f;
 #pragma unroll
-      for (int c = 0; c < MAXC; c++)
+      for (int c = 0; c < MAXC; c++) {
+        float kf[NE], tkf[NE];
+        E::unpack(r.k[u][c], kf);
+        E::unpack(r.tk[u][c], tkf);
 #pragma unroll
         for (int e = 0; e < NE; e++) {
-          dot = fmaf(qf[c][e], kf[u][c][e], dot);
-          tdot = fmaf(tqf[c][e], kf[u][c][e], tdot);
-          tdot = fmaf(qf[c][e], tkf[u][c][e], tdot);
+          dot = fmaf(qf[c][e], kf[e], dot);
+          tdot = fmaf(tqf[c][e], kf[e], tdot);
+          tdot = fmaf(qf[c][e], tkf[e], tdot);
         }
+      }
       dot = sum16(dot);
       tdot = sum16(tdot);
       if (s < s1) {
@@ -547,9 +597,28 @@ __global__ __launch_bounds__(256) void attn_step_jvp_kernel(const T* __restrict_
         if (l16 == 0) mu += w;
 #pragma unroll
         for (int c = 0; c < MAXC; c++)
+          if (c < nch) {
+            float vf[NE], tvf[NE];
+            E::unpack(r.v[u][c], vf);
+            E::unpack(r.tv[u][c], tvf);
 #pragma unroll
-          for (int e = 0; e < NE; e++) acc[c][e] = fmaf(w, vf[u][c][e], fmaf(p, tvf[u][c][e], acc[c][e]));
+            for (int e = 0; e < NE; e++) acc[c][e] = fmaf(w, vf[e], fmaf(p, tvf[e], acc[c][e]));
+          }
       }
+    }
+  };
+  {
+    Set r0, r1;
+    int sb = s0 + slot;
+    issue(sb, r0);
+    while (sb < s1) {
+      const int sb1 = sb + 16 * U;
+      if (sb1 < s1) issue(sb1, r1);
+      consume(sb, r0);
+      if (sb1 >= s1) break;
+      sb = sb1 + 16 * U;
+      if (sb < s1) issue(sb, r0);
+      consume(sb1, r1);
     }
   }
   mu = block_sum(mu, scratch);
