@@ -891,9 +891,13 @@ def attention_block(xb, wq, wk, wv, n_heads, theta=10000.0, scale=None, causal=T
     fused = (xb.dim() == 3 and xb.dtype == torch.bfloat16 and Forward._active is None and wq.shape == wk.shape == wv.shape
              and wq.dtype == wk.dtype == wv.dtype == xb.dtype and wq.dim() == 2 and wq.shape[1] == xb.shape[-1]
              and d * n_heads == D and d in (64, 128))
+    proj_fused = False
     if fused:
         T = xb.shape[0] * xb.shape[1]
-        fused = T % 256 == 0 and D % 256 == 0 and (T // 256) * (D // 256) >= 192 and xb.shape[1] >= 128
+        proj_fused = T % 256 == 0 and D % 256 == 0 and (T // 256) * (D // 256) >= 192 and xb.shape[1] >= 128
+        # smaller projections (one grouped launch, then q and k rotated in place by one launch) still take the
+        # attention adjoint that turns dq and dk back as it stores them
+        fused = proj_fused or (xb.shape[1] >= 128 and D % 8 == 0 and xb.shape[-1] % 8 == 0)
     if table is not None and (table.dtype != torch.float32 or xb.dim() != 3 or tuple(table.shape) != (xb.shape[1], d // 2, 2)
                               or not table.is_contiguous()):
         raise ValueError("attention_block: table %s for x %s with %d heads" % (tuple(table.shape), tuple(xb.shape), n_heads))
@@ -912,11 +916,19 @@ def attention_block(xb, wq, wk, wv, n_heads, theta=10000.0, scale=None, causal=T
     x2 = xb.reshape(-1, K)
     if table is None:
         table = rope_table(S, d, theta, 0, xb.device)
-    q = torch.empty((B, S, D), dtype=xb.dtype, device=xb.device)
-    k = torch.empty_like(q)
-    N.check(lib.emi_gemm_rope(_stream(), _p(x2), _p(wq), _p(q), _p(table), T, D, K, S, d, _code(x2)))
-    N.check(lib.emi_gemm_rope(_stream(), _p(x2), _p(wk), _p(k), _p(table), T, D, K, S, d, _code(x2)))
-    v = gemm(x2, wv, False, True).reshape(B, S, D)
+    if proj_fused:
+        q = torch.empty((B, S, D), dtype=xb.dtype, device=xb.device)
+        k = torch.empty_like(q)
+        N.check(lib.emi_gemm_rope(_stream(), _p(x2), _p(wq), _p(q), _p(table), T, D, K, S, d, _code(x2)))
+        N.check(lib.emi_gemm_rope(_stream(), _p(x2), _p(wk), _p(k), _p(table), T, D, K, S, d, _code(x2)))
+        v = gemm(x2, wv, False, True).reshape(B, S, D)
+    else:
+        q, k, v = (t.reshape(B, S, D) for t in gemm_grouped([x2] * 3, [wq, wk, wv], False, True))
+        if _adjacent(q, k):
+            N.check(lib.emi_rope(_stream(), _p(q), _p(table), _p(q), 2 * B, S, n_heads, d, 0, _code(q)))
+        else:
+            for t in (q, k):
+                N.check(lib.emi_rope(_stream(), _p(t), _p(table), _p(t), B, S, n_heads, d, 0, _code(t)))
     o, lse, (_, _, _, sb, sh, ss) = attention_raw(q, k, v, n_heads, scale, causal, "bshd")
 
     def rule(c, acc):
