@@ -877,6 +877,85 @@ def attention(q, k, v, n_heads, scale=None, causal=True, layout="bshd", return_l
     return (o, lse) if return_lse else o
 
 
+def gemm_rope(x2, w, table):
+    """rope(x2 . w^T) as the custom call `emi_gemm_rope` computes it: x2 [T, K] holds whole sequences of
+    S = table.shape[0] positions, w [n_heads*head_dim, K], table fp32 [S, head_dim/2, 2] (test/llama.py:149-168).
+    Reverse: the cotangent is turned back by the angle, then the DotGeneral rule (dX = c W, dW = c^T X)."""
+    _dev(x2, w, table)
+    _same_dtype(x2, w)
+    if x2.dim() != 2 or w.dim() != 2 or table.dim() != 3 or table.dtype != torch.float32 or table.shape[2] != 2 or not table.is_contiguous():
+        raise ValueError("gemm_rope: x %s, w %s, table %s" % (tuple(x2.shape), tuple(w.shape), tuple(table.shape)))
+    T_, K = x2.shape
+    D, S, d = w.shape[0], table.shape[0], 2 * table.shape[1]
+    if w.shape[1] != K or T_ % S or D % d:
+        raise ValueError("gemm_rope: x %s, w %s, table %s" % (tuple(x2.shape), tuple(w.shape), tuple(table.shape)))
+    lib = N.lib()
+    x2 = x2.contiguous()
+    y = torch.empty((T_, D), dtype=x2.dtype, device=x2.device)
+    N.check(lib.emi_gemm_rope(_stream(), _p(x2), _p(w), _p(y), _p(table), T_, D, K, S, d, _code(x2)))
+
+    def turn(c, inverse):
+        g = torch.empty_like(c)
+        N.check(lib.emi_rope(_stream(), _p(c), _p(table), _p(g), T_ // S, S, D // d, d, int(inverse), _code(c)))
+        return g
+
+    def rule(c, acc):
+        return _group_rule(x2, (w,), (turn(c.contiguous(), True),), acc[:2]) + [None]
+
+    Tape.record((x2, w, table), y, rule)
+    tans = _tan(x2, w)
+    if tans is not None and any(t is not None for t in tans):          # linear in x and in w
+        t = None
+        if tans[0] is not None:
+            t = gemm(tans[0], w, False, True, t)
+        if tans[1] is not None:
+            t = gemm(x2, tans[1], False, True, t)
+        _set_tan(y, turn(t, False))
+    return y
+
+
+def gemm_swiglu(x2, w3, a):
+    """(b, g) = (x2 . w3^T, a * sigmoid(a) * b) as the custom call `emi_gemm_swiglu_fwd` computes them (test/llama.py:
+    224-231 with a = x2 . w1^T given).  Reverse: (da, db) from the cotangent of g through the SwiGLU adjoint, then the
+    DotGeneral rule on the total cotangent of b."""
+    _dev(x2, w3, a)
+    _same_dtype(x2, w3, a)
+    if x2.dim() != 2 or w3.dim() != 2 or w3.shape[1] != x2.shape[1] or tuple(a.shape) != (x2.shape[0], w3.shape[0]):
+        raise ValueError("gemm_swiglu: x %s, w3 %s, a %s" % (tuple(x2.shape), tuple(w3.shape), tuple(a.shape)))
+    lib = N.lib()
+    x2, a = x2.contiguous(), a.contiguous()
+    T_, K = x2.shape
+    Hn = w3.shape[0]
+    b, g = torch.empty_like(a), torch.empty_like(a)
+    N.check(lib.emi_gemm_swiglu_fwd(_stream(), _p(x2), _p(w3), _p(a), _p(b), _p(g), T_, Hn, K, _code(x2)))
+
+    def rule(cs, acc):
+        cb, cg = cs
+        da = None
+        if cg is not None:
+            da, db = torch.empty_like(a), torch.empty_like(a)
+            N.check(lib.emi_swiglu_bwd(_stream(), _p(a), _p(b), _p(cg.contiguous()), _p(da), _p(db), a.numel(), _code(a)))
+            cb = db if cb is None else _quiet(lambda: add(cb, db))
+        out = _group_rule(x2, (w3,), (cb,), acc[:2]) if cb is not None else [None, None]
+        return out + [None if da is None else _accumulate(acc[2], da)]
+
+    Tape.record((x2, w3, a), (b, g), rule)
+    tans = _tan(x2, w3, a)
+    if tans is not None and any(t is not None for t in tans):
+        tx, tw, ta = tans
+        tb = None
+        if tx is not None:
+            tb = gemm(tx, w3, False, True, tb)
+        if tw is not None:
+            tb = gemm(x2, tw, False, True, tb)
+        if tb is not None:
+            _set_tan(b, tb)
+        tg = torch.empty_like(a)
+        N.check(lib.emi_swiglu_jvp(_stream(), _p(a), _p(b), _p(ta), _p(tb), _p(tg), a.numel(), _code(a)))
+        _set_tan(g, tg)
+    return b, g
+
+
 def attention_block(xb, wq, wk, wv, n_heads, theta=10000.0, scale=None, causal=True, table=None):
     """The attention sub-block of test/llama.py:149-209 as one operator: q, k, v = xb Wq^T, xb Wk^T, xb Wv^T;
     q, k = rope(q), rope(k); softmax attention.  xb: [B, S, dim]; returns [B, S, n_heads*head_dim].  The rotation of

@@ -1825,6 +1825,10 @@ def _custom_call_impl(self, op, xs):
         return ([out] if sum_ else list(out)) + [None] * (len(op.results) - (1 if sum_ else n_))
     if target == "emi_add":
         return [ops.add(_packed(xs[0]), _packed(xs[1]))]
+    if target == "emi_gemm_rope":
+        return [ops.gemm_rope(_packed(xs[0]), _packed(xs[1]), _packed(xs[2]))]
+    if target == "emi_gemm_swiglu_fwd":
+        return list(ops.gemm_swiglu(_packed(xs[0]), _packed(xs[1]), _packed(xs[2])))
     if target == "emi_rope":
         x, table = _packed(xs[0]), _packed(xs[1])
         if x.dim() != 4 or tuple(table.shape) != (x.shape[1], x.shape[3] // 2, 2):
@@ -1879,6 +1883,25 @@ def _custom_call_impl(self, op, xs):
         N.check(lib.emi_attn_step_jvp(st, P(q), P(k), P(v), P(o), P(lse), P(tq), P(tk), P(tv), P(to), P(ws), nbytes, 1, h, S, d,
                                       h * d, d, S * h * d, d, h * d, float(cfg["scale"]), ops._code(q)))
         return [to, None][:len(op.results)]
+    if target == "emi_gemm_swiglu_bwd":
+        dy, w2t, a, b_ = (_packed(t) for t in xs)
+        T_, K, Hn = dy.shape[0], dy.shape[1], w2t.shape[0]
+        da, db = torch.empty_like(a), torch.empty_like(a)
+        nbytes = lib.emi_gemm_swiglu_bwd_workspace_bytes(T_, Hn, K, ops._code(dy))
+        ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=dy.device)
+        N.check(lib.emi_gemm_swiglu_bwd(st, P(dy), P(w2t), P(a), P(b_), P(da), P(db), P(ws), nbytes, T_, Hn, K, ops._code(dy)))
+        return [da, db, None][:len(op.results)]
+    if target == "emi_attn_bwd_rope":
+        bshd = bool(cfg.get("bshd", False))
+        q, k, v, o, lse, do, table = (_packed(t) for t in xs)
+        B_, S_, h, d = (q.shape if bshd else (q.shape[0], q.shape[2], q.shape[1], q.shape[3]))
+        sb, sh, ss = (S_ * h * d, d, h * d) if bshd else (h * S_ * d, S_ * d, d)
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        nbytes = lib.emi_attn_bwd_workspace_bytes(B_, h, S_, d)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
+        N.check(lib.emi_attn_bwd_rope(st, P(q), P(k), P(v), P(o), P(lse), P(do), P(dq), P(dk), P(dv), P(table), P(ws), nbytes, B_, h,
+                                      S_, d, sb, sh, ss, float(cfg["scale"]), int(bool(cfg.get("causal", True))), ops._code(q)))
+        return [dq, dk, dv, None][:len(op.results)]
     if target in ("emi_attn_bwd", "emi_attn_jvp"):
         bshd = bool(cfg.get("bshd", False))
         q = _packed(xs[0])

@@ -76,15 +76,17 @@ def _step_workspace(heads, rows, head_dim):
     return heads * ((rows + 511) // 512) * (head_dim + 2) * 4          # emi_attn_step_workspace_bytes for one sequence
 
 
-def lower_fused(func):
+def lower_fused(func, blocks=True):
     """A copy of `func` with the matcher's fused operators written as custom calls to this
     library's FFI targets (api_version 4; scalars in backend_config), wrapped in the reshapes
-    that bring the operands to the handlers' layouts."""
+    that bring the operands to the handlers' layouts.  blocks: the two sub-blocks of a decoder layer are written
+    with the targets that apply RoPE and the SwiGLU in GEMM epilogues (`emi_gemm_rope`, `emi_gemm_swiglu_fwd`)."""
     if not any(op.name.startswith("emi.") for op in func.ops):
         return func
+    from .stablehlo import _fuse_blocks
     b = _Builder(func, "emi")
     T = b.types
-    for op in func.ops:
+    for op in (_fuse_blocks(func.ops, func) if blocks else func.ops):
         n = op.name
         ty = op.types[0] if op.types else None
         if n == "emi.rmsnorm":
@@ -117,6 +119,36 @@ def lower_fused(func):
                                  [TensorType((rows, Nn), ty.dtype)] * len(ws))
             for r_, c2, t_ in zip(op.results, outs, op.types):
                 b.ops.append(Op("reshape", [r_], [c2], {}, [t_]))
+        elif n == "emi.ffn":
+            # a = x w1^T ; (b, g) = (x w3^T, swiglu(a, b)) in one launch ; y = g w2^T [+ r]   (test/llama.py:224-233)
+            x, w1, w3, w2 = op.operands[:4]
+            K, Hn = T[x].shape[-1], T[w1].shape[0]
+            rows = int(np.prod(T[x].shape[:-1])) if len(T[x].shape) > 1 else 1
+            x2 = b.reshape(x, (rows, K))
+            hty = TensorType((rows, Hn), ty.dtype)
+            a, = b.custom_call("emi_gemm", [x2, w1], {"trans_a": False, "trans_b": True}, [hty])
+            _, g = b.custom_call("emi_gemm_swiglu_fwd", [x2, w3, a], {}, [hty, hty])
+            Nn = T[w2].shape[0]
+            y2, = b.custom_call("emi_gemm", [g, w2] + [b.reshape(r_, (rows, Nn)) for r_ in op.operands[4:]],
+                                {"trans_a": False, "trans_b": True}, [TensorType((rows, Nn), ty.dtype)])
+            b.ops.append(Op("reshape", op.results, [y2], {}, op.types))
+        elif n == "emi.attention_block":
+            # q, k = rope(x wq^T), rope(x wk^T) stored rotated by the projections ; v = x wv^T ; attention   (:149-209)
+            x, wq, wk, wv = op.operands
+            B_, S_, K = T[x].shape
+            h = op.attrs["heads"]
+            D_ = T[wq].shape[0]
+            x2 = b.reshape(x, (B_ * S_, K))
+            tab = b.emit("constant", [], {"value": np.asarray(op.attrs["table"], dtype=np.float32)},
+                         TensorType(op.attrs["table"].shape, "f32"))
+            pty = TensorType((B_ * S_, D_), ty.dtype)
+            q2, = b.custom_call("emi_gemm_rope", [x2, wq, tab], {}, [pty])
+            k2, = b.custom_call("emi_gemm_rope", [x2, wk, tab], {}, [pty])
+            v2, = b.custom_call("emi_gemm", [x2, wv], {"trans_a": False, "trans_b": True}, [pty])
+            q4, k4, v4 = (b.reshape(o_, (B_, S_, h, D_ // h)) for o_ in (q2, k2, v2))
+            o4, _ = b.custom_call("emi_attn_fwd", [q4, k4, v4], {"scale": op.attrs["scale"], "causal": bool(op.attrs["causal"]), "bshd": True},
+                                  [T[q4], TensorType((B_, h, S_), "f32")])
+            b.ops.append(Op("reshape", op.results, [o4], {}, op.types))
         elif n == "emi.rmsnorm_rows":
             b.ops.append(Op("custom_call", op.results, list(op.operands), {"target": "emi_rmsnorm_fwd", "config": {"eps": op.attrs["eps"]}},
                             op.types))
@@ -196,6 +228,14 @@ def reverse_function(func, name=None, arg_active=None, ret_active=None):
     func = lower_fused(func)
     b = _Builder(func, "r")
     T = b.types
+    # what the joint rules of the fused targets look at: who produced a value, how often it is used, and which
+    # cotangents already are those of the vector before its rotation
+    b.producer = {r_: op_ for op_ in func.ops for r_ in op_.results}
+    b.uses = {}
+    for op_ in func.ops:
+        for o_ in op_.operands:
+            b.uses[o_] = b.uses.get(o_, 0) + 1
+    b.unrotated = set()
     ret = [op for op in func.ops if op.name == "return"]
     if len(ret) != 1:
         raise ValueError("reverse mode needs exactly one return")
@@ -307,7 +347,10 @@ def reverse_function(func, name=None, arg_active=None, ret_active=None):
         elif n == "convert":
             accum(xs[0], c if T[xs[0]].dtype == T[c].dtype else b.emit("convert", [c], {}, T[xs[0]]))
         elif n == "reshape":
-            accum(xs[0], b.reshape(c, T[xs[0]].shape))
+            g = b.reshape(c, T[xs[0]].shape)
+            if c in b.unrotated:
+                b.unrotated.add(g)
+            accum(xs[0], g)
         elif n == "transpose":
             perm = list(op.attrs["perm"])
             accum(xs[0], b.emit("transpose", [c], {"perm": [perm.index(i) for i in range(len(perm))]}, T[xs[0]]))
@@ -402,7 +445,7 @@ def forward_function(func, name=None, arg_active=None):
     `enzyme_dup` results (primitives.py:1160-1203).  Every operator is followed by the
     operators of its tangent; matched clusters call the tangent targets (`emi_rmsnorm_jvp`,
     `emi_swiglu_jvp`, `emi_attn_step_jvp`, `emi_rope` on the tangent)."""
-    func = lower_fused(func)
+    func = lower_fused(func, blocks=False)
     b = _Builder(func, "f")
     T = b.types
     if arg_active is None:
@@ -656,6 +699,25 @@ def _reverse_custom_call(b, op, cs, accum):
         ta, tb_ = bool(cfg.get("trans_a", False)), bool(cfg.get("trans_b", False))
         A, Bm = xs[0], xs[1]
         gemm = lambda p, q, fa, fb, ty: b.custom_call("emi_gemm", [p, q], {"trans_a": fa, "trans_b": fb}, [ty])[0]
+        src = getattr(b, "producer", {}).get(A)
+        if (not ta and tb_ and src is not None and src.name == "custom_call" and src.attrs["target"] == "emi_gemm_swiglu_fwd"
+                and A == src.results[1] and b.uses.get(A, 0) == 1):
+            # y = g . w2^T with g = swiglu(a, b) of the launch before: dg = c . w2 goes through the SwiGLU adjoint in the
+            # epilogue of that product (emi_gemm_swiglu_bwd on the transposed down projection) and never reaches memory;
+            # da is the cotangent of a, db becomes the cotangent of the b result of the forward call
+            from . import _native as N
+            a_, b_res = src.operands[2], src.results[0]
+            w2t = b.emit("transpose", [Bm], {"perm": [1, 0]}, TensorType(tuple(reversed(T[Bm].shape)), T[Bm].dtype))
+            M_, K_, Hn = T[c].shape[0], T[c].shape[1], T[Bm].shape[1]
+            code = 16 if T[c].dtype == "bf16" else 11
+            nbytes = int(N.lib().emi_gemm_swiglu_bwd_workspace_bytes(M_, Hn, K_, code))
+            da, db, _ = b.custom_call("emi_gemm_swiglu_bwd", [c, w2t, a_, b_res], {}, [T[a_], T[b_res], TensorType((max(nbytes, 16),), "i8")])
+            accum(a_, da)
+            accum(b_res, db)
+            accum(Bm, gemm(c, A, True, False, T[Bm]))
+            if len(xs) > 2:
+                accum(xs[2], c)
+            return
         accum(A, gemm(c, Bm, False, not tb_, T[A]) if not ta else gemm(Bm, c, tb_, True, T[A]))
         accum(Bm, gemm(A, c, not ta, False, T[Bm]) if not tb_ else gemm(c, A, True, ta, T[Bm]))
         if len(xs) > 2:
@@ -681,6 +743,30 @@ def _reverse_custom_call(b, op, cs, accum):
             for i in live:
                 accum(x, b.custom_call("emi_gemm", [cs[i], xs[n_ + i]], {"trans_a": False, "trans_b": False}, [T[x]])[0])
                 accum(xs[n_ + i], b.custom_call("emi_gemm", [cs[i], x], {"trans_a": True, "trans_b": False}, [T[xs[n_ + i]]])[0])
+    elif target == "emi_gemm_rope":
+        # y = rope(x . w^T): the cotangent is turned back by the angle (unless the attention adjoint already did that as
+        # it stored dq / dk), then the DotGeneral rule
+        x, w, tab = xs
+        if c not in getattr(b, "unrotated", ()):
+            S_, d = T[tab].shape[0], 2 * T[tab].shape[1]
+            M_, D_ = T[c].shape
+            c4 = b.reshape(c, (M_ // S_, S_, D_ // d, d))
+            g4, = b.custom_call("emi_rope", [c4, tab], {"inverse": True}, [T[c4]])
+            c = b.reshape(g4, (M_, D_))
+        accum(x, b.custom_call("emi_gemm", [c, w], {"trans_a": False, "trans_b": False}, [T[x]])[0])
+        accum(w, b.custom_call("emi_gemm", [c, x], {"trans_a": True, "trans_b": False}, [T[w]])[0])
+    elif target == "emi_gemm_swiglu_fwd":
+        # (b, g) = (x . w3^T, swiglu(a, b)): a cotangent of g goes through the SwiGLU adjoint (the joint rule of the
+        # product that consumes g has usually taken it already), the total cotangent of b through the DotGeneral rule
+        x, w3, a_ = xs
+        cb, cg = cs[0], cs[1] if len(cs) > 1 else None
+        if cg is not None:
+            da, db = b.custom_call("emi_swiglu_bwd", [a_, op.results[0], cg], {}, [T[a_], T[op.results[0]]])
+            accum(a_, da)
+            cb = db if cb is None else b.binary("add", cb, db)
+        if cb is not None:
+            accum(x, b.custom_call("emi_gemm", [cb, w3], {"trans_a": False, "trans_b": False}, [T[x]])[0])
+            accum(w3, b.custom_call("emi_gemm", [cb, x], {"trans_a": True, "trans_b": False}, [T[w3]])[0])
     elif target == "emi_attn_fwd":
         if any(x is not None for x in cs[1:]):
             raise NotImplementedError("cotangents of the log-sum-exp or workspace results of emi_attn_fwd")
@@ -693,6 +779,26 @@ def _reverse_custom_call(b, op, cs, accum):
         qs = T[q].shape
         B_, S_, h, d = (qs[0], qs[1], qs[2], qs[3]) if bshd else (qs[0], qs[2], qs[1], qs[3])
         nbytes = int(N.lib().emi_attn_bwd_workspace_bytes(B_, h, S_, d))
+        # q and k that are (reshapes of) projections stored rotated with one table, each with this one use: the adjoint
+        # turns dq and dk back as it stores them
+        def rotated_projection(v_):
+            p_ = getattr(b, "producer", {}).get(v_)
+            if p_ is not None and p_.name == "reshape" and b.uses.get(v_, 0) == 1:
+                v_ = p_.operands[0]
+                p_ = b.producer.get(v_)
+            if p_ is not None and p_.name == "custom_call" and p_.attrs["target"] == "emi_gemm_rope" and b.uses.get(v_, 0) == 1:
+                return p_.operands[2]
+            return None
+        tq, tk = rotated_projection(q), rotated_projection(k)
+        if bshd and tq is not None and tq == tk and q != k:
+            dq, dk, dv, _ = b.custom_call("emi_attn_bwd_rope", [q, k, v, o, lse, c, tq],
+                                          {"scale": cfg["scale"], "causal": bool(cfg.get("causal", True)), "bshd": True},
+                                          [T[q], T[k], T[v], TensorType((nbytes,), "i8")])
+            b.unrotated.update((dq, dk))
+            accum(q, dq)
+            accum(k, dk)
+            accum(v, dv)
+            return
         dq, dk, dv, _ = b.custom_call("emi_attn_bwd", [q, k, v, o, lse, c],
                                       {"scale": cfg["scale"], "causal": bool(cfg.get("causal", True)), "bshd": bshd},
                                       [T[q], T[k], T[v], TensorType((nbytes,), "i8")])

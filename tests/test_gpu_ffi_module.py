@@ -99,7 +99,7 @@ def test_layer_modules_through_the_ffi_handlers():
         got = exe.run(ins)
         torch.cuda.synchronize()
         want = hlo_call(*ins, source=low)
-        assert len(calls) == low.count("stablehlo.custom_call") and set(calls) >= {"emi_gemm", "emi_attn_fwd", "emi_rope"}, name
+        assert len(calls) == low.count("stablehlo.custom_call") and set(calls) >= {"emi_gemm", "emi_attn_fwd", "emi_gemm_rope", "emi_gemm_swiglu_fwd"}, name
         for a, b in zip(got, want):
             assert torch.equal(a, b) if name == "primal" else _close(a, b, 2e-2), name
 

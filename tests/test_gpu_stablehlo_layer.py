@@ -107,8 +107,8 @@ def test_layer_text_forward_mode_adjoint_identity():
 
 
 def test_layer_text_lowered_and_symbolic_programs():
-    """optimize_module's three programs for the batched layer (clusters as emi_rmsnorm_fwd /
-    emi_rope / emi_attn_fwd / emi_swiglu_fwd custom calls; the reverse program with emi_attn_bwd
+    """optimize_module's three programs for the batched layer (clusters as emi_rmsnorm_fwd / emi_gemm_rope /
+    emi_attn_fwd / emi_gemm_swiglu_fwd custom calls; the reverse program with emi_attn_bwd_rope, emi_gemm_swiglu_bwd
     & co.; the forward program with emi_attn_jvp & co.) through hlo_call against the tape."""
     from enzyme_ad.jax import hlo_call, jvp, optimize_module, stablehlo_ad, vjp
     from enzyme_ad.jax import primitives as P
@@ -125,13 +125,14 @@ def test_layer_text_lowered_and_symbolic_programs():
         y, f_vjp = vjp(fn, *args)
         grads = f_vjp(dy)
         low = optimize_module(text)
-        assert low.count("stablehlo.custom_call") == 10 and low.count("@emi_gemm_grouped") == 2
+        assert low.count("stablehlo.custom_call") == 10 and low.count("@emi_gemm_rope") == 2 and low.count("@emi_gemm_swiglu_fwd") == 1
         assert "stablehlo.exponential" not in low and "stablehlo.dot_general" not in low
         y_low = hlo_call(*args, source=low)[0]
         assert torch.equal(y_low, y)
         fwd_pipe = P.forward_mode_pipeline(P.JaXPipeline(), [True] * len(args), 1)
         rev = optimize_module(text, P.reverse_mode_pipeline(fwd_pipe, [True]).pass_pipeline())
-        assert rev.count("@emi_attn_bwd") == 1 and rev.count("@emi_rmsnorm_bwd") == 2
+        assert rev.count("@emi_attn_bwd_rope") == 1 and rev.count("@emi_gemm_swiglu_bwd") == 1 and rev.count("@emi_rmsnorm_bwd") == 2
+        assert "@emi_rope" not in rev and "@emi_swiglu_bwd" not in rev
         sym = hlo_call(*(args + [dy]), source=rev)
         for name, g, t in zip(order, sym, grads):
             e = float((g.float() - t.float()).abs().max() / t.float().abs().max())

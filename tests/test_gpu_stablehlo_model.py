@@ -60,7 +60,7 @@ def test_model_text_loss_and_every_gradient(cfg, B, S, dt, loss):
 
 def test_model_text_logits_and_printed_modules_through_the_ffi_handlers():
     """Logits form at a reduced size: value and gradients against the oracle, then the printed primal and reverse
-    modules (sibling projections as `emi_gemm_grouped`, the lookup as `stablehlo.gather`, its adjoint as
+    modules (the sub-blocks of a layer on the targets with RoPE and SwiGLU in GEMM epilogues, the lookup as `stablehlo.gather`, its adjoint as
     `emi_embedding_bwd`) with every custom call
     served by the library's FFI handler, against `hlo_call` on the same text."""
     from enzyme_ad.jax import hlo_call, optimize_module, primitives as P, vjp
@@ -81,18 +81,20 @@ def test_model_text_logits_and_printed_modules_through_the_ffi_handlers():
     for k in MODEL_ORDER:
         check(gw[k], rgw[k], dt, "d" + k)
     low = optimize_module(text)
-    assert low.count("@emi_gemm_grouped") == 2 * cfg["n_layers"] and low.count('"stablehlo.gather"') == 1
+    assert low.count("@emi_gemm_rope") == 2 * cfg["n_layers"] and low.count("@emi_gemm_swiglu_fwd") == cfg["n_layers"]
+    assert low.count('"stablehlo.gather"') == 1
     assert "stablehlo.dot_general" not in low and "stablehlo.exponential" not in low
     active = [False] + [True] * len(MODEL_ORDER)
     fwd_pipe = P.forward_mode_pipeline(P.JaXPipeline(), active, 1)
     rev = optimize_module(text, P.reverse_mode_pipeline(fwd_pipe, [True]).pass_pipeline())
-    assert rev.count("@emi_attn_bwd") == cfg["n_layers"] and rev.count("@emi_embedding_bwd") == 1
+    assert rev.count("@emi_attn_bwd_rope") == cfg["n_layers"] and rev.count("@emi_gemm_swiglu_bwd") == cfg["n_layers"]
+    assert rev.count("@emi_embedding_bwd") == 1 and "@emi_rope" not in rev
     for name, prog, ins in (("primal", low, args), ("reverse", rev, args + [dout])):
         exe, calls = _ffi_executable(prog)
         got = exe.run(ins)
         torch.cuda.synchronize()
         want = hlo_call(*ins, source=prog)
-        assert len(calls) == prog.count("stablehlo.custom_call") and "emi_gemm_grouped" in calls, name
+        assert len(calls) == prog.count("stablehlo.custom_call") and "emi_gemm_rope" in calls and "emi_gemm_swiglu_fwd" in calls, name
         for a, b in zip(got, want):
             assert torch.equal(a, b) if name == "primal" else _close(a, b, 2e-2), name
     # the reverse program's gradients are the tape's

@@ -115,6 +115,35 @@ def test_run_list_joins_the_sub_blocks_of_a_layer():
     assert run["emi.ffn"] == 3 and run["emi.attention_block"] == 3 and run["emi.select"] == 27 and "emi.swiglu" not in run
 
 
+def test_optimize_module_prints_the_fused_epilogue_targets():
+    """The batched layer as optimize_module prints it: q and k projections stored rotated (`emi_gemm_rope`), the SwiGLU
+    in the epilogue of the w3 product (`emi_gemm_swiglu_fwd`); the reverse program turns dq / dk back inside the
+    attention adjoint (`emi_attn_bwd_rope`, no `emi_rope`) and runs the SwiGLU adjoint in the epilogue of dy . w2
+    (`emi_gemm_swiglu_bwd` on the transposed down projection, no `emi_swiglu_bwd`).  The forward-mode program keeps the
+    separate clusters (their tangent targets)."""
+    import re
+    from enzyme_ad.jax import optimize_module, primitives as P, stablehlo as S
+    from enzyme_ad.jax.llama_text import llama_layer_text
+
+    text, _ = llama_layer_text({"dim": 128, "hidden_dim": 352, "n_heads": 2}, 2, 40, "bf16")
+    calls = lambda t: re.findall(r"custom_call @(\w+)", t)
+    low = optimize_module(text)
+    assert calls(low) == ["emi_rmsnorm_fwd", "emi_gemm_rope", "emi_gemm_rope", "emi_gemm", "emi_attn_fwd", "emi_gemm", "emi_rmsnorm_fwd",
+                          "emi_gemm", "emi_gemm_swiglu_fwd", "emi_gemm"]
+    fwd_pipe = P.forward_mode_pipeline(P.JaXPipeline(), [True] * 10, 1)
+    rev = optimize_module(text, P.reverse_mode_pipeline(fwd_pipe, [True]).pass_pipeline())
+    rc = Counter(calls(rev))
+    assert rc["emi_attn_bwd_rope"] == 1 and rc["emi_gemm_swiglu_bwd"] == 1 and rc["emi_rmsnorm_bwd"] == 2
+    assert "emi_rope" not in rc and "emi_swiglu_bwd" not in rc and "emi_attn_bwd" not in rc
+    assert "stablehlo.transpose" in rev                                   # the down projection, transposed for the fused adjoint
+    line = [l for l in rev.splitlines() if "@emi_attn_bwd_rope" in l][0]
+    assert line.count("tensor<2x40x2x64xbf16>") >= 8 and "tensor<40x32x2xf32>" in line and "bshd = true" in line
+    fw = Counter(calls(optimize_module(text, fwd_pipe.pass_pipeline())))
+    assert fw["emi_rope"] == 4 and fw["emi_swiglu_jvp"] == 1 and fw["emi_attn_jvp"] == 1 and "emi_gemm_rope" not in fw
+    for t in (low, rev):
+        S.Executable(t, fuse=False)                                       # the printed text parses back
+
+
 def test_matcher_leaves_clusters_with_outside_uses_alone():
     from enzyme_ad.jax import stablehlo as S
 
