@@ -13,7 +13,10 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.mark.parametrize("dt", ["f32", "bf16"])
-@pytest.mark.parametrize("m,n,k", [(1, 288, 288), (1, 768, 288), (3, 520, 264), (8, 4096, 1024), (1, 11008, 4096)])
+@pytest.mark.parametrize("m,n,k", [(1, 288, 288), (1, 768, 288), (3, 520, 264), (8, 4096, 1024), (1, 11008, 4096),
+                                   (1, 4096, 11008),      # few long rows: two wavefronts share a row of W
+                                   (2, 1000, 20000),      # four wavefronts per row, two rows of x, a ragged last batch
+                                   (5, 301, 9000)])       # four per row in fp32, rows that do not fill the last block
 def test_skinny_gemm_forms(dt, m, n, k):
     """Y = X W^T (M <= 8 tokens), dX = dY W and dW = dY^T X with and without residual."""
     from enzyme_ad.jax import ops
