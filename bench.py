@@ -263,6 +263,28 @@ def bench_kernels(cfg, iters):
         hbm("cross_entropy_bwd_" + tag, lambda: N.check(lib.emi_cross_entropy_bwd(st, P(z), P(tgt), P(lse_t), P(dl), P(dz), Tk, V, code)), 2 * Tk * V * s)
         hbm("cross_entropy_jvp_" + tag, lambda: N.check(lib.emi_cross_entropy_jvp(st, P(z), P(tgt), P(lse_t), P(tz), P(loss), Tk, V, code)), 2 * Tk * V * s)
         del z, tz, dz
+    # The four GEMM launches of the C5 step that carry an elementwise part of the layer in their epilogue, priced as the
+    # plain product they replace (2 M N K flops): what the epilogue costs is the distance to the plain launch next to it.
+    T5, D5, H5, S5, hd5 = cfg["batch"] * cfg["seq"], cfg["dim"], cfg["hidden_dim"], cfg["seq"], cfg["dim"] // cfg["n_heads"]
+    x5 = torch.randn((T5, D5), device="cuda").to(bf)
+    wq5 = (torch.randn((D5, D5), device="cuda") * 0.02).to(bf)
+    w35 = (torch.randn((H5, D5), device="cuda") * 0.02).to(bf)
+    w2t5 = (torch.randn((H5, D5), device="cuda") * 0.02).to(bf)
+    y5 = torch.empty((T5, D5), device="cuda", dtype=bf)
+    a5 = torch.randn((T5, H5), device="cuda").to(bf)
+    b5, g5, d5 = (torch.empty((T5, H5), device="cuda", dtype=bf) for _ in range(3))
+    tab5 = ops.rope_table(S5, hd5)
+    mfma("gemm_plain_16384x4096x4096", lambda: N.check(lib.emi_gemm(st, P(x5), P(wq5), None, P(y5), T5, D5, D5, D5, D5, D5, D5, 0, 1,
+                                                                    N.EMI_BF16)), 2.0 * T5 * D5 * D5)
+    mfma("gemm_rope_16384x4096x4096", lambda: N.check(lib.emi_gemm_rope(st, P(x5), P(wq5), P(y5), P(tab5), T5, D5, D5, S5, hd5,
+                                                                        N.EMI_BF16)), 2.0 * T5 * D5 * D5)
+    mfma("gemm_plain_16384x11008x4096", lambda: N.check(lib.emi_gemm(st, P(x5), P(w35), None, P(b5), T5, H5, D5, D5, D5, H5, H5, 0, 1,
+                                                                     N.EMI_BF16)), 2.0 * T5 * H5 * D5)
+    mfma("gemm_swiglu_fwd_16384x11008x4096", lambda: N.check(lib.emi_gemm_swiglu_fwd(st, P(x5), P(w35), P(a5), P(b5), P(g5), T5, H5, D5,
+                                                                                     N.EMI_BF16)), 2.0 * T5 * H5 * D5)
+    mfma("gemm_swiglu_bwd_16384x11008x4096", lambda: N.check(lib.emi_gemm_swiglu_bwd(st, P(x5), P(w2t5), P(a5), P(b5), P(g5), P(d5), None,
+                                                                                     0, T5, H5, D5, N.EMI_BF16)), 2.0 * T5 * H5 * D5)
+    del x5, wq5, w35, w2t5, y5, a5, b5, g5, d5
     # C3: attention [8, 32, 2048, 128] bf16 causal
     B, h, S, d = 8, 32, 2048, 128
     q, k, v, do = (torch.randn((B, h, S, d), device="cuda").to(bf) for _ in range(4))
