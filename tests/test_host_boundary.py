@@ -119,6 +119,16 @@ def test_ffi_metadata_probe_and_stages():
      [(F.BF16, [1, 2, 64, 128])], {"causal": (F.PRED, 1)}, "scale"),
     ("emi_embedding_fwd_ffi", [(F.S64, [3]), (F.F32, [10, 4])], [(F.F32, [3, 4])], {}, "s32"),
     ("emi_swiglu_bwd_ffi", [(F.F32, [8])] * 3, [(F.F32, [8]), (F.F32, [9])], {}, "shape"),
+    ("emi_gemm_rope_ffi", [(F.BF16, [32, 16]), (F.BF16, [64, 16]), (F.BF16, [16, 32, 2])], [(F.BF16, [32, 64])], {}, "table"),
+    ("emi_gemm_rope_ffi", [(F.BF16, [32, 16]), (F.BF16, [64, 24]), (F.F32, [16, 32, 2])], [(F.BF16, [32, 64])], {}, "contraction"),
+    ("emi_gemm_rope_ffi", [(F.BF16, [32, 16]), (F.BF16, [64, 16]), (F.F32, [16, 32, 2])], [(F.BF16, [32, 60])], {}, "y must be"),
+    ("emi_gemm_swiglu_fwd_ffi", [(F.BF16, [32, 16]), (F.BF16, [64, 16]), (F.BF16, [32, 48])], [(F.BF16, [32, 64])] * 2, {}, "a, b, g"),
+    ("emi_gemm_swiglu_bwd_ffi", [(F.BF16, [32, 16]), (F.BF16, [64, 16]), (F.BF16, [32, 64]), (F.F32, [32, 64])],
+     [(F.BF16, [32, 64])] * 2, {}, "dtype"),
+    ("emi_attn_bwd_rope_ffi", [(F.BF16, [1, 64, 2, 128])] * 4 + [(F.F32, [1, 2, 64]), (F.BF16, [1, 64, 2, 128]), (F.F32, [64, 32, 2])],
+     [(F.BF16, [1, 64, 2, 128])] * 3 + [(F.U8, [1024])], {"scale": (F.F32, 0.1), "bshd": (F.PRED, 1)}, "table"),
+    ("emi_attn_bwd_rope_ffi", [(F.BF16, [1, 64, 2, 128])] * 4 + [(F.F32, [1, 2, 64]), (F.BF16, [1, 64, 2, 128]), (F.F32, [64, 64, 2])],
+     [(F.BF16, [1, 64, 2, 128])] * 3 + [(F.U8, [8])], {"scale": (F.F32, 0.1), "bshd": (F.PRED, 1)}, "workspace"),
 ])
 def test_ffi_rejects_malformed_frames(name, args, rets, attrs, needle):
     xla = F.FakeXla()
