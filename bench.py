@@ -227,6 +227,10 @@ def bench_kernels(cfg, iters):
                                                                          i64([D, 1]), 0, s)), n * s)
         hbm("transpose_copy_" + tag, lambda: N.check(lib.emi_strided_copy(st, P(a), P(y), 2, i64([D, rows]), i64([1, D]), 0,
                                                                           i64([rows, 1]), 0, s)), 2 * n * s)
+        # what a plain read-and-write pass over the same bytes reaches here: torch's device copy (a yardstick for the
+        # transpose above; not a product kernel)
+        hbm("device_copy_yardstick_" + tag, lambda: y.copy_(a), 2 * n * s)
+        out["device_copy_yardstick_" + tag]["yardstick"] = "torch.Tensor.copy_ of the same [32768, 4096] operand"
         rwb = max(lib.emi_reduce_workspace_bytes(1, rows, D, code), lib.emi_reduce_workspace_bytes(1, n, 1, code), 16)
         rws = torch.empty(rwb, dtype=torch.uint8, device="cuda")
         hbm("reduce_rows_" + tag, lambda: N.check(lib.emi_reduce(st, HO.REDUCE["add"], P(a), P(col), None, 0, rows, D, 1, code)), n * s)
@@ -351,7 +355,15 @@ def bench_kernels(cfg, iters):
     hbm("step_matvec_dx_bf16", lambda: N.check(lib.emi_gemm_ws(st, P(dyv), P(rot(wsr)), None, P(dxv), P(gws), gwb, 1, D, H, H, D, D, D,
                                                                0, 0, N.EMI_BF16)), w.numel() * 2, in_graph=True)
     hbm("step_matvec_dw_bf16", lambda: gm(dyv, xv, rot(dwr), H, D, 1, H, D, 1, 0), w.numel() * 2, in_graph=True)
-    for k_ in ("step_matvec_bf16", "step_matvec_dx_bf16", "step_matvec_dw_bf16"):
+    # what reading such a matrix once costs with nothing else to do: a sum over all its elements, timed the same way
+    # (a yardstick for the three mat-vec entries; not a kernel of the step)
+    rwb1 = max(lib.emi_reduce_workspace_bytes(1, w.numel(), 1, N.EMI_BF16), 16)
+    rws1 = torch.empty(rwb1, dtype=torch.uint8, device="cuda")
+    one1 = torch.empty(1, device="cuda").to(bf)
+    hbm("step_read_yardstick_bf16", lambda: N.check(lib.emi_reduce(st, HO.REDUCE["add"], P(rot(wsr)), P(one1), P(rws1), rwb1, 1, w.numel(), 1,
+                                                                   N.EMI_BF16)), w.numel() * 2, in_graph=True)
+    out["step_read_yardstick_bf16"]["yardstick"] = "emi_reduce(add) over one [11008, 4096] matrix, same rotation and timing"
+    for k_ in ("step_matvec_bf16", "step_matvec_dx_bf16", "step_matvec_dw_bf16", "step_read_yardstick_bf16"):
         out[k_]["operands"] = "four [11008, 4096] matrices in rotation (360 MB), none of them cache-resident"
     del wsr, dwr, w, gws
     return out

@@ -74,7 +74,7 @@ def test_elementwise_maps_match_numpy(dt, n):
 
 
 @pytest.mark.parametrize("dt", ["f32", "bf16"])
-@pytest.mark.parametrize("n", [1, 9, 4099])
+@pytest.mark.parametrize("n", [1, 9, 4099, 70001])
 def test_compare_and_select_match_numpy(dt, n):
     from enzyme_ad.jax import hlo_ops as H
 
@@ -136,7 +136,10 @@ def test_strided_copy_forms_match_numpy(dt):
 
 @pytest.mark.parametrize("dt", ["f32", "bf16"])
 @pytest.mark.parametrize("shape,dims", [((37, 5000), [1]), ((37, 5000), [0]), ((4, 33, 7), [1]), ((4, 33, 7), [0, 2]),
-                                        ((2, 3, 4), [0, 1, 2]), ((300, 64), [1]), ((1, 100003), [1])])
+                                        ((2, 3, 4), [0, 1, 2]), ((300, 64), [1]), ((1, 100003), [1]),
+                                        # column sums split into bands of rows: a partial strip of columns, a strip of one
+                                        # wavefront, several outer slices, more strips than one
+                                        ((4096, 1000), [0]), ((3000, 96), [0]), ((2, 700, 520), [1]), ((1500, 5000), [0])])
 def test_reduce_matches_numpy(dt, shape, dims):
     from enzyme_ad.jax import hlo_ops as H
 
