@@ -67,7 +67,7 @@ def test_plain_launchers_reject_bad_arguments_before_touching_the_gpu():
     assert lib.emi_reduce(None, 0, 16, 16, None, 0, 4, 0, 1, 11) == 3          # empty reduction
     assert lib.emi_reduce_workspace_bytes(32768, 4096, 1, 16) == 0             # plenty of rows: one stage
     assert lib.emi_reduce_workspace_bytes(1, 1 << 27, 1, 16) == 2048 * 4       # full sum: 2048 fp32 partials
-    assert lib.emi_reduce_workspace_bytes(1, 32768, 4096, 11) == 512 * 4096 * 4   # column sum: 512 bands of 64 rows
+    assert lib.emi_reduce_workspace_bytes(1, 32768, 4096, 11) == 64 * 4096 * 4    # column sum: 4 strips x 64 bands of 512 rows, a block per CU
 
 
 def _handler(name):
