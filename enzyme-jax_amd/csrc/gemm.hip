@@ -797,8 +797,14 @@ template <int N, typename F> __device__ __forceinline__ void static_for(F&& f) {
 // sum == 0); otherwise the last argument is an empty placeholder.
 // EPI: 0 = the result [+ R]; 1 / 2 = the SwiGLU epilogues (epilogue_swiglu_t16; R is P0, C is Q0, plus P1 and Q1);
 // 3 = the result [+ R] with RoPE applied to it (epilogue_bf16_t16<..., ROPE>); 4 = as 0 for matrices of whole tiles and
-// 16-byte accesses (the launcher checks): without the code for ragged tiles the kernel needs no scratch memory.
+// 16-byte accesses (the launcher checks): without the code for ragged tiles the kernel needs no scratch memory;
+// 5 = split-K: the grid holds tiles x splits blocks, split-major; split z owns k in [z * k_per_split, ...) and leaves its
+// fp32 tile in part[z][M][N] for gemm_splitk_reduce_kernel (k-contiguous operands only).
 struct NoEpi {};
+struct SplitEpi {
+  float* part;
+  int k_per_split;
+};
 struct SwigluEpi {
   const uint16_t* P1;
   uint16_t* Q1;
@@ -811,6 +817,7 @@ template <int EPI> struct EpiArg { using type = NoEpi; };
 template <> struct EpiArg<1> { using type = SwigluEpi; };
 template <> struct EpiArg<2> { using type = SwigluEpi; };
 template <> struct EpiArg<3> { using type = RopeEpi; };
+template <> struct EpiArg<5> { using type = SplitEpi; };
 template <bool AKM, bool BKM, bool GROUPED = false, int EPI = 0>
 __global__ __launch_bounds__(512) void gemm_bf16_pingpong_kernel(const uint16_t* __restrict__ A,
                                                                   const uint16_t* __restrict__ B, const uint16_t* R,
@@ -833,6 +840,7 @@ __global__ __launch_bounds__(512) void gemm_bf16_pingpong_kernel(const uint16_t*
 
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
   int tile_m, tile_n;
+  [[maybe_unused]] int split = 0;
   if constexpr (GROUPED) {
     const int pid = xcd_contiguous_id(), tiles = tiles_m * tiles_n;
     const int prod = pid / tiles;
@@ -841,6 +849,17 @@ __global__ __launch_bounds__(512) void gemm_bf16_pingpong_kernel(const uint16_t*
     B = grp.B[prod];
     R = grp.R[prod];
     C = grp.C[prod];
+  } else if constexpr (EPI == 5) {
+    static_assert(!AKM && !BKM, "split-K serves the k-contiguous layout");
+    const int pid = xcd_contiguous_id(), tiles = tiles_m * tiles_n;
+    split = pid / tiles;
+    tile_coords(pid - split * tiles, tiles_m, tiles_n, &tile_m, &tile_n);
+    const int k_lo = split * epi.k_per_split;                      // < K: the launcher sizes the grid
+    A += k_lo;
+    B += k_lo;
+    a_bytes -= (uint32_t)k_lo * 2u;
+    b_bytes -= (uint32_t)k_lo * 2u;
+    K = K - k_lo < epi.k_per_split ? K - k_lo : epi.k_per_split;
   } else {
     // With a long contraction and k-contiguous operands, groups of 4 tile-rows measured 3 % faster than 8
     // ([16384, 11008] x [4096, 11008]^T: 975 vs 1005 us): an XCD then re-reads the (cache-resident) weight panels
@@ -1063,7 +1082,40 @@ __global__ __launch_bounds__(512) void gemm_bf16_pingpong_kernel(const uint16_t*
   wait_vmcnt<0>();                          // zero-filled loads past the end of K
   slot_end();
 
-  if constexpr (EPI == 3) {
+  if constexpr (EPI == 5) {
+    // accumulator layout (swapped operands): register r of lane l holds row l % 16, column 4 * (l / 16) + r of its 16x16
+    // tile.  Each wavefront stages 32 rows x 64 columns of fp32 at a time through its own slice of the idle LDS (rows 16
+    // bytes further apart than their 256) and writes them as whole 256-byte rows, four per store instruction.
+    constexpr int RS = 64 * 4 + 16;
+    EMI_LDS uint8_t* wl = smem + wave * (32 * RS);
+    float* pz = epi.part + (int64_t)split * M * N;
+    const bool vec4 = (N & 3) == 0;
+    const int lr = lane & 15, lg = lane >> 4;
+#pragma unroll
+    for (int p = 0; p < 4; p++) {
+#pragma unroll
+      for (int ii = 0; ii < 2; ii++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+          *reinterpret_cast<EMI_LDS f32x4_t*>(wl + (16 * ii + lr) * RS + (16 * j + 4 * lg) * 4) = acc[2 * p + ii][j];
+#pragma unroll
+      for (int it = 0; it < 8; it++) {
+        const int row = it * 4 + lg, c = lr * 4;
+        const f32x4_t v = *reinterpret_cast<const EMI_LDS f32x4_t*>(wl + row * RS + c * 4);
+        const int grow = m0 + wm * 128 + 32 * p + row, gcol = n0 + wn * 64 + c;
+        if (grow < M && gcol < N) {
+          float* dst = pz + (int64_t)grow * N + gcol;
+          if (vec4) {
+            *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+              if (gcol + e < N) dst[e] = v[e];
+          }
+        }
+      }
+    }
+  } else if constexpr (EPI == 3) {
     static_assert(!AKM && !BKM && !GROUPED, "the RoPE epilogue belongs to the k-contiguous single product");
     epilogue_bf16_t16<8, 4, 0, true>(acc, smem, wave, lane, m0 + wm * 128, n0 + wn * 64, R, C, M, N, ldr, ldc, vec_ok, epi.table,
                                      epi.seq, epi.head_dim);
@@ -1444,24 +1496,93 @@ __global__ __launch_bounds__(256) void gemm_f32_tiled_kernel(const float* __rest
     }
 }
 
-template <typename T>
+// VEC: a thread owns four consecutive columns of a row (N, ldr and ldc multiples of 4, rows of R and C aligned for one
+// access of four elements): 16-byte loads from every plane.
+template <typename T, bool VEC = false>
 __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __restrict__ part, const T* R, T* C, int M, int N,
                                                                  int splits, int64_t ldr, int64_t ldc) {
-  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  constexpr int V = VEC ? 4 : 1;
+  const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * V;
   if (i >= (int64_t)M * N) return;
   const int row = (int)(i / N), col = (int)(i - (int64_t)row * N);
-  float v = 0.f;
+  const int64_t plane = (int64_t)M * N;
+  float v[V];
+#pragma unroll
+  for (int e = 0; e < V; e++) v[e] = 0.f;
+  auto load = [&](int z, float (&t)[V]) {
+    if constexpr (VEC) {
+      const float4 q = *reinterpret_cast<const float4*>(part + z * plane + i);
+      t[0] = q.x; t[1] = q.y; t[2] = q.z; t[3] = q.w;
+    } else {
+      t[0] = part[z * plane + i];
+    }
+  };
   int z = 0;
   for (; z + 8 <= splits; z += 8) {                       // eight loads in flight, added in plane order
-    float t[8];
+    float t[8][V];
 #pragma unroll
-    for (int u = 0; u < 8; u++) t[u] = part[(int64_t)(z + u) * M * N + i];
+    for (int u = 0; u < 8; u++) load(z + u, t[u]);
 #pragma unroll
-    for (int u = 0; u < 8; u++) v += t[u];
+    for (int u = 0; u < 8; u++)
+#pragma unroll
+      for (int e = 0; e < V; e++) v[e] += t[u][e];
   }
-  for (; z < splits; z++) v += part[(int64_t)z * M * N + i];
-  if (R != nullptr) v += to_f32(R[(int64_t)row * ldr + col]);
-  C[(int64_t)row * ldc + col] = from_f32<T>(v);
+  if (z + 4 <= splits) {
+    float t[4][V];
+#pragma unroll
+    for (int u = 0; u < 4; u++) load(z + u, t[u]);
+#pragma unroll
+    for (int u = 0; u < 4; u++)
+#pragma unroll
+      for (int e = 0; e < V; e++) v[e] += t[u][e];
+    z += 4;
+  }
+  for (; z < splits; z++) {
+    float t[V];
+    load(z, t);
+#pragma unroll
+    for (int e = 0; e < V; e++) v[e] += t[e];
+  }
+  if constexpr (VEC) {
+    if (R != nullptr) {
+      if constexpr (sizeof(T) == 2) {
+        const u32x2_t r = *reinterpret_cast<const u32x2_t*>(R + (int64_t)row * ldr + col);
+        v[0] += __uint_as_float(r[0] << 16); v[1] += __uint_as_float(r[0] & 0xffff0000u);
+        v[2] += __uint_as_float(r[1] << 16); v[3] += __uint_as_float(r[1] & 0xffff0000u);
+      } else {
+        const float4 r = *reinterpret_cast<const float4*>(R + (int64_t)row * ldr + col);
+        v[0] += r.x; v[1] += r.y; v[2] += r.z; v[3] += r.w;
+      }
+    }
+    if constexpr (sizeof(T) == 2) {
+      u32x2_t o;
+      o[0] = pack_bf16x2(v[0], v[1]);
+      o[1] = pack_bf16x2(v[2], v[3]);
+      *reinterpret_cast<u32x2_t*>(C + (int64_t)row * ldc + col) = o;
+    } else {
+      *reinterpret_cast<float4*>(C + (int64_t)row * ldc + col) = make_float4(v[0], v[1], v[2], v[3]);
+    }
+  } else {
+    if (R != nullptr) v[0] += to_f32(R[(int64_t)row * ldr + col]);
+    C[(int64_t)row * ldc + col] = from_f32<T>(v[0]);
+  }
+}
+
+// Launches the reduction of `splits` fp32 planes [M, N] (+ R) into C.
+template <typename T>
+static void launch_splitk_reduce(hipStream_t st, const float* part, const void* R, void* C, int M, int N, int splits, int64_t ldr,
+                                 int64_t ldc) {
+  const uintptr_t al = 4 * sizeof(T) - 1;
+  const bool vec = N % 4 == 0 && ldc % 4 == 0 && (reinterpret_cast<uintptr_t>(C) & al) == 0 && (reinterpret_cast<uintptr_t>(part) & 15) == 0 &&
+                   (R == nullptr || (ldr % 4 == 0 && (reinterpret_cast<uintptr_t>(R) & al) == 0));
+  const int64_t items = vec ? (int64_t)M * N / 4 : (int64_t)M * N;
+  const dim3 grid((unsigned)((items + 255) / 256));
+  if (vec)
+    hipLaunchKernelGGL((gemm_splitk_reduce_kernel<T, true>), grid, dim3(256), 0, st, part, static_cast<const T*>(R), static_cast<T*>(C), M,
+                       N, splits, ldr, ldc);
+  else
+    hipLaunchKernelGGL((gemm_splitk_reduce_kernel<T, false>), grid, dim3(256), 0, st, part, static_cast<const T*>(R), static_cast<T*>(C), M,
+                       N, splits, ldr, ldc);
 }
 
 // Few output tiles and a long contraction (the logits adjoint dX = dY . Wcls of a small batch:
@@ -1501,8 +1622,7 @@ static int launch_bf16(hipStream_t st, const void* A, const void* B, const void*
                        static_cast<const uint16_t*>(B), static_cast<const uint16_t*>(R), static_cast<uint16_t*>(C), M, N, K,
                        lda, ldb, ldr, ldc, a_bytes, b_bytes, vec_ok, part, kps, GemmGroup{});
     EMI_CHECK_LAUNCH("emi_gemm(split-K)");
-    hipLaunchKernelGGL(gemm_splitk_reduce_kernel<bf16>, dim3((unsigned)(((int64_t)M * N + 255) / 256)), dim3(256), 0, st, part,
-                       static_cast<const bf16*>(R), static_cast<bf16*>(C), M, N, nz, (int64_t)ldr, (int64_t)ldc);
+    launch_splitk_reduce<bf16>(st, part, R, C, M, N, nz, (int64_t)ldr, (int64_t)ldc);
     EMI_CHECK_LAUNCH("emi_gemm(split-K reduce)");
     return EMI_OK;
   }
@@ -1570,9 +1690,7 @@ static int launch_bf16_grouped(hipStream_t st, const GemmGroup& g, int M, int N,
                        ldr, ldc, a_bytes, b_bytes, vec_ok, part, kps, g);
     EMI_CHECK_LAUNCH("emi_gemm_grouped(split-K)");
     for (int i = 0; i < g.count; i++) {
-      hipLaunchKernelGGL(gemm_splitk_reduce_kernel<bf16>, dim3((unsigned)(((int64_t)M * N + 255) / 256)), dim3(256), 0, st,
-                         part + (int64_t)i * nz * M * N, reinterpret_cast<const bf16*>(g.R[i]), reinterpret_cast<bf16*>(g.C[i]), M, N,
-                         nz, (int64_t)ldr, (int64_t)ldc);
+      launch_splitk_reduce<bf16>(st, part + (int64_t)i * nz * M * N, g.R[i], g.C[i], M, N, nz, (int64_t)ldr, (int64_t)ldc);
       EMI_CHECK_LAUNCH("emi_gemm_grouped(split-K reduce)");
     }
     return EMI_OK;
@@ -1674,6 +1792,43 @@ static int launch_bf16_rope(hipStream_t st, const void* A, const void* B, void* 
   return EMI_OK;
 }
 
+// Split-K on the 256x256 ping-pong kernel: k-contiguous products with too few 256-tiles for that kernel, too many
+// 128-tiles for bf16_splits and a long contraction (dX of the classifier of a small model, [8192, 32000] x [32000, 768]:
+// 96 tiles of 256, 384 of 128).  The 128-tile kernel runs those at 0.75 PFLOP/s (two blocks on half the CUs, one on the
+// others); four splits are 384 ping-pong blocks at 1.1 PFLOP/s plus the reduction of 4 x M x N fp32 partials.
+static int pingpong_splits(int64_t M, int64_t N, int64_t K, bool k_contiguous) {
+  if (!k_contiguous || K < 8192) return 1;
+  const int64_t big = ((M + 255) / 256) * ((N + 255) / 256), t128 = ((M + 127) / 128) * ((N + 127) / 128);
+  if (big >= 192 || t128 <= 128 || big > 128) return 1;
+  int64_t s = (320 + big - 1) / big;
+  if (s > 8) s = 8;
+  while (s > 1 && K / s < 2048) s--;
+  return (int)s;
+}
+
+static int launch_bf16_pingpong_splitk(hipStream_t st, const void* A, const void* B, const void* R, void* C, int M, int N, int K,
+                                       int lda, int ldb, int ldr, int ldc, uint32_t a_bytes, uint32_t b_bytes, float* part,
+                                       int splits) {
+  auto kern = gemm_bf16_pingpong_kernel<false, false, false, 5>;
+  constexpr int smem = 2 * 65536;
+  static bool configured = false;   // idempotent; a race only repeats the call
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return emi_fail(EMI_INTERNAL, "emi_gemm: cannot reserve %d bytes of LDS: %s", smem, hipGetErrorString(e));
+    configured = true;
+  }
+  const int tiles = ((M + 255) / 256) * ((N + 255) / 256);
+  const int kps = (((K + splits - 1) / splits) + 63) / 64 * 64;
+  const int nz = (K + kps - 1) / kps;
+  hipLaunchKernelGGL(kern, dim3(tiles * nz), dim3(512), smem, st, static_cast<const uint16_t*>(A), static_cast<const uint16_t*>(B),
+                     static_cast<const uint16_t*>(nullptr), static_cast<uint16_t*>(nullptr), M, N, K, lda, ldb, ldr, ldc, a_bytes,
+                     b_bytes, 0, NoGroup{}, SplitEpi{part, kps});
+  EMI_CHECK_LAUNCH("emi_gemm(split-K, 256-tiles)");
+  launch_splitk_reduce<bf16>(st, part, R, C, M, N, nz, (int64_t)ldr, (int64_t)ldc);
+  EMI_CHECK_LAUNCH("emi_gemm(split-K reduce)");
+  return EMI_OK;
+}
+
 // The 128x128 bf16 kernel on few tiles and a long contraction (the weight gradients of a small model:
 // dW[768, 768] over 8192 tokens is 36 tiles): two blocks per CU, at least 1024 of K per block.
 static int bf16_splits(int64_t M, int64_t N, int64_t K) {
@@ -1694,6 +1849,13 @@ static int launch_bf16_layout(hipStream_t st, const void* A, const void* B, cons
       workspace_bytes >= (size_t)splits * M * N * sizeof(float))
     return launch_bf16<128, 128, 64, 2, 2, 2, AK, BKM>(st, A, B, R, C, M, N, K, lda, ldb, ldr, ldc, a_bytes, b_bytes,
                                                       static_cast<float*>(workspace), splits);
+  if constexpr (!AK && !BKM) {
+    const int pps = pingpong_splits(M, N, K, true);
+    if (pps > 1 && workspace != nullptr && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0 &&
+        workspace_bytes >= (size_t)pps * M * N * sizeof(float))
+      return launch_bf16_pingpong_splitk(st, A, B, R, C, M, N, K, lda, ldb, ldr, ldc, a_bytes, b_bytes,
+                                         static_cast<float*>(workspace), pps);
+  }
   // 256x256 tiles (the ping-pong kernel) when they fill the chip, else 128x128.
   const int64_t big_tiles = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
   if (big_tiles >= 192) return launch_bf16_pingpong<AK, BKM>(st, A, B, R, C, M, N, K, lda, ldb, ldr, ldc, a_bytes, b_bytes);
@@ -1723,8 +1885,7 @@ static int launch_generic(hipStream_t st, const void* A, const void* B, const vo
     float* part = static_cast<float*>(workspace);
     EMI_GENERIC(part, kps);
     EMI_CHECK_LAUNCH("emi_gemm(generic split-K)");
-    hipLaunchKernelGGL(gemm_splitk_reduce_kernel<T>, dim3((unsigned)(((int64_t)M * N + 255) / 256)), dim3(256), 0, st, part,
-                       static_cast<const T*>(R), static_cast<T*>(C), M, N, (int)grid.z, ldr, ldc);
+    launch_splitk_reduce<T>(st, part, R, C, M, N, (int)grid.z, ldr, ldc);
     EMI_CHECK_LAUNCH("emi_gemm(generic split-K reduce)");
     return EMI_OK;
   }
@@ -1753,6 +1914,7 @@ extern "C" size_t emi_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int 
   // 128x128 bf16 kernel would use, since alignment decides between them at launch time)
   int splits = generic_splits(M, N, K);
   if (dtype == EMI_BF16 && bf16_splits(M, N, K) > splits) splits = bf16_splits(M, N, K);
+  if (dtype == EMI_BF16 && pingpong_splits(M, N, K, !trans_a && trans_b) > splits) splits = pingpong_splits(M, N, K, true);
   return splits > 1 ? (size_t)splits * M * N * sizeof(float) : 0;
 }
 
@@ -1837,8 +1999,7 @@ extern "C" int emi_gemm_ws(emi_stream_t stream, const void* A, const void* B, co
         else EMI_F32_TILED_SPLIT(true, false);
 #undef EMI_F32_TILED_SPLIT
         EMI_CHECK_LAUNCH("emi_gemm(fp32 tiled split-K)");
-        hipLaunchKernelGGL(gemm_splitk_reduce_kernel<float>, dim3((unsigned)(((int64_t)M * N + 255) / 256)), dim3(256), 0, st, part,
-                           static_cast<const float*>(R), static_cast<float*>(C), (int)M, (int)N, (int)grid.z, ldr, ldc);
+        launch_splitk_reduce<float>(st, part, R, C, (int)M, (int)N, (int)grid.z, ldr, ldc);
         EMI_CHECK_LAUNCH("emi_gemm(fp32 split-K reduce)");
         return EMI_OK;
       }
@@ -1852,8 +2013,7 @@ extern "C" int emi_gemm_ws(emi_stream_t stream, const void* A, const void* B, co
       else EMI_F32_SPLIT(true, false);
 #undef EMI_F32_SPLIT
       EMI_CHECK_LAUNCH("emi_gemm(fp32 split-K)");
-      hipLaunchKernelGGL(gemm_splitk_reduce_kernel<float>, dim3((unsigned)(((int64_t)M * N + 255) / 256)), dim3(256), 0, st, part,
-                         static_cast<const float*>(R), static_cast<float*>(C), (int)M, (int)N, (int)grid.z, ldr, ldc);
+      launch_splitk_reduce<float>(st, part, R, C, (int)M, (int)N, (int)grid.z, ldr, ldc);
       EMI_CHECK_LAUNCH("emi_gemm(fp32 split-K reduce)");
       return EMI_OK;
     }

@@ -115,11 +115,17 @@ int emi_gemm(emi_stream_t stream, const void* A, const void* B, const void* R, v
              int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldr, int64_t ldc,
              int trans_a, int trans_b, int dtype);
 
-/* The same with an optional scratch buffer.  Only the single-token adjoint
- * dX = dY.W (trans_a = trans_b = 0, M <= 8) uses one: with
- * emi_gemm_workspace_bytes() bytes it sums row bands of W in many blocks and
- * adds the partial sums in a fixed order (about 3x faster); without, or for
- * any other shape, the call is emi_gemm. */
+/* The same with an optional scratch buffer of emi_gemm_workspace_bytes() bytes (0
+ * for shapes that need none).  With it, the single-token adjoint dX = dY.W
+ * (trans_a = trans_b = 0, M <= 8) sums row bands of W in many blocks (about 3x
+ * faster), and products with few output tiles and a long contraction split K
+ * over more blocks, each leaving an fp32 partial [M,N] plane: the weight
+ * gradients of a small model on the 128x128 kernel, and in the bf16
+ * Y = X.W^T form the shapes with more than 128 tiles of 128x128 but fewer than
+ * 192 of 256x256 and K >= 8192 (the classifier adjoint [8192,32000].[32000,768]
+ * of a 110M model) on the 256x256 kernel.  The planes are added in a fixed
+ * order, with R, before the single rounding.  Without the buffer, or for any
+ * other shape, the call is emi_gemm. */
 size_t emi_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int trans_a, int trans_b, int dtype);
 int emi_gemm_ws(emi_stream_t stream, const void* A, const void* B, const void* R, void* C,
                 void* workspace, size_t workspace_bytes, int64_t M, int64_t N, int64_t K,

@@ -107,6 +107,8 @@ GEMM_SHAPES = [
     (100, 200, 2600),    # split-K on the generic kernel for both dtypes where M is not a multiple of 8
     (64, 101, 4096),     # split-K with rows of the partials that are not 16-byte aligned (scalar partial stores)
     (256, 288, 32000),   # the logits adjoint dX = dY . Wcls of the 15M model: 50 planes of K
+    (2300, 1000, 8264),  # more than 128 tiles of 128, fewer than 192 of 256, long contraction: in the NT bf16 form split-K
+                         # on the 256-tile kernel (36 tiles x 4 splits, ragged rows and columns, a ragged last k-tile)
 ]
 
 

@@ -68,6 +68,12 @@ def test_plain_launchers_reject_bad_arguments_before_touching_the_gpu():
     assert lib.emi_reduce_workspace_bytes(32768, 4096, 1, 16) == 0             # plenty of rows: one stage
     assert lib.emi_reduce_workspace_bytes(1, 1 << 27, 1, 16) == 2048 * 4       # full sum: 2048 fp32 partials
     assert lib.emi_reduce_workspace_bytes(1, 32768, 4096, 11) == 64 * 4096 * 4    # column sum: 4 strips x 64 bands of 512 rows, a block per CU
+    # split-K partials of the GEMM: none where the 256-tile kernel fills the chip, four planes for the classifier adjoint of
+    # a small model in the NT bf16 form (96 tiles of 256, K = 32000), none for the same shape in another layout or in fp32
+    assert lib.emi_gemm_workspace_bytes(16384, 4096, 4096, 0, 1, 16) == 0
+    assert lib.emi_gemm_workspace_bytes(8192, 768, 32000, 0, 1, 16) == 4 * 8192 * 768 * 4
+    assert lib.emi_gemm_workspace_bytes(8192, 768, 32000, 0, 0, 16) == 0
+    assert lib.emi_gemm_workspace_bytes(8192, 768, 32000, 0, 1, 11) == 0
 
 
 def _handler(name):
