@@ -858,6 +858,10 @@ __device__ __forceinline__ void unrope_quad(const float* t, float& x0, float& x1
 // ---------------------------------------------------------------------------
 // dQ: block = 4 waves x 32 queries; K and V tiles of 64 keys through LDS.
 //   S^T = K Q^T, dP^T = V dO^T, dS^T = P^T (dP^T - delta), dQ^T = K^T dS^T
+// With `o` given the kernel also does the adjoint's pre-pass for its 128 queries: delta = rowsum(dO . O) from the dO
+// fragments it holds anyway and the matching fragments of O (a lane and its partner 32 lanes on hold alternate groups
+// of eight elements of a row), written as delta * delta_sign to delta_out and lse * log2(e) to lse2_out for the dK/dV kernel, which then has
+// to run after this one.  Without `o`, delta comes in through `delta`.
 // ---------------------------------------------------------------------------
 template <int D>
 __global__ __launch_bounds__(256, 2) void attn_bwd_dq_bf16_kernel(const uint16_t* __restrict__ q,
@@ -868,7 +872,9 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_bf16_kernel(const uint16_t
                                                                const float* __restrict__ delta,
                                                                uint16_t* __restrict__ dq, AttnShape sh,
                                                                uint32_t head_bytes, float scale, int causal,
-                                                               float delta_sign, const float* __restrict__ unrope) {
+                                                               float delta_sign, const float* __restrict__ unrope,
+                                                               const uint16_t* __restrict__ o, float* __restrict__ delta_out,
+                                                               float* __restrict__ lse2_out) {
   constexpr int BQ = 128, BKV = 64, NW = 4;
   constexpr int TILE = BKV * D * 2, STAGE = 2 * TILE;
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem_raw[];
@@ -888,7 +894,35 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_bf16_kernel(const uint16_t
   load_reg_rows<D>(q + base, qrow, seq, sh.ss, lane, qf);
   load_reg_rows<D>(d_o + base, qrow, seq, sh.ss, lane, dof);
   const float L2 = qrow < seq ? lse[(int64_t)bh * seq + qrow] * kLog2e : 0.f;
-  const float dl = qrow < seq ? delta[(int64_t)bh * seq + qrow] * delta_sign : 0.f;
+  float dl;
+  if (o != nullptr) {
+    bf16x8_t of[D / 16];
+    load_reg_rows<D>(o + base, qrow, seq, sh.ss, lane, of);
+    // sums of eight products, then pairs of them 8, 4, 2 and 1 apart (the last pair is the partner lane's)
+    float cs[D / 16];
+#pragma unroll
+    for (int t = 0; t < D / 16; t++) {
+      const u32x4_t a = __builtin_bit_cast(u32x4_t, of[t]), b = __builtin_bit_cast(u32x4_t, dof[t]);
+      float c = 0.f;
+#pragma unroll
+      for (int w = 0; w < 4; w++) {
+        c += __uint_as_float(a[w] << 16) * __uint_as_float(b[w] << 16);
+        c += __uint_as_float(a[w] & 0xffff0000u) * __uint_as_float(b[w] & 0xffff0000u);
+      }
+      cs[t] = c;
+    }
+#pragma unroll
+    for (int m = D / 32; m >= 1; m >>= 1)
+#pragma unroll
+      for (int t = 0; t < m; t++) cs[t] += cs[t + m];
+    dl = cs[0] + __shfl_xor(cs[0], 32, 64);
+    if (qrow < seq && lane < 32) {
+      delta_out[(int64_t)bh * seq + qrow] = dl * delta_sign;
+      lse2_out[(int64_t)bh * seq + qrow] = L2;
+    }
+  } else {
+    dl = qrow < seq ? delta[(int64_t)bh * seq + qrow] * delta_sign : 0.f;
+  }
 
   const __amdgpu_buffer_rsrc_t rK = attn_rsrc(k + base, head_bytes);
   const __amdgpu_buffer_rsrc_t rV = attn_rsrc(v + base, head_bytes);
@@ -965,35 +999,6 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_bf16_kernel(const uint16_t
         w.y = pack_bf16x2(x2, x3);
         *reinterpret_cast<uint2*>(out + dcol) = w;
       }
-  }
-}
-
-// ---------------------------------------------------------------------------
-// Adjoint pre-pass for the MFMA kernels: delta[row] = sum_i dO*O (times delta_sign) and
-// lse2[row] = lse * log2(e).  16-byte loads, D/8 lanes per row.
-// ---------------------------------------------------------------------------
-template <int D>
-__global__ __launch_bounds__(256) void attn_prep_kernel(const uint16_t* __restrict__ o, const uint16_t* __restrict__ d_o,
-                                                        const float* __restrict__ lse, float* __restrict__ delta,
-                                                        float* __restrict__ lse2, AttnShape sh, float delta_sign) {
-  constexpr int LPR = D / 8, RPB = 256 / LPR;          // lanes per row, rows per block
-  const int qi = blockIdx.x * RPB + threadIdx.x / LPR;
-  const int bh = blockIdx.y;
-  const int c = threadIdx.x % LPR;
-  float s = 0.f;
-  if (qi < sh.seq) {
-    const int64_t off = (int64_t)(bh / sh.heads) * sh.sb + (int64_t)(bh % sh.heads) * sh.sh + (int64_t)qi * sh.ss + c * 8;
-    float a[8], b[8];
-    Vec8<bf16>::load(reinterpret_cast<const bf16*>(o) + off, a);
-    Vec8<bf16>::load(reinterpret_cast<const bf16*>(d_o) + off, b);
-#pragma unroll
-    for (int e = 0; e < 8; e++) s += a[e] * b[e];
-  }
-#pragma unroll
-  for (int m = LPR / 2; m > 0; m >>= 1) s += __shfl_xor(s, m, 64);
-  if (qi < sh.seq && c == 0) {
-    delta[(int64_t)bh * sh.seq + qi] = s * delta_sign;
-    lse2[(int64_t)bh * sh.seq + qi] = lse[(int64_t)bh * sh.seq + qi] * kLog2e;
   }
 }
 
@@ -1620,12 +1625,7 @@ static int attn_bwd_impl(emi_stream_t stream, const void* q, const void* k, cons
   const bool fast = mfma_ok(a, dtype, {q, k, v, o, d_o, dq, dk, dv});
   const float delta_sign = -1.0f;          // the MFMA kernels accumulate dP onto -delta
   if (fast) {
-    if (head_dim == 128)
-      hipLaunchKernelGGL(attn_prep_kernel<128>, dim3((unsigned)((seq + 15) / 16), bh), dim3(256), 0, st, (const uint16_t*)o,
-                         (const uint16_t*)d_o, lse, delta, lse2, shp, delta_sign);
-    else
-      hipLaunchKernelGGL(attn_prep_kernel<64>, dim3((unsigned)((seq + 31) / 32), bh), dim3(256), 0, st, (const uint16_t*)o,
-                         (const uint16_t*)d_o, lse, delta, lse2, shp, delta_sign);
+    // the dQ kernel computes delta and lse * log2(e) for its own queries and leaves them for the dK/dV kernel
   } else if (dtype == EMI_BF16)
     hipLaunchKernelGGL(attn_delta_kernel<bf16>, grid4, dim3(256), 0, st, (const bf16*)o, (const bf16*)d_o, delta, shp,
                        (int)head_dim);
@@ -1640,20 +1640,20 @@ static int attn_bwd_impl(emi_stream_t stream, const void* q, const void* k, cons
   do {                                                                                                                   \
     constexpr int smem_q = 2 * 2 * 64 * DD * 2;                                                                          \
     constexpr int smem_sp = 6 * 64 * DD * 2 + 3 * 512;                                                                   \
+    if (int rc = reserve_lds(attn_bwd_dq_bf16_kernel<DD>, smem_q, "emi_attn_bwd")) return rc;                            \
+    hipLaunchKernelGGL(attn_bwd_dq_bf16_kernel<DD>, grid, dim3(256), smem_q, st, (const uint16_t*)q, (const uint16_t*)k, \
+                       (const uint16_t*)v, (const uint16_t*)d_o, lse, (const float*)nullptr, (uint16_t*)dq, shp,         \
+                       head_bytes, scale, causal, delta_sign, unrope, (const uint16_t*)o, delta, lse2);                  \
+    EMI_CHECK_LAUNCH("emi_attn_bwd(dq)");                                                                                \
     if (int rc = reserve_lds(attn_bwd_dkv_sp_kernel<DD>, smem_sp, "emi_attn_bwd")) return rc;                            \
     hipLaunchKernelGGL(attn_bwd_dkv_sp_kernel<DD>, grid, dim3(256), smem_sp, st, (const uint16_t*)q,                     \
                        (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse2, delta, (uint16_t*)dk,         \
                        (uint16_t*)dv, shp, head_bytes, scale, causal, unrope);                                           \
-    EMI_CHECK_LAUNCH("emi_attn_bwd(dkv)");                                                                               \
-    if (int rc = reserve_lds(attn_bwd_dq_bf16_kernel<DD>, smem_q, "emi_attn_bwd")) return rc;                            \
-    hipLaunchKernelGGL(attn_bwd_dq_bf16_kernel<DD>, grid, dim3(256), smem_q, st, (const uint16_t*)q, (const uint16_t*)k, \
-                       (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, (uint16_t*)dq, shp, head_bytes, scale,      \
-                       causal, delta_sign, unrope);                                                                      \
   } while (0)
     if (head_dim == 128) EMI_ATTN_BWD_LAUNCH(128);
     else EMI_ATTN_BWD_LAUNCH(64);
 #undef EMI_ATTN_BWD_LAUNCH
-    EMI_CHECK_LAUNCH("emi_attn_bwd(dq)");
+    EMI_CHECK_LAUNCH("emi_attn_bwd(dkv)");
     return EMI_OK;
   }
   if (dtype == EMI_F32) {
