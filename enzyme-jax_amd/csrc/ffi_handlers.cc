@@ -249,7 +249,7 @@ extern "C" XLA_FFI_Error* emi_add_ffi(XLA_FFI_CallFrame* cf) {
 extern "C" XLA_FFI_Error* emi_gemm_ffi(XLA_FFI_CallFrame* cf) {
   EMI_FFI_BEGIN("emi_gemm", 2, 3, 1, 2)
   const XLA_FFI_Buffer *A = f.arg(0), *B = f.arg(1), *R = cf->args.size == 3 ? f.arg(2) : nullptr, *C = f.ret(0);
-  const XLA_FFI_Buffer* ws = cf->rets.size == 2 ? f.ret(1) : nullptr;      // optional scratch (single-token dX)
+  const XLA_FFI_Buffer* ws = cf->rets.size == 2 ? f.ret(1) : nullptr;      // optional scratch (emi_gemm_workspace_bytes)
   if (!is_float(A) || B->dtype != A->dtype || C->dtype != A->dtype || (R && R->dtype != A->dtype))
     return f.invalid("A, B, C (and R) must share one dtype, f32 or bf16 (code %lld)", A->dtype);
   if (A->rank != 2 || B->rank != 2 || C->rank != 2 || (R && R->rank != 2)) return f.invalid("operands must be rank 2 (A rank %lld, B rank %lld)", A->rank, B->rank);
