@@ -432,10 +432,92 @@ def reverse_function(func, name=None, arg_active=None, ret_active=None):
         if t.dtype not in FLOAT:
             raise ValueError("argument %s of type %r cannot be active" % (a, t))
         outs.append(ct[a] if a in ct else b.const(0.0, t))
+    outs = _group_adjoint_products(b, outs)
     b.ops.append(Op("return", [], outs, {}, []))
     rev = Func(name or func.name + "_rev", list(func.args) + ct_args, [T[o] for o in outs], b.ops)
     _drop_dead(rev)
     return rev
+
+
+def _group_adjoint_products(b, outs):
+    """The adjoint products of sibling projections as the tape issues them (ops._group_rule): the fan-in
+    dX = dY_0 . W_0 + dY_1 . W_1 + ... of single products and adds becomes one summed emi_gemm_grouped (one rounding
+    instead of one per product and add), and the weight gradients dW_i = dY_i^T . X that share X become one grouped
+    call.  Works on the emitted list in place; returns the (renamed) results."""
+    ops, T = b.ops, b.types
+    uses = {}
+    for op in ops:
+        for o in op.operands:
+            uses[o] = uses.get(o, 0) + 1
+    for o in outs:
+        uses[o] = uses.get(o, 0) + 1
+    prod = {r: op for op in ops for r in op.results}
+
+    def gemm_flags(op):
+        if op is None or op.name != "custom_call" or op.attrs["target"] != "emi_gemm" or len(op.operands) != 2:
+            return None
+        cfg = op.attrs["config"]
+        return bool(cfg.get("trans_a", False)), bool(cfg.get("trans_b", False))
+
+    # fan-in sums: trees of adds whose leaves are all single-use results of plain products of one shape
+    absorbed = set()
+    for idx in range(len(ops) - 1, -1, -1):
+        op = ops[idx]
+        if op.name != "add" or id(op) in absorbed:
+            continue
+        leaves, inner, stack = [], [], [op]
+        while stack:
+            a = stack.pop()
+            for v in a.operands:
+                p_ = prod.get(v)
+                if p_ is not None and p_.name == "add" and uses.get(v, 0) == 1:
+                    inner.append(p_)
+                    stack.append(p_)
+                else:
+                    leaves.append(v)
+        srcs = [prod.get(v) for v in leaves]
+        if not (2 <= len(leaves) <= 48) or len(set(leaves)) != len(leaves) or \
+                any(gemm_flags(g) != (False, False) or uses.get(v, 0) != 1 for v, g in zip(leaves, srcs)):
+            continue
+        if any(T[g.operands[0]] != T[srcs[0].operands[0]] or T[g.operands[1]] != T[srcs[0].operands[1]] for g in srcs):
+            continue
+        srcs.sort(key=lambda g: next(i for i, o in enumerate(ops) if o is g))       # the order the products were emitted in
+        ops[idx] = Op("custom_call", list(op.results), [g.operands[0] for g in srcs] + [g.operands[1] for g in srcs],
+                      {"target": "emi_gemm_grouped", "config": {"count": len(srcs), "sum": True, "trans_a": False, "trans_b": False}},
+                      list(op.types))
+        absorbed.update(id(a) for a in inner)
+    # weight gradients that share their second operand: one grouped call where the last of them stood
+    groups = {}
+    for idx, op in enumerate(ops):
+        if gemm_flags(op) == (True, False):
+            groups.setdefault((op.operands[1], repr(T[op.operands[0]]), repr(op.types[0])), []).append(idx)
+    first_use = {}
+    for idx, op in enumerate(ops):
+        for o in op.operands:
+            first_use.setdefault(o, idx)
+    rename, drop = {}, set()
+    for (x, _, _), idxs in groups.items():
+        last = idxs[-1]
+        idxs = [i for i in idxs if first_use.get(ops[i].results[0], len(ops)) > last][:48]
+        if len(idxs) < 2 or idxs[-1] != last:
+            continue
+        tys = [ops[i].types[0] for i in idxs]
+        base = b.new(tys[0])
+        names = ["%s#%d" % (base, k) for k in range(len(idxs))]
+        for n_, t_ in zip(names, tys):
+            T[n_] = t_
+        for i, n_ in zip(idxs, names):
+            rename[ops[i].results[0]] = n_
+        grouped = Op("custom_call", names, [ops[i].operands[0] for i in idxs] + [x] * len(idxs),
+                     {"target": "emi_gemm_grouped", "config": {"count": len(idxs), "sum": False, "trans_a": True, "trans_b": False}}, tys)
+        drop.update(idxs[:-1])
+        ops[last] = grouped
+    if rename:
+        for op in ops:
+            op.operands = [rename.get(o, o) for o in op.operands]
+        outs = [rename.get(o, o) for o in outs]
+    b.ops = [op for i, op in enumerate(ops) if i not in drop]
+    return outs
 
 
 def forward_function(func, name=None, arg_active=None):

@@ -136,6 +136,10 @@ def test_optimize_module_prints_the_fused_epilogue_targets():
     assert rc["emi_attn_bwd_rope"] == 1 and rc["emi_gemm_swiglu_bwd"] == 1 and rc["emi_rmsnorm_bwd"] == 2
     assert "emi_rope" not in rc and "emi_swiglu_bwd" not in rc and "emi_attn_bwd" not in rc
     assert "stablehlo.transpose" in rev                                   # the down projection, transposed for the fused adjoint
+    # the adjoint products of sibling projections, as the tape issues them: dxb = dq . wq + dk . wk + dv . wv as one summed
+    # launch and dwq, dwk, dwv as one grouped launch; the same for the pair w1 / w3
+    grouped = sorted(re.findall(r"@emi_gemm_grouped\(.*?count = (\d+).*?sum = (\w+).*?trans_a = (\w+)", rev))
+    assert grouped == [("2", "false", "true"), ("2", "true", "false"), ("3", "false", "true"), ("3", "true", "false")], grouped
     line = [l for l in rev.splitlines() if "@emi_attn_bwd_rope" in l][0]
     assert line.count("tensor<2x40x2x64xbf16>") >= 8 and "tensor<40x32x2xf32>" in line and "bshd = true" in line
     fw = Counter(calls(optimize_module(text, fwd_pipe.pass_pipeline())))
