@@ -1811,16 +1811,17 @@ def _custom_call_impl(self, op, xs):
         a, b_ = _packed(xs[0]), _packed(xs[1])
         r = _packed(xs[2]) if len(xs) > 2 else None
         ta, tb_ = bool(cfg.get("trans_a", False)), bool(cfg.get("trans_b", False))
+        ws = [None] * (len(op.results) - 1)                             # a declared scratch result: ops brings its own
         if not ta and tb_:
-            return [ops.matmul_nt(a, b_, residual=r)]                   # the projection form: differentiable on the tape
-        return [ops.gemm(a, b_, ta, tb_, r)]                            # the forms derivative programs use
+            return [ops.matmul_nt(a, b_, residual=r)] + ws              # the projection form: differentiable on the tape
+        return [ops.gemm(a, b_, ta, tb_, r)] + ws                       # the forms derivative programs use
     if target == "emi_gemm_grouped":
         n_, sum_ = int(cfg["count"]), bool(cfg.get("sum", False))
         ta, tb_ = bool(cfg.get("trans_a", False)), bool(cfg.get("trans_b", False))
         As, Bs = [_packed(t) for t in xs[:n_]], [_packed(t) for t in xs[n_:2 * n_]]
         rs = [_packed(t) for t in xs[2 * n_:]] or None
         if not ta and tb_ and not sum_ and rs is None and all(a is As[0] for a in As):
-            return list(ops.matmul_nt_group(As[0], Bs))                  # sibling projections: differentiable on the tape
+            return list(ops.matmul_nt_group(As[0], Bs)) + [None] * (len(op.results) - n_)      # sibling projections: differentiable on the tape
         out = ops.gemm_grouped(As, Bs, ta, tb_, rs, sum_into_one=sum_)   # the forms derivative programs use
         return ([out] if sum_ else list(out)) + [None] * (len(op.results) - (1 if sum_ else n_))
     if target == "emi_add":

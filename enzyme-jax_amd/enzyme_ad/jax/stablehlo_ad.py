@@ -54,7 +54,32 @@ class _Builder:
         ty = TensorType(shape, self.types[v].dtype)
         return v if self.types[v].shape == ty.shape else self.emit("reshape", [v], {}, ty)
 
+    def _gemm_workspace(self, target, operands, config):
+        """Bytes of scratch the GEMM targets use for split-K partials (0 for most shapes): declared as an extra i8 result,
+        which their handlers take when it is there."""
+        from . import _native as N
+        n = int(config.get("count", 1)) if target == "emi_gemm_grouped" else 1
+        ta, tb = bool(config.get("trans_a", False)), bool(config.get("trans_b", False))
+        at, bt = self.types[operands[0]], self.types[operands[n]]
+        if len(at.shape) != 2 or len(bt.shape) != 2 or at.dtype not in ("f32", "bf16"):
+            return 0
+        M, K = (at.shape[1], at.shape[0]) if ta else at.shape
+        Nn = bt.shape[0] if tb else bt.shape[1]
+        code = 16 if at.dtype == "bf16" else 11
+        if target == "emi_gemm":
+            return int(N.lib().emi_gemm_workspace_bytes(M, Nn, K, int(ta), int(tb), code))
+        return int(N.lib().emi_gemm_grouped_workspace_bytes(n, M, Nn, K, int(ta), int(tb), int(bool(config.get("sum", False))), code))
+
     def custom_call(self, target, operands, config, tys):
+        tys = list(tys)
+        nres = len(tys)
+        if target in ("emi_gemm", "emi_gemm_grouped"):
+            nbytes = self._gemm_workspace(target, operands, config)
+            if nbytes:
+                tys.append(TensorType((nbytes,), "i8"))
+        return self._call(target, operands, config, tys)[:nres]
+
+    def _call(self, target, operands, config, tys):
         base = self.new(tys[0])
         names = [base] if len(tys) == 1 else ["%s#%d" % (base, i) for i in range(len(tys))]
         for n, t in zip(names, tys):
@@ -459,8 +484,9 @@ def _group_adjoint_products(b, outs):
         cfg = op.attrs["config"]
         return bool(cfg.get("trans_a", False)), bool(cfg.get("trans_b", False))
 
-    # fan-in sums: trees of adds whose leaves are all single-use results of plain products of one shape
-    absorbed = set()
+    # fan-in sums: trees of adds whose leaves are all single-use results of plain products of one shape (2 to 4 of them:
+    # what the emi_gemm_grouped handler takes)
+    absorbed, sum_rename = set(), {}
     for idx in range(len(ops) - 1, -1, -1):
         op = ops[idx]
         if op.name != "add" or id(op) in absorbed:
@@ -476,15 +502,23 @@ def _group_adjoint_products(b, outs):
                 else:
                     leaves.append(v)
         srcs = [prod.get(v) for v in leaves]
-        if not (2 <= len(leaves) <= 48) or len(set(leaves)) != len(leaves) or \
+        if not (2 <= len(leaves) <= 4) or len(set(leaves)) != len(leaves) or \
                 any(gemm_flags(g) != (False, False) or uses.get(v, 0) != 1 for v, g in zip(leaves, srcs)):
             continue
         if any(T[g.operands[0]] != T[srcs[0].operands[0]] or T[g.operands[1]] != T[srcs[0].operands[1]] for g in srcs):
             continue
         srcs.sort(key=lambda g: next(i for i, o in enumerate(ops) if o is g))       # the order the products were emitted in
-        ops[idx] = Op("custom_call", list(op.results), [g.operands[0] for g in srcs] + [g.operands[1] for g in srcs],
-                      {"target": "emi_gemm_grouped", "config": {"count": len(srcs), "sum": True, "trans_a": False, "trans_b": False}},
-                      list(op.types))
+        cfg_ = {"count": len(srcs), "sum": True, "trans_a": False, "trans_b": False}
+        operands_ = [g.operands[0] for g in srcs] + [g.operands[1] for g in srcs]
+        nbytes = b._gemm_workspace("emi_gemm_grouped", operands_, cfg_)
+        if nbytes:                    # the sum and its scratch as results #0, #1 of one call
+            base = b.new(op.types[0])
+            names_ = [base + "#0", base + "#1"]
+            T[names_[0]], T[names_[1]] = op.types[0], TensorType((nbytes,), "i8")
+            sum_rename[op.results[0]] = names_[0]
+            ops[idx] = Op("custom_call", names_, operands_, {"target": "emi_gemm_grouped", "config": cfg_}, [op.types[0], T[names_[1]]])
+        else:
+            ops[idx] = Op("custom_call", list(op.results), operands_, {"target": "emi_gemm_grouped", "config": cfg_}, list(op.types))
         absorbed.update(id(a) for a in inner)
     # weight gradients that share their second operand: one grouped call where the last of them stood
     groups = {}
@@ -495,10 +529,10 @@ def _group_adjoint_products(b, outs):
     for idx, op in enumerate(ops):
         for o in op.operands:
             first_use.setdefault(o, idx)
-    rename, drop = {}, set()
+    rename, drop = dict(sum_rename), set()
     for (x, _, _), idxs in groups.items():
         last = idxs[-1]
-        idxs = [i for i in idxs if first_use.get(ops[i].results[0], len(ops)) > last][:48]
+        idxs = [i for i in idxs if first_use.get(ops[i].results[0], len(ops)) > last][-4:]      # 2 to 4 products per call
         if len(idxs) < 2 or idxs[-1] != last:
             continue
         tys = [ops[i].types[0] for i in idxs]
@@ -508,8 +542,14 @@ def _group_adjoint_products(b, outs):
             T[n_] = t_
         for i, n_ in zip(idxs, names):
             rename[ops[i].results[0]] = n_
-        grouped = Op("custom_call", names, [ops[i].operands[0] for i in idxs] + [x] * len(idxs),
-                     {"target": "emi_gemm_grouped", "config": {"count": len(idxs), "sum": False, "trans_a": True, "trans_b": False}}, tys)
+        cfg_ = {"count": len(idxs), "sum": False, "trans_a": True, "trans_b": False}
+        operands_ = [ops[i].operands[0] for i in idxs] + [x] * len(idxs)
+        nbytes = b._gemm_workspace("emi_gemm_grouped", operands_, cfg_)
+        if nbytes:
+            names = names + ["%s#%d" % (base, len(idxs))]
+            tys = tys + [TensorType((nbytes,), "i8")]
+            T[names[-1]] = tys[-1]
+        grouped = Op("custom_call", names, operands_, {"target": "emi_gemm_grouped", "config": cfg_}, tys)
         drop.update(idxs[:-1])
         ops[last] = grouped
     if rename:

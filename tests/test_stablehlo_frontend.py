@@ -262,6 +262,11 @@ def test_symbolic_reverse_of_the_llama_step_calls_the_adjoint_targets():
                        "emi_swiglu_bwd": 1, "emi_attn_step_bwd": 1, "emi_gemm": 7 + 14}      # 7 projections, dX and dW of each
     assert sorted(o.attrs["config"]["inverse"] for o in f.ops if o.name == "custom_call" and o.attrs["target"] == "emi_rope") == \
         [False, False, True, True]
+    # the seven dx = dy . W products of one token declare the scratch their kernel sums row bands in (an extra i8 result
+    # of emi_gemm_workspace_bytes bytes, which the handler takes when it is there); no other product needs one
+    with_ws = [o for o in f.ops if o.name == "custom_call" and o.attrs["target"] == "emi_gemm" and len(o.results) == 2]
+    assert len(with_ws) == 7 and all(o.types[1].dtype == "i8" and not o.attrs["config"]["trans_a"] and not o.attrs["config"]["trans_b"]
+                                     for o in with_ws)
     assert len(f.args) == len(order) + 1 and f.args[-1][1].shape == (288,)
     assert [t.shape for t in f.result_types] == [t.shape for _, t in f.args[:-1]]
     assert S.print_module(S.parse_module(rev)) == rev
