@@ -14,7 +14,10 @@ Prints ONE JSON line on stdout (everything else goes to stderr):
   kernels   the same figure for every other kernel of the path at its
             configuration-C2/C3/C5 shape (HBM GB/s or MFMA TFLOP/s)
             (`vendor`: torch.matmul = hipBLASLt timed on the same launches in the same
-            run, a yardstick only: the library is never on the product path)
+            run, a yardstick only: the library is never on the product path; entries
+            with a `yardstick` key - a device copy, a plain sum over one weight - say
+            what a pass of that size and shape reaches here, next to the transposes and
+            the single-token mat-vec kernels they are measured against)
   cpu_baseline  a PyTorch-CPU fp32 restatement of test/llama.py (oracle/llama_torch.py,
             autograd as the VJP) timed on the host cores on a bounded sample
             (reported next to the GPU number, not a target)
